@@ -1,0 +1,187 @@
+/*
+ * libscn_hip.so -- C ABI of the MI355X (gfx950) implementation of
+ * SparseConvNet's spatially-sparse forward path.
+ *
+ * The reference has no plugin interface; its seam is the set of free functions
+ * that the layer classes' preprocess()/forwards() call with raw device
+ * pointers and a stream.  Each entry point below names the reference function
+ * it stands in for (paths relative to the reference's SparseConvNet/ folder).
+ *
+ * Conventions
+ *   - every function returns SCN_OK or an SCN_ERR_* code; scn_last_error()
+ *     gives the message of the calling thread's last failure (the reference
+ *     prints and exit(-1)s instead, utilities.h:36-67);
+ *   - all device work is issued on the context's single stream
+ *     (cudaMemStream, utilities.cu:171-178) and is asynchronous unless the
+ *     function has to hand a count back to the host;
+ *   - pointers named d_* are device pointers, h_* host pointers;
+ *   - feature matrices are row-major fp32 [rows x channels]; rule books are
+ *     row-major int32 [output rows x rule width]; rows are batch-global;
+ *   - numeric kernels never allocate: every buffer is the caller's
+ *     (SpatiallySparseBatchSubInterface, SpatiallySparseBatchInterface.h:8-17).
+ *     scn_grids objects own their tables and only ever grow them.
+ */
+#ifndef SCN_HIP_H
+#define SCN_HIP_H
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  SCN_OK = 0,
+  SCN_ERR_ARG = 1,      /* bad argument (the reference would assert) */
+  SCN_ERR_HIP = 2,      /* a HIP runtime call failed */
+  SCN_ERR_CAPACITY = 3, /* a caller buffer or an index range is too small */
+  SCN_ERR_STATE = 4     /* call order violated (e.g. fill without plan) */
+};
+
+/* ActivationFunction, types.h:11-20 (same numbering) */
+enum {
+  SCN_NOSIGMOID = 0,
+  SCN_RELU = 1,
+  SCN_VLEAKYRELU = 2,
+  SCN_LEAKYRELU = 3,
+  SCN_TANH = 4, /* not on the forward configs: rejected */
+  SCN_SOFTMAX = 5,
+  SCN_PRELU = 6,
+  SCN_SIGMOID = 7 /* rejected */
+};
+
+enum { SCN_FP32 = 0, SCN_BF16 = 1 }; /* operand precision of the NiN contraction */
+
+typedef struct scn_ctx scn_ctx;
+typedef struct scn_grids scn_grids;
+
+const char *scn_last_error(void);
+const char *scn_version(void);
+
+/* ---- context: device, stream, copies --------------------------------- */
+/* initializeGPU (utilities.cu:105-130) + cudaMemStream ctor (:171-174).
+ * device < 0 selects device 0. */
+int scn_ctx_create(int device, scn_ctx **ctx);
+int scn_ctx_destroy(scn_ctx *ctx);
+/* the hipStream_t all work is issued on */
+void *scn_ctx_stream(scn_ctx *ctx);
+int scn_sync(scn_ctx *ctx);
+/* vectorCUDA<T> device storage (vectorCUDA.cu:26-108): raw allocate / free /
+ * blocking copies / fill. */
+int scn_malloc(scn_ctx *ctx, size_t bytes, void **d_ptr);
+int scn_free(scn_ctx *ctx, void *d_ptr);
+int scn_h2d(scn_ctx *ctx, void *d_dst, const void *h_src, size_t bytes);
+int scn_d2h(scn_ctx *ctx, void *h_dst, const void *d_src, size_t bytes);
+int scn_fill32(scn_ctx *ctx, void *d_dst, uint32_t word, size_t nWords);
+
+/* ---- sparse grids ----------------------------------------------------- */
+/* A scn_grids holds, for one depth of the net, the SparseGrid of every sample
+ * of the batch (SparseGrid.h:26-37, SpatiallySparseBatchInterface.h:36):
+ * an open-addressing hash table in HBM from the packed coordinate
+ * sample * spatialSize^dimension + key to the batch-global row, an occupancy
+ * bit mask over the same packed coordinates, and backgroundCol per sample. */
+int scn_grids_create(scn_ctx *ctx, scn_grids **grids);
+int scn_grids_destroy(scn_ctx *ctx, scn_grids *grids);
+/* The input-layer grids as Picture::codifyInputData leaves them
+ * (Picture.h:10-11; OpenCVPicture.cpp:368-402): n active sites given as
+ * (sample, key, row) in any order, key = row-major site index in the
+ * spatialSize^dimension field, plus backgroundCol per sample (-1: none) and
+ * the interface's nSpatialSites.  Keys must be unique within a sample. */
+int scn_grids_build(scn_ctx *ctx, scn_grids *grids, int batch, int dimension,
+                    int spatialSize, const int32_t *d_sample,
+                    const int64_t *d_key, const int32_t *d_row, int64_t n,
+                    const int32_t *d_background, int32_t nSpatialSites);
+int scn_grids_info(const scn_grids *grids, int *batch, int *dimension,
+                   int *spatialSize, int64_t *nActive, int32_t *nSpatialSites);
+/* Every entry in map iteration order (sample, then ascending key), and
+ * backgroundCol[batch].  Host arrays of nActive / batch elements. */
+int scn_grids_download(scn_ctx *ctx, const scn_grids *grids, int32_t *h_sample,
+                       int64_t *h_key, int32_t *h_row, int32_t *h_background);
+/* mp.find() for n packed queries (sample, key) -> row or -1; device arrays. */
+int scn_grids_find(scn_ctx *ctx, const scn_grids *grids,
+                   const int32_t *d_sample, const int64_t *d_key, int64_t n,
+                   int32_t *d_row);
+
+/* ---- rule books -------------------------------------------------------- */
+/* Rule construction is split in two so that the caller owns the rules buffer
+ * (SpatiallySparseBatchInterface::rules): plan() finds the output sites,
+ * numbers them in the reference's first-touch order under ascending-key map
+ * iteration and builds `out`; fill() writes the rules.
+ *
+ * gridRules(in, out, RegularSquareRegions(nIn, nOut, dimension, size, stride),
+ *           nOutputSpatialSites, rules, true, minActive) for every sample
+ * (Regions.h:84-87; Regions.cu:528-653 NoMin, :338-526 Min, :658-780 Valid,
+ * dispatcher :782-802), as ConvolutionalLayer::preprocess and
+ * MaxPoolingLayer::preprocess call it (ConvolutionalLayer.cu:110-118,
+ * MaxPoolingLayer.cu:113-118).  minActive: 1, >1, or -1 (valid, 2-D size 3). */
+int scn_rules_square_plan(scn_ctx *ctx, const scn_grids *in, scn_grids *out,
+                          int nIn, int nOut, int size, int stride,
+                          int minActive, int64_t *nOutputSpatialSites);
+/* gridRules(in, out, RegularTriangularRegions(...), n, rules, minActive)
+ * (Regions.h:120-127; Regions.cu:834-970 NoMin, :972-1164 Min). */
+int scn_rules_triangular_plan(scn_ctx *ctx, const scn_grids *in,
+                              scn_grids *out, int nIn, int nOut, int size,
+                              int stride, int minActive,
+                              int64_t *nOutputSpatialSites);
+/* TerminalPoolingLayer::preprocess + terminalGridPoolingRules
+ * (TerminalPoolingLayer.cu:8-20,81-97).  *ruleWidth = S. */
+int scn_rules_terminal_plan(scn_ctx *ctx, const scn_grids *in, scn_grids *out,
+                            int64_t *ruleWidth);
+/* Rule width of the plan held by `out` (size^d, triangleSize, or S). */
+int scn_rules_width(const scn_grids *out, int64_t *width);
+/* Writes nOutputSpatialSites * width int32 rules; capacity in int32s. */
+int scn_rules_fill(scn_ctx *ctx, const scn_grids *in, scn_grids *out,
+                   int32_t *d_rules, int64_t capacity);
+
+/* ---- feature kernels --------------------------------------------------- */
+/* propForwardToMatrixMultiply (ConvolutionalLayer.h:38-40;
+ * ConvolutionalLayer.cu:12-41): out[c*nIn + j] = in[rules[c]*nIn + j],
+ * c < count.  A negative rule (the reference does not guard them) is refused
+ * by the host check only in debug builds; rule books from this library never
+ * hold one here. */
+int scn_gather_rows(scn_ctx *ctx, const float *d_in, float *d_out,
+                    const int32_t *d_rules, int64_t count, int nIn);
+/* replicateArray + d_rowMajorSGEMM_alphaAB_betaC(alpha = beta = p) +
+ * applySigmoid / PreLU, test-time branch (NetworkInNetworkLayer.cu:187-200,
+ * NetworkInNetworkPReLULayer.cu:158-169; utilities.cu:135-142;
+ * SigmoidLayer.cu:187-222): out[M x N] = act(p * (A[M x K] W[K x N] + B)).
+ * d_prelu is the per-channel slope vector for SCN_PRELU, else ignored.
+ * SCN_SOFTMAX applies dSigmoidSoftmax (SigmoidLayer.cu:160-177) to the rows. */
+int scn_nin_forward(scn_ctx *ctx, const float *d_A, const float *d_W,
+                    const float *d_B, const float *d_prelu, float *d_out,
+                    int64_t M, int K, int N, float p, int act, int precision);
+/* maxPool (MaxPoolingLayer.h:6-7; MaxPoolingLayer.cu:9-72): first maximum
+ * wins, negative rules skipped, choice = rule * C + channel. */
+int scn_maxpool(scn_ctx *ctx, const float *d_in, float *d_out,
+                const int32_t *d_rules, int64_t nOutSites, int ps, int C,
+                int32_t *d_choice);
+/* terminalPool (TerminalPoolingLayer.cu:22-46): mean over the rows listed
+ * before the first negative rule, summed in rule order. */
+int scn_terminal_pool(scn_ctx *ctx, const float *d_in, float *d_out,
+                      const int32_t *d_rules, int64_t count, int S, int C);
+/* dSigmoidSoftmax (SigmoidLayer.cu:160-177). */
+int scn_softmax_rows(scn_ctx *ctx, const float *d_in, float *d_out, int64_t M,
+                     int N);
+
+/* ---- per-kernel timing -------------------------------------------------- */
+/* HIP events recorded on the context's stream around every kernel of one
+ * family; off by default.  The reference only times whole dataset passes
+ * (SparseConvNetCUDA.cu:277-324). */
+enum {
+  SCN_K_GRID_BUILD = 0,
+  SCN_K_RULES = 1,
+  SCN_K_GATHER = 2,
+  SCN_K_NIN = 3,
+  SCN_K_MAXPOOL = 4,
+  SCN_K_TERMINAL = 5,
+  SCN_K_SOFTMAX = 6,
+  SCN_K_COUNT = 7
+};
+int scn_prof_enable(scn_ctx *ctx, int on);
+int scn_prof_reset(scn_ctx *ctx);
+/* synchronises, then returns accumulated milliseconds and number of calls */
+int scn_prof_read(scn_ctx *ctx, int family, double *ms, int64_t *calls);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,303 @@
+"""ctypes view of ``libscn_hip.so`` (the C ABI in ``include/scn_hip.h``).
+
+This module is plumbing for tests, the smoke check and the benchmark: it loads
+the in-tree HIP library, raises if it is missing (there is no CPU fallback) and
+wraps device buffers.  The product's host side is the C++ library in ``host/``.
+"""
+import ctypes as C
+import os
+import re
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(_HERE)
+LIB_PATH = os.path.join(_HERE, "libscn_hip.so")
+HEADER = os.path.join(ROOT, "include", "scn_hip.h")
+
+# ActivationFunction (reference types.h:11-20)
+NOSIGMOID, RELU, VLEAKYRELU, LEAKYRELU, TANH, SOFTMAX, PRELU, SIGMOID = range(8)
+FP32, BF16 = 0, 1
+K_GRID_BUILD, K_RULES, K_GATHER, K_NIN, K_MAXPOOL, K_TERMINAL, K_SOFTMAX = range(7)
+KERNEL_FAMILIES = ["grid_build", "rules", "gather", "nin", "maxpool", "terminal", "softmax"]
+
+
+class ScnError(RuntimeError):
+    pass
+
+
+def build(force=True):
+    """Compile the HIP library for gfx950 (works without a GPU)."""
+    args = ["make", "-C", os.path.join(_HERE, "csrc"), "-s", "-j8"]
+    if force:
+        args.append("-B")
+    subprocess.check_call(args)
+
+
+def declared_symbols():
+    """Names of every function the C header declares."""
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(scn_[a-z0-9_]+)\s*\(", text)))
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ScnError(
+            "libscn_hip.so is not built (run `python -c 'import __graft_entry__ as g; g.build()'`); "
+            "there is no CPU fallback for the sparse forward path")
+    L = C.CDLL(LIB_PATH)
+    vp, i32, i64, f32, sz = C.c_void_p, C.c_int32, C.c_int64, C.c_float, C.c_size_t
+    P = C.POINTER
+    sig = {
+        "scn_last_error": (C.c_char_p, []),
+        "scn_version": (C.c_char_p, []),
+        "scn_ctx_create": (C.c_int, [C.c_int, P(vp)]),
+        "scn_ctx_destroy": (C.c_int, [vp]),
+        "scn_ctx_stream": (vp, [vp]),
+        "scn_sync": (C.c_int, [vp]),
+        "scn_malloc": (C.c_int, [vp, sz, P(vp)]),
+        "scn_free": (C.c_int, [vp, vp]),
+        "scn_h2d": (C.c_int, [vp, vp, vp, sz]),
+        "scn_d2h": (C.c_int, [vp, vp, vp, sz]),
+        "scn_fill32": (C.c_int, [vp, vp, C.c_uint32, sz]),
+        "scn_grids_create": (C.c_int, [vp, P(vp)]),
+        "scn_grids_destroy": (C.c_int, [vp, vp]),
+        "scn_grids_build": (C.c_int, [vp, vp, C.c_int, C.c_int, C.c_int, vp, vp, vp, i64, vp, i32]),
+        "scn_grids_info": (C.c_int, [vp, P(C.c_int), P(C.c_int), P(C.c_int), P(i64), P(i32)]),
+        "scn_grids_download": (C.c_int, [vp, vp, vp, vp, vp, vp]),
+        "scn_grids_find": (C.c_int, [vp, vp, vp, vp, i64, vp]),
+        "scn_rules_square_plan": (C.c_int, [vp, vp, vp] + [C.c_int] * 5 + [P(i64)]),
+        "scn_rules_triangular_plan": (C.c_int, [vp, vp, vp] + [C.c_int] * 5 + [P(i64)]),
+        "scn_rules_terminal_plan": (C.c_int, [vp, vp, vp, P(i64)]),
+        "scn_rules_width": (C.c_int, [vp, P(i64)]),
+        "scn_rules_fill": (C.c_int, [vp, vp, vp, vp, i64]),
+        "scn_gather_rows": (C.c_int, [vp, vp, vp, vp, i64, C.c_int]),
+        "scn_nin_forward": (C.c_int, [vp] * 6 + [i64, C.c_int, C.c_int, f32, C.c_int, C.c_int]),
+        "scn_maxpool": (C.c_int, [vp, vp, vp, vp, i64, C.c_int, C.c_int, vp]),
+        "scn_terminal_pool": (C.c_int, [vp, vp, vp, vp, i64, C.c_int, C.c_int]),
+        "scn_softmax_rows": (C.c_int, [vp, vp, vp, i64, C.c_int]),
+        "scn_prof_enable": (C.c_int, [vp, C.c_int]),
+        "scn_prof_reset": (C.c_int, [vp]),
+        "scn_prof_read": (C.c_int, [vp, C.c_int, P(C.c_double), P(i64)]),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(L, name)
+        fn.restype = res
+        fn.argtypes = args
+    L._signatures = sig
+    _lib = L
+    return L
+
+
+def _check(rc):
+    if rc != 0:
+        raise ScnError("scn error %d: %s" % (rc, lib().scn_last_error().decode()))
+
+
+class DevArray:
+    """A typed device buffer allocated through the C ABI."""
+
+    def __init__(self, ctx, shape, dtype):
+        self.ctx = ctx
+        self.shape = tuple(int(s) for s in (shape if isinstance(shape, (tuple, list)) else (shape,)))
+        self.dtype = np.dtype(dtype)
+        self.size = int(np.prod(self.shape)) if self.shape else 1
+        self.nbytes = self.size * self.dtype.itemsize
+        p = C.c_void_p()
+        _check(lib().scn_malloc(ctx.h, max(self.nbytes, 16), C.byref(p)))
+        self.ptr = p.value
+
+    def free(self):
+        if getattr(self, "ptr", None):
+            lib().scn_free(self.ctx.h, self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+    def upload(self, a):
+        a = np.ascontiguousarray(a, dtype=self.dtype)
+        assert a.size == self.size, (a.shape, self.shape)
+        _check(lib().scn_h2d(self.ctx.h, self.ptr, a.ctypes.data_as(C.c_void_p), self.nbytes))
+        return self
+
+    def download(self):
+        out = np.empty(self.shape, self.dtype)
+        _check(lib().scn_d2h(self.ctx.h, out.ctypes.data_as(C.c_void_p), self.ptr, self.nbytes))
+        return out
+
+
+class Context:
+    def __init__(self, device=0):
+        h = C.c_void_p()
+        _check(lib().scn_ctx_create(device, C.byref(h)))
+        self.h = h.value
+
+    def close(self):
+        if getattr(self, "h", None):
+            lib().scn_ctx_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def sync(self):
+        _check(lib().scn_sync(self.h))
+
+    def stream(self):
+        return lib().scn_ctx_stream(self.h)
+
+    def array(self, a, dtype=None):
+        a = np.ascontiguousarray(a, dtype=dtype)
+        return DevArray(self, a.shape, a.dtype).upload(a)
+
+    def empty(self, shape, dtype):
+        return DevArray(self, shape, dtype)
+
+    # ---- profiling
+    def prof_enable(self, on=True):
+        _check(lib().scn_prof_enable(self.h, int(on)))
+
+    def prof_reset(self):
+        _check(lib().scn_prof_reset(self.h))
+
+    def prof_read(self):
+        out = {}
+        for i, name in enumerate(KERNEL_FAMILIES):
+            ms, calls = C.c_double(), C.c_int64()
+            _check(lib().scn_prof_read(self.h, i, C.byref(ms), C.byref(calls)))
+            out[name] = (ms.value, calls.value)
+        return out
+
+    # ---- feature kernels
+    def gather_rows(self, d_in, d_out, d_rules, count, nIn):
+        _check(lib().scn_gather_rows(self.h, d_in.ptr, d_out.ptr, d_rules.ptr, count, nIn))
+
+    def nin_forward(self, d_A, d_W, d_B, d_prelu, d_out, M, K, N, p=1.0, act=RELU, precision=FP32):
+        _check(lib().scn_nin_forward(self.h, d_A.ptr, d_W.ptr, d_B.ptr,
+                                     d_prelu.ptr if d_prelu is not None else None,
+                                     d_out.ptr, M, K, N, p, act, precision))
+
+    def maxpool(self, d_in, d_out, d_rules, nOutSites, ps, Cn, d_choice):
+        _check(lib().scn_maxpool(self.h, d_in.ptr, d_out.ptr, d_rules.ptr, nOutSites, ps, Cn, d_choice.ptr))
+
+    def terminal_pool(self, d_in, d_out, d_rules, count, S, Cn):
+        _check(lib().scn_terminal_pool(self.h, d_in.ptr, d_out.ptr, d_rules.ptr, count, S, Cn))
+
+    def softmax_rows(self, d_in, d_out, M, N):
+        _check(lib().scn_softmax_rows(self.h, d_in.ptr, d_out.ptr, M, N))
+
+
+class Grids:
+    """Device-resident SparseGrids of one depth of a batch."""
+
+    def __init__(self, ctx):
+        self.ctx = ctx
+        h = C.c_void_p()
+        _check(lib().scn_grids_create(ctx.h, C.byref(h)))
+        self.h = h.value
+
+    def close(self):
+        if getattr(self, "h", None) and getattr(self.ctx, "h", None):
+            lib().scn_grids_destroy(self.ctx.h, self.h)
+        self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def build(self, batch, dimension, spatialSize, sample, key, row, background, nSpatialSites):
+        """Host arrays in, as Picture::codifyInputData leaves them."""
+        c = self.ctx
+        self._keep = (c.array(sample, np.int32), c.array(key, np.int64), c.array(row, np.int32),
+                      c.array(np.asarray(background, np.int32) if batch else np.zeros(1, np.int32), np.int32))
+        self.build_device(batch, dimension, spatialSize, *self._keep, len(np.asarray(key)), nSpatialSites)
+
+    def build_device(self, batch, dimension, spatialSize, d_sample, d_key, d_row, d_bg, n, nSpatialSites):
+        _check(lib().scn_grids_build(self.ctx.h, self.h, batch, dimension, spatialSize,
+                                     d_sample.ptr, d_key.ptr, d_row.ptr, n, d_bg.ptr, nSpatialSites))
+
+    def info(self):
+        b, d, n = C.c_int(), C.c_int(), C.c_int()
+        na, ns = C.c_int64(), C.c_int32()
+        _check(lib().scn_grids_info(self.h, C.byref(b), C.byref(d), C.byref(n), C.byref(na), C.byref(ns)))
+        return dict(batch=b.value, dimension=d.value, spatialSize=n.value, nActive=na.value, nSpatialSites=ns.value)
+
+    def download(self):
+        info = self.info()
+        n, b = info["nActive"], info["batch"]
+        s = np.empty(n, np.int32)
+        k = np.empty(n, np.int64)
+        r = np.empty(n, np.int32)
+        bg = np.empty(b, np.int32)
+        vp = lambda a: a.ctypes.data_as(C.c_void_p)
+        _check(lib().scn_grids_download(self.ctx.h, self.h, vp(s), vp(k), vp(r), vp(bg)))
+        return s, k, r, bg
+
+    def find(self, sample, key):
+        c = self.ctx
+        ds, dk = c.array(sample, np.int32), c.array(key, np.int64)
+        out = c.empty(len(sample), np.int32)
+        _check(lib().scn_grids_find(c.h, self.h, ds.ptr, dk.ptr, len(sample), out.ptr))
+        return out.download()
+
+    # ---- rule books: plan on `self` as the input, returns (out grids, nOutSites)
+    def plan_square(self, out, nIn, nOut, size, stride, minActive=1):
+        n = C.c_int64()
+        _check(lib().scn_rules_square_plan(self.ctx.h, self.h, out.h, nIn, nOut, size, stride, minActive, C.byref(n)))
+        return n.value
+
+    def plan_triangular(self, out, nIn, nOut, size, stride, minActive=1):
+        n = C.c_int64()
+        _check(lib().scn_rules_triangular_plan(self.ctx.h, self.h, out.h, nIn, nOut, size, stride, minActive, C.byref(n)))
+        return n.value
+
+    def plan_terminal(self, out):
+        S = C.c_int64()
+        _check(lib().scn_rules_terminal_plan(self.ctx.h, self.h, out.h, C.byref(S)))
+        return S.value
+
+    def rules_width(self):
+        w = C.c_int64()
+        _check(lib().scn_rules_width(self.h, C.byref(w)))
+        return w.value
+
+    def fill(self, out, d_rules, capacity=None):
+        cap = d_rules.size if capacity is None else capacity
+        _check(lib().scn_rules_fill(self.ctx.h, self.h, out.h, d_rules.ptr, cap))
+
+
+def rules_square(ctx, grids, nIn, nOut, size, stride, minActive=1, triangular=False):
+    """plan + fill; returns (out grids, device rules, nOutSites, width)."""
+    out = Grids(ctx)
+    plan = grids.plan_triangular if triangular else grids.plan_square
+    n = plan(out, nIn, nOut, size, stride, minActive)
+    w = out.rules_width()
+    rules = ctx.empty(max(n * w, 1), np.int32)
+    grids.fill(out, rules, n * w)
+    return out, rules, n, w
+
+
+def rules_terminal(ctx, grids):
+    out = Grids(ctx)
+    S = grids.plan_terminal(out)
+    batch = grids.info()["batch"]
+    rules = ctx.empty(max(batch * S, 1), np.int32)
+    grids.fill(out, rules, batch * S)
+    return out, rules, S

@@ -1,0 +1,190 @@
+// Context, error reporting, raw device memory and per-kernel timing.
+#include "scn_common.h"
+#include <stdarg.h>
+#include <string.h>
+
+static thread_local char g_err[512] = "";
+
+void scn_set_error(const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+extern "C" const char *scn_last_error(void) { return g_err; }
+extern "C" const char *scn_version(void) { return "scn_hip 0.1 (gfx950)"; }
+
+extern "C" int scn_ctx_create(int device, scn_ctx **out) {
+  SCN_REQUIRE(out != nullptr, SCN_ERR_ARG, "scn_ctx_create: null out pointer");
+  int n = 0;
+  SCN_HIP_CHECK(hipGetDeviceCount(&n));
+  if (device < 0)
+    device = 0;
+  SCN_REQUIRE(device < n, SCN_ERR_ARG, "scn_ctx_create: device %d of %d",
+              device, n);
+  SCN_HIP_CHECK(hipSetDevice(device));
+  scn_ctx *c = new scn_ctx();
+  c->device = device;
+  c->prof = false;
+  memset(c->profMs, 0, sizeof(c->profMs));
+  memset(c->profCalls, 0, sizeof(c->profCalls));
+  hipDeviceProp_t prop;
+  SCN_HIP_CHECK(hipGetDeviceProperties(&prop, device));
+  c->numCU = prop.multiProcessorCount;
+  SCN_HIP_CHECK(hipStreamCreate(&c->stream)); // default priority
+  SCN_HIP_CHECK(hipHostMalloc((void **)&c->h_pinned, 16 * sizeof(int64_t)));
+  SCN_HIP_CHECK(hipMalloc((void **)&c->d_scalars, 16 * sizeof(int64_t)));
+  SCN_HIP_CHECK(hipMemset(c->d_scalars, 0, 16 * sizeof(int64_t)));
+  *out = c;
+  return SCN_OK;
+}
+
+extern "C" int scn_ctx_destroy(scn_ctx *c) {
+  if (!c)
+    return SCN_OK;
+  (void)hipStreamSynchronize(c->stream);
+  for (auto &s : c->spans) {
+    (void)hipEventDestroy(s.a);
+    (void)hipEventDestroy(s.b);
+  }
+  for (auto e : c->freeEvents)
+    (void)hipEventDestroy(e);
+  (void)hipFree(c->d_scalars);
+  (void)hipHostFree(c->h_pinned);
+  (void)hipStreamDestroy(c->stream);
+  delete c;
+  return SCN_OK;
+}
+
+extern "C" void *scn_ctx_stream(scn_ctx *c) { return (void *)c->stream; }
+
+extern "C" int scn_sync(scn_ctx *c) {
+  SCN_HIP_CHECK(hipStreamSynchronize(c->stream));
+  return SCN_OK;
+}
+
+extern "C" int scn_malloc(scn_ctx *c, size_t bytes, void **d_ptr) {
+  SCN_REQUIRE(c && d_ptr, SCN_ERR_ARG, "scn_malloc: null argument");
+  *d_ptr = nullptr;
+  if (bytes == 0)
+    bytes = 16;
+  SCN_HIP_CHECK(hipMalloc(d_ptr, bytes));
+  return SCN_OK;
+}
+
+extern "C" int scn_free(scn_ctx *c, void *d_ptr) {
+  (void)c;
+  if (d_ptr)
+    SCN_HIP_CHECK(hipFree(d_ptr));
+  return SCN_OK;
+}
+
+extern "C" int scn_h2d(scn_ctx *c, void *d_dst, const void *h_src,
+                       size_t bytes) {
+  if (bytes == 0)
+    return SCN_OK;
+  SCN_HIP_CHECK(
+      hipMemcpyAsync(d_dst, h_src, bytes, hipMemcpyHostToDevice, c->stream));
+  SCN_HIP_CHECK(hipStreamSynchronize(c->stream));
+  return SCN_OK;
+}
+
+extern "C" int scn_d2h(scn_ctx *c, void *h_dst, const void *d_src,
+                       size_t bytes) {
+  if (bytes == 0)
+    return SCN_OK;
+  SCN_HIP_CHECK(
+      hipMemcpyAsync(h_dst, d_src, bytes, hipMemcpyDeviceToHost, c->stream));
+  SCN_HIP_CHECK(hipStreamSynchronize(c->stream));
+  return SCN_OK;
+}
+
+__global__ void k_fill32(uint32_t *dst, uint32_t w, size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  size_t step = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += step)
+    dst[i] = w;
+}
+
+extern "C" int scn_fill32(scn_ctx *c, void *d_dst, uint32_t word,
+                          size_t nWords) {
+  if (nWords == 0)
+    return SCN_OK;
+  int blocks = (int)((nWords + 255) / 256);
+  if (blocks > 65536)
+    blocks = 65536;
+  hipLaunchKernelGGL(k_fill32, dim3(blocks), dim3(256), 0, c->stream,
+                     (uint32_t *)d_dst, word, nWords);
+  SCN_HIP_CHECK(hipGetLastError());
+  return SCN_OK;
+}
+
+// ---- profiling ---------------------------------------------------------
+
+static hipEvent_t take_event(scn_ctx *c) {
+  if (!c->freeEvents.empty()) {
+    hipEvent_t e = c->freeEvents.back();
+    c->freeEvents.pop_back();
+    return e;
+  }
+  hipEvent_t e;
+  (void)hipEventCreate(&e);
+  return e;
+}
+
+ProfScope::ProfScope(scn_ctx *c, int family) : ctx(c), idx(-1) {
+  if (!c->prof)
+    return;
+  ProfSpan s;
+  s.family = family;
+  s.a = take_event(c);
+  s.b = take_event(c);
+  (void)hipEventRecord(s.a, c->stream);
+  c->spans.push_back(s);
+  idx = (int)c->spans.size() - 1;
+}
+
+ProfScope::~ProfScope() {
+  if (idx >= 0)
+    (void)hipEventRecord(ctx->spans[idx].b, ctx->stream);
+}
+
+static void drain_spans(scn_ctx *c) {
+  (void)hipStreamSynchronize(c->stream);
+  for (auto &s : c->spans) {
+    float ms = 0.f;
+    if (hipEventElapsedTime(&ms, s.a, s.b) == hipSuccess) {
+      c->profMs[s.family] += ms;
+      c->profCalls[s.family] += 1;
+    }
+    c->freeEvents.push_back(s.a);
+    c->freeEvents.push_back(s.b);
+  }
+  c->spans.clear();
+}
+
+extern "C" int scn_prof_enable(scn_ctx *c, int on) {
+  drain_spans(c);
+  c->prof = on != 0;
+  return SCN_OK;
+}
+
+extern "C" int scn_prof_reset(scn_ctx *c) {
+  drain_spans(c);
+  memset(c->profMs, 0, sizeof(c->profMs));
+  memset(c->profCalls, 0, sizeof(c->profCalls));
+  return SCN_OK;
+}
+
+extern "C" int scn_prof_read(scn_ctx *c, int family, double *ms,
+                             int64_t *calls) {
+  SCN_REQUIRE(family >= 0 && family < SCN_K_COUNT, SCN_ERR_ARG,
+              "scn_prof_read: family %d", family);
+  drain_spans(c);
+  if (ms)
+    *ms = c->profMs[family];
+  if (calls)
+    *calls = c->profCalls[family];
+  return SCN_OK;
+}

@@ -1,0 +1,1006 @@
+// Sparse grids in HBM and rule-book construction.
+//
+// A batch of SparseGrids (SparseGrid.h:26-37) is kept as
+//   * an open-addressing hash table, linear probing, 16-byte slots
+//     {int64 packed coordinate, int32 row}, load factor <= 1/2;
+//     packed coordinate = sample * spatialSize^d + key;
+//   * an occupancy bit mask over the packed coordinates, with an exclusive
+//     popcount prefix per 64-bit word, so that the position of a site in map
+//     iteration order (sample, then ascending key) is prefix + popcount;
+//   * the list of entries (packed coordinate, row) in no particular order.
+//
+// Rule books (Regions.cu gridRules*) number output sites in first-touch order
+// while the input map is iterated in ascending key.  An output site is first
+// touched by the active input with the smallest key inside its window (its
+// "owner"), and one input touches its outputs in ascending output key.  So
+//   row(o) = #outputs owned by inputs that precede owner(o) in iteration order
+//          + position of o among owner(o)'s outputs
+//          + #background rows appended for earlier samples,
+// which needs no sort: count owned outputs per input, scatter the counts to
+// iteration order through the rank, prefix-sum, emit.
+#include "scn_common.h"
+
+struct __align__(16) Slot {
+  long long key;
+  int row;
+  int pad;
+};
+#define SLOT_EMPTY (-1LL)
+
+enum { MODE_SQ_NOMIN = 0, MODE_SQ_MIN, MODE_SQ_VALID, MODE_TRI_NOMIN, MODE_TRI_MIN };
+enum { PLAN_NONE = 0, PLAN_REGIONS = 1, PLAN_TERMINAL = 2 };
+
+struct Geom {
+  int d;
+  int nIn, nOut, size, stride, minActive, mode;
+  long long volIn, volOut;
+  int width; // rule-row width: size^d or triangleSize(size, d)
+  int cube;  // size^d
+};
+
+struct GridView {
+  Slot *table;
+  unsigned shift, mask;
+  unsigned long long *bits;
+  const unsigned *prefix;
+  const int *bg;
+  long long vol;
+  int n, d, batch;
+};
+
+struct scn_grids {
+  int batch = 0, d = 0, n = 0;
+  long long vol = 0;
+  long long nActive = 0;
+  int nSites = 0;
+  unsigned log2cap = 0;
+  size_t nWords = 0;
+  bool rankValid = false;
+  DevBuf<Slot> table;
+  DevBuf<unsigned long long> bits;
+  DevBuf<unsigned> prefix;
+  DevBuf<long long> ekey;
+  DevBuf<int> erow;
+  DevBuf<int> bg;
+  DevBuf<unsigned> scanTmp;
+  // state of the plan that produced this object
+  int planKind = PLAN_NONE;
+  const scn_grids *planIn = nullptr;
+  Geom geom;
+  long long termS = 0;
+  DevBuf<long long> siteKey; // per output row: packed key, or -1 - sample for a background row
+  DevBuf<unsigned> cnt, base;
+  DevBuf<int> bgBefore;
+  DevBuf<unsigned> sampleStart;
+  DevBuf<int> invOrd;
+  // scratch for download
+  DevBuf<int> dlSample, dlRow;
+  DevBuf<long long> dlKey;
+};
+
+// ---------------------------------------------------------------- device
+
+__device__ __forceinline__ unsigned hash_slot(long long p, unsigned shift) {
+  return (unsigned)(((unsigned long long)p * 0x9E3779B97F4A7C15ull) >> shift);
+}
+
+__device__ __forceinline__ void hash_insert(Slot *t, unsigned shift,
+                                            unsigned mask, long long p,
+                                            int row) {
+  unsigned s = hash_slot(p, shift);
+  for (;;) {
+    unsigned long long prev =
+        atomicCAS((unsigned long long *)&t[s].key,
+                  (unsigned long long)SLOT_EMPTY, (unsigned long long)p);
+    if (prev == (unsigned long long)SLOT_EMPTY ||
+        prev == (unsigned long long)p) {
+      t[s].row = row;
+      return;
+    }
+    s = (s + 1) & mask;
+  }
+}
+
+__device__ __forceinline__ int hash_find(const Slot *t, unsigned shift,
+                                         unsigned mask, long long p) {
+  unsigned s = hash_slot(p, shift);
+  for (;;) {
+    const int4 v = *reinterpret_cast<const int4 *>(&t[s]); // one 128-bit load
+    long long k = ((long long)v.y << 32) | (unsigned)v.x;
+    if (k == p)
+      return v.z;
+    if (k == SLOT_EMPTY)
+      return -1;
+    s = (s + 1) & mask;
+  }
+}
+
+// `len` (1..32) mask bits starting at bit position p
+__device__ __forceinline__ unsigned get_bits(const unsigned long long *bits,
+                                             long long p, int len) {
+  long long w = p >> 6;
+  int sh = (int)(p & 63);
+  unsigned long long lo = bits[w] >> sh;
+  if (sh + len > 64)
+    lo |= bits[w + 1] << (64 - sh);
+  unsigned m = (len >= 32) ? 0xFFFFFFFFu : ((1u << len) - 1u);
+  return (unsigned)lo & m;
+}
+
+__device__ __forceinline__ unsigned rank_of(const GridView &g, long long p) {
+  long long w = p >> 6;
+  int sh = (int)(p & 63);
+  unsigned long long below = sh ? (g.bits[w] & ((1ull << sh) - 1ull)) : 0ull;
+  return g.prefix[w] + (unsigned)__popcll(below);
+}
+
+__device__ __forceinline__ int sq_outputL(int size, int stride, int i) {
+  int v = (i - size + stride) / stride; // truncation toward zero, as in C
+  return v > 0 ? v : 0;
+}
+__device__ __forceinline__ int sq_outputR(int stride, int nOut, int i) {
+  int v = i / stride + 1;
+  return v < nOut ? v : nOut;
+}
+
+template <int D>
+__device__ __forceinline__ void decode_key(long long key, int n, int *c) {
+#pragma unroll
+  for (int a = D - 1; a >= 0; --a) {
+    c[a] = (int)(key % n);
+    key /= n;
+  }
+}
+template <int D>
+__device__ __forceinline__ long long encode_key(const int *c, int n) {
+  long long k = 0;
+#pragma unroll
+  for (int a = 0; a < D; ++a)
+    k = k * n + c[a];
+  return k;
+}
+
+// Is any site of the window with origin w active at a window offset that
+// precedes offset a (row-major)?  Square window of side `size`.
+template <int D>
+__device__ __forceinline__ bool any_before(const unsigned long long *bits,
+                                           long long sampleBase, int nIn,
+                                           int size, const int *w,
+                                           const int *a) {
+  if (D == 1) {
+    return a[0] > 0 && get_bits(bits, sampleBase + w[0], a[0]) != 0;
+  } else if (D == 2) {
+    for (int q0 = 0; q0 < a[0]; ++q0)
+      if (get_bits(bits, sampleBase + (long long)(w[0] + q0) * nIn + w[1], size))
+        return true;
+    return a[1] > 0 &&
+           get_bits(bits, sampleBase + (long long)(w[0] + a[0]) * nIn + w[1],
+                    a[1]) != 0;
+  } else {
+    for (int q0 = 0; q0 <= a[0]; ++q0) {
+      int q1max = (q0 < a[0]) ? size : a[1];
+      for (int q1 = 0; q1 < q1max; ++q1)
+        if (get_bits(bits,
+                     sampleBase +
+                         ((long long)(w[0] + q0) * nIn + (w[1] + q1)) * nIn +
+                         w[2],
+                     size))
+          return true;
+    }
+    return a[2] > 0 &&
+           get_bits(bits,
+                    sampleBase +
+                        ((long long)(w[0] + a[0]) * nIn + (w[1] + a[1])) * nIn +
+                        w[2],
+                    a[2]) != 0;
+  }
+}
+
+// number of active sites in the window; TRI counts only offsets with
+// coordinate sum < size
+template <int D, bool TRI>
+__device__ __forceinline__ int count_active(const unsigned long long *bits,
+                                            long long sampleBase, int nIn,
+                                            int size, const int *w) {
+  int c = 0;
+  if (D == 1) {
+    c = __popc(get_bits(bits, sampleBase + w[0], size));
+  } else if (D == 2) {
+    for (int q0 = 0; q0 < size; ++q0) {
+      int len = TRI ? size - q0 : size;
+      c += __popc(get_bits(bits, sampleBase + (long long)(w[0] + q0) * nIn + w[1], len));
+    }
+  } else {
+    for (int q0 = 0; q0 < size; ++q0) {
+      int q1n = TRI ? size - q0 : size;
+      for (int q1 = 0; q1 < q1n; ++q1) {
+        int len = TRI ? size - q0 - q1 : size;
+        c += __popc(get_bits(
+            bits,
+            sampleBase + ((long long)(w[0] + q0) * nIn + (w[1] + q1)) * nIn + w[2],
+            len));
+      }
+    }
+  }
+  return c;
+}
+
+// Visits, in ascending output key, the output sites owned by the input site
+// with coordinates i of sample b; f(outKey) is called for each.
+template <int D, typename F>
+__device__ __forceinline__ void for_each_owned(const GridView &in,
+                                               const Geom &g, int b,
+                                               const int *i, F f) {
+  int lo[D], hi[D];
+  const long long sampleBase = (long long)b * g.volIn;
+  if (g.mode == MODE_SQ_VALID) {
+    // Regions.cu:693-697: output (i0-1, i1-1) when 1 <= i <= nOut on each axis
+#pragma unroll
+    for (int a = 0; a < D; ++a) {
+      if (i[a] < 1 || i[a] > g.nOut)
+        return;
+      lo[a] = i[a] - 1;
+      hi[a] = i[a];
+    }
+  } else {
+#pragma unroll
+    for (int a = 0; a < D; ++a) {
+      lo[a] = sq_outputL(g.size, g.stride, i[a]);
+      hi[a] = sq_outputR(g.stride, g.nOut, i[a]);
+      if (lo[a] >= hi[a])
+        return;
+    }
+  }
+  const bool tri = g.mode == MODE_TRI_NOMIN || g.mode == MODE_TRI_MIN;
+  int j[D];
+#pragma unroll
+  for (int a = 0; a < D; ++a)
+    j[a] = lo[a];
+  for (;;) {
+    bool consider = true;
+    if (tri) {
+      int sum = 0;
+#pragma unroll
+      for (int a = 0; a < D; ++a)
+        sum += j[a];
+      consider = sum < g.nOut; // Regions.cu:874,900
+    }
+    if (consider) {
+      bool own = true;
+      if (g.mode != MODE_SQ_VALID) {
+        int w[D], off[D];
+#pragma unroll
+        for (int a = 0; a < D; ++a) {
+          w[a] = j[a] * g.stride;
+          off[a] = i[a] - w[a];
+        }
+        own = !any_before<D>(in.bits, sampleBase, g.nIn, g.size, w, off);
+        if (own && g.mode == MODE_SQ_MIN)
+          own = count_active<D, false>(in.bits, sampleBase, g.nIn, g.size, w) >=
+                g.minActive;
+        if (own && g.mode == MODE_TRI_MIN)
+          own = count_active<D, true>(in.bits, sampleBase, g.nIn, g.size, w) >=
+                g.minActive;
+      }
+      if (own)
+        f(encode_key<D>(j, g.nOut));
+    }
+    // odometer, last axis fastest
+    int a = D - 1;
+    for (; a >= 0; --a) {
+      if (++j[a] < hi[a])
+        break;
+      j[a] = lo[a];
+    }
+    if (a < 0)
+      break;
+  }
+}
+
+__global__ void k_grid_build(GridView g, const int *sample,
+                             const long long *key, const int *row, long long n,
+                             long long *ekey, int *erow,
+                             unsigned long long *badSites) {
+  long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= n)
+    return;
+  const int b = sample[e];
+  const long long k = key[e];
+  if (b < 0 || b >= g.batch || k < 0 || k >= g.vol) {
+    // outside the field: counted and reported by the next call that
+    // synchronises; stored on the sample-0 origin so every list stays valid
+    atomicAdd(badSites, 1ull);
+    ekey[e] = 0;
+    erow[e] = row[e];
+    return;
+  }
+  long long p = (long long)b * g.vol + k;
+  int r = row[e];
+  hash_insert(g.table, g.shift, g.mask, p, r);
+  atomicOr(&g.bits[p >> 6], 1ull << (p & 63));
+  ekey[e] = p;
+  erow[e] = r;
+}
+
+// pass 1: number of output sites owned by each input, stored at the input's
+// position in iteration order
+template <int D>
+__global__ void k_plan_count(GridView in, Geom g, const long long *ekey,
+                             long long nEntries, unsigned *cntByRank) {
+  long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= nEntries)
+    return;
+  long long p = ekey[e];
+  int b = (int)(p / g.volIn);
+  int i[D];
+  decode_key<D>(p - (long long)b * g.volIn, g.nIn, i);
+  unsigned c = 0;
+  for_each_owned<D>(in, g, b, i, [&](long long) { ++c; });
+  cntByRank[rank_of(in, p)] = c;
+}
+
+// per sample: does it need a background row, and how many were appended
+// before it.  One block.
+__global__ void k_plan_samples(GridView in, const unsigned *base,
+                               long long nEntries, long long fullSize,
+                               int *outBg, int *bgBefore,
+                               unsigned *sampleStart, long long *scalars) {
+  __shared__ int lds[1024];
+  __shared__ int carry;
+  const int t = threadIdx.x;
+  if (t == 0)
+    carry = 0;
+  __syncthreads();
+  for (int b0 = 0; b0 < in.batch; b0 += 1024) {
+    int b = b0 + t;
+    int notFull = 0;
+    unsigned re = 0;
+    if (b < in.batch) {
+      unsigned rs = rank_of(in, (long long)b * in.vol);
+      re = rank_of(in, (long long)(b + 1) * in.vol);
+      sampleStart[b] = rs;
+      long long oc = (long long)base[re] - (long long)base[rs];
+      notFull = oc < fullSize;
+    }
+    lds[t] = notFull;
+    __syncthreads();
+    for (int off = 1; off < 1024; off <<= 1) {
+      int add = (t >= off) ? lds[t - off] : 0;
+      __syncthreads();
+      lds[t] += add;
+      __syncthreads();
+    }
+    int excl = lds[t] - notFull + carry;
+    if (b < in.batch) {
+      bgBefore[b] = excl;
+      outBg[b] = notFull ? (int)base[re] + excl : -1;
+    }
+    __syncthreads();
+    if (t == 1023)
+      carry += lds[1023];
+    __syncthreads();
+  }
+  if (t == 0) {
+    scalars[0] = (long long)base[nEntries] + carry; // nOutputSpatialSites
+    scalars[1] = (long long)base[nEntries];         // active output sites
+  }
+}
+
+// pass 2: emit the owned outputs
+template <int D>
+__global__ void k_plan_emit(GridView in, GridView out, Geom g,
+                            const long long *ekey, long long nEntries,
+                            const unsigned *base, const int *bgBefore,
+                            const int *outBg, long long *okey, int *orow,
+                            long long *siteKey) {
+  long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e < in.batch) { // background rows
+    int r = outBg[e];
+    if (r >= 0)
+      siteKey[r] = -1 - e;
+  }
+  if (e >= nEntries)
+    return;
+  long long p = ekey[e];
+  int b = (int)(p / g.volIn);
+  int i[D];
+  decode_key<D>(p - (long long)b * g.volIn, g.nIn, i);
+  unsigned idx = base[rank_of(in, p)];
+  const int shiftRows = bgBefore[b];
+  for_each_owned<D>(in, g, b, i, [&](long long outKey) {
+    long long po = (long long)b * g.volOut + outKey;
+    int row = (int)idx + shiftRows;
+    hash_insert(out.table, out.shift, out.mask, po, row);
+    atomicOr(&out.bits[po >> 6], 1ull << (po & 63));
+    okey[idx] = po;
+    orow[idx] = row;
+    siteKey[row] = po;
+    ++idx;
+  });
+}
+
+// inverse of RegularTriangularRegions::ord (Regions.cu:810-826)
+__global__ void k_tri_table(int size, int d, int *invOrd) {
+  if (blockIdx.x != 0 || threadIdx.x != 0)
+    return;
+  int cube = 1;
+  for (int a = 0; a < d; ++a)
+    cube *= size;
+  int S = 0;
+  for (int i = 0; i < cube; ++i) {
+    int j = i, J = 0;
+    while (j > 0) {
+      J += j % size;
+      j /= size;
+    }
+    if (J < size)
+      invOrd[S++] = i;
+  }
+}
+
+// one thread per rule: rules[row * width + q]
+template <int D>
+__global__ void k_rules_fill(GridView in, Geom g, const long long *siteKey,
+                             long long nSites, const int *invOrd, int *rules) {
+  long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  long long total = nSites * g.width;
+  if (idx >= total)
+    return;
+  long long r = idx / g.width;
+  int q = (int)(idx - r * g.width);
+  long long sk = siteKey[r];
+  if (sk < 0) { // all-background row (Regions.cu:647-652)
+    rules[idx] = in.bg[-1 - sk];
+    return;
+  }
+  int b = (int)(sk / g.volOut);
+  int j[D], c[D];
+  decode_key<D>(sk - (long long)b * g.volOut, g.nOut, j);
+  int cubeOff = invOrd ? invOrd[q] : q;
+#pragma unroll
+  for (int a = D - 1; a >= 0; --a) {
+    c[a] = j[a] * g.stride + cubeOff % g.size;
+    cubeOff /= g.size;
+  }
+  long long p = (long long)b * g.volIn + encode_key<D>(c, g.nIn);
+  int val;
+  if ((in.bits[p >> 6] >> (p & 63)) & 1ull)
+    val = hash_find(in.table, in.shift, in.mask, p);
+  else
+    val = in.bg[b];
+  rules[idx] = val;
+}
+
+// terminal pooling: sample sizes and their maximum.  One block.
+__global__ void k_terminal_plan(GridView in, unsigned *sampleStart,
+                                long long *scalars) {
+  __shared__ long long lds[1024];
+  const int t = threadIdx.x;
+  long long mx = 1; // TerminalPoolingLayer.cu:90
+  for (int b = t; b < in.batch; b += 1024) {
+    unsigned rs = rank_of(in, (long long)b * in.vol);
+    unsigned re = rank_of(in, (long long)(b + 1) * in.vol);
+    sampleStart[b] = rs;
+    if (b == in.batch - 1)
+      sampleStart[in.batch] = re;
+    long long c = (long long)re - rs;
+    mx = c > mx ? c : mx;
+  }
+  lds[t] = mx;
+  __syncthreads();
+  for (int off = 512; off > 0; off >>= 1) {
+    if (t < off && lds[t + off] > lds[t])
+      lds[t] = lds[t + off];
+    __syncthreads();
+  }
+  if (t == 0)
+    scalars[0] = lds[0];
+}
+
+// out grid of the terminal layer: key 0 of sample b -> row b
+__global__ void k_terminal_out(GridView out, long long *okey, int *orow,
+                               int *outBg) {
+  int b = blockIdx.x * blockDim.x + threadIdx.x;
+  if (b >= out.batch)
+    return;
+  long long p = (long long)b * out.vol;
+  hash_insert(out.table, out.shift, out.mask, p, b);
+  atomicOr(&out.bits[p >> 6], 1ull << (p & 63));
+  okey[b] = p;
+  orow[b] = b;
+  outBg[b] = -1;
+}
+
+__global__ void k_terminal_init(GridView in, const unsigned *sampleStart,
+                                long long S, int *rules) {
+  long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long long)in.batch * S)
+    return;
+  int b = (int)(idx / S);
+  long long s = idx - (long long)b * S;
+  int v = -1;
+  // a sample without active sites pools its background row
+  // (TerminalPoolingLayer.cu:12-13)
+  if (s == 0 && sampleStart[b + 1] == sampleStart[b])
+    v = in.bg[b];
+  rules[idx] = v;
+}
+
+__global__ void k_terminal_scatter(GridView in, const long long *ekey,
+                                   const int *erow, long long nEntries,
+                                   const unsigned *sampleStart, long long S,
+                                   int *rules) {
+  long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= nEntries)
+    return;
+  long long p = ekey[e];
+  int b = (int)(p / in.vol);
+  unsigned r = rank_of(in, p) - sampleStart[b];
+  rules[(long long)b * S + r] = erow[e];
+}
+
+__global__ void k_download(GridView g, const long long *ekey, const int *erow,
+                           long long n, int *sample, long long *key, int *row) {
+  long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= n)
+    return;
+  long long p = ekey[e];
+  unsigned r = rank_of(g, p);
+  int b = (int)(p / g.vol);
+  sample[r] = b;
+  key[r] = p - (long long)b * g.vol;
+  row[r] = erow[e];
+}
+
+__global__ void k_find(GridView g, const int *sample, const long long *key,
+                       long long n, int *row) {
+  long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= n)
+    return;
+  long long k = key[e];
+  int b = sample[e];
+  int r = -1;
+  if (b >= 0 && b < g.batch && k >= 0 && k < g.vol)
+    r = hash_find(g.table, g.shift, g.mask, (long long)b * g.vol + k);
+  row[e] = r;
+}
+
+// ------------------------------------------------------------------ host
+
+static GridView view_of(const scn_grids *g) {
+  GridView v;
+  v.table = g->table.p;
+  v.shift = 64 - g->log2cap;
+  v.mask = (1u << g->log2cap) - 1u;
+  v.bits = g->bits.p;
+  v.prefix = g->prefix.p;
+  v.bg = g->bg.p;
+  v.vol = g->vol;
+  v.n = g->n;
+  v.d = g->d;
+  v.batch = g->batch;
+  return v;
+}
+
+static long long ipow_ll(long long b, int e) {
+  long long r = 1;
+  for (int i = 0; i < e; ++i)
+    r *= b;
+  return r;
+}
+
+// (re)shape a grids object for `batch` samples of an n^d field holding up to
+// nActive sites; clears the table and the mask
+static int grids_prepare(scn_ctx *ctx, scn_grids *g, int batch, int d, int n,
+                         long long nActive) {
+  SCN_REQUIRE(batch >= 0 && d >= 1 && d <= 3 && n >= 1, SCN_ERR_ARG,
+              "grids: batch %d dimension %d spatialSize %d (dimension must be 1..3)",
+              batch, d, n);
+  long long vol = ipow_ll(n, d);
+  SCN_REQUIRE((double)vol * (double)(batch > 0 ? batch : 1) < 6.0e10,
+              SCN_ERR_CAPACITY,
+              "grids: %d samples of %lld sites exceed the occupancy-mask limit",
+              batch, vol);
+  g->batch = batch;
+  g->d = d;
+  g->n = n;
+  g->vol = vol;
+  g->nActive = nActive;
+  g->rankValid = false;
+  g->planKind = PLAN_NONE;
+  g->planIn = nullptr;
+  unsigned lg = 6;
+  while ((1ll << lg) < 2 * nActive)
+    ++lg;
+  SCN_REQUIRE(lg <= 31, SCN_ERR_CAPACITY, "grids: %lld active sites", nActive);
+  g->log2cap = lg;
+  size_t cap = (size_t)1 << lg;
+  g->nWords = (size_t)(((long long)batch * vol + 63) / 64);
+  SCN_TRY(g->table.reserve(cap));
+  SCN_TRY(g->bits.reserve(g->nWords + 2));
+  SCN_TRY(g->prefix.reserve(g->nWords + 2));
+  SCN_TRY(g->ekey.reserve((size_t)nActive + 1));
+  SCN_TRY(g->erow.reserve((size_t)nActive + 1));
+  SCN_TRY(g->bg.reserve((size_t)batch + 1));
+  SCN_TRY(scn_fill32(ctx, g->table.p, 0xFFFFFFFFu, cap * 4));
+  SCN_TRY(scn_fill32(ctx, g->bits.p, 0u, (g->nWords + 2) * 2));
+  return SCN_OK;
+}
+
+static int ensure_rank(scn_ctx *ctx, scn_grids *g) {
+  if (g->rankValid)
+    return SCN_OK;
+  SCN_TRY(g->scanTmp.reserve(scn_scan_tmp_elems(g->nWords + 1)));
+  // one word past the mask so that the rank of the end position is defined
+  SCN_TRY(scn_scan_exclusive_popc64(ctx->stream,
+                                    (const uint64_t *)g->bits.p, g->prefix.p,
+                                    g->nWords + 1, g->scanTmp.p));
+  g->rankValid = true;
+  return SCN_OK;
+}
+
+static int read_scalars(scn_ctx *ctx) {
+  SCN_HIP_CHECK(hipMemcpyAsync(ctx->h_pinned, ctx->d_scalars,
+                               16 * sizeof(int64_t), hipMemcpyDeviceToHost,
+                               ctx->stream));
+  SCN_HIP_CHECK(hipStreamSynchronize(ctx->stream));
+  if (ctx->h_pinned[15] != 0) {
+    long long bad = ctx->h_pinned[15];
+    SCN_TRY(scn_fill32(ctx, ctx->d_scalars + 15, 0u, 2));
+    SCN_REQUIRE(false, SCN_ERR_ARG,
+                "scn_grids_build was given %lld sites outside the field", bad);
+  }
+  return SCN_OK;
+}
+
+extern "C" int scn_grids_create(scn_ctx *ctx, scn_grids **out) {
+  SCN_REQUIRE(ctx && out, SCN_ERR_ARG, "scn_grids_create: null argument");
+  *out = new scn_grids();
+  return SCN_OK;
+}
+
+extern "C" int scn_grids_destroy(scn_ctx *ctx, scn_grids *g) {
+  if (!g)
+    return SCN_OK;
+  if (ctx)
+    (void)hipStreamSynchronize(ctx->stream);
+  g->table.release();
+  g->bits.release();
+  g->prefix.release();
+  g->ekey.release();
+  g->erow.release();
+  g->bg.release();
+  g->scanTmp.release();
+  g->siteKey.release();
+  g->cnt.release();
+  g->base.release();
+  g->bgBefore.release();
+  g->sampleStart.release();
+  g->invOrd.release();
+  g->dlSample.release();
+  g->dlRow.release();
+  g->dlKey.release();
+  delete g;
+  return SCN_OK;
+}
+
+extern "C" int scn_grids_build(scn_ctx *ctx, scn_grids *g, int batch,
+                               int dimension, int spatialSize,
+                               const int32_t *d_sample, const int64_t *d_key,
+                               const int32_t *d_row, int64_t n,
+                               const int32_t *d_background,
+                               int32_t nSpatialSites) {
+  SCN_REQUIRE(ctx && g, SCN_ERR_ARG, "scn_grids_build: null argument");
+  SCN_REQUIRE(n >= 0 && (n == 0 || (d_sample && d_key && d_row)), SCN_ERR_ARG,
+              "scn_grids_build: null site arrays");
+  SCN_REQUIRE(batch == 0 || d_background, SCN_ERR_ARG,
+              "scn_grids_build: null background array");
+  ProfScope ps(ctx, SCN_K_GRID_BUILD);
+  SCN_TRY(grids_prepare(ctx, g, batch, dimension, spatialSize, n));
+  g->nSites = nSpatialSites;
+  if (batch > 0)
+    SCN_HIP_CHECK(hipMemcpyAsync(g->bg.p, d_background, batch * sizeof(int),
+                                 hipMemcpyDeviceToDevice, ctx->stream));
+  if (n > 0) {
+    hipLaunchKernelGGL(k_grid_build, dim3(scn_ceil_div(n, 256)), dim3(256), 0,
+                       ctx->stream, view_of(g), d_sample,
+                       (const long long *)d_key, d_row, (long long)n, g->ekey.p,
+                       g->erow.p, (unsigned long long *)(ctx->d_scalars + 15));
+    SCN_HIP_CHECK(hipGetLastError());
+  }
+  return SCN_OK;
+}
+
+extern "C" int scn_grids_info(const scn_grids *g, int *batch, int *dimension,
+                              int *spatialSize, int64_t *nActive,
+                              int32_t *nSpatialSites) {
+  SCN_REQUIRE(g, SCN_ERR_ARG, "scn_grids_info: null grids");
+  if (batch)
+    *batch = g->batch;
+  if (dimension)
+    *dimension = g->d;
+  if (spatialSize)
+    *spatialSize = g->n;
+  if (nActive)
+    *nActive = g->nActive;
+  if (nSpatialSites)
+    *nSpatialSites = g->nSites;
+  return SCN_OK;
+}
+
+extern "C" int scn_grids_download(scn_ctx *ctx, const scn_grids *cg,
+                                  int32_t *h_sample, int64_t *h_key,
+                                  int32_t *h_row, int32_t *h_background) {
+  scn_grids *g = const_cast<scn_grids *>(cg);
+  SCN_REQUIRE(ctx && g, SCN_ERR_ARG, "scn_grids_download: null argument");
+  SCN_TRY(ensure_rank(ctx, g));
+  long long n = g->nActive;
+  if (n > 0) {
+    SCN_TRY(g->dlSample.reserve((size_t)n));
+    SCN_TRY(g->dlRow.reserve((size_t)n));
+    SCN_TRY(g->dlKey.reserve((size_t)n));
+    hipLaunchKernelGGL(k_download, dim3(scn_ceil_div(n, 256)), dim3(256), 0,
+                       ctx->stream, view_of(g), g->ekey.p, g->erow.p, n,
+                       g->dlSample.p, g->dlKey.p, g->dlRow.p);
+    SCN_HIP_CHECK(hipGetLastError());
+    SCN_TRY(scn_d2h(ctx, h_sample, g->dlSample.p, n * sizeof(int)));
+    SCN_TRY(scn_d2h(ctx, h_key, g->dlKey.p, n * sizeof(long long)));
+    SCN_TRY(scn_d2h(ctx, h_row, g->dlRow.p, n * sizeof(int)));
+  }
+  if (g->batch > 0)
+    SCN_TRY(scn_d2h(ctx, h_background, g->bg.p, g->batch * sizeof(int)));
+  return SCN_OK;
+}
+
+extern "C" int scn_grids_find(scn_ctx *ctx, const scn_grids *g,
+                              const int32_t *d_sample, const int64_t *d_key,
+                              int64_t n, int32_t *d_row) {
+  SCN_REQUIRE(ctx && g, SCN_ERR_ARG, "scn_grids_find: null argument");
+  if (n <= 0)
+    return SCN_OK;
+  hipLaunchKernelGGL(k_find, dim3(scn_ceil_div(n, 256)), dim3(256), 0,
+                     ctx->stream, view_of(g), d_sample,
+                     (const long long *)d_key, (long long)n, d_row);
+  SCN_HIP_CHECK(hipGetLastError());
+  return SCN_OK;
+}
+
+static int triangle_size(int n, int d) { // utilities.cu:27-32
+  int fs = 1;
+  for (int i = 1; i <= d; ++i)
+    fs = fs * (n + d - i) / i;
+  return fs;
+}
+
+template <int D>
+static int plan_regions_d(scn_ctx *ctx, scn_grids *in, scn_grids *out,
+                          const Geom &g, long long fullSize,
+                          int64_t *nOutSites) {
+  const long long nE = in->nActive;
+  SCN_TRY(out->cnt.reserve((size_t)nE + 2));
+  SCN_TRY(out->base.reserve((size_t)nE + 2));
+  SCN_TRY(out->bgBefore.reserve((size_t)in->batch + 2));
+  SCN_TRY(out->sampleStart.reserve((size_t)in->batch + 2));
+  SCN_TRY(out->bg.reserve((size_t)in->batch + 1));
+  SCN_TRY(out->scanTmp.reserve(scn_scan_tmp_elems((size_t)nE + 1)));
+  GridView vin = view_of(in);
+  if (nE > 0) {
+    hipLaunchKernelGGL(k_plan_count<D>, dim3(scn_ceil_div(nE, 256)), dim3(256),
+                       0, ctx->stream, vin, g, in->ekey.p, nE, out->cnt.p);
+    SCN_HIP_CHECK(hipGetLastError());
+  }
+  SCN_TRY(scn_scan_exclusive_u32(ctx->stream, out->cnt.p, out->base.p,
+                                 (size_t)nE, out->scanTmp.p));
+  hipLaunchKernelGGL(k_plan_samples, dim3(1), dim3(1024), 0, ctx->stream, vin,
+                     out->base.p, nE, fullSize, out->bg.p, out->bgBefore.p,
+                     out->sampleStart.p, (long long *)ctx->d_scalars);
+  SCN_HIP_CHECK(hipGetLastError());
+  SCN_TRY(read_scalars(ctx));
+  long long nSites = ctx->h_pinned[0], nOutActive = ctx->h_pinned[1];
+  SCN_REQUIRE(nSites < 2147483647ll, SCN_ERR_CAPACITY,
+              "rules: %lld output rows do not fit 32-bit row numbers", nSites);
+  // out->bg already holds what k_plan_samples wrote: grids_prepare only
+  // reserves it (no reallocation at the same size) and clears table and mask
+  SCN_TRY(grids_prepare(ctx, out, in->batch, g.d, g.nOut, nOutActive));
+  out->nSites = (int)nSites;
+  SCN_TRY(out->siteKey.reserve((size_t)nSites + 1));
+  long long nThreads = nE > in->batch ? nE : in->batch;
+  if (nThreads > 0) {
+    hipLaunchKernelGGL(k_plan_emit<D>, dim3(scn_ceil_div(nThreads, 256)),
+                       dim3(256), 0, ctx->stream, vin, view_of(out), g,
+                       in->ekey.p, nE, out->base.p, out->bgBefore.p, out->bg.p,
+                       out->ekey.p, out->erow.p, out->siteKey.p);
+    SCN_HIP_CHECK(hipGetLastError());
+  }
+  *nOutSites = nSites;
+  return SCN_OK;
+}
+
+static int plan_regions(scn_ctx *ctx, const scn_grids *cin, scn_grids *out,
+                        int nIn, int nOut, int size, int stride, int minActive,
+                        bool tri, int64_t *nOutSites) {
+  scn_grids *in = const_cast<scn_grids *>(cin);
+  SCN_REQUIRE(ctx && in && out && nOutSites, SCN_ERR_ARG,
+              "rules plan: null argument");
+  SCN_REQUIRE(in != out, SCN_ERR_ARG, "rules plan: in and out are the same object");
+  SCN_REQUIRE(size >= 1 && size <= 32 && stride >= 1 && nOut >= 1,
+              SCN_ERR_ARG, "rules plan: size %d stride %d nOut %d", size,
+              stride, nOut);
+  // Regions.cu:17,823
+  SCN_REQUIRE(nIn == size + (nOut - 1) * stride, SCN_ERR_ARG,
+              "rules plan: nIn %d != size %d + (nOut %d - 1) * stride %d", nIn,
+              size, nOut, stride);
+  SCN_REQUIRE(in->n == nIn, SCN_ERR_ARG,
+              "rules plan: input grids have spatialSize %d, regions say %d",
+              in->n, nIn);
+  Geom g;
+  g.d = in->d;
+  g.nIn = nIn;
+  g.nOut = nOut;
+  g.size = size;
+  g.stride = stride;
+  g.minActive = minActive;
+  g.volIn = in->vol;
+  g.volOut = ipow_ll(nOut, in->d);
+  g.cube = (int)ipow_ll(size, in->d);
+  SCN_REQUIRE(ipow_ll(size, in->d) <= 32768, SCN_ERR_ARG,
+              "rules plan: window of %d^%d sites", size, in->d);
+  long long fullSize;
+  if (tri) {
+    SCN_REQUIRE(minActive >= 1, SCN_ERR_ARG,
+                "triangular rules: minActive %d", minActive);
+    g.mode = minActive == 1 ? MODE_TRI_NOMIN : MODE_TRI_MIN;
+    g.width = triangle_size(size, in->d);
+    fullSize = triangle_size(nOut, in->d);
+  } else {
+    SCN_REQUIRE(minActive >= 1 || minActive == -1, SCN_ERR_ARG,
+                "square rules: minActive %d", minActive);
+    if (minActive == -1) {
+      // Regions.cu:668,671,714,748: only the 2-D, size-3 case is live
+      SCN_REQUIRE(size == 3 && in->d == 2, SCN_ERR_ARG,
+                  "valid-mode rules need dimension 2 and size 3");
+      g.mode = MODE_SQ_VALID;
+    } else
+      g.mode = minActive == 1 ? MODE_SQ_NOMIN : MODE_SQ_MIN;
+    g.width = g.cube;
+    fullSize = g.volOut;
+  }
+  ProfScope ps(ctx, SCN_K_RULES);
+  SCN_TRY(ensure_rank(ctx, in));
+  int rc;
+  switch (in->d) {
+  case 1:
+    rc = plan_regions_d<1>(ctx, in, out, g, fullSize, nOutSites);
+    break;
+  case 2:
+    rc = plan_regions_d<2>(ctx, in, out, g, fullSize, nOutSites);
+    break;
+  default:
+    rc = plan_regions_d<3>(ctx, in, out, g, fullSize, nOutSites);
+    break;
+  }
+  SCN_TRY(rc);
+  if (tri) {
+    SCN_TRY(out->invOrd.reserve((size_t)g.cube));
+    hipLaunchKernelGGL(k_tri_table, dim3(1), dim3(64), 0, ctx->stream, size,
+                       in->d, out->invOrd.p);
+    SCN_HIP_CHECK(hipGetLastError());
+  }
+  out->geom = g;
+  out->planKind = PLAN_REGIONS;
+  out->planIn = in;
+  return SCN_OK;
+}
+
+extern "C" int scn_rules_square_plan(scn_ctx *ctx, const scn_grids *in,
+                                     scn_grids *out, int nIn, int nOut,
+                                     int size, int stride, int minActive,
+                                     int64_t *nOutSites) {
+  return plan_regions(ctx, in, out, nIn, nOut, size, stride, minActive, false,
+                      nOutSites);
+}
+
+extern "C" int scn_rules_triangular_plan(scn_ctx *ctx, const scn_grids *in,
+                                         scn_grids *out, int nIn, int nOut,
+                                         int size, int stride, int minActive,
+                                         int64_t *nOutSites) {
+  return plan_regions(ctx, in, out, nIn, nOut, size, stride, minActive, true,
+                      nOutSites);
+}
+
+extern "C" int scn_rules_terminal_plan(scn_ctx *ctx, const scn_grids *cin,
+                                       scn_grids *out, int64_t *ruleWidth) {
+  scn_grids *in = const_cast<scn_grids *>(cin);
+  SCN_REQUIRE(ctx && in && out && ruleWidth, SCN_ERR_ARG,
+              "terminal rules plan: null argument");
+  SCN_REQUIRE(in != out, SCN_ERR_ARG,
+              "terminal rules plan: in and out are the same object");
+  ProfScope ps(ctx, SCN_K_RULES);
+  SCN_TRY(ensure_rank(ctx, in));
+  SCN_TRY(out->sampleStart.reserve((size_t)in->batch + 2));
+  hipLaunchKernelGGL(k_terminal_plan, dim3(1), dim3(1024), 0, ctx->stream,
+                     view_of(in), out->sampleStart.p,
+                     (long long *)ctx->d_scalars);
+  SCN_HIP_CHECK(hipGetLastError());
+  SCN_TRY(read_scalars(ctx));
+  long long S = ctx->h_pinned[0];
+  SCN_TRY(grids_prepare(ctx, out, in->batch, in->d, 1, in->batch));
+  out->nSites = in->batch;
+  if (in->batch > 0) {
+    hipLaunchKernelGGL(k_terminal_out, dim3(scn_ceil_div(in->batch, 256)),
+                       dim3(256), 0, ctx->stream, view_of(out), out->ekey.p,
+                       out->erow.p, out->bg.p);
+    SCN_HIP_CHECK(hipGetLastError());
+  }
+  out->termS = S;
+  out->planKind = PLAN_TERMINAL;
+  out->planIn = in;
+  *ruleWidth = S;
+  return SCN_OK;
+}
+
+extern "C" int scn_rules_width(const scn_grids *out, int64_t *width) {
+  SCN_REQUIRE(out && width, SCN_ERR_ARG, "scn_rules_width: null argument");
+  SCN_REQUIRE(out->planKind != PLAN_NONE, SCN_ERR_STATE,
+              "scn_rules_width: no plan on these grids");
+  *width = out->planKind == PLAN_TERMINAL ? out->termS : out->geom.width;
+  return SCN_OK;
+}
+
+extern "C" int scn_rules_fill(scn_ctx *ctx, const scn_grids *in,
+                              scn_grids *out, int32_t *d_rules,
+                              int64_t capacity) {
+  SCN_REQUIRE(ctx && in && out, SCN_ERR_ARG, "scn_rules_fill: null argument");
+  SCN_REQUIRE(out->planKind != PLAN_NONE && out->planIn == in, SCN_ERR_STATE,
+              "scn_rules_fill: `out` does not hold a plan made from `in`");
+  ProfScope ps(ctx, SCN_K_RULES);
+  GridView vin = view_of(in);
+  if (out->planKind == PLAN_TERMINAL) {
+    long long total = (long long)in->batch * out->termS;
+    SCN_REQUIRE(capacity >= total, SCN_ERR_CAPACITY,
+                "scn_rules_fill: %lld rules, capacity %lld", total,
+                (long long)capacity);
+    if (total == 0)
+      return SCN_OK;
+    SCN_REQUIRE(d_rules, SCN_ERR_ARG, "scn_rules_fill: null rules buffer");
+    hipLaunchKernelGGL(k_terminal_init, dim3(scn_ceil_div(total, 256)),
+                       dim3(256), 0, ctx->stream, vin, out->sampleStart.p,
+                       out->termS, d_rules);
+    SCN_HIP_CHECK(hipGetLastError());
+    if (in->nActive > 0) {
+      hipLaunchKernelGGL(k_terminal_scatter,
+                         dim3(scn_ceil_div(in->nActive, 256)), dim3(256), 0,
+                         ctx->stream, vin, in->ekey.p, in->erow.p, in->nActive,
+                         out->sampleStart.p, out->termS, d_rules);
+      SCN_HIP_CHECK(hipGetLastError());
+    }
+    return SCN_OK;
+  }
+  const Geom &g = out->geom;
+  long long total = (long long)out->nSites * g.width;
+  SCN_REQUIRE(capacity >= total, SCN_ERR_CAPACITY,
+              "scn_rules_fill: %lld rules, capacity %lld", total,
+              (long long)capacity);
+  if (total == 0)
+    return SCN_OK;
+  SCN_REQUIRE(d_rules, SCN_ERR_ARG, "scn_rules_fill: null rules buffer");
+  const bool tri = g.mode == MODE_TRI_NOMIN || g.mode == MODE_TRI_MIN;
+  const int *inv = tri ? out->invOrd.p : nullptr;
+  dim3 grid(scn_ceil_div(total, 256)), block(256);
+  switch (g.d) {
+  case 1:
+    hipLaunchKernelGGL(k_rules_fill<1>, grid, block, 0, ctx->stream, vin, g,
+                       out->siteKey.p, (long long)out->nSites, inv, d_rules);
+    break;
+  case 2:
+    hipLaunchKernelGGL(k_rules_fill<2>, grid, block, 0, ctx->stream, vin, g,
+                       out->siteKey.p, (long long)out->nSites, inv, d_rules);
+    break;
+  default:
+    hipLaunchKernelGGL(k_rules_fill<3>, grid, block, 0, ctx->stream, vin, g,
+                       out->siteKey.p, (long long)out->nSites, inv, d_rules);
+    break;
+  }
+  SCN_HIP_CHECK(hipGetLastError());
+  return SCN_OK;
+}

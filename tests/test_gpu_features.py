@@ -1,0 +1,131 @@
+"""Feature kernels against the CPU oracle (through the C ABI)."""
+import numpy as np
+import pytest
+
+import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("nIn", [1, 3, 4, 32, 33, 64, 160, 288, 1030])
+def test_gather_bit_exact(scn, ctx, nIn):
+    rng = np.random.default_rng(nIn)
+    rows = 501
+    inp = rng.standard_normal((rows, nIn)).astype(np.float32)
+    for count in (1, 255, 256, 257, 5000):
+        print("gather nIn=%d count=%d" % (nIn, count), flush=True)
+        rules = rng.integers(0, rows, size=count).astype(np.int32)
+        d_out = ctx.empty((count, nIn), np.float32)
+        ctx.gather_rows(ctx.array(inp), d_out, ctx.array(rules), count, nIn)
+        assert np.array_equal(d_out.download(), orc.gather_rows(inp, rules, nIn))
+
+
+@pytest.mark.parametrize("C,ps", [(32, 4), (32, 9), (64, 8), (96, 27), (3, 4), (160, 9), (5, 3)])
+def test_maxpool_values_and_argmax_bit_exact(scn, ctx, C, ps):
+    rng = np.random.default_rng(C * 100 + ps)
+    rows, nOut = 300, 777
+    # quantised values force ties; the first maximum in window order must win
+    inp = rng.integers(-2, 3, size=(rows, C)).astype(np.float32)
+    rules = rng.integers(-1, rows, size=(nOut, ps)).astype(np.int32)
+    rules[:, 0] = np.abs(rules[:, 0])
+    print("maxpool C=%d ps=%d" % (C, ps), flush=True)
+    d_out = ctx.empty((nOut, C), np.float32)
+    d_choice = ctx.empty((nOut, C), np.int32)
+    ctx.maxpool(ctx.array(inp), d_out, ctx.array(rules), nOut, ps, C, d_choice)
+    o_out, o_choice = orc.maxpool(inp, rules, nOut, ps, C)
+    assert np.array_equal(d_out.download(), o_out)
+    assert np.array_equal(d_choice.download(), o_choice)
+    # random floats as well
+    inp = rng.standard_normal((rows, C)).astype(np.float32)
+    ctx.maxpool(ctx.array(inp), d_out, ctx.array(rules), nOut, ps, C, d_choice)
+    o_out, o_choice = orc.maxpool(inp, rules, nOut, ps, C)
+    assert np.array_equal(d_out.download(), o_out)
+    assert np.array_equal(d_choice.download(), o_choice)
+
+
+def test_terminal_pool_bit_exact(scn, ctx):
+    rng = np.random.default_rng(1)
+    rows, C, B, S = 400, 192, 37, 9
+    inp = rng.standard_normal((rows, C)).astype(np.float32)
+    rules = np.full((B, S), -1, np.int32)
+    for b in range(B):
+        n = 1 + b % S
+        rules[b, :n] = rng.integers(0, rows, n)
+    d_out = ctx.empty((B, C), np.float32)
+    ctx.terminal_pool(ctx.array(inp), d_out, ctx.array(rules), B, S, C)
+    assert np.array_equal(d_out.download(), orc.terminal_pool(inp, rules, B, S, C))
+
+
+def test_softmax(scn, ctx):
+    rng = np.random.default_rng(2)
+    for M, N in ((100, 100), (7, 40), (3, 1), (130, 1000)):
+        x = (rng.standard_normal((M, N)) * 4).astype(np.float32)
+        d_out = ctx.empty((M, N), np.float32)
+        ctx.softmax_rows(ctx.array(x), d_out, M, N)
+        got = d_out.download()
+        want = orc.softmax_rows(x)
+        # tolerance: fp32 forward path, 1e-4 relative
+        assert np.allclose(got, want, rtol=1e-4, atol=1e-7)
+        assert np.array_equal(got.argmax(1), want.argmax(1))
+    lo = np.full((1, 3), -10050.0, np.float32)
+    lo[0, 1] = -10040.0
+    d_out = ctx.empty((1, 3), np.float32)
+    ctx.softmax_rows(ctx.array(lo), d_out, 1, 3)
+    assert np.allclose(d_out.download(), orc.softmax_rows(lo), rtol=1e-4)
+
+
+SHAPES = [(1000, 12, 32), (777, 128, 64), (513, 256, 96), (300, 384, 128), (129, 512, 160), (400, 160, 192),
+          (100, 192, 100), (64, 288, 64), (5, 7, 3), (2000, 27, 32), (257, 1728, 64)]
+
+
+@pytest.mark.parametrize("M,K,N", SHAPES)
+@pytest.mark.parametrize("act", ["NOSIGMOID", "RELU", "LEAKYRELU", "VLEAKYRELU", "PRELU", "SOFTMAX"])
+def test_nin_fp32(scn, ctx, M, K, N, act):
+    """fp32 activations within 1e-4 relative of the oracle (scaled by the
+    magnitude of the contraction, since individual outputs can cancel)."""
+    a = getattr(scn, act)
+    rng = np.random.default_rng(M + K + N + a)
+    A = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    W = (rng.standard_normal((K, N)) * np.sqrt(2.0 / K)).astype(np.float32)
+    B = rng.uniform(-0.5, 0.5, N).astype(np.float32)
+    pr = rng.uniform(0.1, 0.4, N).astype(np.float32)
+    p = 0.75 if act == "RELU" else 1.0
+    print("nin M=%d K=%d N=%d act=%s" % (M, K, N, act), flush=True)
+    d_out = ctx.empty((M, N), np.float32)
+    ctx.nin_forward(ctx.array(A), ctx.array(W), ctx.array(B), ctx.array(pr), d_out, M, K, N, p, a, scn.FP32)
+    got = d_out.download()
+    want64 = orc.nin_forward(A, W, B, pr, p, a, f64=True)
+    want32 = orc.nin_forward(A, W, B, pr, p, a)
+    if act == "SOFTMAX":
+        assert np.allclose(got, want64, rtol=1e-4, atol=1e-6)
+        return
+    scale = np.abs(A).astype(np.float64) @ np.abs(W).astype(np.float64) + np.abs(B)
+    assert np.all(np.abs(got - want64) <= 1e-4 * scale)
+    # and no further from fp64 than the oracle's own fp32 accumulation, within a factor
+    err_gpu = np.abs(got - want64).max()
+    err_cpu = np.abs(want32 - want64).max()
+    assert err_gpu <= 4 * err_cpu + 1e-6
+    rel = np.linalg.norm(got - want64) / max(np.linalg.norm(want64), 1e-30)
+    assert rel <= 1e-4
+
+
+def test_nin_special_cases(scn, ctx):
+    rng = np.random.default_rng(3)
+    M, K = 70, 64
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = rng.standard_normal(K).astype(np.float32)
+    d_out = ctx.empty((M, K), np.float32)
+    ctx.nin_forward(ctx.array(A), ctx.array(np.eye(K, dtype=np.float32)), ctx.array(B), None, d_out, M, K, K, 1.0,
+                    scn.NOSIGMOID)
+    assert np.array_equal(d_out.download(), A + B)
+    W = np.zeros((K, K), np.float32)
+    W[3, 7] = 2.0
+    ctx.nin_forward(ctx.array(A), ctx.array(W), ctx.array(np.zeros(K, np.float32)), None, d_out, M, K, K, 1.0,
+                    scn.NOSIGMOID)
+    want = np.zeros((M, K), np.float32)
+    want[:, 7] = 2.0 * A[:, 3]
+    assert np.array_equal(d_out.download(), want)
+    with pytest.raises(scn.ScnError):
+        ctx.nin_forward(ctx.array(A), ctx.array(W), ctx.array(B), None, d_out, M, K, K, 1.0, scn.TANH)
+    with pytest.raises(scn.ScnError):
+        ctx.nin_forward(ctx.array(A), ctx.array(W), ctx.array(B), None, d_out, M, K, K, 1.0, scn.PRELU)
