@@ -1,0 +1,260 @@
+#!/usr/bin/env python3
+"""Forward-path benchmark on one MI355X.
+
+A step is one forward pass of one synthetic batch through the C++ host classes
+(SparseConvNet) on top of libscn_hip.so: grid hash build, every rule book,
+gather / NiN / max-pool / terminal pool / softmax kernels, and the copy of the
+class probabilities back to the host.  The batch's active sites and input
+features are already in HBM when the timed region starts.
+
+Prints ONE JSON line: active sites/s (value) and samples/s, the roofline of the
+kernel family that takes the most time, a per-kernel table, and the CPU oracle
+timed on this host's cores beside it.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "oracle"))
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+MFMA_PEAK_TFLOPS = {"fp32": 157.3, "bf16": 2500.0}
+BALANCE_FLOP_PER_BYTE = {"fp32": 157.3e12 / 8e12, "bf16": 2500e12 / 8e12}
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--config", type=int, default=2, help="1..5, the synthetic configs; 2 is the headline one")
+    ap.add_argument("--batch", type=int, default=None)
+    ap.add_argument("--precision", choices=["fp32", "bf16"], default="fp32")
+    ap.add_argument("--seed", type=int, default=2015)
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 disables it)")
+    return ap.parse_args()
+
+
+def algorithmic_work(layers, ifaces, batch, precision):
+    """{(family, layer): (bytes, flops)} per step, from the sizes of one forward
+    pass.  N_in / N_out are active sites of the grids, rows include the
+    background rows."""
+    work = {}
+    n0 = ifaces[0]["gridEntries"]
+    work[("grid_build", -1)] = (28 * n0, 0)
+    esz = 4
+    for i, l in enumerate(layers):
+        a, b = ifaces[i], ifaces[i + 1]
+        k = l["kind"]
+        if k in ("conv", "conv_tri", "maxpool", "maxpool_tri"):
+            width = b["nRules"] // max(b["rows"], 1)
+            work[("rules", i)] = (12 * a["gridEntries"] + 12 * b["gridEntries"] + 4 * width * b["rows"], 0)
+            if k.startswith("conv"):
+                count = b["nRules"]
+                work[("gather", i)] = (4 * count + 2 * esz * count * a["nFeatures"], 0)
+            else:
+                C = a["nFeatures"]
+                work[("maxpool", i)] = (4 * width * b["rows"] + esz * C * width * b["rows"] + 8 * C * b["rows"], 0)
+        elif k == "terminal":
+            S = b["nRules"] // max(batch, 1)
+            work[("rules", i)] = (12 * a["gridEntries"] + 4 * batch * S, 0)
+            work[("terminal", i)] = (esz * a["nFeatures"] * a["gridEntries"] + 4 * batch * S + 4 * batch * a["nFeatures"], 0)
+        else:
+            M, K, N = b["rows"], l["nIn"], l["nOut"]
+            asz = 2 if precision == "bf16" else 4
+            work[("nin", i)] = (asz * (M * K + K * N) + 4 * (M * N + N), 2 * M * K * N)
+    return work
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; --gpus %d is not supported (the forward path shards by sample "
+              "with no exchange, see DESIGN.md)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    # the host classes announce every layer on stdout like the reference does;
+    # keep stdout for the one JSON line and send that chatter to stderr
+    sys.stdout.flush()
+    saved_stdout = os.dup(1)
+    os.dup2(2, 1)
+    from __graft_entry__ import load_package
+    scn = load_package()
+    from sparseconvnet_archived_amd import hostapi, synthetic
+
+    cfg = synthetic.config(args.config, batch=args.batch)
+    B = cfg.batch
+    net = hostapi.Net(cfg.dimension, cfg.nInputFeatures, max(cfg.nClasses, 1), threads=1)
+    cfg.build(net)
+    if args.precision == "bf16":
+        net.setPrecision(scn.BF16)
+    layers = net.layers()
+    weights = synthetic.he_normal_weights(layers, args.seed + 1)
+    for i, (W, Bv, pr) in weights.items():
+        net.set_weights(i, W, Bv, pr)
+    samples = synthetic.make_samples(cfg, args.seed)
+    S, K, R, bg, feats, nSites = synthetic.codify(samples, cfg.dimension, cfg.lattice, net.inputSpatialSize,
+                                                  cfg.nInputFeatures)
+    active = int(len(K))
+    ctx = scn.Context(handle=net.context_handle())
+    dS, dK, dR, dBg, dF = ctx.array(S, np.int32), ctx.array(K, np.int64), ctx.array(R, np.int32), ctx.array(bg, np.int32), ctx.array(feats, np.float32)
+    probs = np.zeros((B, max(cfg.nClasses, 1)), np.float32)
+
+    def step():
+        net.forward_resident(B, dS.ptr, dK.ptr, dR.ptr, dBg.ptr, active, nSites, dF.ptr, probs)
+
+    for _ in range(args.warmup):
+        step()
+    ctx.sync()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    ctx.sync()
+    dt = time.perf_counter() - t0
+    ms_per_step = 1e3 * dt / args.steps
+    mac = hostapi.take_multiply_add_count()  # resets the counter
+    step()
+    mac = hostapi.take_multiply_add_count()
+
+    # sizes of every interface, for the algorithmic byte / flop counts
+    ifaces = []
+    for i in range(len(layers) + 1):
+        info = net.interface(i, want_features=False)
+        ifaces.append(dict(rows=info["nSpatialSites"], nFeatures=info["nFeatures"], nRules=int(info["rules"].size),
+                           gridEntries=int(info["grids"][0].size)))
+    work = algorithmic_work(layers, ifaces, B, args.precision)
+
+    # per-kernel durations: HIP events on the library's stream, same steps again
+    ctx.prof_reset()
+    ctx.prof_enable(True)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    ctx.sync()
+    dt_prof = time.perf_counter() - t0
+    spans = ctx.prof_spans()
+    ctx.prof_enable(False)
+    tot, cnt = {}, {}
+    for fam, tag, ms in spans:
+        key = (fam, tag)
+        tot[key] = tot.get(key, 0.0) + ms
+        cnt[key] = cnt.get(key, 0) + 1
+    kernels = []
+    for key, ms_total in tot.items():
+        fam, tag = key
+        ms = ms_total / args.steps
+        byts, flops = work.get(key, (0, 0))
+        entry = dict(kernel=fam, layer=tag, ms_per_step=round(ms, 5), launches_per_step=cnt[key] / args.steps)
+        if fam == "nin" and flops:
+            K_, N_ = layers[tag]["nIn"], layers[tag]["nOut"]
+            intensity = flops / max(byts, 1)
+            entry["shape"] = [ifaces[tag + 1]["rows"], K_, N_]
+            if intensity >= BALANCE_FLOP_PER_BYTE[args.precision]:
+                a = flops / (ms * 1e-3) / 1e12
+                entry.update(bound="mfma", achieved=a, peak=MFMA_PEAK_TFLOPS[args.precision], unit="TFLOP/s")
+            else:
+                a = byts / (ms * 1e-3) / 1e9
+                entry.update(bound="hbm", achieved=a, peak=HBM_PEAK_GBS, unit="GB/s")
+        elif byts:
+            a = byts / (ms * 1e-3) / 1e9
+            entry.update(bound="hbm", achieved=a, peak=HBM_PEAK_GBS, unit="GB/s")
+        if "achieved" in entry:
+            entry["frac"] = entry["achieved"] / entry["peak"]
+            entry["achieved"] = round(entry["achieved"], 3)
+            entry["frac"] = round(entry["frac"], 5)
+        kernels.append(entry)
+    kernels.sort(key=lambda e: -e["ms_per_step"])
+    fam_ms = {}
+    for e in kernels:
+        fam_ms[e["kernel"]] = fam_ms.get(e["kernel"], 0.0) + e["ms_per_step"]
+    dominant = next((e for e in kernels if "achieved" in e), None)
+    roofline = None
+    if dominant:
+        roofline = dict(kernel="%s[layer %d]" % (dominant["kernel"], dominant["layer"]), bound=dominant["bound"],
+                        achieved=dominant["achieved"], peak=dominant["peak"], unit=dominant["unit"], frac=dominant["frac"],
+                        traffic=None)
+
+    cpu_baseline = None
+    if args.cpu_seconds > 0:
+        cpu_baseline = cpu_leg(cfg, layers, weights, samples, net.inputSpatialSize, args.cpu_seconds)
+
+    out = {
+        "metric": "active sites/sec + samples/sec fwd at 1 GPU; % HBM GB/s and % MFMA peak",
+        "value": active * args.steps / dt,
+        "unit": "active sites/s",
+        "samples_per_s": B * args.steps / dt,
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "ms_per_step_with_event_timing": 1e3 * dt_prof / args.steps,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32" if args.precision == "fp32" else "bf16",
+        "data": "synthetic",
+        "config": {"workload": cfg.name, "batch": B, "input_field": net.inputSpatialSize, "lattice": cfg.lattice,
+                   "dimension": cfg.dimension, "active_sites": active, "input_rows": nSites,
+                   "stack": [list(c) for c in cfg.stack], "precision": args.precision, "seed": args.seed},
+        "mega_multiply_adds_per_sample": mac / B / 1e6,
+        "giga_multiply_adds_per_s": mac / (ms_per_step * 1e-3) / 1e9,
+        "roofline": roofline,
+        "kernel_family_ms_per_step": {k: round(v, 5) for k, v in fam_ms.items()},
+        "kernels": kernels,
+        "cpu_baseline": cpu_baseline,
+    }
+    net.close()
+    sys.stdout.flush()
+    os.dup2(saved_stdout, 1)
+    print(json.dumps(out))
+
+
+def cpu_leg(cfg, layers, weights, samples, spatialSize, budget_s):
+    """The CPU oracle on this host's cores, same batch, bounded wall time."""
+    import oracle as orc
+    import oracle_net
+    from sparseconvnet_archived_amd import synthetic
+    cores = min(os.cpu_count() or 1, 16)
+    ora = oracle_net.Net(cfg.dimension, cfg.nInputFeatures, max(cfg.nClasses, 1))
+    cfg.build(ora)
+    for i, (W, Bv, pr) in weights.items():
+        ora.set_weights(i, W, Bv, pr)
+    # bounded sample: shrink the batch until one pass fits the budget
+    sub = samples
+    if cfg.number == 5:
+        sub = samples[:2]
+    elif cfg.number == 4:
+        sub = samples[:16]
+    S, K, R, bg, feats, n = synthetic.codify(sub, cfg.dimension, cfg.lattice, spatialSize, cfg.nInputFeatures)
+    orc.set_threads(cores)
+    times, t_start = [], time.perf_counter()
+    while len(times) < 2 or (time.perf_counter() - t_start < budget_s and len(times) < 20):
+        t0 = time.perf_counter()
+        ora.forward(len(sub), S, K, R, bg, feats, n, keep=False)
+        times.append(time.perf_counter() - t0)
+    full = float(np.median(times))
+    # rule books only, one thread (the reference's own CPU code on this path)
+    g = orc.Grids.from_flat(len(sub), S, K, R, bg)
+    t0 = time.perf_counter()
+    cur = g
+    for l in ora.layers:
+        if l["kind"] in ("conv", "maxpool"):
+            cur, _, _ = orc.rules_square(cur, cfg.dimension, l["inSize"], l["outSize"], l["size"], l["stride"], l.get("minActive", 1))
+        elif l["kind"] == "terminal":
+            cur, _, _ = orc.rules_terminal(cur)
+    rules_only = time.perf_counter() - t0
+    orc.set_threads(1)
+    return {"value": len(K) / full, "unit": "active sites/s", "cores": cores, "kind": "port",
+            "sample": "%s, %d of %d samples, %d passes, median" % (cfg.name, len(sub), len(samples), len(times)),
+            "ms_per_batch": 1e3 * full, "samples_per_s": len(sub) / full,
+            "rulebooks_only_1_thread_ms": 1e3 * rules_only,
+            "rulebooks_only_active_sites_per_s": len(K) / rules_only}
+
+
+if __name__ == "__main__":
+    main()

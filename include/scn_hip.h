@@ -71,6 +71,8 @@ int scn_malloc(scn_ctx *ctx, size_t bytes, void **d_ptr);
 int scn_free(scn_ctx *ctx, void *d_ptr);
 int scn_h2d(scn_ctx *ctx, void *d_dst, const void *h_src, size_t bytes);
 int scn_d2h(scn_ctx *ctx, void *h_dst, const void *d_src, size_t bytes);
+/* device-to-device, asynchronous on the context's stream */
+int scn_d2d(scn_ctx *ctx, void *d_dst, const void *d_src, size_t bytes);
 int scn_fill32(scn_ctx *ctx, void *d_dst, uint32_t word, size_t nWords);
 
 /* ---- sparse grids ----------------------------------------------------- */
@@ -177,6 +179,13 @@ enum {
   SCN_K_COUNT = 7
 };
 int scn_prof_enable(scn_ctx *ctx, int on);
+/* label attached to the spans recorded from now on (e.g. the layer index) */
+int scn_prof_tag(scn_ctx *ctx, int tag);
+/* synchronises and hands back every span recorded since the last read:
+ * family, tag and milliseconds of up to `capacity` spans, *n = their number
+ * (spans beyond the capacity are dropped).  Also adds them to the totals. */
+int scn_prof_spans(scn_ctx *ctx, int capacity, int32_t *family, int32_t *tag,
+                   double *ms, int32_t *n);
 int scn_prof_reset(scn_ctx *ctx);
 /* synchronises, then returns accumulated milliseconds and number of calls */
 int scn_prof_read(scn_ctx *ctx, int family, double *ms, int64_t *calls);

@@ -1,0 +1,139 @@
+"""Net-level CPU oracle: the reference's layer builders and per-batch forward
+restated over the C oracle.  TEST INFRASTRUCTURE ONLY.
+
+Builders follow SparseConvNetCUDA.cu:50-111 (addLearntLayer rounding to 32,
+filterSize 1 adds no gather layer, poolSize 1 adds no pooling layer),
+:165-196 (triangular builders, including the argument mix-up that makes the
+convolution's minActiveInputs equal to the pool size) and :198-210 (spatial
+sizes worked out from the top).  forward() follows BatchProducer.cu:40-87
+(every layer's preprocess) and SparseConvNetCUDA.cu:227-247 (forwards loop,
+then SoftmaxClassifier).
+"""
+import numpy as np
+
+import oracle as orc
+
+RELU, SOFTMAX, PRELU = orc.RELU, orc.SOFTMAX, orc.PRELU
+
+
+def int_round(a, d):  # utilities.cu:103
+    return int(np.floor(a * 1.0 / d + 0.5)) * d if a >= 0 else -int(np.floor(-a * 1.0 / d + 0.5)) * d
+
+
+class Net:
+    def __init__(self, dimension, nInputFeatures, nClasses, nTop=1, triangular=False):
+        self.dimension, self.nInputFeatures, self.nClasses, self.nTop = dimension, nInputFeatures, nClasses, nTop
+        self.triangular = triangular
+        self.nOutputFeatures = nInputFeatures
+        self.layers = []  # dicts: kind, geometry, nIn, nOut, act, dropout
+        self.weights = {}
+        self.inputSpatialSize = None
+
+    # ---- builders
+    def _learnt(self, nFeatures, act, dropout):
+        if act != SOFTMAX:
+            nFeatures = max(32, int_round(nFeatures, 32))
+        if dropout > 0:
+            kept = int(np.float32(nFeatures) * (np.float32(1) - np.float32(dropout)))  # float -> int argument
+            dropout = np.float32(1) - (np.float32(int_round(kept, 32)) + np.float32(0.01)) * np.float32(1.0) / np.float32(nFeatures)
+        dropout = max(float(dropout), 0.0)
+        kind = "nin_prelu" if act == PRELU else "nin"
+        self.layers.append(dict(kind=kind, nIn=self.nOutputFeatures, nOut=nFeatures, act=act, dropout=dropout))
+        self.nOutputFeatures = nFeatures
+
+    def addLeNetLayerMP(self, nFeatures, filterSize, filterStride, poolSize, poolStride, activationFn=RELU, dropout=0.0,
+                        minActiveInputs=1):
+        tri = self.triangular
+        if tri:
+            minActiveInputs = poolSize  # SparseConvNetCUDA.cu:165-168 vs :183-185
+        if filterSize > 1:
+            fs = orc.lib.orc_triangle_size(filterSize, self.dimension) if tri else filterSize ** self.dimension
+            self.layers.append(dict(kind="conv_tri" if tri else "conv", size=filterSize, stride=filterStride,
+                                    minActive=minActiveInputs, nIn=self.nOutputFeatures,
+                                    nOut=self.nOutputFeatures * fs, fs=fs))
+            self.nOutputFeatures *= fs
+        self._learnt(nFeatures, activationFn, dropout)
+        if poolSize > 1:
+            self.layers.append(dict(kind="maxpool_tri" if tri else "maxpool", size=poolSize, stride=poolStride, nIn=0, nOut=0))
+
+    def addTerminalPoolingLayer(self, poolSize):
+        self.layers.append(dict(kind="terminal", size=poolSize, nIn=0, nOut=0))
+
+    def _sizes_from(self, top):
+        s = top
+        for l in reversed(self.layers):
+            l["outSize"] = s
+            if l["kind"] in ("conv", "conv_tri", "maxpool", "maxpool_tri"):
+                s = l["size"] + (s - 1) * l["stride"]
+            elif l["kind"] == "terminal":
+                assert s == 1
+                s = l["size"]
+            l["inSize"] = s
+        self.inputSpatialSize = s
+        return s
+
+    def addSoftmaxLayer(self):
+        self._learnt(self.nClasses, SOFTMAX, 0.0)
+        self._sizes_from(1)
+
+    def finishHeadless(self, topSpatialSize):
+        return self._sizes_from(topSpatialSize)
+
+    def layer_list(self):
+        return [dict(kind=l["kind"], nIn=l.get("nIn", 0) if l["kind"] in ("conv", "conv_tri", "nin", "nin_prelu") else 0,
+                     nOut=l.get("nOut", 0) if l["kind"] in ("conv", "conv_tri", "nin", "nin_prelu") else 0,
+                     act=l.get("act", -1) if l["kind"] in ("nin", "nin_prelu") else -1) for l in self.layers]
+
+    def set_weights(self, layer, W, B, prelu=None):
+        self.weights[layer] = (np.asarray(W, np.float32), np.asarray(B, np.float32),
+                               None if prelu is None else np.asarray(prelu, np.float32))
+
+    # ---- forward over one batch
+    def forward(self, batch, sample, key, row, bg, features, nSpatialSites, labels=None, keep=True):
+        """Returns a list of interfaces (dicts with grids, rules, features,
+        choices, nSpatialSites, nFeatures, spatialSize) and, when the net ends
+        in the classifier, probabilities / predictions / mistakes / nll."""
+        d = self.dimension
+        g = orc.Grids.from_flat(batch, sample, key, row, bg)
+        feats = np.ascontiguousarray(features, np.float32)
+        ifaces = [dict(grids=g, rules=np.zeros(0, np.int32), features=feats, choices=np.zeros(0, np.int32),
+                       nSpatialSites=nSpatialSites, nFeatures=self.nInputFeatures, spatialSize=self.inputSpatialSize)]
+        for i, l in enumerate(self.layers):
+            k = l["kind"]
+            cur = ifaces[-1]
+            nxt = dict(grids=cur["grids"], rules=np.zeros(0, np.int32), choices=np.zeros(0, np.int32),
+                       nFeatures=cur["nFeatures"], spatialSize=cur["spatialSize"], nSpatialSites=cur["nSpatialSites"])
+            if k in ("conv", "conv_tri", "maxpool", "maxpool_tri"):
+                fn = orc.rules_triangular if k.endswith("_tri") else orc.rules_square
+                minActive = l.get("minActive", 1)
+                og, rules, n = fn(cur["grids"], d, l["inSize"], l["outSize"], l["size"], l["stride"], minActive)
+                nxt.update(grids=og, rules=rules, nSpatialSites=n, spatialSize=l["outSize"])
+                if k.startswith("conv"):
+                    nxt["features"] = orc.gather_rows(cur["features"], rules, cur["nFeatures"]).reshape(n, -1)
+                    nxt["nFeatures"] = cur["nFeatures"] * l["fs"]
+                else:
+                    width = rules.size // max(n, 1)
+                    nxt["features"], ch = orc.maxpool(cur["features"], rules, n, width, cur["nFeatures"])
+                    nxt["choices"] = ch.reshape(-1)
+            elif k in ("nin", "nin_prelu"):
+                W, B, pr = self.weights[i]
+                p = np.float32(1.0) - np.float32(l["dropout"])
+                nxt["features"] = orc.nin_forward(cur["features"], W, B, pr, p, l["act"])
+                nxt["nFeatures"] = l["nOut"]
+            elif k == "terminal":
+                og, rules, S = orc.rules_terminal(cur["grids"])
+                nxt.update(grids=og, rules=rules, nSpatialSites=batch, spatialSize=1)
+                nxt["features"] = orc.terminal_pool(cur["features"], rules, batch, S, cur["nFeatures"])
+            if not keep:
+                cur.pop("features", None)
+            ifaces.append(nxt)
+        out = dict(interfaces=ifaces)
+        if self.layers and self.layers[-1].get("act") == SOFTMAX:
+            probs = ifaces[-1]["features"]
+            out["probabilities"] = probs
+            if labels is not None:
+                pred, mistakes, nll = orc.softmax_classifier(probs, labels, self.nTop)
+                out.update(predictions=pred, mistakes=mistakes, nll=nll)
+            else:
+                out["predictions"] = np.stack([orc.top_indices(p, self.nTop) for p in probs])
+        return out

@@ -67,6 +67,7 @@ def lib():
         "scn_free": (C.c_int, [vp, vp]),
         "scn_h2d": (C.c_int, [vp, vp, vp, sz]),
         "scn_d2h": (C.c_int, [vp, vp, vp, sz]),
+        "scn_d2d": (C.c_int, [vp, vp, vp, sz]),
         "scn_fill32": (C.c_int, [vp, vp, C.c_uint32, sz]),
         "scn_grids_create": (C.c_int, [vp, P(vp)]),
         "scn_grids_destroy": (C.c_int, [vp, vp]),
@@ -86,6 +87,8 @@ def lib():
         "scn_softmax_rows": (C.c_int, [vp, vp, vp, i64, C.c_int]),
         "scn_prof_enable": (C.c_int, [vp, C.c_int]),
         "scn_prof_reset": (C.c_int, [vp]),
+        "scn_prof_tag": (C.c_int, [vp, C.c_int]),
+        "scn_prof_spans": (C.c_int, [vp, C.c_int, vp, vp, vp, P(i32)]),
         "scn_prof_read": (C.c_int, [vp, C.c_int, P(C.c_double), P(i64)]),
     }
     for name, (res, args) in sig.items():
@@ -139,13 +142,17 @@ class DevArray:
 
 
 class Context:
-    def __init__(self, device=0):
-        h = C.c_void_p()
-        _check(lib().scn_ctx_create(device, C.byref(h)))
-        self.h = h.value
+    def __init__(self, device=0, handle=None):
+        """A new context, or a view of one owned elsewhere (handle)."""
+        self.owned = handle is None
+        if handle is None:
+            h = C.c_void_p()
+            _check(lib().scn_ctx_create(device, C.byref(h)))
+            handle = h.value
+        self.h = handle
 
     def close(self):
-        if getattr(self, "h", None):
+        if getattr(self, "h", None) and self.owned:
             lib().scn_ctx_destroy(self.h)
             self.h = None
 
@@ -182,6 +189,16 @@ class Context:
             _check(lib().scn_prof_read(self.h, i, C.byref(ms), C.byref(calls)))
             out[name] = (ms.value, calls.value)
         return out
+
+    def prof_spans(self, capacity=1 << 16):
+        """[(family name, tag, ms)] of every span since the last read."""
+        fam = np.empty(capacity, np.int32)
+        tag = np.empty(capacity, np.int32)
+        ms = np.empty(capacity, np.float64)
+        n = C.c_int32()
+        vp = lambda a: a.ctypes.data_as(C.c_void_p)
+        _check(lib().scn_prof_spans(self.h, capacity, vp(fam), vp(tag), vp(ms), C.byref(n)))
+        return [(KERNEL_FAMILIES[fam[i]], int(tag[i]), float(ms[i])) for i in range(n.value)]
 
     # ---- feature kernels
     def gather_rows(self, d_in, d_out, d_rules, count, nIn):

@@ -35,6 +35,7 @@ void scn_set_error(const char *fmt, ...);
 
 struct ProfSpan {
   int family;
+  int tag;
   hipEvent_t a, b;
 };
 
@@ -47,6 +48,7 @@ struct scn_ctx {
   int64_t *d_scalars; // 16 int64
   // profiling
   bool prof;
+  int profTag;
   std::vector<ProfSpan> spans;
   std::vector<hipEvent_t> freeEvents;
   double profMs[SCN_K_COUNT];

@@ -27,6 +27,7 @@ extern "C" int scn_ctx_create(int device, scn_ctx **out) {
   scn_ctx *c = new scn_ctx();
   c->device = device;
   c->prof = false;
+  c->profTag = 0;
   memset(c->profMs, 0, sizeof(c->profMs));
   memset(c->profCalls, 0, sizeof(c->profCalls));
   hipDeviceProp_t prop;
@@ -100,6 +101,15 @@ extern "C" int scn_d2h(scn_ctx *c, void *h_dst, const void *d_src,
   return SCN_OK;
 }
 
+extern "C" int scn_d2d(scn_ctx *c, void *d_dst, const void *d_src,
+                       size_t bytes) {
+  if (bytes == 0)
+    return SCN_OK;
+  SCN_HIP_CHECK(
+      hipMemcpyAsync(d_dst, d_src, bytes, hipMemcpyDeviceToDevice, c->stream));
+  return SCN_OK;
+}
+
 __global__ void k_fill32(uint32_t *dst, uint32_t w, size_t n) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   size_t step = (size_t)gridDim.x * blockDim.x;
@@ -138,6 +148,7 @@ ProfScope::ProfScope(scn_ctx *c, int family) : ctx(c), idx(-1) {
     return;
   ProfSpan s;
   s.family = family;
+  s.tag = c->profTag;
   s.a = take_event(c);
   s.b = take_event(c);
   (void)hipEventRecord(s.a, c->stream);
@@ -150,18 +161,42 @@ ProfScope::~ProfScope() {
     (void)hipEventRecord(ctx->spans[idx].b, ctx->stream);
 }
 
-static void drain_spans(scn_ctx *c) {
+static void drain_spans(scn_ctx *c, int capacity = 0, int32_t *family = nullptr,
+                        int32_t *tag = nullptr, double *msOut = nullptr,
+                        int32_t *n = nullptr) {
   (void)hipStreamSynchronize(c->stream);
+  int kept = 0;
   for (auto &s : c->spans) {
     float ms = 0.f;
     if (hipEventElapsedTime(&ms, s.a, s.b) == hipSuccess) {
       c->profMs[s.family] += ms;
       c->profCalls[s.family] += 1;
+      if (kept < capacity) {
+        family[kept] = s.family;
+        tag[kept] = s.tag;
+        msOut[kept] = ms;
+        ++kept;
+      }
     }
     c->freeEvents.push_back(s.a);
     c->freeEvents.push_back(s.b);
   }
   c->spans.clear();
+  if (n)
+    *n = kept;
+}
+
+extern "C" int scn_prof_tag(scn_ctx *c, int tag) {
+  c->profTag = tag;
+  return SCN_OK;
+}
+
+extern "C" int scn_prof_spans(scn_ctx *c, int capacity, int32_t *family,
+                              int32_t *tag, double *ms, int32_t *n) {
+  SCN_REQUIRE(capacity >= 0 && n && (capacity == 0 || (family && tag && ms)),
+              SCN_ERR_ARG, "scn_prof_spans: null output");
+  drain_spans(c, capacity, family, tag, ms, n);
+  return SCN_OK;
 }
 
 extern "C" int scn_prof_enable(scn_ctx *c, int on) {

@@ -1,0 +1,76 @@
+// The net runtime behind the SparseConvNet facade: layer list, layer builders,
+// per-batch forward driver, weight files (SparseConvNetCUDA.h:25-114).  The
+// class keeps the reference's name; the device code underneath is HIP.
+#pragma once
+#include <fstream>
+#include <iostream>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+#include "SpatiallySparseBatch.h"
+#include "SpatiallySparseDataset.h"
+#include "SpatiallySparseLayer.h"
+
+#define N_MAX_BATCH_PRODUCER_THREADS 20
+
+class SparseConvNetCUDA {
+public:
+  cudaMemStream memStream; // first member: the context outlives every buffer
+  std::vector<SpatiallySparseLayer *> layers;
+  std::vector<float> inputNormalizingConstants;
+  int dimension;
+  int nClasses;
+  int nTop;
+  int inputSpatialSize;
+  int nInputFeatures;
+  int nOutputFeatures;
+  int deviceID;
+  int nBatchProducerThreads;
+  std::mutex batchLock[N_MAX_BATCH_PRODUCER_THREADS];
+  std::vector<SpatiallySparseBatch> batchPool;
+  std::vector<SpatiallySparseBatchSubInterface *> initialSubInterfaces;
+  std::vector<SpatiallySparseBatchSubInterface *> sharedSubInterfaces;
+  SparseConvNetCUDA(int dimension, int nInputFeatures, int nClasses,
+                    int pciBusID = -1, int nTop = 1,
+                    int nBatchProducerThreads = 10);
+  ~SparseConvNetCUDA();
+  void processBatch(SpatiallySparseBatch &batch, float learningRate,
+                    float momentum, std::ofstream &f, std::ofstream &g);
+  void addLearntLayer(int nFeatures, ActivationFunction activationFn = RELU,
+                      float dropout = 0.0f, float alpha = 1.0f);
+  void addNetworkInNetworkLayer(int nFeatures,
+                                ActivationFunction activationFn = RELU,
+                                float dropout = 0.0f);
+  void addConvolutionalLayer(int nFeatures, int filterSize, int filterStride,
+                             ActivationFunction activationFn = RELU,
+                             float dropout = 0.0f, int minActiveInputs = 1,
+                             float poolingToFollow = 1.0f);
+  void addLeNetLayerMP(int nFeatures, int filterSize, int filterStride,
+                       int poolSize, int poolStride,
+                       ActivationFunction activationFn = RELU,
+                       float dropout = 0.0f, int minActiveInputs = 1);
+  void addTriangularConvolutionalLayer(int nFeatures, int filterSize,
+                                       int filterStride,
+                                       ActivationFunction activationFn = RELU,
+                                       float dropout = 0.0f,
+                                       int minActiveInputs = 1,
+                                       float poolingToFollow = 1.0f);
+  void addTriangularLeNetLayerMP(int nFeatures, int filterSize,
+                                 int filterStride, int poolSize, int poolStride,
+                                 ActivationFunction activationFn = RELU,
+                                 float dropout = 0.0f, int minActiveInputs = 1);
+  void addSoftmaxLayer();
+  void addTerminalPoolingLayer(int poolSize, int S);
+  float processDataset(SpatiallySparseDataset &dataset, int batchSize = 100,
+                       float learningRate = 0, float momentum = 0.99);
+  void processDatasetRepeatTest(SpatiallySparseDataset &dataset,
+                                int batchSize = 100, int nReps = 12,
+                                std::string predictionsFilename = "",
+                                std::string confusionMatrixFilename = "");
+  void loadWeights(std::string baseName, int epoch, bool momentum,
+                   int firstNlayers = 1000000);
+  void saveWeights(std::string baseName, int epoch, bool momentum);
+  // set the operand precision of every NiN contraction (SCN_FP32 / SCN_BF16)
+  void setPrecision(int precision);
+};

@@ -1,0 +1,39 @@
+// Data carried between layers (SpatiallySparseBatchInterface.h:8-46).
+#pragma once
+#include <vector>
+#include "SparseGrid.h"
+#include "vectorCUDA.h"
+
+// The large vectors of one depth; they stay in HBM and are shared by every
+// batch slot (BatchProducer.cu:28-33).
+class SpatiallySparseBatchSubInterface {
+public:
+  vectorCUDA<float> features;
+  vectorCUDA<float> dfeatures; // backward pass only; never filled here
+  vectorCUDA<int> poolingChoices;
+  SpatiallySparseBatchSubInterface();
+  void reset();
+};
+
+class SpatiallySparseBatchInterface {
+public:
+  SpatiallySparseBatchSubInterface *sub;
+  int nFeatures;                   // features per spatial location
+  vectorCUDA<int> featuresPresent; // identity at test time
+  int nSpatialSites; // active rows of the whole batch, background rows included
+  int spatialSize;
+  bool backpropErrors;
+  // Host view of the sparse grids.  Filled by the Pictures for the input
+  // interface; for deeper interfaces the grids are built in HBM
+  // (deviceGrids) and this view is only materialised by downloadGrids().
+  std::vector<SparseGrid> grids;
+  scn_grids *deviceGrids;
+  bool ownsDeviceGrids;
+  vectorCUDA<int> rules;
+  SpatiallySparseBatchInterface(SpatiallySparseBatchSubInterface *s);
+  SpatiallySparseBatchInterface(SpatiallySparseBatchInterface &&o);
+  ~SpatiallySparseBatchInterface();
+  void downloadGrids(int batchSize);
+  void summary();
+  void reset();
+};

@@ -1,0 +1,223 @@
+// The layer interface and every layer class of the forward path.
+//
+// preprocess() builds the output interface's grids and rule book, forwards()
+// runs the feature kernels (SpatiallySparseLayer.h:6-27).  In the reference
+// preprocess() is CPU code run by batch-producer threads; here it issues the
+// rule-book kernels on the GPU.  The backward pass is outside this library:
+// backwards() exists so that subclasses written against the reference still
+// compile, and reports an error when called.
+#pragma once
+#include <fstream>
+#include <iostream>
+#include "Rng.h"
+#include "SpatiallySparseBatch.h"
+#include "SpatiallySparseBatchInterface.h"
+
+class SpatiallySparseLayer {
+public:
+  cudaMemStream &memStream;
+  virtual void preprocess(SpatiallySparseBatch &batch,
+                          SpatiallySparseBatchInterface &input,
+                          SpatiallySparseBatchInterface &output) = 0;
+  virtual void forwards(SpatiallySparseBatch &batch,
+                        SpatiallySparseBatchInterface &input,
+                        SpatiallySparseBatchInterface &output) = 0;
+  virtual void scaleWeights(SpatiallySparseBatchInterface &input,
+                            SpatiallySparseBatchInterface &output,
+                            float &scalingUnderneath, bool topLayer);
+  virtual void backwards(SpatiallySparseBatch &batch,
+                         SpatiallySparseBatchInterface &input,
+                         SpatiallySparseBatchInterface &output,
+                         float learningRate, float momentum);
+  SpatiallySparseLayer(cudaMemStream &memStream);
+  virtual ~SpatiallySparseLayer();
+  virtual void loadWeightsFromStream(std::ifstream &f, bool momentum);
+  virtual void putWeightsToStream(std::ofstream &f, bool momentum);
+  virtual int calculateInputSpatialSize(int outputSpatialSize) = 0;
+};
+
+// ConvolutionalLayer.h:3-33 -- gathers each output site's receptive field
+// into one row of the matrix the following NiN layer multiplies.
+class ConvolutionalLayer : public SpatiallySparseLayer {
+private:
+  int fs;
+
+public:
+  int inSpatialSize;
+  int outSpatialSize;
+  int filterSize;
+  int filterStride;
+  int dimension;
+  int nFeaturesIn;
+  int nFeaturesOut;
+  int minActiveInputs; // 1; > 1; or -1 for 'valid' mode
+  ConvolutionalLayer(cudaMemStream &memStream, int filterSize,
+                     int filterStride, int dimension, int nFeaturesIn,
+                     int minActiveInputs = 1);
+  void preprocess(SpatiallySparseBatch &batch,
+                  SpatiallySparseBatchInterface &input,
+                  SpatiallySparseBatchInterface &output);
+  void forwards(SpatiallySparseBatch &batch,
+                SpatiallySparseBatchInterface &input,
+                SpatiallySparseBatchInterface &output);
+  int calculateInputSpatialSize(int outputSpatialSize);
+};
+
+// ConvolutionalTriangularLayer.h
+class ConvolutionalTriangularLayer : public SpatiallySparseLayer {
+private:
+  int fs;
+
+public:
+  int inSpatialSize;
+  int outSpatialSize;
+  int filterSize;
+  int filterStride;
+  int dimension;
+  int nFeaturesIn;
+  int nFeaturesOut;
+  int minActiveInputs;
+  ConvolutionalTriangularLayer(cudaMemStream &memStream, int filterSize,
+                               int filterStride, int dimension,
+                               int nFeaturesIn, int minActiveInputs = 1);
+  void preprocess(SpatiallySparseBatch &batch,
+                  SpatiallySparseBatchInterface &input,
+                  SpatiallySparseBatchInterface &output);
+  void forwards(SpatiallySparseBatch &batch,
+                SpatiallySparseBatchInterface &input,
+                SpatiallySparseBatchInterface &output);
+  int calculateInputSpatialSize(int outputSpatialSize);
+};
+
+// NetworkInNetworkLayer.h:5-49 -- W [nFeaturesIn x nFeaturesOut] row-major,
+// B [nFeaturesOut]; public so that a harness can set them.
+class NetworkInNetworkLayer : public SpatiallySparseLayer {
+private:
+  RNG rng;
+
+public:
+  vectorCUDA<float> W;
+  vectorCUDA<float> MW; // momentum: read and written by the weight files only
+  vectorCUDA<float> B;
+  vectorCUDA<float> MB;
+  ActivationFunction fn;
+  int nFeaturesIn;
+  int nFeaturesOut;
+  float dropout;
+  int precision; // SCN_FP32 or SCN_BF16 operands for the contraction
+  NetworkInNetworkLayer(cudaMemStream &memStream, int nFeaturesIn,
+                        int nFeaturesOut, float dropout = 0,
+                        ActivationFunction fn = NOSIGMOID, float alpha = 1);
+  void preprocess(SpatiallySparseBatch &batch,
+                  SpatiallySparseBatchInterface &input,
+                  SpatiallySparseBatchInterface &output);
+  void forwards(SpatiallySparseBatch &batch,
+                SpatiallySparseBatchInterface &input,
+                SpatiallySparseBatchInterface &output);
+  void loadWeightsFromStream(std::ifstream &f, bool momentum);
+  void putWeightsToStream(std::ofstream &f, bool momentum);
+  int calculateInputSpatialSize(int outputSpatialSize);
+};
+
+// NetworkInNetworkPReLULayer.h
+class NetworkInNetworkPReLULayer : public SpatiallySparseLayer {
+private:
+  RNG rng;
+
+public:
+  vectorCUDA<float> W;
+  vectorCUDA<float> MW;
+  vectorCUDA<float> B;
+  vectorCUDA<float> MB;
+  vectorCUDA<float> PReLU; // per-channel slope, initialised to 0.25
+  vectorCUDA<float> MPReLU;
+  int nFeaturesIn;
+  int nFeaturesOut;
+  float dropout;
+  int precision;
+  NetworkInNetworkPReLULayer(cudaMemStream &memStream, int nFeaturesIn,
+                             int nFeaturesOut, float dropout = 0,
+                             float alpha = 1);
+  void preprocess(SpatiallySparseBatch &batch,
+                  SpatiallySparseBatchInterface &input,
+                  SpatiallySparseBatchInterface &output);
+  void forwards(SpatiallySparseBatch &batch,
+                SpatiallySparseBatchInterface &input,
+                SpatiallySparseBatchInterface &output);
+  void loadWeightsFromStream(std::ifstream &f, bool momentum);
+  void putWeightsToStream(std::ofstream &f, bool momentum);
+  int calculateInputSpatialSize(int outputSpatialSize);
+};
+
+// MaxPoolingLayer.h:11-31
+class MaxPoolingLayer : public SpatiallySparseLayer {
+public:
+  int inSpatialSize;
+  int outSpatialSize;
+  int poolSize;
+  int poolStride;
+  int dimension;
+  int sd;
+  MaxPoolingLayer(cudaMemStream &memStream, int poolSize, int poolStride,
+                  int dimension);
+  void preprocess(SpatiallySparseBatch &batch,
+                  SpatiallySparseBatchInterface &input,
+                  SpatiallySparseBatchInterface &output);
+  void forwards(SpatiallySparseBatch &batch,
+                SpatiallySparseBatchInterface &input,
+                SpatiallySparseBatchInterface &output);
+  int calculateInputSpatialSize(int outputSpatialSize);
+};
+
+// MaxPoolingTriangularLayer.h
+class MaxPoolingTriangularLayer : public SpatiallySparseLayer {
+public:
+  int inSpatialSize;
+  int outSpatialSize;
+  int poolSize;
+  int poolStride;
+  int dimension;
+  int S;
+  MaxPoolingTriangularLayer(cudaMemStream &memStream, int poolSize,
+                            int poolStride, int dimension);
+  void preprocess(SpatiallySparseBatch &batch,
+                  SpatiallySparseBatchInterface &input,
+                  SpatiallySparseBatchInterface &output);
+  void forwards(SpatiallySparseBatch &batch,
+                SpatiallySparseBatchInterface &input,
+                SpatiallySparseBatchInterface &output);
+  int calculateInputSpatialSize(int outputSpatialSize);
+};
+
+// TerminalPoolingLayer.h:5-25 -- averages every active site of a sample.
+class TerminalPoolingLayer : public SpatiallySparseLayer {
+public:
+  int inSpatialSize;  // == poolSize
+  int outSpatialSize; // 1
+  int poolSize;
+  int S; // only printed; the rule width is the batch's largest site count
+  TerminalPoolingLayer(cudaMemStream &memStream, int poolSize, int S);
+  void preprocess(SpatiallySparseBatch &batch,
+                  SpatiallySparseBatchInterface &input,
+                  SpatiallySparseBatchInterface &output);
+  void forwards(SpatiallySparseBatch &batch,
+                SpatiallySparseBatchInterface &input,
+                SpatiallySparseBatchInterface &output);
+  int calculateInputSpatialSize(int outputSpatialSize);
+};
+
+// SoftmaxClassifier.h:10-12 -- copies the class probabilities to the host,
+// takes the top nTop classes per sample, counts mistakes and adds up the
+// negative log-likelihood.
+void SoftmaxClassifier(SpatiallySparseBatchInterface &input,
+                       SpatiallySparseBatch &batch, int nTop,
+                       cudaMemStream &memStream);
+
+// utilities.h
+int ipow(int base, int exp);
+int triangleSize(int linearSize, int dimension);
+int intRound(int a, int d);
+int intRoundUp(int a, int d);
+std::vector<int> range(int n);
+template <typename t>
+std::vector<int> vectorTopIndices(std::vector<t> &test, int k);

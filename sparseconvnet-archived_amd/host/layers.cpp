@@ -1,0 +1,516 @@
+// Layer classes of the forward path.  preprocess() issues the rule-book
+// kernels, forwards() the feature kernels, all through the C ABI of
+// libscn_hip.so on the net's stream.
+#include <cassert>
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include "SpatiallySparseLayer.h"
+
+static void unsupported(const char *what) {
+  std::fprintf(stderr, "%s is outside the forward path of this library\n", what);
+  std::exit(EXIT_FAILURE);
+}
+
+SpatiallySparseLayer::SpatiallySparseLayer(cudaMemStream &memStream)
+    : memStream(memStream) {}
+SpatiallySparseLayer::~SpatiallySparseLayer() {}
+void SpatiallySparseLayer::loadWeightsFromStream(std::ifstream &, bool) {}
+void SpatiallySparseLayer::putWeightsToStream(std::ofstream &, bool) {}
+void SpatiallySparseLayer::scaleWeights(SpatiallySparseBatchInterface &,
+                                        SpatiallySparseBatchInterface &,
+                                        float &, bool) {}
+void SpatiallySparseLayer::backwards(SpatiallySparseBatch &,
+                                     SpatiallySparseBatchInterface &,
+                                     SpatiallySparseBatchInterface &, float,
+                                     float) {
+  unsupported("backwards()");
+}
+
+// the output interface's own grids object, created on first use and kept for
+// later batches (its tables only grow)
+static scn_grids *own_grids(cudaMemStream &ms,
+                            SpatiallySparseBatchInterface &output) {
+  if (!output.deviceGrids || !output.ownsDeviceGrids) {
+    scn_grids *g = nullptr;
+    SCN_CHECKED(scn_grids_create(ms.ctx, &g));
+    output.deviceGrids = g;
+    output.ownsDeviceGrids = true;
+  }
+  return output.deviceGrids;
+}
+// a layer that leaves the grids alone passes its input's object on
+// (NetworkInNetworkLayer.cu:152: output.grids = input.grids)
+static void share_grids(SpatiallySparseBatchInterface &input,
+                        SpatiallySparseBatchInterface &output) {
+  if (output.deviceGrids && output.ownsDeviceGrids)
+    scn_grids_destroy(scnDefaultContext(), output.deviceGrids);
+  output.deviceGrids = input.deviceGrids;
+  output.ownsDeviceGrids = false;
+}
+
+static void fill_rules(cudaMemStream &ms, SpatiallySparseBatchInterface &input,
+                       SpatiallySparseBatchInterface &output, int64_t nRules) {
+  output.rules.copyToGPU();
+  output.rules.resize64((size_t)nRules);
+  SCN_CHECKED(scn_rules_fill(ms.ctx, input.deviceGrids, output.deviceGrids,
+                             output.rules.dPtr(), nRules));
+}
+
+// featuresPresent of a convolution's output: fs copies of the input's list,
+// shifted by nf per copy (ConvolutionalLayer.cu:74-80)
+static void convolutionFeaturesPresent(std::vector<int> &src,
+                                       std::vector<int> &dest, int nf, int nfp,
+                                       int nCopies) {
+  dest.resize((size_t)nfp * nCopies);
+  for (int i = 0; i < nfp * nCopies; ++i)
+    dest[i] = src[i % nfp] + nf * (i / nfp);
+}
+
+// ---- ConvolutionalLayer (ConvolutionalLayer.cu:82-156) ------------------------
+ConvolutionalLayer::ConvolutionalLayer(cudaMemStream &memStream,
+                                       int filterSize, int filterStride,
+                                       int dimension, int nFeaturesIn,
+                                       int minActiveInputs)
+    : SpatiallySparseLayer(memStream), inSpatialSize(0), outSpatialSize(0),
+      filterSize(filterSize), filterStride(filterStride), dimension(dimension),
+      nFeaturesIn(nFeaturesIn), minActiveInputs(minActiveInputs) {
+  fs = ipow(filterSize, dimension);
+  nFeaturesOut = fs * nFeaturesIn;
+  std::cout << "Convolution " << filterSize << "^" << dimension << "x"
+            << nFeaturesIn << "->" << nFeaturesOut;
+  if (filterStride != 1)
+    std::cout << " stride:" << filterStride;
+  if (minActiveInputs != 1)
+    std::cout << " minActiveInputs:" << minActiveInputs;
+  std::cout << std::endl;
+}
+void ConvolutionalLayer::preprocess(SpatiallySparseBatch &batch,
+                                    SpatiallySparseBatchInterface &input,
+                                    SpatiallySparseBatchInterface &output) {
+  (void)batch;
+  assert(input.nFeatures == nFeaturesIn);
+  assert(input.spatialSize >= filterSize);
+  assert((input.spatialSize - filterSize) % filterStride == 0);
+  output.nFeatures = nFeaturesOut;
+  output.spatialSize = (input.spatialSize - filterSize) / filterStride + 1;
+  output.backpropErrors = input.backpropErrors;
+  int64_t n = 0;
+  SCN_CHECKED(scn_rules_square_plan(memStream.ctx, input.deviceGrids,
+                                    own_grids(memStream, output),
+                                    inSpatialSize, outSpatialSize, filterSize,
+                                    filterStride, minActiveInputs, &n));
+  output.nSpatialSites = (int)n;
+  fill_rules(memStream, input, output, n * fs);
+  convolutionFeaturesPresent(input.featuresPresent.hVector(),
+                             output.featuresPresent.hVector(), input.nFeatures,
+                             (int)input.featuresPresent.size(), fs);
+}
+void ConvolutionalLayer::forwards(SpatiallySparseBatch &batch,
+                                  SpatiallySparseBatchInterface &input,
+                                  SpatiallySparseBatchInterface &output) {
+  (void)batch;
+  const size_t nIn = input.featuresPresent.size();
+  output.sub->features.resize64((size_t)output.nSpatialSites * nIn * fs);
+  SCN_CHECKED(scn_gather_rows(memStream.ctx, input.sub->features.dPtr(),
+                              output.sub->features.dPtr(), output.rules.dPtr(),
+                              (int64_t)output.nSpatialSites * fs, (int)nIn));
+}
+int ConvolutionalLayer::calculateInputSpatialSize(int outputSpatialSize) {
+  outSpatialSize = outputSpatialSize;
+  inSpatialSize = filterSize + (outputSpatialSize - 1) * filterStride;
+  std::cout << "-(C" << filterSize;
+  if (filterStride != 1)
+    std::cout << "/" << filterStride;
+  std::cout << ")-" << inSpatialSize;
+  return inSpatialSize;
+}
+
+// ---- ConvolutionalTriangularLayer (ConvolutionalTriangularLayer.cu) -----------
+ConvolutionalTriangularLayer::ConvolutionalTriangularLayer(
+    cudaMemStream &memStream, int filterSize, int filterStride, int dimension,
+    int nFeaturesIn, int minActiveInputs)
+    : SpatiallySparseLayer(memStream), inSpatialSize(0), outSpatialSize(0),
+      filterSize(filterSize), filterStride(filterStride), dimension(dimension),
+      nFeaturesIn(nFeaturesIn), minActiveInputs(minActiveInputs) {
+  fs = triangleSize(filterSize, dimension);
+  nFeaturesOut = fs * nFeaturesIn;
+  std::cout << dimension
+            << "D ConvolutionalTriangularLayer side-length=" << filterSize
+            << " " << nFeaturesIn << "x" << fs << "->" << nFeaturesOut;
+  if (filterStride > 1)
+    std::cout << ", stride " << filterStride;
+  std::cout << std::endl;
+}
+void ConvolutionalTriangularLayer::preprocess(
+    SpatiallySparseBatch &batch, SpatiallySparseBatchInterface &input,
+    SpatiallySparseBatchInterface &output) {
+  (void)batch;
+  assert(input.nFeatures == nFeaturesIn);
+  assert(input.spatialSize >= filterSize);
+  assert((input.spatialSize - filterSize) % filterStride == 0);
+  output.nFeatures = nFeaturesOut;
+  output.spatialSize = (input.spatialSize - filterSize) / filterStride + 1;
+  output.backpropErrors = input.backpropErrors;
+  int64_t n = 0;
+  SCN_CHECKED(scn_rules_triangular_plan(
+      memStream.ctx, input.deviceGrids, own_grids(memStream, output),
+      inSpatialSize, outSpatialSize, filterSize, filterStride, minActiveInputs,
+      &n));
+  output.nSpatialSites = (int)n;
+  fill_rules(memStream, input, output, n * fs);
+  convolutionFeaturesPresent(input.featuresPresent.hVector(),
+                             output.featuresPresent.hVector(), input.nFeatures,
+                             (int)input.featuresPresent.size(), fs);
+}
+void ConvolutionalTriangularLayer::forwards(
+    SpatiallySparseBatch &batch, SpatiallySparseBatchInterface &input,
+    SpatiallySparseBatchInterface &output) {
+  (void)batch;
+  const size_t nIn = input.featuresPresent.size();
+  output.sub->features.resize64((size_t)output.nSpatialSites * nIn * fs);
+  SCN_CHECKED(scn_gather_rows(memStream.ctx, input.sub->features.dPtr(),
+                              output.sub->features.dPtr(), output.rules.dPtr(),
+                              (int64_t)output.nSpatialSites * fs, (int)nIn));
+}
+int ConvolutionalTriangularLayer::calculateInputSpatialSize(
+    int outputSpatialSize) {
+  outSpatialSize = outputSpatialSize;
+  inSpatialSize = filterSize + (outputSpatialSize - 1) * filterStride;
+  std::cout << "-(C" << filterSize;
+  if (filterStride != 1)
+    std::cout << "/" << filterStride;
+  std::cout << ")-" << inSpatialSize;
+  return inSpatialSize;
+}
+
+// ---- NetworkInNetworkLayer (NetworkInNetworkLayer.cu:125-202,290-331) ---------
+static void nin_preprocess(int nFeaturesIn, int nFeaturesOut,
+                           SpatiallySparseBatchInterface &input,
+                           SpatiallySparseBatchInterface &output) {
+  assert(input.nFeatures == nFeaturesIn);
+  (void)nFeaturesIn;
+  output.nFeatures = nFeaturesOut;
+  output.spatialSize = input.spatialSize;
+  output.nSpatialSites = input.nSpatialSites;
+  share_grids(input, output);
+  // no dropout outside training: every output feature is present
+  output.featuresPresent.hVector() = range(nFeaturesOut);
+  output.backpropErrors = true;
+}
+static void read_floats(std::ifstream &f, vectorCUDA<float> &v) {
+  std::vector<float> &h = v.hVector();
+  f.read((char *)h.data(), sizeof(float) * h.size());
+  v.copyToGPU();
+}
+static void write_floats(std::ofstream &f, vectorCUDA<float> &v) {
+  std::vector<float> &h = v.hVector();
+  f.write((char *)h.data(), sizeof(float) * h.size());
+  v.copyToGPU();
+}
+
+NetworkInNetworkLayer::NetworkInNetworkLayer(cudaMemStream &memStream,
+                                             int nFeaturesIn, int nFeaturesOut,
+                                             float dropout,
+                                             ActivationFunction fn,
+                                             float alpha)
+    : SpatiallySparseLayer(memStream),
+      W(true, (size_t)nFeaturesIn * nFeaturesOut),
+      MW(true, (size_t)nFeaturesIn * nFeaturesOut), B(true, nFeaturesOut),
+      MB(true, nFeaturesOut), fn(fn), nFeaturesIn(nFeaturesIn),
+      nFeaturesOut(nFeaturesOut), dropout(dropout), precision(SCN_FP32) {
+  if (fn == TANH || fn == SIGMOID)
+    unsupported("the tanh / logistic activation");
+  float scale = std::pow(6.0f / (nFeaturesIn + nFeaturesOut * alpha), 0.5f);
+  W.setUniform(-scale, scale);
+  MW.setZero();
+  B.setZero();
+  MB.setZero();
+  std::cout << "Learn " << nFeaturesIn << "->" << nFeaturesOut
+            << " dropout=" << dropout << " " << sigmoidNames[fn] << std::endl;
+}
+void NetworkInNetworkLayer::preprocess(SpatiallySparseBatch &batch,
+                                       SpatiallySparseBatchInterface &input,
+                                       SpatiallySparseBatchInterface &output) {
+  if (batch.type == TRAINBATCH)
+    unsupported("a TRAINBATCH (dropout and the backward pass)");
+  nin_preprocess(nFeaturesIn, nFeaturesOut, input, output);
+}
+void NetworkInNetworkLayer::forwards(SpatiallySparseBatch &batch,
+                                     SpatiallySparseBatchInterface &input,
+                                     SpatiallySparseBatchInterface &output) {
+  output.sub->features.resize64((size_t)output.nSpatialSites * nFeaturesOut);
+  // test-time scaling by the kept fraction (NetworkInNetworkLayer.cu:188)
+  float p = 1.0f - (batch.type != RESCALEBATCH ? dropout : 0.0f);
+  SCN_CHECKED(scn_nin_forward(memStream.ctx, input.sub->features.dPtr(),
+                              W.dPtr(), B.dPtr(), nullptr,
+                              output.sub->features.dPtr(),
+                              output.nSpatialSites, nFeaturesIn, nFeaturesOut,
+                              p, (int)fn, precision));
+  multiplyAddCount +=
+      (__int128_t)output.nSpatialSites * nFeaturesIn * nFeaturesOut;
+}
+void NetworkInNetworkLayer::loadWeightsFromStream(std::ifstream &f,
+                                                  bool momentum) {
+  read_floats(f, W);
+  read_floats(f, B);
+  if (momentum) {
+    read_floats(f, MW);
+    read_floats(f, MB);
+  } else {
+    MW.setZero();
+    MB.setZero();
+  }
+}
+void NetworkInNetworkLayer::putWeightsToStream(std::ofstream &f,
+                                               bool momentum) {
+  write_floats(f, W);
+  write_floats(f, B);
+  if (momentum) {
+    write_floats(f, MW);
+    write_floats(f, MB);
+  }
+}
+int NetworkInNetworkLayer::calculateInputSpatialSize(int outputSpatialSize) {
+  return outputSpatialSize;
+}
+
+// ---- NetworkInNetworkPReLULayer (NetworkInNetworkPReLULayer.cu:86-335) --------
+NetworkInNetworkPReLULayer::NetworkInNetworkPReLULayer(
+    cudaMemStream &memStream, int nFeaturesIn, int nFeaturesOut, float dropout,
+    float alpha)
+    : SpatiallySparseLayer(memStream),
+      W(true, (size_t)nFeaturesIn * nFeaturesOut),
+      MW(true, (size_t)nFeaturesIn * nFeaturesOut), B(true, nFeaturesOut),
+      MB(true, nFeaturesOut), PReLU(true, nFeaturesOut),
+      MPReLU(true, nFeaturesOut), nFeaturesIn(nFeaturesIn),
+      nFeaturesOut(nFeaturesOut), dropout(dropout), precision(SCN_FP32) {
+  float scale = std::pow(6.0f / (nFeaturesIn + nFeaturesOut * alpha), 0.5f);
+  W.setUniform(-scale, scale);
+  PReLU.setConstant(0.25f); // NetworkInNetworkPReLULayer.cu:6
+  MW.setZero();
+  B.setZero();
+  MB.setZero();
+  MPReLU.setZero();
+  std::cout << "Learn " << nFeaturesIn << "->" << nFeaturesOut
+            << " dropout=" << dropout << " " << sigmoidNames[PRELU]
+            << std::endl;
+}
+void NetworkInNetworkPReLULayer::preprocess(
+    SpatiallySparseBatch &batch, SpatiallySparseBatchInterface &input,
+    SpatiallySparseBatchInterface &output) {
+  if (batch.type == TRAINBATCH)
+    unsupported("a TRAINBATCH (dropout and the backward pass)");
+  nin_preprocess(nFeaturesIn, nFeaturesOut, input, output);
+}
+void NetworkInNetworkPReLULayer::forwards(
+    SpatiallySparseBatch &batch, SpatiallySparseBatchInterface &input,
+    SpatiallySparseBatchInterface &output) {
+  output.sub->features.resize64((size_t)output.nSpatialSites * nFeaturesOut);
+  float p = 1.0f - (batch.type != RESCALEBATCH ? dropout : 0.0f);
+  SCN_CHECKED(scn_nin_forward(memStream.ctx, input.sub->features.dPtr(),
+                              W.dPtr(), B.dPtr(), PReLU.dPtr(),
+                              output.sub->features.dPtr(),
+                              output.nSpatialSites, nFeaturesIn, nFeaturesOut,
+                              p, (int)PRELU, precision));
+  multiplyAddCount +=
+      (__int128_t)output.nSpatialSites * nFeaturesIn * nFeaturesOut;
+}
+void NetworkInNetworkPReLULayer::loadWeightsFromStream(std::ifstream &f,
+                                                       bool momentum) {
+  read_floats(f, W);
+  read_floats(f, B);
+  read_floats(f, PReLU);
+  if (momentum) {
+    read_floats(f, MW);
+    read_floats(f, MB);
+    read_floats(f, MPReLU);
+  } else {
+    MW.setZero();
+    MB.setZero();
+    MPReLU.setZero();
+  }
+}
+void NetworkInNetworkPReLULayer::putWeightsToStream(std::ofstream &f,
+                                                    bool momentum) {
+  write_floats(f, W);
+  write_floats(f, B);
+  write_floats(f, PReLU);
+  if (momentum) {
+    write_floats(f, MW);
+    write_floats(f, MB);
+    write_floats(f, MPReLU);
+  }
+}
+int NetworkInNetworkPReLULayer::calculateInputSpatialSize(
+    int outputSpatialSize) {
+  return outputSpatialSize;
+}
+
+// ---- MaxPoolingLayer (MaxPoolingLayer.cu:97-155) ------------------------------
+MaxPoolingLayer::MaxPoolingLayer(cudaMemStream &memStream, int poolSize,
+                                 int poolStride, int dimension)
+    : SpatiallySparseLayer(memStream), inSpatialSize(0), outSpatialSize(0),
+      poolSize(poolSize), poolStride(poolStride), dimension(dimension) {
+  sd = ipow(poolSize, dimension);
+  std::cout << "MaxPooling " << poolSize << " " << poolStride << std::endl;
+}
+void MaxPoolingLayer::preprocess(SpatiallySparseBatch &batch,
+                                 SpatiallySparseBatchInterface &input,
+                                 SpatiallySparseBatchInterface &output) {
+  (void)batch;
+  assert(input.spatialSize == inSpatialSize);
+  output.nFeatures = input.nFeatures;
+  output.featuresPresent.hVector() = input.featuresPresent.hVector();
+  output.spatialSize = outSpatialSize;
+  output.backpropErrors = input.backpropErrors;
+  int64_t n = 0;
+  SCN_CHECKED(scn_rules_square_plan(memStream.ctx, input.deviceGrids,
+                                    own_grids(memStream, output),
+                                    inSpatialSize, outSpatialSize, poolSize,
+                                    poolStride, 1, &n));
+  output.nSpatialSites = (int)n;
+  fill_rules(memStream, input, output, n * sd);
+}
+static void pool_forwards(cudaMemStream &ms,
+                          SpatiallySparseBatchInterface &input,
+                          SpatiallySparseBatchInterface &output, int width) {
+  const size_t nf = output.featuresPresent.size();
+  output.sub->poolingChoices.resize64((size_t)output.nSpatialSites * nf);
+  output.sub->features.resize64((size_t)output.nSpatialSites * nf);
+  SCN_CHECKED(scn_maxpool(ms.ctx, input.sub->features.dPtr(),
+                          output.sub->features.dPtr(), output.rules.dPtr(),
+                          output.nSpatialSites, width, (int)nf,
+                          output.sub->poolingChoices.dPtr()));
+}
+void MaxPoolingLayer::forwards(SpatiallySparseBatch &batch,
+                               SpatiallySparseBatchInterface &input,
+                               SpatiallySparseBatchInterface &output) {
+  (void)batch;
+  pool_forwards(memStream, input, output, sd);
+}
+int MaxPoolingLayer::calculateInputSpatialSize(int outputSpatialSize) {
+  outSpatialSize = outputSpatialSize;
+  inSpatialSize = poolSize + (outputSpatialSize - 1) * poolStride;
+  std::cout << "-(MP" << poolSize;
+  if (poolStride != poolSize)
+    std::cout << "/" << poolStride;
+  std::cout << ")-" << inSpatialSize;
+  return inSpatialSize;
+}
+
+// ---- MaxPoolingTriangularLayer (MaxPoolingTriangularLayer.cu) -----------------
+MaxPoolingTriangularLayer::MaxPoolingTriangularLayer(cudaMemStream &memStream,
+                                                     int poolSize,
+                                                     int poolStride,
+                                                     int dimension)
+    : SpatiallySparseLayer(memStream), inSpatialSize(0), outSpatialSize(0),
+      poolSize(poolSize), poolStride(poolStride), dimension(dimension) {
+  S = triangleSize(poolSize, dimension);
+  std::cout << dimension
+            << "D MaxPoolingTriangularLayer side-length=" << poolSize
+            << " volume=" << S << " stride " << poolStride << std::endl;
+}
+void MaxPoolingTriangularLayer::preprocess(
+    SpatiallySparseBatch &batch, SpatiallySparseBatchInterface &input,
+    SpatiallySparseBatchInterface &output) {
+  (void)batch;
+  assert(input.spatialSize == inSpatialSize);
+  output.nFeatures = input.nFeatures;
+  output.featuresPresent.hVector() = input.featuresPresent.hVector();
+  output.spatialSize = outSpatialSize;
+  output.backpropErrors = input.backpropErrors;
+  int64_t n = 0;
+  SCN_CHECKED(scn_rules_triangular_plan(
+      memStream.ctx, input.deviceGrids, own_grids(memStream, output),
+      inSpatialSize, outSpatialSize, poolSize, poolStride, 1, &n));
+  output.nSpatialSites = (int)n;
+  fill_rules(memStream, input, output, n * S);
+}
+void MaxPoolingTriangularLayer::forwards(SpatiallySparseBatch &batch,
+                                         SpatiallySparseBatchInterface &input,
+                                         SpatiallySparseBatchInterface &output) {
+  (void)batch;
+  pool_forwards(memStream, input, output, S);
+}
+int MaxPoolingTriangularLayer::calculateInputSpatialSize(
+    int outputSpatialSize) {
+  outSpatialSize = outputSpatialSize;
+  inSpatialSize = poolSize + (outputSpatialSize - 1) * poolStride;
+  std::cout << "-(MP" << poolSize;
+  if (poolStride != poolSize)
+    std::cout << "/" << poolStride;
+  std::cout << ")-" << inSpatialSize;
+  return inSpatialSize;
+}
+
+// ---- TerminalPoolingLayer (TerminalPoolingLayer.cu:75-130) --------------------
+TerminalPoolingLayer::TerminalPoolingLayer(cudaMemStream &memStream,
+                                           int poolSize, int S)
+    : SpatiallySparseLayer(memStream), inSpatialSize(poolSize),
+      outSpatialSize(1), poolSize(poolSize), S(S) {
+  std::cout << "TerminalPooling " << poolSize << " " << S << std::endl;
+}
+void TerminalPoolingLayer::preprocess(SpatiallySparseBatch &batch,
+                                      SpatiallySparseBatchInterface &input,
+                                      SpatiallySparseBatchInterface &output) {
+  assert(input.spatialSize == inSpatialSize);
+  output.nFeatures = input.nFeatures;
+  output.featuresPresent.hVector() = input.featuresPresent.hVector();
+  output.spatialSize = outSpatialSize;
+  output.backpropErrors = input.backpropErrors;
+  int64_t width = 0;
+  SCN_CHECKED(scn_rules_terminal_plan(memStream.ctx, input.deviceGrids,
+                                      own_grids(memStream, output), &width));
+  output.nSpatialSites = batch.batchSize;
+  fill_rules(memStream, input, output, width * batch.batchSize);
+}
+void TerminalPoolingLayer::forwards(SpatiallySparseBatch &batch,
+                                    SpatiallySparseBatchInterface &input,
+                                    SpatiallySparseBatchInterface &output) {
+  const size_t nf = output.featuresPresent.size();
+  output.sub->poolingChoices.resize64((size_t)output.nSpatialSites * nf);
+  output.sub->features.resize64((size_t)output.nSpatialSites * nf);
+  SCN_CHECKED(scn_terminal_pool(
+      memStream.ctx, input.sub->features.dPtr(), output.sub->features.dPtr(),
+      output.rules.dPtr(), output.nSpatialSites,
+      (int)(output.rules.size64() / batch.batchSize), (int)nf));
+}
+int TerminalPoolingLayer::calculateInputSpatialSize(int outputSpatialSize) {
+  assert(outputSpatialSize == 1);
+  (void)outputSpatialSize;
+  std::cout << "-(TP)-" << inSpatialSize;
+  return inSpatialSize;
+}
+
+// ---- SoftmaxClassifier (SoftmaxClassifier.cu:16-58) ---------------------------
+void SoftmaxClassifier(SpatiallySparseBatchInterface &input,
+                       SpatiallySparseBatch &batch, int nTop,
+                       cudaMemStream &memStream) {
+  assert(batch.batchSize == input.nSpatialSites);
+  assert(input.nFeatures == (int)input.featuresPresent.size());
+  if (batch.type == TRAINBATCH)
+    unsupported("a TRAINBATCH (dropout and the backward pass)");
+  const int nClasses = input.nFeatures;
+  std::vector<float> probs((size_t)batch.batchSize * nClasses);
+  SCN_CHECKED(scn_d2h(memStream.ctx, probs.data(),
+                      input.sub->features.dPtr(),
+                      probs.size() * sizeof(float)));
+  for (int i = 0; i < batch.batchSize; ++i)
+    batch.probabilities.push_back(std::vector<float>(
+        probs.begin() + (size_t)i * nClasses,
+        probs.begin() + (size_t)(i + 1) * nClasses));
+  for (int i = 0; i < batch.batchSize; i++)
+    batch.predictions.push_back(vectorTopIndices(batch.probabilities[i], nTop));
+  if (batch.type != UNLABELEDBATCH) {
+    std::vector<int> &labels = batch.labels.hVector();
+    batch.mistakes += batch.batchSize;
+    for (int i = 0; i < batch.batchSize; i++) {
+      double pr = batch.probabilities[i][labels[i]];
+      batch.negativeLogLikelihood -= (float)std::log(std::max(pr, 1.0e-15));
+      for (int j = 0; j < nTop; j++)
+        if (batch.predictions[i][j] == labels[i])
+          batch.mistakes--;
+    }
+  }
+}

@@ -1,0 +1,635 @@
+// Net runtime, batch production, public facades and canned architectures.
+#include <algorithm>
+#include <cassert>
+#include <chrono>
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include "BatchProducer.h"
+#include "NetworkArchitectures.h"
+#include "SparseConvNet.h"
+#include "SparseConvNetCUDA.h"
+
+#define FEATURE_QUANTUM 32 // KERNELBLOCKSIZE of the reference (utilities.h:73)
+
+// ================================================================ runtime
+SparseConvNetCUDA::SparseConvNetCUDA(int dimension, int nInputFeatures,
+                                     int nClasses, int pciBusID, int nTop,
+                                     int nBatchProducerThreads)
+    : dimension(dimension), nClasses(nClasses), nTop(nTop),
+      inputSpatialSize(0), nInputFeatures(nInputFeatures),
+      nOutputFeatures(nInputFeatures), deviceID(0),
+      nBatchProducerThreads(nBatchProducerThreads) {
+  (void)pciBusID; // one GPU per process: the context picks device 0
+  assert(nBatchProducerThreads >= 1 &&
+         nBatchProducerThreads <= N_MAX_BATCH_PRODUCER_THREADS);
+  std::cout << "Sparse CNN - dimension=" << dimension
+            << " nInputFeatures=" << nInputFeatures << " nClasses=" << nClasses
+            << std::endl;
+  batchPool.reserve(nBatchProducerThreads);
+  for (int c = 0; c < nBatchProducerThreads; c++) {
+    initialSubInterfaces.push_back(new SpatiallySparseBatchSubInterface());
+    batchPool.emplace_back(initialSubInterfaces.back());
+  }
+}
+SparseConvNetCUDA::~SparseConvNetCUDA() {
+  memStream.synchronize();
+  batchPool.clear();
+  for (auto p : layers)
+    delete p;
+  for (auto p : initialSubInterfaces)
+    delete p;
+  for (auto p : sharedSubInterfaces)
+    delete p;
+}
+// SparseConvNetCUDA.cu:50-70
+void SparseConvNetCUDA::addLearntLayer(int nFeatures,
+                                       ActivationFunction activationFn,
+                                       float dropout, float alpha) {
+  // every learnt layer but the classifier is rounded to a multiple of 32
+  if (activationFn != SOFTMAX)
+    nFeatures = std::max(FEATURE_QUANTUM, intRound(nFeatures, FEATURE_QUANTUM));
+  if (dropout > 0)
+    dropout = 1 - (intRound(nFeatures * (1 - dropout), FEATURE_QUANTUM) + 0.01f) *
+                      1.0f / nFeatures;
+  if (dropout < 0)
+    dropout = 0;
+  std::cout << layers.size() << ":";
+  if (activationFn == PRELU)
+    layers.push_back(new NetworkInNetworkPReLULayer(
+        memStream, nOutputFeatures, nFeatures, dropout, alpha));
+  else
+    layers.push_back(new NetworkInNetworkLayer(memStream, nOutputFeatures,
+                                               nFeatures, dropout,
+                                               activationFn, alpha));
+  nOutputFeatures = nFeatures;
+}
+void SparseConvNetCUDA::addNetworkInNetworkLayer(
+    int nFeatures, ActivationFunction activationFn, float dropout) {
+  addLearntLayer(nFeatures, activationFn, dropout, 1.0f);
+}
+// SparseConvNetCUDA.cu:75-98: filterSize 1 adds no gather layer
+void SparseConvNetCUDA::addConvolutionalLayer(int nFeatures, int filterSize,
+                                              int filterStride,
+                                              ActivationFunction activationFn,
+                                              float dropout,
+                                              int minActiveInputs,
+                                              float poolingToFollow) {
+  if (filterSize > 1) {
+    std::cout << layers.size() << ":";
+    layers.push_back(new ConvolutionalLayer(memStream, filterSize, filterStride,
+                                            dimension, nOutputFeatures,
+                                            minActiveInputs));
+    nOutputFeatures *= ipow(filterSize, dimension);
+  }
+  addLearntLayer(nFeatures, activationFn, dropout,
+                 powf(filterSize * 1.0 / filterStride / poolingToFollow, 2));
+}
+void SparseConvNetCUDA::addLeNetLayerMP(int nFeatures, int filterSize,
+                                        int filterStride, int poolSize,
+                                        int poolStride,
+                                        ActivationFunction activationFn,
+                                        float dropout, int minActiveInputs) {
+  addConvolutionalLayer(nFeatures, filterSize, filterStride, activationFn,
+                        dropout, minActiveInputs, poolSize);
+  if (poolSize > 1) {
+    std::cout << layers.size() << ":";
+    layers.push_back(
+        new MaxPoolingLayer(memStream, poolSize, poolStride, dimension));
+  }
+}
+void SparseConvNetCUDA::addTriangularConvolutionalLayer(
+    int nFeatures, int filterSize, int filterStride,
+    ActivationFunction activationFn, float dropout, int minActiveInputs,
+    float poolingToFollow) {
+  if (filterSize > 1) {
+    std::cout << layers.size() << ":";
+    layers.push_back(new ConvolutionalTriangularLayer(
+        memStream, filterSize, filterStride, dimension, nOutputFeatures,
+        minActiveInputs));
+    nOutputFeatures *= triangleSize(filterSize, dimension);
+  }
+  addLearntLayer(nFeatures, activationFn, dropout,
+                 powf(filterSize * 1.0 / filterStride / poolingToFollow, 2));
+}
+// The reference hands (.., dropout, poolSize, minActiveInputs) to a callee
+// whose parameters are (.., dropout, minActiveInputs, poolingToFollow)
+// (SparseConvNetCUDA.cu:165-168 against :183-185): through this builder the
+// convolution's minActiveInputs is the pool size.  Kept, because nets built
+// with the reference behave that way.
+void SparseConvNetCUDA::addTriangularLeNetLayerMP(
+    int nFeatures, int filterSize, int filterStride, int poolSize,
+    int poolStride, ActivationFunction activationFn, float dropout,
+    int minActiveInputs) {
+  addTriangularConvolutionalLayer(nFeatures, filterSize, filterStride,
+                                  activationFn, dropout, poolSize,
+                                  minActiveInputs);
+  if (poolSize > 1) {
+    std::cout << layers.size() << ":";
+    layers.push_back(new MaxPoolingTriangularLayer(memStream, poolSize,
+                                                   poolStride, dimension));
+  }
+}
+void SparseConvNetCUDA::addTerminalPoolingLayer(int poolSize, int S) {
+  std::cout << layers.size() << ":";
+  layers.push_back(new TerminalPoolingLayer(memStream, poolSize, S));
+}
+// SparseConvNetCUDA.cu:198-210: classifier, then the spatial sizes are worked
+// out from the top (size 1) down to the input field
+void SparseConvNetCUDA::addSoftmaxLayer() {
+  addLearntLayer(nClasses, SOFTMAX, 0.0f, 1);
+  inputSpatialSize = 1;
+  std::cout << "Spatially sparse CNN with layer sizes: " << inputSpatialSize;
+  for (int i = (int)layers.size() - 1; i >= 0; i--)
+    inputSpatialSize = layers[i]->calculateInputSpatialSize(inputSpatialSize);
+  std::cout << std::endl;
+  std::cout << "Input-field dimensions = " << inputSpatialSize;
+  for (int i = 1; i < dimension; ++i)
+    std::cout << "x" << inputSpatialSize;
+  std::cout << std::endl;
+}
+void SparseConvNetCUDA::setPrecision(int precision) {
+  for (auto *l : layers) {
+    if (auto *n = dynamic_cast<NetworkInNetworkLayer *>(l))
+      n->precision = precision;
+    if (auto *n = dynamic_cast<NetworkInNetworkPReLULayer *>(l))
+      n->precision = precision;
+  }
+}
+// SparseConvNetCUDA.cu:227-271, forward branch
+void SparseConvNetCUDA::processBatch(SpatiallySparseBatch &batch,
+                                     float learningRate, float momentum,
+                                     std::ofstream &f, std::ofstream &g) {
+  (void)learningRate;
+  (void)momentum;
+  for (size_t i = 0; i < layers.size(); i++) {
+    batch.interfaces[i + 1].sub->reset();
+    scn_prof_tag(memStream.ctx, (int)i);
+    layers[i]->forwards(batch, batch.interfaces[i], batch.interfaces[i + 1]);
+  }
+  SoftmaxClassifier(batch.interfaces.back(), batch, nTop, memStream);
+  if (f.is_open())
+    for (auto &p : batch.predictions) {
+      for (size_t k = 0; k < p.size(); k++)
+        f << (k ? " " : "") << p[k];
+      f << std::endl;
+    }
+  if (g.is_open())
+    for (auto &p : batch.probabilities) {
+      for (size_t k = 0; k < p.size(); k++)
+        g << (k ? " " : "") << p[k];
+      g << std::endl;
+    }
+}
+static void printThroughput(long long nanoseconds, size_t nPictures) {
+  std::cout << " MegaMultiplyAdds/sample:"
+            << roundf(multiplyAddCount / nPictures / 1000000)
+            << " time:" << nanoseconds / 1000000000L
+            << "s GigaMultiplyAdds/s:" << roundf(multiplyAddCount / nanoseconds)
+            << " rate:" << roundf(nPictures * 1000000000.0f / nanoseconds)
+            << "/s" << std::endl;
+}
+// SparseConvNetCUDA.cu:272-326
+float SparseConvNetCUDA::processDataset(SpatiallySparseDataset &dataset,
+                                        int batchSize, float learningRate,
+                                        float momentum) {
+  assert(dataset.pictures.size() > 0);
+  if (dataset.type == TRAINBATCH || dataset.type == RESCALEBATCH) {
+    std::fprintf(stderr, "processDataset: %s passes are outside the forward "
+                         "path of this library\n",
+                 batchTypeNames[dataset.type]);
+    std::exit(EXIT_FAILURE);
+  }
+  float errorRate = 0, nll = 0;
+  multiplyAddCount = 0;
+  auto start = std::chrono::system_clock::now();
+  std::ofstream f, g;
+  BatchProducer bp(*this, dataset, inputSpatialSize, batchSize);
+  if (dataset.type == UNLABELEDBATCH) {
+    f.open("unlabelledData.predictions");
+    g.open("unlabelledData.probabilities");
+  }
+  while (SpatiallySparseBatch *batch = bp.nextBatch()) {
+    processBatch(*batch, learningRate, momentum, f, g);
+    errorRate += batch->mistakes * 1.0 / dataset.pictures.size();
+    nll += batch->negativeLogLikelihood * 1.0 / dataset.pictures.size();
+  }
+  auto end = std::chrono::system_clock::now();
+  auto diff =
+      std::chrono::duration_cast<std::chrono::nanoseconds>(end - start).count();
+  std::cout << dataset.name;
+  if (dataset.type != UNLABELEDBATCH)
+    std::cout << " Mistakes:" << 100.0 * errorRate << "% NLL:" << nll;
+  printThroughput(diff, dataset.pictures.size());
+  return nll;
+}
+// SparseConvNetCUDA.cu:327-405: nReps forward passes, probabilities averaged
+void SparseConvNetCUDA::processDatasetRepeatTest(
+    SpatiallySparseDataset &dataset, int batchSize, int nReps,
+    std::string predictionsFilename, std::string confusionMatrixFilename) {
+  assert(dataset.pictures.size() > 0);
+  multiplyAddCount = 0;
+  auto start = std::chrono::system_clock::now();
+  const size_t nPictures = dataset.pictures.size();
+  std::vector<std::vector<int>> votes(nPictures,
+                                      std::vector<int>(dataset.nClasses));
+  std::vector<std::vector<float>> probs(nPictures,
+                                        std::vector<float>(dataset.nClasses));
+  for (int rep = 1; rep <= nReps; ++rep) {
+    {
+      BatchProducer bp(*this, dataset, inputSpatialSize, batchSize);
+      while (SpatiallySparseBatch *batch = bp.nextBatch()) {
+        std::ofstream f, g;
+        processBatch(*batch, 0, 0, f, g);
+        for (int i = 0; i < batch->batchSize; ++i) {
+          int ii = batch->sampleNumbers[i];
+          votes[ii][batch->predictions[i][0]]++;
+          for (int j = 0; j < dataset.nClasses; ++j)
+            probs[ii][j] += batch->probabilities[i][j];
+        }
+      }
+    }
+    int errors = (int)nPictures;
+    float nll = 0;
+    if (dataset.type != UNLABELEDBATCH)
+      for (size_t i = 0; i < nPictures; ++i) {
+        std::vector<int> predictions = vectorTopIndices(probs[i], nTop);
+        for (int j = 0; j < nTop; j++)
+          if (predictions[j] == dataset.pictures[i]->label)
+            errors--;
+        nll -= log(std::max(probs[i][dataset.pictures[i]->label] / rep,
+                            (float)1.0e-15));
+      }
+    if (!predictionsFilename.empty()) {
+      std::cout << predictionsFilename << std::endl;
+      std::ofstream f(predictionsFilename.c_str());
+      if (!dataset.header.empty())
+        f << dataset.header << std::endl;
+      for (size_t i = 0; i < nPictures; ++i) {
+        f << dataset.pictures[i]->identify();
+        if (dataset.type != UNLABELEDBATCH)
+          f << "," << dataset.pictures[i]->label;
+        for (int j = 0; j < dataset.nClasses; ++j)
+          f << "," << probs[i][j] / rep;
+        f << std::endl;
+      }
+    }
+    if (!confusionMatrixFilename.empty() && dataset.type != UNLABELEDBATCH) {
+      std::vector<float> cm((size_t)dataset.nClasses * dataset.nClasses);
+      for (size_t i = 0; i < nPictures; ++i)
+        for (int j = 0; j < dataset.nClasses; ++j)
+          cm[dataset.pictures[i]->label * dataset.nClasses + j] +=
+              probs[i][j] / rep;
+      std::ofstream f(confusionMatrixFilename.c_str());
+      for (int i = 0; i < dataset.nClasses; ++i) {
+        for (int j = 0; j < dataset.nClasses; ++j)
+          f << cm[i * dataset.nClasses + j] << " ";
+        f << std::endl;
+      }
+    }
+    auto end = std::chrono::system_clock::now();
+    auto diff = std::chrono::duration_cast<std::chrono::nanoseconds>(end - start)
+                    .count();
+    std::cout << dataset.name << " rep " << rep << "/" << nReps;
+    if (dataset.type != UNLABELEDBATCH)
+      std::cout << " Mistakes: " << 100.0 * errors / nPictures << "% NLL "
+                << nll / nPictures;
+    printThroughput(diff, nPictures);
+  }
+}
+// raw little-endian fp32, no header (SparseConvNetCUDA.cu:406-442)
+void SparseConvNetCUDA::loadWeights(std::string baseName, int epoch,
+                                    bool momentum, int firstNlayers) {
+  std::string filename = baseName + "_epoch-" + std::to_string(epoch) + ".cnn";
+  std::ifstream f(filename.c_str(), std::ios::in | std::ios::binary);
+  if (!f) {
+    std::cout << "Cannot find " << filename << std::endl;
+    std::exit(EXIT_FAILURE);
+  }
+  std::cout << "Loading network parameters from " << filename << std::endl;
+  for (int i = 0; i < std::min((int)layers.size(), firstNlayers); i++)
+    layers[i]->loadWeightsFromStream(f, momentum);
+  if (inputNormalizingConstants.size() > 0)
+    f.read((char *)&inputNormalizingConstants[0],
+           sizeof(float) * inputNormalizingConstants.size());
+}
+void SparseConvNetCUDA::saveWeights(std::string baseName, int epoch,
+                                    bool momentum) {
+  std::string filename = baseName + "_epoch-" + std::to_string(epoch) + ".cnn";
+  std::ofstream f(filename.c_str(), std::ios::binary);
+  if (!f) {
+    std::cout << "Cannot write " << filename << std::endl;
+    std::exit(EXIT_FAILURE);
+  }
+  for (auto *l : layers)
+    l->putWeightsToStream(f, momentum);
+  if (inputNormalizingConstants.size() > 0)
+    f.write((char *)&inputNormalizingConstants[0],
+            sizeof(float) * inputNormalizingConstants.size());
+}
+
+// ========================================================== batch producer
+BatchProducer::BatchProducer(SparseConvNetCUDA &cnn,
+                             SpatiallySparseDataset &dataset, int spatialSize,
+                             int batchSize)
+    : cnn(cnn), batchCounter(-1), dataset(dataset), batchSize(batchSize),
+      spatialSize(spatialSize), stopping(false) {
+  assert(batchSize > 0);
+  nBatches = ((int)dataset.pictures.size() + batchSize - 1) / batchSize;
+  permutation = range((int)dataset.pictures.size());
+  // one shared sub-interface per depth, one interface per depth and slot
+  while (cnn.batchPool[0].interfaces.size() <= cnn.layers.size()) {
+    cnn.sharedSubInterfaces.push_back(new SpatiallySparseBatchSubInterface());
+    for (int c = 0; c < cnn.nBatchProducerThreads; c++)
+      cnn.batchPool[c].interfaces.emplace_back(cnn.sharedSubInterfaces.back());
+  }
+  slotFull.assign(cnn.nBatchProducerThreads, 0);
+  for (int c = 0; c < cnn.nBatchProducerThreads; c++)
+    cnn.batchPool[c].batchSize = 0;
+  for (int nThread = 0; nThread < cnn.nBatchProducerThreads; ++nThread)
+    workers.emplace_back(&BatchProducer::batchProducerThread, this, nThread);
+}
+BatchProducer::~BatchProducer() {
+  {
+    std::lock_guard<std::mutex> lock(slotMutex);
+    stopping = true;
+  }
+  slotChanged.notify_all();
+  for (auto &w : workers)
+    if (w.joinable())
+      w.join();
+}
+// CPU half of BatchProducer.cu:40-87: distort, codify, normalise
+void BatchProducer::preprocessBatch(int c, int cc, RNG &rng) {
+  SpatiallySparseBatch &b = cnn.batchPool[cc];
+  b.reset();
+  b.type = dataset.type;
+  SpatiallySparseBatchInterface &in = b.interfaces[0];
+  in.nFeatures = dataset.nFeatures;
+  in.spatialSize = spatialSize;
+  in.featuresPresent.hVector() = range(dataset.nFeatures);
+  const int last = std::min((c + 1) * batchSize, (int)dataset.pictures.size());
+  for (int i = c * batchSize; i < last; i++) {
+    Picture *pic = dataset.pictures[permutation[i]]->distort(rng, dataset.type);
+    b.sampleNumbers.push_back(permutation[i]);
+    b.batchSize++;
+    in.grids.push_back(SparseGrid());
+    b.labels.hVector().push_back(pic->label);
+    pic->codifyInputData(in.grids.back(), in.sub->features.hVector(),
+                         in.nSpatialSites, in.spatialSize);
+    if (pic != dataset.pictures[permutation[i]])
+      delete pic;
+  }
+  assert(in.sub->features.size64() ==
+         (size_t)in.nFeatures * (size_t)in.nSpatialSites);
+  if (cnn.inputNormalizingConstants.size() > 0) {
+    std::vector<float> &features = in.sub->features.hVector();
+    for (size_t i = 0; i < features.size(); ++i)
+      features[i] *= cnn.inputNormalizingConstants[i % in.nFeatures];
+  }
+}
+// GPU half: the input grids go to HBM, then every layer builds its rule book
+void BatchProducer::preprocessBatchOnDevice(int cc) {
+  SpatiallySparseBatch &b = cnn.batchPool[cc];
+  SpatiallySparseBatchInterface &in = b.interfaces[0];
+  std::vector<int32_t> sample, row, bg;
+  std::vector<int64_t> key;
+  size_t n = 0;
+  for (auto &g : in.grids)
+    n += g.mp.size();
+  sample.reserve(n);
+  row.reserve(n);
+  key.reserve(n);
+  for (int item = 0; item < b.batchSize; ++item) {
+    bg.push_back(in.grids[item].backgroundCol);
+    for (auto &e : in.grids[item].mp.entries()) {
+      sample.push_back(item);
+      key.push_back(e.first);
+      row.push_back(e.second);
+    }
+  }
+  scn_ctx *ctx = cnn.memStream.ctx;
+  void *d_sample, *d_key, *d_row, *d_bg;
+  SCN_CHECKED(scn_malloc(ctx, n * 4, &d_sample));
+  SCN_CHECKED(scn_malloc(ctx, n * 8, &d_key));
+  SCN_CHECKED(scn_malloc(ctx, n * 4, &d_row));
+  SCN_CHECKED(scn_malloc(ctx, bg.size() * 4, &d_bg));
+  SCN_CHECKED(scn_h2d(ctx, d_sample, sample.data(), n * 4));
+  SCN_CHECKED(scn_h2d(ctx, d_key, key.data(), n * 8));
+  SCN_CHECKED(scn_h2d(ctx, d_row, row.data(), n * 4));
+  SCN_CHECKED(scn_h2d(ctx, d_bg, bg.data(), bg.size() * 4));
+  if (!in.deviceGrids) {
+    SCN_CHECKED(scn_grids_create(ctx, &in.deviceGrids));
+    in.ownsDeviceGrids = true;
+  }
+  scn_prof_tag(ctx, -1);
+  SCN_CHECKED(scn_grids_build(ctx, in.deviceGrids, b.batchSize, cnn.dimension,
+                              in.spatialSize, (const int32_t *)d_sample,
+                              (const int64_t *)d_key, (const int32_t *)d_row,
+                              (int64_t)n, (const int32_t *)d_bg,
+                              in.nSpatialSites));
+  in.sub->features.copyToGPU();
+  for (size_t i = 0; i < cnn.layers.size(); i++) {
+    scn_prof_tag(ctx, (int)i);
+    cnn.layers[i]->preprocess(b, b.interfaces[i], b.interfaces[i + 1]);
+  }
+  SCN_CHECKED(scn_sync(ctx));
+  scn_free(ctx, d_sample);
+  scn_free(ctx, d_key);
+  scn_free(ctx, d_row);
+  scn_free(ctx, d_bg);
+}
+void BatchProducer::batchProducerThread(int nThread) {
+  RNG rng;
+  for (int c = nThread; c < nBatches; c += cnn.nBatchProducerThreads) {
+    {
+      std::unique_lock<std::mutex> lock(slotMutex);
+      slotChanged.wait(lock, [&] { return stopping || !slotFull[nThread]; });
+      if (stopping)
+        return;
+    }
+    {
+      std::lock_guard<std::mutex> slot(cnn.batchLock[nThread]);
+      preprocessBatch(c, nThread, rng);
+    }
+    {
+      std::lock_guard<std::mutex> lock(slotMutex);
+      slotFull[nThread] = 1;
+    }
+    slotChanged.notify_all();
+  }
+}
+SpatiallySparseBatch *BatchProducer::nextBatch() {
+  if (batchCounter >= 0) { // hand the previous slot back to its worker
+    int cc = batchCounter % cnn.nBatchProducerThreads;
+    cnn.batchPool[cc].batchSize = 0;
+    {
+      std::lock_guard<std::mutex> lock(slotMutex);
+      slotFull[cc] = 0;
+    }
+    slotChanged.notify_all();
+  }
+  batchCounter++;
+  if (batchCounter >= nBatches) {
+    for (auto &w : workers)
+      if (w.joinable())
+        w.join();
+    return NULL;
+  }
+  int cc = batchCounter % cnn.nBatchProducerThreads;
+  {
+    std::unique_lock<std::mutex> lock(slotMutex);
+    slotChanged.wait(lock, [&] { return slotFull[cc] != 0; });
+  }
+  std::lock_guard<std::mutex> slot(cnn.batchLock[cc]);
+  preprocessBatchOnDevice(cc);
+  return &cnn.batchPool[cc];
+}
+
+// ================================================================= facades
+SparseConvNet::SparseConvNet(int dimension, int nInputFeatures, int nClasses,
+                             int pciBusID, int nTop)
+    : cnn(new SparseConvNetCUDA(dimension, nInputFeatures, nClasses, pciBusID,
+                                nTop)) {}
+SparseConvNet::~SparseConvNet() {}
+void SparseConvNet::addLeNetLayerMP(int nFeatures, int filterSize,
+                                    int filterStride, int poolSize,
+                                    int poolStride,
+                                    ActivationFunction activationFn,
+                                    float dropout, int minActiveInputs) {
+  cnn->addLeNetLayerMP(nFeatures, filterSize, filterStride, poolSize,
+                       poolStride, activationFn, dropout, minActiveInputs);
+}
+void SparseConvNet::addTerminalPoolingLayer(int poolSize) {
+  cnn->addTerminalPoolingLayer(poolSize, ipow(poolSize, cnn->dimension));
+}
+void SparseConvNet::addSoftmaxLayer() { cnn->addSoftmaxLayer(); }
+float SparseConvNet::processDataset(SpatiallySparseDataset &dataset,
+                                    int batchSize, float learningRate,
+                                    float momentum) {
+  return cnn->processDataset(dataset, batchSize, learningRate, momentum);
+}
+void SparseConvNet::processDatasetRepeatTest(
+    SpatiallySparseDataset &dataset, int batchSize, int nReps,
+    std::string predictionsFilename, std::string confusionMatrixFilename) {
+  cnn->processDatasetRepeatTest(dataset, batchSize, nReps, predictionsFilename,
+                                confusionMatrixFilename);
+}
+void SparseConvNet::loadWeights(std::string baseName, int epoch, bool momentum,
+                                int firstNlayers) {
+  cnn->loadWeights(baseName, epoch, momentum, firstNlayers);
+}
+void SparseConvNet::saveWeights(std::string baseName, int epoch,
+                                bool momentum) {
+  cnn->saveWeights(baseName, epoch, momentum);
+}
+
+SparseConvTriangLeNet::SparseConvTriangLeNet(int dimension, int nInputFeatures,
+                                             int nClasses, int pciBusID,
+                                             int nTop)
+    : cnn(new SparseConvNetCUDA(dimension, nInputFeatures, nClasses, pciBusID,
+                                nTop)) {}
+SparseConvTriangLeNet::~SparseConvTriangLeNet() {}
+void SparseConvTriangLeNet::addLeNetLayerMP(int nFeatures, int filterSize,
+                                            int filterStride, int poolSize,
+                                            int poolStride,
+                                            ActivationFunction activationFn,
+                                            float dropout,
+                                            int minActiveInputs) {
+  cnn->addTriangularLeNetLayerMP(nFeatures, filterSize, filterStride, poolSize,
+                                 poolStride, activationFn, dropout,
+                                 minActiveInputs);
+}
+void SparseConvTriangLeNet::addTerminalPoolingLayer(int poolSize) {
+  cnn->addTerminalPoolingLayer(poolSize,
+                               triangleSize(poolSize, cnn->dimension));
+}
+void SparseConvTriangLeNet::addSoftmaxLayer() { cnn->addSoftmaxLayer(); }
+float SparseConvTriangLeNet::processDataset(SpatiallySparseDataset &dataset,
+                                            int batchSize, float learningRate,
+                                            float momentum) {
+  return cnn->processDataset(dataset, batchSize, learningRate, momentum);
+}
+void SparseConvTriangLeNet::processDatasetRepeatTest(
+    SpatiallySparseDataset &dataset, int batchSize, int nReps,
+    std::string predictionsFilename, std::string confusionMatrixFilename) {
+  cnn->processDatasetRepeatTest(dataset, batchSize, nReps, predictionsFilename,
+                                confusionMatrixFilename);
+}
+void SparseConvTriangLeNet::loadWeights(std::string baseName, int epoch,
+                                        bool momentum, int firstNlayers) {
+  cnn->loadWeights(baseName, epoch, momentum, firstNlayers);
+}
+void SparseConvTriangLeNet::saveWeights(std::string baseName, int epoch,
+                                        bool momentum) {
+  cnn->saveWeights(baseName, epoch, momentum);
+}
+
+// ============================================================ architectures
+// NetworkArchitectures.cpp:3-68
+DeepCNet::DeepCNet(int dimension, int l, int k, ActivationFunction fn,
+                   int nInputFeatures, int nClasses, float p, int cudaDevice,
+                   int nTop)
+    : SparseConvNet(dimension, nInputFeatures, nClasses, cudaDevice, nTop) {
+  for (int i = 0; i <= l; i++)
+    addLeNetLayerMP((i + 1) * k, i == 0 ? 3 : 2, 1, i < l ? 3 : 1,
+                    i < l ? 2 : 1, fn, p * i * 1.0f / l);
+  addSoftmaxLayer();
+}
+DeepC2::DeepC2(int dimension, int l, int k, ActivationFunction fn,
+               int nInputFeatures, int nClasses, float p, int cudaDevice,
+               int nTop)
+    : SparseConvNet(dimension, nInputFeatures, nClasses, cudaDevice, nTop) {
+  for (int i = 0; i <= l; i++)
+    addLeNetLayerMP((i + 1) * k, 2, 1, i < l ? 3 : 1, i < l ? 2 : 1, fn,
+                    p * i * 1.0f / l);
+  addSoftmaxLayer();
+}
+DeepCNiN::DeepCNiN(int dimension, int l, int k, ActivationFunction fn,
+                   int nInputFeatures, int nClasses, float p, int cudaDevice,
+                   int nTop)
+    : SparseConvNet(dimension, nInputFeatures, nClasses, cudaDevice, nTop) {
+  for (int i = 0; i <= l; i++) {
+    addLeNetLayerMP((i + 1) * k, 2, 1, i < l ? 3 : 1, i < l ? 2 : 1, fn,
+                    p * i * 1.0f / l);
+    addLeNetLayerMP((i + 1) * k, 1, 1, 1, 1, fn, p * i * 1.0f / l);
+  }
+  addSoftmaxLayer();
+}
+DeepC2C2::DeepC2C2(int dimension, int l, int k, ActivationFunction fn,
+                   int nInputFeatures, int nClasses, float p, int cudaDevice,
+                   int nTop)
+    : SparseConvNet(dimension, nInputFeatures, nClasses, cudaDevice, nTop) {
+  for (int i = 0; i < l; i++) {
+    addLeNetLayerMP((i + 1) * k, 2, 1, 1, 1, fn, p * i * 1.0f / l);
+    addLeNetLayerMP((i + 1) * k, 2, 1, 3, 2, fn, p * i * 1.0f / l);
+  }
+  addLeNetLayerMP((l + 1) * k, 2, 1, 1, 1, fn, p);
+  addLeNetLayerMP((l + 1) * k, 1, 1, 1, 1, fn, p);
+  addSoftmaxLayer();
+}
+DeepC3C3::DeepC3C3(int dimension, int l, int k, ActivationFunction fn,
+                   int nInputFeatures, int nClasses, float p, int cudaDevice,
+                   int nTop)
+    : SparseConvNet(dimension, nInputFeatures, nClasses, cudaDevice, nTop) {
+  for (int i = 0; i < l; i++) {
+    addLeNetLayerMP((i + 1) * k, 3, 1, 1, 1, fn, p * i * 1.0f / l);
+    addLeNetLayerMP((i + 1) * k, 3, 1, 3, 2, fn, p * i * 1.0f / l);
+  }
+  addLeNetLayerMP((l + 1) * k, 3, 1, 1, 1, fn, p);
+  addLeNetLayerMP((l + 1) * k, 1, 1, 1, 1, fn, p);
+  addSoftmaxLayer();
+}
+DeepC3C3Valid::DeepC3C3Valid(int dimension, int l, int k,
+                             ActivationFunction fn, int nInputFeatures,
+                             int nClasses, float p, int cudaDevice, int nTop)
+    : SparseConvNet(dimension, nInputFeatures, nClasses, cudaDevice, nTop) {
+  for (int i = 0; i < l; i++) {
+    addLeNetLayerMP((i + 1) * k, 3, 1, 1, 1, fn, p * i * 1.0f / l, -1);
+    addLeNetLayerMP((i + 1) * k, 3, 1, 3, 2, fn, p * i * 1.0f / l, -1);
+  }
+  // one ordinary convolution at the end, in case no site survived
+  addLeNetLayerMP((l + 1) * k, 3, 1, 1, 1, fn, p, +1);
+  addLeNetLayerMP((l + 1) * k, 1, 1, 1, 1, fn, p);
+  addSoftmaxLayer();
+}

@@ -1,0 +1,325 @@
+// C view of the host classes (see scn_host_c.h).
+#include "scn_host_c.h"
+#include <cstdio>
+#include <cstdlib>
+#include <memory>
+#include "BatchProducer.h"
+#include "SparseConvNet.h"
+#include "SparseConvNetCUDA.h"
+
+struct scnh_net {
+  std::unique_ptr<SparseConvNet> square;
+  std::unique_ptr<SparseConvTriangLeNet> triangular;
+  SparseConvNetCUDA *cnn = nullptr;
+  std::unique_ptr<BatchProducer> producer;
+  SpatiallySparseBatch *batch = nullptr;
+  bool hasClassifier = false;
+};
+struct scnh_dataset {
+  SpatiallySparseDataset ds;
+  ~scnh_dataset() {
+    for (auto *p : ds.pictures)
+      delete p;
+  }
+};
+
+extern "C" {
+
+scnh_net *scnh_net_create(int dimension, int nInputFeatures, int nClasses,
+                          int nTop, int nBatchProducerThreads,
+                          int triangular) {
+  scnh_net *n = new scnh_net();
+  if (triangular) {
+    n->triangular.reset(new SparseConvTriangLeNet(dimension, nInputFeatures,
+                                                  nClasses, -1, nTop));
+    n->cnn = n->triangular->runtime();
+  } else {
+    n->square.reset(
+        new SparseConvNet(dimension, nInputFeatures, nClasses, -1, nTop));
+    n->cnn = n->square->cnn.get();
+  }
+  // the thread count is fixed at construction in the reference (default 10);
+  // a smaller pool is allowed here because every slot owns device tables
+  if (nBatchProducerThreads >= 1 &&
+      nBatchProducerThreads < n->cnn->nBatchProducerThreads) {
+    n->cnn->nBatchProducerThreads = nBatchProducerThreads;
+    while ((int)n->cnn->batchPool.size() > nBatchProducerThreads)
+      n->cnn->batchPool.pop_back();
+  }
+  return n;
+}
+void scnh_net_destroy(scnh_net *net) {
+  if (!net)
+    return;
+  net->producer.reset();
+  delete net;
+}
+void scnh_add_lenet_layer_mp(scnh_net *net, int nFeatures, int filterSize,
+                             int filterStride, int poolSize, int poolStride,
+                             int activationFn, float dropout,
+                             int minActiveInputs) {
+  if (net->triangular)
+    net->triangular->addLeNetLayerMP(nFeatures, filterSize, filterStride,
+                                     poolSize, poolStride,
+                                     (ActivationFunction)activationFn, dropout,
+                                     minActiveInputs);
+  else
+    net->square->addLeNetLayerMP(nFeatures, filterSize, filterStride, poolSize,
+                                 poolStride, (ActivationFunction)activationFn,
+                                 dropout, minActiveInputs);
+}
+void scnh_add_terminal_pooling_layer(scnh_net *net, int poolSize) {
+  if (net->triangular)
+    net->triangular->addTerminalPoolingLayer(poolSize);
+  else
+    net->square->addTerminalPoolingLayer(poolSize);
+}
+void scnh_add_softmax_layer(scnh_net *net) {
+  if (net->triangular)
+    net->triangular->addSoftmaxLayer();
+  else
+    net->square->addSoftmaxLayer();
+  net->hasClassifier = true;
+}
+int scnh_finish_headless(scnh_net *net, int topSpatialSize) {
+  SparseConvNetCUDA *cnn = net->cnn;
+  cnn->inputSpatialSize = topSpatialSize;
+  std::cout << "Headless stack with layer sizes: " << topSpatialSize;
+  for (int i = (int)cnn->layers.size() - 1; i >= 0; i--)
+    cnn->inputSpatialSize =
+        cnn->layers[i]->calculateInputSpatialSize(cnn->inputSpatialSize);
+  std::cout << std::endl;
+  return cnn->inputSpatialSize;
+}
+void scnh_set_precision(scnh_net *net, int precision) {
+  net->cnn->setPrecision(precision);
+}
+int scnh_input_spatial_size(scnh_net *net) { return net->cnn->inputSpatialSize; }
+int scnh_n_layers(scnh_net *net) { return (int)net->cnn->layers.size(); }
+int scnh_layer_info(scnh_net *net, int layer, int *nIn, int *nOut, int *act) {
+  SpatiallySparseLayer *l = net->cnn->layers.at(layer);
+  int a = -1, i = 0, o = 0, kind = -1;
+  if (auto *c = dynamic_cast<ConvolutionalLayer *>(l)) {
+    kind = 0, i = c->nFeaturesIn, o = c->nFeaturesOut;
+  } else if (auto *c = dynamic_cast<ConvolutionalTriangularLayer *>(l)) {
+    kind = 1, i = c->nFeaturesIn, o = c->nFeaturesOut;
+  } else if (auto *c = dynamic_cast<NetworkInNetworkLayer *>(l)) {
+    kind = 2, i = c->nFeaturesIn, o = c->nFeaturesOut, a = c->fn;
+  } else if (auto *c = dynamic_cast<NetworkInNetworkPReLULayer *>(l)) {
+    kind = 3, i = c->nFeaturesIn, o = c->nFeaturesOut, a = PRELU;
+  } else if (dynamic_cast<MaxPoolingLayer *>(l)) {
+    kind = 4;
+  } else if (dynamic_cast<MaxPoolingTriangularLayer *>(l)) {
+    kind = 5;
+  } else if (dynamic_cast<TerminalPoolingLayer *>(l)) {
+    kind = 6;
+  }
+  if (nIn)
+    *nIn = i;
+  if (nOut)
+    *nOut = o;
+  if (act)
+    *act = a;
+  return kind;
+}
+static void put(vectorCUDA<float> &v, const float *src) {
+  std::vector<float> &h = v.hVector();
+  std::copy(src, src + h.size(), h.begin());
+  v.copyToGPU();
+}
+int scnh_set_weights(scnh_net *net, int layer, const float *W, const float *B,
+                     const float *prelu) {
+  SpatiallySparseLayer *l = net->cnn->layers.at(layer);
+  if (auto *c = dynamic_cast<NetworkInNetworkLayer *>(l)) {
+    put(c->W, W);
+    put(c->B, B);
+    return 0;
+  }
+  if (auto *c = dynamic_cast<NetworkInNetworkPReLULayer *>(l)) {
+    put(c->W, W);
+    put(c->B, B);
+    if (prelu)
+      put(c->PReLU, prelu);
+    return 0;
+  }
+  return -1;
+}
+void scnh_save_weights(scnh_net *net, const char *baseName, int epoch) {
+  net->cnn->saveWeights(baseName, epoch, false);
+}
+void scnh_load_weights(scnh_net *net, const char *baseName, int epoch) {
+  net->cnn->loadWeights(baseName, epoch, false);
+}
+
+scnh_dataset *scnh_dataset_create(const char *name, int nFeatures,
+                                  int nClasses, int type) {
+  scnh_dataset *d = new scnh_dataset();
+  d->ds.name = name ? name : "";
+  d->ds.nFeatures = nFeatures;
+  d->ds.nClasses = nClasses;
+  d->ds.type = (batchType)type;
+  return d;
+}
+void scnh_dataset_destroy(scnh_dataset *ds) { delete ds; }
+void scnh_dataset_add_points(scnh_dataset *ds, int dimension, int latticeSize,
+                             int64_t nSites, const int32_t *coords,
+                             const float *features, int label) {
+  auto *p = new SparsePointsPicture(dimension, latticeSize, ds->ds.nFeatures,
+                                    label);
+  p->coords.assign(coords, coords + nSites * dimension);
+  p->features.assign(features, features + nSites * ds->ds.nFeatures);
+  ds->ds.pictures.push_back(p);
+}
+int64_t scnh_dataset_size(scnh_dataset *ds) {
+  return (int64_t)ds->ds.pictures.size();
+}
+
+float scnh_process_dataset(scnh_net *net, scnh_dataset *ds, int batchSize) {
+  return net->cnn->processDataset(ds->ds, batchSize);
+}
+void scnh_process_dataset_repeat_test(scnh_net *net, scnh_dataset *ds,
+                                      int batchSize, int nReps) {
+  net->cnn->processDatasetRepeatTest(ds->ds, batchSize, nReps);
+}
+
+void scnh_begin(scnh_net *net, scnh_dataset *ds, int batchSize) {
+  net->batch = nullptr;
+  net->producer.reset(new BatchProducer(*net->cnn, ds->ds,
+                                        net->cnn->inputSpatialSize, batchSize));
+}
+static void forward_layers(scnh_net *net, SpatiallySparseBatch &b) {
+  SparseConvNetCUDA *cnn = net->cnn;
+  if (net->hasClassifier) {
+    std::ofstream f, g;
+    cnn->processBatch(b, 0, 0, f, g);
+  } else {
+    for (size_t i = 0; i < cnn->layers.size(); i++) {
+      b.interfaces[i + 1].sub->reset();
+      scn_prof_tag(cnn->memStream.ctx, (int)i);
+      cnn->layers[i]->forwards(b, b.interfaces[i], b.interfaces[i + 1]);
+    }
+  }
+}
+int scnh_next_batch(scnh_net *net) {
+  if (!net->producer)
+    return 0;
+  net->batch = net->producer->nextBatch();
+  if (!net->batch) {
+    net->producer.reset();
+    return 0;
+  }
+  forward_layers(net, *net->batch);
+  net->cnn->memStream.synchronize();
+  return 1;
+}
+void scnh_end(scnh_net *net) {
+  net->batch = nullptr;
+  net->producer.reset();
+}
+int scnh_batch_size(scnh_net *net) { return net->batch->batchSize; }
+int scnh_batch_mistakes(scnh_net *net) { return net->batch->mistakes; }
+float scnh_batch_nll(scnh_net *net) { return net->batch->negativeLogLikelihood; }
+void scnh_batch_probabilities(scnh_net *net, float *out) {
+  for (auto &p : net->batch->probabilities)
+    out = std::copy(p.begin(), p.end(), out);
+}
+void scnh_batch_predictions(scnh_net *net, int32_t *out) {
+  for (auto &p : net->batch->predictions)
+    out = std::copy(p.begin(), p.end(), out);
+}
+void scnh_batch_sample_numbers(scnh_net *net, int32_t *out) {
+  std::copy(net->batch->sampleNumbers.begin(), net->batch->sampleNumbers.end(),
+            out);
+}
+void scnh_iface_info(scnh_net *net, int i, int *nFeatures, int *nSpatialSites,
+                     int *spatialSize, int64_t *nRules, int64_t *nFeatureElems,
+                     int64_t *nChoices, int64_t *nGridEntries) {
+  SpatiallySparseBatchInterface &f = net->batch->interfaces.at(i);
+  *nFeatures = f.nFeatures;
+  *nSpatialSites = f.nSpatialSites;
+  *spatialSize = f.spatialSize;
+  *nRules = (int64_t)f.rules.size64();
+  *nFeatureElems = (int64_t)f.nSpatialSites * f.nFeatures;
+  *nChoices = (int64_t)f.sub->poolingChoices.size64();
+  int64_t n = 0;
+  if (f.deviceGrids)
+    SCN_CHECKED(scn_grids_info(f.deviceGrids, nullptr, nullptr, nullptr, &n,
+                               nullptr));
+  *nGridEntries = n;
+}
+void scnh_iface_rules(scnh_net *net, int i, int32_t *out) {
+  SpatiallySparseBatchInterface &f = net->batch->interfaces.at(i);
+  SCN_CHECKED(scn_d2h(net->cnn->memStream.ctx, out, f.rules.dPtr(),
+                      f.rules.size64() * sizeof(int32_t)));
+}
+void scnh_iface_features(scnh_net *net, int i, float *out) {
+  SpatiallySparseBatchInterface &f = net->batch->interfaces.at(i);
+  SCN_CHECKED(scn_d2h(net->cnn->memStream.ctx, out, f.sub->features.dPtr(),
+                      (size_t)f.nSpatialSites * f.nFeatures * sizeof(float)));
+}
+void scnh_iface_choices(scnh_net *net, int i, int32_t *out) {
+  SpatiallySparseBatchInterface &f = net->batch->interfaces.at(i);
+  SCN_CHECKED(scn_d2h(net->cnn->memStream.ctx, out,
+                      f.sub->poolingChoices.dPtr(),
+                      f.sub->poolingChoices.size64() * sizeof(int32_t)));
+}
+void scnh_iface_grids(scnh_net *net, int i, int32_t *sample, int64_t *key,
+                      int32_t *row, int32_t *background) {
+  SpatiallySparseBatchInterface &f = net->batch->interfaces.at(i);
+  SCN_CHECKED(scn_grids_download(net->cnn->memStream.ctx, f.deviceGrids,
+                                 sample, key, row, background));
+}
+
+int scnh_forward_resident(scnh_net *net, int batch, const int32_t *d_sample,
+                          const int64_t *d_key, const int32_t *d_row,
+                          const int32_t *d_background, int64_t nActive,
+                          int nSpatialSites, const float *d_features,
+                          float *h_probs) {
+  SparseConvNetCUDA *cnn = net->cnn;
+  scn_ctx *ctx = cnn->memStream.ctx;
+  SpatiallySparseBatch &b = cnn->batchPool[0];
+  while (b.interfaces.size() <= cnn->layers.size()) {
+    cnn->sharedSubInterfaces.push_back(new SpatiallySparseBatchSubInterface());
+    for (auto &slot : cnn->batchPool)
+      slot.interfaces.emplace_back(cnn->sharedSubInterfaces.back());
+  }
+  b.reset();
+  b.type = UNLABELEDBATCH;
+  b.batchSize = batch;
+  SpatiallySparseBatchInterface &in = b.interfaces[0];
+  in.nFeatures = cnn->nInputFeatures;
+  in.spatialSize = cnn->inputSpatialSize;
+  in.nSpatialSites = nSpatialSites;
+  in.featuresPresent.hVector() = range(cnn->nInputFeatures);
+  if (!in.deviceGrids) {
+    SCN_CHECKED(scn_grids_create(ctx, &in.deviceGrids));
+    in.ownsDeviceGrids = true;
+  }
+  scn_prof_tag(ctx, -1);
+  SCN_CHECKED(scn_grids_build(ctx, in.deviceGrids, batch, cnn->dimension,
+                              in.spatialSize, d_sample, d_key, d_row, nActive,
+                              d_background, nSpatialSites));
+  in.sub->features.copyToGPU();
+  size_t nElems = (size_t)nSpatialSites * cnn->nInputFeatures;
+  in.sub->features.resize64(nElems);
+  SCN_CHECKED(scn_d2d(ctx, in.sub->features.dPtr(), d_features,
+                      nElems * sizeof(float)));
+  for (size_t i = 0; i < cnn->layers.size(); i++) {
+    scn_prof_tag(ctx, (int)i);
+    cnn->layers[i]->preprocess(b, b.interfaces[i], b.interfaces[i + 1]);
+  }
+  net->batch = &b;
+  forward_layers(net, b);
+  if (net->hasClassifier && h_probs)
+    scnh_batch_probabilities(net, h_probs);
+  cnn->memStream.synchronize();
+  return b.interfaces.back().nSpatialSites;
+}
+void *scnh_context(scnh_net *net) { return net->cnn->memStream.ctx; }
+double scnh_take_multiply_add_count(void) {
+  double v = (double)multiplyAddCount;
+  multiplyAddCount = 0;
+  return v;
+}
+
+} // extern "C"

@@ -1,0 +1,94 @@
+/* C view of the C++ host classes, for callers that cannot link C++ (the
+ * Python test and benchmark harness loads it with ctypes).  Every function
+ * forwards to the class method named in its comment. */
+#ifndef SCN_HOST_C_H
+#define SCN_HOST_C_H
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct scnh_net scnh_net;
+typedef struct scnh_dataset scnh_dataset;
+
+/* SparseConvNet / SparseConvTriangLeNet constructors */
+scnh_net *scnh_net_create(int dimension, int nInputFeatures, int nClasses,
+                          int nTop, int nBatchProducerThreads, int triangular);
+void scnh_net_destroy(scnh_net *net);
+/* addLeNetLayerMP of the square or triangular facade */
+void scnh_add_lenet_layer_mp(scnh_net *net, int nFeatures, int filterSize,
+                             int filterStride, int poolSize, int poolStride,
+                             int activationFn, float dropout,
+                             int minActiveInputs);
+void scnh_add_terminal_pooling_layer(scnh_net *net, int poolSize);
+void scnh_add_softmax_layer(scnh_net *net);
+/* A stack without a classifier: fixes the spatial sizes from the size of the
+ * last layer's output; returns the input field size. */
+int scnh_finish_headless(scnh_net *net, int topSpatialSize);
+void scnh_set_precision(scnh_net *net, int precision);
+int scnh_input_spatial_size(scnh_net *net);
+int scnh_n_layers(scnh_net *net);
+/* kind: 0 conv, 1 triangular conv, 2 NiN, 3 NiN PReLU, 4 max-pool,
+ * 5 triangular max-pool, 6 terminal pool; NiN layers report nIn/nOut/act */
+int scnh_layer_info(scnh_net *net, int layer, int *nIn, int *nOut, int *act);
+/* NetworkInNetwork(PReLU)Layer::W, B, PReLU */
+int scnh_set_weights(scnh_net *net, int layer, const float *W, const float *B,
+                     const float *prelu);
+void scnh_save_weights(scnh_net *net, const char *baseName, int epoch);
+void scnh_load_weights(scnh_net *net, const char *baseName, int epoch);
+
+scnh_dataset *scnh_dataset_create(const char *name, int nFeatures,
+                                  int nClasses, int type);
+void scnh_dataset_destroy(scnh_dataset *ds);
+/* appends a SparsePointsPicture */
+void scnh_dataset_add_points(scnh_dataset *ds, int dimension, int latticeSize,
+                             int64_t nSites, const int32_t *coords,
+                             const float *features, int label);
+int64_t scnh_dataset_size(scnh_dataset *ds);
+
+/* SparseConvNet::processDataset / processDatasetRepeatTest */
+float scnh_process_dataset(scnh_net *net, scnh_dataset *ds, int batchSize);
+void scnh_process_dataset_repeat_test(scnh_net *net, scnh_dataset *ds,
+                                      int batchSize, int nReps);
+
+/* Batch-by-batch processing with the batch left in place for inspection:
+ * BatchProducer::nextBatch + SparseConvNetCUDA::processBatch. */
+void scnh_begin(scnh_net *net, scnh_dataset *ds, int batchSize);
+int scnh_next_batch(scnh_net *net); /* 0 when the dataset is exhausted */
+void scnh_end(scnh_net *net);
+int scnh_batch_size(scnh_net *net);
+int scnh_batch_mistakes(scnh_net *net);
+float scnh_batch_nll(scnh_net *net);
+void scnh_batch_probabilities(scnh_net *net, float *out);
+void scnh_batch_predictions(scnh_net *net, int32_t *out);
+void scnh_batch_sample_numbers(scnh_net *net, int32_t *out);
+/* interface i (0 = input): sizes, then the vectors themselves */
+void scnh_iface_info(scnh_net *net, int i, int *nFeatures, int *nSpatialSites,
+                     int *spatialSize, int64_t *nRules, int64_t *nFeatureElems,
+                     int64_t *nChoices, int64_t *nGridEntries);
+void scnh_iface_rules(scnh_net *net, int i, int32_t *out);
+void scnh_iface_features(scnh_net *net, int i, float *out);
+void scnh_iface_choices(scnh_net *net, int i, int32_t *out);
+void scnh_iface_grids(scnh_net *net, int i, int32_t *sample, int64_t *key,
+                      int32_t *row, int32_t *background);
+
+/* One forward pass over a batch whose input already sits in HBM: active
+ * sites (sample, key, row), backgroundCol per sample and the input feature
+ * matrix [nSpatialSites x nInputFeatures], all device pointers.  Builds the
+ * grids and every rule book, runs every layer and, when the net ends in the
+ * softmax classifier, copies the probabilities [batch x nClasses] to h_probs.
+ * Returns the number of rows of the last interface. */
+int scnh_forward_resident(scnh_net *net, int batch, const int32_t *d_sample,
+                          const int64_t *d_key, const int32_t *d_row,
+                          const int32_t *d_background, int64_t nActive,
+                          int nSpatialSites, const float *d_features,
+                          float *h_probs);
+/* the library context of the net (scn_ctx *), for timing and raw buffers */
+void *scnh_context(scnh_net *net);
+/* multiply-accumulates of the NiN layers since the last call */
+double scnh_take_multiply_add_count(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

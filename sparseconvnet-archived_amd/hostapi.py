@@ -1,0 +1,236 @@
+"""ctypes view of ``libscn_host.so``: the C++ host classes (SparseConvNet,
+SparseConvTriangLeNet, SpatiallySparseDataset, BatchProducer) through the C
+facade in ``host/scn_host_c.h``.  Harness plumbing only."""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libscn_host.so")
+
+TRAINBATCH, TESTBATCH, UNLABELEDBATCH, RESCALEBATCH = range(4)
+LAYER_KINDS = ["conv", "conv_tri", "nin", "nin_prelu", "maxpool", "maxpool_tri", "terminal"]
+
+
+def build(force=True):
+    args = ["make", "-C", os.path.join(_HERE, "host"), "-s", "-j8"]
+    if force:
+        args.append("-B")
+    subprocess.check_call(args)
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError("libscn_host.so is not built; run __graft_entry__.build()")
+    L = C.CDLL(LIB_PATH)
+    vp, i32, i64, f32 = C.c_void_p, C.c_int, C.c_int64, C.c_float
+    P = C.POINTER
+    sig = {
+        "scnh_net_create": (vp, [i32] * 6),
+        "scnh_net_destroy": (None, [vp]),
+        "scnh_add_lenet_layer_mp": (None, [vp] + [i32] * 6 + [f32, i32]),
+        "scnh_add_terminal_pooling_layer": (None, [vp, i32]),
+        "scnh_add_softmax_layer": (None, [vp]),
+        "scnh_finish_headless": (i32, [vp, i32]),
+        "scnh_set_precision": (None, [vp, i32]),
+        "scnh_input_spatial_size": (i32, [vp]),
+        "scnh_n_layers": (i32, [vp]),
+        "scnh_layer_info": (i32, [vp, i32, P(i32), P(i32), P(i32)]),
+        "scnh_set_weights": (i32, [vp, i32, vp, vp, vp]),
+        "scnh_save_weights": (None, [vp, C.c_char_p, i32]),
+        "scnh_load_weights": (None, [vp, C.c_char_p, i32]),
+        "scnh_dataset_create": (vp, [C.c_char_p, i32, i32, i32]),
+        "scnh_dataset_destroy": (None, [vp]),
+        "scnh_dataset_add_points": (None, [vp, i32, i32, i64, vp, vp, i32]),
+        "scnh_dataset_size": (i64, [vp]),
+        "scnh_process_dataset": (f32, [vp, vp, i32]),
+        "scnh_process_dataset_repeat_test": (None, [vp, vp, i32, i32]),
+        "scnh_begin": (None, [vp, vp, i32]),
+        "scnh_next_batch": (i32, [vp]),
+        "scnh_end": (None, [vp]),
+        "scnh_batch_size": (i32, [vp]),
+        "scnh_batch_mistakes": (i32, [vp]),
+        "scnh_batch_nll": (f32, [vp]),
+        "scnh_batch_probabilities": (None, [vp, vp]),
+        "scnh_batch_predictions": (None, [vp, vp]),
+        "scnh_batch_sample_numbers": (None, [vp, vp]),
+        "scnh_iface_info": (None, [vp, i32, P(i32), P(i32), P(i32), P(i64), P(i64), P(i64), P(i64)]),
+        "scnh_iface_rules": (None, [vp, i32, vp]),
+        "scnh_iface_features": (None, [vp, i32, vp]),
+        "scnh_iface_choices": (None, [vp, i32, vp]),
+        "scnh_iface_grids": (None, [vp, i32, vp, vp, vp, vp]),
+        "scnh_forward_resident": (i32, [vp, i32, vp, vp, vp, vp, i64, i32, vp, vp]),
+        "scnh_context": (vp, [vp]),
+        "scnh_take_multiply_add_count": (C.c_double, []),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(L, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = L
+    return L
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+class Dataset:
+    def __init__(self, name, nFeatures, nClasses, batch_type=TESTBATCH):
+        self.nFeatures, self.nClasses = nFeatures, nClasses
+        self.h = lib().scnh_dataset_create(name.encode(), nFeatures, nClasses, batch_type)
+
+    def add_points(self, dimension, latticeSize, coords, features, label=-1):
+        coords = np.ascontiguousarray(coords, np.int32).reshape(-1, dimension)
+        features = np.ascontiguousarray(features, np.float32).reshape(coords.shape[0], self.nFeatures)
+        lib().scnh_dataset_add_points(self.h, dimension, latticeSize, coords.shape[0], _p(coords), _p(features), label)
+
+    def __len__(self):
+        return lib().scnh_dataset_size(self.h)
+
+    def close(self):
+        if getattr(self, "h", None):
+            lib().scnh_dataset_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Net:
+    """SparseConvNet (or SparseConvTriangLeNet with triangular=True)."""
+
+    def __init__(self, dimension, nInputFeatures, nClasses, nTop=1, threads=2, triangular=False):
+        self.dimension, self.nInputFeatures, self.nClasses, self.nTop = dimension, nInputFeatures, nClasses, nTop
+        self.h = lib().scnh_net_create(dimension, nInputFeatures, nClasses, nTop, threads, int(triangular))
+
+    def close(self):
+        if getattr(self, "h", None):
+            lib().scnh_net_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    # builders, named as in the reference
+    def addLeNetLayerMP(self, nFeatures, filterSize, filterStride, poolSize, poolStride, activationFn=1, dropout=0.0,
+                        minActiveInputs=1):
+        lib().scnh_add_lenet_layer_mp(self.h, nFeatures, filterSize, filterStride, poolSize, poolStride, activationFn,
+                                      dropout, minActiveInputs)
+
+    def addTerminalPoolingLayer(self, poolSize):
+        lib().scnh_add_terminal_pooling_layer(self.h, poolSize)
+
+    def addSoftmaxLayer(self):
+        lib().scnh_add_softmax_layer(self.h)
+
+    def finishHeadless(self, topSpatialSize):
+        return lib().scnh_finish_headless(self.h, topSpatialSize)
+
+    def setPrecision(self, precision):
+        lib().scnh_set_precision(self.h, precision)
+
+    @property
+    def inputSpatialSize(self):
+        return lib().scnh_input_spatial_size(self.h)
+
+    def layers(self):
+        out = []
+        for i in range(lib().scnh_n_layers(self.h)):
+            a, b, c = C.c_int(), C.c_int(), C.c_int()
+            kind = lib().scnh_layer_info(self.h, i, C.byref(a), C.byref(b), C.byref(c))
+            out.append(dict(kind=LAYER_KINDS[kind], nIn=a.value, nOut=b.value, act=c.value))
+        return out
+
+    def set_weights(self, layer, W, B, prelu=None):
+        W = np.ascontiguousarray(W, np.float32)
+        B = np.ascontiguousarray(B, np.float32)
+        pr = np.ascontiguousarray(prelu, np.float32) if prelu is not None else None
+        rc = lib().scnh_set_weights(self.h, layer, _p(W), _p(B), _p(pr) if pr is not None else None)
+        assert rc == 0, "layer %d has no weights" % layer
+
+    def saveWeights(self, base, epoch):
+        lib().scnh_save_weights(self.h, base.encode(), epoch)
+
+    def loadWeights(self, base, epoch):
+        lib().scnh_load_weights(self.h, base.encode(), epoch)
+
+    def processDataset(self, ds, batchSize=100):
+        return lib().scnh_process_dataset(self.h, ds.h, batchSize)
+
+    def processDatasetRepeatTest(self, ds, batchSize=100, nReps=2):
+        lib().scnh_process_dataset_repeat_test(self.h, ds.h, batchSize, nReps)
+
+    # batch-by-batch with inspection
+    def begin(self, ds, batchSize):
+        lib().scnh_begin(self.h, ds.h, batchSize)
+
+    def next_batch(self):
+        return bool(lib().scnh_next_batch(self.h))
+
+    def end(self):
+        lib().scnh_end(self.h)
+
+    def batch_outputs(self):
+        L = lib()
+        b = L.scnh_batch_size(self.h)
+        probs = np.empty((b, self.nClasses), np.float32)
+        pred = np.empty((b, self.nTop), np.int32)
+        nums = np.empty(b, np.int32)
+        L.scnh_batch_probabilities(self.h, _p(probs))
+        L.scnh_batch_predictions(self.h, _p(pred))
+        L.scnh_batch_sample_numbers(self.h, _p(nums))
+        return dict(probabilities=probs, predictions=pred, sampleNumbers=nums, mistakes=L.scnh_batch_mistakes(self.h),
+                    nll=L.scnh_batch_nll(self.h), batchSize=b)
+
+    def interface(self, i, want_features=True):
+        L = lib()
+        nf, ns, ss = C.c_int(), C.c_int(), C.c_int()
+        nr, ne, nc, ng = C.c_int64(), C.c_int64(), C.c_int64(), C.c_int64()
+        L.scnh_iface_info(self.h, i, C.byref(nf), C.byref(ns), C.byref(ss), C.byref(nr), C.byref(ne), C.byref(nc),
+                          C.byref(ng))
+        out = dict(nFeatures=nf.value, nSpatialSites=ns.value, spatialSize=ss.value)
+        rules = np.empty(nr.value, np.int32)
+        if nr.value:
+            L.scnh_iface_rules(self.h, i, _p(rules))
+        out["rules"] = rules
+        if want_features:
+            feats = np.empty((ns.value, nf.value), np.float32)
+            if ne.value:
+                L.scnh_iface_features(self.h, i, _p(feats))
+            out["features"] = feats
+        ch = np.empty(nc.value, np.int32)
+        if nc.value:
+            L.scnh_iface_choices(self.h, i, _p(ch))
+        out["choices"] = ch
+        b = L.scnh_batch_size(self.h)
+        s, k, r, bg = np.empty(ng.value, np.int32), np.empty(ng.value, np.int64), np.empty(ng.value, np.int32), np.empty(b, np.int32)
+        L.scnh_iface_grids(self.h, i, _p(s), _p(k), _p(r), _p(bg))
+        out["grids"] = (s, k, r, bg)
+        return out
+
+    # resident input (device pointers as integers)
+    def forward_resident(self, batch, d_sample, d_key, d_row, d_bg, nActive, nSpatialSites, d_features, h_probs=None):
+        return lib().scnh_forward_resident(self.h, batch, d_sample, d_key, d_row, d_bg, nActive, nSpatialSites,
+                                           d_features, _p(h_probs) if h_probs is not None else None)
+
+    def context_handle(self):
+        return lib().scnh_context(self.h)
+
+
+def take_multiply_add_count():
+    return lib().scnh_take_multiply_add_count()

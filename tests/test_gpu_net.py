@@ -1,0 +1,159 @@
+"""Whole stacks through the C++ host classes (SparseConvNet builders,
+BatchProducer, processBatch) against the net-level oracle."""
+import os
+
+import numpy as np
+import pytest
+
+import oracle as orc
+import oracle_net
+from conftest import load_scn
+
+pytestmark = pytest.mark.gpu
+
+
+def rel_l2(a, b):
+    a = a.astype(np.float64).ravel()
+    b = b.astype(np.float64).ravel()
+    return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30))
+
+
+def build_pair(cfg, hostapi, triangular=False):
+    net = hostapi.Net(cfg.dimension, cfg.nInputFeatures, cfg.nClasses, nTop=1, threads=2, triangular=triangular)
+    ora = oracle_net.Net(cfg.dimension, cfg.nInputFeatures, cfg.nClasses, nTop=1, triangular=triangular)
+    cfg.build(net)
+    cfg.build(ora)
+    assert net.layers() == ora.layer_list()
+    assert net.inputSpatialSize == ora.inputSpatialSize
+    return net, ora
+
+
+def run_config(scn, cfg, seed, tol=1e-4, triangular=False, samples=None):
+    from sparseconvnet_archived_amd import hostapi, synthetic
+    net, ora = build_pair(cfg, hostapi, triangular)
+    weights = synthetic.he_normal_weights(net.layers(), seed + 1)
+    for i, (W, B, pr) in weights.items():
+        net.set_weights(i, W, B, pr)
+        ora.set_weights(i, W, B, pr)
+    samples = samples or synthetic.make_samples(cfg, seed)
+    ds = hostapi.Dataset(cfg.name, cfg.nInputFeatures, max(cfg.nClasses, 1), hostapi.TESTBATCH)
+    for pts, f, label in samples:
+        ds.add_points(cfg.dimension, cfg.lattice, pts, f, label)
+    S, K, R, bg, feats, n = synthetic.codify(samples, cfg.dimension, cfg.lattice, net.inputSpatialSize, cfg.nInputFeatures)
+    labels = np.array([s[2] for s in samples], np.int32)
+    want = ora.forward(len(samples), S, K, R, bg, feats, n, labels)
+    print("config", cfg.name, "batch", len(samples), "input rows", n, flush=True)
+    net.begin(ds, len(samples))
+    assert net.next_batch()
+    layers = net.layers()
+    for i, wi in enumerate(want["interfaces"]):
+        gi = net.interface(i)
+        print("  interface", i, "rows", gi["nSpatialSites"], "features", gi["nFeatures"], flush=True)
+        assert gi["nSpatialSites"] == wi["nSpatialSites"]
+        assert gi["nFeatures"] == wi["nFeatures"]
+        assert gi["spatialSize"] == wi["spatialSize"]
+        # rule books, grids and background rows: bit-exact
+        assert np.array_equal(gi["rules"], wi["rules"])
+        s, k, r, b = gi["grids"]
+        os_, ok, or_, ob = wi["grids"].flat()
+        assert np.array_equal(s, os_) and np.array_equal(k, ok) and np.array_equal(r, or_) and np.array_equal(b, ob)
+        # activations: 1e-4 relative (fp32)
+        err = rel_l2(gi["features"], wi["features"])
+        print("    rel-L2 error %.3g" % err, flush=True)
+        assert err <= tol
+        if i > 0:
+            kind = layers[i - 1]["kind"]
+            prev = net.interface(i - 1)
+            if kind.startswith("maxpool"):
+                # values and argmax indices bit-exact on identical inputs
+                width = gi["rules"].size // gi["nSpatialSites"]
+                v, ch = orc.maxpool(prev["features"], gi["rules"], gi["nSpatialSites"], width, gi["nFeatures"])
+                assert np.array_equal(gi["features"], v)
+                assert np.array_equal(gi["choices"], ch.ravel())
+            if kind.startswith("conv"):
+                assert np.array_equal(gi["features"].ravel(),
+                                      orc.gather_rows(prev["features"], gi["rules"], prev["nFeatures"]).ravel())
+    if "probabilities" in want:
+        out = net.batch_outputs()
+        assert np.allclose(out["probabilities"], want["probabilities"], rtol=1e-3, atol=1e-6)
+        agree = np.mean(out["predictions"][:, 0] == want["predictions"][:, 0])
+        assert agree >= 0.995
+        assert out["mistakes"] == want["mistakes"] or agree < 1.0
+        assert np.isclose(out["nll"], want["nll"], rtol=1e-3)
+    assert not net.next_batch()
+    net.close()
+    return want
+
+
+def test_config1_single_conv(scn):
+    from sparseconvnet_archived_amd import synthetic
+    run_config(scn, synthetic.config(1), 101)
+
+
+def test_config2_sparse_net_2d(scn):
+    from sparseconvnet_archived_amd import synthetic
+    run_config(scn, synthetic.config(2, batch=20), 102)
+
+
+def test_config3_voxel_net_3d(scn):
+    from sparseconvnet_archived_amd import synthetic
+    run_config(scn, synthetic.config(3, batch=6), 103)
+
+
+def test_config4_wide_net_small_batch(scn):
+    from sparseconvnet_archived_amd import synthetic
+    run_config(scn, synthetic.config(4, batch=3), 104)
+
+
+def test_config5_spatiotemporal_small_batch(scn):
+    from sparseconvnet_archived_amd import synthetic
+    run_config(scn, synthetic.config(5, batch=1), 105)
+
+
+def test_triangular_net(scn):
+    """SparseConvTriangLeNet: triangular filters, and the builder quirk that
+    makes the convolution's minActiveInputs equal to the pool size."""
+    from sparseconvnet_archived_amd import synthetic
+    stack = [("addLeNetLayerMP", 32, 2, 1, 2, 2, synthetic.RELU), ("addLeNetLayerMP", 64, 2, 1, 2, 2, synthetic.RELU),
+             ("addLeNetLayerMP", 64, 2, 1, 1, 1, synthetic.VLEAKYRELU), ("addTerminalPoolingLayer", 2), ("addSoftmaxLayer",)]
+    cfg = synthetic.Config("tri", 2, 3, 10, 8, 13, stack)
+    cfg.number = 2
+    rng = np.random.default_rng(5)
+    samples = []
+    for _ in range(8):
+        pts = np.array([(a, b) for a in range(13) for b in range(13 - a) if rng.random() < 0.4], np.int32)
+        samples.append((pts, rng.uniform(-1, 1, (len(pts), 3)).astype(np.float32), int(rng.integers(0, 10))))
+    run_config(scn, cfg, 7, triangular=True, samples=samples)
+
+
+def test_process_dataset_and_weight_files(scn, tmp_path):
+    from sparseconvnet_archived_amd import hostapi, synthetic
+    cfg = synthetic.config(2, batch=10)
+    net, ora = build_pair(cfg, hostapi)
+    for i, (W, B, pr) in synthetic.he_normal_weights(net.layers(), 9).items():
+        net.set_weights(i, W, B, pr)
+        ora.set_weights(i, W, B, pr)
+    samples = synthetic.make_samples(cfg, 33, batch=25)
+    ds = hostapi.Dataset("synthetic", 3, 100, hostapi.TESTBATCH)
+    for pts, f, label in samples:
+        ds.add_points(2, cfg.lattice, pts, f, label)
+    # three batches (10, 10, 5) through processDataset
+    nll = net.processDataset(ds, 10)
+    want_nll = 0.0
+    for lo in range(0, 25, 10):
+        chunk = samples[lo:lo + 10]
+        S, K, R, bg, feats, n = synthetic.codify(chunk, 2, cfg.lattice, net.inputSpatialSize, 3)
+        w = ora.forward(len(chunk), S, K, R, bg, feats, n, np.array([s[2] for s in chunk], np.int32), keep=False)
+        want_nll += w["nll"] / 25
+    assert np.isclose(nll, want_nll, rtol=1e-3)
+    # weights survive a save / load round trip through the .cnn format
+    base = str(tmp_path / "w")
+    net.saveWeights(base, 3)
+    size = os.path.getsize(base + "_epoch-3.cnn")
+    expect = sum(l["nIn"] * l["nOut"] + l["nOut"] * (2 if l["kind"] == "nin_prelu" else 1)
+                 for l in net.layers() if l["kind"].startswith("nin"))
+    assert size == 4 * expect
+    net2, _ = build_pair(cfg, hostapi)
+    net2.loadWeights(base, 3)
+    assert np.isclose(net2.processDataset(ds, 10), nll, rtol=1e-6)
+    net2.processDatasetRepeatTest(ds, 10, 2)
