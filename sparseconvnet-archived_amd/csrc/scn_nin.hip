@@ -102,6 +102,139 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// ---- MFMA path: fp32 operands, v_mfma_f32_32x32x2_f32 ----------------------
+// Block = 4 wavefronts laid out WM x WN; every wavefront owns a 32 x (32 NT)
+// patch of the output as NT accumulator tiles of 32x32 (16 VGPRs per lane
+// each).  Operands are staged through LDS in k-slabs of MF_BK, double
+// buffered: A transposed to [k][row] (row stride odd, so both the transposing
+// stores and the operand reads hit every bank evenly), W as [k][col].  One
+// MFMA consumes k = 2: lane l supplies A[row = l % 32][k = l / 32] and
+// W[k = l / 32][col = l % 32]; accumulator register v of lane l is
+// D[row = 8 (v / 4) + 4 (l / 32) + v % 4][col = l % 32].
+#define MF_BK 32
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+template <int WM, int WN, int NT>
+__global__ void __launch_bounds__(256)
+    k_nin_mfma(const float *__restrict__ A, const float *__restrict__ W,
+               float *__restrict__ out, long long M, int K, int N,
+               Epilogue ep) {
+  constexpr int BM = 32 * WM;
+  constexpr int BN = 32 * NT * WN;
+  constexpr int BMP = BM + 1;
+  constexpr int A_CHUNKS = BM * MF_BK / 4; // float4 chunks per slab
+  constexpr int W_CHUNKS = MF_BK * BN / 4;
+  constexpr int A_PER = (A_CHUNKS + 255) / 256;
+  constexpr int W_PER = (W_CHUNKS + 255) / 256;
+  __shared__ float sA[2][MF_BK * BMP];
+  __shared__ float sW[2][MF_BK * BN];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+  const int nBlocksN = (N + BN - 1) / BN; // n-blocks fastest: the blocks that
+  const long long m0 = (long long)(blockIdx.x / nBlocksN) * BM; // share an A
+  const int n0 = (int)(blockIdx.x % nBlocksN) * BN;             // slab run together
+  floatx16 acc[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int v = 0; v < 16; ++v)
+      acc[j][v] = 0.f;
+
+  float4 ra[A_PER], rw[W_PER];
+  auto load_slab = [&](int k0) {
+#pragma unroll
+    for (int u = 0; u < A_PER; ++u) {
+      int c = tid + u * 256;
+      int r = c / (MF_BK / 4), kc = c % (MF_BK / 4);
+      long long m = m0 + r;
+      int k = k0 + kc * 4;
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (c < A_CHUNKS && m < M && k < K) // K % 4 == 0: a chunk is all in or all out
+        v = *reinterpret_cast<const float4 *>(A + m * K + k);
+      ra[u] = v;
+    }
+#pragma unroll
+    for (int u = 0; u < W_PER; ++u) {
+      int c = tid + u * 256;
+      int kk = c / (BN / 4), nc = c % (BN / 4);
+      int k = k0 + kk, n = n0 + nc * 4;
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (c < W_CHUNKS && k < K && n < N) // N % 4 == 0
+        v = *reinterpret_cast<const float4 *>(W + (long long)k * N + n);
+      rw[u] = v;
+    }
+  };
+  auto store_slab = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < A_PER; ++u) {
+      int c = tid + u * 256;
+      if (c < A_CHUNKS) {
+        int r = c / (MF_BK / 4), kc = c % (MF_BK / 4);
+        float *dst = &sA[buf][(kc * 4) * BMP + r];
+        dst[0] = ra[u].x;
+        dst[BMP] = ra[u].y;
+        dst[2 * BMP] = ra[u].z;
+        dst[3 * BMP] = ra[u].w;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < W_PER; ++u) {
+      int c = tid + u * 256;
+      if (c < W_CHUNKS)
+        *reinterpret_cast<float4 *>(&sW[buf][c * 4]) = rw[u];
+    }
+  };
+
+  const int nSlabs = (K + MF_BK - 1) / MF_BK;
+  load_slab(0);
+  store_slab(0);
+  __syncthreads();
+  for (int s = 0; s < nSlabs; ++s) {
+    const int buf = s & 1;
+    if (s + 1 < nSlabs)
+      load_slab((s + 1) * MF_BK); // in flight while this slab is multiplied
+    const float *pa = &sA[buf][(lane >> 5) * BMP + wm * 32 + (lane & 31)];
+    const float *pw = &sW[buf][(lane >> 5) * BN + wn * 32 * NT + (lane & 31)];
+#pragma unroll
+    for (int kk = 0; kk < MF_BK; kk += 2) {
+      float a = pa[kk * BMP];
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        float b = pw[kk * BN + 32 * j];
+        acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[j], 0, 0, 0);
+      }
+    }
+    if (s + 1 < nSlabs)
+      store_slab(buf ^ 1);
+    __syncthreads();
+  }
+
+  const int col = lane & 31;
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    int n = n0 + (wn * NT + j) * 32 + col;
+    if (n >= N)
+      continue;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      long long m = m0 + wm * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+      if (m < M)
+        out[m * N + n] = apply_act(acc[j][v], n, ep);
+    }
+  }
+}
+
+template <int WM, int WN, int NT>
+static void launch_mfma(scn_ctx *ctx, const float *A, const float *W,
+                        float *out, long long M, int K, int N,
+                        const Epilogue &ep) {
+  constexpr int BM = 32 * WM, BN = 32 * NT * WN;
+  dim3 grid((unsigned)((long long)scn_ceil_div(N, BN) * scn_ceil_div(M, BM)));
+  hipLaunchKernelGGL((k_nin_mfma<WM, WN, NT>), grid, dim3(256), 0, ctx->stream,
+                     A, W, out, M, K, N, ep);
+}
+
 extern "C" int scn_nin_forward(scn_ctx *ctx, const float *d_A,
                                const float *d_W, const float *d_B,
                                const float *d_prelu, float *d_out, int64_t M,
@@ -129,9 +262,21 @@ extern "C" int scn_nin_forward(scn_ctx *ctx, const float *d_A,
   ep.slope = act == SCN_LEAKYRELU ? 0.01f : (act == SCN_VLEAKYRELU ? 0.333f : 0.f);
   ep.act = act;
   ProfScope prof(ctx, SCN_K_NIN);
-  dim3 grid(scn_ceil_div(M, GT_BM), scn_ceil_div(N, GT_BN));
-  hipLaunchKernelGGL(k_nin_generic, grid, dim3(256), 0, ctx->stream, d_A, d_W,
-                     d_out, (long long)M, K, N, ep);
+  const bool vec = K % 4 == 0 && N % 4 == 0 && ((uintptr_t)d_A & 15) == 0 &&
+                   ((uintptr_t)d_W & 15) == 0;
+  if (vec && K >= 8) {
+    long long blocksLarge = (long long)scn_ceil_div(M, 128) * scn_ceil_div(N, 64);
+    if (N <= 32)
+      launch_mfma<4, 1, 1>(ctx, d_A, d_W, d_out, M, K, N, ep);
+    else if (blocksLarge >= ctx->numCU)
+      launch_mfma<4, 1, 2>(ctx, d_A, d_W, d_out, M, K, N, ep);
+    else // too few rows to fill the chip with tall tiles: 32-row tiles
+      launch_mfma<1, 4, 1>(ctx, d_A, d_W, d_out, M, K, N, ep);
+  } else {
+    dim3 grid(scn_ceil_div(M, GT_BM), scn_ceil_div(N, GT_BN));
+    hipLaunchKernelGGL(k_nin_generic, grid, dim3(256), 0, ctx->stream, d_A,
+                       d_W, d_out, (long long)M, K, N, ep);
+  }
   SCN_HIP_CHECK(hipGetLastError());
   if (act == SCN_SOFTMAX)
     SCN_TRY(scn_softmax_launch(ctx, d_out, d_out, (long long)M, N));
