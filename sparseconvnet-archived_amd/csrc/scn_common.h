@@ -44,7 +44,8 @@ struct scn_ctx {
   hipStream_t stream;
   int numCU;
   // small pinned buffer for counts that must come back to the host
-  int64_t *h_pinned; // 16 int64
+  int64_t *h_pinned; // 16 int64, host view
+  int64_t *d_pinned; // the same memory as the device sees it
   int64_t *d_scalars; // 16 int64
   // profiling
   bool prof;

@@ -19,6 +19,7 @@
 // which needs no sort: count owned outputs per input, scatter the counts to
 // iteration order through the rank, prefix-sum, emit.
 #include "scn_common.h"
+#include "scn_scan_dev.h"
 
 struct __align__(16) Slot {
   long long key;
@@ -70,6 +71,8 @@ struct scn_grids {
   long long termS = 0;
   DevBuf<long long> siteKey; // per output row: packed key, or -1 - sample for a background row
   DevBuf<unsigned> cnt, base;
+  DevBuf<unsigned long long> ownMask;
+  DevBuf<unsigned> rankOf;
   DevBuf<int> bgBefore;
   DevBuf<unsigned> sampleStart;
   DevBuf<int> invOrd;
@@ -225,20 +228,17 @@ __device__ __forceinline__ int count_active(const unsigned long long *bits,
   return c;
 }
 
-// Visits, in ascending output key, the output sites owned by the input site
-// with coordinates i of sample b; f(outKey) is called for each.
-template <int D, typename F>
-__device__ __forceinline__ void for_each_owned(const GridView &in,
-                                               const Geom &g, int b,
-                                               const int *i, F f) {
-  int lo[D], hi[D];
-  const long long sampleBase = (long long)b * g.volIn;
+// The box [lo, hi) of output sites whose window holds the input site i
+// (Regions.cu:13-29), or for valid mode the single site (i0-1, i1-1) when
+// 1 <= i <= nOut on each axis (Regions.cu:693-697).  False when empty.
+template <int D>
+__device__ __forceinline__ bool cand_box(const Geom &g, const int *i, int *lo,
+                                         int *hi) {
   if (g.mode == MODE_SQ_VALID) {
-    // Regions.cu:693-697: output (i0-1, i1-1) when 1 <= i <= nOut on each axis
 #pragma unroll
     for (int a = 0; a < D; ++a) {
       if (i[a] < 1 || i[a] > g.nOut)
-        return;
+        return false;
       lo[a] = i[a] - 1;
       hi[a] = i[a];
     }
@@ -248,43 +248,64 @@ __device__ __forceinline__ void for_each_owned(const GridView &in,
       lo[a] = sq_outputL(g.size, g.stride, i[a]);
       hi[a] = sq_outputR(g.stride, g.nOut, i[a]);
       if (lo[a] >= hi[a])
-        return;
+        return false;
     }
   }
-  const bool tri = g.mode == MODE_TRI_NOMIN || g.mode == MODE_TRI_MIN;
+  return true;
+}
+
+// Does input site i of sample b own candidate output j?  (the active input
+// with the smallest key in j's window owns it; Min modes also need enough
+// active inputs; the triangular lattice only has outputs with sum(j) < nOut)
+template <int D>
+__device__ __forceinline__ bool owns(const GridView &in, const Geom &g,
+                                     long long sampleBase, const int *i,
+                                     const int *j) {
+  if (g.mode == MODE_TRI_NOMIN || g.mode == MODE_TRI_MIN) {
+    int sum = 0;
+#pragma unroll
+    for (int a = 0; a < D; ++a)
+      sum += j[a];
+    if (sum >= g.nOut) // Regions.cu:874,900
+      return false;
+  }
+  if (g.mode == MODE_SQ_VALID)
+    return true;
+  int w[D], off[D];
+#pragma unroll
+  for (int a = 0; a < D; ++a) {
+    w[a] = j[a] * g.stride;
+    off[a] = i[a] - w[a];
+  }
+  if (any_before<D>(in.bits, sampleBase, g.nIn, g.size, w, off))
+    return false;
+  if (g.mode == MODE_SQ_MIN)
+    return count_active<D, false>(in.bits, sampleBase, g.nIn, g.size, w) >=
+           g.minActive;
+  if (g.mode == MODE_TRI_MIN)
+    return count_active<D, true>(in.bits, sampleBase, g.nIn, g.size, w) >=
+           g.minActive;
+  return true;
+}
+
+// Visits, in ascending output key, the output sites owned by the input site
+// with coordinates i of sample b; f(outKey, c) is called for each, c being the
+// position of the site among the candidates of the box.
+template <int D, typename F>
+__device__ __forceinline__ void for_each_owned(const GridView &in,
+                                               const Geom &g, int b,
+                                               const int *i, F f) {
+  int lo[D], hi[D];
+  if (!cand_box<D>(g, i, lo, hi))
+    return;
+  const long long sampleBase = (long long)b * g.volIn;
   int j[D];
 #pragma unroll
   for (int a = 0; a < D; ++a)
     j[a] = lo[a];
-  for (;;) {
-    bool consider = true;
-    if (tri) {
-      int sum = 0;
-#pragma unroll
-      for (int a = 0; a < D; ++a)
-        sum += j[a];
-      consider = sum < g.nOut; // Regions.cu:874,900
-    }
-    if (consider) {
-      bool own = true;
-      if (g.mode != MODE_SQ_VALID) {
-        int w[D], off[D];
-#pragma unroll
-        for (int a = 0; a < D; ++a) {
-          w[a] = j[a] * g.stride;
-          off[a] = i[a] - w[a];
-        }
-        own = !any_before<D>(in.bits, sampleBase, g.nIn, g.size, w, off);
-        if (own && g.mode == MODE_SQ_MIN)
-          own = count_active<D, false>(in.bits, sampleBase, g.nIn, g.size, w) >=
-                g.minActive;
-        if (own && g.mode == MODE_TRI_MIN)
-          own = count_active<D, true>(in.bits, sampleBase, g.nIn, g.size, w) >=
-                g.minActive;
-      }
-      if (own)
-        f(encode_key<D>(j, g.nOut));
-    }
+  for (int c = 0;; ++c) {
+    if (owns<D>(in, g, sampleBase, i, j))
+      f(encode_key<D>(j, g.nOut), c);
     // odometer, last axis fastest
     int a = D - 1;
     for (; a >= 0; --a) {
@@ -326,7 +347,8 @@ __global__ void k_grid_build(GridView g, const int *sample,
 // position in iteration order
 template <int D>
 __global__ void k_plan_count(GridView in, Geom g, const long long *ekey,
-                             long long nEntries, unsigned *cntByRank) {
+                             long long nEntries, unsigned *cntByRank,
+                             unsigned long long *ownMask, unsigned *rankOf) {
   long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (e >= nEntries)
     return;
@@ -334,17 +356,27 @@ __global__ void k_plan_count(GridView in, Geom g, const long long *ekey,
   int b = (int)(p / g.volIn);
   int i[D];
   decode_key<D>(p - (long long)b * g.volIn, g.nIn, i);
-  unsigned c = 0;
-  for_each_owned<D>(in, g, b, i, [&](long long) { ++c; });
-  cntByRank[rank_of(in, p)] = c;
+  unsigned n = 0;
+  unsigned long long mask = 0;
+  for_each_owned<D>(in, g, b, i, [&](long long, int c) {
+    ++n;
+    mask |= 1ull << (c & 63);
+  });
+  unsigned r = rank_of(in, p);
+  cntByRank[r] = n;
+  if (ownMask) { // only when a box never has more than 64 candidates
+    ownMask[e] = mask; // kept per entry, with the rank, so that the emit pass
+    rankOf[e] = r;     // reads them without walking the mask again
+  }
 }
 
 // per sample: does it need a background row, and how many were appended
-// before it.  One block.
-__global__ void k_plan_samples(GridView in, const unsigned *base,
-                               long long nEntries, long long fullSize,
-                               int *outBg, int *bgBefore,
-                               unsigned *sampleStart, long long *scalars) {
+// before it.  One block of 1024 lanes.
+__device__ __forceinline__ void
+plan_samples_body(const GridView &in, const unsigned *base, long long nEntries,
+                  long long fullSize, int *outBg, int *bgBefore,
+                  unsigned *sampleStart, volatile long long *scalars,
+                  const long long *badSites) {
   __shared__ int lds[1024];
   __shared__ int carry;
   const int t = threadIdx.x;
@@ -386,6 +418,29 @@ __global__ void k_plan_samples(GridView in, const unsigned *base,
   }
 }
 
+__global__ void __launch_bounds__(1024)
+    k_plan_samples(GridView in, const unsigned *base, long long nEntries,
+                   long long fullSize, int *outBg, int *bgBefore,
+                   unsigned *sampleStart, long long *scalars,
+                   const long long *badSites) {
+  plan_samples_body(in, base, nEntries, fullSize, outBg, bgBefore, sampleStart,
+                    scalars, badSites);
+}
+
+// small batches: prefix sum of the owned counts and the per-sample pass in
+// one launch
+__global__ void __launch_bounds__(1024)
+    k_plan_scan_samples(GridView in, const unsigned *cnt, unsigned *base,
+                        long long nEntries, long long fullSize, int *outBg,
+                        int *bgBefore, unsigned *sampleStart,
+                        long long *scalars, const long long *badSites) {
+  __shared__ uint32_t ldsScan[17];
+  (void)block_scan_loop<false>(cnt, base, (size_t)nEntries, ldsScan);
+  __syncthreads(); // the block's own writes to base[] are visible to it
+  plan_samples_body(in, base, nEntries, fullSize, outBg, bgBefore, sampleStart,
+                    scalars, badSites);
+}
+
 // pass 2: emit the owned outputs
 template <int D>
 __global__ void k_plan_emit(GridView in, GridView out, Geom g,
@@ -407,7 +462,7 @@ __global__ void k_plan_emit(GridView in, GridView out, Geom g,
   decode_key<D>(p - (long long)b * g.volIn, g.nIn, i);
   unsigned idx = base[rank_of(in, p)];
   const int shiftRows = bgBefore[b];
-  for_each_owned<D>(in, g, b, i, [&](long long outKey) {
+  for_each_owned<D>(in, g, b, i, [&](long long outKey, int) {
     long long po = (long long)b * g.volOut + outKey;
     int row = (int)idx + shiftRows;
     hash_insert(out.table, out.shift, out.mask, po, row);
@@ -417,6 +472,64 @@ __global__ void k_plan_emit(GridView in, GridView out, Geom g,
     siteKey[row] = po;
     ++idx;
   });
+}
+
+// pass 2 when the ownership masks are available: one lane per (input,
+// candidate), candidate index on blockIdx.y, so no lane walks a chain of
+// dependent atomics.
+template <int D>
+__global__ void k_plan_emit_masked(GridView in, GridView out, Geom g,
+                                   const long long *ekey, long long nEntries,
+                                   const unsigned *base,
+                                   const unsigned long long *ownMask,
+                                   const unsigned *rankOf,
+                                   const int *bgBefore, const int *outBg,
+                                   long long *okey, int *orow,
+                                   long long *siteKey) {
+  long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const int c = blockIdx.y;
+  if (c == 0 && e < in.batch) { // background rows
+    int r = outBg[e];
+    if (r >= 0)
+      siteKey[r] = -1 - e;
+  }
+  if (e >= nEntries)
+    return;
+  unsigned long long mask = ownMask[e];
+  if (!((mask >> c) & 1ull))
+    return;
+  long long p = ekey[e];
+  unsigned r = rankOf[e];
+  int b = (int)(p / g.volIn);
+  int i[D], lo[D], hi[D], j[D];
+  decode_key<D>(p - (long long)b * g.volIn, g.nIn, i);
+  (void)cand_box<D>(g, i, lo, hi);
+  int rem = c;
+#pragma unroll
+  for (int a = D - 1; a >= 0; --a) {
+    int ext = hi[a] - lo[a];
+    j[a] = lo[a] + rem % ext;
+    rem /= ext;
+  }
+  unsigned idx = base[r] + (unsigned)__popcll(mask & ((1ull << c) - 1ull));
+  long long po = (long long)b * g.volOut + encode_key<D>(j, g.nOut);
+  int row = (int)idx + bgBefore[b];
+  hash_insert(out.table, out.shift, out.mask, po, row);
+  atomicOr(&out.bits[po >> 6], 1ull << (po & 63));
+  okey[idx] = po;
+  orow[idx] = row;
+  siteKey[row] = po;
+}
+
+// clears a hash table (all-ones = empty slots) and an occupancy mask at once
+__global__ void k_clear_grid(uint4 *slots, size_t nSlots,
+                             unsigned long long *bits, size_t nWords) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  size_t step = (size_t)gridDim.x * blockDim.x;
+  for (size_t k = i; k < nSlots; k += step)
+    slots[k] = make_uint4(0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu);
+  for (size_t k = i; k < nWords; k += step)
+    bits[k] = 0ull;
 }
 
 // inverse of RegularTriangularRegions::ord (Regions.cu:810-826)
@@ -622,8 +735,16 @@ static int grids_prepare(scn_ctx *ctx, scn_grids *g, int batch, int d, int n,
   SCN_TRY(g->ekey.reserve((size_t)nActive + 1));
   SCN_TRY(g->erow.reserve((size_t)nActive + 1));
   SCN_TRY(g->bg.reserve((size_t)batch + 1));
-  SCN_TRY(scn_fill32(ctx, g->table.p, 0xFFFFFFFFu, cap * 4));
-  SCN_TRY(scn_fill32(ctx, g->bits.p, 0u, (g->nWords + 2) * 2));
+  {
+    size_t most = cap > g->nWords + 2 ? cap : g->nWords + 2;
+    size_t blocks = (most + 255) / 256;
+    if (blocks > 16384)
+      blocks = 16384;
+    hipLaunchKernelGGL(k_clear_grid, dim3((unsigned)blocks), dim3(256), 0,
+                       ctx->stream, (uint4 *)g->table.p, cap, g->bits.p,
+                       g->nWords + 2);
+    SCN_HIP_CHECK(hipGetLastError());
+  }
   return SCN_OK;
 }
 
@@ -646,6 +767,7 @@ static int read_scalars(scn_ctx *ctx) {
   SCN_HIP_CHECK(hipStreamSynchronize(ctx->stream));
   if (ctx->h_pinned[15] != 0) {
     long long bad = ctx->h_pinned[15];
+    ctx->h_pinned[15] = 0;
     SCN_TRY(scn_fill32(ctx, ctx->d_scalars + 15, 0u, 2));
     SCN_REQUIRE(false, SCN_ERR_ARG,
                 "scn_grids_build was given %lld sites outside the field", bad);
@@ -673,6 +795,8 @@ extern "C" int scn_grids_destroy(scn_ctx *ctx, scn_grids *g) {
   g->scanTmp.release();
   g->siteKey.release();
   g->cnt.release();
+  g->ownMask.release();
+  g->rankOf.release();
   g->base.release();
   g->bgBefore.release();
   g->sampleStart.release();
@@ -784,16 +908,34 @@ static int plan_regions_d(scn_ctx *ctx, scn_grids *in, scn_grids *out,
   SCN_TRY(out->bg.reserve((size_t)in->batch + 1));
   SCN_TRY(out->scanTmp.reserve(scn_scan_tmp_elems((size_t)nE + 1)));
   GridView vin = view_of(in);
+  // number of candidates of one input: (ceil(size / stride))^d at most
+  long long maxCand = 1;
+  for (int a = 0; a < D; ++a)
+    maxCand *= g.mode == MODE_SQ_VALID ? 1 : (g.size + g.stride - 1) / g.stride;
+  const bool masked = maxCand <= 64;
+  if (masked) {
+    SCN_TRY(out->ownMask.reserve((size_t)nE + 2));
+    SCN_TRY(out->rankOf.reserve((size_t)nE + 2));
+  }
   if (nE > 0) {
     hipLaunchKernelGGL(k_plan_count<D>, dim3(scn_ceil_div(nE, 256)), dim3(256),
-                       0, ctx->stream, vin, g, in->ekey.p, nE, out->cnt.p);
+                       0, ctx->stream, vin, g, in->ekey.p, nE, out->cnt.p,
+                       masked ? out->ownMask.p : nullptr, out->rankOf.p);
     SCN_HIP_CHECK(hipGetLastError());
   }
-  SCN_TRY(scn_scan_exclusive_u32(ctx->stream, out->cnt.p, out->base.p,
-                                 (size_t)nE, out->scanTmp.p));
-  hipLaunchKernelGGL(k_plan_samples, dim3(1), dim3(1024), 0, ctx->stream, vin,
-                     out->base.p, nE, fullSize, out->bg.p, out->bgBefore.p,
-                     out->sampleStart.p, (long long *)ctx->d_scalars);
+  const long long *bad = (const long long *)(ctx->d_scalars + 15);
+  if ((size_t)nE <= SCAN1_MAX_ELEMS) {
+    hipLaunchKernelGGL(k_plan_scan_samples, dim3(1), dim3(1024), 0, ctx->stream,
+                       vin, out->cnt.p, out->base.p, nE, fullSize, out->bg.p,
+                       out->bgBefore.p, out->sampleStart.p,
+                       (long long *)ctx->d_scalars, bad);
+  } else {
+    SCN_TRY(scn_scan_exclusive_u32(ctx->stream, out->cnt.p, out->base.p,
+                                   (size_t)nE, out->scanTmp.p));
+    hipLaunchKernelGGL(k_plan_samples, dim3(1), dim3(1024), 0, ctx->stream, vin,
+                       out->base.p, nE, fullSize, out->bg.p, out->bgBefore.p,
+                       out->sampleStart.p, (long long *)ctx->d_scalars, bad);
+  }
   SCN_HIP_CHECK(hipGetLastError());
   SCN_TRY(read_scalars(ctx));
   long long nSites = ctx->h_pinned[0], nOutActive = ctx->h_pinned[1];
@@ -805,7 +947,15 @@ static int plan_regions_d(scn_ctx *ctx, scn_grids *in, scn_grids *out,
   out->nSites = (int)nSites;
   SCN_TRY(out->siteKey.reserve((size_t)nSites + 1));
   long long nThreads = nE > in->batch ? nE : in->batch;
-  if (nThreads > 0) {
+  if (nThreads > 0 && masked) {
+    hipLaunchKernelGGL(k_plan_emit_masked<D>,
+                       dim3(scn_ceil_div(nThreads, 256), (unsigned)maxCand),
+                       dim3(256), 0, ctx->stream, vin, view_of(out), g,
+                       in->ekey.p, nE, out->base.p, out->ownMask.p,
+                       out->rankOf.p, out->bgBefore.p, out->bg.p, out->ekey.p,
+                       out->erow.p, out->siteKey.p);
+    SCN_HIP_CHECK(hipGetLastError());
+  } else if (nThreads > 0) {
     hipLaunchKernelGGL(k_plan_emit<D>, dim3(scn_ceil_div(nThreads, 256)),
                        dim3(256), 0, ctx->stream, vin, view_of(out), g,
                        in->ekey.p, nE, out->base.p, out->bgBefore.p, out->bg.p,

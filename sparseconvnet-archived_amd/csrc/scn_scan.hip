@@ -1,6 +1,7 @@
 // Exclusive prefix sums over uint32 counts (or popcounts of 64-bit words),
 // three-phase: per-tile totals, recursive scan of the totals, per-tile rescan.
 #include "scn_common.h"
+#include "scn_scan_dev.h"
 
 #define SCAN_THREADS 256
 #define SCAN_PER_THREAD 8
@@ -77,6 +78,13 @@ __global__ void __launch_bounds__(SCAN_THREADS)
     out[n] = off + total;
 }
 
+template <bool POPC>
+__global__ void __launch_bounds__(SCAN1_THREADS)
+    k_scan_single(const void *in, uint32_t *out, size_t n) {
+  __shared__ uint32_t lds[17];
+  (void)block_scan_loop<POPC>(in, out, n, lds);
+}
+
 size_t scn_scan_tmp_elems(size_t n) {
   size_t total = 0;
   while (n > SCAN_TILE) {
@@ -90,8 +98,14 @@ size_t scn_scan_tmp_elems(size_t n) {
 template <bool POPC>
 static int scan_impl(hipStream_t s, const void *in, uint32_t *out, size_t n,
                      uint32_t *tmp) {
+  if (n <= SCAN1_MAX_ELEMS) { // one launch; n == 0 still writes out[0] = 0
+    hipLaunchKernelGGL(k_scan_single<POPC>, dim3(1), dim3(SCAN1_THREADS), 0, s,
+                       in, out, n);
+    SCN_HIP_CHECK(hipGetLastError());
+    return SCN_OK;
+  }
   size_t nb = (n + SCAN_TILE - 1) / SCAN_TILE;
-  if (nb <= 1) { // n == 0 still writes out[0] = 0
+  if (nb <= 1) {
     hipLaunchKernelGGL(k_scan_final<POPC>, dim3(1), dim3(SCAN_THREADS), 0, s, in,
                        out, n, (const uint32_t *)nullptr);
     SCN_HIP_CHECK(hipGetLastError());
