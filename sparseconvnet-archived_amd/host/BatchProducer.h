@@ -1,7 +1,10 @@
-// Builds batches for processDataset (BatchProducer.h:8-25).  Worker threads
-// run the CPU part (distort + codifyInputData) one batch slot each;
-// nextBatch() uploads the slot and issues every layer's preprocess() -- the
-// rule-book kernels -- from the calling thread, on the net's stream.
+// Builds batches for processDataset (BatchProducer.h:8-25).  As in the
+// reference, each worker thread owns one batch slot and runs the whole
+// preprocessing of its batches: distort + codifyInputData on the CPU, then the
+// upload of the input sites and every layer's preprocess() -- here GPU rule-book
+// kernels -- on the slot's own stream.  nextBatch() hands finished slots to the
+// caller in order, so rule books of the next batches are built while the
+// forward pass of the current one runs on the net's stream.
 #pragma once
 #include <condition_variable>
 #include <thread>
@@ -22,6 +25,9 @@ public:
   std::vector<int> permutation;
   BatchProducer(SparseConvNetCUDA &cnn, SpatiallySparseDataset &dataset,
                 int spatialSize, int batchSize);
+  // nBatches passes over one batch that is resident in HBM (benchmarking)
+  BatchProducer(SparseConvNetCUDA &cnn, const ResidentBatch &resident,
+                int nBatches);
   ~BatchProducer();
   SpatiallySparseBatch *nextBatch();
   void batchProducerThread(int nThread);
@@ -31,6 +37,10 @@ public:
   void preprocessBatchOnDevice(int cc);
 
 private:
+  static SpatiallySparseDataset emptyDataset;
+  const ResidentBatch *resident;
+  ResidentBatch residentCopy;
+  void start();
   std::vector<char> slotFull;
   std::condition_variable slotChanged;
   std::mutex slotMutex;

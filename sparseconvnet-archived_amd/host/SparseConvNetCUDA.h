@@ -14,6 +14,20 @@
 
 #define N_MAX_BATCH_PRODUCER_THREADS 20
 
+// A batch whose input is already in HBM: active sites (sample, key, row),
+// backgroundCol per sample, and the feature matrix [nSpatialSites x
+// nInputFeatures]; all device pointers.
+struct ResidentBatch {
+  int batchSize;
+  const int32_t *d_sample;
+  const int64_t *d_key;
+  const int32_t *d_row;
+  const int32_t *d_background;
+  int64_t nActive;
+  int nSpatialSites;
+  const float *d_features;
+};
+
 class SparseConvNetCUDA {
 public:
   cudaMemStream memStream; // first member: the context outlives every buffer
@@ -27,6 +41,11 @@ public:
   int nOutputFeatures;
   int deviceID;
   int nBatchProducerThreads;
+  // one stream per batch slot: the slot's producer thread issues the grid
+  // upload and the rule-book kernels of its batch there, while the forward
+  // pass of another batch runs on memStream (the reference declares the same
+  // array, SparseConvNetCUDA.h:38, and leaves it unused)
+  std::vector<std::unique_ptr<cudaMemStream>> batchMemStreams;
   std::mutex batchLock[N_MAX_BATCH_PRODUCER_THREADS];
   std::vector<SpatiallySparseBatch> batchPool;
   std::vector<SpatiallySparseBatchSubInterface *> initialSubInterfaces;
@@ -73,4 +92,9 @@ public:
   void saveWeights(std::string baseName, int epoch, bool momentum);
   // set the operand precision of every NiN contraction (SCN_FP32 / SCN_BF16)
   void setPrecision(int precision);
+  // grows every slot's interface list to layers.size() + 1
+  void ensureInterfaces();
+  // Fills slot cc's input interface from a batch that already sits in HBM
+  // (see ResidentBatch) and builds every rule book, on the slot's stream.
+  void preprocessResident(int cc, const struct ResidentBatch &input);
 };

@@ -11,6 +11,9 @@ class SpatiallySparseBatch {
 public:
   SpatiallySparseBatch(SpatiallySparseBatchSubInterface *inputSub);
   SpatiallySparseBatch(SpatiallySparseBatch &&) = default;
+  // The stream this slot's preprocess() -- grid upload and rule-book kernels
+  // -- is issued on (one of the net's batchMemStreams); null: the layer's own.
+  cudaMemStream *preprocessStream;
   batchType type;
   int batchSize;
   std::vector<int> sampleNumbers;
@@ -20,5 +23,8 @@ public:
   std::vector<std::vector<float>> probabilities;
   float negativeLogLikelihood;
   int mistakes;
+  // device staging of the input sites (sample, key as two ints, row,
+  // backgroundCol), reused from batch to batch
+  vectorCUDA<int> stagingSample, stagingKey, stagingRow, stagingBackground;
   void reset();
 };

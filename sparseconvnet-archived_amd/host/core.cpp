@@ -104,7 +104,7 @@ std::vector<int> RNG::NchooseM(int n, int m) {
 
 // ---- context --------------------------------------------------------------------
 static scn_ctx *g_defaultCtx = nullptr;
-static int g_ctxUsers = 0;
+static std::vector<scn_ctx *> g_liveCtx; // oldest first
 static std::mutex g_ctxMutex;
 
 void scnCheck(int rc, const char *file, int line) {
@@ -122,19 +122,17 @@ scn_ctx *scnDefaultContext() {
   }
   return g_defaultCtx;
 }
-cudaMemStream::cudaMemStream() {
+cudaMemStream::cudaMemStream() : ctx(nullptr) {
   std::lock_guard<std::mutex> lock(g_ctxMutex);
-  if (!g_defaultCtx)
-    SCN_CHECKED(scn_ctx_create(-1, &g_defaultCtx));
-  ++g_ctxUsers;
-  ctx = g_defaultCtx;
+  SCN_CHECKED(scn_ctx_create(-1, &ctx));
+  g_liveCtx.push_back(ctx);
+  g_defaultCtx = g_liveCtx.front();
 }
 cudaMemStream::~cudaMemStream() {
   std::lock_guard<std::mutex> lock(g_ctxMutex);
-  if (--g_ctxUsers == 0) {
-    scn_ctx_destroy(g_defaultCtx);
-    g_defaultCtx = nullptr;
-  }
+  g_liveCtx.erase(std::find(g_liveCtx.begin(), g_liveCtx.end(), ctx));
+  g_defaultCtx = g_liveCtx.empty() ? nullptr : g_liveCtx.front();
+  scn_ctx_destroy(ctx);
 }
 void *cudaMemStream::stream() const { return scn_ctx_stream(ctx); }
 void cudaMemStream::synchronize() const { SCN_CHECKED(scn_sync(ctx)); }
@@ -159,38 +157,44 @@ vectorCUDA<t>::vectorCUDA(vectorCUDA &&o)
   o.dAllocated = 0;
 }
 template <typename t> vectorCUDA<t>::~vectorCUDA() {
-  if (d_vec && g_defaultCtx)
-    scn_free(g_defaultCtx, d_vec);
+  if (d_vec)
+    scn_free(nullptr, d_vec);
 }
 template <typename t> void vectorCUDA<t>::copyToCPU() {
   if (!onGPU)
     return;
-  onGPU = false;
-  vec.resize(dsize);
-  if (dsize > 0)
-    SCN_CHECKED(scn_d2h(scnDefaultContext(), vec.data(), d_vec,
-                        sizeof(t) * (size_t)dsize));
+  toCPU(scnDefaultContext());
 }
 template <typename t> void vectorCUDA<t>::copyToGPU() {
   if (onGPU)
     return;
+  toGPU(scnDefaultContext());
+}
+template <typename t> void vectorCUDA<t>::toCPU(scn_ctx *ctx) {
+  onGPU = false;
+  vec.resize(dsize);
+  if (dsize > 0)
+    SCN_CHECKED(scn_d2h(ctx, vec.data(), d_vec, sizeof(t) * (size_t)dsize));
+}
+template <typename t> void vectorCUDA<t>::toGPU(scn_ctx *ctx) {
   onGPU = true;
   dsize = 0;
   resize64(vec.size());
   if (dsize > 0)
-    SCN_CHECKED(scn_h2d(scnDefaultContext(), d_vec, vec.data(),
-                        sizeof(t) * (size_t)dsize));
+    SCN_CHECKED(scn_h2d(ctx, d_vec, vec.data(), sizeof(t) * (size_t)dsize));
   vec.clear();
 }
+// the copies go on the named stream and return when they are done, as the
+// reference's do (vectorCUDA.cu:58-108 synchronise the stream)
 template <typename t>
 void vectorCUDA<t>::copyToCPUAsync(cudaMemStream &memStream) {
-  (void)memStream; // the context's stream; the copy returns when it is done
-  copyToCPU();
+  if (onGPU)
+    toCPU(memStream.ctx);
 }
 template <typename t>
 void vectorCUDA<t>::copyToGPUAsync(cudaMemStream &memStream) {
-  (void)memStream;
-  copyToGPU();
+  if (!onGPU)
+    toGPU(memStream.ctx);
 }
 template <typename t> t *&vectorCUDA<t>::dPtr() {
   copyToGPU();
@@ -245,12 +249,11 @@ template <typename t> void vectorCUDA<t>::resize64(size_t n) {
     return;
   }
   if (n > dAllocated) {
-    scn_ctx *ctx = scnDefaultContext();
     if (d_vec)
-      SCN_CHECKED(scn_free(ctx, d_vec));
+      SCN_CHECKED(scn_free(nullptr, d_vec));
     size_t want = n + n / 4;
     void *p = nullptr;
-    SCN_CHECKED(scn_malloc(ctx, want * sizeof(t), &p));
+    SCN_CHECKED(scn_malloc(scnDefaultContext(), want * sizeof(t), &p));
     d_vec = (t *)p;
     dAllocated = want;
   }
@@ -325,7 +328,9 @@ void SpatiallySparseBatchInterface::summary() {
 
 SpatiallySparseBatch::SpatiallySparseBatch(
     SpatiallySparseBatchSubInterface *inputSub)
-    : inputSub(inputSub), labels(false, 0) {
+    : inputSub(inputSub), preprocessStream(nullptr), labels(false, 0),
+      stagingSample(true, 0), stagingKey(true, 0), stagingRow(true, 0),
+      stagingBackground(true, 0) {
   interfaces.emplace_back(inputSub);
   reset();
 }

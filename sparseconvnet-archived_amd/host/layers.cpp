@@ -27,13 +27,19 @@ void SpatiallySparseLayer::backwards(SpatiallySparseBatch &,
   unsupported("backwards()");
 }
 
+// preprocess() runs on the batch slot's own stream when it has one, so that
+// rule books of several batches are built side by side
+static scn_ctx *pre_ctx(SpatiallySparseBatch &batch, cudaMemStream &ms) {
+  return batch.preprocessStream ? batch.preprocessStream->ctx : ms.ctx;
+}
+
 // the output interface's own grids object, created on first use and kept for
 // later batches (its tables only grow)
-static scn_grids *own_grids(cudaMemStream &ms,
+static scn_grids *own_grids(scn_ctx *ctx,
                             SpatiallySparseBatchInterface &output) {
   if (!output.deviceGrids || !output.ownsDeviceGrids) {
     scn_grids *g = nullptr;
-    SCN_CHECKED(scn_grids_create(ms.ctx, &g));
+    SCN_CHECKED(scn_grids_create(ctx, &g));
     output.deviceGrids = g;
     output.ownsDeviceGrids = true;
   }
@@ -49,11 +55,11 @@ static void share_grids(SpatiallySparseBatchInterface &input,
   output.ownsDeviceGrids = false;
 }
 
-static void fill_rules(cudaMemStream &ms, SpatiallySparseBatchInterface &input,
+static void fill_rules(scn_ctx *ctx, SpatiallySparseBatchInterface &input,
                        SpatiallySparseBatchInterface &output, int64_t nRules) {
   output.rules.copyToGPU();
   output.rules.resize64((size_t)nRules);
-  SCN_CHECKED(scn_rules_fill(ms.ctx, input.deviceGrids, output.deviceGrids,
+  SCN_CHECKED(scn_rules_fill(ctx, input.deviceGrids, output.deviceGrids,
                              output.rules.dPtr(), nRules));
 }
 
@@ -88,7 +94,7 @@ ConvolutionalLayer::ConvolutionalLayer(cudaMemStream &memStream,
 void ConvolutionalLayer::preprocess(SpatiallySparseBatch &batch,
                                     SpatiallySparseBatchInterface &input,
                                     SpatiallySparseBatchInterface &output) {
-  (void)batch;
+  scn_ctx *ctx = pre_ctx(batch, memStream);
   assert(input.nFeatures == nFeaturesIn);
   assert(input.spatialSize >= filterSize);
   assert((input.spatialSize - filterSize) % filterStride == 0);
@@ -96,12 +102,12 @@ void ConvolutionalLayer::preprocess(SpatiallySparseBatch &batch,
   output.spatialSize = (input.spatialSize - filterSize) / filterStride + 1;
   output.backpropErrors = input.backpropErrors;
   int64_t n = 0;
-  SCN_CHECKED(scn_rules_square_plan(memStream.ctx, input.deviceGrids,
-                                    own_grids(memStream, output),
-                                    inSpatialSize, outSpatialSize, filterSize,
-                                    filterStride, minActiveInputs, &n));
+  SCN_CHECKED(scn_rules_square_plan(ctx, input.deviceGrids,
+                                    own_grids(ctx, output), inSpatialSize,
+                                    outSpatialSize, filterSize, filterStride,
+                                    minActiveInputs, &n));
   output.nSpatialSites = (int)n;
-  fill_rules(memStream, input, output, n * fs);
+  fill_rules(ctx, input, output, n * fs);
   convolutionFeaturesPresent(input.featuresPresent.hVector(),
                              output.featuresPresent.hVector(), input.nFeatures,
                              (int)input.featuresPresent.size(), fs);
@@ -145,7 +151,7 @@ ConvolutionalTriangularLayer::ConvolutionalTriangularLayer(
 void ConvolutionalTriangularLayer::preprocess(
     SpatiallySparseBatch &batch, SpatiallySparseBatchInterface &input,
     SpatiallySparseBatchInterface &output) {
-  (void)batch;
+  scn_ctx *ctx = pre_ctx(batch, memStream);
   assert(input.nFeatures == nFeaturesIn);
   assert(input.spatialSize >= filterSize);
   assert((input.spatialSize - filterSize) % filterStride == 0);
@@ -154,11 +160,10 @@ void ConvolutionalTriangularLayer::preprocess(
   output.backpropErrors = input.backpropErrors;
   int64_t n = 0;
   SCN_CHECKED(scn_rules_triangular_plan(
-      memStream.ctx, input.deviceGrids, own_grids(memStream, output),
-      inSpatialSize, outSpatialSize, filterSize, filterStride, minActiveInputs,
-      &n));
+      ctx, input.deviceGrids, own_grids(ctx, output), inSpatialSize,
+      outSpatialSize, filterSize, filterStride, minActiveInputs, &n));
   output.nSpatialSites = (int)n;
-  fill_rules(memStream, input, output, n * fs);
+  fill_rules(ctx, input, output, n * fs);
   convolutionFeaturesPresent(input.featuresPresent.hVector(),
                              output.featuresPresent.hVector(), input.nFeatures,
                              (int)input.featuresPresent.size(), fs);
@@ -358,19 +363,19 @@ MaxPoolingLayer::MaxPoolingLayer(cudaMemStream &memStream, int poolSize,
 void MaxPoolingLayer::preprocess(SpatiallySparseBatch &batch,
                                  SpatiallySparseBatchInterface &input,
                                  SpatiallySparseBatchInterface &output) {
-  (void)batch;
+  scn_ctx *ctx = pre_ctx(batch, memStream);
   assert(input.spatialSize == inSpatialSize);
   output.nFeatures = input.nFeatures;
   output.featuresPresent.hVector() = input.featuresPresent.hVector();
   output.spatialSize = outSpatialSize;
   output.backpropErrors = input.backpropErrors;
   int64_t n = 0;
-  SCN_CHECKED(scn_rules_square_plan(memStream.ctx, input.deviceGrids,
-                                    own_grids(memStream, output),
-                                    inSpatialSize, outSpatialSize, poolSize,
-                                    poolStride, 1, &n));
+  SCN_CHECKED(scn_rules_square_plan(ctx, input.deviceGrids,
+                                    own_grids(ctx, output), inSpatialSize,
+                                    outSpatialSize, poolSize, poolStride, 1,
+                                    &n));
   output.nSpatialSites = (int)n;
-  fill_rules(memStream, input, output, n * sd);
+  fill_rules(ctx, input, output, n * sd);
 }
 static void pool_forwards(cudaMemStream &ms,
                           SpatiallySparseBatchInterface &input,
@@ -414,18 +419,19 @@ MaxPoolingTriangularLayer::MaxPoolingTriangularLayer(cudaMemStream &memStream,
 void MaxPoolingTriangularLayer::preprocess(
     SpatiallySparseBatch &batch, SpatiallySparseBatchInterface &input,
     SpatiallySparseBatchInterface &output) {
-  (void)batch;
+  scn_ctx *ctx = pre_ctx(batch, memStream);
   assert(input.spatialSize == inSpatialSize);
   output.nFeatures = input.nFeatures;
   output.featuresPresent.hVector() = input.featuresPresent.hVector();
   output.spatialSize = outSpatialSize;
   output.backpropErrors = input.backpropErrors;
   int64_t n = 0;
-  SCN_CHECKED(scn_rules_triangular_plan(
-      memStream.ctx, input.deviceGrids, own_grids(memStream, output),
-      inSpatialSize, outSpatialSize, poolSize, poolStride, 1, &n));
+  SCN_CHECKED(scn_rules_triangular_plan(ctx, input.deviceGrids,
+                                        own_grids(ctx, output), inSpatialSize,
+                                        outSpatialSize, poolSize, poolStride, 1,
+                                        &n));
   output.nSpatialSites = (int)n;
-  fill_rules(memStream, input, output, n * S);
+  fill_rules(ctx, input, output, n * S);
 }
 void MaxPoolingTriangularLayer::forwards(SpatiallySparseBatch &batch,
                                          SpatiallySparseBatchInterface &input,
@@ -459,11 +465,12 @@ void TerminalPoolingLayer::preprocess(SpatiallySparseBatch &batch,
   output.featuresPresent.hVector() = input.featuresPresent.hVector();
   output.spatialSize = outSpatialSize;
   output.backpropErrors = input.backpropErrors;
+  scn_ctx *ctx = pre_ctx(batch, memStream);
   int64_t width = 0;
-  SCN_CHECKED(scn_rules_terminal_plan(memStream.ctx, input.deviceGrids,
-                                      own_grids(memStream, output), &width));
+  SCN_CHECKED(scn_rules_terminal_plan(ctx, input.deviceGrids,
+                                      own_grids(ctx, output), &width));
   output.nSpatialSites = batch.batchSize;
-  fill_rules(memStream, input, output, width * batch.batchSize);
+  fill_rules(ctx, input, output, width * batch.batchSize);
 }
 void TerminalPoolingLayer::forwards(SpatiallySparseBatch &batch,
                                     SpatiallySparseBatchInterface &input,

@@ -30,9 +30,13 @@ SparseConvNetCUDA::SparseConvNetCUDA(int dimension, int nInputFeatures,
   for (int c = 0; c < nBatchProducerThreads; c++) {
     initialSubInterfaces.push_back(new SpatiallySparseBatchSubInterface());
     batchPool.emplace_back(initialSubInterfaces.back());
+    batchMemStreams.emplace_back(new cudaMemStream());
+    batchPool.back().preprocessStream = batchMemStreams.back().get();
   }
 }
 SparseConvNetCUDA::~SparseConvNetCUDA() {
+  for (auto &s : batchMemStreams)
+    s->synchronize();
   memStream.synchronize();
   batchPool.clear();
   for (auto p : layers)
@@ -147,6 +151,46 @@ void SparseConvNetCUDA::addSoftmaxLayer() {
   for (int i = 1; i < dimension; ++i)
     std::cout << "x" << inputSpatialSize;
   std::cout << std::endl;
+}
+void SparseConvNetCUDA::ensureInterfaces() {
+  // one shared sub-interface per depth, one interface per depth and slot
+  // (BatchProducer.cu:28-33)
+  while (batchPool[0].interfaces.size() <= layers.size()) {
+    sharedSubInterfaces.push_back(new SpatiallySparseBatchSubInterface());
+    for (auto &slot : batchPool)
+      slot.interfaces.emplace_back(sharedSubInterfaces.back());
+  }
+}
+void SparseConvNetCUDA::preprocessResident(int cc, const ResidentBatch &input) {
+  SpatiallySparseBatch &b = batchPool[cc];
+  scn_ctx *ctx = b.preprocessStream ? b.preprocessStream->ctx : memStream.ctx;
+  b.reset();
+  b.type = UNLABELEDBATCH;
+  b.batchSize = input.batchSize;
+  SpatiallySparseBatchInterface &in = b.interfaces[0];
+  in.nFeatures = nInputFeatures;
+  in.spatialSize = inputSpatialSize;
+  in.nSpatialSites = input.nSpatialSites;
+  in.featuresPresent.hVector() = range(nInputFeatures);
+  if (!in.deviceGrids) {
+    SCN_CHECKED(scn_grids_create(ctx, &in.deviceGrids));
+    in.ownsDeviceGrids = true;
+  }
+  scn_prof_tag(ctx, -1);
+  SCN_CHECKED(scn_grids_build(ctx, in.deviceGrids, input.batchSize, dimension,
+                              in.spatialSize, input.d_sample, input.d_key,
+                              input.d_row, input.nActive, input.d_background,
+                              input.nSpatialSites));
+  in.sub->features.copyToGPU();
+  size_t nElems = (size_t)input.nSpatialSites * nInputFeatures;
+  in.sub->features.resize64(nElems);
+  SCN_CHECKED(scn_d2d(ctx, in.sub->features.dPtr(), input.d_features,
+                      nElems * sizeof(float)));
+  for (size_t i = 0; i < layers.size(); i++) {
+    scn_prof_tag(ctx, (int)i);
+    layers[i]->preprocess(b, b.interfaces[i], b.interfaces[i + 1]);
+  }
+  SCN_CHECKED(scn_sync(ctx));
 }
 void SparseConvNetCUDA::setPrecision(int precision) {
   for (auto *l : layers) {
@@ -329,20 +373,27 @@ void SparseConvNetCUDA::saveWeights(std::string baseName, int epoch,
 }
 
 // ========================================================== batch producer
+SpatiallySparseDataset BatchProducer::emptyDataset;
+
 BatchProducer::BatchProducer(SparseConvNetCUDA &cnn,
                              SpatiallySparseDataset &dataset, int spatialSize,
                              int batchSize)
     : cnn(cnn), batchCounter(-1), dataset(dataset), batchSize(batchSize),
-      spatialSize(spatialSize), stopping(false) {
+      spatialSize(spatialSize), resident(nullptr), stopping(false) {
   assert(batchSize > 0);
   nBatches = ((int)dataset.pictures.size() + batchSize - 1) / batchSize;
   permutation = range((int)dataset.pictures.size());
-  // one shared sub-interface per depth, one interface per depth and slot
-  while (cnn.batchPool[0].interfaces.size() <= cnn.layers.size()) {
-    cnn.sharedSubInterfaces.push_back(new SpatiallySparseBatchSubInterface());
-    for (int c = 0; c < cnn.nBatchProducerThreads; c++)
-      cnn.batchPool[c].interfaces.emplace_back(cnn.sharedSubInterfaces.back());
-  }
+  start();
+}
+BatchProducer::BatchProducer(SparseConvNetCUDA &cnn,
+                             const ResidentBatch &residentBatch, int nBatches)
+    : cnn(cnn), batchCounter(-1), nBatches(nBatches), dataset(emptyDataset),
+      batchSize(residentBatch.batchSize), spatialSize(cnn.inputSpatialSize),
+      resident(&residentCopy), residentCopy(residentBatch), stopping(false) {
+  start();
+}
+void BatchProducer::start() {
+  cnn.ensureInterfaces();
   slotFull.assign(cnn.nBatchProducerThreads, 0);
   for (int c = 0; c < cnn.nBatchProducerThreads; c++)
     cnn.batchPool[c].batchSize = 0;
@@ -388,10 +439,13 @@ void BatchProducer::preprocessBatch(int c, int cc, RNG &rng) {
       features[i] *= cnn.inputNormalizingConstants[i % in.nFeatures];
   }
 }
-// GPU half: the input grids go to HBM, then every layer builds its rule book
+// GPU half: the input grids go to HBM, then every layer builds its rule book,
+// all on the slot's stream
 void BatchProducer::preprocessBatchOnDevice(int cc) {
   SpatiallySparseBatch &b = cnn.batchPool[cc];
   SpatiallySparseBatchInterface &in = b.interfaces[0];
+  cudaMemStream &ms = b.preprocessStream ? *b.preprocessStream : cnn.memStream;
+  scn_ctx *ctx = ms.ctx;
   std::vector<int32_t> sample, row, bg;
   std::vector<int64_t> key;
   size_t n = 0;
@@ -408,36 +462,30 @@ void BatchProducer::preprocessBatchOnDevice(int cc) {
       row.push_back(e.second);
     }
   }
-  scn_ctx *ctx = cnn.memStream.ctx;
-  void *d_sample, *d_key, *d_row, *d_bg;
-  SCN_CHECKED(scn_malloc(ctx, n * 4, &d_sample));
-  SCN_CHECKED(scn_malloc(ctx, n * 8, &d_key));
-  SCN_CHECKED(scn_malloc(ctx, n * 4, &d_row));
-  SCN_CHECKED(scn_malloc(ctx, bg.size() * 4, &d_bg));
-  SCN_CHECKED(scn_h2d(ctx, d_sample, sample.data(), n * 4));
-  SCN_CHECKED(scn_h2d(ctx, d_key, key.data(), n * 8));
-  SCN_CHECKED(scn_h2d(ctx, d_row, row.data(), n * 4));
-  SCN_CHECKED(scn_h2d(ctx, d_bg, bg.data(), bg.size() * 4));
+  b.stagingSample.resize64(n);
+  b.stagingKey.resize64(2 * n);
+  b.stagingRow.resize64(n);
+  b.stagingBackground.resize64(bg.size());
+  SCN_CHECKED(scn_h2d(ctx, b.stagingSample.dPtr(), sample.data(), n * 4));
+  SCN_CHECKED(scn_h2d(ctx, b.stagingKey.dPtr(), key.data(), n * 8));
+  SCN_CHECKED(scn_h2d(ctx, b.stagingRow.dPtr(), row.data(), n * 4));
+  SCN_CHECKED(scn_h2d(ctx, b.stagingBackground.dPtr(), bg.data(), bg.size() * 4));
   if (!in.deviceGrids) {
     SCN_CHECKED(scn_grids_create(ctx, &in.deviceGrids));
     in.ownsDeviceGrids = true;
   }
   scn_prof_tag(ctx, -1);
   SCN_CHECKED(scn_grids_build(ctx, in.deviceGrids, b.batchSize, cnn.dimension,
-                              in.spatialSize, (const int32_t *)d_sample,
-                              (const int64_t *)d_key, (const int32_t *)d_row,
-                              (int64_t)n, (const int32_t *)d_bg,
-                              in.nSpatialSites));
-  in.sub->features.copyToGPU();
+                              in.spatialSize, b.stagingSample.dPtr(),
+                              (const int64_t *)b.stagingKey.dPtr(),
+                              b.stagingRow.dPtr(), (int64_t)n,
+                              b.stagingBackground.dPtr(), in.nSpatialSites));
+  in.sub->features.copyToGPUAsync(ms);
   for (size_t i = 0; i < cnn.layers.size(); i++) {
     scn_prof_tag(ctx, (int)i);
     cnn.layers[i]->preprocess(b, b.interfaces[i], b.interfaces[i + 1]);
   }
   SCN_CHECKED(scn_sync(ctx));
-  scn_free(ctx, d_sample);
-  scn_free(ctx, d_key);
-  scn_free(ctx, d_row);
-  scn_free(ctx, d_bg);
 }
 void BatchProducer::batchProducerThread(int nThread) {
   RNG rng;
@@ -450,7 +498,12 @@ void BatchProducer::batchProducerThread(int nThread) {
     }
     {
       std::lock_guard<std::mutex> slot(cnn.batchLock[nThread]);
-      preprocessBatch(c, nThread, rng);
+      if (resident) {
+        cnn.preprocessResident(nThread, *resident);
+      } else {
+        preprocessBatch(c, nThread, rng);
+        preprocessBatchOnDevice(nThread);
+      }
     }
     {
       std::lock_guard<std::mutex> lock(slotMutex);
@@ -481,8 +534,6 @@ SpatiallySparseBatch *BatchProducer::nextBatch() {
     std::unique_lock<std::mutex> lock(slotMutex);
     slotChanged.wait(lock, [&] { return slotFull[cc] != 0; });
   }
-  std::lock_guard<std::mutex> slot(cnn.batchLock[cc]);
-  preprocessBatchOnDevice(cc);
   return &cnn.batchPool[cc];
 }
 

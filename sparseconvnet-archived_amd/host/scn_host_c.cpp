@@ -43,8 +43,10 @@ scnh_net *scnh_net_create(int dimension, int nInputFeatures, int nClasses,
   if (nBatchProducerThreads >= 1 &&
       nBatchProducerThreads < n->cnn->nBatchProducerThreads) {
     n->cnn->nBatchProducerThreads = nBatchProducerThreads;
-    while ((int)n->cnn->batchPool.size() > nBatchProducerThreads)
+    while ((int)n->cnn->batchPool.size() > nBatchProducerThreads) {
       n->cnn->batchPool.pop_back();
+      n->cnn->batchMemStreams.pop_back();
+    }
   }
   return n;
 }
@@ -270,50 +272,66 @@ void scnh_iface_grids(scnh_net *net, int i, int32_t *sample, int64_t *key,
                                  sample, key, row, background));
 }
 
+static ResidentBatch resident_of(int batch, const int32_t *d_sample,
+                                 const int64_t *d_key, const int32_t *d_row,
+                                 const int32_t *d_background, int64_t nActive,
+                                 int nSpatialSites, const float *d_features) {
+  ResidentBatch r;
+  r.batchSize = batch;
+  r.d_sample = d_sample;
+  r.d_key = d_key;
+  r.d_row = d_row;
+  r.d_background = d_background;
+  r.nActive = nActive;
+  r.nSpatialSites = nSpatialSites;
+  r.d_features = d_features;
+  return r;
+}
+
 int scnh_forward_resident(scnh_net *net, int batch, const int32_t *d_sample,
                           const int64_t *d_key, const int32_t *d_row,
                           const int32_t *d_background, int64_t nActive,
                           int nSpatialSites, const float *d_features,
                           float *h_probs) {
   SparseConvNetCUDA *cnn = net->cnn;
-  scn_ctx *ctx = cnn->memStream.ctx;
+  cnn->ensureInterfaces();
+  // everything on the net's own stream: one batch, start to end
+  cudaMemStream *keep = cnn->batchPool[0].preprocessStream;
+  cnn->batchPool[0].preprocessStream = nullptr;
+  cnn->preprocessResident(0, resident_of(batch, d_sample, d_key, d_row,
+                                         d_background, nActive, nSpatialSites,
+                                         d_features));
+  cnn->batchPool[0].preprocessStream = keep;
   SpatiallySparseBatch &b = cnn->batchPool[0];
-  while (b.interfaces.size() <= cnn->layers.size()) {
-    cnn->sharedSubInterfaces.push_back(new SpatiallySparseBatchSubInterface());
-    for (auto &slot : cnn->batchPool)
-      slot.interfaces.emplace_back(cnn->sharedSubInterfaces.back());
-  }
-  b.reset();
-  b.type = UNLABELEDBATCH;
-  b.batchSize = batch;
-  SpatiallySparseBatchInterface &in = b.interfaces[0];
-  in.nFeatures = cnn->nInputFeatures;
-  in.spatialSize = cnn->inputSpatialSize;
-  in.nSpatialSites = nSpatialSites;
-  in.featuresPresent.hVector() = range(cnn->nInputFeatures);
-  if (!in.deviceGrids) {
-    SCN_CHECKED(scn_grids_create(ctx, &in.deviceGrids));
-    in.ownsDeviceGrids = true;
-  }
-  scn_prof_tag(ctx, -1);
-  SCN_CHECKED(scn_grids_build(ctx, in.deviceGrids, batch, cnn->dimension,
-                              in.spatialSize, d_sample, d_key, d_row, nActive,
-                              d_background, nSpatialSites));
-  in.sub->features.copyToGPU();
-  size_t nElems = (size_t)nSpatialSites * cnn->nInputFeatures;
-  in.sub->features.resize64(nElems);
-  SCN_CHECKED(scn_d2d(ctx, in.sub->features.dPtr(), d_features,
-                      nElems * sizeof(float)));
-  for (size_t i = 0; i < cnn->layers.size(); i++) {
-    scn_prof_tag(ctx, (int)i);
-    cnn->layers[i]->preprocess(b, b.interfaces[i], b.interfaces[i + 1]);
-  }
   net->batch = &b;
   forward_layers(net, b);
   if (net->hasClassifier && h_probs)
     scnh_batch_probabilities(net, h_probs);
   cnn->memStream.synchronize();
   return b.interfaces.back().nSpatialSites;
+}
+
+int scnh_forward_resident_stream(scnh_net *net, int nBatches, int batch,
+                                 const int32_t *d_sample, const int64_t *d_key,
+                                 const int32_t *d_row,
+                                 const int32_t *d_background, int64_t nActive,
+                                 int nSpatialSites, const float *d_features,
+                                 float *h_probs) {
+  SparseConvNetCUDA *cnn = net->cnn;
+  ResidentBatch r = resident_of(batch, d_sample, d_key, d_row, d_background,
+                                nActive, nSpatialSites, d_features);
+  BatchProducer bp(*cnn, r, nBatches);
+  int done = 0;
+  while (SpatiallySparseBatch *b = bp.nextBatch()) {
+    net->batch = b;
+    forward_layers(net, *b);
+    if (net->hasClassifier && h_probs)
+      scnh_batch_probabilities(net, h_probs);
+    cnn->memStream.synchronize();
+    ++done;
+  }
+  net->batch = nullptr;
+  return done;
 }
 void *scnh_context(scnh_net *net) { return net->cnn->memStream.ctx; }
 double scnh_take_multiply_add_count(void) {

@@ -83,6 +83,16 @@ int scnh_forward_resident(scnh_net *net, int batch, const int32_t *d_sample,
                           const int32_t *d_background, int64_t nActive,
                           int nSpatialSites, const float *d_features,
                           float *h_probs);
+/* nBatches forward passes over the same resident batch, produced the way
+ * processDataset produces them: the net's batch-producer threads build grids
+ * and rule books on their slots' streams while the calling thread runs the
+ * forward pass of the previous batch.  Returns the number of batches done. */
+int scnh_forward_resident_stream(scnh_net *net, int nBatches, int batch,
+                                 const int32_t *d_sample, const int64_t *d_key,
+                                 const int32_t *d_row,
+                                 const int32_t *d_background, int64_t nActive,
+                                 int nSpatialSites, const float *d_features,
+                                 float *h_probs);
 /* the library context of the net (scn_ctx *), for timing and raw buffers */
 void *scnh_context(scnh_net *net);
 /* multiply-accumulates of the NiN layers since the last call */

@@ -8,19 +8,21 @@
 #include <vector>
 #include "scn_hip.h"
 
-// The stream object layer constructors take (utilities.h:105-112).  Here it
-// carries the library context, which owns the HIP stream.
+// The stream object layer constructors take (utilities.h:105-112).  Every
+// instance owns one library context, i.e. one HIP stream on the GPU.
 class cudaMemStream {
 public:
   scn_ctx *ctx;
   cudaMemStream();
   ~cudaMemStream();
+  cudaMemStream(const cudaMemStream &) = delete;
+  cudaMemStream &operator=(const cudaMemStream &) = delete;
   void *stream() const;
   void synchronize() const;
 };
 
-// the context vectorCUDA objects allocate from: the first cudaMemStream
-// constructed in the process (one GPU, one stream, as in the reference)
+// the context vectorCUDA objects use when no stream is named: the one of the
+// oldest live cudaMemStream (the net's own memStream)
 scn_ctx *scnDefaultContext();
 void scnCheck(int rc, const char *file, int line);
 #define SCN_CHECKED(expr) scnCheck((expr), __FILE__, __LINE__)
@@ -31,6 +33,8 @@ private:
   size_t dsize;       // size while on the GPU
   size_t dAllocated;  // elements allocated on the GPU (>= dsize)
   std::vector<t> vec;
+  void toCPU(scn_ctx *ctx);
+  void toGPU(scn_ctx *ctx);
 
 public:
   vectorCUDA(bool onGPU = true, size_t dsize = 0);

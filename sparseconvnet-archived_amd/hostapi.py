@@ -68,6 +68,7 @@ def lib():
         "scnh_iface_choices": (None, [vp, i32, vp]),
         "scnh_iface_grids": (None, [vp, i32, vp, vp, vp, vp]),
         "scnh_forward_resident": (i32, [vp, i32, vp, vp, vp, vp, i64, i32, vp, vp]),
+        "scnh_forward_resident_stream": (i32, [vp, i32, i32, vp, vp, vp, vp, i64, i32, vp, vp]),
         "scnh_context": (vp, [vp]),
         "scnh_take_multiply_add_count": (C.c_double, []),
     }
@@ -227,6 +228,11 @@ class Net:
     def forward_resident(self, batch, d_sample, d_key, d_row, d_bg, nActive, nSpatialSites, d_features, h_probs=None):
         return lib().scnh_forward_resident(self.h, batch, d_sample, d_key, d_row, d_bg, nActive, nSpatialSites,
                                            d_features, _p(h_probs) if h_probs is not None else None)
+
+    def forward_resident_stream(self, nBatches, batch, d_sample, d_key, d_row, d_bg, nActive, nSpatialSites, d_features,
+                                h_probs=None):
+        return lib().scnh_forward_resident_stream(self.h, nBatches, batch, d_sample, d_key, d_row, d_bg, nActive,
+                                                  nSpatialSites, d_features, _p(h_probs) if h_probs is not None else None)
 
     def context_handle(self):
         return lib().scnh_context(self.h)
