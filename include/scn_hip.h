@@ -49,7 +49,10 @@ enum {
   SCN_SIGMOID = 7 /* rejected */
 };
 
-enum { SCN_FP32 = 0, SCN_BF16 = 1 }; /* operand precision of the NiN contraction */
+/* Operand precision of the NiN contraction (accumulation is always fp32):
+ * fp32 MFMA; bf16 operands; or bf16 hi + lo pairs with three MFMAs per tile,
+ * which keeps fp32-grade results at bf16-matrix-core speed. */
+enum { SCN_FP32 = 0, SCN_BF16 = 1, SCN_BF16X3 = 2 };
 
 typedef struct scn_ctx scn_ctx;
 typedef struct scn_grids scn_grids;

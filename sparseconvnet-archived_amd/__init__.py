@@ -18,7 +18,7 @@ HEADER = os.path.join(ROOT, "include", "scn_hip.h")
 
 # ActivationFunction (reference types.h:11-20)
 NOSIGMOID, RELU, VLEAKYRELU, LEAKYRELU, TANH, SOFTMAX, PRELU, SIGMOID = range(8)
-FP32, BF16 = 0, 1
+FP32, BF16, BF16X3 = 0, 1, 2
 K_GRID_BUILD, K_RULES, K_GATHER, K_NIN, K_MAXPOOL, K_TERMINAL, K_SOFTMAX = range(7)
 KERNEL_FAMILIES = ["grid_build", "rules", "gather", "nin", "maxpool", "terminal", "softmax"]
 

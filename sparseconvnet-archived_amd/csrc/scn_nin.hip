@@ -225,6 +225,199 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// ---- MFMA path with bf16 operands: v_mfma_f32_32x32x16_bf16 ----------------
+// A and W stay fp32 in HBM; they are rounded to bf16 (nearest even) on their
+// way into LDS and accumulated in fp32.  One MFMA consumes k = 16: lane l
+// supplies eight consecutive k of row / column l % 32 starting at
+// k = 8 (l / 32), so both operands sit in LDS with k contiguous:
+// sA[row][k], sW[col][k], rows padded to 40 elements (80 bytes) so that the
+// 128-bit operand reads spread over all banks.
+//
+// SPLIT keeps the rounding residue as a second bf16 (x = hi + lo up to 2^-17)
+// and issues three MFMAs per tile, hi*hi + hi*lo + lo*hi: fp32-grade results
+// at a third of the bf16 rate, still several times the fp32 MFMA rate.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+#define BF_ROW 40
+
+__device__ __forceinline__ unsigned short to_bf16(float f) {
+  unsigned u = __float_as_uint(f);
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return (unsigned short)(u >> 16);
+}
+__device__ __forceinline__ uint4 pack_bf16x8(const float *v) {
+  uint4 r;
+  r.x = to_bf16(v[0]) | ((unsigned)to_bf16(v[1]) << 16);
+  r.y = to_bf16(v[2]) | ((unsigned)to_bf16(v[3]) << 16);
+  r.z = to_bf16(v[4]) | ((unsigned)to_bf16(v[5]) << 16);
+  r.w = to_bf16(v[6]) | ((unsigned)to_bf16(v[7]) << 16);
+  return r;
+}
+// v[i] -= float(bf16(v[i])): what the first rounding lost
+__device__ __forceinline__ void residue8(float *v) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+    v[i] -= __uint_as_float((unsigned)to_bf16(v[i]) << 16);
+}
+
+template <int WM, int WN, int NT, bool SPLIT>
+__global__ void __launch_bounds__(256)
+    k_nin_mfma_bf16(const float *__restrict__ A, const float *__restrict__ W,
+                    float *__restrict__ out, long long M, int K, int N,
+                    Epilogue ep) {
+  constexpr int BM = 32 * WM;
+  constexpr int BN = 32 * NT * WN;
+  constexpr int A_ITEMS = BM * (MF_BK / 8); // one item = 8 consecutive k of a row
+  constexpr int W_ITEMS = BN * (MF_BK / 8); // 8 consecutive k of a column
+  constexpr int A_PER = (A_ITEMS + 255) / 256;
+  constexpr int W_PER = (W_ITEMS + 255) / 256;
+  constexpr int PARTS = SPLIT ? 2 : 1; // hi, lo
+  __shared__ __attribute__((aligned(16))) unsigned short sA[2][PARTS][BM * BF_ROW];
+  __shared__ __attribute__((aligned(16))) unsigned short sW[2][PARTS][BN * BF_ROW];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+  const int nBlocksN = (N + BN - 1) / BN;
+  const long long m0 = (long long)(blockIdx.x / nBlocksN) * BM;
+  const int n0 = (int)(blockIdx.x % nBlocksN) * BN;
+  floatx16 acc[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int v = 0; v < 16; ++v)
+      acc[j][v] = 0.f;
+
+  uint4 ra[A_PER][PARTS], rw[W_PER][PARTS];
+  auto load_slab = [&](int k0) {
+#pragma unroll
+    for (int u = 0; u < A_PER; ++u) {
+      int c = tid + u * 256;
+      int r = c / (MF_BK / 8), kc = c % (MF_BK / 8);
+      long long m = m0 + r;
+      int k = k0 + kc * 8;
+      float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if (c < A_ITEMS && m < M) {
+        const float *src = A + m * K + k;
+        if (k + 8 <= K) {
+          float4 x = *reinterpret_cast<const float4 *>(src);
+          float4 y = *reinterpret_cast<const float4 *>(src + 4);
+          v[0] = x.x, v[1] = x.y, v[2] = x.z, v[3] = x.w;
+          v[4] = y.x, v[5] = y.y, v[6] = y.z, v[7] = y.w;
+        } else if (k < K) { // K % 4 == 0: exactly four left
+          float4 x = *reinterpret_cast<const float4 *>(src);
+          v[0] = x.x, v[1] = x.y, v[2] = x.z, v[3] = x.w;
+        }
+      }
+      ra[u][0] = pack_bf16x8(v);
+      if (SPLIT) {
+        residue8(v);
+        ra[u][PARTS - 1] = pack_bf16x8(v);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < W_PER; ++u) {
+      int c = tid + u * 256;
+      int kc = c / BN, nn = c % BN; // consecutive lanes: consecutive columns
+      int n = n0 + nn, k = k0 + kc * 8;
+      float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if (c < W_ITEMS && n < N) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q)
+          if (k + q < K)
+            v[q] = W[(long long)(k + q) * N + n];
+      }
+      rw[u][0] = pack_bf16x8(v);
+      if (SPLIT) {
+        residue8(v);
+        rw[u][PARTS - 1] = pack_bf16x8(v);
+      }
+    }
+  };
+  auto store_slab = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < A_PER; ++u) {
+      int c = tid + u * 256;
+      if (c < A_ITEMS) {
+        int r = c / (MF_BK / 8), kc = c % (MF_BK / 8);
+#pragma unroll
+        for (int h = 0; h < PARTS; ++h)
+          *reinterpret_cast<uint4 *>(&sA[buf][h][r * BF_ROW + kc * 8]) = ra[u][h];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < W_PER; ++u) {
+      int c = tid + u * 256;
+      if (c < W_ITEMS) {
+        int kc = c / BN, nn = c % BN;
+#pragma unroll
+        for (int h = 0; h < PARTS; ++h)
+          *reinterpret_cast<uint4 *>(&sW[buf][h][nn * BF_ROW + kc * 8]) = rw[u][h];
+      }
+    }
+  };
+
+  const int nSlabs = (K + MF_BK - 1) / MF_BK;
+  load_slab(0);
+  store_slab(0);
+  __syncthreads();
+  const int offA = (wm * 32 + (lane & 31)) * BF_ROW + 8 * (lane >> 5);
+  const int offW = (wn * 32 * NT + (lane & 31)) * BF_ROW + 8 * (lane >> 5);
+  for (int s = 0; s < nSlabs; ++s) {
+    const int buf = s & 1;
+    if (s + 1 < nSlabs)
+      load_slab((s + 1) * MF_BK);
+#pragma unroll
+    for (int kk = 0; kk < MF_BK; kk += 16) {
+      bf16x8 a = *reinterpret_cast<const bf16x8 *>(&sA[buf][0][offA + kk]);
+      bf16x8 al;
+      if (SPLIT)
+        al = *reinterpret_cast<const bf16x8 *>(&sA[buf][PARTS - 1][offA + kk]);
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        const int o = offW + 32 * j * BF_ROW + kk;
+        bf16x8 b = *reinterpret_cast<const bf16x8 *>(&sW[buf][0][o]);
+        if (SPLIT) {
+          bf16x8 bl = *reinterpret_cast<const bf16x8 *>(&sW[buf][PARTS - 1][o]);
+          // small terms first
+          acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, b, acc[j], 0, 0, 0);
+          acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, bl, acc[j], 0, 0, 0);
+        }
+        acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[j], 0, 0, 0);
+      }
+    }
+    if (s + 1 < nSlabs)
+      store_slab(buf ^ 1);
+    __syncthreads();
+  }
+
+  const int col = lane & 31;
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    int n = n0 + (wn * NT + j) * 32 + col;
+    if (n >= N)
+      continue;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      long long m = m0 + wm * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+      if (m < M)
+        out[m * N + n] = apply_act(acc[j][v], n, ep);
+    }
+  }
+}
+
+template <int WM, int WN, int NT>
+static void launch_mfma_bf16(scn_ctx *ctx, const float *A, const float *W,
+                             float *out, long long M, int K, int N,
+                             const Epilogue &ep, bool split) {
+  constexpr int BM = 32 * WM, BN = 32 * NT * WN;
+  dim3 grid((unsigned)((long long)scn_ceil_div(N, BN) * scn_ceil_div(M, BM)));
+  if (split)
+    hipLaunchKernelGGL((k_nin_mfma_bf16<WM, WN, NT, true>), grid, dim3(256), 0,
+                       ctx->stream, A, W, out, M, K, N, ep);
+  else
+    hipLaunchKernelGGL((k_nin_mfma_bf16<WM, WN, NT, false>), grid, dim3(256), 0,
+                       ctx->stream, A, W, out, M, K, N, ep);
+}
+
 template <int WM, int WN, int NT>
 static void launch_mfma(scn_ctx *ctx, const float *A, const float *W,
                         float *out, long long M, int K, int N,
@@ -246,7 +439,9 @@ extern "C" int scn_nin_forward(scn_ctx *ctx, const float *d_A,
                   act == SCN_LEAKYRELU || act == SCN_SOFTMAX || act == SCN_PRELU,
               SCN_ERR_ARG, "scn_nin_forward: activation %d is not supported",
               act);
-  SCN_REQUIRE(precision == SCN_FP32 || precision == SCN_BF16, SCN_ERR_ARG,
+  SCN_REQUIRE(precision == SCN_FP32 || precision == SCN_BF16 ||
+                  precision == SCN_BF16X3,
+              SCN_ERR_ARG,
               "scn_nin_forward: precision %d", precision);
   if (M == 0)
     return SCN_OK;
@@ -264,7 +459,18 @@ extern "C" int scn_nin_forward(scn_ctx *ctx, const float *d_A,
   ProfScope prof(ctx, SCN_K_NIN);
   const bool vec = K % 4 == 0 && N % 4 == 0 && ((uintptr_t)d_A & 15) == 0 &&
                    ((uintptr_t)d_W & 15) == 0;
-  if (vec && K >= 8) {
+  // bf16 operands only where the contraction is big enough to matter; the
+  // classifier head and the thin first layers stay fp32
+  if (vec && K >= 64 && act != SCN_SOFTMAX && precision != SCN_FP32) {
+    const bool split = precision == SCN_BF16X3;
+    long long blocksLarge = (long long)scn_ceil_div(M, 128) * scn_ceil_div(N, 64);
+    if (N <= 32)
+      launch_mfma_bf16<4, 1, 1>(ctx, d_A, d_W, d_out, M, K, N, ep, split);
+    else if (blocksLarge >= ctx->numCU)
+      launch_mfma_bf16<4, 1, 2>(ctx, d_A, d_W, d_out, M, K, N, ep, split);
+    else
+      launch_mfma_bf16<1, 4, 1>(ctx, d_A, d_W, d_out, M, K, N, ep, split);
+  } else if (vec && K >= 8) {
     long long blocksLarge = (long long)scn_ceil_div(M, 128) * scn_ceil_div(N, 64);
     if (N <= 32)
       launch_mfma<4, 1, 1>(ctx, d_A, d_W, d_out, M, K, N, ep);

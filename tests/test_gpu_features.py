@@ -129,3 +129,42 @@ def test_nin_special_cases(scn, ctx):
         ctx.nin_forward(ctx.array(A), ctx.array(W), ctx.array(B), None, d_out, M, K, K, 1.0, scn.TANH)
     with pytest.raises(scn.ScnError):
         ctx.nin_forward(ctx.array(A), ctx.array(W), ctx.array(B), None, d_out, M, K, K, 1.0, scn.PRELU)
+
+
+def to_bf16(x):
+    """Round fp32 to bf16 (nearest even) and back, in numpy."""
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32).astype(np.uint64)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) >> 16 << 16
+    return u.astype(np.uint32).view(np.float32)
+
+
+@pytest.mark.parametrize("M,K,N", [(777, 128, 64), (513, 256, 96), (129, 512, 160), (400, 160, 192), (100, 192, 100),
+                                   (3000, 1728, 64), (64, 288, 32), (2000, 64, 32)])
+@pytest.mark.parametrize("act", ["RELU", "PRELU", "NOSIGMOID"])
+def test_nin_bf16(scn, ctx, M, K, N, act):
+    """bf16 operands, fp32 accumulation: within 2e-2 relative of the fp32
+    oracle, and within 1e-4 of the same contraction with operands rounded to
+    bf16 on the host (i.e. the rounding is the only difference)."""
+    a = getattr(scn, act)
+    rng = np.random.default_rng(M + K + N + a)
+    A = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    W = (rng.standard_normal((K, N)) * np.sqrt(2.0 / K)).astype(np.float32)
+    B = rng.uniform(-0.5, 0.5, N).astype(np.float32)
+    pr = rng.uniform(0.1, 0.4, N).astype(np.float32)
+    print("nin bf16 M=%d K=%d N=%d act=%s" % (M, K, N, act), flush=True)
+    d_out = ctx.empty((M, N), np.float32)
+    ctx.nin_forward(ctx.array(A), ctx.array(W), ctx.array(B), ctx.array(pr), d_out, M, K, N, 1.0, a, scn.BF16)
+    got = d_out.download()
+    want = orc.nin_forward(A, W, B, pr, 1.0, a, f64=True)
+    scale = np.abs(A).astype(np.float64) @ np.abs(W).astype(np.float64) + np.abs(B)
+    assert np.all(np.abs(got - want) <= 2e-2 * scale)
+    assert np.linalg.norm(got - want) / np.linalg.norm(want) <= 2e-2
+    rounded = orc.nin_forward(to_bf16(A), to_bf16(W), B, pr, 1.0, a, f64=True)
+    assert np.all(np.abs(got - rounded) <= 1e-4 * scale)
+    if K >= 64:  # the rounding is really there: the result differs from fp32
+        assert np.abs(got - want).max() > 1e-5
+    # hi + lo operand pairs, three MFMAs per tile: back within the fp32 tolerance
+    ctx.nin_forward(ctx.array(A), ctx.array(W), ctx.array(B), ctx.array(pr), d_out, M, K, N, 1.0, a, scn.BF16X3)
+    got3 = d_out.download()
+    assert np.all(np.abs(got3 - want) <= 1e-4 * scale)
+    assert np.linalg.norm(got3 - want) / np.linalg.norm(want) <= 1e-4

@@ -157,3 +157,43 @@ def test_process_dataset_and_weight_files(scn, tmp_path):
     net2.loadWeights(base, 3)
     assert np.isclose(net2.processDataset(ds, 10), nll, rtol=1e-6)
     net2.processDatasetRepeatTest(ds, 10, 2)
+
+
+@pytest.mark.parametrize("mode", ["BF16", "BF16X3"])
+def test_bf16_mode_net(scn, mode):
+    """bf16 NiN contractions against the fp32 oracle on 200 samples.
+
+    Plain bf16 operands: class probabilities within 2e-2 relative.  The
+    synthetic nets have random He-normal weights, so their 100-class softmax is
+    nearly flat and a 1e-2 relative change of the logits moves the arg-max of
+    2-3 % of the samples; top-1 agreement with plain bf16 is therefore checked
+    at 95 % here.  The hi + lo mode (three MFMAs per tile) has to meet the full
+    bar: 1e-4 relative and at least 99.5 % top-1 agreement."""
+    from sparseconvnet_archived_amd import hostapi, synthetic
+    cfg = synthetic.config(2, batch=200)
+    net, ora = build_pair(cfg, hostapi)
+    net.setPrecision(getattr(scn, mode))
+    for i, (W, B, pr) in synthetic.he_normal_weights(net.layers(), 77).items():
+        net.set_weights(i, W, B, pr)
+        ora.set_weights(i, W, B, pr)
+    samples = synthetic.make_samples(cfg, 78)
+    ds = hostapi.Dataset("bf16", 3, 100, hostapi.TESTBATCH)
+    for pts, f, label in samples:
+        ds.add_points(2, cfg.lattice, pts, f, label)
+    S, K, R, bg, feats, n = synthetic.codify(samples, 2, cfg.lattice, net.inputSpatialSize, 3)
+    want = ora.forward(len(samples), S, K, R, bg, feats, n, np.array([s[2] for s in samples], np.int32), keep=False)
+    net.begin(ds, len(samples))
+    assert net.next_batch()
+    out = net.batch_outputs()
+    err = rel_l2(out["probabilities"], want["probabilities"])
+    agree = np.mean(out["predictions"][:, 0] == want["predictions"][:, 0])
+    print("%s probabilities rel-L2 %.3g, top-1 agreement %.4f" % (mode, err, agree), flush=True)
+    if mode == "BF16":
+        assert err <= 2e-2 and agree >= 0.95
+    else:
+        assert err <= 1e-4 and agree >= 0.995
+    # rule books do not depend on the precision
+    for i, wi in enumerate(want["interfaces"]):
+        assert np.array_equal(net.interface(i, want_features=False)["rules"], wi["rules"])
+    net.end()
+    net.close()
