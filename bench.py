@@ -39,6 +39,9 @@ def parse():
     ap.add_argument("--precision", choices=["fp32", "bf16", "bf16x3"], default="fp32")
     ap.add_argument("--seed", type=int, default=2015)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 disables it)")
+    ap.add_argument("--calibration-copy-mb", type=int, default=0,
+                    help="first launch a plain row copy (gather with identity rules) of this many MB, so that "
+                         "hardware byte counters collected over the run can be scaled by a kernel of known traffic")
     ap.add_argument("--producers", type=int, default=4,
                     help="batch-producer threads / streams building rule books ahead of the forward pass")
     return ap.parse_args()
@@ -110,6 +113,20 @@ def main():
 
     def step():
         net.forward_resident(B, dS.ptr, dK.ptr, dR.ptr, dBg.ptr, active, nSites, dF.ptr, probs)
+
+    if args.calibration_copy_mb > 0:
+        # rows of 64 floats copied through the gather kernel with rules 0..n-1:
+        # reads n*256 + n*4 bytes, writes n*256 bytes
+        n_rows = args.calibration_copy_mb * (1 << 20) // 256
+        src = ctx.empty((n_rows, 64), np.float32)
+        dst = ctx.empty((n_rows, 64), np.float32)
+        ident = ctx.array(np.arange(n_rows, dtype=np.int32))
+        scn.lib().scn_fill32(ctx.h, src.ptr, 0x3F800000, n_rows * 64)
+        ctx.gather_rows(src, dst, ident, n_rows, 64)
+        ctx.sync()
+        print("calibration copy: %d rows of 256 B: read %d B, written %d B" % (n_rows, n_rows * 260, n_rows * 256),
+              file=sys.stderr)
+        del src, dst, ident
 
     def run(n):
         # n batches the way processDataset runs them: producer threads build

@@ -114,7 +114,7 @@ __global__ void __launch_bounds__(256)
 #define MF_BK 32
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-template <int WM, int WN, int NT>
+template <int WM, int WN, int NT, int BK>
 __global__ void __launch_bounds__(256)
     k_nin_mfma(const float *__restrict__ A, const float *__restrict__ W,
                float *__restrict__ out, long long M, int K, int N,
@@ -122,18 +122,26 @@ __global__ void __launch_bounds__(256)
   constexpr int BM = 32 * WM;
   constexpr int BN = 32 * NT * WN;
   constexpr int BMP = BM + 1;
-  constexpr int A_CHUNKS = BM * MF_BK / 4; // float4 chunks per slab
-  constexpr int W_CHUNKS = MF_BK * BN / 4;
+  constexpr int A_CHUNKS = BM * BK / 4; // float4 chunks per slab
+  constexpr int W_CHUNKS = BK * BN / 4;
   constexpr int A_PER = (A_CHUNKS + 255) / 256;
   constexpr int W_PER = (W_CHUNKS + 255) / 256;
-  __shared__ float sA[2][MF_BK * BMP];
-  __shared__ float sW[2][MF_BK * BN];
+  __shared__ float sA[2][BK * BMP];
+  __shared__ float sW[2][BK * BN];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WN, wn = wave % WN;
-  const int nBlocksN = (N + BN - 1) / BN; // n-blocks fastest: the blocks that
-  const long long m0 = (long long)(blockIdx.x / nBlocksN) * BM; // share an A
-  const int n0 = (int)(blockIdx.x % nBlocksN) * BN;             // slab run together
+  // Consecutive workgroup ids go to consecutive XCDs (8, each with its own
+  // L2).  The n-blocks that share an A slab are given ids that land on ONE
+  // XCD: id = slot * 8 + xcd  ->  tile = xcd * (grid / 8) + slot.
+  const int nBlocksN = (N + BN - 1) / BN;
+  const long long nTiles = ((M + BM - 1) / BM) * nBlocksN;
+  const long long tile =
+      (long long)(blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  if (tile >= nTiles)
+    return; // the grid is rounded up to a multiple of 8
+  const long long m0 = (tile / nBlocksN) * BM;
+  const int n0 = (int)(tile % nBlocksN) * BN;
   floatx16 acc[NT];
 #pragma unroll
   for (int j = 0; j < NT; ++j)
@@ -146,7 +154,7 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
     for (int u = 0; u < A_PER; ++u) {
       int c = tid + u * 256;
-      int r = c / (MF_BK / 4), kc = c % (MF_BK / 4);
+      int r = c / (BK / 4), kc = c % (BK / 4);
       long long m = m0 + r;
       int k = k0 + kc * 4;
       float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -170,7 +178,7 @@ __global__ void __launch_bounds__(256)
     for (int u = 0; u < A_PER; ++u) {
       int c = tid + u * 256;
       if (c < A_CHUNKS) {
-        int r = c / (MF_BK / 4), kc = c % (MF_BK / 4);
+        int r = c / (BK / 4), kc = c % (BK / 4);
         float *dst = &sA[buf][(kc * 4) * BMP + r];
         dst[0] = ra[u].x;
         dst[BMP] = ra[u].y;
@@ -186,18 +194,18 @@ __global__ void __launch_bounds__(256)
     }
   };
 
-  const int nSlabs = (K + MF_BK - 1) / MF_BK;
+  const int nSlabs = (K + BK - 1) / BK;
   load_slab(0);
   store_slab(0);
   __syncthreads();
   for (int s = 0; s < nSlabs; ++s) {
     const int buf = s & 1;
     if (s + 1 < nSlabs)
-      load_slab((s + 1) * MF_BK); // in flight while this slab is multiplied
+      load_slab((s + 1) * BK); // in flight while this slab is multiplied
     const float *pa = &sA[buf][(lane >> 5) * BMP + wm * 32 + (lane & 31)];
     const float *pw = &sW[buf][(lane >> 5) * BN + wn * 32 * NT + (lane & 31)];
 #pragma unroll
-    for (int kk = 0; kk < MF_BK; kk += 2) {
+    for (int kk = 0; kk < BK; kk += 2) {
       float a = pa[kk * BMP];
 #pragma unroll
       for (int j = 0; j < NT; ++j) {
@@ -418,14 +426,15 @@ static void launch_mfma_bf16(scn_ctx *ctx, const float *A, const float *W,
                        ctx->stream, A, W, out, M, K, N, ep);
 }
 
-template <int WM, int WN, int NT>
+template <int WM, int WN, int NT, int BK = MF_BK>
 static void launch_mfma(scn_ctx *ctx, const float *A, const float *W,
                         float *out, long long M, int K, int N,
                         const Epilogue &ep) {
   constexpr int BM = 32 * WM, BN = 32 * NT * WN;
-  dim3 grid((unsigned)((long long)scn_ceil_div(N, BN) * scn_ceil_div(M, BM)));
-  hipLaunchKernelGGL((k_nin_mfma<WM, WN, NT>), grid, dim3(256), 0, ctx->stream,
-                     A, W, out, M, K, N, ep);
+  long long tiles = (long long)scn_ceil_div(N, BN) * scn_ceil_div(M, BM);
+  dim3 grid((unsigned)((tiles + 7) / 8 * 8));
+  hipLaunchKernelGGL((k_nin_mfma<WM, WN, NT, BK>), grid, dim3(256), 0,
+                     ctx->stream, A, W, out, M, K, N, ep);
 }
 
 extern "C" int scn_nin_forward(scn_ctx *ctx, const float *d_A,
@@ -471,13 +480,38 @@ extern "C" int scn_nin_forward(scn_ctx *ctx, const float *d_A,
     else
       launch_mfma_bf16<1, 4, 1>(ctx, d_A, d_W, d_out, M, K, N, ep, split);
   } else if (vec && K >= 8) {
-    long long blocksLarge = (long long)scn_ceil_div(M, 128) * scn_ceil_div(N, 64);
-    if (N <= 32)
-      launch_mfma<4, 1, 1>(ctx, d_A, d_W, d_out, M, K, N, ep);
-    else if (blocksLarge >= ctx->numCU)
-      launch_mfma<4, 1, 2>(ctx, d_A, d_W, d_out, M, K, N, ep);
-    else // too few rows to fill the chip with tall tiles: 32-row tiles
+    // Tall tiles (128 rows), 64 columns wide, or 96 where that divides N
+    // (measured on 12928 x 1280 x 480: 93 TFLOP/s against 73 with 64-column
+    // tiles; wider tiles leave too few workgroups for 256 compute units).
+    const int maxCols = N % 96 == 0 ? 96 : 64;
+    const int nChunks = (N + maxCols - 1) / maxCols;
+    const int nt = ((N + 31) / 32 + nChunks - 1) / nChunks; // 1..6
+    long long blocksTall = (long long)scn_ceil_div(M, 128) * nChunks;
+    if (blocksTall * 2 < ctx->numCU && N > 32) {
+      // too few rows to fill the chip with tall tiles: 32-row tiles
       launch_mfma<1, 4, 1>(ctx, d_A, d_W, d_out, M, K, N, ep);
+    } else {
+      switch (nt) {
+      case 1:
+        launch_mfma<4, 1, 1>(ctx, d_A, d_W, d_out, M, K, N, ep);
+        break;
+      case 2:
+        launch_mfma<4, 1, 2>(ctx, d_A, d_W, d_out, M, K, N, ep);
+        break;
+      case 3:
+        launch_mfma<4, 1, 3>(ctx, d_A, d_W, d_out, M, K, N, ep);
+        break;
+      case 4:
+        launch_mfma<4, 1, 4, 16>(ctx, d_A, d_W, d_out, M, K, N, ep);
+        break;
+      case 5:
+        launch_mfma<4, 1, 5, 16>(ctx, d_A, d_W, d_out, M, K, N, ep);
+        break;
+      default:
+        launch_mfma<4, 1, 6, 16>(ctx, d_A, d_W, d_out, M, K, N, ep);
+        break;
+      }
+    }
   } else {
     dim3 grid(scn_ceil_div(M, GT_BM), scn_ceil_div(N, GT_BN));
     hipLaunchKernelGGL(k_nin_generic, grid, dim3(256), 0, ctx->stream, d_A,
