@@ -29,6 +29,25 @@ MFMA_PEAK_TFLOPS = {"fp32": 157.3, "bf16": 2500.0, "bf16x3": 2500.0 / 3}
 BALANCE_FLOP_PER_BYTE = {k: v * 1e12 / 8e12 for k, v in MFMA_PEAK_TFLOPS.items()}
 
 
+# HBM bytes per launch (read + written) measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by
+# a copy kernel of known size; the runs are summarised in profiles/hbm_traffic_c2.txt and hbm_traffic_c5.txt.
+# Only valid for the default batch and seed of the config.
+MEASURED_TRAFFIC = {
+    ("c2_sparse_net_2d", "gather", 3): 8.03e6 + 30.96e6,
+    ("c2_sparse_net_2d", "nin", 4): 31.44e6 + 15.48e6,
+    ("c2_sparse_net_2d", "maxpool", 5): 22.66e6 + 11.76e6,
+    ("c2_sparse_net_2d", "gather", 6): 7.92e6 + 30.54e6,
+    ("c2_sparse_net_2d", "nin", 7): 31.61e6 + 11.45e6,
+    ("c2_sparse_net_2d", "nin", 10): 20.50e6 + 5.98e6,
+    ("c2_sparse_net_2d", "nin", 13): 7.80e6 + 1.58e6,
+    ("c5_spatiotemporal_3d", "gather", 0): 3031.14e6 + 22831.83e6,
+    ("c5_spatiotemporal_3d", "nin", 1): 23188.35e6 + 845.62e6,
+    ("c5_spatiotemporal_3d", "gather", 2): 9378.68e6 + 43599.93e6,
+    ("c5_spatiotemporal_3d", "nin", 3): 44336.62e6 + 1614.81e6,
+    ("c5_spatiotemporal_3d", "maxpool", 4): 1650.98e6 + 522.02e6,
+}
+
+
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -206,12 +225,19 @@ def main():
     fam_ms = {}
     for e in kernels:
         fam_ms[e["kernel"]] = fam_ms.get(e["kernel"], 0.0) + e["ms_per_step"]
-    dominant = next((e for e in kernels if "achieved" in e), None)
+    default_input = args.batch is None and args.seed == 2015 and args.precision == "fp32"
+    for e in kernels:
+        e["traffic"] = MEASURED_TRAFFIC.get((cfg.name, e["kernel"], e["layer"])) if default_input else None
+    # the dominant kernel: the single-kernel span that takes the most time (a "rules" or "grid_build" span covers
+    # several small kernels and a host round trip, so it has no one roofline)
+    dominant = next((e for e in kernels if "achieved" in e and e["kernel"] in ("gather", "nin", "maxpool", "terminal")), None)
     roofline = None
     if dominant:
         roofline = dict(kernel="%s[layer %d]" % (dominant["kernel"], dominant["layer"]), bound=dominant["bound"],
                         achieved=dominant["achieved"], peak=dominant["peak"], unit=dominant["unit"], frac=dominant["frac"],
-                        traffic=None)
+                        traffic=dominant["traffic"])
+        if "shape" in dominant:
+            roofline["shape_MKN"] = dominant["shape"]
 
     cpu_baseline = None
     if args.cpu_seconds > 0:
