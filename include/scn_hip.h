@@ -140,9 +140,9 @@ int scn_rules_fill(scn_ctx *ctx, const scn_grids *in, scn_grids *out,
 /* ---- feature kernels --------------------------------------------------- */
 /* propForwardToMatrixMultiply (ConvolutionalLayer.h:38-40;
  * ConvolutionalLayer.cu:12-41): out[c*nIn + j] = in[rules[c]*nIn + j],
- * c < count.  A negative rule (the reference does not guard them) is refused
- * by the host check only in debug builds; rule books from this library never
- * hold one here. */
+ * c < count.  A negative rule, which the reference's kernel does not guard
+ * (ConvolutionalLayer.cu:20-27), gathers a row of zeros; rule books built by
+ * this library never hold one here. */
 int scn_gather_rows(scn_ctx *ctx, const float *d_in, float *d_out,
                     const int32_t *d_rules, int64_t count, int nIn);
 /* replicateArray + d_rowMajorSGEMM_alphaAB_betaC(alpha = beta = p) +

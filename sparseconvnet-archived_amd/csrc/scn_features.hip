@@ -9,7 +9,8 @@
 
 // out[c * nIn + j] = in[rules[c] * nIn + j]   (ConvolutionalLayer.cu:12-31)
 // The output is one contiguous run per tile, so consecutive lanes write
-// consecutive 16-byte chunks; reads are contiguous per rule.
+// consecutive 16-byte chunks; reads are contiguous per rule.  A negative rule
+// (the reference reads out of bounds on one) gathers a row of zeros.
 template <typename VecT, int VEC>
 __global__ void __launch_bounds__(GATHER_THREADS)
     k_gather(const float *__restrict__ in, float *__restrict__ out,
@@ -23,8 +24,10 @@ __global__ void __launch_bounds__(GATHER_THREADS)
        c0 += (long long)gridDim.x * GATHER_TILE) {
     long long left = count - c0;
     const int n = left < GATHER_TILE ? (int)left : GATHER_TILE;
-    if (tid < n)
-      roff[tid] = (long long)rules[c0 + tid] * nIn;
+    if (tid < n) {
+      int rule = rules[c0 + tid];
+      roff[tid] = rule < 0 ? -1 : (long long)rule * nIn;
+    }
     __syncthreads();
     const int items = n * chunks;
     VecT *dst = reinterpret_cast<VecT *>(out + c0 * nIn);
@@ -36,7 +39,8 @@ __global__ void __launch_bounds__(GATHER_THREADS)
       int qq = q, cc = ch;
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        v[u] = *reinterpret_cast<const VecT *>(in + roff[qq] + cc * VEC);
+        long long ro = roff[qq];
+        v[u] = ro < 0 ? VecT{} : *reinterpret_cast<const VecT *>(in + ro + cc * VEC);
         qq += dq;
         cc += dch;
         if (cc >= chunks) {
@@ -51,7 +55,8 @@ __global__ void __launch_bounds__(GATHER_THREADS)
       ch = cc;
     }
     for (; idx < items; idx += GATHER_THREADS) {
-      dst[idx] = *reinterpret_cast<const VecT *>(in + roff[q] + ch * VEC);
+      long long ro = roff[q];
+      dst[idx] = ro < 0 ? VecT{} : *reinterpret_cast<const VecT *>(in + ro + ch * VEC);
       q += dq;
       ch += dch;
       if (ch >= chunks) {

@@ -25,3 +25,15 @@ def test_version_and_error_string_without_gpu():
     scn = load_scn()
     assert b"gfx950" in scn.lib().scn_version()
     assert isinstance(scn.lib().scn_last_error(), bytes)
+
+
+def test_host_library_exports_the_c_facade():
+    scn = load_scn()
+    from sparseconvnet_archived_amd import hostapi
+    assert os.path.exists(hostapi.LIB_PATH)
+    L = hostapi.lib()
+    import re
+    hdr = open(os.path.join(os.path.dirname(hostapi.LIB_PATH), "host", "scn_host_c.h")).read()
+    hdr = re.sub(r"/\*.*?\*/", "", hdr, flags=re.S)
+    for name in sorted(set(re.findall(r"\b(scnh_[a-z0-9_]+)\s*\(", hdr))):
+        assert hasattr(L, name), name

@@ -168,3 +168,31 @@ def test_nin_bf16(scn, ctx, M, K, N, act):
     got3 = d_out.download()
     assert np.all(np.abs(got3 - want) <= 1e-4 * scale)
     assert np.linalg.norm(got3 - want) / np.linalg.norm(want) <= 1e-4
+
+
+def test_gather_negative_rule_is_zero_row(scn, ctx):
+    rng = np.random.default_rng(4)
+    inp = rng.standard_normal((50, 32)).astype(np.float32)
+    rules = rng.integers(0, 50, 1000).astype(np.int32)
+    rules[::7] = -1
+    d_out = ctx.empty((1000, 32), np.float32)
+    ctx.gather_rows(ctx.array(inp), d_out, ctx.array(rules), 1000, 32)
+    want = np.where(rules[:, None] < 0, np.float32(0), inp[np.maximum(rules, 0)])
+    assert np.array_equal(d_out.download(), want)
+
+
+def test_argument_errors(scn, ctx):
+    d = ctx.empty(16, np.float32)
+    r = ctx.empty(16, np.int32)
+    with pytest.raises(scn.ScnError):
+        ctx.gather_rows(d, d, r, 4, 0)
+    with pytest.raises(scn.ScnError):
+        ctx.maxpool(d, d, r, 4, 0, 4, r)
+    with pytest.raises(scn.ScnError):
+        ctx.terminal_pool(d, d, r, 1, 0, 4)
+    with pytest.raises(scn.ScnError):
+        ctx.softmax_rows(d, d, 1, 0)
+    # zero-sized work is accepted and does nothing
+    ctx.gather_rows(d, d, r, 0, 4)
+    ctx.maxpool(d, d, r, 0, 2, 4, r)
+    ctx.sync()

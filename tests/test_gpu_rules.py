@@ -148,3 +148,21 @@ def test_find_and_errors(scn, ctx):
     with pytest.raises(scn.ScnError):
         g.fill(out, ctx.empty(4, np.int32), 4)  # capacity
     assert n == 9
+
+
+def test_sites_outside_the_field_are_reported(scn, ctx):
+    g = scn.Grids(ctx)
+    # key 30 does not exist in a 5 x 5 field; sample 3 does not exist in a batch of 1
+    g.build(1, 2, 5, [0, 0, 3], [7, 30, 2], [1, 2, 3], [0], 4)
+    out = scn.Grids(ctx)
+    with pytest.raises(scn.ScnError, match="outside the field"):
+        g.plan_square(out, 5, 4, 2, 1)
+    # the context stays usable
+    g.build(1, 2, 5, [0, 0], [7, 6], [1, 2], [0], 3)
+    assert g.plan_square(out, 5, 4, 2, 1) == 7
+
+
+def test_empty_batch_and_empty_samples(scn, ctx):
+    samples = [(0, {}), (1, {3: 2}), (3, {})]
+    run_both(scn, ctx, samples, 2, 5, 4, 2, 1, 1, False, 4)
+    run_both(scn, ctx, [(0, {})], 3, 4, 2, 3, 1, 1, False, 1)
