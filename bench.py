@@ -61,6 +61,8 @@ def parse():
     ap.add_argument("--calibration-copy-mb", type=int, default=0,
                     help="first launch a plain row copy (gather with identity rules) of this many MB, so that "
                          "hardware byte counters collected over the run can be scaled by a kernel of known traffic")
+    ap.add_argument("--from-host", action="store_true",
+                    help="also time processDataset() on host-resident Pictures (CPU codify + PCIe upload included)")
     ap.add_argument("--producers", type=int, default=4,
                     help="batch-producer threads / streams building rule books ahead of the forward pass")
     return ap.parse_args()
@@ -239,6 +241,25 @@ def main():
         if "shape" in dominant:
             roofline["shape_MKN"] = dominant["shape"]
 
+    from_host = None
+    if args.from_host:
+        # the reference's own entry point: Pictures in host memory, codifyInputData on the producer threads, input
+        # sites and features uploaded over PCIe for every batch
+        reps = max(2, min(args.steps, 20))
+        ds = hostapi.Dataset(cfg.name, cfg.nInputFeatures, max(cfg.nClasses, 1), hostapi.TESTBATCH)
+        for _ in range(reps):
+            for pts, f, label in samples:
+                ds.add_points(cfg.dimension, cfg.lattice, pts, f, label)
+        if net.layers()[-1]["act"] == synthetic.SOFTMAX:
+            net.processDataset(ds, B)  # warm-up pass (buffers grow)
+            t0 = time.perf_counter()
+            net.processDataset(ds, B)
+            dth = time.perf_counter() - t0
+            from_host = {"ms_per_batch": 1e3 * dth / reps, "active_sites_per_s": active * reps / dth,
+                         "samples_per_s": B * reps / dth, "batches": reps,
+                         "note": "processDataset on host Pictures: CPU codify + H2D of sites and features included"}
+        ds.close()
+
     cpu_baseline = None
     if args.cpu_seconds > 0:
         cpu_baseline = cpu_leg(cfg, layers, weights, samples, net.inputSpatialSize, args.cpu_seconds)
@@ -270,6 +291,8 @@ def main():
         "kernels": kernels,
         "cpu_baseline": cpu_baseline,
     }
+    if from_host:
+        out["from_host_pictures"] = from_host
     net.close()
     sys.stdout.flush()
     os.dup2(saved_stdout, 1)

@@ -197,3 +197,15 @@ def test_bf16_mode_net(scn, mode):
         assert np.array_equal(net.interface(i, want_features=False)["rules"], wi["rules"])
     net.end()
     net.close()
+
+
+def test_reference_style_cpp_driver(scn):
+    """A C++ driver written against the public headers only (DeepC2, a Picture
+    subclass, processDataset, weight save/load, repeat test) runs end to end."""
+    import subprocess
+    exe = os.path.join(os.path.dirname(scn.LIB_PATH), "scn_example_driver")
+    assert os.path.exists(exe), "built by make -C sparseconvnet-archived_amd/host"
+    out = subprocess.run([exe, "250", "100"], capture_output=True, text=True, timeout=170)
+    print(out.stdout[-1500:], out.stderr[-500:], flush=True)
+    assert out.returncode == 0
+    assert "example driver ok" in out.stdout and "rate:" in out.stdout
