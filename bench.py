@@ -65,6 +65,9 @@ def parse():
                     help="also time processDataset() on host-resident Pictures (CPU codify + PCIe upload included)")
     ap.add_argument("--producers", type=int, default=4,
                     help="batch-producer threads / streams building rule books ahead of the forward pass")
+    ap.add_argument("--fused", type=int, choices=[0, 1], default=1,
+                    help="1: setFusedConvolutions, a convolution's gather runs inside the next NiN kernel (same "
+                         "results bit for bit); 0: the reference's two steps, gather then NiN")
     return ap.parse_args()
 
 
@@ -96,6 +99,11 @@ def algorithmic_work(layers, ifaces, batch, precision):
             M, K, N = b["rows"], l["nIn"], l["nOut"]
             asz = 4  # operands are fp32 in HBM in every mode; bf16 rounding happens on the way into LDS
             work[("nin", i)] = (asz * (M * K + K * N) + 4 * (M * N + N), 2 * M * K * N)
+            if i > 0 and layers[i - 1]["kind"].startswith("conv"):
+                # gather fused in: the rules and the convolution's input rows are read instead of the wide matrix
+                src = ifaces[i - 1]
+                work[("conv_nin", i)] = (4 * a["nRules"] + asz * (src["rows"] * src["nFeatures"] + K * N) + 4 * (M * N + N),
+                                         2 * M * K * N)
     return work
 
 
@@ -118,6 +126,7 @@ def main():
     B = cfg.batch
     net = hostapi.Net(cfg.dimension, cfg.nInputFeatures, max(cfg.nClasses, 1), threads=max(1, args.producers))
     cfg.build(net)
+    net.setFusedConvolutions(bool(args.fused))
     if args.precision != "fp32":
         net.setPrecision(scn.BF16 if args.precision == "bf16" else scn.BF16X3)
     layers = net.layers()
@@ -205,7 +214,7 @@ def main():
         ms = ms_total / args.steps
         byts, flops = work.get(key, (0, 0))
         entry = dict(kernel=fam, layer=tag, ms_per_step=round(ms, 5), launches_per_step=cnt[key] / args.steps)
-        if fam == "nin" and flops:
+        if fam in ("nin", "conv_nin") and flops:
             K_, N_ = layers[tag]["nIn"], layers[tag]["nOut"]
             intensity = flops / max(byts, 1)
             entry["shape"] = [ifaces[tag + 1]["rows"], K_, N_]
@@ -228,11 +237,12 @@ def main():
     for e in kernels:
         fam_ms[e["kernel"]] = fam_ms.get(e["kernel"], 0.0) + e["ms_per_step"]
     default_input = args.batch is None and args.seed == 2015 and args.precision == "fp32"
+    fused_layers = {e["layer"] for e in kernels if e["kernel"] == "conv_nin"}
     for e in kernels:
         e["traffic"] = MEASURED_TRAFFIC.get((cfg.name, e["kernel"], e["layer"])) if default_input else None
     # the dominant kernel: the single-kernel span that takes the most time (a "rules" or "grid_build" span covers
     # several small kernels and a host round trip, so it has no one roofline)
-    dominant = next((e for e in kernels if "achieved" in e and e["kernel"] in ("gather", "nin", "maxpool", "terminal")), None)
+    dominant = next((e for e in kernels if "achieved" in e and e["kernel"] in ("gather", "nin", "conv_nin", "maxpool", "terminal")), None)
     roofline = None
     if dominant:
         roofline = dict(kernel="%s[layer %d]" % (dominant["kernel"], dominant["layer"]), bound=dominant["bound"],
@@ -276,6 +286,7 @@ def main():
         "ms_single_batch_latency": ms_latency,
         "ms_per_step_with_event_timing": 1e3 * dt_prof / args.steps,
         "producer_threads": max(1, args.producers),
+        "fused_convolutions": sorted(fused_layers),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -283,7 +294,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": cfg.name, "batch": B, "input_field": net.inputSpatialSize, "lattice": cfg.lattice,
                    "dimension": cfg.dimension, "active_sites": active, "input_rows": nSites,
-                   "stack": [list(c) for c in cfg.stack], "precision": args.precision, "seed": args.seed},
+                   "stack": [list(c) for c in cfg.stack], "precision": args.precision, "seed": args.seed,
+                   "fused": bool(args.fused)},
         "mega_multiply_adds_per_sample": mac / B / 1e6,
         "giga_multiply_adds_per_s": mac / (ms_per_step * 1e-3) / 1e9,
         "roofline": roofline,

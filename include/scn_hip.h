@@ -154,6 +154,22 @@ int scn_gather_rows(scn_ctx *ctx, const float *d_in, float *d_out,
 int scn_nin_forward(scn_ctx *ctx, const float *d_A, const float *d_W,
                     const float *d_B, const float *d_prelu, float *d_out,
                     int64_t M, int K, int N, float p, int act, int precision);
+/* Gather and NiN in one kernel: out[M x N] = act(p * (G W + B)) where row m of
+ * G is the receptive field of output site m, G[m][q * nIn + c] =
+ * in[rules[m * fs + q] * nIn + c], without ever writing G to memory.  Same
+ * result as scn_gather_rows followed by scn_nin_forward (fp32), bit for bit.
+ * The reference keeps such a fused layer as disabled code
+ * (ReallyConvolutionalLayer.cu:27-60, switched off at SparseConvNetCUDA.cu:81);
+ * what it replaces on the live path is ConvolutionalLayer::forwards +
+ * NetworkInNetwork(PReLU)Layer::forwards (ConvolutionalLayer.cu:125-133,
+ * NetworkInNetworkLayer.cu:187-200).  W is [fs * nIn x N].
+ * scn_conv_nin_supported tells whether (fs, nIn, N) is in the kernel's range. */
+int scn_conv_nin_supported(int fs, int nIn, int N);
+int scn_conv_nin_forward(scn_ctx *ctx, const float *d_in,
+                         const int32_t *d_rules, int fs, int nIn,
+                         const float *d_W, const float *d_B,
+                         const float *d_prelu, float *d_out, int64_t M, int N,
+                         float p, int act);
 /* maxPool (MaxPoolingLayer.h:6-7; MaxPoolingLayer.cu:9-72): first maximum
  * wins, negative rules skipped, choice = rule * C + channel. */
 int scn_maxpool(scn_ctx *ctx, const float *d_in, float *d_out,
@@ -179,7 +195,8 @@ enum {
   SCN_K_MAXPOOL = 4,
   SCN_K_TERMINAL = 5,
   SCN_K_SOFTMAX = 6,
-  SCN_K_COUNT = 7
+  SCN_K_CONV_NIN = 7, /* gather fused into the NiN contraction */
+  SCN_K_COUNT = 8
 };
 int scn_prof_enable(scn_ctx *ctx, int on);
 /* label attached to the spans recorded from now on (e.g. the layer index) */

@@ -19,8 +19,8 @@ HEADER = os.path.join(ROOT, "include", "scn_hip.h")
 # ActivationFunction (reference types.h:11-20)
 NOSIGMOID, RELU, VLEAKYRELU, LEAKYRELU, TANH, SOFTMAX, PRELU, SIGMOID = range(8)
 FP32, BF16, BF16X3 = 0, 1, 2
-K_GRID_BUILD, K_RULES, K_GATHER, K_NIN, K_MAXPOOL, K_TERMINAL, K_SOFTMAX = range(7)
-KERNEL_FAMILIES = ["grid_build", "rules", "gather", "nin", "maxpool", "terminal", "softmax"]
+K_GRID_BUILD, K_RULES, K_GATHER, K_NIN, K_MAXPOOL, K_TERMINAL, K_SOFTMAX, K_CONV_NIN = range(8)
+KERNEL_FAMILIES = ["grid_build", "rules", "gather", "nin", "maxpool", "terminal", "softmax", "conv_nin"]
 
 
 class ScnError(RuntimeError):
@@ -82,6 +82,8 @@ def lib():
         "scn_rules_fill": (C.c_int, [vp, vp, vp, vp, i64]),
         "scn_gather_rows": (C.c_int, [vp, vp, vp, vp, i64, C.c_int]),
         "scn_nin_forward": (C.c_int, [vp] * 6 + [i64, C.c_int, C.c_int, f32, C.c_int, C.c_int]),
+        "scn_conv_nin_supported": (C.c_int, [C.c_int, C.c_int, C.c_int]),
+        "scn_conv_nin_forward": (C.c_int, [vp, vp, vp, C.c_int, C.c_int, vp, vp, vp, vp, i64, C.c_int, f32, C.c_int]),
         "scn_maxpool": (C.c_int, [vp, vp, vp, vp, i64, C.c_int, C.c_int, vp]),
         "scn_terminal_pool": (C.c_int, [vp, vp, vp, vp, i64, C.c_int, C.c_int]),
         "scn_softmax_rows": (C.c_int, [vp, vp, vp, i64, C.c_int]),
@@ -208,6 +210,10 @@ class Context:
         _check(lib().scn_nin_forward(self.h, d_A.ptr, d_W.ptr, d_B.ptr,
                                      d_prelu.ptr if d_prelu is not None else None,
                                      d_out.ptr, M, K, N, p, act, precision))
+
+    def conv_nin_forward(self, d_in, d_rules, fs, nIn, d_W, d_B, d_prelu, d_out, M, N, p=1.0, act=RELU):
+        _check(lib().scn_conv_nin_forward(self.h, d_in.ptr, d_rules.ptr, fs, nIn, d_W.ptr, d_B.ptr,
+                                          d_prelu.ptr if d_prelu is not None else None, d_out.ptr, M, N, p, act))
 
     def maxpool(self, d_in, d_out, d_rules, nOutSites, ps, Cn, d_choice):
         _check(lib().scn_maxpool(self.h, d_in.ptr, d_out.ptr, d_rules.ptr, nOutSites, ps, Cn, d_choice.ptr))

@@ -114,11 +114,23 @@ __global__ void __launch_bounds__(256)
 #define MF_BK 32
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-template <int WM, int WN, int NT, int BK>
+//
+// GATHER: A is never materialised.  Row m of A is the receptive field of
+// output site m, column q * nIn + c = channel c of input row
+// rules[m * fs + q] (what scn_gather_rows would have written); the block's
+// rules are staged in LDS once and the A slabs are fetched through them.
+#define GF_MAX_FS 27
+struct GatherSource {
+  const int *rules; // [M x fs]
+  int fs;           // rule-row width
+  int nIn;          // channels of the gathered matrix, nIn % 4 == 0
+};
+
+template <int WM, int WN, int NT, int BK, bool GATHER>
 __global__ void __launch_bounds__(256)
     k_nin_mfma(const float *__restrict__ A, const float *__restrict__ W,
                float *__restrict__ out, long long M, int K, int N,
-               Epilogue ep) {
+               Epilogue ep, GatherSource gs) {
   constexpr int BM = 32 * WM;
   constexpr int BN = 32 * NT * WN;
   constexpr int BMP = BM + 1;
@@ -148,6 +160,15 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
     for (int v = 0; v < 16; ++v)
       acc[j][v] = 0.f;
+  __shared__ int sR[GATHER ? BM * GF_MAX_FS : 1];
+  if (GATHER) {
+    // the rules of rows m0 .. m0 + BM are one contiguous run
+    const long long first = m0 * gs.fs;
+    const long long limit = M * gs.fs;
+    for (int idx = tid; idx < BM * gs.fs; idx += 256)
+      sR[idx] = first + idx < limit ? gs.rules[first + idx] : -1;
+    __syncthreads();
+  }
 
   float4 ra[A_PER], rw[W_PER];
   auto load_slab = [&](int k0) {
@@ -158,8 +179,17 @@ __global__ void __launch_bounds__(256)
       long long m = m0 + r;
       int k = k0 + kc * 4;
       float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (c < A_CHUNKS && m < M && k < K) // K % 4 == 0: a chunk is all in or all out
-        v = *reinterpret_cast<const float4 *>(A + m * K + k);
+      if (c < A_CHUNKS && m < M && k < K) { // K % 4 == 0: a chunk is all in or all out
+        if (GATHER) {
+          int q = k / gs.nIn;
+          int rule = sR[r * gs.fs + q];
+          if (rule >= 0)
+            v = *reinterpret_cast<const float4 *>(
+                A + (long long)rule * gs.nIn + (k - q * gs.nIn));
+        } else {
+          v = *reinterpret_cast<const float4 *>(A + m * K + k);
+        }
+      }
       ra[u] = v;
     }
 #pragma unroll
@@ -429,18 +459,22 @@ static void launch_mfma_bf16(scn_ctx *ctx, const float *A, const float *W,
 template <int WM, int WN, int NT, int BK = MF_BK>
 static void launch_mfma(scn_ctx *ctx, const float *A, const float *W,
                         float *out, long long M, int K, int N,
-                        const Epilogue &ep) {
+                        const Epilogue &ep, const GatherSource *gs = nullptr) {
   constexpr int BM = 32 * WM, BN = 32 * NT * WN;
   long long tiles = (long long)scn_ceil_div(N, BN) * scn_ceil_div(M, BM);
   dim3 grid((unsigned)((tiles + 7) / 8 * 8));
-  hipLaunchKernelGGL((k_nin_mfma<WM, WN, NT, BK>), grid, dim3(256), 0,
-                     ctx->stream, A, W, out, M, K, N, ep);
+  if (gs)
+    hipLaunchKernelGGL((k_nin_mfma<WM, WN, NT, BK, true>), grid, dim3(256), 0,
+                       ctx->stream, A, W, out, M, K, N, ep, *gs);
+  else
+    hipLaunchKernelGGL((k_nin_mfma<WM, WN, NT, BK, false>), grid, dim3(256), 0,
+                       ctx->stream, A, W, out, M, K, N, ep, GatherSource());
 }
 
-extern "C" int scn_nin_forward(scn_ctx *ctx, const float *d_A,
-                               const float *d_W, const float *d_B,
-                               const float *d_prelu, float *d_out, int64_t M,
-                               int K, int N, float p, int act, int precision) {
+static int nin_forward(scn_ctx *ctx, const float *d_A, const float *d_W,
+                       const float *d_B, const float *d_prelu, float *d_out,
+                       int64_t M, int K, int N, float p, int act, int precision,
+                       const GatherSource *gs) {
   SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_nin_forward: null context");
   SCN_REQUIRE(M >= 0 && K >= 1 && N >= 1, SCN_ERR_ARG,
               "scn_nin_forward: M %lld K %d N %d", (long long)M, K, N);
@@ -465,7 +499,7 @@ extern "C" int scn_nin_forward(scn_ctx *ctx, const float *d_A,
   // SigmoidLayer.cu:204-213
   ep.slope = act == SCN_LEAKYRELU ? 0.01f : (act == SCN_VLEAKYRELU ? 0.333f : 0.f);
   ep.act = act;
-  ProfScope prof(ctx, SCN_K_NIN);
+  ProfScope prof(ctx, gs ? SCN_K_CONV_NIN : SCN_K_NIN);
   const bool vec = K % 4 == 0 && N % 4 == 0 && ((uintptr_t)d_A & 15) == 0 &&
                    ((uintptr_t)d_W & 15) == 0;
   // bf16 operands only where the contraction is big enough to matter; the
@@ -479,7 +513,7 @@ extern "C" int scn_nin_forward(scn_ctx *ctx, const float *d_A,
       launch_mfma_bf16<4, 1, 2>(ctx, d_A, d_W, d_out, M, K, N, ep, split);
     else
       launch_mfma_bf16<1, 4, 1>(ctx, d_A, d_W, d_out, M, K, N, ep, split);
-  } else if (vec && K >= 8) {
+  } else if ((vec && K >= 8) || gs) {
     // Tall tiles (128 rows), 64 columns wide, or 96 where that divides N
     // (measured on 12928 x 1280 x 480: 93 TFLOP/s against 73 with 64-column
     // tiles; wider tiles leave too few workgroups for 256 compute units).
@@ -489,26 +523,17 @@ extern "C" int scn_nin_forward(scn_ctx *ctx, const float *d_A,
     long long blocksTall = (long long)scn_ceil_div(M, 128) * nChunks;
     if (blocksTall * 2 < ctx->numCU && N > 32) {
       // too few rows to fill the chip with tall tiles: 32-row tiles
-      launch_mfma<1, 4, 1>(ctx, d_A, d_W, d_out, M, K, N, ep);
+      launch_mfma<1, 4, 1>(ctx, d_A, d_W, d_out, M, K, N, ep, gs);
     } else {
       switch (nt) {
       case 1:
-        launch_mfma<4, 1, 1>(ctx, d_A, d_W, d_out, M, K, N, ep);
+        launch_mfma<4, 1, 1>(ctx, d_A, d_W, d_out, M, K, N, ep, gs);
         break;
       case 2:
-        launch_mfma<4, 1, 2>(ctx, d_A, d_W, d_out, M, K, N, ep);
-        break;
-      case 3:
-        launch_mfma<4, 1, 3>(ctx, d_A, d_W, d_out, M, K, N, ep);
-        break;
-      case 4:
-        launch_mfma<4, 1, 4, 16>(ctx, d_A, d_W, d_out, M, K, N, ep);
-        break;
-      case 5:
-        launch_mfma<4, 1, 5, 16>(ctx, d_A, d_W, d_out, M, K, N, ep);
+        launch_mfma<4, 1, 2>(ctx, d_A, d_W, d_out, M, K, N, ep, gs);
         break;
       default:
-        launch_mfma<4, 1, 6, 16>(ctx, d_A, d_W, d_out, M, K, N, ep);
+        launch_mfma<4, 1, 3>(ctx, d_A, d_W, d_out, M, K, N, ep, gs);
         break;
       }
     }
@@ -521,4 +546,37 @@ extern "C" int scn_nin_forward(scn_ctx *ctx, const float *d_A,
   if (act == SCN_SOFTMAX)
     SCN_TRY(scn_softmax_launch(ctx, d_out, d_out, (long long)M, N));
   return SCN_OK;
+}
+
+extern "C" int scn_nin_forward(scn_ctx *ctx, const float *d_A,
+                               const float *d_W, const float *d_B,
+                               const float *d_prelu, float *d_out, int64_t M,
+                               int K, int N, float p, int act, int precision) {
+  return nin_forward(ctx, d_A, d_W, d_B, d_prelu, d_out, M, K, N, p, act,
+                     precision, nullptr);
+}
+
+extern "C" int scn_conv_nin_supported(int fs, int nIn, int N) {
+  return fs >= 1 && fs <= GF_MAX_FS && nIn >= 4 && nIn % 4 == 0 && N % 4 == 0;
+}
+
+extern "C" int scn_conv_nin_forward(scn_ctx *ctx, const float *d_in,
+                                    const int32_t *d_rules, int fs, int nIn,
+                                    const float *d_W, const float *d_B,
+                                    const float *d_prelu, float *d_out,
+                                    int64_t M, int N, float p, int act) {
+  SCN_REQUIRE(scn_conv_nin_supported(fs, nIn, N), SCN_ERR_ARG,
+              "scn_conv_nin_forward: fs %d nIn %d N %d is outside the fused "
+              "kernel's range (fs <= %d, nIn and N multiples of 4)",
+              fs, nIn, N, GF_MAX_FS);
+  SCN_REQUIRE(d_rules || M == 0, SCN_ERR_ARG,
+              "scn_conv_nin_forward: null rules");
+  SCN_REQUIRE(((uintptr_t)d_in & 15) == 0 && ((uintptr_t)d_W & 15) == 0,
+              SCN_ERR_ARG, "scn_conv_nin_forward: buffers must be 16-byte aligned");
+  GatherSource gs;
+  gs.rules = d_rules;
+  gs.fs = fs;
+  gs.nIn = nIn;
+  return nin_forward(ctx, d_in, d_W, d_B, d_prelu, d_out, M, fs * nIn, N, p,
+                     act, SCN_FP32, &gs);
 }

@@ -92,6 +92,11 @@ public:
   void saveWeights(std::string baseName, int epoch, bool momentum);
   // set the operand precision of every NiN contraction (SCN_FP32 / SCN_BF16)
   void setPrecision(int precision);
+  // Fuse every convolutional layer's gather into the NiN layer that follows
+  // it (one kernel, the im2col-like matrix is never written).  Same results;
+  // the convolution's output interface then holds rules but no features.
+  // Off by default, as the reference materialises that matrix.
+  void setFusedConvolutions(bool on);
   // grows every slot's interface list to layers.size() + 1
   void ensureInterfaces();
   // Fills slot cc's input interface from a batch that already sits in HBM

@@ -30,6 +30,10 @@ public:
   scn_grids *deviceGrids;
   bool ownsDeviceGrids;
   vectorCUDA<int> rules;
+  // Set by a convolutional layer that left its gather to the following NiN
+  // layer (fused kernel): the interface whose features the rules index.  The
+  // feature matrix of THIS interface is then not materialised.
+  SpatiallySparseBatchInterface *deferredGatherFrom;
   SpatiallySparseBatchInterface(SpatiallySparseBatchSubInterface *s);
   SpatiallySparseBatchInterface(SpatiallySparseBatchInterface &&o);
   ~SpatiallySparseBatchInterface();

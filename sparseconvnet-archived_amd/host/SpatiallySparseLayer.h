@@ -51,6 +51,9 @@ public:
   int nFeaturesIn;
   int nFeaturesOut;
   int minActiveInputs; // 1; > 1; or -1 for 'valid' mode
+  // leave the gather to the NiN layer that follows (fused kernel); set by
+  // SparseConvNetCUDA::setFusedConvolutions
+  bool deferGather;
   ConvolutionalLayer(cudaMemStream &memStream, int filterSize,
                      int filterStride, int dimension, int nFeaturesIn,
                      int minActiveInputs = 1);
@@ -77,6 +80,7 @@ public:
   int nFeaturesIn;
   int nFeaturesOut;
   int minActiveInputs;
+  bool deferGather;
   ConvolutionalTriangularLayer(cudaMemStream &memStream, int filterSize,
                                int filterStride, int dimension,
                                int nFeaturesIn, int minActiveInputs = 1);

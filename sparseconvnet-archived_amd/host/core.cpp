@@ -275,7 +275,7 @@ void SpatiallySparseBatchSubInterface::reset() {
 SpatiallySparseBatchInterface::SpatiallySparseBatchInterface(
     SpatiallySparseBatchSubInterface *s)
     : sub(s), featuresPresent(false, 0), deviceGrids(nullptr),
-      ownsDeviceGrids(false), rules(true, 0) {
+      ownsDeviceGrids(false), rules(true, 0), deferredGatherFrom(nullptr) {
   reset();
 }
 SpatiallySparseBatchInterface::SpatiallySparseBatchInterface(
@@ -285,7 +285,7 @@ SpatiallySparseBatchInterface::SpatiallySparseBatchInterface(
       nSpatialSites(o.nSpatialSites), spatialSize(o.spatialSize),
       backpropErrors(o.backpropErrors), grids(std::move(o.grids)),
       deviceGrids(o.deviceGrids), ownsDeviceGrids(o.ownsDeviceGrids),
-      rules(std::move(o.rules)) {
+      rules(std::move(o.rules)), deferredGatherFrom(nullptr) {
   o.deviceGrids = nullptr;
   o.ownsDeviceGrids = false;
 }
@@ -299,6 +299,7 @@ void SpatiallySparseBatchInterface::reset() {
   grids.resize(0);
   rules.resize(0);
   backpropErrors = false;
+  deferredGatherFrom = nullptr;
   // deviceGrids keeps its tables for the next batch
 }
 // Rebuilds the host SparseGrid view from the tables in HBM.

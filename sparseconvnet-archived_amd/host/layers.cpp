@@ -63,6 +63,19 @@ static void fill_rules(scn_ctx *ctx, SpatiallySparseBatchInterface &input,
                              output.rules.dPtr(), nRules));
 }
 
+// materialise the im2col-like matrix of a convolution's output interface
+static void gather_now(cudaMemStream &ms, SpatiallySparseBatchInterface &input,
+                       SpatiallySparseBatchInterface &output) {
+  const size_t nIn = input.featuresPresent.size();
+  const size_t width = output.featuresPresent.size(); // fs * nIn
+  output.sub->features.resize64((size_t)output.nSpatialSites * width);
+  SCN_CHECKED(scn_gather_rows(ms.ctx, input.sub->features.dPtr(),
+                              output.sub->features.dPtr(), output.rules.dPtr(),
+                              (int64_t)output.nSpatialSites * (width / nIn),
+                              (int)nIn));
+  output.deferredGatherFrom = nullptr;
+}
+
 // featuresPresent of a convolution's output: fs copies of the input's list,
 // shifted by nf per copy (ConvolutionalLayer.cu:74-80)
 static void convolutionFeaturesPresent(std::vector<int> &src,
@@ -80,7 +93,8 @@ ConvolutionalLayer::ConvolutionalLayer(cudaMemStream &memStream,
                                        int minActiveInputs)
     : SpatiallySparseLayer(memStream), inSpatialSize(0), outSpatialSize(0),
       filterSize(filterSize), filterStride(filterStride), dimension(dimension),
-      nFeaturesIn(nFeaturesIn), minActiveInputs(minActiveInputs) {
+      nFeaturesIn(nFeaturesIn), minActiveInputs(minActiveInputs),
+      deferGather(false) {
   fs = ipow(filterSize, dimension);
   nFeaturesOut = fs * nFeaturesIn;
   std::cout << "Convolution " << filterSize << "^" << dimension << "x"
@@ -116,11 +130,11 @@ void ConvolutionalLayer::forwards(SpatiallySparseBatch &batch,
                                   SpatiallySparseBatchInterface &input,
                                   SpatiallySparseBatchInterface &output) {
   (void)batch;
-  const size_t nIn = input.featuresPresent.size();
-  output.sub->features.resize64((size_t)output.nSpatialSites * nIn * fs);
-  SCN_CHECKED(scn_gather_rows(memStream.ctx, input.sub->features.dPtr(),
-                              output.sub->features.dPtr(), output.rules.dPtr(),
-                              (int64_t)output.nSpatialSites * fs, (int)nIn));
+  if (deferGather) { // the following NiN layer reads the input through the rules
+    output.deferredGatherFrom = &input;
+    return;
+  }
+  gather_now(memStream, input, output);
 }
 int ConvolutionalLayer::calculateInputSpatialSize(int outputSpatialSize) {
   outSpatialSize = outputSpatialSize;
@@ -138,7 +152,8 @@ ConvolutionalTriangularLayer::ConvolutionalTriangularLayer(
     int nFeaturesIn, int minActiveInputs)
     : SpatiallySparseLayer(memStream), inSpatialSize(0), outSpatialSize(0),
       filterSize(filterSize), filterStride(filterStride), dimension(dimension),
-      nFeaturesIn(nFeaturesIn), minActiveInputs(minActiveInputs) {
+      nFeaturesIn(nFeaturesIn), minActiveInputs(minActiveInputs),
+      deferGather(false) {
   fs = triangleSize(filterSize, dimension);
   nFeaturesOut = fs * nFeaturesIn;
   std::cout << dimension
@@ -172,11 +187,11 @@ void ConvolutionalTriangularLayer::forwards(
     SpatiallySparseBatch &batch, SpatiallySparseBatchInterface &input,
     SpatiallySparseBatchInterface &output) {
   (void)batch;
-  const size_t nIn = input.featuresPresent.size();
-  output.sub->features.resize64((size_t)output.nSpatialSites * nIn * fs);
-  SCN_CHECKED(scn_gather_rows(memStream.ctx, input.sub->features.dPtr(),
-                              output.sub->features.dPtr(), output.rules.dPtr(),
-                              (int64_t)output.nSpatialSites * fs, (int)nIn));
+  if (deferGather) { // the following NiN layer reads the input through the rules
+    output.deferredGatherFrom = &input;
+    return;
+  }
+  gather_now(memStream, input, output);
 }
 int ConvolutionalTriangularLayer::calculateInputSpatialSize(
     int outputSpatialSize) {
@@ -203,6 +218,30 @@ static void nin_preprocess(int nFeaturesIn, int nFeaturesOut,
   output.featuresPresent.hVector() = range(nFeaturesOut);
   output.backpropErrors = true;
 }
+// When the preceding convolutional layer deferred its gather: run the fused
+// kernel (fp32 operands), or gather now if this layer wants bf16 operands.
+// Returns false when the input is an ordinary feature matrix.
+static bool nin_fused(cudaMemStream &ms, SpatiallySparseBatchInterface &input,
+                      SpatiallySparseBatchInterface &output,
+                      vectorCUDA<float> &W, vectorCUDA<float> &B,
+                      vectorCUDA<float> *prelu, int nFeaturesOut, float p,
+                      int act, int precision) {
+  SpatiallySparseBatchInterface *src = input.deferredGatherFrom;
+  if (!src)
+    return false;
+  const int nIn = src->nFeatures;
+  const int fs = input.nFeatures / nIn;
+  if (precision != SCN_FP32 || !scn_conv_nin_supported(fs, nIn, nFeaturesOut)) {
+    gather_now(ms, *src, input);
+    return false;
+  }
+  SCN_CHECKED(scn_conv_nin_forward(
+      ms.ctx, src->sub->features.dPtr(), input.rules.dPtr(), fs, nIn, W.dPtr(),
+      B.dPtr(), prelu ? prelu->dPtr() : nullptr, output.sub->features.dPtr(),
+      output.nSpatialSites, nFeaturesOut, p, act));
+  return true;
+}
+
 static void read_floats(std::ifstream &f, vectorCUDA<float> &v) {
   std::vector<float> &h = v.hVector();
   f.read((char *)h.data(), sizeof(float) * h.size());
@@ -247,11 +286,13 @@ void NetworkInNetworkLayer::forwards(SpatiallySparseBatch &batch,
   output.sub->features.resize64((size_t)output.nSpatialSites * nFeaturesOut);
   // test-time scaling by the kept fraction (NetworkInNetworkLayer.cu:188)
   float p = 1.0f - (batch.type != RESCALEBATCH ? dropout : 0.0f);
-  SCN_CHECKED(scn_nin_forward(memStream.ctx, input.sub->features.dPtr(),
-                              W.dPtr(), B.dPtr(), nullptr,
-                              output.sub->features.dPtr(),
-                              output.nSpatialSites, nFeaturesIn, nFeaturesOut,
-                              p, (int)fn, precision));
+  if (!nin_fused(memStream, input, output, W, B, nullptr, nFeaturesOut, p,
+                 (int)fn, precision))
+    SCN_CHECKED(scn_nin_forward(memStream.ctx, input.sub->features.dPtr(),
+                                W.dPtr(), B.dPtr(), nullptr,
+                                output.sub->features.dPtr(),
+                                output.nSpatialSites, nFeaturesIn, nFeaturesOut,
+                                p, (int)fn, precision));
   multiplyAddCount +=
       (__int128_t)output.nSpatialSites * nFeaturesIn * nFeaturesOut;
 }
@@ -313,11 +354,13 @@ void NetworkInNetworkPReLULayer::forwards(
     SpatiallySparseBatchInterface &output) {
   output.sub->features.resize64((size_t)output.nSpatialSites * nFeaturesOut);
   float p = 1.0f - (batch.type != RESCALEBATCH ? dropout : 0.0f);
-  SCN_CHECKED(scn_nin_forward(memStream.ctx, input.sub->features.dPtr(),
-                              W.dPtr(), B.dPtr(), PReLU.dPtr(),
-                              output.sub->features.dPtr(),
-                              output.nSpatialSites, nFeaturesIn, nFeaturesOut,
-                              p, (int)PRELU, precision));
+  if (!nin_fused(memStream, input, output, W, B, &PReLU, nFeaturesOut, p,
+                 (int)PRELU, precision))
+    SCN_CHECKED(scn_nin_forward(memStream.ctx, input.sub->features.dPtr(),
+                                W.dPtr(), B.dPtr(), PReLU.dPtr(),
+                                output.sub->features.dPtr(),
+                                output.nSpatialSites, nFeaturesIn, nFeaturesOut,
+                                p, (int)PRELU, precision));
   multiplyAddCount +=
       (__int128_t)output.nSpatialSites * nFeaturesIn * nFeaturesOut;
 }

@@ -152,6 +152,25 @@ void SparseConvNetCUDA::addSoftmaxLayer() {
     std::cout << "x" << inputSpatialSize;
   std::cout << std::endl;
 }
+void SparseConvNetCUDA::setFusedConvolutions(bool on) {
+  for (size_t i = 0; i + 1 < layers.size(); ++i) {
+    int nOut = 0;
+    if (auto *n = dynamic_cast<NetworkInNetworkLayer *>(layers[i + 1]))
+      nOut = n->nFeaturesOut;
+    else if (auto *n = dynamic_cast<NetworkInNetworkPReLULayer *>(layers[i + 1]))
+      nOut = n->nFeaturesOut;
+    if (auto *c = dynamic_cast<ConvolutionalLayer *>(layers[i]))
+      c->deferGather =
+          on && nOut > 0 &&
+          scn_conv_nin_supported(c->nFeaturesOut / c->nFeaturesIn,
+                                 c->nFeaturesIn, nOut);
+    if (auto *c = dynamic_cast<ConvolutionalTriangularLayer *>(layers[i]))
+      c->deferGather =
+          on && nOut > 0 &&
+          scn_conv_nin_supported(c->nFeaturesOut / c->nFeaturesIn,
+                                 c->nFeaturesIn, nOut);
+  }
+}
 void SparseConvNetCUDA::ensureInterfaces() {
   // one shared sub-interface per depth, one interface per depth and slot
   // (BatchProducer.cu:28-33)

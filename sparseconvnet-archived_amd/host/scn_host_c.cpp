@@ -93,6 +93,9 @@ int scnh_finish_headless(scnh_net *net, int topSpatialSize) {
   std::cout << std::endl;
   return cnn->inputSpatialSize;
 }
+void scnh_set_fused_convolutions(scnh_net *net, int on) {
+  net->cnn->setFusedConvolutions(on != 0);
+}
 void scnh_set_precision(scnh_net *net, int precision) {
   net->cnn->setPrecision(precision);
 }
@@ -241,7 +244,8 @@ void scnh_iface_info(scnh_net *net, int i, int *nFeatures, int *nSpatialSites,
   *nSpatialSites = f.nSpatialSites;
   *spatialSize = f.spatialSize;
   *nRules = (int64_t)f.rules.size64();
-  *nFeatureElems = (int64_t)f.nSpatialSites * f.nFeatures;
+  *nFeatureElems =
+      f.deferredGatherFrom ? 0 : (int64_t)f.nSpatialSites * f.nFeatures;
   *nChoices = (int64_t)f.sub->poolingChoices.size64();
   int64_t n = 0;
   if (f.deviceGrids)

@@ -41,6 +41,7 @@ def lib():
         "scnh_add_softmax_layer": (None, [vp]),
         "scnh_finish_headless": (i32, [vp, i32]),
         "scnh_set_precision": (None, [vp, i32]),
+        "scnh_set_fused_convolutions": (None, [vp, i32]),
         "scnh_input_spatial_size": (i32, [vp]),
         "scnh_n_layers": (i32, [vp]),
         "scnh_layer_info": (i32, [vp, i32, P(i32), P(i32), P(i32)]),
@@ -142,6 +143,9 @@ class Net:
     def finishHeadless(self, topSpatialSize):
         return lib().scnh_finish_headless(self.h, topSpatialSize)
 
+    def setFusedConvolutions(self, on=True):
+        lib().scnh_set_fused_convolutions(self.h, int(on))
+
     def setPrecision(self, precision):
         lib().scnh_set_precision(self.h, precision)
 
@@ -210,7 +214,8 @@ class Net:
             L.scnh_iface_rules(self.h, i, _p(rules))
         out["rules"] = rules
         if want_features:
-            feats = np.empty((ns.value, nf.value), np.float32)
+            # None: a convolution's output whose gather was fused into the next NiN layer
+            feats = np.empty((ns.value, nf.value), np.float32) if (ne.value or ns.value == 0) else None
             if ne.value:
                 L.scnh_iface_features(self.h, i, _p(feats))
             out["features"] = feats

@@ -196,3 +196,33 @@ def test_argument_errors(scn, ctx):
     ctx.gather_rows(d, d, r, 0, 4)
     ctx.maxpool(d, d, r, 0, 2, 4, r)
     ctx.sync()
+
+
+@pytest.mark.parametrize("rows,fs,nIn,N", [(700, 4, 32, 64), (3000, 9, 64, 96), (513, 27, 64, 64), (129, 8, 96, 128),
+                                           (5000, 4, 128, 160), (64, 1, 4, 32), (300, 25, 8, 100)])
+@pytest.mark.parametrize("act", ["RELU", "PRELU"])
+def test_fused_gather_nin_matches_the_two_kernels_bit_for_bit(scn, ctx, rows, fs, nIn, N, act):
+    a = getattr(scn, act)
+    rng = np.random.default_rng(rows + fs + nIn + N)
+    nInRows = 400
+    inp = rng.uniform(-1, 1, (nInRows, nIn)).astype(np.float32)
+    rules = rng.integers(0, nInRows, (rows, fs)).astype(np.int32)
+    K = fs * nIn
+    W = (rng.standard_normal((K, N)) * np.sqrt(2.0 / K)).astype(np.float32)
+    B = rng.uniform(-0.5, 0.5, N).astype(np.float32)
+    pr = rng.uniform(0.1, 0.4, N).astype(np.float32)
+    assert scn.lib().scn_conv_nin_supported(fs, nIn, N)
+    print("fused rows=%d fs=%d nIn=%d N=%d" % (rows, fs, nIn, N), flush=True)
+    d_in, d_rules, d_W, d_B, d_pr = ctx.array(inp), ctx.array(rules), ctx.array(W), ctx.array(B), ctx.array(pr)
+    fused = ctx.empty((rows, N), np.float32)
+    ctx.conv_nin_forward(d_in, d_rules, fs, nIn, d_W, d_B, d_pr, fused, rows, N, 1.0, a)
+    g = ctx.empty((rows, K), np.float32)
+    two = ctx.empty((rows, N), np.float32)
+    ctx.gather_rows(d_in, g, d_rules, rows * fs, nIn)
+    ctx.nin_forward(g, d_W, d_B, d_pr, two, rows, K, N, 1.0, a, scn.FP32)
+    assert np.array_equal(fused.download(), two.download())
+    want = orc.nin_forward(orc.gather_rows(inp, rules.ravel(), nIn).reshape(rows, K), W, B, pr, 1.0, a, f64=True)
+    scale = np.abs(inp[rules].reshape(rows, K)).astype(np.float64) @ np.abs(W).astype(np.float64) + np.abs(B)
+    assert np.all(np.abs(fused.download() - want) <= 1e-4 * scale)
+    assert not scn.lib().scn_conv_nin_supported(64, 32, 64)  # window too large for the staged rules
+    assert not scn.lib().scn_conv_nin_supported(4, 3, 32)  # channels not a multiple of 4

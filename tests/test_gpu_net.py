@@ -28,9 +28,10 @@ def build_pair(cfg, hostapi, triangular=False):
     return net, ora
 
 
-def run_config(scn, cfg, seed, tol=1e-4, triangular=False, samples=None):
+def run_config(scn, cfg, seed, tol=1e-4, triangular=False, samples=None, fused=False):
     from sparseconvnet_archived_amd import hostapi, synthetic
     net, ora = build_pair(cfg, hostapi, triangular)
+    net.setFusedConvolutions(fused)
     weights = synthetic.he_normal_weights(net.layers(), seed + 1)
     for i, (W, B, pr) in weights.items():
         net.set_weights(i, W, B, pr)
@@ -57,6 +58,10 @@ def run_config(scn, cfg, seed, tol=1e-4, triangular=False, samples=None):
         s, k, r, b = gi["grids"]
         os_, ok, or_, ob = wi["grids"].flat()
         assert np.array_equal(s, os_) and np.array_equal(k, ok) and np.array_equal(r, or_) and np.array_equal(b, ob)
+        if gi["features"] is None:
+            # the gather of this convolution runs inside the next NiN kernel
+            assert fused and layers[i - 1]["kind"].startswith("conv") and layers[i]["kind"].startswith("nin")
+            continue
         # activations: 1e-4 relative (fp32)
         err = rel_l2(gi["features"], wi["features"])
         print("    rel-L2 error %.3g" % err, flush=True)
@@ -124,6 +129,67 @@ def test_triangular_net(scn):
         pts = np.array([(a, b) for a in range(13) for b in range(13 - a) if rng.random() < 0.4], np.int32)
         samples.append((pts, rng.uniform(-1, 1, (len(pts), 3)).astype(np.float32), int(rng.integers(0, 10))))
     run_config(scn, cfg, 7, triangular=True, samples=samples)
+
+
+@pytest.mark.parametrize("number,batch,seed", [(2, 20, 202), (3, 6, 203), (4, 2, 204), (5, 1, 205)])
+def test_fused_convolutions_against_oracle(scn, number, batch, seed):
+    """setFusedConvolutions: the gather runs inside the NiN kernel; everything
+    downstream has to meet the same bars against the oracle."""
+    from sparseconvnet_archived_amd import synthetic
+    run_config(scn, synthetic.config(number, batch=batch), seed, fused=True)
+
+
+def test_fused_convolutions_triangular(scn):
+    from sparseconvnet_archived_amd import synthetic
+    stack = [("addLeNetLayerMP", 32, 2, 1, 2, 2, synthetic.RELU), ("addLeNetLayerMP", 64, 2, 1, 2, 2, synthetic.RELU),
+             ("addLeNetLayerMP", 64, 2, 1, 1, 1, synthetic.VLEAKYRELU), ("addTerminalPoolingLayer", 2), ("addSoftmaxLayer",)]
+    cfg = synthetic.Config("tri", 2, 3, 10, 8, 13, stack)
+    cfg.number = 2
+    rng = np.random.default_rng(6)
+    samples = []
+    for _ in range(8):
+        pts = np.array([(a, b) for a in range(13) for b in range(13 - a) if rng.random() < 0.4], np.int32)
+        samples.append((pts, rng.uniform(-1, 1, (len(pts), 3)).astype(np.float32), int(rng.integers(0, 10))))
+    run_config(scn, cfg, 8, triangular=True, samples=samples, fused=True)
+
+
+@pytest.mark.parametrize("precision", ["FP32", "BF16X3"])
+def test_fused_convolutions_change_no_bit(scn, precision):
+    """The same net, weights and batch with and without fusion: every
+    materialised interface and the class probabilities are identical bit for
+    bit, and at least one convolution really was fused.  With bf16 operands
+    the NiN layer gathers first, so nothing may change either."""
+    from sparseconvnet_archived_amd import hostapi, synthetic
+    cfg = synthetic.config(2, batch=12)
+    samples = synthetic.make_samples(cfg, 55)
+    runs = []
+    for fused in (False, True):
+        net, _ = build_pair(cfg, hostapi)
+        net.setPrecision(getattr(scn, precision))
+        net.setFusedConvolutions(fused)
+        for i, (W, B, pr) in synthetic.he_normal_weights(net.layers(), 56).items():
+            net.set_weights(i, W, B, pr)
+        ds = hostapi.Dataset("fused", 3, 100, hostapi.TESTBATCH)
+        for pts, f, label in samples:
+            ds.add_points(2, cfg.lattice, pts, f, label)
+        net.begin(ds, len(samples))
+        assert net.next_batch()
+        ifaces = [net.interface(i) for i in range(len(net.layers()) + 1)]
+        runs.append((ifaces, net.batch_outputs()))
+        net.end()
+        net.close()
+    (plain, out0), (fusedrun, out1) = runs
+    skipped = 0
+    for a, b in zip(plain, fusedrun):
+        assert np.array_equal(a["rules"], b["rules"]) and np.array_equal(a["choices"], b["choices"])
+        if b["features"] is None:
+            skipped += 1
+            continue
+        assert np.array_equal(a["features"], b["features"])
+    assert np.array_equal(out0["probabilities"], out1["probabilities"])
+    assert skipped >= (3 if precision == "FP32" else 0)
+    if precision != "FP32":
+        assert skipped == 0
 
 
 def test_process_dataset_and_weight_files(scn, tmp_path):
