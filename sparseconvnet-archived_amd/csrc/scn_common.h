@@ -39,6 +39,7 @@ struct ProfSpan {
   hipEvent_t a, b;
 };
 
+#define SCN_ZERO_FLOATS 4096
 struct scn_ctx {
   int device;
   hipStream_t stream;
@@ -47,6 +48,7 @@ struct scn_ctx {
   int64_t *h_pinned; // 16 int64, host view
   int64_t *d_pinned; // the same memory as the device sees it
   int64_t *d_scalars; // 16 int64
+  float *d_zeros;     // SCN_ZERO_FLOATS zeros: the row a negative rule stands for
   // profiling
   bool prof;
   int profTag;

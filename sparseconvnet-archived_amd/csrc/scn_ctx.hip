@@ -40,6 +40,8 @@ extern "C" int scn_ctx_create(int device, scn_ctx **out) {
   SCN_HIP_CHECK(hipHostGetDevicePointer((void **)&c->d_pinned, c->h_pinned, 0));
   SCN_HIP_CHECK(hipMalloc((void **)&c->d_scalars, 16 * sizeof(int64_t)));
   SCN_HIP_CHECK(hipMemset(c->d_scalars, 0, 16 * sizeof(int64_t)));
+  SCN_HIP_CHECK(hipMalloc((void **)&c->d_zeros, SCN_ZERO_FLOATS * sizeof(float)));
+  SCN_HIP_CHECK(hipMemset(c->d_zeros, 0, SCN_ZERO_FLOATS * sizeof(float)));
   *out = c;
   return SCN_OK;
 }
@@ -55,6 +57,7 @@ extern "C" int scn_ctx_destroy(scn_ctx *c) {
   for (auto e : c->freeEvents)
     (void)hipEventDestroy(e);
   (void)hipFree(c->d_scalars);
+  (void)hipFree(c->d_zeros);
   (void)hipHostFree(c->h_pinned);
   (void)hipStreamDestroy(c->stream);
   delete c;

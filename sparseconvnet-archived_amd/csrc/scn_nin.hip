@@ -32,6 +32,30 @@ __device__ __forceinline__ float apply_act(float acc, int n,
   }
 }
 
+// The same, branch-free, for kernels that keep the column's constants in
+// registers: every supported activation is v > 0 ? v : v * slope with slope
+// 1 (none), 0 (ReLU), a constant (leaky) or PReLU's learnt per-column value.
+struct ColEpilogue {
+  float pb;    // p * bias[n]
+  float p;
+  float slope;
+};
+__device__ __forceinline__ ColEpilogue load_col(const Epilogue &e, int n) {
+  ColEpilogue c;
+  c.p = e.p;
+  c.pb = e.p * e.bias[n];
+  c.slope = e.act == SCN_PRELU
+                ? e.prelu[n]
+                : (e.act == SCN_RELU ? 0.f
+                                     : (e.act == SCN_LEAKYRELU || e.act == SCN_VLEAKYRELU ? e.slope : 1.f));
+  return c;
+}
+__device__ __forceinline__ float finish(float acc, const ColEpilogue &c) {
+  const float v = c.p * acc + c.pb;
+  const float neg = c.slope == 0.f ? 0.f : v * c.slope;
+  return v > 0.f ? v : neg;
+}
+
 // ---- generic path: any M, K, N; 64x64 tile, 4x4 per lane, fp32 FMA --------
 #define GT_BM 64
 #define GT_BN 64
@@ -121,9 +145,11 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 // rules are staged in LDS once and the A slabs are fetched through them.
 #define GF_MAX_FS 27
 struct GatherSource {
-  const int *rules; // [M x fs]
-  int fs;           // rule-row width
-  int nIn;          // channels of the gathered matrix, nIn % 4 == 0
+  const int *rules;   // [M x fs]
+  int fs;             // rule-row width
+  int nIn;            // channels of the gathered matrix, nIn % 4 == 0
+  unsigned magic;     // floor(2^32 / nIn) + 1: k / nIn == mulhi(k, magic) for k nIn < 2^32
+  const float *zeros; // at least nIn zeros: the row a negative rule stands for
 };
 
 template <int WM, int WN, int NT, int BK, bool GATHER>
@@ -261,6 +287,372 @@ __global__ void __launch_bounds__(256)
         out[m * N + n] = apply_act(acc[j][v], n, ep);
     }
   }
+}
+
+// ---- MFMA shapes used by the W-resident path --------------------------------
+//   ROWS 32: v_mfma_f32_32x32x2_f32, lane = (c = l % 32, q = l / 32)
+//   ROWS 16: v_mfma_f32_16x16x4_f32, lane = (c = l % 16, q = l / 16)
+// Lane (c, q) supplies A[row c][k-slot q] and W[k-slot q][column c]; accumulator
+// register v of that lane is D[row 4 q + v][column c] (16 rows) or
+// D[row 8 (v / 4) + 4 q + v % 4][column c] (32 rows).
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+template <int ROWS> struct DirectAcc;
+template <> struct DirectAcc<32> {
+  typedef floatx16 type;
+  static __device__ __forceinline__ type mfma(float a, float b, type c) {
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct DirectAcc<16> {
+  typedef floatx4 type;
+  static __device__ __forceinline__ type mfma(float a, float b, type c) {
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+  }
+};
+
+// ---- W-resident MFMA path ---------------------------------------------------
+// For the many layers whose weight slice fits in LDS (K x NW floats, up to
+// 160 KB).  A workgroup of eight wavefronts copies its slice of W into LDS once
+// and then every wavefront walks its own row panels (ROWS rows x NW columns):
+// A goes from global memory straight into the MFMA register layout (a lane
+// fetches 16 contiguous bytes of its row, k = KS t + 4 q + i, and MFMA i of
+// the step consumes element i, so k-slot q of that MFMA stands for that k in
+// both operands), prefetched SA - 1 k-steps ahead and across panel boundaries,
+// W is read from LDS one step ahead.  No barrier is executed after the W copy.
+// LDS row pitch NW + 4 keeps the two or four k-rows a wavefront reads at once
+// in different banks.
+//
+// Loads and stores retire in issue order through one counter, and the compiler
+// derives every wait from what it can prove is in flight.  So (1) every load in
+// the pipeline is unconditional (addresses are clamped instead); (2) a panel's
+// first k-steps, which run while the previous panel's stores drain, are a code
+// copy of their own, entered only from an epilogue, so that their waits count
+// those stores instead of waiting for them; (3) the one ragged panel (M not a
+// multiple of ROWS), whose stores are predicated, is handled after the loop.
+template <int ROWS, int NT, int SA> struct WresPipe {
+  typedef typename DirectAcc<ROWS>::type acc_t;
+  static constexpr int KQ = 64 / ROWS;
+  static constexpr int KS = 4 * KQ;
+  static constexpr int VPT = ROWS * ROWS / 64;
+  static constexpr int NW = ROWS * NT;
+  static constexpr int PITCH = NW + 4;
+
+  float4 a[SA];
+  float b[2][4][NT];
+  acc_t acc[NT];
+
+  __device__ __forceinline__ void read_w(const float *wl, int t, int slot) {
+    const float *wk = wl + KS * t * PITCH;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+        b[slot][i][j] = wk[i * PITCH + ROWS * j];
+  }
+  __device__ __forceinline__ void clear() {
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int v = 0; v < VPT; ++v)
+        acc[j][v] = 0.f;
+  }
+  // SA k-steps starting at t0 (t0 % SA == 0; SA is even, so the W slot parity
+  // survives from group to group).  addr(tt) is where this lane's 16 bytes of
+  // k-step tt are; it is called with consecutive tt, and tt >= T means step
+  // tt - T of the next panel.
+  template <class Addr>
+  __device__ __forceinline__ void group(int t0, int T, Addr &addr,
+                                        const float *wl) {
+#pragma unroll
+    for (int s = 0; s < SA; ++s) {
+      const int t = t0 + s;
+      a[(s + SA - 1) % SA] =
+          *reinterpret_cast<const float4 *>(addr(t + SA - 1));
+      read_w(wl, t + 1 < T ? t + 1 : 0, (s + 1) & 1);
+      // keep this step's prefetches ahead of its MFMAs and inside the step
+      __builtin_amdgcn_sched_barrier(0);
+      const float av[4] = {a[s].x, a[s].y, a[s].z, a[s].w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+          acc[j] = DirectAcc<ROWS>::mfma(av[i], b[s & 1][i][j], acc[j]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  template <bool GUARDED>
+  __device__ __forceinline__ void store(float *orow, int N, long long rowsLeft,
+                                        int q, const ColEpilogue (&col)[NT]) {
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int v = 0; v < VPT; ++v) {
+        const int r = ROWS == 32 ? 8 * (v / 4) + (v % 4) : v;
+        if (!GUARDED || 4 * q + r < rowsLeft)
+          orow[(long long)r * N + ROWS * j] = finish(acc[j][v], col[j]);
+      }
+  }
+};
+
+template <int ROWS, int NT, int SA, bool GATHER>
+__global__ void __launch_bounds__(512)
+    k_nin_wres(const float *__restrict__ A, const float *__restrict__ W,
+               float *__restrict__ out, long long M, int K, int N, Epilogue ep,
+               GatherSource gs, int nSplits) {
+  typedef WresPipe<ROWS, NT, SA> Pipe;
+  constexpr int KS = Pipe::KS, NW = Pipe::NW, PITCH = Pipe::PITCH;
+  extern __shared__ __attribute__((aligned(16))) float sW[]; // [K][PITCH]
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int c = lane % ROWS, q = lane / ROWS;
+  const int split = blockIdx.x % nSplits; // workgroups that share rows are neighbours
+  const int wg = blockIdx.x / nSplits;
+  const int wgs = gridDim.x / nSplits;
+  const int n0 = split * NW;
+  const long long nFull = M / ROWS;
+  const long long nPanels = (M + ROWS - 1) / ROWS;
+  const long long stride = (long long)wgs * 8;
+  long long panel = (long long)wave * wgs + wg;
+  const int T = K / KS;
+
+  // Where lane (c, q) finds k-steps of a panel.  Plain: a row of A.  GATHER:
+  // through this wavefront's copy of the panel's rules in LDS, two buffers
+  // (this panel, next panel); the rule for the next call is fetched one call
+  // ahead so that its LDS latency is off the path.
+  int *const sRw = reinterpret_cast<int *>(sW + (size_t)K * PITCH) +
+                   wave * (2 * ROWS * gs.fs);
+  const int rulesPerPanel = ROWS * gs.fs;
+  auto row_of = [&](long long pnl) {
+    long long m = pnl * ROWS + c;
+    return m < M ? m : M - 1; // rows past the end: read a valid row, store nothing
+  };
+  struct {
+    const float *cur, *nxt; // plain
+    long long wrap;
+    int bufCur, bufNext, rule, ch; // gather
+  } st;
+  auto addr = [&](int tt) -> const float * {
+    if (!GATHER)
+      return st.cur + KS * tt + (tt >= T ? st.wrap : 0ll);
+    const float *p =
+        (st.rule >= 0 ? A + (long long)st.rule * gs.nIn : gs.zeros) + st.ch;
+    const int tn = tt + 1;
+    const int kn = KS * (tn >= T ? tn - T : tn) + 4 * q;
+    const int fn = (int)__umulhi((unsigned)kn, gs.magic);
+    st.ch = kn - fn * gs.nIn;
+    st.rule = sRw[(tn >= T ? st.bufNext : st.bufCur) + c * gs.fs + fn];
+    return p;
+  };
+  // GATHER: the rules of panel pnl, 64 consecutive ints per load
+  constexpr int RU = GATHER ? (ROWS * GF_MAX_FS + 63) / 64 : 1;
+  int rr[RU];
+  auto fetch_rules = [&](long long pnl) {
+    if (pnl >= nPanels)
+      pnl = nPanels - 1;
+    const long long first = pnl * rulesPerPanel, last = M * gs.fs - 1;
+#pragma unroll
+    for (int u = 0; u < RU; ++u) {
+      long long i = first + lane + 64 * u;
+      rr[u] = gs.rules[i < last ? i : last];
+    }
+  };
+  auto keep_rules = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < RU; ++u)
+      if (lane + 64 * u < rulesPerPanel)
+        sRw[buf + lane + 64 * u] = rr[u];
+  };
+
+  Pipe pipe;
+  if (GATHER) {
+    st.bufCur = 0;
+    st.bufNext = rulesPerPanel;
+    fetch_rules(panel);
+    keep_rules(0);
+    fetch_rules(panel + stride);
+    st.ch = 4 * q - (int)__umulhi((unsigned)(4 * q), gs.magic) * gs.nIn;
+    st.rule = sRw[c * gs.fs + (int)__umulhi((unsigned)(4 * q), gs.magic)];
+    if (panel + stride >= nPanels)
+      st.bufNext = 0; // no next panel: the prefetch past the end re-reads this one
+  } else {
+    st.cur = A + row_of(panel < nPanels ? panel : 0) * K + 4 * q;
+  }
+  // with T >= SA the first SA - 1 steps are all inside the first panel
+  st.wrap = 0;
+#pragma unroll
+  for (int s = 0; s < SA - 1; ++s)
+    pipe.a[s] = *reinterpret_cast<const float4 *>(addr(s));
+  // this workgroup's columns of W into LDS
+  {
+    const int perRow = NW / 4;
+    const int chunks = K * perRow;
+    constexpr int U = 12; // loads in flight per lane
+    for (int base = tid; base < chunks; base += 512 * U) {
+      float4 w[U];
+      int dst[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        // past the end: the last chunk again (same value to the same place)
+        int x = base + 512 * u;
+        x = x < chunks ? x : chunks - 1;
+        const int k = x / perRow, nc = x - k * perRow;
+        dst[u] = k * PITCH + 4 * nc;
+        w[u] = *reinterpret_cast<const float4 *>(W + (long long)k * N + n0 + 4 * nc);
+      }
+      // all loads in flight before the first store (left alone the compiler
+      // sinks each load to its store and waits for them one by one)
+#define SCN_PIN4(v) "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w)
+      asm volatile("" : SCN_PIN4(w[0]), SCN_PIN4(w[1]), SCN_PIN4(w[2]),
+                        SCN_PIN4(w[3]), SCN_PIN4(w[4]), SCN_PIN4(w[5]));
+      asm volatile("" : SCN_PIN4(w[6]), SCN_PIN4(w[7]), SCN_PIN4(w[8]),
+                        SCN_PIN4(w[9]), SCN_PIN4(w[10]), SCN_PIN4(w[11]));
+#undef SCN_PIN4
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        *reinterpret_cast<float4 *>(&sW[dst[u]]) = w[u];
+    }
+  }
+  __syncthreads();
+
+  const float *wl = sW + 4 * q * PITCH + c;
+  pipe.read_w(wl, 0, 0);
+  ColEpilogue col[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+    col[j] = load_col(ep, n0 + ROWS * j + c);
+
+  // aim: set up the prefetch that runs past this panel's end into the next
+  auto aim = [&]() {
+    const long long next = panel + stride;
+    if (GATHER) {
+      // rr holds the next panel's rules (fetched a panel ago): into the
+      // buffer the previous panel has finished with; then fetch the ones after
+      if (next < nPanels)
+        keep_rules(st.bufNext);
+      fetch_rules(next + stride);
+    } else {
+      // past the last panel the prefetch re-reads this panel's first steps
+      st.nxt = next < nPanels ? A + row_of(next) * K + 4 * q : st.cur;
+      st.wrap = (st.nxt - st.cur) - (long long)KS * T;
+    }
+    pipe.clear();
+  };
+  auto advance = [&]() {
+    panel += stride;
+    if (GATHER) {
+      const int b = st.bufCur;
+      st.bufCur = st.bufNext;
+      st.bufNext = panel + stride < nPanels ? b : st.bufCur;
+    } else {
+      st.cur = st.nxt;
+    }
+  };
+  float *const obase = out + (long long)(4 * q) * N + n0 + c;
+
+  if (panel < nFull) { // first panel: entered with only loads in flight
+    aim();
+    for (int t0 = 0; t0 < T; t0 += SA)
+      pipe.group(t0, T, addr, wl);
+    pipe.template store<false>(obase + panel * ROWS * N, N, ROWS, q, col);
+    advance();
+    while (panel < nFull) { // entered with the previous panel's stores in flight
+      aim();
+      pipe.group(0, T, addr, wl);
+      for (int t0 = SA; t0 < T; t0 += SA)
+        pipe.group(t0, T, addr, wl);
+      pipe.template store<false>(obase + panel * ROWS * N, N, ROWS, q, col);
+      advance();
+    }
+  }
+  if (panel < nPanels) { // the ragged last panel
+    aim();
+    for (int t0 = 0; t0 < T; t0 += SA)
+      pipe.group(t0, T, addr, wl);
+    pipe.template store<true>(obase + panel * ROWS * N, N, M - panel * ROWS, q, col);
+  }
+}
+
+// T = K / KS must be a multiple of SA (the prefetch ring wraps at panel ends)
+#define WRES_LDS_BYTES (160 * 1024)
+// LDS the gathering variant adds: 8 wavefronts x 2 buffers x 16 rows x fs rules
+#define WRES_RULE_BYTES(fs) (8 * 2 * 16 * (fs) * 4)
+template <int NT, int SA>
+static int launch_wres(scn_ctx *ctx, const float *A, const float *W, float *out,
+                       long long M, int K, int N, const Epilogue &ep,
+                       const GatherSource *gs) {
+  constexpr int ROWS = 16, NW = ROWS * NT;
+  const int nSplits = N / NW;
+  const size_t lds = (size_t)K * (NW + 4) * sizeof(float) +
+                     (gs ? WRES_RULE_BYTES(gs->fs) : 0);
+  long long wgs = scn_ceil_div(scn_ceil_div(M, ROWS), 8);
+  const long long cap = (long long)ctx->numCU * (lds * 2 <= WRES_LDS_BYTES ? 2 : 1);
+  if (wgs > cap)
+    wgs = cap;
+  static bool configured = false; // one pair of attribute calls per instantiation
+  if (!configured) {
+    SCN_HIP_CHECK(hipFuncSetAttribute(
+        reinterpret_cast<const void *>(k_nin_wres<ROWS, NT, SA, false>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, WRES_LDS_BYTES));
+    SCN_HIP_CHECK(hipFuncSetAttribute(
+        reinterpret_cast<const void *>(k_nin_wres<ROWS, NT, SA, true>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, WRES_LDS_BYTES));
+    configured = true;
+  }
+  const dim3 grid((unsigned)(wgs * nSplits));
+  if (gs)
+    hipLaunchKernelGGL((k_nin_wres<ROWS, NT, SA, true>), grid, dim3(512), lds,
+                       ctx->stream, A, W, out, M, K, N, ep, *gs, nSplits);
+  else
+    hipLaunchKernelGGL((k_nin_wres<ROWS, NT, SA, false>), grid, dim3(512), lds,
+                       ctx->stream, A, W, out, M, K, N, ep, GatherSource(),
+                       nSplits);
+  return SCN_OK;
+}
+
+// Picks the column width of the W slices and launches; false when the shape is
+// not one for this path (the tiled kernel takes it then).  The choice depends
+// on M, K, N only, so that a fused convolution and the gather + NiN pair it
+// replaces run the same arithmetic in the same order.
+static bool wres_forward(scn_ctx *ctx, const float *A, const float *W,
+                         float *out, long long M, int K, int N,
+                         const Epilogue &ep, const GatherSource *gs) {
+  if (K % 32 != 0 || N % 16 != 0)
+    return false; // 16 k per step, an even number of steps
+  const int sa = (K / 16) % 4 == 0 ? 4 : 2;
+  const long long panels = scn_ceil_div(M, 16);
+  // widest slice that fits LDS (with room for the rules of the widest filter)
+  // and still gives every SIMD a wavefront; else the narrowest
+  static const int widths[] = {6, 4, 3, 2, 1};
+  int nt = 0;
+  for (int w : widths) {
+    const int nw = 16 * w;
+    if (N % nw != 0 ||
+        (size_t)K * (nw + 4) * 4 + WRES_RULE_BYTES(GF_MAX_FS) > WRES_LDS_BYTES)
+      continue;
+    nt = w;
+    if (panels * (N / nw) >= 1024)
+      break;
+  }
+  if (nt == 0)
+    return false;
+  // every slice re-reads A: fine while that stays in the caches
+  const int nSplits = N / (16 * nt);
+  if (nSplits > 1 && (double)M * K * 4 * nSplits > 64e6)
+    return false;
+#define SCN_WRES_CASE(T)                                                       \
+  case T:                                                                      \
+    return (sa == 4 ? launch_wres<T, 4>(ctx, A, W, out, M, K, N, ep, gs)       \
+                    : launch_wres<T, 2>(ctx, A, W, out, M, K, N, ep, gs)) ==   \
+           SCN_OK;
+  switch (nt) {
+    SCN_WRES_CASE(1)
+    SCN_WRES_CASE(2)
+    SCN_WRES_CASE(3)
+    SCN_WRES_CASE(4)
+    SCN_WRES_CASE(6)
+  }
+#undef SCN_WRES_CASE
+  return false;
 }
 
 // ---- MFMA path with bf16 operands: v_mfma_f32_32x32x16_bf16 ----------------
@@ -513,6 +905,8 @@ static int nin_forward(scn_ctx *ctx, const float *d_A, const float *d_W,
       launch_mfma_bf16<4, 1, 2>(ctx, d_A, d_W, d_out, M, K, N, ep, split);
     else
       launch_mfma_bf16<1, 4, 1>(ctx, d_A, d_W, d_out, M, K, N, ep, split);
+  } else if (vec && wres_forward(ctx, d_A, d_W, d_out, M, K, N, ep, gs)) {
+    // W-resident kernel took it
   } else if ((vec && K >= 8) || gs) {
     // Tall tiles (128 rows), 64 columns wide, or 96 where that divides N
     // (measured on 12928 x 1280 x 480: 93 TFLOP/s against 73 with 64-column
@@ -557,7 +951,8 @@ extern "C" int scn_nin_forward(scn_ctx *ctx, const float *d_A,
 }
 
 extern "C" int scn_conv_nin_supported(int fs, int nIn, int N) {
-  return fs >= 1 && fs <= GF_MAX_FS && nIn >= 4 && nIn % 4 == 0 && N % 4 == 0;
+  return fs >= 1 && fs <= GF_MAX_FS && nIn >= 4 && nIn % 4 == 0 &&
+         nIn <= SCN_ZERO_FLOATS && N % 4 == 0;
 }
 
 extern "C" int scn_conv_nin_forward(scn_ctx *ctx, const float *d_in,
@@ -565,6 +960,7 @@ extern "C" int scn_conv_nin_forward(scn_ctx *ctx, const float *d_in,
                                     const float *d_W, const float *d_B,
                                     const float *d_prelu, float *d_out,
                                     int64_t M, int N, float p, int act) {
+  SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_conv_nin_forward: null context");
   SCN_REQUIRE(scn_conv_nin_supported(fs, nIn, N), SCN_ERR_ARG,
               "scn_conv_nin_forward: fs %d nIn %d N %d is outside the fused "
               "kernel's range (fs <= %d, nIn and N multiples of 4)",
@@ -577,6 +973,8 @@ extern "C" int scn_conv_nin_forward(scn_ctx *ctx, const float *d_in,
   gs.rules = d_rules;
   gs.fs = fs;
   gs.nIn = nIn;
+  gs.magic = (unsigned)((1ull << 32) / (unsigned)nIn + 1);
+  gs.zeros = ctx->d_zeros;
   return nin_forward(ctx, d_in, d_W, d_B, d_prelu, d_out, M, fs * nIn, N, p,
                      act, SCN_FP32, &gs);
 }
