@@ -74,6 +74,21 @@ int scn_malloc(scn_ctx *ctx, size_t bytes, void **d_ptr);
 int scn_free(scn_ctx *ctx, void *d_ptr);
 int scn_h2d(scn_ctx *ctx, void *d_dst, const void *h_src, size_t bytes);
 int scn_d2h(scn_ctx *ctx, void *h_dst, const void *d_src, size_t bytes);
+/* The asynchronous half of the same interface (vectorCUDA<T>::copyToCPUAsync,
+ * vectorCUDA.cu:110-127, followed by cudaStreamSynchronize in
+ * SoftmaxClassifier.cu:24-27): pinned host memory, a copy that is only queued
+ * on the context's stream, and an event to wait for it while later work is
+ * already queued behind it. */
+typedef struct scn_event scn_event;
+int scn_host_alloc(scn_ctx *ctx, size_t bytes, void **h_ptr);
+int scn_host_free(scn_ctx *ctx, void *h_ptr);
+int scn_d2h_async(scn_ctx *ctx, void *h_pinned_dst, const void *d_src, size_t bytes);
+int scn_event_create(scn_ctx *ctx, scn_event **event);
+int scn_event_destroy(scn_event *event);
+/* marks the point the stream has reached */
+int scn_event_record(scn_ctx *ctx, scn_event *event);
+/* blocks the calling thread until the stream has passed the recorded point */
+int scn_event_wait(scn_event *event);
 /* device-to-device, asynchronous on the context's stream */
 int scn_d2d(scn_ctx *ctx, void *d_dst, const void *d_src, size_t bytes);
 int scn_fill32(scn_ctx *ctx, void *d_dst, uint32_t word, size_t nWords);

@@ -67,6 +67,13 @@ def lib():
         "scn_free": (C.c_int, [vp, vp]),
         "scn_h2d": (C.c_int, [vp, vp, vp, sz]),
         "scn_d2h": (C.c_int, [vp, vp, vp, sz]),
+        "scn_host_alloc": (C.c_int, [vp, sz, C.POINTER(vp)]),
+        "scn_host_free": (C.c_int, [vp, vp]),
+        "scn_d2h_async": (C.c_int, [vp, vp, vp, sz]),
+        "scn_event_create": (C.c_int, [vp, C.POINTER(vp)]),
+        "scn_event_destroy": (C.c_int, [vp]),
+        "scn_event_record": (C.c_int, [vp, vp]),
+        "scn_event_wait": (C.c_int, [vp]),
         "scn_d2d": (C.c_int, [vp, vp, vp, sz]),
         "scn_fill32": (C.c_int, [vp, vp, C.c_uint32, sz]),
         "scn_grids_create": (C.c_int, [vp, P(vp)]),

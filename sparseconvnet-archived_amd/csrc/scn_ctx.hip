@@ -107,6 +107,64 @@ extern "C" int scn_d2h(scn_ctx *c, void *h_dst, const void *d_src,
   return SCN_OK;
 }
 
+struct scn_event {
+  hipEvent_t ev;
+};
+extern "C" int scn_host_alloc(scn_ctx *c, size_t bytes, void **h_ptr) {
+  SCN_REQUIRE(c && h_ptr, SCN_ERR_ARG, "scn_host_alloc: null argument");
+  *h_ptr = nullptr;
+  if (bytes == 0)
+    return SCN_OK;
+  SCN_HIP_CHECK(hipSetDevice(c->device));
+  SCN_HIP_CHECK(hipHostMalloc(h_ptr, bytes, hipHostMallocDefault));
+  return SCN_OK;
+}
+extern "C" int scn_host_free(scn_ctx *c, void *h_ptr) {
+  (void)c;
+  if (h_ptr)
+    SCN_HIP_CHECK(hipHostFree(h_ptr));
+  return SCN_OK;
+}
+extern "C" int scn_d2h_async(scn_ctx *c, void *h_dst, const void *d_src,
+                             size_t bytes) {
+  SCN_REQUIRE(c, SCN_ERR_ARG, "scn_d2h_async: null context");
+  if (bytes == 0)
+    return SCN_OK;
+  SCN_REQUIRE(h_dst && d_src, SCN_ERR_ARG, "scn_d2h_async: null buffer");
+  SCN_HIP_CHECK(
+      hipMemcpyAsync(h_dst, d_src, bytes, hipMemcpyDeviceToHost, c->stream));
+  return SCN_OK;
+}
+extern "C" int scn_event_create(scn_ctx *c, scn_event **event) {
+  SCN_REQUIRE(c && event, SCN_ERR_ARG, "scn_event_create: null argument");
+  SCN_HIP_CHECK(hipSetDevice(c->device));
+  scn_event *e = new scn_event;
+  hipError_t rc = hipEventCreateWithFlags(&e->ev, hipEventDisableTiming);
+  if (rc != hipSuccess) {
+    delete e;
+    SCN_HIP_CHECK(rc);
+  }
+  *event = e;
+  return SCN_OK;
+}
+extern "C" int scn_event_destroy(scn_event *event) {
+  if (event) {
+    (void)hipEventDestroy(event->ev);
+    delete event;
+  }
+  return SCN_OK;
+}
+extern "C" int scn_event_record(scn_ctx *c, scn_event *event) {
+  SCN_REQUIRE(c && event, SCN_ERR_ARG, "scn_event_record: null argument");
+  SCN_HIP_CHECK(hipEventRecord(event->ev, c->stream));
+  return SCN_OK;
+}
+extern "C" int scn_event_wait(scn_event *event) {
+  SCN_REQUIRE(event, SCN_ERR_ARG, "scn_event_wait: null event");
+  SCN_HIP_CHECK(hipEventSynchronize(event->ev));
+  return SCN_OK;
+}
+
 extern "C" int scn_d2d(scn_ctx *c, void *d_dst, const void *d_src,
                        size_t bytes) {
   if (bytes == 0)

@@ -29,6 +29,10 @@ public:
   BatchProducer(SparseConvNetCUDA &cnn, const ResidentBatch &resident,
                 int nBatches);
   ~BatchProducer();
+  // nextBatch() hands the slot of the batch it returned keepAlive + 1 calls
+  // ago back to the workers: 0 is the reference's behaviour; 1 lets the caller
+  // still read batch i after asking for batch i + 1 (needs >= 2 slots).
+  int keepAlive = 0;
   SpatiallySparseBatch *nextBatch();
   void batchProducerThread(int nThread);
   // CPU half: fills slot cc with batch c (codify only)

@@ -54,6 +54,9 @@ public:
                     int pciBusID = -1, int nTop = 1,
                     int nBatchProducerThreads = 10);
   ~SparseConvNetCUDA();
+  void forwardBatch(SpatiallySparseBatch &batch);
+  void finishBatch(SpatiallySparseBatch &batch, std::ofstream &f,
+                   std::ofstream &g);
   void processBatch(SpatiallySparseBatch &batch, float learningRate,
                     float momentum, std::ofstream &f, std::ofstream &g);
   void addLearntLayer(int nFeatures, ActivationFunction activationFn = RELU,

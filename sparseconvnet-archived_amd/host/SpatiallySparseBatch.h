@@ -1,9 +1,24 @@
 // One batch travelling through the net (SpatiallySparseBatch.h:7-22).
 #pragma once
+#include <memory>
 #include <vector>
 #include "SpatiallySparseBatchInterface.h"
 #include "types.h"
 #include "vectorCUDA.h"
+
+// Where a batch's class probabilities land: pinned host memory filled by a
+// copy queued behind the batch's forward pass, and the event that says it has
+// arrived.  Lets the caller queue the next batch before reading this one.
+struct BatchResultStage {
+  float *pinned;
+  size_t capacity; // floats
+  scn_event *arrived;
+  bool pending;
+  BatchResultStage();
+  ~BatchResultStage();
+  BatchResultStage(const BatchResultStage &) = delete;
+  BatchResultStage &operator=(const BatchResultStage &) = delete;
+};
 
 class SpatiallySparseBatch {
   SpatiallySparseBatchSubInterface *inputSub;
@@ -26,5 +41,6 @@ public:
   // device staging of the input sites (sample, key as two ints, row,
   // backgroundCol), reused from batch to batch
   vectorCUDA<int> stagingSample, stagingKey, stagingRow, stagingBackground;
+  std::unique_ptr<BatchResultStage> result;
   void reset();
 };

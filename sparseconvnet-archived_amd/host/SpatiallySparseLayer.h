@@ -216,6 +216,12 @@ public:
 void SoftmaxClassifier(SpatiallySparseBatchInterface &input,
                        SpatiallySparseBatch &batch, int nTop,
                        cudaMemStream &memStream);
+// its two halves: queue the copy of the probabilities; wait for it and count
+void SoftmaxClassifierLaunch(SpatiallySparseBatchInterface &input,
+                             SpatiallySparseBatch &batch,
+                             cudaMemStream &memStream);
+void SoftmaxClassifierCollect(SpatiallySparseBatchInterface &input,
+                              SpatiallySparseBatch &batch, int nTop);
 
 // utilities.h
 int ipow(int base, int exp);

@@ -327,11 +327,20 @@ void SpatiallySparseBatchInterface::summary() {
             << sub->features.size() << " rules " << rules.size() << std::endl;
 }
 
+BatchResultStage::BatchResultStage()
+    : pinned(nullptr), capacity(0), arrived(nullptr), pending(false) {}
+BatchResultStage::~BatchResultStage() {
+  if (arrived)
+    scn_event_destroy(arrived);
+  if (pinned)
+    scn_host_free(scnDefaultContext(), pinned);
+}
+
 SpatiallySparseBatch::SpatiallySparseBatch(
     SpatiallySparseBatchSubInterface *inputSub)
     : inputSub(inputSub), preprocessStream(nullptr), labels(false, 0),
       stagingSample(true, 0), stagingKey(true, 0), stagingRow(true, 0),
-      stagingBackground(true, 0) {
+      stagingBackground(true, 0), result(new BatchResultStage()) {
   interfaces.emplace_back(inputSub);
   reset();
 }

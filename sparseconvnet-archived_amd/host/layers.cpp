@@ -534,22 +534,45 @@ int TerminalPoolingLayer::calculateInputSpatialSize(int outputSpatialSize) {
 }
 
 // ---- SoftmaxClassifier (SoftmaxClassifier.cu:16-58) ---------------------------
-void SoftmaxClassifier(SpatiallySparseBatchInterface &input,
-                       SpatiallySparseBatch &batch, int nTop,
-                       cudaMemStream &memStream) {
+// In two halves, so that a caller may queue the next batch's forward pass
+// between them: the copy of the probabilities to the host is only queued
+// (SoftmaxClassifier.cu:24, copyToCPUAsync), the statistics are computed once
+// it has arrived (:27 onwards).
+void SoftmaxClassifierLaunch(SpatiallySparseBatchInterface &input,
+                             SpatiallySparseBatch &batch,
+                             cudaMemStream &memStream) {
   assert(batch.batchSize == input.nSpatialSites);
   assert(input.nFeatures == (int)input.featuresPresent.size());
   if (batch.type == TRAINBATCH)
     unsupported("a TRAINBATCH (dropout and the backward pass)");
+  BatchResultStage &r = *batch.result;
+  const size_t n = (size_t)batch.batchSize * input.nFeatures;
+  if (n > r.capacity) {
+    if (r.pinned)
+      SCN_CHECKED(scn_host_free(memStream.ctx, r.pinned));
+    r.capacity = n + n / 2;
+    SCN_CHECKED(scn_host_alloc(memStream.ctx, r.capacity * sizeof(float),
+                               (void **)&r.pinned));
+  }
+  if (!r.arrived)
+    SCN_CHECKED(scn_event_create(memStream.ctx, &r.arrived));
+  SCN_CHECKED(scn_d2h_async(memStream.ctx, r.pinned, input.sub->features.dPtr(),
+                            n * sizeof(float)));
+  SCN_CHECKED(scn_event_record(memStream.ctx, r.arrived));
+  r.pending = true;
+}
+void SoftmaxClassifierCollect(SpatiallySparseBatchInterface &input,
+                              SpatiallySparseBatch &batch, int nTop) {
+  BatchResultStage &r = *batch.result;
+  if (!r.pending)
+    return;
+  SCN_CHECKED(scn_event_wait(r.arrived));
+  r.pending = false;
   const int nClasses = input.nFeatures;
-  std::vector<float> probs((size_t)batch.batchSize * nClasses);
-  SCN_CHECKED(scn_d2h(memStream.ctx, probs.data(),
-                      input.sub->features.dPtr(),
-                      probs.size() * sizeof(float)));
+  const float *probs = r.pinned;
   for (int i = 0; i < batch.batchSize; ++i)
     batch.probabilities.push_back(std::vector<float>(
-        probs.begin() + (size_t)i * nClasses,
-        probs.begin() + (size_t)(i + 1) * nClasses));
+        probs + (size_t)i * nClasses, probs + (size_t)(i + 1) * nClasses));
   for (int i = 0; i < batch.batchSize; i++)
     batch.predictions.push_back(vectorTopIndices(batch.probabilities[i], nTop));
   if (batch.type != UNLABELEDBATCH) {
@@ -563,4 +586,10 @@ void SoftmaxClassifier(SpatiallySparseBatchInterface &input,
           batch.mistakes--;
     }
   }
+}
+void SoftmaxClassifier(SpatiallySparseBatchInterface &input,
+                       SpatiallySparseBatch &batch, int nTop,
+                       cudaMemStream &memStream) {
+  SoftmaxClassifierLaunch(input, batch, memStream);
+  SoftmaxClassifierCollect(input, batch, nTop);
 }

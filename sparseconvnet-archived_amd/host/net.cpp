@@ -225,12 +225,25 @@ void SparseConvNetCUDA::processBatch(SpatiallySparseBatch &batch,
                                      std::ofstream &f, std::ofstream &g) {
   (void)learningRate;
   (void)momentum;
+  forwardBatch(batch);
+  finishBatch(batch, f, g);
+}
+// The two halves of processBatch.  forwardBatch only queues work on the net's
+// stream (every layer, then the copy of the probabilities to the host);
+// finishBatch waits for that copy and does the host-side statistics.  The
+// dataset loops queue batch i + 1 before finishing batch i, so the stream never
+// runs dry while the host is busy.
+void SparseConvNetCUDA::forwardBatch(SpatiallySparseBatch &batch) {
   for (size_t i = 0; i < layers.size(); i++) {
     batch.interfaces[i + 1].sub->reset();
     scn_prof_tag(memStream.ctx, (int)i);
     layers[i]->forwards(batch, batch.interfaces[i], batch.interfaces[i + 1]);
   }
-  SoftmaxClassifier(batch.interfaces.back(), batch, nTop, memStream);
+  SoftmaxClassifierLaunch(batch.interfaces.back(), batch, memStream);
+}
+void SparseConvNetCUDA::finishBatch(SpatiallySparseBatch &batch,
+                                    std::ofstream &f, std::ofstream &g) {
+  SoftmaxClassifierCollect(batch.interfaces.back(), batch, nTop);
   if (f.is_open())
     for (auto &p : batch.predictions) {
       for (size_t k = 0; k < p.size(); k++)
@@ -272,11 +285,27 @@ float SparseConvNetCUDA::processDataset(SpatiallySparseDataset &dataset,
     f.open("unlabelledData.predictions");
     g.open("unlabelledData.probabilities");
   }
-  while (SpatiallySparseBatch *batch = bp.nextBatch()) {
-    processBatch(*batch, learningRate, momentum, f, g);
+  (void)learningRate;
+  (void)momentum;
+  bp.keepAlive = nBatchProducerThreads >= 2 ? 1 : 0;
+  SpatiallySparseBatch *queued = nullptr; // forward pass queued, not yet read
+  auto finish = [&](SpatiallySparseBatch *batch) {
+    finishBatch(*batch, f, g);
     errorRate += batch->mistakes * 1.0 / dataset.pictures.size();
     nll += batch->negativeLogLikelihood * 1.0 / dataset.pictures.size();
+  };
+  while (SpatiallySparseBatch *batch = bp.nextBatch()) {
+    forwardBatch(*batch);
+    if (queued)
+      finish(queued);
+    queued = batch;
+    if (!bp.keepAlive) {
+      finish(queued);
+      queued = nullptr;
+    }
   }
+  if (queued)
+    finish(queued);
   auto end = std::chrono::system_clock::now();
   auto diff =
       std::chrono::duration_cast<std::chrono::nanoseconds>(end - start).count();
@@ -301,16 +330,30 @@ void SparseConvNetCUDA::processDatasetRepeatTest(
   for (int rep = 1; rep <= nReps; ++rep) {
     {
       BatchProducer bp(*this, dataset, inputSpatialSize, batchSize);
-      while (SpatiallySparseBatch *batch = bp.nextBatch()) {
+      bp.keepAlive = nBatchProducerThreads >= 2 ? 1 : 0;
+      SpatiallySparseBatch *queued = nullptr;
+      auto finish = [&](SpatiallySparseBatch *batch) {
         std::ofstream f, g;
-        processBatch(*batch, 0, 0, f, g);
+        finishBatch(*batch, f, g);
         for (int i = 0; i < batch->batchSize; ++i) {
           int ii = batch->sampleNumbers[i];
           votes[ii][batch->predictions[i][0]]++;
           for (int j = 0; j < dataset.nClasses; ++j)
             probs[ii][j] += batch->probabilities[i][j];
         }
+      };
+      while (SpatiallySparseBatch *batch = bp.nextBatch()) {
+        forwardBatch(*batch);
+        if (queued)
+          finish(queued);
+        queued = batch;
+        if (!bp.keepAlive) {
+          finish(queued);
+          queued = nullptr;
+        }
       }
+      if (queued)
+        finish(queued);
     }
     int errors = (int)nPictures;
     float nll = 0;
@@ -532,8 +575,8 @@ void BatchProducer::batchProducerThread(int nThread) {
   }
 }
 SpatiallySparseBatch *BatchProducer::nextBatch() {
-  if (batchCounter >= 0) { // hand the previous slot back to its worker
-    int cc = batchCounter % cnn.nBatchProducerThreads;
+  if (batchCounter - keepAlive >= 0) { // hand a finished slot back to its worker
+    int cc = (batchCounter - keepAlive) % cnn.nBatchProducerThreads;
     cnn.batchPool[cc].batchSize = 0;
     {
       std::lock_guard<std::mutex> lock(slotMutex);

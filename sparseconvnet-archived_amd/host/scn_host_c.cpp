@@ -325,15 +325,35 @@ int scnh_forward_resident_stream(scnh_net *net, int nBatches, int batch,
   ResidentBatch r = resident_of(batch, d_sample, d_key, d_row, d_background,
                                 nActive, nSpatialSites, d_features);
   BatchProducer bp(*cnn, r, nBatches);
+  bp.keepAlive = cnn->nBatchProducerThreads >= 2 ? 1 : 0;
   int done = 0;
-  while (SpatiallySparseBatch *b = bp.nextBatch()) {
-    net->batch = b;
-    forward_layers(net, *b);
-    if (net->hasClassifier && h_probs)
-      scnh_batch_probabilities(net, h_probs);
-    cnn->memStream.synchronize();
+  SpatiallySparseBatch *queued = nullptr; // forward pass queued, not yet read
+  auto finish = [&](SpatiallySparseBatch *b) {
+    if (net->hasClassifier) {
+      std::ofstream f, g;
+      cnn->finishBatch(*b, f, g);
+      net->batch = b;
+      if (h_probs)
+        scnh_batch_probabilities(net, h_probs);
+    }
     ++done;
+  };
+  while (SpatiallySparseBatch *b = bp.nextBatch()) {
+    if (net->hasClassifier)
+      cnn->forwardBatch(*b);
+    else
+      forward_layers(net, *b);
+    if (queued)
+      finish(queued);
+    queued = b;
+    if (!bp.keepAlive) {
+      finish(queued);
+      queued = nullptr;
+    }
   }
+  if (queued)
+    finish(queued);
+  cnn->memStream.synchronize();
   net->batch = nullptr;
   return done;
 }
