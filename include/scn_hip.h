@@ -211,7 +211,8 @@ enum {
   SCN_K_TERMINAL = 5,
   SCN_K_SOFTMAX = 6,
   SCN_K_CONV_NIN = 7, /* gather fused into the NiN contraction */
-  SCN_K_COUNT = 8
+  SCN_K_PROBE = 8,    /* scn_prof_probe: what a span costs by itself */
+  SCN_K_COUNT = 9
 };
 int scn_prof_enable(scn_ctx *ctx, int on);
 /* label attached to the spans recorded from now on (e.g. the layer index) */
@@ -222,6 +223,10 @@ int scn_prof_tag(scn_ctx *ctx, int tag);
 int scn_prof_spans(scn_ctx *ctx, int capacity, int32_t *family, int32_t *tag,
                    double *ms, int32_t *n);
 int scn_prof_reset(scn_ctx *ctx);
+/* Records one span of family SCN_K_PROBE around nothing (with_kernel == 0) or
+ * around a kernel of one wavefront that does nothing (with_kernel != 0): the
+ * floor under every other span, for callers that want to subtract it. */
+int scn_prof_probe(scn_ctx *ctx, int with_kernel);
 /* synchronises, then returns accumulated milliseconds and number of calls */
 int scn_prof_read(scn_ctx *ctx, int family, double *ms, int64_t *calls);
 

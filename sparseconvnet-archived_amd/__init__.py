@@ -19,8 +19,8 @@ HEADER = os.path.join(ROOT, "include", "scn_hip.h")
 # ActivationFunction (reference types.h:11-20)
 NOSIGMOID, RELU, VLEAKYRELU, LEAKYRELU, TANH, SOFTMAX, PRELU, SIGMOID = range(8)
 FP32, BF16, BF16X3 = 0, 1, 2
-K_GRID_BUILD, K_RULES, K_GATHER, K_NIN, K_MAXPOOL, K_TERMINAL, K_SOFTMAX, K_CONV_NIN = range(8)
-KERNEL_FAMILIES = ["grid_build", "rules", "gather", "nin", "maxpool", "terminal", "softmax", "conv_nin"]
+K_GRID_BUILD, K_RULES, K_GATHER, K_NIN, K_MAXPOOL, K_TERMINAL, K_SOFTMAX, K_CONV_NIN, K_PROBE = range(9)
+KERNEL_FAMILIES = ["grid_build", "rules", "gather", "nin", "maxpool", "terminal", "softmax", "conv_nin", "probe"]
 
 
 class ScnError(RuntimeError):
@@ -96,6 +96,7 @@ def lib():
         "scn_softmax_rows": (C.c_int, [vp, vp, vp, i64, C.c_int]),
         "scn_prof_enable": (C.c_int, [vp, C.c_int]),
         "scn_prof_reset": (C.c_int, [vp]),
+        "scn_prof_probe": (C.c_int, [vp, C.c_int]),
         "scn_prof_tag": (C.c_int, [vp, C.c_int]),
         "scn_prof_spans": (C.c_int, [vp, C.c_int, vp, vp, vp, P(i32)]),
         "scn_prof_read": (C.c_int, [vp, C.c_int, P(C.c_double), P(i64)]),
@@ -187,6 +188,9 @@ class Context:
     # ---- profiling
     def prof_enable(self, on=True):
         _check(lib().scn_prof_enable(self.h, int(on)))
+
+    def prof_probe(self, with_kernel=True):
+        _check(lib().scn_prof_probe(self.h, int(with_kernel)))
 
     def prof_reset(self):
         _check(lib().scn_prof_reset(self.h))

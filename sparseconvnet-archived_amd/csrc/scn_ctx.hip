@@ -225,6 +225,17 @@ ProfScope::~ProfScope() {
     (void)hipEventRecord(ctx->spans[idx].b, ctx->stream);
 }
 
+__global__ void k_nothing() {}
+extern "C" int scn_prof_probe(scn_ctx *c, int with_kernel) {
+  SCN_REQUIRE(c, SCN_ERR_ARG, "scn_prof_probe: null context");
+  ProfScope prof(c, SCN_K_PROBE);
+  if (with_kernel) {
+    hipLaunchKernelGGL(k_nothing, dim3(1), dim3(64), 0, c->stream);
+    SCN_HIP_CHECK(hipGetLastError());
+  }
+  return SCN_OK;
+}
+
 static void drain_spans(scn_ctx *c, int capacity = 0, int32_t *family = nullptr,
                         int32_t *tag = nullptr, double *msOut = nullptr,
                         int32_t *n = nullptr) {

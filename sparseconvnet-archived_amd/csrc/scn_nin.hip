@@ -126,18 +126,6 @@ __global__ void __launch_bounds__(256)
   }
 }
 
-// ---- MFMA path: fp32 operands, v_mfma_f32_32x32x2_f32 ----------------------
-// Block = 4 wavefronts laid out WM x WN; every wavefront owns a 32 x (32 NT)
-// patch of the output as NT accumulator tiles of 32x32 (16 VGPRs per lane
-// each).  Operands are staged through LDS in k-slabs of MF_BK, double
-// buffered: A transposed to [k][row] (row stride odd, so both the transposing
-// stores and the operand reads hit every bank evenly), W as [k][col].  One
-// MFMA consumes k = 2: lane l supplies A[row = l % 32][k = l / 32] and
-// W[k = l / 32][col = l % 32]; accumulator register v of lane l is
-// D[row = 8 (v / 4) + 4 (l / 32) + v % 4][col = l % 32].
-#define MF_BK 32
-typedef float floatx16 __attribute__((ext_vector_type(16)));
-
 //
 // GATHER: A is never materialised.  Row m of A is the receptive field of
 // output site m, column q * nIn + c = channel c of input row
@@ -151,6 +139,19 @@ struct GatherSource {
   unsigned magic;     // floor(2^32 / nIn) + 1: k / nIn == mulhi(k, magic) for k nIn < 2^32
   const float *zeros; // at least nIn zeros: the row a negative rule stands for
 };
+
+
+// ---- MFMA path: fp32 operands, v_mfma_f32_32x32x2_f32 ----------------------
+// Block = 4 wavefronts laid out WM x WN; every wavefront owns a 32 x (32 NT)
+// patch of the output as NT accumulator tiles of 32x32 (16 VGPRs per lane
+// each).  Operands are staged through LDS in k-slabs of MF_BK, double
+// buffered: A transposed to [k][row] (row stride odd, so both the transposing
+// stores and the operand reads hit every bank evenly), W as [k][col].  One
+// MFMA consumes k = 2: lane l supplies A[row = l % 32][k = l / 32] and
+// W[k = l / 32][col = l % 32]; accumulator register v of lane l is
+// D[row = 8 (v / 4) + 4 (l / 32) + v % 4][col = l % 32].
+#define MF_BK 32
+typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 template <int WM, int WN, int NT, int BK, bool GATHER>
 __global__ void __launch_bounds__(256)

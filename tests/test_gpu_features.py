@@ -77,7 +77,9 @@ def test_softmax(scn, ctx):
 SHAPES = [(1000, 12, 32), (777, 128, 64), (513, 256, 96), (300, 384, 128), (129, 512, 160), (400, 160, 192),
           (100, 192, 100), (64, 288, 64), (5, 7, 3), (2000, 27, 32), (257, 1728, 64),
           # enough 16-row panels that wavefronts of the W-resident kernel walk several, last one ragged
-          (70001, 128, 64), (40003, 256, 96)]
+          (70001, 128, 64), (40003, 256, 96),
+          # W-resident kernel: an odd number of prefetch groups, a 48-column slice, many narrow slices
+          (600, 160, 192), (1000, 64, 48), (2469, 512, 160)]
 
 
 @pytest.mark.parametrize("M,K,N", SHAPES)
