@@ -429,13 +429,14 @@ __global__ void __launch_bounds__(1024)
 
 // small batches: prefix sum of the owned counts and the per-sample pass in
 // one launch
+template <int PER>
 __global__ void __launch_bounds__(1024)
     k_plan_scan_samples(GridView in, const unsigned *cnt, unsigned *base,
                         long long nEntries, long long fullSize, int *outBg,
                         int *bgBefore, unsigned *sampleStart,
                         long long *scalars, const long long *badSites) {
   __shared__ uint32_t ldsScan[17];
-  (void)block_scan_loop<false>(cnt, base, (size_t)nEntries, ldsScan);
+  (void)block_scan_loop<false, PER>(cnt, base, (size_t)nEntries, ldsScan);
   __syncthreads(); // the block's own writes to base[] are visible to it
   plan_samples_body(in, base, nEntries, fullSize, outBg, bgBefore, sampleStart,
                     scalars, badSites);
@@ -730,7 +731,7 @@ static int grids_prepare(scn_ctx *ctx, scn_grids *g, int batch, int d, int n,
   size_t cap = (size_t)1 << lg;
   g->nWords = (size_t)(((long long)batch * vol + 63) / 64);
   SCN_TRY(g->table.reserve(cap));
-  SCN_TRY(g->bits.reserve(g->nWords + 2));
+  SCN_TRY(g->bits.reserve(g->nWords + 8)); // the scan reads whole 32-byte groups
   SCN_TRY(g->prefix.reserve(g->nWords + 2));
   SCN_TRY(g->ekey.reserve((size_t)nActive + 1));
   SCN_TRY(g->erow.reserve((size_t)nActive + 1));
@@ -901,7 +902,7 @@ static int plan_regions_d(scn_ctx *ctx, scn_grids *in, scn_grids *out,
                           const Geom &g, long long fullSize,
                           int64_t *nOutSites) {
   const long long nE = in->nActive;
-  SCN_TRY(out->cnt.reserve((size_t)nE + 2));
+  SCN_TRY(out->cnt.reserve((size_t)nE + 8)); // the scan reads whole 16-byte groups
   SCN_TRY(out->base.reserve((size_t)nE + 2));
   SCN_TRY(out->bgBefore.reserve((size_t)in->batch + 2));
   SCN_TRY(out->sampleStart.reserve((size_t)in->batch + 2));
@@ -925,10 +926,16 @@ static int plan_regions_d(scn_ctx *ctx, scn_grids *in, scn_grids *out,
   }
   const long long *bad = (const long long *)(ctx->d_scalars + 15);
   if ((size_t)nE <= SCAN1_MAX_ELEMS) {
-    hipLaunchKernelGGL(k_plan_scan_samples, dim3(1), dim3(1024), 0, ctx->stream,
-                       vin, out->cnt.p, out->base.p, nE, fullSize, out->bg.p,
-                       out->bgBefore.p, out->sampleStart.p,
-                       (long long *)ctx->d_scalars, bad);
+    if ((size_t)nE <= SCAN1_SMALL_ELEMS)
+      hipLaunchKernelGGL((k_plan_scan_samples<32>), dim3(1), dim3(1024), 0,
+                         ctx->stream, vin, out->cnt.p, out->base.p, nE, fullSize,
+                         out->bg.p, out->bgBefore.p, out->sampleStart.p,
+                         (long long *)ctx->d_scalars, bad);
+    else
+      hipLaunchKernelGGL((k_plan_scan_samples<64>), dim3(1), dim3(1024), 0,
+                         ctx->stream, vin, out->cnt.p, out->base.p, nE, fullSize,
+                         out->bg.p, out->bgBefore.p, out->sampleStart.p,
+                         (long long *)ctx->d_scalars, bad);
   } else {
     SCN_TRY(scn_scan_exclusive_u32(ctx->stream, out->cnt.p, out->base.p,
                                    (size_t)nE, out->scanTmp.p));

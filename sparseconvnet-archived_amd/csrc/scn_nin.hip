@@ -395,12 +395,15 @@ template <int ROWS, int NT, int SA> struct WresPipe {
   }
 };
 
-template <int ROWS, int NT, int SA, bool GATHER>
+// GRU: 0 = A is a plain matrix; else A is gathered through the rules and GRU
+// is the number of 64-int loads that cover one panel's rules (16 fs <= 64 GRU)
+template <int ROWS, int NT, int SA, int GRU>
 __global__ void __launch_bounds__(512)
     k_nin_wres(const float *__restrict__ A, const float *__restrict__ W,
                float *__restrict__ out, long long M, int K, int N, Epilogue ep,
                GatherSource gs, int nSplits) {
   typedef WresPipe<ROWS, NT, SA> Pipe;
+  constexpr bool GATHER = GRU > 0;
   constexpr int KS = Pipe::KS, NW = Pipe::NW, PITCH = Pipe::PITCH;
   extern __shared__ __attribute__((aligned(16))) float sW[]; // [K][PITCH]
   const int tid = threadIdx.x;
@@ -445,7 +448,7 @@ __global__ void __launch_bounds__(512)
     return p;
   };
   // GATHER: the rules of panel pnl, 64 consecutive ints per load
-  constexpr int RU = GATHER ? (ROWS * GF_MAX_FS + 63) / 64 : 1;
+  constexpr int RU = GATHER ? GRU : 1;
   int rr[RU];
   auto fetch_rules = [&](long long pnl) {
     if (pnl >= nPanels)
@@ -464,11 +467,45 @@ __global__ void __launch_bounds__(512)
         sRw[buf + lane + 64 * u] = rr[u];
   };
 
+  // this workgroup's columns of W go to LDS in batches of U 16-byte loads per lane
+  const int perRow = NW / 4;
+  const int chunks = K * perRow;
+  constexpr int U = 12;
+  float4 w[U];
+  int dst[U];
+  auto w_load = [&](int base) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      // past the end: the last chunk again (same value to the same place)
+      int x = base + 512 * u;
+      x = x < chunks ? x : chunks - 1;
+      const int k = x / perRow, nc = x - k * perRow;
+      dst[u] = k * PITCH + 4 * nc;
+      w[u] = *reinterpret_cast<const float4 *>(W + (long long)k * N + n0 + 4 * nc);
+    }
+  };
+  auto w_store = [&]() {
+    // all of the batch's loads are in flight before the first store (left
+    // alone the compiler sinks each load to its store and waits one by one)
+#define SCN_PIN4(v) "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w)
+    asm volatile("" : SCN_PIN4(w[0]), SCN_PIN4(w[1]), SCN_PIN4(w[2]),
+                      SCN_PIN4(w[3]), SCN_PIN4(w[4]), SCN_PIN4(w[5]));
+    asm volatile("" : SCN_PIN4(w[6]), SCN_PIN4(w[7]), SCN_PIN4(w[8]),
+                      SCN_PIN4(w[9]), SCN_PIN4(w[10]), SCN_PIN4(w[11]));
+#undef SCN_PIN4
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      *reinterpret_cast<float4 *>(&sW[dst[u]]) = w[u];
+  };
+
+  // Prologue.  Order of issue = order of arrival: what is needed first goes
+  // first, and the first batch of W travels while the rules are put in place.
   Pipe pipe;
   if (GATHER) {
     st.bufCur = 0;
     st.bufNext = rulesPerPanel;
     fetch_rules(panel);
+    w_load(tid);
     keep_rules(0);
     fetch_rules(panel + stride);
     st.ch = 4 * q - (int)__umulhi((unsigned)(4 * q), gs.magic) * gs.nIn;
@@ -483,35 +520,12 @@ __global__ void __launch_bounds__(512)
 #pragma unroll
   for (int s = 0; s < SA - 1; ++s)
     pipe.a[s] = *reinterpret_cast<const float4 *>(addr(s));
-  // this workgroup's columns of W into LDS
-  {
-    const int perRow = NW / 4;
-    const int chunks = K * perRow;
-    constexpr int U = 12; // loads in flight per lane
-    for (int base = tid; base < chunks; base += 512 * U) {
-      float4 w[U];
-      int dst[U];
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        // past the end: the last chunk again (same value to the same place)
-        int x = base + 512 * u;
-        x = x < chunks ? x : chunks - 1;
-        const int k = x / perRow, nc = x - k * perRow;
-        dst[u] = k * PITCH + 4 * nc;
-        w[u] = *reinterpret_cast<const float4 *>(W + (long long)k * N + n0 + 4 * nc);
-      }
-      // all loads in flight before the first store (left alone the compiler
-      // sinks each load to its store and waits for them one by one)
-#define SCN_PIN4(v) "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w)
-      asm volatile("" : SCN_PIN4(w[0]), SCN_PIN4(w[1]), SCN_PIN4(w[2]),
-                        SCN_PIN4(w[3]), SCN_PIN4(w[4]), SCN_PIN4(w[5]));
-      asm volatile("" : SCN_PIN4(w[6]), SCN_PIN4(w[7]), SCN_PIN4(w[8]),
-                        SCN_PIN4(w[9]), SCN_PIN4(w[10]), SCN_PIN4(w[11]));
-#undef SCN_PIN4
-#pragma unroll
-      for (int u = 0; u < U; ++u)
-        *reinterpret_cast<float4 *>(&sW[dst[u]]) = w[u];
-    }
+  if (!GATHER)
+    w_load(tid);
+  w_store();
+  for (int base = tid + 512 * U; base < chunks; base += 512 * U) {
+    w_load(base);
+    w_store();
   }
   __syncthreads();
 
@@ -589,24 +603,29 @@ static int launch_wres(scn_ctx *ctx, const float *A, const float *W, float *out,
   const long long cap = (long long)ctx->numCU * (lds * 2 <= WRES_LDS_BYTES ? 2 : 1);
   if (wgs > cap)
     wgs = cap;
-  static bool configured = false; // one pair of attribute calls per instantiation
+  static bool configured = false; // one set of attribute calls per instantiation
   if (!configured) {
-    SCN_HIP_CHECK(hipFuncSetAttribute(
-        reinterpret_cast<const void *>(k_nin_wres<ROWS, NT, SA, false>),
-        hipFuncAttributeMaxDynamicSharedMemorySize, WRES_LDS_BYTES));
-    SCN_HIP_CHECK(hipFuncSetAttribute(
-        reinterpret_cast<const void *>(k_nin_wres<ROWS, NT, SA, true>),
-        hipFuncAttributeMaxDynamicSharedMemorySize, WRES_LDS_BYTES));
+#define SCN_WRES_LDS(G)                                                        \
+  SCN_HIP_CHECK(hipFuncSetAttribute(                                           \
+      reinterpret_cast<const void *>(k_nin_wres<ROWS, NT, SA, G>),             \
+      hipFuncAttributeMaxDynamicSharedMemorySize, WRES_LDS_BYTES));
+    SCN_WRES_LDS(0) SCN_WRES_LDS(1) SCN_WRES_LDS(3) SCN_WRES_LDS(7)
+#undef SCN_WRES_LDS
     configured = true;
   }
   const dim3 grid((unsigned)(wgs * nSplits));
-  if (gs)
-    hipLaunchKernelGGL((k_nin_wres<ROWS, NT, SA, true>), grid, dim3(512), lds,
-                       ctx->stream, A, W, out, M, K, N, ep, *gs, nSplits);
+#define SCN_WRES_GO(G, src)                                                    \
+  hipLaunchKernelGGL((k_nin_wres<ROWS, NT, SA, G>), grid, dim3(512), lds,      \
+                     ctx->stream, A, W, out, M, K, N, ep, src, nSplits)
+  if (!gs)
+    SCN_WRES_GO(0, GatherSource());
+  else if (gs->fs <= 4)
+    SCN_WRES_GO(1, *gs);
+  else if (gs->fs <= 12)
+    SCN_WRES_GO(3, *gs);
   else
-    hipLaunchKernelGGL((k_nin_wres<ROWS, NT, SA, false>), grid, dim3(512), lds,
-                       ctx->stream, A, W, out, M, K, N, ep, GatherSource(),
-                       nSplits);
+    SCN_WRES_GO(7, *gs);
+#undef SCN_WRES_GO
   return SCN_OK;
 }
 

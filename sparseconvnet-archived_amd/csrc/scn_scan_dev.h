@@ -1,68 +1,68 @@
 // Device-side exclusive prefix sum by ONE workgroup of 1024 lanes.  For arrays
-// up to about a hundred thousand elements this is one launch instead of the
-// three of the tiled scan, and launch count is what small batches pay for.
+// up to 65536 elements this is one launch instead of the three of the tiled
+// scan, and launch count is what small batches pay for.
 //
-// Every lane owns one contiguous chunk: it sums the chunk (all loads in flight
-// at once, no barrier in between), the 1024 chunk sums are scanned through
-// wavefront shuffles and 17 words of LDS, and the lane walks its chunk a
-// second time (served by the caches) to write the prefixes.
+// Every lane owns 32 (or 64) consecutive elements and keeps them in registers: all of
+// its loads are issued back to back (one memory latency, not one per load),
+// the 1024 lane sums are scanned through wavefront shuffles and 17 words of
+// LDS, and the prefixes are written from the registers.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
 #define SCAN1_THREADS 1024
-#define SCAN1_MAX_ELEMS (SCAN1_THREADS * 32) // above this one compute unit's bandwidth loses to the three-launch tiled scan
+// elements per lane: 32, or 64 for arrays of up to 65536 elements (64 value
+// registers per lane, which a 1024-lane workgroup can still afford)
+#define SCAN1_SMALL_ELEMS (SCAN1_THREADS * 32)
+#define SCAN1_MAX_ELEMS (SCAN1_THREADS * 64)
 
+// Four consecutive elements starting at i (i % 4 == 0); elements at or past n
+// read as zero.  The loads are unconditional: a group that starts past the end
+// reads group 0 instead, and the group that straddles n reads up to 12 bytes
+// (24 for 64-bit words) past it -- inside the same aligned 16 / 32 bytes, so
+// which the caller must have allocated (in must be 16-byte aligned).
 template <bool POPC>
-__device__ __forceinline__ uint32_t scan1_load(const void *in, size_t i) {
-  if (POPC)
-    return (uint32_t)__popcll(((const unsigned long long *)in)[i]);
-  return ((const uint32_t *)in)[i];
-}
-
-// four consecutive elements starting at i (i % 4 == 0); elements at or past n
-// read as zero
-template <bool POPC>
-__device__ __forceinline__ uint4 scan1_load4(const void *in, size_t i,
-                                             size_t n) {
-  uint4 v = make_uint4(0u, 0u, 0u, 0u);
-  if (i + 4 <= n) {
-    if (POPC) {
-      const ulonglong2 *p =
-          reinterpret_cast<const ulonglong2 *>((const unsigned long long *)in + i);
-      ulonglong2 a = p[0], b = p[1];
-      v = make_uint4(__popcll(a.x), __popcll(a.y), __popcll(b.x), __popcll(b.y));
-    } else {
-      v = *reinterpret_cast<const uint4 *>((const uint32_t *)in + i);
-    }
+__device__ __forceinline__ uint4 scan1_load4(const void *in, size_t i, size_t n) {
+  const size_t at = i < n ? i : 0;
+  uint4 v;
+  if (POPC) {
+    const ulonglong2 *p =
+        reinterpret_cast<const ulonglong2 *>((const unsigned long long *)in + at);
+    const ulonglong2 a = p[0], b = p[1];
+    v = make_uint4(__popcll(a.x), __popcll(a.y), __popcll(b.x), __popcll(b.y));
   } else {
-    if (i < n)
-      v.x = scan1_load<POPC>(in, i);
-    if (i + 1 < n)
-      v.y = scan1_load<POPC>(in, i + 1);
-    if (i + 2 < n)
-      v.z = scan1_load<POPC>(in, i + 2);
+    v = *reinterpret_cast<const uint4 *>((const uint32_t *)in + at);
   }
+  v.x = i < n ? v.x : 0u;
+  v.y = i + 1 < n ? v.y : 0u;
+  v.z = i + 2 < n ? v.z : 0u;
+  v.w = i + 3 < n ? v.w : 0u;
   return v;
 }
 
-// out[i] = sum of in[0..i), out[n] = total.  Must be called by all 1024 lanes
-// of a workgroup; lds needs 17 words; in and out 16-byte aligned.  Returns the
-// total to every lane.
-template <bool POPC>
+// out[i] = sum of in[0..i), out[n] = total, n <= 1024 SCAN1_PER_LANE.  Must be
+// called by all 1024 lanes of a workgroup; lds needs 17 words; in and out
+// 16-byte aligned.  Returns the total to every lane.
+template <bool POPC, int SCAN1_PER_LANE>
 __device__ __forceinline__ uint32_t block_scan_loop(const void *in,
                                                     uint32_t *out, size_t n,
                                                     uint32_t *lds) {
   const int t = threadIdx.x;
   const int lane = t & 63, wave = t >> 6;
-  size_t chunk = (n + SCAN1_THREADS - 1) / SCAN1_THREADS;
-  chunk = (chunk + 3) & ~(size_t)3;
-  const size_t start = (size_t)t * chunk;
-  uint32_t s = 0;
-  for (size_t k = 0; k < chunk && start + k < n; k += 4) {
-    uint4 v = scan1_load4<POPC>(in, start + k, n);
-    s += v.x + v.y + v.z + v.w;
+  if (n == 0) { // nothing to read (in may be null); uniform, so no barrier is skipped by some
+    if (t == 0)
+      out[0] = 0;
+    return 0;
   }
+  const size_t start = (size_t)t * SCAN1_PER_LANE;
+  uint4 v[SCAN1_PER_LANE / 4];
+#pragma unroll
+  for (int j = 0; j < SCAN1_PER_LANE / 4; ++j)
+    v[j] = scan1_load4<POPC>(in, start + 4 * j, n);
+  uint32_t s = 0;
+#pragma unroll
+  for (int j = 0; j < SCAN1_PER_LANE / 4; ++j)
+    s += v[j].x + v[j].y + v[j].z + v[j].w;
   // inclusive scan of s across the wavefront, then across the 16 wavefronts
   uint32_t incl = s;
 #pragma unroll
@@ -91,18 +91,18 @@ __device__ __forceinline__ uint32_t block_scan_loop(const void *in,
   __syncthreads();
   uint32_t run = lds[wave] + (incl - s);
   const uint32_t total = lds[16];
-  for (size_t k = 0; k < chunk && start + k < n; k += 4) {
-    uint4 v = scan1_load4<POPC>(in, start + k, n);
+#pragma unroll
+  for (int j = 0; j < SCAN1_PER_LANE / 4; ++j) {
     uint4 o;
     o.x = run;
-    o.y = o.x + v.x;
-    o.z = o.y + v.y;
-    o.w = o.z + v.z;
-    run = o.w + v.w;
-    size_t i = start + k;
+    o.y = o.x + v[j].x;
+    o.z = o.y + v[j].y;
+    o.w = o.z + v[j].z;
+    run = o.w + v[j].w;
+    const size_t i = start + 4 * j;
     if (i + 4 <= n) {
       *reinterpret_cast<uint4 *>(out + i) = o;
-    } else {
+    } else if (i < n) {
       out[i] = o.x;
       if (i + 1 < n)
         out[i + 1] = o.y;
