@@ -101,6 +101,12 @@ int scn_fill32(scn_ctx *ctx, void *d_dst, uint32_t word, size_t nWords);
  * bit mask over the same packed coordinates, and backgroundCol per sample. */
 int scn_grids_create(scn_ctx *ctx, scn_grids **grids);
 int scn_grids_destroy(scn_ctx *ctx, scn_grids *grids);
+/* Start of a batch (SpatiallySparseBatch::reset, SpatiallySparseBatch.cu:14-27,
+ * which empties every interface's grids): empties the hash tables and masks
+ * of all n objects in one launch, so that the build / plan calls of the batch
+ * need not do it one by one.  Optional; objects it has not seen are emptied
+ * by the call that fills them. */
+int scn_grids_clear_many(scn_ctx *ctx, scn_grids **grids, int n);
 /* The input-layer grids as Picture::codifyInputData leaves them
  * (Picture.h:10-11; OpenCVPicture.cpp:368-402): n active sites given as
  * (sample, key, row) in any order, key = row-major site index in the

@@ -77,6 +77,7 @@ def lib():
         "scn_d2d": (C.c_int, [vp, vp, vp, sz]),
         "scn_fill32": (C.c_int, [vp, vp, C.c_uint32, sz]),
         "scn_grids_create": (C.c_int, [vp, P(vp)]),
+        "scn_grids_clear_many": (C.c_int, [vp, C.POINTER(vp), C.c_int]),
         "scn_grids_destroy": (C.c_int, [vp, vp]),
         "scn_grids_build": (C.c_int, [vp, vp, C.c_int, C.c_int, C.c_int, vp, vp, vp, i64, vp, i32]),
         "scn_grids_info": (C.c_int, [vp, P(C.c_int), P(C.c_int), P(C.c_int), P(i64), P(i32)]),
@@ -317,9 +318,15 @@ class Grids:
         _check(lib().scn_rules_fill(self.ctx.h, self.h, out.h, d_rules.ptr, cap))
 
 
-def rules_square(ctx, grids, nIn, nOut, size, stride, minActive=1, triangular=False):
+def clear_many(ctx, grids):
+    """Empty the tables and masks of several Grids in one launch (start of a batch)."""
+    arr = (C.c_void_p * len(grids))(*[g.h for g in grids])
+    _check(lib().scn_grids_clear_many(ctx.h, arr, len(grids)))
+
+
+def rules_square(ctx, grids, nIn, nOut, size, stride, minActive=1, triangular=False, out=None):
     """plan + fill; returns (out grids, device rules, nOutSites, width)."""
-    out = Grids(ctx)
+    out = out if out is not None else Grids(ctx)
     plan = grids.plan_triangular if triangular else grids.plan_square
     n = plan(out, nIn, nOut, size, stride, minActive)
     w = out.rules_width()

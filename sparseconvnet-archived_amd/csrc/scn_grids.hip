@@ -57,6 +57,8 @@ struct scn_grids {
   unsigned log2cap = 0;
   size_t nWords = 0;
   bool rankValid = false;
+  // how much of table / bits is known to be empty right now (scn_grids_clear_many)
+  size_t cleanSlots = 0, cleanWords = 0;
   DevBuf<Slot> table;
   DevBuf<unsigned long long> bits;
   DevBuf<unsigned> prefix;
@@ -413,8 +415,11 @@ plan_samples_body(const GridView &in, const unsigned *base, long long nEntries,
     __syncthreads();
   }
   if (t == 0) {
+    // scalars is host memory the device can write (the caller waits for the
+    // stream and reads it, no copy kernel in between)
     scalars[0] = (long long)base[nEntries] + carry; // nOutputSpatialSites
     scalars[1] = (long long)base[nEntries];         // active output sites
+    scalars[15] = *badSites; // sites scn_grids_build found outside the field
   }
 }
 
@@ -730,13 +735,18 @@ static int grids_prepare(scn_ctx *ctx, scn_grids *g, int batch, int d, int n,
   g->log2cap = lg;
   size_t cap = (size_t)1 << lg;
   g->nWords = (size_t)(((long long)batch * vol + 63) / 64);
+  const void *hadTable = g->table.p, *hadBits = g->bits.p;
   SCN_TRY(g->table.reserve(cap));
   SCN_TRY(g->bits.reserve(g->nWords + 8)); // the scan reads whole 32-byte groups
+  if (g->table.p != hadTable || g->bits.p != hadBits)
+    g->cleanSlots = g->cleanWords = 0; // fresh memory
   SCN_TRY(g->prefix.reserve(g->nWords + 2));
   SCN_TRY(g->ekey.reserve((size_t)nActive + 1));
   SCN_TRY(g->erow.reserve((size_t)nActive + 1));
   SCN_TRY(g->bg.reserve((size_t)batch + 1));
-  {
+  const bool clean = cap <= g->cleanSlots && g->nWords + 2 <= g->cleanWords;
+  g->cleanSlots = g->cleanWords = 0; // about to be written
+  if (!clean) {
     size_t most = cap > g->nWords + 2 ? cap : g->nWords + 2;
     size_t blocks = (most + 255) / 256;
     if (blocks > 16384)
@@ -744,6 +754,58 @@ static int grids_prepare(scn_ctx *ctx, scn_grids *g, int batch, int d, int n,
     hipLaunchKernelGGL(k_clear_grid, dim3((unsigned)blocks), dim3(256), 0,
                        ctx->stream, (uint4 *)g->table.p, cap, g->bits.p,
                        g->nWords + 2);
+    SCN_HIP_CHECK(hipGetLastError());
+  }
+  return SCN_OK;
+}
+
+// One launch empties the tables and masks of up to CLEAR_MANY grids objects.
+#define CLEAR_MANY 24
+struct ClearList {
+  uint4 *slots[CLEAR_MANY];
+  unsigned long long *bits[CLEAR_MANY];
+  size_t nSlots[CLEAR_MANY], nWords[CLEAR_MANY];
+};
+__global__ void k_clear_many(ClearList l) {
+  const int g = blockIdx.y;
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t step = (size_t)gridDim.x * blockDim.x;
+  uint4 *slots = l.slots[g];
+  for (size_t k = i; k < l.nSlots[g]; k += step)
+    slots[k] = make_uint4(0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu);
+  unsigned long long *bits = l.bits[g];
+  for (size_t k = i; k < l.nWords[g]; k += step)
+    bits[k] = 0ull;
+}
+
+extern "C" int scn_grids_clear_many(scn_ctx *ctx, scn_grids **grids, int n) {
+  SCN_REQUIRE(ctx && (grids || n == 0) && n >= 0, SCN_ERR_ARG,
+              "scn_grids_clear_many: bad argument");
+  for (int first = 0; first < n; first += CLEAR_MANY) {
+    ClearList l;
+    int m = 0;
+    size_t most = 0;
+    for (int i = first; i < n && i < first + CLEAR_MANY; ++i) {
+      scn_grids *g = grids[i];
+      if (!g || (!g->table.p && !g->bits.p))
+        continue;
+      l.slots[m] = (uint4 *)g->table.p;
+      l.nSlots[m] = g->table.p ? g->table.cap : 0;
+      l.bits[m] = g->bits.p;
+      l.nWords[m] = g->bits.p ? g->bits.cap : 0;
+      most = l.nSlots[m] > most ? l.nSlots[m] : most;
+      most = l.nWords[m] > most ? l.nWords[m] : most;
+      g->cleanSlots = l.nSlots[m];
+      g->cleanWords = l.nWords[m];
+      g->rankValid = false;
+      ++m;
+    }
+    if (m == 0)
+      continue;
+    size_t blocks = (most + 1023) / 1024; // four elements per lane
+    blocks = blocks < 1 ? 1 : (blocks > 2048 ? 2048 : blocks);
+    hipLaunchKernelGGL(k_clear_many, dim3((unsigned)blocks, (unsigned)m),
+                       dim3(256), 0, ctx->stream, l);
     SCN_HIP_CHECK(hipGetLastError());
   }
   return SCN_OK;
@@ -761,10 +823,8 @@ static int ensure_rank(scn_ctx *ctx, scn_grids *g) {
   return SCN_OK;
 }
 
+// waits for the kernels that wrote the counts into the mapped host words
 static int read_scalars(scn_ctx *ctx) {
-  SCN_HIP_CHECK(hipMemcpyAsync(ctx->h_pinned, ctx->d_scalars,
-                               16 * sizeof(int64_t), hipMemcpyDeviceToHost,
-                               ctx->stream));
   SCN_HIP_CHECK(hipStreamSynchronize(ctx->stream));
   if (ctx->h_pinned[15] != 0) {
     long long bad = ctx->h_pinned[15];
@@ -930,18 +990,18 @@ static int plan_regions_d(scn_ctx *ctx, scn_grids *in, scn_grids *out,
       hipLaunchKernelGGL((k_plan_scan_samples<32>), dim3(1), dim3(1024), 0,
                          ctx->stream, vin, out->cnt.p, out->base.p, nE, fullSize,
                          out->bg.p, out->bgBefore.p, out->sampleStart.p,
-                         (long long *)ctx->d_scalars, bad);
+                         (long long *)ctx->d_pinned, bad);
     else
       hipLaunchKernelGGL((k_plan_scan_samples<64>), dim3(1), dim3(1024), 0,
                          ctx->stream, vin, out->cnt.p, out->base.p, nE, fullSize,
                          out->bg.p, out->bgBefore.p, out->sampleStart.p,
-                         (long long *)ctx->d_scalars, bad);
+                         (long long *)ctx->d_pinned, bad);
   } else {
     SCN_TRY(scn_scan_exclusive_u32(ctx->stream, out->cnt.p, out->base.p,
                                    (size_t)nE, out->scanTmp.p));
     hipLaunchKernelGGL(k_plan_samples, dim3(1), dim3(1024), 0, ctx->stream, vin,
                        out->base.p, nE, fullSize, out->bg.p, out->bgBefore.p,
-                       out->sampleStart.p, (long long *)ctx->d_scalars, bad);
+                       out->sampleStart.p, (long long *)ctx->d_pinned, bad);
   }
   SCN_HIP_CHECK(hipGetLastError());
   SCN_TRY(read_scalars(ctx));
@@ -1077,7 +1137,7 @@ extern "C" int scn_rules_terminal_plan(scn_ctx *ctx, const scn_grids *cin,
   SCN_TRY(out->sampleStart.reserve((size_t)in->batch + 2));
   hipLaunchKernelGGL(k_terminal_plan, dim3(1), dim3(1024), 0, ctx->stream,
                      view_of(in), out->sampleStart.p,
-                     (long long *)ctx->d_scalars);
+                     (long long *)ctx->d_pinned);
   SCN_HIP_CHECK(hipGetLastError());
   SCN_TRY(read_scalars(ctx));
   long long S = ctx->h_pinned[0];

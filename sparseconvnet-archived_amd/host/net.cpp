@@ -180,6 +180,15 @@ void SparseConvNetCUDA::ensureInterfaces() {
       slot.interfaces.emplace_back(sharedSubInterfaces.back());
   }
 }
+// every grids object the slot owns, emptied in one launch at the start of a batch
+static void clearDeviceGrids(scn_ctx *ctx, SpatiallySparseBatch &b) {
+  std::vector<scn_grids *> owned;
+  for (auto &iface : b.interfaces)
+    if (iface.deviceGrids && iface.ownsDeviceGrids)
+      owned.push_back(iface.deviceGrids);
+  if (!owned.empty())
+    SCN_CHECKED(scn_grids_clear_many(ctx, owned.data(), (int)owned.size()));
+}
 void SparseConvNetCUDA::preprocessResident(int cc, const ResidentBatch &input) {
   SpatiallySparseBatch &b = batchPool[cc];
   scn_ctx *ctx = b.preprocessStream ? b.preprocessStream->ctx : memStream.ctx;
@@ -196,6 +205,7 @@ void SparseConvNetCUDA::preprocessResident(int cc, const ResidentBatch &input) {
     in.ownsDeviceGrids = true;
   }
   scn_prof_tag(ctx, -1);
+  clearDeviceGrids(ctx, b);
   SCN_CHECKED(scn_grids_build(ctx, in.deviceGrids, input.batchSize, dimension,
                               in.spatialSize, input.d_sample, input.d_key,
                               input.d_row, input.nActive, input.d_background,
@@ -537,6 +547,7 @@ void BatchProducer::preprocessBatchOnDevice(int cc) {
     in.ownsDeviceGrids = true;
   }
   scn_prof_tag(ctx, -1);
+  clearDeviceGrids(ctx, b);
   SCN_CHECKED(scn_grids_build(ctx, in.deviceGrids, b.batchSize, cnn.dimension,
                               in.spatialSize, b.stagingSample.dPtr(),
                               (const int64_t *)b.stagingKey.dPtr(),

@@ -1,5 +1,8 @@
 // C view of the host classes (see scn_host_c.h).
 #include "scn_host_c.h"
+#include <time.h>
+#include <stdlib.h>
+#include <stdio.h>
 #include <cstdio>
 #include <cstdlib>
 #include <memory>
@@ -338,13 +341,19 @@ int scnh_forward_resident_stream(scnh_net *net, int nBatches, int batch,
     }
     ++done;
   };
+  double tNext = 0, tFwd = 0, tFin = 0;
+  auto now = [] { timespec ts; clock_gettime(CLOCK_MONOTONIC, &ts); return ts.tv_sec * 1e3 + ts.tv_nsec * 1e-6; };
+  double t0 = now();
   while (SpatiallySparseBatch *b = bp.nextBatch()) {
+    double t1 = now(); tNext += t1 - t0;
     if (net->hasClassifier)
       cnn->forwardBatch(*b);
     else
       forward_layers(net, *b);
+    double t2 = now(); tFwd += t2 - t1;
     if (queued)
       finish(queued);
+    t0 = now(); tFin += t0 - t2;
     queued = b;
     if (!bp.keepAlive) {
       finish(queued);
@@ -354,6 +363,8 @@ int scnh_forward_resident_stream(scnh_net *net, int nBatches, int batch,
   if (queued)
     finish(queued);
   cnn->memStream.synchronize();
+  if (getenv("SCN_TIMING_TMP"))
+    fprintf(stderr, "TIMING per batch: nextBatch %.3f ms, forwardBatch (launch) %.3f ms, finish %.3f ms\n", tNext / nBatches, tFwd / nBatches, tFin / nBatches);
   net->batch = nullptr;
   return done;
 }

@@ -119,6 +119,29 @@ def test_chained_layers_2d(scn, ctx):
     assert S == o_S and np.array_equal(d_rules.download()[: 6 * S], o_rules)
 
 
+def test_grids_reused_across_batches_with_one_clear(scn, ctx):
+    """The same grids objects take three batches in a row (large, small, large)
+    with scn_grids_clear_many at the start of each, as the host classes do:
+    nothing of an earlier batch may survive in a table or a mask."""
+    rng = np.random.default_rng(21)
+    sizes = [18, 17, 8]
+    geoms = [(2, 1), (3, 2)]
+    dg = scn.Grids(ctx)
+    outs = [scn.Grids(ctx), scn.Grids(ctx)]
+    for batch, density in ((7, 0.08), (2, 0.02), (5, 0.3)):
+        samples, nSites = brute.random_samples(rng, batch, 2, sizes[0], density)
+        scn.clear_many(ctx, [dg] + outs)
+        s, k, r, bg = flatten_samples(samples)
+        dg.build(len(samples), 2, sizes[0], s, k, r, bg, nSites)
+        og, cur = oracle_grids(samples), dg
+        for (size, stride), nIn, nOut, out in zip(geoms, sizes[:-1], sizes[1:], outs):
+            og2, o_rules, o_n = orc.rules_square(og, 2, nIn, nOut, size, stride, 1)
+            d2, d_rules, n, w = scn.rules_square(ctx, cur, nIn, nOut, size, stride, 1, out=out)
+            assert n == o_n and np.array_equal(d_rules.download()[: n * w], o_rules)
+            assert_same_grids(d2, og2)
+            og, cur = og2, d2
+
+
 def test_larger_3d_batch(scn, ctx):
     rng = np.random.default_rng(12)
     nOut, size, stride = 22, 3, 1
