@@ -153,6 +153,19 @@ int scn_rules_triangular_plan(scn_ctx *ctx, const scn_grids *in,
 int scn_rules_terminal_plan(scn_ctx *ctx, const scn_grids *in, scn_grids *out,
                             int64_t *ruleWidth);
 /* Rule width of the plan held by `out` (size^d, triangleSize, or S). */
+/* Deferred counts.  BatchProducer::preprocessBatch (BatchProducer.cu:40-87)
+ * runs every layer's preprocess() back to back on the CPU; on the GPU every
+ * plan call above would wait for its counts, one host round trip per layer.
+ * With deferral on, a plan whose `out` object has held a plan before returns
+ * at once: *nOutSites (or *ruleWidth) is an UPPER BOUND derived from the
+ * largest counts that object has seen, buffers sized by it are large enough,
+ * and scn_rules_fill on such a pair is bounded the same way.  scn_rules_settle
+ * then waits once for the stream and makes the real counts readable
+ * (scn_grids_info, scn_rules_width).  It returns SCN_ERR_CAPACITY when a
+ * batch outgrew a bound: nothing out of range was written, and the caller
+ * plans the batch again with deferral off (that also raises the bounds). */
+int scn_ctx_defer_counts(scn_ctx *ctx, int on);
+int scn_rules_settle(scn_ctx *ctx);
 int scn_rules_width(const scn_grids *out, int64_t *width);
 /* Writes nOutputSpatialSites * width int32 rules; capacity in int32s. */
 int scn_rules_fill(scn_ctx *ctx, const scn_grids *in, scn_grids *out,

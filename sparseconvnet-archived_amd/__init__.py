@@ -19,6 +19,7 @@ HEADER = os.path.join(ROOT, "include", "scn_hip.h")
 # ActivationFunction (reference types.h:11-20)
 NOSIGMOID, RELU, VLEAKYRELU, LEAKYRELU, TANH, SOFTMAX, PRELU, SIGMOID = range(8)
 FP32, BF16, BF16X3 = 0, 1, 2
+OK, ERR_ARG, ERR_HIP, ERR_CAPACITY, ERR_STATE = range(5)
 K_GRID_BUILD, K_RULES, K_GATHER, K_NIN, K_MAXPOOL, K_TERMINAL, K_SOFTMAX, K_CONV_NIN, K_PROBE = range(9)
 KERNEL_FAMILIES = ["grid_build", "rules", "gather", "nin", "maxpool", "terminal", "softmax", "conv_nin", "probe"]
 
@@ -78,6 +79,8 @@ def lib():
         "scn_fill32": (C.c_int, [vp, vp, C.c_uint32, sz]),
         "scn_grids_create": (C.c_int, [vp, P(vp)]),
         "scn_grids_clear_many": (C.c_int, [vp, C.POINTER(vp), C.c_int]),
+        "scn_ctx_defer_counts": (C.c_int, [vp, C.c_int]),
+        "scn_rules_settle": (C.c_int, [vp]),
         "scn_grids_destroy": (C.c_int, [vp, vp]),
         "scn_grids_build": (C.c_int, [vp, vp, C.c_int, C.c_int, C.c_int, vp, vp, vp, i64, vp, i32]),
         "scn_grids_info": (C.c_int, [vp, P(C.c_int), P(C.c_int), P(C.c_int), P(i64), P(i32)]),
@@ -316,6 +319,19 @@ class Grids:
     def fill(self, out, d_rules, capacity=None):
         cap = d_rules.size if capacity is None else capacity
         _check(lib().scn_rules_fill(self.ctx.h, self.h, out.h, d_rules.ptr, cap))
+
+
+def defer_counts(ctx, on):
+    _check(lib().scn_ctx_defer_counts(ctx.h, int(on)))
+
+
+def settle(ctx):
+    """Collect deferred counts; returns False when a bound was outgrown (plan again with deferral off)."""
+    rc = lib().scn_rules_settle(ctx.h)
+    if rc == ERR_CAPACITY:
+        return False
+    _check(rc)
+    return True
 
 
 def clear_many(ctx, grids):

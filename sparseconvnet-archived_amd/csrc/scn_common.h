@@ -40,15 +40,22 @@ struct ProfSpan {
 };
 
 #define SCN_ZERO_FLOATS 4096
+#define SCN_MAX_PENDING 62 // plans per settle; 16 + 4 * 62 = 264 pinned words
+#define SCN_PINNED_WORDS (16 + 4 * SCN_MAX_PENDING)
 struct scn_ctx {
   int device;
   hipStream_t stream;
   int numCU;
   // small pinned buffer for counts that must come back to the host
-  int64_t *h_pinned; // 16 int64, host view
+  int64_t *h_pinned; // SCN_PINNED_WORDS int64, host view
   int64_t *d_pinned; // the same memory as the device sees it
   int64_t *d_scalars; // 16 int64
   float *d_zeros;     // SCN_ZERO_FLOATS zeros: the row a negative rule stands for
+  long long ticket;   // number of the last count readback (h_pinned[14] echoes it)
+  // deferred counts (scn_ctx_defer_counts): plans whose counts are still on
+  // their way; slot i of them reports into h_pinned[16 + 4 i ..]
+  bool deferCounts;
+  std::vector<struct scn_grids *> pendingGrids;
   // profiling
   bool prof;
   int profTag;

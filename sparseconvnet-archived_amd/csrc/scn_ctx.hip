@@ -28,15 +28,17 @@ extern "C" int scn_ctx_create(int device, scn_ctx **out) {
   c->device = device;
   c->prof = false;
   c->profTag = 0;
+  c->ticket = 0;
+  c->deferCounts = false;
   memset(c->profMs, 0, sizeof(c->profMs));
   memset(c->profCalls, 0, sizeof(c->profCalls));
   hipDeviceProp_t prop;
   SCN_HIP_CHECK(hipGetDeviceProperties(&prop, device));
   c->numCU = prop.multiProcessorCount;
   SCN_HIP_CHECK(hipStreamCreate(&c->stream)); // default priority
-  SCN_HIP_CHECK(hipHostMalloc((void **)&c->h_pinned, 16 * sizeof(int64_t),
+  SCN_HIP_CHECK(hipHostMalloc((void **)&c->h_pinned, SCN_PINNED_WORDS * sizeof(int64_t),
                               hipHostMallocMapped));
-  memset(c->h_pinned, 0, 16 * sizeof(int64_t));
+  memset(c->h_pinned, 0, SCN_PINNED_WORDS * sizeof(int64_t));
   SCN_HIP_CHECK(hipHostGetDevicePointer((void **)&c->d_pinned, c->h_pinned, 0));
   SCN_HIP_CHECK(hipMalloc((void **)&c->d_scalars, 16 * sizeof(int64_t)));
   SCN_HIP_CHECK(hipMemset(c->d_scalars, 0, 16 * sizeof(int64_t)));

@@ -19,6 +19,7 @@
 // which needs no sort: count owned outputs per input, scatter the counts to
 // iteration order through the rank, prefix-sum, emit.
 #include "scn_common.h"
+#include <atomic>
 #include "scn_scan_dev.h"
 
 struct __align__(16) Slot {
@@ -49,6 +50,22 @@ struct GridView {
   int n, d, batch;
 };
 
+// A count the host may not know yet: an upper bound, and where the real value
+// is (device memory written by an earlier kernel of the same stream); live ==
+// null means the bound is exact.
+struct Count {
+  long long bound;
+  const long long *live;
+};
+__device__ __forceinline__ long long count_now(const Count &c) {
+  if (!c.live)
+    return c.bound;
+  const long long v = *c.live;
+  return v < c.bound ? v : c.bound;
+}
+// per-grids device record
+enum { META_SITES = 0, META_ACTIVE = 1, META_OVERFLOW = 2, META_WIDTH = 3 };
+
 struct scn_grids {
   int batch = 0, d = 0, n = 0;
   long long vol = 0;
@@ -59,6 +76,14 @@ struct scn_grids {
   bool rankValid = false;
   // how much of table / bits is known to be empty right now (scn_grids_clear_many)
   size_t cleanSlots = 0, cleanWords = 0;
+  // Deferred counts: while pending, nActive / nSites / termS hold upper bounds
+  // and the real values are in meta (device) and on their way to the pinned
+  // slot; seen* are the largest values this object has ever held, from which
+  // the next bounds are derived.
+  bool pending = false;
+  int pinnedSlot = -1;
+  long long seenRows = 0, seenActive = 0, seenWidth = 0;
+  DevBuf<long long> meta; // META_* words
   DevBuf<Slot> table;
   DevBuf<unsigned long long> bits;
   DevBuf<unsigned> prefix;
@@ -349,11 +374,20 @@ __global__ void k_grid_build(GridView g, const int *sample,
 // position in iteration order
 template <int D>
 __global__ void k_plan_count(GridView in, Geom g, const long long *ekey,
-                             long long nEntries, unsigned *cntByRank,
-                             unsigned long long *ownMask, unsigned *rankOf) {
+                             Count nEntries, const long long *inMeta,
+                             unsigned *cntByRank, unsigned long long *ownMask,
+                             unsigned *rankOf) {
   long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (e >= nEntries)
+  if (e >= nEntries.bound)
     return;
+  // an input whose own deferred plan outgrew its bounds holds no entries worth
+  // reading (its emit pass wrote nothing): count nothing
+  if (e >= count_now(nEntries) || (inMeta && inMeta[META_OVERFLOW])) {
+    // past the real entries: the ranks of the real ones are below their
+    // number, so these lanes zero exactly the rest of what the scan covers
+    cntByRank[e] = 0;
+    return;
+  }
   long long p = ekey[e];
   int b = (int)(p / g.volIn);
   int i[D];
@@ -378,7 +412,9 @@ __device__ __forceinline__ void
 plan_samples_body(const GridView &in, const unsigned *base, long long nEntries,
                   long long fullSize, int *outBg, int *bgBefore,
                   unsigned *sampleStart, volatile long long *scalars,
-                  const long long *badSites) {
+                  const long long *badSites, long long ticket,
+                  long long *meta, const long long *inMeta, long long boundRows,
+                  long long boundActive, int pinnedSlot) {
   __shared__ int lds[1024];
   __shared__ int carry;
   const int t = threadIdx.x;
@@ -415,11 +451,28 @@ plan_samples_body(const GridView &in, const unsigned *base, long long nEntries,
     __syncthreads();
   }
   if (t == 0) {
+    const long long nSites = (long long)base[nEntries] + carry; // nOutputSpatialSites
+    const long long nActive = (long long)base[nEntries];        // active output sites
+    const long long over = (inMeta && inMeta[META_OVERFLOW]) || nSites > boundRows ||
+                           nActive > boundActive;
+    meta[META_SITES] = nSites;
+    meta[META_ACTIVE] = nActive;
+    meta[META_OVERFLOW] = over;
     // scalars is host memory the device can write (the caller waits for the
     // stream and reads it, no copy kernel in between)
-    scalars[0] = (long long)base[nEntries] + carry; // nOutputSpatialSites
-    scalars[1] = (long long)base[nEntries];         // active output sites
-    scalars[15] = *badSites; // sites scn_grids_build found outside the field
+    if (pinnedSlot >= 0) { // deferred: read at settle time
+      volatile long long *slot = scalars + 16 + 4 * pinnedSlot;
+      slot[0] = nSites;
+      slot[1] = nActive;
+      slot[2] = over;
+      scalars[15] = *badSites;
+    } else {
+      scalars[0] = nSites;
+      scalars[1] = nActive;
+      scalars[15] = *badSites; // sites scn_grids_build found outside the field
+      __threadfence_system();
+      scalars[14] = ticket; // last: the host spins on this word
+    }
   }
 }
 
@@ -427,9 +480,12 @@ __global__ void __launch_bounds__(1024)
     k_plan_samples(GridView in, const unsigned *base, long long nEntries,
                    long long fullSize, int *outBg, int *bgBefore,
                    unsigned *sampleStart, long long *scalars,
-                   const long long *badSites) {
+                   const long long *badSites, long long ticket, long long *meta,
+                   const long long *inMeta, long long boundRows,
+                   long long boundActive, int pinnedSlot) {
   plan_samples_body(in, base, nEntries, fullSize, outBg, bgBefore, sampleStart,
-                    scalars, badSites);
+                    scalars, badSites, ticket, meta, inMeta, boundRows,
+                    boundActive, pinnedSlot);
 }
 
 // small batches: prefix sum of the owned counts and the per-sample pass in
@@ -439,28 +495,35 @@ __global__ void __launch_bounds__(1024)
     k_plan_scan_samples(GridView in, const unsigned *cnt, unsigned *base,
                         long long nEntries, long long fullSize, int *outBg,
                         int *bgBefore, unsigned *sampleStart,
-                        long long *scalars, const long long *badSites) {
+                        long long *scalars, const long long *badSites,
+                        long long ticket, long long *meta,
+                        const long long *inMeta, long long boundRows,
+                        long long boundActive, int pinnedSlot) {
   __shared__ uint32_t ldsScan[17];
   (void)block_scan_loop<false, PER>(cnt, base, (size_t)nEntries, ldsScan);
   __syncthreads(); // the block's own writes to base[] are visible to it
   plan_samples_body(in, base, nEntries, fullSize, outBg, bgBefore, sampleStart,
-                    scalars, badSites);
+                    scalars, badSites, ticket, meta, inMeta, boundRows,
+                    boundActive, pinnedSlot);
 }
 
 // pass 2: emit the owned outputs
 template <int D>
 __global__ void k_plan_emit(GridView in, GridView out, Geom g,
-                            const long long *ekey, long long nEntries,
+                            const long long *ekey, Count nEntries,
+                            const long long *outMeta,
                             const unsigned *base, const int *bgBefore,
                             const int *outBg, long long *okey, int *orow,
                             long long *siteKey) {
   long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (outMeta[META_OVERFLOW])
+    return; // the bounds did not hold: nothing may be written
   if (e < in.batch) { // background rows
     int r = outBg[e];
     if (r >= 0)
       siteKey[r] = -1 - e;
   }
-  if (e >= nEntries)
+  if (e >= count_now(nEntries))
     return;
   long long p = ekey[e];
   int b = (int)(p / g.volIn);
@@ -485,7 +548,8 @@ __global__ void k_plan_emit(GridView in, GridView out, Geom g,
 // dependent atomics.
 template <int D>
 __global__ void k_plan_emit_masked(GridView in, GridView out, Geom g,
-                                   const long long *ekey, long long nEntries,
+                                   const long long *ekey, Count nEntries,
+                                   const long long *outMeta,
                                    const unsigned *base,
                                    const unsigned long long *ownMask,
                                    const unsigned *rankOf,
@@ -494,12 +558,14 @@ __global__ void k_plan_emit_masked(GridView in, GridView out, Geom g,
                                    long long *siteKey) {
   long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   const int c = blockIdx.y;
+  if (outMeta[META_OVERFLOW])
+    return; // the bounds did not hold: nothing may be written
   if (c == 0 && e < in.batch) { // background rows
     int r = outBg[e];
     if (r >= 0)
       siteKey[r] = -1 - e;
   }
-  if (e >= nEntries)
+  if (e >= count_now(nEntries))
     return;
   unsigned long long mask = ownMask[e];
   if (!((mask >> c) & 1ull))
@@ -560,9 +626,12 @@ __global__ void k_tri_table(int size, int d, int *invOrd) {
 // one thread per rule: rules[row * width + q]
 template <int D>
 __global__ void k_rules_fill(GridView in, Geom g, const long long *siteKey,
-                             long long nSites, const int *invOrd, int *rules) {
+                             Count nSites, const long long *outMeta,
+                             const int *invOrd, int *rules) {
   long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  long long total = nSites * g.width;
+  if (outMeta[META_OVERFLOW])
+    return;
+  long long total = count_now(nSites) * g.width;
   if (idx >= total)
     return;
   long long r = idx / g.width;
@@ -592,7 +661,10 @@ __global__ void k_rules_fill(GridView in, Geom g, const long long *siteKey,
 
 // terminal pooling: sample sizes and their maximum.  One block.
 __global__ void k_terminal_plan(GridView in, unsigned *sampleStart,
-                                long long *scalars) {
+                                volatile long long *scalars,
+                                long long ticket, long long *meta,
+                                const long long *inMeta, long long boundWidth,
+                                int pinnedSlot) {
   __shared__ long long lds[1024];
   const int t = threadIdx.x;
   long long mx = 1; // TerminalPoolingLayer.cu:90
@@ -612,8 +684,24 @@ __global__ void k_terminal_plan(GridView in, unsigned *sampleStart,
       lds[t] = lds[t + off];
     __syncthreads();
   }
-  if (t == 0)
-    scalars[0] = lds[0];
+  if (t == 0) {
+    const long long over = (inMeta && inMeta[META_OVERFLOW]) || lds[0] > boundWidth;
+    meta[META_SITES] = in.batch;
+    meta[META_ACTIVE] = in.batch;
+    meta[META_OVERFLOW] = over;
+    meta[META_WIDTH] = lds[0];
+    if (pinnedSlot >= 0) { // deferred: read at settle time
+      volatile long long *slot = scalars + 16 + 4 * pinnedSlot;
+      slot[0] = in.batch;
+      slot[1] = in.batch;
+      slot[2] = over;
+      slot[3] = lds[0];
+    } else {
+      scalars[0] = lds[0];
+      __threadfence_system();
+      scalars[14] = ticket;
+    }
+  }
 }
 
 // out grid of the terminal layer: key 0 of sample b -> row b
@@ -631,8 +719,12 @@ __global__ void k_terminal_out(GridView out, long long *okey, int *orow,
 }
 
 __global__ void k_terminal_init(GridView in, const unsigned *sampleStart,
-                                long long S, int *rules) {
+                                Count width, const long long *outMeta,
+                                int *rules) {
   long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (outMeta[META_OVERFLOW])
+    return;
+  const long long S = count_now(width);
   if (idx >= (long long)in.batch * S)
     return;
   int b = (int)(idx / S);
@@ -646,12 +738,13 @@ __global__ void k_terminal_init(GridView in, const unsigned *sampleStart,
 }
 
 __global__ void k_terminal_scatter(GridView in, const long long *ekey,
-                                   const int *erow, long long nEntries,
-                                   const unsigned *sampleStart, long long S,
-                                   int *rules) {
+                                   const int *erow, Count nEntries,
+                                   const unsigned *sampleStart, Count width,
+                                   const long long *outMeta, int *rules) {
   long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (e >= nEntries)
+  if (outMeta[META_OVERFLOW] || e >= count_now(nEntries))
     return;
+  const long long S = count_now(width);
   long long p = ekey[e];
   int b = (int)(p / in.vol);
   unsigned r = rank_of(in, p) - sampleStart[b];
@@ -728,6 +821,7 @@ static int grids_prepare(scn_ctx *ctx, scn_grids *g, int batch, int d, int n,
   g->rankValid = false;
   g->planKind = PLAN_NONE;
   g->planIn = nullptr;
+  g->pending = false;
   unsigned lg = 6;
   while ((1ll << lg) < 2 * nActive)
     ++lg;
@@ -823,9 +917,27 @@ static int ensure_rank(scn_ctx *ctx, scn_grids *g) {
   return SCN_OK;
 }
 
-// waits for the kernels that wrote the counts into the mapped host words
-static int read_scalars(scn_ctx *ctx) {
-  SCN_HIP_CHECK(hipStreamSynchronize(ctx->stream));
+// Waits for the kernel that wrote the counts into the mapped host words.  The
+// kernel writes its ticket last; watching that word costs a microsecond or two
+// where a stream synchronisation costs ten, and this wait is on the critical
+// path of every layer.  A kernel that does not deliver falls back to the
+// stream (which also surfaces its error).
+static int read_scalars(scn_ctx *ctx, long long ticket) {
+  volatile int64_t *word = ctx->h_pinned + 14;
+  bool seen = false;
+  for (int spin = 0; spin < 400000; ++spin) {
+    if (*word == ticket) {
+      seen = true;
+      break;
+    }
+    __builtin_ia32_pause();
+  }
+  std::atomic_thread_fence(std::memory_order_acquire);
+  if (!seen) {
+    SCN_HIP_CHECK(hipStreamSynchronize(ctx->stream));
+    SCN_REQUIRE(*word == ticket, SCN_ERR_STATE,
+                "rules: the planning kernel did not deliver its counts");
+  }
   if (ctx->h_pinned[15] != 0) {
     long long bad = ctx->h_pinned[15];
     ctx->h_pinned[15] = 0;
@@ -834,6 +946,85 @@ static int read_scalars(scn_ctx *ctx) {
                 "scn_grids_build was given %lld sites outside the field", bad);
   }
   return SCN_OK;
+}
+
+static Count count_active(const scn_grids *g) {
+  Count c;
+  c.bound = g->nActive;
+  c.live = g->pending ? g->meta.p + META_ACTIVE : nullptr;
+  return c;
+}
+static Count count_sites(const scn_grids *g) {
+  Count c;
+  c.bound = g->nSites;
+  c.live = g->pending ? g->meta.p + META_SITES : nullptr;
+  return c;
+}
+static Count count_width(const scn_grids *g) {
+  Count c;
+  c.bound = g->termS;
+  c.live = g->pending ? g->meta.p + META_WIDTH : nullptr;
+  return c;
+}
+static long long grow_bound(long long seen, long long slack, long long cap) {
+  long long b = seen + seen / 4 + slack;
+  return b < cap ? b : cap;
+}
+
+// Deferred counts.  With deferral on, a plan whose output object has held a
+// plan before does not wait for its counts: it sizes everything by bounds
+// derived from the largest counts the object has seen, its kernels read the
+// real counts from device memory, and scn_rules_settle() collects them all
+// with one synchronisation.
+extern "C" int scn_ctx_defer_counts(scn_ctx *ctx, int on) {
+  SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_ctx_defer_counts: null context");
+  ctx->deferCounts = on != 0;
+  return SCN_OK;
+}
+extern "C" int scn_rules_settle(scn_ctx *ctx) {
+  SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_rules_settle: null context");
+  if (ctx->pendingGrids.empty())
+    return SCN_OK;
+  SCN_HIP_CHECK(hipStreamSynchronize(ctx->stream));
+  std::atomic_thread_fence(std::memory_order_acquire);
+  bool overflowed = false;
+  for (scn_grids *g : ctx->pendingGrids) {
+    const volatile int64_t *slot = ctx->h_pinned + 16 + 4 * g->pinnedSlot;
+    if (slot[2]) {
+      overflowed = true;
+      g->planKind = PLAN_NONE; // nothing was emitted
+      g->nSites = 0;
+      g->nActive = 0;
+    } else {
+      g->nSites = (int)slot[0];
+      g->nActive = slot[1];
+      g->seenRows = slot[0] > g->seenRows ? slot[0] : g->seenRows;
+      g->seenActive = slot[1] > g->seenActive ? slot[1] : g->seenActive;
+      if (g->planKind == PLAN_TERMINAL) {
+        g->termS = slot[3];
+        g->seenWidth = slot[3] > g->seenWidth ? slot[3] : g->seenWidth;
+      }
+    }
+    g->pending = false;
+    g->pinnedSlot = -1;
+  }
+  ctx->pendingGrids.clear();
+  if (ctx->h_pinned[15] != 0) {
+    long long bad = ctx->h_pinned[15];
+    ctx->h_pinned[15] = 0;
+    SCN_TRY(scn_fill32(ctx, ctx->d_scalars + 15, 0u, 2));
+    SCN_REQUIRE(false, SCN_ERR_ARG,
+                "scn_grids_build was given %lld sites outside the field", bad);
+  }
+  SCN_REQUIRE(!overflowed, SCN_ERR_CAPACITY,
+              "scn_rules_settle: a batch outgrew the bounds of its deferred "
+              "plans; plan it again with deferral off");
+  return SCN_OK;
+}
+static void mark_pending(scn_ctx *ctx, scn_grids *g, int slot) {
+  g->pending = true;
+  g->pinnedSlot = slot;
+  ctx->pendingGrids.push_back(g);
 }
 
 extern "C" int scn_grids_create(scn_ctx *ctx, scn_grids **out) {
@@ -845,8 +1036,16 @@ extern "C" int scn_grids_create(scn_ctx *ctx, scn_grids **out) {
 extern "C" int scn_grids_destroy(scn_ctx *ctx, scn_grids *g) {
   if (!g)
     return SCN_OK;
-  if (ctx)
+  if (ctx) {
     (void)hipStreamSynchronize(ctx->stream);
+    auto &pl = ctx->pendingGrids;
+    for (size_t i = 0; i < pl.size(); ++i)
+      if (pl[i] == g) {
+        pl.erase(pl.begin() + i);
+        break;
+      }
+  }
+  g->meta.release();
   g->table.release();
   g->bits.release();
   g->prefix.release();
@@ -900,6 +1099,9 @@ extern "C" int scn_grids_info(const scn_grids *g, int *batch, int *dimension,
                               int *spatialSize, int64_t *nActive,
                               int32_t *nSpatialSites) {
   SCN_REQUIRE(g, SCN_ERR_ARG, "scn_grids_info: null grids");
+  SCN_REQUIRE(!g->pending, SCN_ERR_STATE,
+              "scn_grids_info: the counts of these grids are deferred; call "
+              "scn_rules_settle first");
   if (batch)
     *batch = g->batch;
   if (dimension)
@@ -918,6 +1120,9 @@ extern "C" int scn_grids_download(scn_ctx *ctx, const scn_grids *cg,
                                   int32_t *h_row, int32_t *h_background) {
   scn_grids *g = const_cast<scn_grids *>(cg);
   SCN_REQUIRE(ctx && g, SCN_ERR_ARG, "scn_grids_download: null argument");
+  SCN_REQUIRE(!g->pending, SCN_ERR_STATE,
+              "scn_grids_download: the counts of these grids are deferred; "
+              "call scn_rules_settle first");
   SCN_TRY(ensure_rank(ctx, g));
   long long n = g->nActive;
   if (n > 0) {
@@ -961,7 +1166,22 @@ template <int D>
 static int plan_regions_d(scn_ctx *ctx, scn_grids *in, scn_grids *out,
                           const Geom &g, long long fullSize,
                           int64_t *nOutSites) {
-  const long long nE = in->nActive;
+  // deferred: size by bounds, leave the counts on the device (see scn_rules_settle)
+  const bool deferred = ctx->deferCounts && out->seenRows > 0 &&
+                        (int)ctx->pendingGrids.size() < SCN_MAX_PENDING;
+  if (!deferred && in->pending)
+    SCN_TRY(scn_rules_settle(ctx)); // the exact path needs the exact input count
+  const long long nE = in->nActive; // a bound while `in` is pending
+  const Count nEc = count_active(in);
+  const long long *inMeta = in->pending ? in->meta.p : nullptr;
+  const long long volOutAll = (long long)in->batch * g.volOut;
+  const long long boundActive =
+      deferred ? grow_bound(out->seenActive, 64, volOutAll) : 0x7FFFFFFFFFFFll;
+  const long long boundRows =
+      deferred ? grow_bound(out->seenRows, 64, boundActive + in->batch)
+               : 0x7FFFFFFFFFFFll;
+  const int slot = deferred ? (int)ctx->pendingGrids.size() : -1;
+  SCN_TRY(out->meta.reserve(8));
   SCN_TRY(out->cnt.reserve((size_t)nE + 8)); // the scan reads whole 16-byte groups
   SCN_TRY(out->base.reserve((size_t)nE + 2));
   SCN_TRY(out->bgBefore.reserve((size_t)in->batch + 2));
@@ -980,52 +1200,65 @@ static int plan_regions_d(scn_ctx *ctx, scn_grids *in, scn_grids *out,
   }
   if (nE > 0) {
     hipLaunchKernelGGL(k_plan_count<D>, dim3(scn_ceil_div(nE, 256)), dim3(256),
-                       0, ctx->stream, vin, g, in->ekey.p, nE, out->cnt.p,
+                       0, ctx->stream, vin, g, in->ekey.p, nEc, inMeta, out->cnt.p,
                        masked ? out->ownMask.p : nullptr, out->rankOf.p);
     SCN_HIP_CHECK(hipGetLastError());
   }
   const long long *bad = (const long long *)(ctx->d_scalars + 15);
+  const long long ticket = ++ctx->ticket;
   if ((size_t)nE <= SCAN1_MAX_ELEMS) {
     if ((size_t)nE <= SCAN1_SMALL_ELEMS)
       hipLaunchKernelGGL((k_plan_scan_samples<32>), dim3(1), dim3(1024), 0,
                          ctx->stream, vin, out->cnt.p, out->base.p, nE, fullSize,
                          out->bg.p, out->bgBefore.p, out->sampleStart.p,
-                         (long long *)ctx->d_pinned, bad);
+                         (long long *)ctx->d_pinned, bad, ticket, out->meta.p,
+                         inMeta, boundRows, boundActive, slot);
     else
       hipLaunchKernelGGL((k_plan_scan_samples<64>), dim3(1), dim3(1024), 0,
                          ctx->stream, vin, out->cnt.p, out->base.p, nE, fullSize,
                          out->bg.p, out->bgBefore.p, out->sampleStart.p,
-                         (long long *)ctx->d_pinned, bad);
+                         (long long *)ctx->d_pinned, bad, ticket, out->meta.p,
+                         inMeta, boundRows, boundActive, slot);
   } else {
     SCN_TRY(scn_scan_exclusive_u32(ctx->stream, out->cnt.p, out->base.p,
                                    (size_t)nE, out->scanTmp.p));
     hipLaunchKernelGGL(k_plan_samples, dim3(1), dim3(1024), 0, ctx->stream, vin,
                        out->base.p, nE, fullSize, out->bg.p, out->bgBefore.p,
-                       out->sampleStart.p, (long long *)ctx->d_pinned, bad);
+                       out->sampleStart.p, (long long *)ctx->d_pinned, bad, ticket, out->meta.p,
+                         inMeta, boundRows, boundActive, slot);
   }
   SCN_HIP_CHECK(hipGetLastError());
-  SCN_TRY(read_scalars(ctx));
-  long long nSites = ctx->h_pinned[0], nOutActive = ctx->h_pinned[1];
+  long long nSites = boundRows, nOutActive = boundActive;
+  if (!deferred) {
+    SCN_TRY(read_scalars(ctx, ticket));
+    nSites = ctx->h_pinned[0];
+    nOutActive = ctx->h_pinned[1];
+    out->seenRows = nSites > out->seenRows ? nSites : out->seenRows;
+    out->seenActive = nOutActive > out->seenActive ? nOutActive : out->seenActive;
+  }
   SCN_REQUIRE(nSites < 2147483647ll, SCN_ERR_CAPACITY,
               "rules: %lld output rows do not fit 32-bit row numbers", nSites);
   // out->bg already holds what k_plan_samples wrote: grids_prepare only
   // reserves it (no reallocation at the same size) and clears table and mask
   SCN_TRY(grids_prepare(ctx, out, in->batch, g.d, g.nOut, nOutActive));
   out->nSites = (int)nSites;
+  if (deferred)
+    mark_pending(ctx, out, slot);
   SCN_TRY(out->siteKey.reserve((size_t)nSites + 1));
   long long nThreads = nE > in->batch ? nE : in->batch;
   if (nThreads > 0 && masked) {
     hipLaunchKernelGGL(k_plan_emit_masked<D>,
                        dim3(scn_ceil_div(nThreads, 256), (unsigned)maxCand),
                        dim3(256), 0, ctx->stream, vin, view_of(out), g,
-                       in->ekey.p, nE, out->base.p, out->ownMask.p,
+                       in->ekey.p, nEc, out->meta.p, out->base.p, out->ownMask.p,
                        out->rankOf.p, out->bgBefore.p, out->bg.p, out->ekey.p,
                        out->erow.p, out->siteKey.p);
     SCN_HIP_CHECK(hipGetLastError());
   } else if (nThreads > 0) {
     hipLaunchKernelGGL(k_plan_emit<D>, dim3(scn_ceil_div(nThreads, 256)),
                        dim3(256), 0, ctx->stream, vin, view_of(out), g,
-                       in->ekey.p, nE, out->base.p, out->bgBefore.p, out->bg.p,
+                       in->ekey.p, nEc, out->meta.p, out->base.p, out->bgBefore.p,
+                       out->bg.p,
                        out->ekey.p, out->erow.p, out->siteKey.p);
     SCN_HIP_CHECK(hipGetLastError());
   }
@@ -1133,16 +1366,30 @@ extern "C" int scn_rules_terminal_plan(scn_ctx *ctx, const scn_grids *cin,
   SCN_REQUIRE(in != out, SCN_ERR_ARG,
               "terminal rules plan: in and out are the same object");
   ProfScope ps(ctx, SCN_K_RULES);
+  const bool deferred = ctx->deferCounts && out->seenWidth > 0 &&
+                        (int)ctx->pendingGrids.size() < SCN_MAX_PENDING;
   SCN_TRY(ensure_rank(ctx, in));
   SCN_TRY(out->sampleStart.reserve((size_t)in->batch + 2));
+  SCN_TRY(out->meta.reserve(8));
+  const long long boundWidth =
+      deferred ? grow_bound(out->seenWidth, 8, in->vol) : 0x7FFFFFFFFFFFll;
+  const int slot = deferred ? (int)ctx->pendingGrids.size() : -1;
+  const long long ticket = ++ctx->ticket;
   hipLaunchKernelGGL(k_terminal_plan, dim3(1), dim3(1024), 0, ctx->stream,
                      view_of(in), out->sampleStart.p,
-                     (long long *)ctx->d_pinned);
+                     (long long *)ctx->d_pinned, ticket, out->meta.p,
+                     in->pending ? in->meta.p : nullptr, boundWidth, slot);
   SCN_HIP_CHECK(hipGetLastError());
-  SCN_TRY(read_scalars(ctx));
-  long long S = ctx->h_pinned[0];
+  long long S = boundWidth;
+  if (!deferred) {
+    SCN_TRY(read_scalars(ctx, ticket));
+    S = ctx->h_pinned[0];
+    out->seenWidth = S > out->seenWidth ? S : out->seenWidth;
+  }
   SCN_TRY(grids_prepare(ctx, out, in->batch, in->d, 1, in->batch));
   out->nSites = in->batch;
+  if (deferred)
+    mark_pending(ctx, out, slot);
   if (in->batch > 0) {
     hipLaunchKernelGGL(k_terminal_out, dim3(scn_ceil_div(in->batch, 256)),
                        dim3(256), 0, ctx->stream, view_of(out), out->ekey.p,
@@ -1182,13 +1429,14 @@ extern "C" int scn_rules_fill(scn_ctx *ctx, const scn_grids *in,
     SCN_REQUIRE(d_rules, SCN_ERR_ARG, "scn_rules_fill: null rules buffer");
     hipLaunchKernelGGL(k_terminal_init, dim3(scn_ceil_div(total, 256)),
                        dim3(256), 0, ctx->stream, vin, out->sampleStart.p,
-                       out->termS, d_rules);
+                       count_width(out), out->meta.p, d_rules);
     SCN_HIP_CHECK(hipGetLastError());
     if (in->nActive > 0) {
       hipLaunchKernelGGL(k_terminal_scatter,
                          dim3(scn_ceil_div(in->nActive, 256)), dim3(256), 0,
-                         ctx->stream, vin, in->ekey.p, in->erow.p, in->nActive,
-                         out->sampleStart.p, out->termS, d_rules);
+                         ctx->stream, vin, in->ekey.p, in->erow.p,
+                         count_active(in), out->sampleStart.p, count_width(out),
+                         out->meta.p, d_rules);
       SCN_HIP_CHECK(hipGetLastError());
     }
     return SCN_OK;
@@ -1207,15 +1455,18 @@ extern "C" int scn_rules_fill(scn_ctx *ctx, const scn_grids *in,
   switch (g.d) {
   case 1:
     hipLaunchKernelGGL(k_rules_fill<1>, grid, block, 0, ctx->stream, vin, g,
-                       out->siteKey.p, (long long)out->nSites, inv, d_rules);
+                       out->siteKey.p, count_sites(out), out->meta.p, inv,
+                       d_rules);
     break;
   case 2:
     hipLaunchKernelGGL(k_rules_fill<2>, grid, block, 0, ctx->stream, vin, g,
-                       out->siteKey.p, (long long)out->nSites, inv, d_rules);
+                       out->siteKey.p, count_sites(out), out->meta.p, inv,
+                       d_rules);
     break;
   default:
     hipLaunchKernelGGL(k_rules_fill<3>, grid, block, 0, ctx->stream, vin, g,
-                       out->siteKey.p, (long long)out->nSites, inv, d_rules);
+                       out->siteKey.p, count_sites(out), out->meta.p, inv,
+                       d_rules);
     break;
   }
   SCN_HIP_CHECK(hipGetLastError());

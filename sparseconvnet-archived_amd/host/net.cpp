@@ -189,6 +189,44 @@ static void clearDeviceGrids(scn_ctx *ctx, SpatiallySparseBatch &b) {
   if (!owned.empty())
     SCN_CHECKED(scn_grids_clear_many(ctx, owned.data(), (int)owned.size()));
 }
+// Every layer's rule book for the batch in slot b, on ctx's stream.  First with
+// deferred counts: no host round trip per layer, sizes are upper bounds until
+// one scn_rules_settle at the end, after which the real sizes are put in
+// place.  A batch that outgrows the bounds (or the first batch of a slot, which
+// has no bounds yet: its plans simply wait) is planned again the exact way.
+static void buildRuleBooks(SparseConvNetCUDA &cnn, scn_ctx *ctx,
+                           SpatiallySparseBatch &b) {
+  auto all = [&]() {
+    for (size_t i = 0; i < cnn.layers.size(); i++) {
+      scn_prof_tag(ctx, (int)i);
+      cnn.layers[i]->preprocess(b, b.interfaces[i], b.interfaces[i + 1]);
+    }
+  };
+  SCN_CHECKED(scn_ctx_defer_counts(ctx, 1));
+  all();
+  SCN_CHECKED(scn_ctx_defer_counts(ctx, 0));
+  const int rc = scn_rules_settle(ctx);
+  if (rc == SCN_ERR_CAPACITY) {
+    all(); // every plan empties its own output tables again
+    return;
+  }
+  SCN_CHECKED(rc);
+  // real sizes: a layer that owns its grids asks them, the others inherit
+  for (size_t i = 0; i < cnn.layers.size(); i++) {
+    SpatiallySparseBatchInterface &in = b.interfaces[i], &out = b.interfaces[i + 1];
+    if (out.ownsDeviceGrids && out.deviceGrids) {
+      int32_t nSites = 0;
+      int64_t width = 0;
+      SCN_CHECKED(scn_grids_info(out.deviceGrids, nullptr, nullptr, nullptr,
+                                 nullptr, &nSites));
+      SCN_CHECKED(scn_rules_width(out.deviceGrids, &width));
+      out.nSpatialSites = nSites;
+      out.rules.resize64((size_t)nSites * (size_t)width);
+    } else {
+      out.nSpatialSites = in.nSpatialSites;
+    }
+  }
+}
 void SparseConvNetCUDA::preprocessResident(int cc, const ResidentBatch &input) {
   SpatiallySparseBatch &b = batchPool[cc];
   scn_ctx *ctx = b.preprocessStream ? b.preprocessStream->ctx : memStream.ctx;
@@ -215,10 +253,7 @@ void SparseConvNetCUDA::preprocessResident(int cc, const ResidentBatch &input) {
   in.sub->features.resize64(nElems);
   SCN_CHECKED(scn_d2d(ctx, in.sub->features.dPtr(), input.d_features,
                       nElems * sizeof(float)));
-  for (size_t i = 0; i < layers.size(); i++) {
-    scn_prof_tag(ctx, (int)i);
-    layers[i]->preprocess(b, b.interfaces[i], b.interfaces[i + 1]);
-  }
+  buildRuleBooks(*this, ctx, b);
   SCN_CHECKED(scn_sync(ctx));
 }
 void SparseConvNetCUDA::setPrecision(int precision) {
@@ -554,10 +589,7 @@ void BatchProducer::preprocessBatchOnDevice(int cc) {
                               b.stagingRow.dPtr(), (int64_t)n,
                               b.stagingBackground.dPtr(), in.nSpatialSites));
   in.sub->features.copyToGPUAsync(ms);
-  for (size_t i = 0; i < cnn.layers.size(); i++) {
-    scn_prof_tag(ctx, (int)i);
-    cnn.layers[i]->preprocess(b, b.interfaces[i], b.interfaces[i + 1]);
-  }
+  buildRuleBooks(cnn, ctx, b);
   SCN_CHECKED(scn_sync(ctx));
 }
 void BatchProducer::batchProducerThread(int nThread) {

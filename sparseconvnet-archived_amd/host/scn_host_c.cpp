@@ -346,6 +346,20 @@ int scnh_forward_resident_stream(scnh_net *net, int nBatches, int batch,
   double t0 = now();
   while (SpatiallySparseBatch *b = bp.nextBatch()) {
     double t1 = now(); tNext += t1 - t0;
+    const char *mode = getenv("SCN_TMP_MODE");
+    if (mode && mode[0] == 'p') { t0 = now(); ++done; continue; } // producers only
+    if (mode && mode[0] == 'f') { // forward only: the same batch over and over
+      double ta = now();
+      for (int rep = 0; rep < 200; ++rep) { cnn->forwardBatch(*b); std::ofstream f, g; cnn->finishBatch(*b, f, g); b->predictions.clear(); b->probabilities.clear(); }
+      cnn->memStream.synchronize();
+      fprintf(stderr, "FWDONLY %.3f ms per forward (sync each)\n", (now() - ta) / 200);
+      ta = now();
+      for (int rep = 0; rep < 200; ++rep) { cnn->forwardBatch(*b); }
+      cnn->memStream.synchronize();
+      fprintf(stderr, "FWDONLY %.3f ms per forward (queued back to back)\n", (now() - ta) / 200);
+      std::ofstream f, g; cnn->finishBatch(*b, f, g);
+      exit(0);
+    }
     if (net->hasClassifier)
       cnn->forwardBatch(*b);
     else

@@ -142,6 +142,89 @@ def test_grids_reused_across_batches_with_one_clear(scn, ctx):
             og, cur = og2, d2
 
 
+def _chain(scn, ctx, dg, outs, term, samples, sizes, geoms):
+    """conv/pool chain + terminal layer into existing grids objects; returns what fill produced."""
+    got, cur = [], dg
+    for (size, stride), nIn, nOut, out in zip(geoms, sizes[:-1], sizes[1:], outs):
+        d2, d_rules, n, w = scn.rules_square(ctx, cur, nIn, nOut, size, stride, 1, out=out)
+        got.append((d2, d_rules, n, w))
+        cur = d2
+    S = cur.plan_terminal(term)
+    t_rules = ctx.empty(max(len(samples) * S, 1), np.int32)
+    cur.fill(term, t_rules, len(samples) * S)
+    got.append((term, t_rules, len(samples), S))
+    return got
+
+
+def test_deferred_counts(scn, ctx):
+    """scn_ctx_defer_counts / scn_rules_settle: a batch that fits the bounds of
+    the previous one is planned without waiting and gives the same rule books
+    and grids; a batch that outgrows them is reported and planned again."""
+    rng = np.random.default_rng(31)
+    sizes = [18, 17, 8, 7]
+    geoms = [(2, 1), (3, 2), (2, 1)]
+    dg = scn.Grids(ctx)
+    outs = [scn.Grids(ctx) for _ in geoms]
+    term = scn.Grids(ctx)
+
+    def oracle_chain(samples):
+        og, want = oracle_grids(samples), []
+        for (size, stride), nIn, nOut in zip(geoms, sizes[:-1], sizes[1:]):
+            og2, o_rules, o_n = orc.rules_square(og, 2, nIn, nOut, size, stride, 1)
+            want.append((og2, o_rules, o_n))
+            og = og2
+        o_out, o_rules, o_S = orc.rules_terminal(og)
+        want.append((o_out, o_rules, o_S))
+        return want
+
+    def check(got, want, batch):
+        for (dgr, d_rules, n, w), (ogr, o_rules, o_n) in zip(got[:-1], want[:-1]):
+            info = dgr.info()
+            assert info["nSpatialSites"] == o_n
+            assert np.array_equal(d_rules.download()[: o_n * w], o_rules)
+            assert_same_grids(dgr, ogr)
+        (dgr, d_rules, _, _), (ogr, o_rules, o_S) = got[-1], want[-1]
+        assert dgr.rules_width() == o_S
+        assert np.array_equal(d_rules.download()[: batch * o_S], o_rules)
+
+    def build(samples, nSites):
+        scn.clear_many(ctx, [dg] + outs + [term])
+        s, k, r, bg = flatten_samples(samples)
+        dg.build(len(samples), 2, sizes[0], s, k, r, bg, nSites)
+
+    # 1: exact (no history yet), establishes the bounds
+    samples, nSites = brute.random_samples(rng, 6, 2, sizes[0], 0.10)
+    build(samples, nSites)
+    check(_chain(scn, ctx, dg, outs, term, samples, sizes, geoms), oracle_chain(samples), 6)
+    # 2: deferred, a little smaller and a little larger than batch 1 (within the 25 % head room)
+    for density in (0.07, 0.11):
+        samples, nSites = brute.random_samples(rng, 6, 2, sizes[0], density)
+        build(samples, nSites)
+        scn.defer_counts(ctx, True)
+        got = _chain(scn, ctx, dg, outs, term, samples, sizes, geoms)
+        with pytest.raises(scn.ScnError):
+            got[0][0].info()  # not readable before the counts are settled
+        scn.defer_counts(ctx, False)
+        assert scn.settle(ctx)
+        check(got, oracle_chain(samples), 6)
+    # 3: deferred, far denser: outgrows the bounds, is reported, and planned again the exact way
+    samples, nSites = brute.random_samples(rng, 6, 2, sizes[0], 0.6)
+    build(samples, nSites)
+    scn.defer_counts(ctx, True)
+    _chain(scn, ctx, dg, outs, term, samples, sizes, geoms)
+    scn.defer_counts(ctx, False)
+    assert not scn.settle(ctx)
+    check(_chain(scn, ctx, dg, outs, term, samples, sizes, geoms), oracle_chain(samples), 6)
+    # 4: and the raised bounds now hold for a batch of that size
+    samples, nSites = brute.random_samples(rng, 6, 2, sizes[0], 0.55)
+    build(samples, nSites)
+    scn.defer_counts(ctx, True)
+    got = _chain(scn, ctx, dg, outs, term, samples, sizes, geoms)
+    scn.defer_counts(ctx, False)
+    assert scn.settle(ctx)
+    check(got, oracle_chain(samples), 6)
+
+
 def test_larger_3d_batch(scn, ctx):
     rng = np.random.default_rng(12)
     nOut, size, stride = 22, 3, 1
