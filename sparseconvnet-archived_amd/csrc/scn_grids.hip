@@ -415,9 +415,10 @@ plan_samples_body(const GridView &in, const unsigned *base, long long nEntries,
                   const long long *badSites, long long ticket,
                   long long *meta, const long long *inMeta, long long boundRows,
                   long long boundActive, int pinnedSlot) {
-  __shared__ int lds[1024];
+  __shared__ int waveSum[17];
   __shared__ int carry;
   const int t = threadIdx.x;
+  const int lane = t & 63, wave = t >> 6;
   if (t == 0)
     carry = 0;
   __syncthreads();
@@ -432,22 +433,41 @@ plan_samples_body(const GridView &in, const unsigned *base, long long nEntries,
       long long oc = (long long)base[re] - (long long)base[rs];
       notFull = oc < fullSize;
     }
-    lds[t] = notFull;
-    __syncthreads();
-    for (int off = 1; off < 1024; off <<= 1) {
-      int add = (t >= off) ? lds[t - off] : 0;
-      __syncthreads();
-      lds[t] += add;
-      __syncthreads();
+    // prefix of notFull over the 1024 lanes: shuffles inside a wavefront, the
+    // 16 wavefront totals through LDS (two barriers instead of thirty)
+    int incl = notFull;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      int up = __shfl_up(incl, off, 64);
+      if (lane >= off)
+        incl += up;
     }
-    int excl = lds[t] - notFull + carry;
+    if (lane == 63)
+      waveSum[wave] = incl;
+    __syncthreads();
+    if (wave == 0) {
+      int w = lane < 16 ? waveSum[lane] : 0;
+      int wi = w;
+#pragma unroll
+      for (int off = 1; off < 16; off <<= 1) {
+        int up = __shfl_up(wi, off, 64);
+        if (lane >= off)
+          wi += up;
+      }
+      if (lane < 16)
+        waveSum[lane] = wi - w;
+      if (lane == 15)
+        waveSum[16] = wi;
+    }
+    __syncthreads();
+    int excl = waveSum[wave] + incl - notFull + carry;
     if (b < in.batch) {
       bgBefore[b] = excl;
       outBg[b] = notFull ? (int)base[re] + excl : -1;
     }
     __syncthreads();
-    if (t == 1023)
-      carry += lds[1023];
+    if (t == 0)
+      carry += waveSum[16];
     __syncthreads();
   }
   if (t == 0) {
@@ -567,11 +587,12 @@ __global__ void k_plan_emit_masked(GridView in, GridView out, Geom g,
   }
   if (e >= count_now(nEntries))
     return;
-  unsigned long long mask = ownMask[e];
+  // all three at once: one memory latency instead of two in a row
+  const unsigned long long mask = ownMask[e];
+  const long long p = ekey[e];
+  const unsigned r = rankOf[e];
   if (!((mask >> c) & 1ull))
     return;
-  long long p = ekey[e];
-  unsigned r = rankOf[e];
   int b = (int)(p / g.volIn);
   int i[D], lo[D], hi[D], j[D];
   decode_key<D>(p - (long long)b * g.volIn, g.nIn, i);

@@ -1,8 +1,6 @@
 // C view of the host classes (see scn_host_c.h).
 #include "scn_host_c.h"
-#include <time.h>
-#include <stdlib.h>
-#include <stdio.h>
+
 #include <cstdio>
 #include <cstdlib>
 #include <memory>
@@ -341,33 +339,13 @@ int scnh_forward_resident_stream(scnh_net *net, int nBatches, int batch,
     }
     ++done;
   };
-  double tNext = 0, tFwd = 0, tFin = 0;
-  auto now = [] { timespec ts; clock_gettime(CLOCK_MONOTONIC, &ts); return ts.tv_sec * 1e3 + ts.tv_nsec * 1e-6; };
-  double t0 = now();
   while (SpatiallySparseBatch *b = bp.nextBatch()) {
-    double t1 = now(); tNext += t1 - t0;
-    const char *mode = getenv("SCN_TMP_MODE");
-    if (mode && mode[0] == 'p') { t0 = now(); ++done; continue; } // producers only
-    if (mode && mode[0] == 'f') { // forward only: the same batch over and over
-      double ta = now();
-      for (int rep = 0; rep < 200; ++rep) { cnn->forwardBatch(*b); std::ofstream f, g; cnn->finishBatch(*b, f, g); b->predictions.clear(); b->probabilities.clear(); }
-      cnn->memStream.synchronize();
-      fprintf(stderr, "FWDONLY %.3f ms per forward (sync each)\n", (now() - ta) / 200);
-      ta = now();
-      for (int rep = 0; rep < 200; ++rep) { cnn->forwardBatch(*b); }
-      cnn->memStream.synchronize();
-      fprintf(stderr, "FWDONLY %.3f ms per forward (queued back to back)\n", (now() - ta) / 200);
-      std::ofstream f, g; cnn->finishBatch(*b, f, g);
-      exit(0);
-    }
     if (net->hasClassifier)
       cnn->forwardBatch(*b);
     else
       forward_layers(net, *b);
-    double t2 = now(); tFwd += t2 - t1;
     if (queued)
       finish(queued);
-    t0 = now(); tFin += t0 - t2;
     queued = b;
     if (!bp.keepAlive) {
       finish(queued);
@@ -377,8 +355,6 @@ int scnh_forward_resident_stream(scnh_net *net, int nBatches, int batch,
   if (queued)
     finish(queued);
   cnn->memStream.synchronize();
-  if (getenv("SCN_TIMING_TMP"))
-    fprintf(stderr, "TIMING per batch: nextBatch %.3f ms, forwardBatch (launch) %.3f ms, finish %.3f ms\n", tNext / nBatches, tFwd / nBatches, tFin / nBatches);
   net->batch = nullptr;
   return done;
 }
