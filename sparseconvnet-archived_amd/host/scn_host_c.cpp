@@ -1,5 +1,6 @@
 // C view of the host classes (see scn_host_c.h).
 #include "scn_host_c.h"
+#include "Off3DFormatPicture.h"
 
 #include <cstdio>
 #include <cstdlib>
@@ -175,6 +176,50 @@ void scnh_dataset_add_points(scnh_dataset *ds, int dimension, int latticeSize,
   p->coords.assign(coords, coords + nSites * dimension);
   p->features.assign(features, features + nSites * ds->ds.nFeatures);
   ds->ds.pictures.push_back(p);
+}
+int scnh_dataset_add_off_file(scnh_dataset *ds, const char *path, int renderSize,
+                              int label) {
+  auto *p = new OffSurfaceModelPicture(path, renderSize, label);
+  if (!p->loaded) {
+    delete p;
+    return -1;
+  }
+  ds->ds.pictures.push_back(p);
+  return 0;
+}
+void scnh_dataset_add_mesh(scnh_dataset *ds, int64_t nPoints,
+                           const double *points, int64_t nTriangles,
+                           const int32_t *triangles, int renderSize,
+                           int label) {
+  ds->ds.pictures.push_back(new OffSurfaceModelPicture(
+      points, (int)nPoints, triangles, (int)nTriangles, renderSize, label));
+}
+int64_t scnh_codify_picture(scnh_dataset *ds, int64_t index, int spatialSize,
+                            int64_t seed, int64_t capacity, int64_t *keys,
+                            int32_t *rows, int32_t *backgroundRow,
+                            float *features) {
+  Picture *original = ds->ds.pictures.at((size_t)index);
+  Picture *pic = original;
+  if (seed >= 0) {
+    RNG rng((unsigned)seed);
+    pic = original->distort(rng, ds->ds.type);
+  }
+  SparseGrid grid;
+  std::vector<float> f;
+  int n = 0;
+  pic->codifyInputData(grid, f, n, spatialSize);
+  if (pic != original)
+    delete pic;
+  if (n <= capacity) {
+    size_t k = 0;
+    for (auto &e : grid.mp.entries()) {
+      keys[k] = e.first;
+      rows[k++] = e.second;
+    }
+    *backgroundRow = grid.backgroundCol;
+    std::copy(f.begin(), f.end(), features);
+  }
+  return n;
 }
 int64_t scnh_dataset_size(scnh_dataset *ds) {
   return (int64_t)ds->ds.pictures.size();

@@ -47,6 +47,23 @@ void scnh_dataset_add_points(scnh_dataset *ds, int dimension, int latticeSize,
                              int64_t nSites, const int32_t *coords,
                              const float *features, int label);
 int64_t scnh_dataset_size(scnh_dataset *ds);
+/* OffSurfaceModelPicture (Off3DFormatPicture.h): from an OFF file (returns -1
+ * when it cannot be read) or from arrays (points: nPoints x 3 doubles,
+ * triangles: nTriangles x 3 vertex indices).  The dataset needs nFeatures 1. */
+int scnh_dataset_add_off_file(scnh_dataset *ds, const char *path, int renderSize,
+                              int label);
+void scnh_dataset_add_mesh(scnh_dataset *ds, int64_t nPoints,
+                           const double *points, int64_t nTriangles,
+                           const int32_t *triangles, int renderSize, int label);
+/* Picture::distort (when seed >= 0, with RNG(seed) and the dataset's batch
+ * type) followed by Picture::codifyInputData into an empty grid, on the CPU.
+ * Returns the number of rows (background row included); when that fits
+ * `capacity`, writes key / row of every site in insertion order, the
+ * background row and the rows x nFeatures feature matrix. */
+int64_t scnh_codify_picture(scnh_dataset *ds, int64_t index, int spatialSize,
+                            int64_t seed, int64_t capacity, int64_t *keys,
+                            int32_t *rows, int32_t *backgroundRow,
+                            float *features);
 
 /* SparseConvNet::processDataset / processDatasetRepeatTest */
 float scnh_process_dataset(scnh_net *net, scnh_dataset *ds, int batchSize);

@@ -52,6 +52,9 @@ def lib():
         "scnh_dataset_destroy": (None, [vp]),
         "scnh_dataset_add_points": (None, [vp, i32, i32, i64, vp, vp, i32]),
         "scnh_dataset_size": (i64, [vp]),
+        "scnh_dataset_add_off_file": (i32, [vp, C.c_char_p, i32, i32]),
+        "scnh_dataset_add_mesh": (None, [vp, i64, vp, i64, vp, i32, i32]),
+        "scnh_codify_picture": (i64, [vp, i64, i32, i64, i64, vp, vp, vp, vp]),
         "scnh_process_dataset": (f32, [vp, vp, i32]),
         "scnh_process_dataset_repeat_test": (None, [vp, vp, i32, i32]),
         "scnh_begin": (None, [vp, vp, i32]),
@@ -94,6 +97,30 @@ class Dataset:
         coords = np.ascontiguousarray(coords, np.int32).reshape(-1, dimension)
         features = np.ascontiguousarray(features, np.float32).reshape(coords.shape[0], self.nFeatures)
         lib().scnh_dataset_add_points(self.h, dimension, latticeSize, coords.shape[0], _p(coords), _p(features), label)
+
+    def add_off_file(self, path, renderSize, label=-1):
+        """OffSurfaceModelPicture from an OFF file."""
+        if lib().scnh_dataset_add_off_file(self.h, str(path).encode(), renderSize, label) != 0:
+            raise IOError("%s is not a readable OFF mesh" % path)
+
+    def add_mesh(self, points, triangles, renderSize, label=-1):
+        """OffSurfaceModelPicture from arrays (points n x 3, triangles m x 3)."""
+        points = np.ascontiguousarray(points, np.float64).reshape(-1, 3)
+        triangles = np.ascontiguousarray(triangles, np.int32).reshape(-1, 3)
+        lib().scnh_dataset_add_mesh(self.h, len(points), _p(points), len(triangles), _p(triangles), renderSize, label)
+
+    def codify(self, index, spatialSize, seed=-1):
+        """distort (seed >= 0) + codifyInputData of one picture on the CPU:
+        (keys, rows in insertion order, background row, features [rows x nFeatures])."""
+        cap = 1 << 12
+        while True:
+            keys, rows = np.empty(cap, np.int64), np.empty(cap, np.int32)
+            bg = C.c_int32()
+            feats = np.empty((cap, self.nFeatures), np.float32)
+            n = lib().scnh_codify_picture(self.h, index, spatialSize, seed, cap, _p(keys), _p(rows), C.byref(bg), _p(feats))
+            if n <= cap:
+                return keys[:n - 1].copy(), rows[:n - 1].copy(), bg.value, feats[:n].copy()
+            cap = int(n)
 
     def __len__(self):
         return lib().scnh_dataset_size(self.h)
