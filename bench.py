@@ -36,15 +36,15 @@ MEASURED_TRAFFIC = {
     ("c2_sparse_net_2d", "gather", 0): 2.66e6 + 4.01e6,
     ("c2_sparse_net_2d", "nin", 1): 4.16e6 + 10.70e6,
     ("c2_sparse_net_2d", "maxpool", 2): 14.57e6 + 10.77e6,
-    ("c2_sparse_net_2d", "conv_nin", 4): 17.44e6 + 15.48e6,
+    ("c2_sparse_net_2d", "conv_nin", 4): 11.64e6 + 15.48e6,
     ("c2_sparse_net_2d", "maxpool", 5): 22.67e6 + 11.76e6,
-    ("c2_sparse_net_2d", "conv_nin", 7): 15.49e6 + 11.46e6,
+    ("c2_sparse_net_2d", "conv_nin", 7): 12.65e6 + 11.46e6,
     ("c2_sparse_net_2d", "maxpool", 8): 17.42e6 + 8.01e6,
-    ("c2_sparse_net_2d", "conv_nin", 10): 15.87e6 + 5.98e6,
+    ("c2_sparse_net_2d", "conv_nin", 10): 14.74e6 + 5.98e6,
     ("c2_sparse_net_2d", "maxpool", 11): 8.42e6 + 3.35e6,
-    ("c2_sparse_net_2d", "conv_nin", 13): 16.47e6 + 1.58e6,
+    ("c2_sparse_net_2d", "conv_nin", 13): 16.45e6 + 1.58e6,
     ("c2_sparse_net_2d", "maxpool", 14): 1.79e6 + 0.51e6,
-    ("c2_sparse_net_2d", "nin", 15): 2.63e6 + 0.31e6,
+    ("c2_sparse_net_2d", "nin", 15): 2.65e6 + 0.31e6,
     ("c2_sparse_net_2d", "nin", 17): 0.47e6 + 0.04e6,
     ("c5_spatiotemporal_3d", "conv_nin", 1): 651.74e6 + 845.62e6,
     ("c5_spatiotemporal_3d", "conv_nin", 3): 1538.63e6 + 1614.81e6,
@@ -368,11 +368,32 @@ def cpu_leg(cfg, layers, weights, samples, spatialSize, budget_s):
             cur, _, _ = orc.rules_terminal(cur)
     rules_only = time.perf_counter() - t0
     orc.set_threads(1)
+    # the same with T producer-style threads, one batch slot each (BatchProducer.cu:90-106 runs up to 10)
+    import threading
+    T = min(10, cores)
+
+    def one_slot():
+        cur = orc.Grids.from_flat(len(sub), S, K, R, bg)
+        for l in ora.layers:
+            if l["kind"] in ("conv", "maxpool"):
+                cur, _, _ = orc.rules_square(cur, cfg.dimension, l["inSize"], l["outSize"], l["size"], l["stride"],
+                                             l.get("minActive", 1))
+            elif l["kind"] == "terminal":
+                cur, _, _ = orc.rules_terminal(cur)
+
+    threads = [threading.Thread(target=one_slot) for _ in range(T)]
+    t0 = time.perf_counter()
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    rules_T = time.perf_counter() - t0
     return {"value": len(K) / full, "unit": "active sites/s", "cores": cores, "kind": "port",
             "sample": "%s, %d of %d samples, %d passes, median" % (cfg.name, len(sub), len(samples), len(times)),
             "ms_per_batch": 1e3 * full, "samples_per_s": len(sub) / full,
             "rulebooks_only_1_thread_ms": 1e3 * rules_only,
-            "rulebooks_only_active_sites_per_s": len(K) / rules_only}
+            "rulebooks_only_active_sites_per_s": len(K) / rules_only,
+            "rulebooks_only_threads": T, "rulebooks_only_T_threads_active_sites_per_s": T * len(K) / rules_T}
 
 
 if __name__ == "__main__":
