@@ -141,6 +141,130 @@ struct GatherSource {
 };
 
 
+// ---- few rows: split-k FMA kernel --------------------------------------------
+// The classifier head and the deepest layers of small batches have a few
+// hundred rows: tiles would leave most of the chip idle and run a long k-loop
+// in a handful of workgroups.  Here a workgroup owns FR_ROWS rows x 64 columns
+// and its four wavefronts split K between them: a lane owns one column, loads
+// its quarter of that column of W with FR_DEPTH loads in flight (W is small
+// and served by the caches) and multiplies it with the rows of A staged in LDS
+// (gathered through the rules if asked); the four partial sums meet in LDS.
+#define FR_ROWS 8
+#define FR_DEPTH 24
+#define FR_MAX_M 512
+#define FR_MAX_K 1024
+__global__ void __launch_bounds__(256)
+    k_nin_fewrows(const float *__restrict__ A, const float *__restrict__ W,
+                  float *__restrict__ out, long long M, int K, int N,
+                  Epilogue ep, GatherSource gs, bool gather) {
+  __shared__ float sA[FR_ROWS * FR_MAX_K];
+  __shared__ float part[4][FR_ROWS][64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const long long m0 = (long long)blockIdx.x * FR_ROWS;
+  const int n = blockIdx.y * 64 + lane;
+  for (int x = tid; x < FR_ROWS * K; x += 256) {
+    const int r = x / K, k = x - r * K;
+    const long long m = m0 + r;
+    float v = 0.f;
+    if (m < M) {
+      if (gather) {
+        const int f = k / gs.nIn;
+        const int rule = gs.rules[m * gs.fs + f];
+        if (rule >= 0)
+          v = A[(long long)rule * gs.nIn + (k - f * gs.nIn)];
+      } else {
+        v = A[m * K + k];
+      }
+    }
+    sA[x] = v;
+  }
+  __syncthreads();
+  // this wavefront's share of K
+  const int per = (K + 3) / 4;
+  const int k0 = wave * per, k1 = min(K, k0 + per);
+  float acc[FR_ROWS];
+#pragma unroll
+  for (int r = 0; r < FR_ROWS; ++r)
+    acc[r] = 0.f;
+  const bool col = n < N;
+  const float *w = W + (col ? n : 0);
+  for (int k = k0; k < k1; k += FR_DEPTH) {
+    float wv[FR_DEPTH];
+#pragma unroll
+    for (int i = 0; i < FR_DEPTH; ++i) {
+      const int kk = k + i < k1 ? k + i : k1 - 1; // clamped, the product is dropped below
+      wv[i] = w[(long long)kk * N];
+    }
+#pragma unroll
+    for (int i = 0; i < FR_DEPTH; ++i)
+      if (k + i < k1) {
+#pragma unroll
+        for (int r = 0; r < FR_ROWS; ++r)
+          acc[r] = fmaf(sA[r * K + k + i], wv[i], acc[r]);
+      }
+  }
+#pragma unroll
+  for (int r = 0; r < FR_ROWS; ++r)
+    part[wave][r][lane] = acc[r];
+  __syncthreads();
+  // 512 sums, two per lane, always added in wavefront order
+  for (int x = tid; x < FR_ROWS * 64; x += 256) {
+    const int r = x >> 6, c = x & 63;
+    const long long m = m0 + r;
+    const int nn = blockIdx.y * 64 + c;
+    if (m < M && nn < N) {
+      const float v = ((part[0][r][c] + part[1][r][c]) + part[2][r][c]) + part[3][r][c];
+      out[m * N + nn] = apply_act(v, nn, ep);
+    }
+  }
+}
+
+// ---- few input channels: one lane per four outputs ------------------------
+// The first NiN layer of a net multiplies a tall matrix by a tiny W (K = 3 fs
+// or so): bandwidth only.  W sits in LDS; a lane reads its row of A (16-byte
+// loads, shared by the eight lanes of the row through the cache) and writes
+// four adjacent outputs.
+#define TK_MAX_K 32
+__global__ void __launch_bounds__(256)
+    k_nin_thin(const float *__restrict__ A, const float *__restrict__ W,
+               float *__restrict__ out, long long M, int K, int N, Epilogue ep) {
+  __shared__ __attribute__((aligned(16))) float sW[TK_MAX_K * 32];
+  const int tid = threadIdx.x;
+  const int n0 = blockIdx.y * 32;
+  for (int x = tid; x < K * 32; x += 256) {
+    const int k = x >> 5, c = x & 31;
+    sW[x] = n0 + c < N ? W[(long long)k * N + n0 + c] : 0.f;
+  }
+  __syncthreads();
+  const long long m = (long long)blockIdx.x * 32 + (tid >> 3);
+  const int c4 = (tid & 7) * 4;
+  if (m >= M)
+    return;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  const float4 *arow = reinterpret_cast<const float4 *>(A + m * K);
+  for (int k4 = 0; k4 < K / 4; ++k4) { // K % 4 == 0
+    const float4 a = arow[k4];
+    const float av[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float4 wv = *reinterpret_cast<const float4 *>(&sW[(4 * k4 + i) * 32 + c4]);
+      acc.x = fmaf(av[i], wv.x, acc.x);
+      acc.y = fmaf(av[i], wv.y, acc.y);
+      acc.z = fmaf(av[i], wv.z, acc.z);
+      acc.w = fmaf(av[i], wv.w, acc.w);
+    }
+  }
+  const int n = n0 + c4;
+  if (n < N) { // N % 4 == 0: the four columns are in or out together
+    float4 r;
+    r.x = apply_act(acc.x, n, ep);
+    r.y = apply_act(acc.y, n + 1, ep);
+    r.z = apply_act(acc.z, n + 2, ep);
+    r.w = apply_act(acc.w, n + 3, ep);
+    *reinterpret_cast<float4 *>(out + m * N + n) = r;
+  }
+}
+
 // ---- MFMA path: fp32 operands, v_mfma_f32_32x32x2_f32 ----------------------
 // Block = 4 wavefronts laid out WM x WN; every wavefront owns a 32 x (32 NT)
 // patch of the output as NT accumulator tiles of 32x32 (16 VGPRs per lane
@@ -925,6 +1049,17 @@ static int nin_forward(scn_ctx *ctx, const float *d_A, const float *d_W,
       launch_mfma_bf16<4, 1, 2>(ctx, d_A, d_W, d_out, M, K, N, ep, split);
     else
       launch_mfma_bf16<1, 4, 1>(ctx, d_A, d_W, d_out, M, K, N, ep, split);
+  } else if (M <= FR_MAX_M && K <= FR_MAX_K && !(vec && K % 32 == 0 && N % 16 == 0)) {
+    // (shapes the W-resident kernel takes are faster there)
+    GatherSource none = GatherSource();
+    hipLaunchKernelGGL(k_nin_fewrows,
+                       dim3(scn_ceil_div(M, FR_ROWS), scn_ceil_div(N, 64)),
+                       dim3(256), 0, ctx->stream, d_A, d_W, d_out, (long long)M,
+                       K, N, ep, gs ? *gs : none, gs != nullptr);
+  } else if (vec && !gs && K <= TK_MAX_K) {
+    hipLaunchKernelGGL(k_nin_thin, dim3(scn_ceil_div(M, 32), scn_ceil_div(N, 32)),
+                       dim3(256), 0, ctx->stream, d_A, d_W, d_out, (long long)M,
+                       K, N, ep);
   } else if (vec && wres_forward(ctx, d_A, d_W, d_out, M, K, N, ep, gs)) {
     // W-resident kernel took it
   } else if ((vec && K >= 8) || gs) {

@@ -79,7 +79,9 @@ SHAPES = [(1000, 12, 32), (777, 128, 64), (513, 256, 96), (300, 384, 128), (129,
           # enough 16-row panels that wavefronts of the W-resident kernel walk several, last one ragged
           (70001, 128, 64), (40003, 256, 96),
           # W-resident kernel: an odd number of prefetch groups, a 48-column slice, many narrow slices
-          (600, 160, 192), (1000, 64, 48), (2469, 512, 160)]
+          (600, 160, 192), (1000, 64, 48), (2469, 512, 160),
+          # few rows (split-k kernel): ragged row and column blocks; few input channels (thin kernel)
+          (3, 40, 100), (511, 1024, 36), (83, 9, 5), (5000, 12, 32), (4097, 28, 100)]
 
 
 @pytest.mark.parametrize("M,K,N", SHAPES)
