@@ -614,6 +614,58 @@ __global__ void k_plan_emit_masked(GridView in, GridView out, Geom g,
   siteKey[row] = po;
 }
 
+// The same with one lane per input walking the set bits of its ownership
+// mask: for boxes of many candidates (3-D: 27) of which an input owns a few,
+// where a lane per (input, candidate) would mostly read masks and leave.
+template <int D>
+__global__ void k_plan_emit_walk(GridView in, GridView out, Geom g,
+                                 const long long *ekey, Count nEntries,
+                                 const long long *outMeta, const unsigned *base,
+                                 const unsigned long long *ownMask,
+                                 const unsigned *rankOf, const int *bgBefore,
+                                 const int *outBg, long long *okey, int *orow,
+                                 long long *siteKey) {
+  long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (outMeta[META_OVERFLOW])
+    return; // the bounds did not hold: nothing may be written
+  if (e < in.batch) { // background rows
+    int r = outBg[e];
+    if (r >= 0)
+      siteKey[r] = -1 - e;
+  }
+  if (e >= count_now(nEntries))
+    return;
+  unsigned long long mask = ownMask[e];
+  const long long p = ekey[e];
+  const unsigned r = rankOf[e];
+  if (mask == 0)
+    return;
+  const int b = (int)(p / g.volIn);
+  int i[D], lo[D], hi[D], j[D];
+  decode_key<D>(p - (long long)b * g.volIn, g.nIn, i);
+  (void)cand_box<D>(g, i, lo, hi);
+  unsigned idx = base[r];
+  const int shiftRows = bgBefore[b];
+  while (mask) { // ascending candidate = ascending output key
+    int rem = __ffsll((long long)mask) - 1;
+    mask &= mask - 1;
+#pragma unroll
+    for (int a = D - 1; a >= 0; --a) {
+      int ext = hi[a] - lo[a];
+      j[a] = lo[a] + rem % ext;
+      rem /= ext;
+    }
+    const long long po = (long long)b * g.volOut + encode_key<D>(j, g.nOut);
+    const int row = (int)idx + shiftRows;
+    hash_insert(out.table, out.shift, out.mask, po, row);
+    atomicOr(&out.bits[po >> 6], 1ull << (po & 63));
+    okey[idx] = po;
+    orow[idx] = row;
+    siteKey[row] = po;
+    ++idx;
+  }
+}
+
 // clears a hash table (all-ones = empty slots) and an occupancy mask at once
 __global__ void k_clear_grid(uint4 *slots, size_t nSlots,
                              unsigned long long *bits, size_t nWords) {
@@ -678,6 +730,47 @@ __global__ void k_rules_fill(GridView in, Geom g, const long long *siteKey,
   else
     val = in.bg[b];
   rules[idx] = val;
+}
+
+// Square windows: one lane per run of `size` rule entries along the innermost
+// axis.  Their input sites are neighbours in the mask, so one mask read serves
+// the whole run (a lane per entry reads a 64-byte line of the mask for every
+// entry, and that line traffic is what bounds the kernel on 3-D batches).
+template <int D>
+__global__ void k_rules_fill_runs(GridView in, Geom g, const long long *siteKey,
+                                  Count nSites, const long long *outMeta,
+                                  int *rules) {
+  long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (outMeta[META_OVERFLOW])
+    return;
+  const int runsPerRow = g.width / g.size;
+  if (idx >= count_now(nSites) * runsPerRow)
+    return;
+  const long long r = idx / runsPerRow;
+  int run = (int)(idx - r * runsPerRow);
+  int *dst = rules + r * g.width + (long long)run * g.size;
+  const long long sk = siteKey[r];
+  if (sk < 0) { // all-background row (Regions.cu:647-652)
+    const int v = in.bg[-1 - sk];
+    for (int t = 0; t < g.size; ++t)
+      dst[t] = v;
+    return;
+  }
+  const int b = (int)(sk / g.volOut);
+  int j[D], c[D];
+  decode_key<D>(sk - (long long)b * g.volOut, g.nOut, j);
+  c[D - 1] = j[D - 1] * g.stride;
+#pragma unroll
+  for (int a = D - 2; a >= 0; --a) {
+    c[a] = j[a] * g.stride + run % g.size;
+    run /= g.size;
+  }
+  const long long p0 = (long long)b * g.volIn + encode_key<D>(c, g.nIn);
+  const unsigned present = get_bits(in.bits, p0, g.size);
+  const int bgRow = in.bg[b];
+  for (int t = 0; t < g.size; ++t)
+    dst[t] = (present >> t) & 1u ? hash_find(in.table, in.shift, in.mask, p0 + t)
+                                 : bgRow;
 }
 
 // terminal pooling: sample sizes and their maximum.  One block.
@@ -1267,7 +1360,14 @@ static int plan_regions_d(scn_ctx *ctx, scn_grids *in, scn_grids *out,
     mark_pending(ctx, out, slot);
   SCN_TRY(out->siteKey.reserve((size_t)nSites + 1));
   long long nThreads = nE > in->batch ? nE : in->batch;
-  if (nThreads > 0 && masked) {
+  if (nThreads > 0 && masked && maxCand > 9) {
+    hipLaunchKernelGGL(k_plan_emit_walk<D>, dim3(scn_ceil_div(nThreads, 256)),
+                       dim3(256), 0, ctx->stream, vin, view_of(out), g,
+                       in->ekey.p, nEc, out->meta.p, out->base.p, out->ownMask.p,
+                       out->rankOf.p, out->bgBefore.p, out->bg.p, out->ekey.p,
+                       out->erow.p, out->siteKey.p);
+    SCN_HIP_CHECK(hipGetLastError());
+  } else if (nThreads > 0 && masked) {
     hipLaunchKernelGGL(k_plan_emit_masked<D>,
                        dim3(scn_ceil_div(nThreads, 256), (unsigned)maxCand),
                        dim3(256), 0, ctx->stream, vin, view_of(out), g,
@@ -1473,6 +1573,28 @@ extern "C" int scn_rules_fill(scn_ctx *ctx, const scn_grids *in,
   const bool tri = g.mode == MODE_TRI_NOMIN || g.mode == MODE_TRI_MIN;
   const int *inv = tri ? out->invOrd.p : nullptr;
   dim3 grid(scn_ceil_div(total, 256)), block(256);
+  if (!tri && g.size >= 2) {
+    dim3 runs(scn_ceil_div(total / g.size, 256));
+    switch (g.d) {
+    case 1:
+      hipLaunchKernelGGL(k_rules_fill_runs<1>, runs, block, 0, ctx->stream, vin,
+                         g, out->siteKey.p, count_sites(out), out->meta.p,
+                         d_rules);
+      break;
+    case 2:
+      hipLaunchKernelGGL(k_rules_fill_runs<2>, runs, block, 0, ctx->stream, vin,
+                         g, out->siteKey.p, count_sites(out), out->meta.p,
+                         d_rules);
+      break;
+    default:
+      hipLaunchKernelGGL(k_rules_fill_runs<3>, runs, block, 0, ctx->stream, vin,
+                         g, out->siteKey.p, count_sites(out), out->meta.p,
+                         d_rules);
+      break;
+    }
+    SCN_HIP_CHECK(hipGetLastError());
+    return SCN_OK;
+  }
   switch (g.d) {
   case 1:
     hipLaunchKernelGGL(k_rules_fill<1>, grid, block, 0, ctx->stream, vin, g,

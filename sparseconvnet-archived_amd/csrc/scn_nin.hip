@@ -321,38 +321,51 @@ __global__ void __launch_bounds__(256)
     __syncthreads();
   }
 
+  // Slab loads are unconditional: addresses are clamped into the operands and
+  // what lies outside is replaced by zero afterwards, so that the loads sit in
+  // one basic block with the MFMAs around them and the compiler can count them.
   float4 ra[A_PER], rw[W_PER];
+  const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
   auto load_slab = [&](int k0) {
+    const float *src[A_PER];
+    bool inside[A_PER];
 #pragma unroll
     for (int u = 0; u < A_PER; ++u) {
       int c = tid + u * 256;
-      int r = c / (BK / 4), kc = c % (BK / 4);
-      long long m = m0 + r;
-      int k = k0 + kc * 4;
-      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (c < A_CHUNKS && m < M && k < K) { // K % 4 == 0: a chunk is all in or all out
-        if (GATHER) {
-          int q = k / gs.nIn;
-          int rule = sR[r * gs.fs + q];
-          if (rule >= 0)
-            v = *reinterpret_cast<const float4 *>(
-                A + (long long)rule * gs.nIn + (k - q * gs.nIn));
-        } else {
-          v = *reinterpret_cast<const float4 *>(A + m * K + k);
-        }
+      c = c < A_CHUNKS ? c : A_CHUNKS - 1;
+      const int r = c / (BK / 4), kc = c % (BK / 4);
+      const long long m = m0 + r;
+      const int k = k0 + kc * 4;
+      const int kIn = k < K ? k : K - 4; // K % 4 == 0: a chunk is all in or all out
+      inside[u] = k < K && m < M;
+      if (GATHER) {
+        const int q = (int)__umulhi((unsigned)kIn, gs.magic); // kIn / nIn
+        const int rule = sR[r * gs.fs + q]; // -1 for rows past M
+        src[u] = (rule >= 0 ? A + (long long)rule * gs.nIn : gs.zeros) +
+                 (kIn - q * gs.nIn);
+      } else {
+        src[u] = A + (m < M ? m : M - 1) * K + kIn;
       }
-      ra[u] = v;
     }
+#pragma unroll
+    for (int u = 0; u < A_PER; ++u)
+      ra[u] = *reinterpret_cast<const float4 *>(src[u]);
 #pragma unroll
     for (int u = 0; u < W_PER; ++u) {
       int c = tid + u * 256;
-      int kk = c / (BN / 4), nc = c % (BN / 4);
-      int k = k0 + kk, n = n0 + nc * 4;
-      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (c < W_CHUNKS && k < K && n < N) // N % 4 == 0
-        v = *reinterpret_cast<const float4 *>(W + (long long)k * N + n);
-      rw[u] = v;
+      c = c < W_CHUNKS ? c : W_CHUNKS - 1;
+      const int kk = c / (BN / 4), nc = c % (BN / 4);
+      const int k = k0 + kk, n = n0 + nc * 4;
+      const bool in = k < K && n < N; // N % 4 == 0
+      rw[u] = *reinterpret_cast<const float4 *>(
+          W + (long long)(k < K ? k : K - 1) * N + (n < N ? n : N - 4));
+      if (!in)
+        rw[u] = zero4;
     }
+#pragma unroll
+    for (int u = 0; u < A_PER; ++u)
+      if (!inside[u])
+        ra[u] = zero4;
   };
   auto store_slab = [&](int buf) {
 #pragma unroll
