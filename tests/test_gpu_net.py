@@ -192,6 +192,52 @@ def test_fused_convolutions_change_no_bit(scn, precision):
         assert skipped == 0
 
 
+@pytest.mark.parametrize("threads", [1, 3])
+def test_batches_of_changing_size_through_one_slot(scn, threads):
+    """Rule books are planned with counts deferred and sized by what the slot
+    has seen before: sparse batches, then one several times denser (outgrows
+    the bounds, is planned again the exact way), then sparse again, then a short
+    last batch.  Every batch's rule books and probabilities against the oracle."""
+    from sparseconvnet_archived_amd import hostapi, synthetic
+    cfg = synthetic.config(2, batch=8)
+    net = hostapi.Net(cfg.dimension, cfg.nInputFeatures, cfg.nClasses, nTop=1, threads=threads)
+    ora = oracle_net.Net(cfg.dimension, cfg.nInputFeatures, cfg.nClasses, nTop=1)
+    cfg.build(net)
+    cfg.build(ora)
+    net.setFusedConvolutions(True)
+    for i, (W, B, pr) in synthetic.he_normal_weights(net.layers(), 41).items():
+        net.set_weights(i, W, B, pr)
+        ora.set_weights(i, W, B, pr)
+    rng = np.random.default_rng(42)
+    sparse = synthetic.make_samples(cfg, 43, batch=8 * 4 + 3)
+    samples = []
+    for k, (pts, f, label) in enumerate(sparse):
+        if 16 <= k < 24:  # the third batch: a dense blob instead of strokes
+            side = 60
+            pts = np.array([(a, b) for a in range(side) for b in range(side) if rng.random() < 0.5], np.int32) + 18
+            f = rng.uniform(-1, 1, (len(pts), cfg.nInputFeatures)).astype(np.float32)
+        samples.append((pts, f, label))
+    ds = hostapi.Dataset("changing", cfg.nInputFeatures, cfg.nClasses, hostapi.TESTBATCH)
+    for pts, f, label in samples:
+        ds.add_points(cfg.dimension, cfg.lattice, pts, f, label)
+    net.begin(ds, 8)
+    for lo in range(0, len(samples), 8):
+        chunk = samples[lo:lo + 8]
+        assert net.next_batch()
+        S, K, R, bg, feats, n = synthetic.codify(chunk, cfg.dimension, cfg.lattice, net.inputSpatialSize,
+                                                 cfg.nInputFeatures)
+        want = ora.forward(len(chunk), S, K, R, bg, feats, n, np.array([c[2] for c in chunk], np.int32))
+        print("batch at", lo, "input rows", n, flush=True)
+        for i, wi in enumerate(want["interfaces"]):
+            gi = net.interface(i, want_features=False)
+            assert gi["nSpatialSites"] == wi["nSpatialSites"]
+            assert np.array_equal(gi["rules"], wi["rules"])
+        out = net.batch_outputs()
+        assert np.allclose(out["probabilities"], want["probabilities"], rtol=1e-3, atol=1e-6)
+    assert not net.next_batch()
+    net.close()
+
+
 def test_process_dataset_and_weight_files(scn, tmp_path):
     from sparseconvnet_archived_amd import hostapi, synthetic
     cfg = synthetic.config(2, batch=10)
