@@ -55,6 +55,7 @@ struct scn_ctx {
   // deferred counts (scn_ctx_defer_counts): plans whose counts are still on
   // their way; slot i of them reports into h_pinned[16 + 4 i ..]
   bool deferCounts;
+  bool wstream; // NiN: W-streaming kernel allowed (SCN_NIN_WSTREAM=0 turns it off)
   std::vector<struct scn_grids *> pendingGrids;
   // profiling
   bool prof;

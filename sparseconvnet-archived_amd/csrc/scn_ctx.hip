@@ -1,5 +1,6 @@
 // Context, error reporting, raw device memory and per-kernel timing.
 #include "scn_common.h"
+#include <stdlib.h>
 #include <stdarg.h>
 #include <string.h>
 
@@ -30,6 +31,10 @@ extern "C" int scn_ctx_create(int device, scn_ctx **out) {
   c->profTag = 0;
   c->ticket = 0;
   c->deferCounts = false;
+  {
+    const char *e = getenv("SCN_NIN_WSTREAM");
+    c->wstream = !(e && e[0] == '0');
+  }
   memset(c->profMs, 0, sizeof(c->profMs));
   memset(c->profCalls, 0, sizeof(c->profCalls));
   hipDeviceProp_t prop;

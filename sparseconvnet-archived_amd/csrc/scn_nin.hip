@@ -2,6 +2,8 @@
 // fused into the contraction's epilogue (the reference runs replicateArray,
 // cublasSgemm and applySigmoid / PreLU as three passes over the output).
 #include "scn_common.h"
+#include <mutex>
+#include <type_traits>
 
 int scn_softmax_launch(scn_ctx *ctx, const float *d_in, float *d_out,
                        long long M, int N);
@@ -479,13 +481,34 @@ template <int ROWS, int NT, int SA> struct WresPipe {
   float b[2][4][NT];
   acc_t acc[NT];
 
+  // Lane (c, q) owns columns NT c .. NT c + NT - 1 of the slice: tile j of the
+  // MFMA is the columns {NT c + j}.  Its NT operands of a k are then adjacent
+  // in LDS (one wide read) and its NT results of a row adjacent in the output
+  // (one wide store).  wl points at sW + 4 q PITCH + NT c.
   __device__ __forceinline__ void read_w(const float *wl, int t, int slot) {
     const float *wk = wl + KS * t * PITCH;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 4; ++i) {
+      const float *p = wk + i * PITCH;
+      if (NT % 4 == 0) {
 #pragma unroll
-      for (int j = 0; j < NT; ++j)
-        b[slot][i][j] = wk[i * PITCH + ROWS * j];
+        for (int j = 0; j < NT; j += 4) {
+          const float4 v = *reinterpret_cast<const float4 *>(p + j);
+          b[slot][i][j] = v.x, b[slot][i][j + 1] = v.y;
+          b[slot][i][j + 2] = v.z, b[slot][i][j + 3] = v.w;
+        }
+      } else if (NT % 2 == 0) {
+#pragma unroll
+        for (int j = 0; j < NT; j += 2) {
+          const float2 v = *reinterpret_cast<const float2 *>(p + j);
+          b[slot][i][j] = v.x, b[slot][i][j + 1] = v.y;
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+          b[slot][i][j] = p[j];
+      }
+    }
   }
   __device__ __forceinline__ void clear() {
 #pragma unroll
@@ -518,17 +541,63 @@ template <int ROWS, int NT, int SA> struct WresPipe {
       __builtin_amdgcn_sched_barrier(0);
     }
   }
+  // SA k-steps whose W is the slab at wslab (lane-offset as wl is); b[0] holds
+  // its first step's W on entry.  Before the last step's MFMAs, handover()
+  // puts the next slab in place (stores + barrier): every wavefront has by
+  // then read all it needs of this slab, and the first W of the next slab
+  // (at wnext) is read under those MFMAs.
+  template <class Addr, class Handover>
+  __device__ __forceinline__ void slab(int t0, Addr &addr, const float *wslab,
+                                       const float *wnext, Handover &handover) {
+#pragma unroll
+    for (int s = 0; s < SA; ++s) {
+      a[(s + SA - 1) % SA] =
+          *reinterpret_cast<const float4 *>(addr(t0 + s + SA - 1));
+      if (s + 1 < SA) {
+        read_w(wslab, s + 1, (s + 1) & 1);
+      } else {
+        handover();
+        read_w(wnext, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      const float av[4] = {a[s].x, a[s].y, a[s].z, a[s].w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+          acc[j] = DirectAcc<ROWS>::mfma(av[i], b[s & 1][i][j], acc[j]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  // orow: row 4 q of the panel, column NT c of the slice
   template <bool GUARDED>
   __device__ __forceinline__ void store(float *orow, int N, long long rowsLeft,
                                         int q, const ColEpilogue (&col)[NT]) {
+    static_assert(ROWS == 16, "lane-contiguous columns are laid out for 16-row panels");
 #pragma unroll
-    for (int j = 0; j < NT; ++j)
+    for (int v = 0; v < VPT; ++v) {
+      if (GUARDED && 4 * q + v >= rowsLeft)
+        continue;
+      float r[NT];
 #pragma unroll
-      for (int v = 0; v < VPT; ++v) {
-        const int r = ROWS == 32 ? 8 * (v / 4) + (v % 4) : v;
-        if (!GUARDED || 4 * q + r < rowsLeft)
-          orow[(long long)r * N + ROWS * j] = finish(acc[j][v], col[j]);
+      for (int j = 0; j < NT; ++j)
+        r[j] = finish(acc[j][v], col[j]);
+      float *o = orow + (long long)v * N;
+      if (NT % 4 == 0) {
+#pragma unroll
+        for (int j = 0; j < NT; j += 4)
+          *reinterpret_cast<float4 *>(o + j) =
+              make_float4(r[j], r[j + 1], r[j + 2], r[j + 3]);
+      } else if (NT % 2 == 0) {
+#pragma unroll
+        for (int j = 0; j < NT; j += 2)
+          *reinterpret_cast<float2 *>(o + j) = make_float2(r[j], r[j + 1]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+          o[j] = r[j];
       }
+    }
   }
 };
 
@@ -666,12 +735,12 @@ __global__ void __launch_bounds__(512)
   }
   __syncthreads();
 
-  const float *wl = sW + 4 * q * PITCH + c;
+  const float *wl = sW + 4 * q * PITCH + NT * c;
   pipe.read_w(wl, 0, 0);
   ColEpilogue col[NT];
 #pragma unroll
   for (int j = 0; j < NT; ++j)
-    col[j] = load_col(ep, n0 + ROWS * j + c);
+    col[j] = load_col(ep, n0 + NT * c + j);
 
   // aim: set up the prefetch that runs past this panel's end into the next
   auto aim = [&]() {
@@ -699,7 +768,7 @@ __global__ void __launch_bounds__(512)
       st.cur = st.nxt;
     }
   };
-  float *const obase = out + (long long)(4 * q) * N + n0 + c;
+  float *const obase = out + (long long)(4 * q) * N + n0 + NT * c;
 
   if (panel < nFull) { // first panel: entered with only loads in flight
     aim();
@@ -740,16 +809,19 @@ static int launch_wres(scn_ctx *ctx, const float *A, const float *W, float *out,
   const long long cap = (long long)ctx->numCU * (lds * 2 <= WRES_LDS_BYTES ? 2 : 1);
   if (wgs > cap)
     wgs = cap;
-  static bool configured = false; // one set of attribute calls per instantiation
-  if (!configured) {
+  static std::once_flag configured; // one set of attribute calls per instantiation
+  int rc = SCN_OK;
+  std::call_once(configured, [&]() {
 #define SCN_WRES_LDS(G)                                                        \
-  SCN_HIP_CHECK(hipFuncSetAttribute(                                           \
-      reinterpret_cast<const void *>(k_nin_wres<ROWS, NT, SA, G>),             \
-      hipFuncAttributeMaxDynamicSharedMemorySize, WRES_LDS_BYTES));
+  if (hipFuncSetAttribute(                                                     \
+          reinterpret_cast<const void *>(k_nin_wres<ROWS, NT, SA, G>),         \
+          hipFuncAttributeMaxDynamicSharedMemorySize,                          \
+          WRES_LDS_BYTES) != hipSuccess)                                       \
+    rc = SCN_ERR_HIP;
     SCN_WRES_LDS(0) SCN_WRES_LDS(1) SCN_WRES_LDS(3) SCN_WRES_LDS(7)
 #undef SCN_WRES_LDS
-    configured = true;
-  }
+  });
+  SCN_REQUIRE(rc == SCN_OK, SCN_ERR_HIP, "hipFuncSetAttribute failed");
   const dim3 grid((unsigned)(wgs * nSplits));
 #define SCN_WRES_GO(G, src)                                                    \
   hipLaunchKernelGGL((k_nin_wres<ROWS, NT, SA, G>), grid, dim3(512), lds,      \
@@ -809,6 +881,269 @@ static bool wres_forward(scn_ctx *ctx, const float *A, const float *W,
     SCN_WRES_CASE(6)
   }
 #undef SCN_WRES_CASE
+  return false;
+}
+
+// ---- W streamed through LDS, A direct to registers ---------------------------
+// For contractions whose slice of W does not fit LDS.  The inner loop is the
+// W-resident kernel's (A goes from global memory straight into the MFMA
+// operand registers, only W is read from LDS), but W passes through two LDS
+// buffers in slabs of SA k-steps.  The eight wavefronts of a workgroup take
+// eight consecutive 16-row panels and walk k in step, so one slab serves all
+// of them: one barrier per slab, none inside it.  Each thread fetches its part
+// of the next slab at the start of a slab and puts it into the other buffer
+// at the end; the slab after a panel's last is the next panel's first, so the
+// stream never drains.
+template <int NT, int SA, int GRU>
+__global__ void __launch_bounds__(512, NT <= 4 ? 2 : 1)
+    k_nin_wstream(const float *__restrict__ A, const float *__restrict__ W,
+                  float *__restrict__ out, long long M, int K, int N,
+                  Epilogue ep, GatherSource gs, int nSplits) {
+  constexpr int ROWS = 16;
+  typedef WresPipe<ROWS, NT, SA> Pipe;
+  constexpr bool GATHER = GRU > 0;
+  constexpr int KS = Pipe::KS, NW = Pipe::NW, PITCH = Pipe::PITCH;
+  constexpr int SLAB = KS * SA;            // k per slab
+  constexpr int SLAB_FLOATS = SLAB * PITCH;
+  extern __shared__ __attribute__((aligned(16))) float sW[]; // [2][SLAB][PITCH]
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int c = lane % ROWS, q = lane / ROWS;
+  const int split = blockIdx.x % nSplits;
+  const int wg = blockIdx.x / nSplits;
+  const int wgs = gridDim.x / nSplits;
+  const int n0 = split * NW;
+  const long long nPanels = (M + ROWS - 1) / ROWS;
+  const long long nGroups = (nPanels + 7) / 8;    // eight panels, one per wavefront
+  const long long nFullGroups = (M / ROWS) / 8;   // ... all of them whole
+  const int T = K / KS, nSlabs = T / SA;
+  long long pg = wg;
+  long long panel = pg * 8 + wave; // may lie past the end in the last group
+
+  int *const sRw = reinterpret_cast<int *>(sW + 2 * SLAB_FLOATS) +
+                   wave * (2 * ROWS * gs.fs);
+  const int rulesPerPanel = ROWS * gs.fs;
+  auto row_of = [&](long long pnl) {
+    long long m = pnl * ROWS + c;
+    return m < M ? m : M - 1; // rows past the end: read a valid row, store nothing
+  };
+  struct {
+    const float *cur, *nxt; // plain
+    long long wrap;
+    int bufCur, bufNext, rule, ch; // gather
+  } st;
+  // as in the W-resident kernel: tt >= T means step tt - T of the next panel
+  auto addr = [&](int tt) -> const float * {
+    if (!GATHER)
+      return st.cur + KS * tt + (tt >= T ? st.wrap : 0ll);
+    const float *p =
+        (st.rule >= 0 ? A + (long long)st.rule * gs.nIn : gs.zeros) + st.ch;
+    const int tn = tt + 1;
+    const int kn = KS * (tn >= T ? tn - T : tn) + 4 * q;
+    const int fn = (int)__umulhi((unsigned)kn, gs.magic);
+    st.ch = kn - fn * gs.nIn;
+    st.rule = sRw[(tn >= T ? st.bufNext : st.bufCur) + c * gs.fs + fn];
+    return p;
+  };
+  constexpr int RU = GATHER ? GRU : 1;
+  int rr[RU];
+  auto fetch_rules = [&](long long pnl) {
+    if (pnl >= nPanels)
+      pnl = nPanels - 1;
+    const long long first = pnl * rulesPerPanel, last = M * gs.fs - 1;
+#pragma unroll
+    for (int u = 0; u < RU; ++u) {
+      long long i = first + lane + 64 * u;
+      rr[u] = gs.rules[i < last ? i : last];
+    }
+  };
+  auto keep_rules = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < RU; ++u)
+      if (lane + 64 * u < rulesPerPanel)
+        sRw[buf + lane + 64 * u] = rr[u];
+  };
+
+  // a slab of this workgroup's columns of W: WPER 16-byte pieces per thread,
+  // the same pieces of every slab
+  constexpr int PER_ROW = NW / 4;
+  constexpr int CHUNKS = SLAB * PER_ROW;
+  constexpr int WPER = (CHUNKS + 511) / 512;
+  float4 w[WPER];
+  int dst[WPER];
+  const float *src[WPER];
+#pragma unroll
+  for (int u = 0; u < WPER; ++u) {
+    // past the end: the last piece again (same value to the same place)
+    int x = tid + 512 * u;
+    x = x < CHUNKS ? x : CHUNKS - 1;
+    const int k = x / PER_ROW, nc = x - k * PER_ROW;
+    dst[u] = k * PITCH + 4 * nc;
+    src[u] = W + (long long)k * N + n0 + 4 * nc;
+  }
+  auto w_load = [&](int slab) {
+    const long long off = (long long)slab * SLAB * N;
+#pragma unroll
+    for (int u = 0; u < WPER; ++u)
+      w[u] = *reinterpret_cast<const float4 *>(src[u] + off);
+  };
+  auto w_store = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < WPER; ++u) {
+      // the loads stay where they were issued, a slab earlier
+      asm volatile("" : "+v"(w[u].x), "+v"(w[u].y), "+v"(w[u].z), "+v"(w[u].w));
+      *reinterpret_cast<float4 *>(&sW[buf * SLAB_FLOATS + dst[u]]) = w[u];
+    }
+  };
+
+  Pipe pipe;
+  const bool more = pg + wgs < nGroups; // uniform over the workgroup
+  if (GATHER) {
+    st.bufCur = 0;
+    st.bufNext = rulesPerPanel;
+    fetch_rules(panel);
+    w_load(0);
+    keep_rules(0);
+    fetch_rules(panel + 8ll * wgs);
+    st.ch = 4 * q - (int)__umulhi((unsigned)(4 * q), gs.magic) * gs.nIn;
+    st.rule = sRw[c * gs.fs + (int)__umulhi((unsigned)(4 * q), gs.magic)];
+    if (!more)
+      st.bufNext = 0; // no next panel: the prefetch past the end re-reads this one
+  } else {
+    st.cur = A + row_of(panel) * K + 4 * q;
+  }
+  st.wrap = 0;
+#pragma unroll
+  for (int s = 0; s < SA - 1; ++s)
+    pipe.a[s] = *reinterpret_cast<const float4 *>(addr(s));
+  if (!GATHER)
+    w_load(0);
+  w_store(0);
+  __syncthreads();
+  int cur = 0; // the buffer the next slab is read from
+  pipe.read_w(sW + 4 * q * PITCH + NT * c, 0, 0);
+
+  const float *const wl = sW + 4 * q * PITCH + NT * c;
+  ColEpilogue col[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+    col[j] = load_col(ep, n0 + NT * c + j);
+  float *const obase = out + (long long)(4 * q) * N + n0 + NT * c;
+
+  auto run_panel = [&](auto guarded) {
+    const long long next = panel + 8ll * wgs;
+    const bool hasNext = pg + wgs < nGroups;
+    if (GATHER) {
+      if (hasNext)
+        keep_rules(st.bufNext);
+      fetch_rules(next + 8ll * wgs);
+    } else {
+      st.nxt = hasNext ? A + row_of(next) * K + 4 * q : st.cur;
+      st.wrap = (st.nxt - st.cur) - (long long)KS * T;
+    }
+    pipe.clear();
+    for (int g = 0; g < nSlabs; ++g) {
+      w_load(g + 1 < nSlabs ? g + 1 : 0);
+      auto handover = [&]() {
+        w_store(cur ^ 1);
+        __syncthreads();
+      };
+      pipe.slab(g * SA, addr, wl + cur * SLAB_FLOATS,
+                wl + (cur ^ 1) * SLAB_FLOATS, handover);
+      cur ^= 1;
+    }
+    pipe.template store<decltype(guarded)::value>(obase + panel * ROWS * N, N,
+                                                  M - panel * ROWS, q, col);
+    pg += wgs;
+    panel = next;
+    if (GATHER) {
+      const int b = st.bufCur;
+      st.bufCur = st.bufNext;
+      st.bufNext = pg + wgs < nGroups ? b : st.bufCur;
+    } else {
+      st.cur = st.nxt;
+    }
+  };
+  while (pg < nFullGroups)
+    run_panel(std::false_type());
+  if (pg < nGroups) // the last group: a ragged panel, panels past the end
+    run_panel(std::true_type());
+}
+
+#define WSTREAM_LDS_BYTES(nw, sa) (2 * 16 * (sa) * ((nw) + 4) * 4)
+template <int NT, int SA>
+static int launch_wstream(scn_ctx *ctx, const float *A, const float *W,
+                          float *out, long long M, int K, int N,
+                          const Epilogue &ep, const GatherSource *gs) {
+  constexpr int NW = 16 * NT;
+  const int nSplits = N / NW;
+  const size_t lds =
+      WSTREAM_LDS_BYTES(NW, SA) + (gs ? WRES_RULE_BYTES(gs->fs) : 0);
+  long long wgs = scn_ceil_div(scn_ceil_div(M, 16), 8);
+  const long long cap = (long long)ctx->numCU * (lds * 2 <= WRES_LDS_BYTES ? 2 : 1);
+  if (wgs > cap)
+    wgs = cap;
+  static std::once_flag configured; // one set of attribute calls per instantiation
+  int rc = SCN_OK;
+  std::call_once(configured, [&]() {
+#define SCN_WSTREAM_LDS(G)                                                     \
+  if (hipFuncSetAttribute(                                                     \
+          reinterpret_cast<const void *>(k_nin_wstream<NT, SA, G>),            \
+          hipFuncAttributeMaxDynamicSharedMemorySize,                          \
+          WRES_LDS_BYTES) != hipSuccess)                                       \
+    rc = SCN_ERR_HIP;
+    SCN_WSTREAM_LDS(0) SCN_WSTREAM_LDS(1) SCN_WSTREAM_LDS(3) SCN_WSTREAM_LDS(7)
+#undef SCN_WSTREAM_LDS
+  });
+  SCN_REQUIRE(rc == SCN_OK, SCN_ERR_HIP, "hipFuncSetAttribute failed");
+  const dim3 grid((unsigned)(wgs * nSplits));
+#define SCN_WSTREAM_GO(G, src)                                                 \
+  hipLaunchKernelGGL((k_nin_wstream<NT, SA, G>), grid, dim3(512), lds,         \
+                     ctx->stream, A, W, out, M, K, N, ep, src, nSplits)
+  if (!gs)
+    SCN_WSTREAM_GO(0, GatherSource());
+  else if (gs->fs <= 4)
+    SCN_WSTREAM_GO(1, *gs);
+  else if (gs->fs <= 12)
+    SCN_WSTREAM_GO(3, *gs);
+  else
+    SCN_WSTREAM_GO(7, *gs);
+#undef SCN_WSTREAM_GO
+  return SCN_OK;
+}
+
+// As wres_forward: the choice depends on M, K, N only.
+static bool wstream_forward(scn_ctx *ctx, const float *A, const float *W,
+                            float *out, long long M, int K, int N,
+                            const Epilogue &ep, const GatherSource *gs) {
+  if (K % 32 != 0 || K < 64 || N % 16 != 0 || M < 1024)
+    return false;
+  const int sa = K % 64 == 0 ? 4 : 2;
+  // widest slice that still fills every compute unit; else the narrowest
+  static const int widths[] = {6, 4, 3, 2};
+  const long long groups = scn_ceil_div(scn_ceil_div(M, 16), 8);
+  int nt = 0;
+  for (int w : widths) {
+    if (N % (16 * w) != 0)
+      continue;
+    nt = w;
+    if (groups * (N / (16 * w)) >= (long long)ctx->numCU * (w <= 4 ? 2 : 1))
+      break; // (the widest runs one workgroup per compute unit)
+  }
+  if (nt == 0)
+    return false;
+#define SCN_WSTREAM_CASE(T)                                                    \
+  case T:                                                                      \
+    return (sa == 4 ? launch_wstream<T, 4>(ctx, A, W, out, M, K, N, ep, gs)    \
+                    : launch_wstream<T, 2>(ctx, A, W, out, M, K, N, ep, gs)) == \
+           SCN_OK;
+  switch (nt) {
+    SCN_WSTREAM_CASE(2)
+    SCN_WSTREAM_CASE(3)
+    SCN_WSTREAM_CASE(4)
+    SCN_WSTREAM_CASE(6)
+  }
+#undef SCN_WSTREAM_CASE
   return false;
 }
 
@@ -1050,7 +1385,7 @@ static int nin_forward(scn_ctx *ctx, const float *d_A, const float *d_W,
   ep.act = act;
   ProfScope prof(ctx, gs ? SCN_K_CONV_NIN : SCN_K_NIN);
   const bool vec = K % 4 == 0 && N % 4 == 0 && ((uintptr_t)d_A & 15) == 0 &&
-                   ((uintptr_t)d_W & 15) == 0;
+                   ((uintptr_t)d_W & 15) == 0 && ((uintptr_t)d_out & 15) == 0;
   // bf16 operands only where the contraction is big enough to matter; the
   // classifier head and the thin first layers stay fp32
   if (vec && K >= 64 && act != SCN_SOFTMAX && precision != SCN_FP32) {
@@ -1075,6 +1410,9 @@ static int nin_forward(scn_ctx *ctx, const float *d_A, const float *d_W,
                        K, N, ep);
   } else if (vec && wres_forward(ctx, d_A, d_W, d_out, M, K, N, ep, gs)) {
     // W-resident kernel took it
+  } else if (vec && ctx->wstream &&
+             wstream_forward(ctx, d_A, d_W, d_out, M, K, N, ep, gs)) {
+    // W-streaming kernel took it
   } else if ((vec && K >= 8) || gs) {
     // Tall tiles (128 rows), 64 columns wide, or 96 where that divides N
     // (measured on 12928 x 1280 x 480: 93 TFLOP/s against 73 with 64-column

@@ -81,7 +81,12 @@ SHAPES = [(1000, 12, 32), (777, 128, 64), (513, 256, 96), (300, 384, 128), (129,
           # W-resident kernel: an odd number of prefetch groups, a 48-column slice, many narrow slices
           (600, 160, 192), (1000, 64, 48), (2469, 512, 160),
           # few rows (split-k kernel): ragged row and column blocks; few input channels (thin kernel)
-          (3, 40, 100), (511, 1024, 36), (83, 9, 5), (5000, 12, 32), (4097, 28, 100)]
+          (3, 40, 100), (511, 1024, 36), (83, 9, 5), (5000, 12, 32), (4097, 28, 100),
+          # contractions too long for W to stay in LDS (W-streaming kernel): narrow slices with a ragged
+          # last group of panels, two-step slabs with a 48-column slice, many slices
+          (1500, 1728, 64), (1100, 2016, 48), (1025, 3200, 320)]
+# ... and with enough rows for its wide slices (64 and 96 columns)
+STREAMED_WIDE = [(66001, 1728, 64), (33005, 1728, 96)]
 
 
 @pytest.mark.parametrize("M,K,N", SHAPES)
@@ -113,6 +118,12 @@ def test_nin_fp32(scn, ctx, M, K, N, act):
     assert err_gpu <= 4 * err_cpu + 1e-6
     rel = np.linalg.norm(got - want64) / max(np.linalg.norm(want64), 1e-30)
     assert rel <= 1e-4
+
+
+@pytest.mark.parametrize("M,K,N", STREAMED_WIDE)
+@pytest.mark.parametrize("act", ["RELU", "PRELU"])
+def test_nin_fp32_streamed_w_wide_slices(scn, ctx, M, K, N, act):
+    test_nin_fp32(scn, ctx, M, K, N, act)
 
 
 def test_nin_special_cases(scn, ctx):
@@ -205,7 +216,10 @@ def test_argument_errors(scn, ctx):
 
 
 @pytest.mark.parametrize("rows,fs,nIn,N", [(700, 4, 32, 64), (3000, 9, 64, 96), (513, 27, 64, 64), (129, 8, 96, 128),
-                                           (5000, 4, 128, 160), (64, 1, 4, 32), (300, 25, 8, 100)])
+                                           (5000, 4, 128, 160), (64, 1, 4, 32), (300, 25, 8, 100),
+                                           # W-streaming kernel: every width of slice, every size of rule load
+                                           (1500, 27, 64, 64), (66001, 27, 64, 64), (33005, 9, 192, 96),
+                                           (1100, 4, 504, 48)])
 @pytest.mark.parametrize("act", ["RELU", "PRELU"])
 def test_fused_gather_nin_matches_the_two_kernels_bit_for_bit(scn, ctx, rows, fs, nIn, N, act):
     a = getattr(scn, act)
@@ -213,6 +227,7 @@ def test_fused_gather_nin_matches_the_two_kernels_bit_for_bit(scn, ctx, rows, fs
     nInRows = 400
     inp = rng.uniform(-1, 1, (nInRows, nIn)).astype(np.float32)
     rules = rng.integers(0, nInRows, (rows, fs)).astype(np.int32)
+    rules[rng.random((rows, fs)) < 0.2] = -1  # no input site there
     K = fs * nIn
     W = (rng.standard_normal((K, N)) * np.sqrt(2.0 / K)).astype(np.float32)
     B = rng.uniform(-0.5, 0.5, N).astype(np.float32)
@@ -227,8 +242,10 @@ def test_fused_gather_nin_matches_the_two_kernels_bit_for_bit(scn, ctx, rows, fs
     ctx.gather_rows(d_in, g, d_rules, rows * fs, nIn)
     ctx.nin_forward(g, d_W, d_B, d_pr, two, rows, K, N, 1.0, a, scn.FP32)
     assert np.array_equal(fused.download(), two.download())
-    want = orc.nin_forward(orc.gather_rows(inp, rules.ravel(), nIn).reshape(rows, K), W, B, pr, 1.0, a, f64=True)
-    scale = np.abs(inp[rules].reshape(rows, K)).astype(np.float64) @ np.abs(W).astype(np.float64) + np.abs(B)
+    # (a rule of -1 reads as a row of zeros; the oracle's gather has the reference's rules, which name a zero row)
+    gathered = np.where(rules[:, :, None] >= 0, inp[np.maximum(rules, 0)], 0).reshape(rows, K).astype(np.float32)
+    want = orc.nin_forward(gathered, W, B, pr, 1.0, a, f64=True)
+    scale = np.abs(gathered).astype(np.float64) @ np.abs(W).astype(np.float64) + np.abs(B)
     assert np.all(np.abs(fused.download() - want) <= 1e-4 * scale)
     assert not scn.lib().scn_conv_nin_supported(64, 32, 64)  # window too large for the staged rules
     assert not scn.lib().scn_conv_nin_supported(4, 3, 32)  # channels not a multiple of 4
