@@ -407,7 +407,7 @@ __global__ void k_plan_count(GridView in, Geom g, const long long *ekey,
 }
 
 // per sample: does it need a background row, and how many were appended
-// before it.  One block of 1024 lanes.
+// before it.  One block of SCAN1_THREADS lanes.
 __device__ __forceinline__ void
 plan_samples_body(const GridView &in, const unsigned *base, long long nEntries,
                   long long fullSize, int *outBg, int *bgBefore,
@@ -415,14 +415,11 @@ plan_samples_body(const GridView &in, const unsigned *base, long long nEntries,
                   const long long *badSites, long long ticket,
                   long long *meta, const long long *inMeta, long long boundRows,
                   long long boundActive, int pinnedSlot) {
-  __shared__ int waveSum[17];
-  __shared__ int carry;
+  __shared__ int waveSum[2 * SCAN1_WAVES];
   const int t = threadIdx.x;
   const int lane = t & 63, wave = t >> 6;
-  if (t == 0)
-    carry = 0;
-  __syncthreads();
-  for (int b0 = 0; b0 < in.batch; b0 += 1024) {
+  int carry = 0, flip = 0; // the same in every lane
+  for (int b0 = 0; b0 < in.batch; b0 += SCAN1_THREADS) {
     int b = b0 + t;
     int notFull = 0;
     unsigned re = 0;
@@ -433,8 +430,8 @@ plan_samples_body(const GridView &in, const unsigned *base, long long nEntries,
       long long oc = (long long)base[re] - (long long)base[rs];
       notFull = oc < fullSize;
     }
-    // prefix of notFull over the 1024 lanes: shuffles inside a wavefront, the
-    // 16 wavefront totals through LDS (two barriers instead of thirty)
+    // prefix of notFull over the lanes: shuffles inside a wavefront, the
+    // wavefront totals through LDS (two sets of words: one barrier per round)
     int incl = notFull;
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {
@@ -442,33 +439,24 @@ plan_samples_body(const GridView &in, const unsigned *base, long long nEntries,
       if (lane >= off)
         incl += up;
     }
+    int *ws = waveSum + flip * SCAN1_WAVES;
     if (lane == 63)
-      waveSum[wave] = incl;
+      ws[wave] = incl;
     __syncthreads();
-    if (wave == 0) {
-      int w = lane < 16 ? waveSum[lane] : 0;
-      int wi = w;
+    int before = 0, total = 0;
 #pragma unroll
-      for (int off = 1; off < 16; off <<= 1) {
-        int up = __shfl_up(wi, off, 64);
-        if (lane >= off)
-          wi += up;
-      }
-      if (lane < 16)
-        waveSum[lane] = wi - w;
-      if (lane == 15)
-        waveSum[16] = wi;
+    for (int w = 0; w < SCAN1_WAVES; ++w) {
+      const int x = ws[w];
+      before += w < wave ? x : 0;
+      total += x;
     }
-    __syncthreads();
-    int excl = waveSum[wave] + incl - notFull + carry;
+    int excl = before + incl - notFull + carry;
     if (b < in.batch) {
       bgBefore[b] = excl;
       outBg[b] = notFull ? (int)base[re] + excl : -1;
     }
-    __syncthreads();
-    if (t == 0)
-      carry += waveSum[16];
-    __syncthreads();
+    carry += total;
+    flip ^= 1;
   }
   if (t == 0) {
     const long long nSites = (long long)base[nEntries] + carry; // nOutputSpatialSites
@@ -496,7 +484,7 @@ plan_samples_body(const GridView &in, const unsigned *base, long long nEntries,
   }
 }
 
-__global__ void __launch_bounds__(1024)
+__global__ void __launch_bounds__(SCAN1_THREADS)
     k_plan_samples(GridView in, const unsigned *base, long long nEntries,
                    long long fullSize, int *outBg, int *bgBefore,
                    unsigned *sampleStart, long long *scalars,
@@ -510,8 +498,7 @@ __global__ void __launch_bounds__(1024)
 
 // small batches: prefix sum of the owned counts and the per-sample pass in
 // one launch
-template <int PER>
-__global__ void __launch_bounds__(1024)
+__global__ void __launch_bounds__(SCAN1_THREADS)
     k_plan_scan_samples(GridView in, const unsigned *cnt, unsigned *base,
                         long long nEntries, long long fullSize, int *outBg,
                         int *bgBefore, unsigned *sampleStart,
@@ -519,8 +506,8 @@ __global__ void __launch_bounds__(1024)
                         long long ticket, long long *meta,
                         const long long *inMeta, long long boundRows,
                         long long boundActive, int pinnedSlot) {
-  __shared__ uint32_t ldsScan[17];
-  (void)block_scan_loop<false, PER>(cnt, base, (size_t)nEntries, ldsScan);
+  __shared__ uint32_t ldsScan[SCAN1_LDS_WORDS];
+  (void)block_scan_loop<false>(cnt, base, (size_t)nEntries, ldsScan);
   __syncthreads(); // the block's own writes to base[] are visible to it
   plan_samples_body(in, base, nEntries, fullSize, outBg, bgBefore, sampleStart,
                     scalars, badSites, ticket, meta, inMeta, boundRows,
@@ -774,15 +761,15 @@ __global__ void k_rules_fill_runs(GridView in, Geom g, const long long *siteKey,
 }
 
 // terminal pooling: sample sizes and their maximum.  One block.
-__global__ void k_terminal_plan(GridView in, unsigned *sampleStart,
+__global__ void __launch_bounds__(SCAN1_THREADS) k_terminal_plan(GridView in, unsigned *sampleStart,
                                 volatile long long *scalars,
                                 long long ticket, long long *meta,
                                 const long long *inMeta, long long boundWidth,
                                 int pinnedSlot) {
-  __shared__ long long lds[1024];
+  __shared__ long long lds[SCAN1_THREADS];
   const int t = threadIdx.x;
   long long mx = 1; // TerminalPoolingLayer.cu:90
-  for (int b = t; b < in.batch; b += 1024) {
+  for (int b = t; b < in.batch; b += SCAN1_THREADS) {
     unsigned rs = rank_of(in, (long long)b * in.vol);
     unsigned re = rank_of(in, (long long)(b + 1) * in.vol);
     sampleStart[b] = rs;
@@ -793,7 +780,7 @@ __global__ void k_terminal_plan(GridView in, unsigned *sampleStart,
   }
   lds[t] = mx;
   __syncthreads();
-  for (int off = 512; off > 0; off >>= 1) {
+  for (int off = SCAN1_THREADS / 2; off > 0; off >>= 1) {
     if (t < off && lds[t + off] > lds[t])
       lds[t] = lds[t + off];
     __syncthreads();
@@ -1321,22 +1308,15 @@ static int plan_regions_d(scn_ctx *ctx, scn_grids *in, scn_grids *out,
   const long long *bad = (const long long *)(ctx->d_scalars + 15);
   const long long ticket = ++ctx->ticket;
   if ((size_t)nE <= SCAN1_MAX_ELEMS) {
-    if ((size_t)nE <= SCAN1_SMALL_ELEMS)
-      hipLaunchKernelGGL((k_plan_scan_samples<32>), dim3(1), dim3(1024), 0,
-                         ctx->stream, vin, out->cnt.p, out->base.p, nE, fullSize,
-                         out->bg.p, out->bgBefore.p, out->sampleStart.p,
-                         (long long *)ctx->d_pinned, bad, ticket, out->meta.p,
-                         inMeta, boundRows, boundActive, slot);
-    else
-      hipLaunchKernelGGL((k_plan_scan_samples<64>), dim3(1), dim3(1024), 0,
-                         ctx->stream, vin, out->cnt.p, out->base.p, nE, fullSize,
-                         out->bg.p, out->bgBefore.p, out->sampleStart.p,
-                         (long long *)ctx->d_pinned, bad, ticket, out->meta.p,
-                         inMeta, boundRows, boundActive, slot);
+    hipLaunchKernelGGL(k_plan_scan_samples, dim3(1), dim3(SCAN1_THREADS), 0,
+                       ctx->stream, vin, out->cnt.p, out->base.p, nE, fullSize,
+                       out->bg.p, out->bgBefore.p, out->sampleStart.p,
+                       (long long *)ctx->d_pinned, bad, ticket, out->meta.p,
+                       inMeta, boundRows, boundActive, slot);
   } else {
     SCN_TRY(scn_scan_exclusive_u32(ctx->stream, out->cnt.p, out->base.p,
                                    (size_t)nE, out->scanTmp.p));
-    hipLaunchKernelGGL(k_plan_samples, dim3(1), dim3(1024), 0, ctx->stream, vin,
+    hipLaunchKernelGGL(k_plan_samples, dim3(1), dim3(SCAN1_THREADS), 0, ctx->stream, vin,
                        out->base.p, nE, fullSize, out->bg.p, out->bgBefore.p,
                        out->sampleStart.p, (long long *)ctx->d_pinned, bad, ticket, out->meta.p,
                          inMeta, boundRows, boundActive, slot);
@@ -1496,7 +1476,7 @@ extern "C" int scn_rules_terminal_plan(scn_ctx *ctx, const scn_grids *cin,
       deferred ? grow_bound(out->seenWidth, 8, in->vol) : 0x7FFFFFFFFFFFll;
   const int slot = deferred ? (int)ctx->pendingGrids.size() : -1;
   const long long ticket = ++ctx->ticket;
-  hipLaunchKernelGGL(k_terminal_plan, dim3(1), dim3(1024), 0, ctx->stream,
+  hipLaunchKernelGGL(k_terminal_plan, dim3(1), dim3(SCAN1_THREADS), 0, ctx->stream,
                      view_of(in), out->sampleStart.p,
                      (long long *)ctx->d_pinned, ticket, out->meta.p,
                      in->pending ? in->meta.p : nullptr, boundWidth, slot);

@@ -78,11 +78,11 @@ __global__ void __launch_bounds__(SCAN_THREADS)
     out[n] = off + total;
 }
 
-template <bool POPC, int PER>
+template <bool POPC>
 __global__ void __launch_bounds__(SCAN1_THREADS)
     k_scan_single(const void *in, uint32_t *out, size_t n) {
-  __shared__ uint32_t lds[17];
-  (void)block_scan_loop<POPC, PER>(in, out, n, lds);
+  __shared__ uint32_t lds[SCAN1_LDS_WORDS];
+  (void)block_scan_loop<POPC>(in, out, n, lds);
 }
 
 size_t scn_scan_tmp_elems(size_t n) {
@@ -99,12 +99,8 @@ template <bool POPC>
 static int scan_impl(hipStream_t s, const void *in, uint32_t *out, size_t n,
                      uint32_t *tmp) {
   if (n <= SCAN1_MAX_ELEMS) { // one launch; n == 0 still writes out[0] = 0
-    if (n <= SCAN1_SMALL_ELEMS)
-      hipLaunchKernelGGL((k_scan_single<POPC, 32>), dim3(1), dim3(SCAN1_THREADS),
-                         0, s, in, out, n);
-    else
-      hipLaunchKernelGGL((k_scan_single<POPC, 64>), dim3(1), dim3(SCAN1_THREADS),
-                         0, s, in, out, n);
+    hipLaunchKernelGGL(k_scan_single<POPC>, dim3(1), dim3(SCAN1_THREADS), 0, s,
+                       in, out, n);
     SCN_HIP_CHECK(hipGetLastError());
     return SCN_OK;
   }
