@@ -67,8 +67,11 @@ def parse():
                          "hardware byte counters collected over the run can be scaled by a kernel of known traffic")
     ap.add_argument("--from-host", action="store_true",
                     help="also time processDataset() on host-resident Pictures (CPU codify + PCIe upload included)")
-    ap.add_argument("--producers", type=int, default=6,
-                    help="batch-producer threads / streams building rule books ahead of the forward pass")
+    ap.add_argument("--producers", type=int, default=5,
+                    help="batch-producer threads / streams building rule books ahead of the forward pass.  HIP "
+                         "spreads streams over 4 hardware queues, and kernels of streams that share a queue run "
+                         "in order: with 5 producer streams the forward pass's stream (created first) still has "
+                         "its queue to itself (measured: 0.30 ms per batch of config 2, 0.35 with 6 or 4)")
     ap.add_argument("--fused", type=int, choices=[0, 1], default=1,
                     help="1: setFusedConvolutions, a convolution's gather runs inside the next NiN kernel (same "
                          "results bit for bit); 0: the reference's two steps, gather then NiN")
