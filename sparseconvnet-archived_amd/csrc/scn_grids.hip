@@ -406,6 +406,19 @@ __global__ void k_plan_count(GridView in, Geom g, const long long *ekey,
   }
 }
 
+// where sample t starts and ends in iteration order: what the first round of
+// plan_samples_body needs of the input grids (independent of the counts, so
+// a caller that scans first can have these loads in flight meanwhile)
+__device__ __forceinline__ void sample_ranks(const GridView &in, unsigned &rs,
+                                             unsigned &re) {
+  const int t = threadIdx.x;
+  rs = re = 0;
+  if (t < in.batch) {
+    rs = rank_of(in, (long long)t * in.vol);
+    re = rank_of(in, (long long)(t + 1) * in.vol);
+  }
+}
+
 // per sample: does it need a background row, and how many were appended
 // before it.  One block of SCAN1_THREADS lanes.
 __device__ __forceinline__ void
@@ -414,7 +427,8 @@ plan_samples_body(const GridView &in, const unsigned *base, long long nEntries,
                   unsigned *sampleStart, volatile long long *scalars,
                   const long long *badSites, long long ticket,
                   long long *meta, const long long *inMeta, long long boundRows,
-                  long long boundActive, int pinnedSlot) {
+                  long long boundActive, int pinnedSlot, unsigned rs0,
+                  unsigned re0) {
   __shared__ int waveSum[2 * SCAN1_WAVES];
   const int t = threadIdx.x;
   const int lane = t & 63, wave = t >> 6;
@@ -424,8 +438,9 @@ plan_samples_body(const GridView &in, const unsigned *base, long long nEntries,
     int notFull = 0;
     unsigned re = 0;
     if (b < in.batch) {
-      unsigned rs = rank_of(in, (long long)b * in.vol);
-      re = rank_of(in, (long long)(b + 1) * in.vol);
+      // (the first round's ranks were fetched by the caller, ahead of its scan)
+      unsigned rs = b0 == 0 ? rs0 : rank_of(in, (long long)b * in.vol);
+      re = b0 == 0 ? re0 : rank_of(in, (long long)(b + 1) * in.vol);
       sampleStart[b] = rs;
       long long oc = (long long)base[re] - (long long)base[rs];
       notFull = oc < fullSize;
@@ -491,9 +506,11 @@ __global__ void __launch_bounds__(SCAN1_THREADS)
                    const long long *badSites, long long ticket, long long *meta,
                    const long long *inMeta, long long boundRows,
                    long long boundActive, int pinnedSlot) {
+  unsigned rs0, re0;
+  sample_ranks(in, rs0, re0);
   plan_samples_body(in, base, nEntries, fullSize, outBg, bgBefore, sampleStart,
                     scalars, badSites, ticket, meta, inMeta, boundRows,
-                    boundActive, pinnedSlot);
+                    boundActive, pinnedSlot, rs0, re0);
 }
 
 // small batches: prefix sum of the owned counts and the per-sample pass in
@@ -507,11 +524,13 @@ __global__ void __launch_bounds__(SCAN1_THREADS)
                         const long long *inMeta, long long boundRows,
                         long long boundActive, int pinnedSlot) {
   __shared__ uint32_t ldsScan[SCAN1_LDS_WORDS];
+  unsigned rs0, re0;
+  sample_ranks(in, rs0, re0);
   (void)block_scan_loop<false>(cnt, base, (size_t)nEntries, ldsScan);
   __syncthreads(); // the block's own writes to base[] are visible to it
   plan_samples_body(in, base, nEntries, fullSize, outBg, bgBefore, sampleStart,
                     scalars, badSites, ticket, meta, inMeta, boundRows,
-                    boundActive, pinnedSlot);
+                    boundActive, pinnedSlot, rs0, re0);
 }
 
 // pass 2: emit the owned outputs
