@@ -1,6 +1,7 @@
 // C view of the host classes (see scn_host_c.h).
 #include "scn_host_c.h"
 #include "Off3DFormatPicture.h"
+#include "OnlineHandwritingPicture.h"
 
 #include <cstdio>
 #include <cstdlib>
@@ -193,6 +194,61 @@ void scnh_dataset_add_mesh(scnh_dataset *ds, int64_t nPoints,
                            int label) {
   ds->ds.pictures.push_back(new OffSurfaceModelPicture(
       points, (int)nPoints, triangles, (int)nTriangles, renderSize, label));
+}
+static bool stroke_encoding_ok(const scnh_dataset *ds, int encoding) {
+  const bool known = encoding == Simple || encoding == Octogram ||
+                     encoding == UndirectedOctogram || encoding == SpaceTime3d ||
+                     encoding == VectorSpaceTime3d;
+  return known && ds->ds.nFeatures == OnlineHandwritingEncodingSize[encoding];
+}
+int scnh_dataset_add_strokes(scnh_dataset *ds, int nStrokes,
+                             const int32_t *strokeLengths, const double *xy,
+                             int renderSize, int encoding, int label,
+                             int normalize) {
+  if (!stroke_encoding_ok(ds, encoding))
+    return -1;
+  auto *p = new OnlineHandwritingPicture(
+      renderSize, (OnlineHandwritingEncoding)encoding, label);
+  for (int s = 0; s < nStrokes; ++s) {
+    p->addStroke(xy, strokeLengths[s]);
+    xy += 2 * (size_t)strokeLengths[s];
+  }
+  if (p->ops.empty()) {
+    delete p;
+    return -1;
+  }
+  if (normalize) {
+    try {
+      p->normalize();
+    } catch (const std::exception &) {
+      delete p;
+      return -1;
+    }
+  }
+  ds->ds.pictures.push_back(p);
+  return 0;
+}
+int64_t scnh_dataset_add_pendigits_file(scnh_dataset *ds, const char *path,
+                                        int renderSize, int encoding) {
+  if (!stroke_encoding_ok(ds, encoding))
+    return -1;
+  try {
+    return readPenDigitsFile(ds->ds.pictures, path, renderSize,
+                             (OnlineHandwritingEncoding)encoding);
+  } catch (const std::exception &) {
+    return -1;
+  }
+}
+int64_t scnh_constant_speed(const double *xy, int nPoints, float density,
+                            int multiplier, double *out, int64_t capacity) {
+  if (nPoints <= 0)
+    return 0;
+  std::vector<double> s(xy, xy + 2 * (size_t)nPoints);
+  std::vector<double> r = constantSpeed(s, density, multiplier);
+  const int64_t n = (int64_t)(r.size() / 2);
+  if (n <= capacity)
+    std::copy(r.begin(), r.end(), out);
+  return n;
 }
 int64_t scnh_codify_picture(scnh_dataset *ds, int64_t index, int spatialSize,
                             int64_t seed, int64_t capacity, int64_t *keys,

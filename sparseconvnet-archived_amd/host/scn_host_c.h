@@ -55,6 +55,25 @@ int scnh_dataset_add_off_file(scnh_dataset *ds, const char *path, int renderSize
 void scnh_dataset_add_mesh(scnh_dataset *ds, int64_t nPoints,
                            const double *points, int64_t nTriangles,
                            const int32_t *triangles, int renderSize, int label);
+/* OnlineHandwritingPicture (OnlineHandwritingPicture.h): a character from
+ * arrays -- nStrokes strokes, stroke s has strokeLengths[s] points, xy holds
+ * all points in order as (x, y) doubles -- optionally normalize()d; or every
+ * character of a UCI pen-digits file (readPenDigitsFile,
+ * SpatiallySparseDatasetPenDigits.cpp:15-63; returns how many were appended).
+ * encoding: 0 Simple, 1 Octogram, 2 UndirectedOctogram, 7 SpaceTime3d,
+ * 8 VectorSpaceTime3d; the dataset needs the matching nFeatures (1, 8, 4, 1,
+ * 3).  Both return -1 for an encoding that is not available (3..6, the
+ * LogSignature ones), a wrong nFeatures, or a file that cannot be opened. */
+int scnh_dataset_add_strokes(scnh_dataset *ds, int nStrokes,
+                             const int32_t *strokeLengths, const double *xy,
+                             int renderSize, int encoding, int label,
+                             int normalize);
+int64_t scnh_dataset_add_pendigits_file(scnh_dataset *ds, const char *path,
+                                        int renderSize, int encoding);
+/* constantSpeed (OnlineHandwritingPicture.cpp:27-53) of one stroke: returns the
+ * number of points and, when that fits capacity, writes them to out. */
+int64_t scnh_constant_speed(const double *xy, int nPoints, float density,
+                            int multiplier, double *out, int64_t capacity);
 /* Picture::distort (when seed >= 0, with RNG(seed) and the dataset's batch
  * type) followed by Picture::codifyInputData into an empty grid, on the CPU.
  * Returns the number of rows (background row included); when that fits

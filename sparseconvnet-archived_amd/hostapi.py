@@ -54,6 +54,9 @@ def lib():
         "scnh_dataset_size": (i64, [vp]),
         "scnh_dataset_add_off_file": (i32, [vp, C.c_char_p, i32, i32]),
         "scnh_dataset_add_mesh": (None, [vp, i64, vp, i64, vp, i32, i32]),
+        "scnh_dataset_add_strokes": (i32, [vp, i32, vp, vp, i32, i32, i32, i32]),
+        "scnh_dataset_add_pendigits_file": (i64, [vp, C.c_char_p, i32, i32]),
+        "scnh_constant_speed": (i64, [vp, i32, f32, i32, vp, i64]),
         "scnh_codify_picture": (i64, [vp, i64, i32, i64, i64, vp, vp, vp, vp]),
         "scnh_process_dataset": (f32, [vp, vp, i32]),
         "scnh_process_dataset_repeat_test": (None, [vp, vp, i32, i32]),
@@ -108,6 +111,24 @@ class Dataset:
         points = np.ascontiguousarray(points, np.float64).reshape(-1, 3)
         triangles = np.ascontiguousarray(triangles, np.int32).reshape(-1, 3)
         lib().scnh_dataset_add_mesh(self.h, len(points), _p(points), len(triangles), _p(triangles), renderSize, label)
+
+    def add_strokes(self, strokes, renderSize, encoding, label=-1, normalize=True):
+        """OnlineHandwritingPicture from a list of strokes (each n x 2)."""
+        strokes = [np.ascontiguousarray(s, np.float64).reshape(-1, 2) for s in strokes]
+        lengths = np.array([len(s) for s in strokes], np.int32)
+        xy = np.ascontiguousarray(np.concatenate(strokes) if strokes else np.zeros((0, 2)))
+        if lib().scnh_dataset_add_strokes(self.h, len(strokes), _p(lengths), _p(xy), renderSize, encoding, label,
+                                          1 if normalize else 0) != 0:
+            raise ValueError("strokes: encoding %d is not available, does not match nFeatures %d, or the "
+                             "character is empty" % (encoding, self.nFeatures))
+
+    def add_pendigits_file(self, path, renderSize, encoding):
+        """every character of a UCI pen-digits file; returns how many."""
+        n = lib().scnh_dataset_add_pendigits_file(self.h, str(path).encode(), renderSize, encoding)
+        if n < 0:
+            raise IOError("%s: not readable, or encoding %d not available for nFeatures %d"
+                          % (path, encoding, self.nFeatures))
+        return int(n)
 
     def codify(self, index, spatialSize, seed=-1):
         """distort (seed >= 0) + codifyInputData of one picture on the CPU:
@@ -268,6 +289,23 @@ class Net:
 
     def context_handle(self):
         return lib().scnh_context(self.h)
+
+
+# OnlineHandwritingEncoding (types.h:29-39 of the reference)
+SIMPLE, OCTOGRAM, UNDIRECTED_OCTOGRAM, SPACETIME3D, VECTOR_SPACETIME3D = 0, 1, 2, 7, 8
+ENCODING_FEATURES = {0: 1, 1: 8, 2: 4, 7: 1, 8: 3}
+
+
+def constant_speed(stroke, density, multiplier=1):
+    """constantSpeed of one stroke (n x 2) -> resampled points."""
+    xy = np.ascontiguousarray(stroke, np.float64).reshape(-1, 2)
+    cap = 1 << 12
+    while True:
+        out = np.empty((cap, 2), np.float64)
+        n = lib().scnh_constant_speed(_p(xy), len(xy), density, multiplier, _p(out), cap)
+        if n <= cap:
+            return out[:n].copy()
+        cap = int(n)
 
 
 def take_multiply_add_count():
