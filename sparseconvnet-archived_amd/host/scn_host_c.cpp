@@ -2,6 +2,7 @@
 #include "scn_host_c.h"
 #include "Off3DFormatPicture.h"
 #include "OnlineHandwritingPicture.h"
+#include "OpenCVPicture.h"
 
 #include <cstdio>
 #include <cstdlib>
@@ -238,6 +239,31 @@ int64_t scnh_dataset_add_pendigits_file(scnh_dataset *ds, const char *path,
   } catch (const std::exception &) {
     return -1;
   }
+}
+int scnh_dataset_add_image(scnh_dataset *ds, int xSize, int ySize, int channels,
+                           const float *pixels, int backgroundColor, int label,
+                           int trainingJiggle) {
+  if (channels != ds->ds.nFeatures || xSize <= 0 || ySize <= 0 ||
+      backgroundColor < 0 || backgroundColor > 255)
+    return -1;
+  auto *p = new OpenCVPicture(xSize, ySize, channels,
+                              (unsigned char)backgroundColor, label);
+  p->trainingJiggle = trainingJiggle;
+  std::copy(pixels, pixels + (size_t)xSize * ySize * channels,
+            reinterpret_cast<float *>(p->mat.data));
+  ds->ds.pictures.push_back(p);
+  return 0;
+}
+int64_t scnh_dataset_add_mnist_files(scnh_dataset *ds, const char *imagesPath,
+                                     const char *labelsPath) {
+  if (ds->ds.nFeatures != 1)
+    return -1;
+  return loadMnist(imagesPath, labelsPath, ds->ds.pictures);
+}
+int64_t scnh_dataset_add_cifar10_file(scnh_dataset *ds, const char *path) {
+  if (ds->ds.nFeatures != 3)
+    return -1;
+  return readCIFAR10File(ds->ds.pictures, path);
 }
 int64_t scnh_constant_speed(const double *xy, int nPoints, float density,
                             int multiplier, double *out, int64_t capacity) {

@@ -70,6 +70,20 @@ int scnh_dataset_add_strokes(scnh_dataset *ds, int nStrokes,
                              int normalize);
 int64_t scnh_dataset_add_pendigits_file(scnh_dataset *ds, const char *path,
                                         int renderSize, int encoding);
+/* OpenCVPicture (OpenCVPicture.h), array-backed: pixels is rows x cols x
+ * channels floats in 0..255 with rows = xSize (the reference's constructor
+ * passes xSize as the row count); the MNIST idx pair and a CIFAR-10 binary
+ * batch through the reference's readers (SpatiallySparseDatasetMnist.cpp,
+ * SpatiallySparseDatasetCIFAR10.cpp).  trainingJiggle: what distort() moves a
+ * training picture by.  The readers return how many pictures they appended;
+ * all return -1 on a channel count that is not the dataset's nFeatures or an
+ * unreadable file. */
+int scnh_dataset_add_image(scnh_dataset *ds, int xSize, int ySize, int channels,
+                           const float *pixels, int backgroundColor, int label,
+                           int trainingJiggle);
+int64_t scnh_dataset_add_mnist_files(scnh_dataset *ds, const char *imagesPath,
+                                     const char *labelsPath);
+int64_t scnh_dataset_add_cifar10_file(scnh_dataset *ds, const char *path);
 /* constantSpeed (OnlineHandwritingPicture.cpp:27-53) of one stroke: returns the
  * number of points and, when that fits capacity, writes them to out. */
 int64_t scnh_constant_speed(const double *xy, int nPoints, float density,

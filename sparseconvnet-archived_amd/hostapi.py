@@ -57,6 +57,9 @@ def lib():
         "scnh_dataset_add_strokes": (i32, [vp, i32, vp, vp, i32, i32, i32, i32]),
         "scnh_dataset_add_pendigits_file": (i64, [vp, C.c_char_p, i32, i32]),
         "scnh_constant_speed": (i64, [vp, i32, f32, i32, vp, i64]),
+        "scnh_dataset_add_image": (i32, [vp, i32, i32, i32, vp, i32, i32, i32]),
+        "scnh_dataset_add_mnist_files": (i64, [vp, C.c_char_p, C.c_char_p]),
+        "scnh_dataset_add_cifar10_file": (i64, [vp, C.c_char_p]),
         "scnh_codify_picture": (i64, [vp, i64, i32, i64, i64, vp, vp, vp, vp]),
         "scnh_process_dataset": (f32, [vp, vp, i32]),
         "scnh_process_dataset_repeat_test": (None, [vp, vp, i32, i32]),
@@ -121,6 +124,27 @@ class Dataset:
                                           1 if normalize else 0) != 0:
             raise ValueError("strokes: encoding %d is not available, does not match nFeatures %d, or the "
                              "character is empty" % (encoding, self.nFeatures))
+
+    def add_image(self, pixels, backgroundColor, label=-1, trainingJiggle=0):
+        """OpenCVPicture from an array [rows x cols x channels] of values 0..255."""
+        pixels = np.ascontiguousarray(pixels, np.float32)
+        if pixels.ndim == 2:
+            pixels = pixels[:, :, None]
+        r, c, ch = pixels.shape
+        if lib().scnh_dataset_add_image(self.h, r, c, ch, _p(pixels), backgroundColor, label, trainingJiggle) != 0:
+            raise ValueError("image: %d channels into a dataset of %d features" % (ch, self.nFeatures))
+
+    def add_mnist_files(self, images, labels):
+        n = lib().scnh_dataset_add_mnist_files(self.h, str(images).encode(), str(labels).encode())
+        if n < 0:
+            raise IOError("%s / %s: not a readable MNIST idx pair (or nFeatures != 1)" % (images, labels))
+        return int(n)
+
+    def add_cifar10_file(self, path):
+        n = lib().scnh_dataset_add_cifar10_file(self.h, str(path).encode())
+        if n < 0:
+            raise IOError("%s: not a readable CIFAR-10 batch (or nFeatures != 3)" % path)
+        return int(n)
 
     def add_pendigits_file(self, path, renderSize, encoding):
         """every character of a UCI pen-digits file; returns how many."""
