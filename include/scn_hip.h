@@ -43,10 +43,10 @@ enum {
   SCN_RELU = 1,
   SCN_VLEAKYRELU = 2,
   SCN_LEAKYRELU = 3,
-  SCN_TANH = 4, /* not on the forward configs: rejected */
+  SCN_TANH = 4,
   SCN_SOFTMAX = 5,
   SCN_PRELU = 6,
-  SCN_SIGMOID = 7 /* rejected */
+  SCN_SIGMOID = 7
 };
 
 /* Operand precision of the NiN contraction (accumulation is always fp32):

@@ -581,6 +581,10 @@ static float activate(float v, int act, float slope) {
   case A_LEAKYRELU:
   case A_PRELU:
     return v > 0 ? v : v * slope;
+  case A_TANH: /* SigmoidLayer.cu:80-85 */
+    return tanhf(v);
+  case A_SIGMOID: /* SigmoidLayer.cu:43-48 */
+    return 1.0f / (1.0f + expf(-v));
   default:
     return v;
   }
@@ -642,6 +646,10 @@ void orc_nin_forward_f64(const float *A, const float *W, const float *B,
         v = v > 0 ? v : 0;
       else if (act == A_LEAKYRELU || act == A_VLEAKYRELU || act == A_PRELU)
         v = v > 0 ? v : v * sl;
+      else if (act == A_TANH)
+        v = tanh(v);
+      else if (act == A_SIGMOID)
+        v = 1.0 / (1.0 + exp(-v));
       o[n] = v;
     }
     if (act == A_SOFTMAX) {

@@ -250,6 +250,34 @@ __global__ void __launch_bounds__(256)
     b[k] = b[k] / acc;
 }
 
+// dSigmoidTanh / dSigmoidLogistic (SigmoidLayer.cu:43-48, 80-85): in place,
+// four elements per lane where the count allows
+__global__ void __launch_bounds__(256)
+    k_squash(float *x, long long n, int logistic) {
+  const long long i = ((long long)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (i + 4 <= n && ((uintptr_t)x & 15) == 0) {
+    float4 v = *reinterpret_cast<float4 *>(x + i);
+    if (logistic) {
+      v.x = 1.0f / (1.0f + expf(-v.x)), v.y = 1.0f / (1.0f + expf(-v.y));
+      v.z = 1.0f / (1.0f + expf(-v.z)), v.w = 1.0f / (1.0f + expf(-v.w));
+    } else {
+      v.x = tanhf(v.x), v.y = tanhf(v.y), v.z = tanhf(v.z), v.w = tanhf(v.w);
+    }
+    *reinterpret_cast<float4 *>(x + i) = v;
+  } else {
+    for (long long k = i; k < n && k < i + 4; ++k)
+      x[k] = logistic ? 1.0f / (1.0f + expf(-x[k])) : tanhf(x[k]);
+  }
+}
+int scn_squash_launch(scn_ctx *ctx, float *d_x, long long n, int logistic) {
+  if (n <= 0)
+    return SCN_OK;
+  hipLaunchKernelGGL(k_squash, dim3((unsigned)scn_ceil_div(scn_ceil_div(n, 4), 256)),
+                     dim3(256), 0, ctx->stream, d_x, n, logistic);
+  SCN_HIP_CHECK(hipGetLastError());
+  return SCN_OK;
+}
+
 int scn_softmax_launch(scn_ctx *ctx, const float *d_in, float *d_out,
                        long long M, int N) {
   hipLaunchKernelGGL(k_softmax, dim3(scn_ceil_div(M, 4)), dim3(256), 0,

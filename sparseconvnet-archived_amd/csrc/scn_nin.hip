@@ -5,6 +5,7 @@
 #include <mutex>
 #include <type_traits>
 
+int scn_squash_launch(scn_ctx *ctx, float *d_x, long long n, int logistic);
 int scn_softmax_launch(scn_ctx *ctx, const float *d_in, float *d_out,
                        long long M, int N);
 
@@ -1362,10 +1363,8 @@ static int nin_forward(scn_ctx *ctx, const float *d_A, const float *d_W,
   SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_nin_forward: null context");
   SCN_REQUIRE(M >= 0 && K >= 1 && N >= 1, SCN_ERR_ARG,
               "scn_nin_forward: M %lld K %d N %d", (long long)M, K, N);
-  SCN_REQUIRE(act == SCN_NOSIGMOID || act == SCN_RELU || act == SCN_VLEAKYRELU ||
-                  act == SCN_LEAKYRELU || act == SCN_SOFTMAX || act == SCN_PRELU,
-              SCN_ERR_ARG, "scn_nin_forward: activation %d is not supported",
-              act);
+  SCN_REQUIRE(act >= SCN_NOSIGMOID && act <= SCN_SIGMOID, SCN_ERR_ARG,
+              "scn_nin_forward: activation %d", act);
   SCN_REQUIRE(precision == SCN_FP32 || precision == SCN_BF16 ||
                   precision == SCN_BF16X3,
               SCN_ERR_ARG,
@@ -1443,8 +1442,13 @@ static int nin_forward(scn_ctx *ctx, const float *d_A, const float *d_W,
                        d_W, d_out, (long long)M, K, N, ep);
   }
   SCN_HIP_CHECK(hipGetLastError());
+  // softmax, tanh and the logistic function are a pass of their own over the
+  // layer's output, as in the reference (the kernels above treat them as
+  // "no activation")
   if (act == SCN_SOFTMAX)
     SCN_TRY(scn_softmax_launch(ctx, d_out, d_out, (long long)M, N));
+  if (act == SCN_TANH || act == SCN_SIGMOID)
+    SCN_TRY(scn_squash_launch(ctx, d_out, (long long)M * N, act == SCN_SIGMOID));
   return SCN_OK;
 }
 

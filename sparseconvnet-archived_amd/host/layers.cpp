@@ -263,8 +263,6 @@ NetworkInNetworkLayer::NetworkInNetworkLayer(cudaMemStream &memStream,
       MW(true, (size_t)nFeaturesIn * nFeaturesOut), B(true, nFeaturesOut),
       MB(true, nFeaturesOut), fn(fn), nFeaturesIn(nFeaturesIn),
       nFeaturesOut(nFeaturesOut), dropout(dropout), precision(SCN_FP32) {
-  if (fn == TANH || fn == SIGMOID)
-    unsupported("the tanh / logistic activation");
   float scale = std::pow(6.0f / (nFeaturesIn + nFeaturesOut * alpha), 0.5f);
   W.setUniform(-scale, scale);
   MW.setZero();

@@ -6,7 +6,7 @@ CPU oracle always see identical inputs and weights.
 """
 import numpy as np
 
-RELU, VLEAKYRELU, LEAKYRELU, SOFTMAX, PRELU = 1, 2, 3, 5, 6
+RELU, VLEAKYRELU, LEAKYRELU, TANH, SOFTMAX, PRELU, SIGMOID = 1, 2, 3, 4, 5, 6, 7
 
 
 # --------------------------------------------------------------- site patterns
@@ -184,7 +184,7 @@ def codify(samples, dimension, lattice, spatialSize, nFeatures):
     """What BatchProducer + SparsePointsPicture::codifyInputData produce for a
     batch: flat (sample, key, row), backgroundCol per sample, the feature
     matrix [nSpatialSites x nFeatures] and nSpatialSites."""
-    shift = (spatialSize - lattice) // 2
+    shift = int((spatialSize - lattice) / 2)  # toward zero, as the C++ division
     S, K, R, bg, feats = [], [], [], [], []
     n = 0
     for i, (pts, f, _) in enumerate(samples):
@@ -196,10 +196,12 @@ def codify(samples, dimension, lattice, spatialSize, nFeatures):
         key = np.zeros(len(c), np.int64)
         for a in range(dimension):
             key = key * spatialSize + c[:, a]
-        _, first = np.unique(key, return_index=True)
+        # first occurrence of every key among the points inside the field (a point outside has a key that
+        # aliases some other cell's: it must not stand in for that cell)
+        idx = np.flatnonzero(inside)
+        _, first = np.unique(key[idx], return_index=True)
         keep = np.zeros(len(c), bool)
-        keep[first] = True
-        keep &= inside
+        keep[idx[first]] = True
         k = key[keep]
         S.append(np.full(len(k), i, np.int32))
         K.append(k)

@@ -126,6 +126,28 @@ def test_nin_fp32_streamed_w_wide_slices(scn, ctx, M, K, N, act):
     test_nin_fp32(scn, ctx, M, K, N, act)
 
 
+@pytest.mark.parametrize("M,K,N", [(777, 128, 64), (5, 7, 3), (40003, 256, 96), (1500, 1728, 64), (4097, 28, 100)])
+@pytest.mark.parametrize("act", ["TANH", "SIGMOID"])
+def test_nin_fp32_squashing_activations(scn, ctx, M, K, N, act):
+    """tanh and the logistic function (SigmoidLayer.cu:43-48, 80-85): a pass over the output of any NiN kernel."""
+    a = getattr(scn, act)
+    rng = np.random.default_rng(M + K + N + a)
+    A = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    W = (rng.standard_normal((K, N)) * np.sqrt(2.0 / K)).astype(np.float32)
+    B = rng.uniform(-0.5, 0.5, N).astype(np.float32)
+    d_out = ctx.empty((M, N), np.float32)
+    ctx.nin_forward(ctx.array(A), ctx.array(W), ctx.array(B), None, d_out, M, K, N, 0.9, a, scn.FP32)
+    got = d_out.download()
+    want64 = orc.nin_forward(A, W, B, None, 0.9, a, f64=True)
+    # both functions have slope <= 1: the error of the contraction carries over at most unchanged
+    scale = np.abs(A).astype(np.float64) @ np.abs(W).astype(np.float64) + np.abs(B)
+    assert np.all(np.abs(got - want64) <= 1e-4 * scale + 1e-6)
+    pre = np.float64(np.float32(0.9)) * (A.astype(np.float64) @ W.astype(np.float64) + B)
+    closed = np.tanh(pre) if act == "TANH" else 1.0 / (1.0 + np.exp(-pre))
+    assert np.allclose(want64, closed, rtol=1e-9, atol=1e-12)  # the oracle against the closed form
+    assert np.allclose(orc.nin_forward(A, W, B, None, 0.9, a), closed, rtol=1e-4, atol=1e-5)
+
+
 def test_nin_special_cases(scn, ctx):
     rng = np.random.default_rng(3)
     M, K = 70, 64
@@ -143,7 +165,7 @@ def test_nin_special_cases(scn, ctx):
     want[:, 7] = 2.0 * A[:, 3]
     assert np.array_equal(d_out.download(), want)
     with pytest.raises(scn.ScnError):
-        ctx.nin_forward(ctx.array(A), ctx.array(W), ctx.array(B), None, d_out, M, K, K, 1.0, scn.TANH)
+        ctx.nin_forward(ctx.array(A), ctx.array(W), ctx.array(B), None, d_out, M, K, K, 1.0, 8)  # no such activation
     with pytest.raises(scn.ScnError):
         ctx.nin_forward(ctx.array(A), ctx.array(W), ctx.array(B), None, d_out, M, K, K, 1.0, scn.PRELU)
 

@@ -131,6 +131,21 @@ def test_triangular_net(scn):
     run_config(scn, cfg, 7, triangular=True, samples=samples)
 
 
+@pytest.mark.parametrize("fused", [False, True])
+def test_net_with_tanh_and_logistic_layers(scn, fused):
+    from sparseconvnet_archived_amd import synthetic
+    stack = [("addLeNetLayerMP", 32, 3, 1, 2, 2, synthetic.TANH), ("addLeNetLayerMP", 64, 2, 1, 2, 2, synthetic.SIGMOID),
+             ("addLeNetLayerMP", 64, 1, 1, 1, 1, synthetic.TANH), ("addTerminalPoolingLayer", 2), ("addSoftmaxLayer",)]
+    cfg = synthetic.Config("squash", 2, 3, 10, 8, 20, stack)
+    cfg.number = 2
+    rng = np.random.default_rng(9)
+    samples = []
+    for _ in range(8):
+        pts = np.array([(a, b) for a in range(20) for b in range(20) if rng.random() < 0.3], np.int32)
+        samples.append((pts, rng.uniform(-1, 1, (len(pts), 3)).astype(np.float32), int(rng.integers(0, 10))))
+    run_config(scn, cfg, 9, samples=samples, fused=fused)
+
+
 @pytest.mark.parametrize("number,batch,seed", [(2, 20, 202), (3, 6, 203), (4, 2, 204), (5, 1, 205)])
 def test_fused_convolutions_against_oracle(scn, number, batch, seed):
     """setFusedConvolutions: the gather runs inside the NiN kernel; everything
