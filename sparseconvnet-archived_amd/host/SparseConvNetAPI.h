@@ -58,6 +58,9 @@ class SparseConvNetCUDA;
                                 int batchSize = 100, int nReps = 12,           \
                                 std::string predictionsFilename = "",          \
                                 std::string confusionMatrixFilename = "");     \
+  void processDatasetDumpTopLevelFeatures(SpatiallySparseDataset &dataset,     \
+                                          int batchSize, int reps = 1);        \
+  void calculateInputRegularizingConstants(SpatiallySparseDataset dataset);    \
   void loadWeights(std::string baseName, int epoch, bool momentum = false,     \
                    int firstNlayers = 1000000);                                \
   void saveWeights(std::string baseName, int epoch, bool momentum = false);

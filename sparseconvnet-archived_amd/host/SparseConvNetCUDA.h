@@ -90,6 +90,14 @@ public:
                                 int batchSize = 100, int nReps = 12,
                                 std::string predictionsFilename = "",
                                 std::string confusionMatrixFilename = "");
+  // every layer but the last; "<sample> <label> <features...>" per sample into
+  // "<dataset.name>.features" (SparseConvNetCUDA.cu:507-538)
+  void processDatasetDumpTopLevelFeatures(SpatiallySparseDataset &dataset,
+                                          int batchSize, int reps = 1);
+  // 1 / max |x| per input feature over (at most 10000 pictures of) the
+  // dataset; the producers scale every batch's input by these from then on,
+  // and saveWeights / loadWeights carry them (SparseConvNetCUDA.cu:540-566)
+  void calculateInputRegularizingConstants(SpatiallySparseDataset dataset);
   void loadWeights(std::string baseName, int epoch, bool momentum,
                    int firstNlayers = 1000000);
   void saveWeights(std::string baseName, int epoch, bool momentum);

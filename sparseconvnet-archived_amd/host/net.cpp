@@ -360,6 +360,61 @@ float SparseConvNetCUDA::processDataset(SpatiallySparseDataset &dataset,
   printThroughput(diff, dataset.pictures.size());
   return nll;
 }
+// SparseConvNetCUDA.cu:507-538
+void SparseConvNetCUDA::processDatasetDumpTopLevelFeatures(
+    SpatiallySparseDataset &dataset, int batchSize, int reps) {
+  assert(dataset.pictures.size() > 0);
+  assert(dataset.type != TRAINBATCH);
+  std::ofstream f((dataset.name + ".features").c_str());
+  const size_t n = layers.size();
+  for (int rep = 0; rep < reps; rep++) {
+    BatchProducer bp(*this, dataset, inputSpatialSize, batchSize);
+    while (SpatiallySparseBatch *batch = bp.nextBatch()) {
+      for (size_t i = 0; i + 1 < n; i++) {
+        batch->interfaces[i + 1].sub->reset();
+        layers[i]->forwards(*batch, batch->interfaces[i], batch->interfaces[i + 1]);
+      }
+      SpatiallySparseBatchInterface &top = batch->interfaces[n - 1];
+      assert(top.nFeatures == (int)top.featuresPresent.size());
+      assert(!top.deferredGatherFrom); // (a convolution is never the last-but-one layer's output here)
+      std::vector<float> &v = top.sub->features.hVector(); // waits for the stream
+      std::vector<int> &labels = batch->labels.hVector();
+      for (int i = 0; i < batch->batchSize; i++) {
+        f << batch->sampleNumbers[i] << " " << labels[i];
+        for (int j = 0; j < top.nFeatures; j++)
+          f << " " << v[(size_t)i * top.nFeatures + j];
+        f << std::endl;
+      }
+    }
+  }
+}
+// SparseConvNetCUDA.cu:540-566
+void SparseConvNetCUDA::calculateInputRegularizingConstants(
+    SpatiallySparseDataset dataset) { // a copy of the dataset
+  inputNormalizingConstants.resize(0); // no rescaling while measuring
+  std::cout << "Using " << std::min(10000, (int)dataset.pictures.size())
+            << " out of " << dataset.pictures.size()
+            << " training samples to calculate regularizing constants."
+            << std::endl;
+  if (dataset.pictures.size() > 10000)
+    dataset.pictures.resize(10000);
+  dataset.type = TESTBATCH; // no dropout, no augmentation
+  std::vector<float> c(nInputFeatures, 0);
+  {
+    BatchProducer bp(*this, dataset, inputSpatialSize, 100);
+    while (SpatiallySparseBatch *batch = bp.nextBatch()) {
+      std::vector<float> &features = batch->interfaces[0].sub->features.hVector();
+      for (size_t i = 0; i < features.size(); ++i)
+        c[i % nInputFeatures] =
+            std::max(c[i % nInputFeatures], std::fabs(features[i]));
+    }
+  }
+  for (int i = 0; i < nInputFeatures; ++i) {
+    inputNormalizingConstants.push_back(c[i] > 0 ? 1.0f / c[i] : 0);
+    std::cout << inputNormalizingConstants.back() << " ";
+  }
+  std::cout << std::endl;
+}
 // SparseConvNetCUDA.cu:327-405: nReps forward passes, probabilities averaged
 void SparseConvNetCUDA::processDatasetRepeatTest(
     SpatiallySparseDataset &dataset, int batchSize, int nReps,
@@ -671,6 +726,14 @@ void SparseConvNet::processDatasetRepeatTest(
   cnn->processDatasetRepeatTest(dataset, batchSize, nReps, predictionsFilename,
                                 confusionMatrixFilename);
 }
+void SparseConvNet::processDatasetDumpTopLevelFeatures(
+    SpatiallySparseDataset &dataset, int batchSize, int reps) {
+  cnn->processDatasetDumpTopLevelFeatures(dataset, batchSize, reps);
+}
+void SparseConvNet::calculateInputRegularizingConstants(
+    SpatiallySparseDataset dataset) {
+  cnn->calculateInputRegularizingConstants(dataset);
+}
 void SparseConvNet::loadWeights(std::string baseName, int epoch, bool momentum,
                                 int firstNlayers) {
   cnn->loadWeights(baseName, epoch, momentum, firstNlayers);
@@ -711,6 +774,14 @@ void SparseConvTriangLeNet::processDatasetRepeatTest(
     std::string predictionsFilename, std::string confusionMatrixFilename) {
   cnn->processDatasetRepeatTest(dataset, batchSize, nReps, predictionsFilename,
                                 confusionMatrixFilename);
+}
+void SparseConvTriangLeNet::processDatasetDumpTopLevelFeatures(
+    SpatiallySparseDataset &dataset, int batchSize, int reps) {
+  cnn->processDatasetDumpTopLevelFeatures(dataset, batchSize, reps);
+}
+void SparseConvTriangLeNet::calculateInputRegularizingConstants(
+    SpatiallySparseDataset dataset) {
+  cnn->calculateInputRegularizingConstants(dataset);
 }
 void SparseConvTriangLeNet::loadWeights(std::string baseName, int epoch,
                                         bool momentum, int firstNlayers) {

@@ -315,6 +315,22 @@ void scnh_process_dataset_repeat_test(scnh_net *net, scnh_dataset *ds,
   net->cnn->processDatasetRepeatTest(ds->ds, batchSize, nReps);
 }
 
+void scnh_process_dataset_dump_top_level_features(scnh_net *net,
+                                                  scnh_dataset *ds,
+                                                  int batchSize, int reps) {
+  net->cnn->processDatasetDumpTopLevelFeatures(ds->ds, batchSize, reps);
+}
+void scnh_calculate_input_regularizing_constants(scnh_net *net,
+                                                 scnh_dataset *ds) {
+  net->cnn->calculateInputRegularizingConstants(ds->ds);
+}
+int scnh_input_normalizing_constants(scnh_net *net, float *out, int capacity) {
+  const auto &c = net->cnn->inputNormalizingConstants;
+  if ((int)c.size() <= capacity)
+    std::copy(c.begin(), c.end(), out);
+  return (int)c.size();
+}
+
 void scnh_begin(scnh_net *net, scnh_dataset *ds, int batchSize) {
   net->batch = nullptr;
   net->producer.reset(new BatchProducer(*net->cnn, ds->ds,

@@ -103,6 +103,17 @@ float scnh_process_dataset(scnh_net *net, scnh_dataset *ds, int batchSize);
 void scnh_process_dataset_repeat_test(scnh_net *net, scnh_dataset *ds,
                                       int batchSize, int nReps);
 
+/* SparseConvNet::processDatasetDumpTopLevelFeatures (writes
+ * "<dataset name>.features" in the working directory) and
+ * calculateInputRegularizingConstants; the constants (nInputFeatures floats,
+ * empty before the call) can be read back. */
+void scnh_process_dataset_dump_top_level_features(scnh_net *net,
+                                                  scnh_dataset *ds,
+                                                  int batchSize, int reps);
+void scnh_calculate_input_regularizing_constants(scnh_net *net,
+                                                 scnh_dataset *ds);
+int scnh_input_normalizing_constants(scnh_net *net, float *out, int capacity);
+
 /* Batch-by-batch processing with the batch left in place for inspection:
  * BatchProducer::nextBatch + SparseConvNetCUDA::processBatch. */
 void scnh_begin(scnh_net *net, scnh_dataset *ds, int batchSize);

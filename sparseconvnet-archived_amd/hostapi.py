@@ -63,6 +63,9 @@ def lib():
         "scnh_codify_picture": (i64, [vp, i64, i32, i64, i64, vp, vp, vp, vp]),
         "scnh_process_dataset": (f32, [vp, vp, i32]),
         "scnh_process_dataset_repeat_test": (None, [vp, vp, i32, i32]),
+        "scnh_process_dataset_dump_top_level_features": (None, [vp, vp, i32, i32]),
+        "scnh_calculate_input_regularizing_constants": (None, [vp, vp]),
+        "scnh_input_normalizing_constants": (i32, [vp, vp, i32]),
         "scnh_begin": (None, [vp, vp, i32]),
         "scnh_next_batch": (i32, [vp]),
         "scnh_end": (None, [vp]),
@@ -253,6 +256,19 @@ class Net:
         lib().scnh_process_dataset_repeat_test(self.h, ds.h, batchSize, nReps)
 
     # batch-by-batch with inspection
+    def processDatasetDumpTopLevelFeatures(self, ds, batchSize=100, reps=1):
+        """writes "<dataset name>.features" into the working directory."""
+        lib().scnh_process_dataset_dump_top_level_features(self.h, ds.h, batchSize, reps)
+
+    def calculateInputRegularizingConstants(self, ds):
+        lib().scnh_calculate_input_regularizing_constants(self.h, ds.h)
+        return self.inputNormalizingConstants()
+
+    def inputNormalizingConstants(self):
+        out = np.zeros(4096, np.float32)
+        n = lib().scnh_input_normalizing_constants(self.h, _p(out), len(out))
+        return out[:n].copy()
+
     def begin(self, ds, batchSize):
         lib().scnh_begin(self.h, ds.h, batchSize)
 

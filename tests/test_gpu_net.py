@@ -286,6 +286,60 @@ def test_process_dataset_and_weight_files(scn, tmp_path):
     net2.processDatasetRepeatTest(ds, 10, 2)
 
 
+def test_dump_top_level_features_and_input_regularizing_constants(scn, tmp_path, monkeypatch):
+    """processDatasetDumpTopLevelFeatures (every layer but the last, one text line per sample) and
+    calculateInputRegularizingConstants (1 / max |x| per input feature, applied to every later batch and
+    carried by the weight file)."""
+    from sparseconvnet_archived_amd import hostapi, synthetic
+    monkeypatch.chdir(tmp_path)
+    cfg = synthetic.config(2, batch=12)
+    net, ora = build_pair(cfg, hostapi)
+    for i, (W, B, pr) in synthetic.he_normal_weights(net.layers(), 19).items():
+        net.set_weights(i, W, B, pr)
+        ora.set_weights(i, W, B, pr)
+    samples = synthetic.make_samples(cfg, 34, batch=12)
+    # make the three input features of very different size
+    samples = [(p, f * np.array([1.0, 7.0, 0.25], np.float32), l) for p, f, l in samples]
+    ds = hostapi.Dataset("dumped", 3, 100, hostapi.TESTBATCH)
+    for pts, f, label in samples:
+        ds.add_points(2, cfg.lattice, pts, f, label)
+    labels = np.array([s[2] for s in samples], np.int32)
+
+    def oracle(scale):
+        scaled = [(p, f * scale, l) for p, f, l in samples]
+        S, K, R, bg, feats, n = synthetic.codify(scaled, 2, cfg.lattice, net.inputSpatialSize, 3)
+        return ora.forward(len(samples), S, K, R, bg, feats, n, labels)
+
+    want = oracle(np.ones(3, np.float32))
+    net.processDatasetDumpTopLevelFeatures(ds, 12)
+    rows = [line.split() for line in open(tmp_path / "dumped.features")]
+    assert len(rows) == 12 and sorted(int(r[0]) for r in rows) == list(range(12))
+    top = want["interfaces"][-2]["features"]  # the input of the last (softmax) layer
+    for r in rows:
+        i = int(r[0])
+        assert int(r[1]) == labels[i] and len(r) == 2 + top.shape[1]
+        assert np.allclose(np.array(r[2:], np.float64), top[i], rtol=2e-3, atol=1e-5)  # 6 significant digits of text
+    assert len(net.inputNormalizingConstants()) == 0
+    c = net.calculateInputRegularizingConstants(ds)
+    allf = np.concatenate([f for _, f, _ in samples])
+    assert np.allclose(c, 1.0 / np.abs(allf).max(0), rtol=1e-6)
+    net.begin(ds, 12)
+    assert net.next_batch()
+    got = net.batch_outputs()["probabilities"]
+    net.end()
+    assert np.allclose(got, oracle(c)["probabilities"], rtol=1e-3, atol=1e-6)
+    assert not np.allclose(got, want["probabilities"], rtol=1e-3, atol=1e-6)
+    # the weight file carries the constants: a net that has them loads them
+    net.saveWeights(str(tmp_path / "w"), 1)
+    net2, _ = build_pair(cfg, hostapi)
+    net2.calculateInputRegularizingConstants(ds)  # (sizes the vector, as the reference's drivers do before loading)
+    net2.loadWeights(str(tmp_path / "w"), 1)
+    net2.begin(ds, 12)
+    assert net2.next_batch()
+    assert np.allclose(net2.batch_outputs()["probabilities"], got, rtol=1e-6)
+    net2.end()
+
+
 @pytest.mark.parametrize("mode", ["BF16", "BF16X3"])
 def test_bf16_mode_net(scn, mode):
     """bf16 NiN contractions against the fp32 oracle on 200 samples.
