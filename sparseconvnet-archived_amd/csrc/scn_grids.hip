@@ -702,12 +702,32 @@ __global__ void k_tri_table(int size, int d, int *invOrd) {
   }
 }
 
+// The rank prefix of the output mask (which the next rule book needs of its
+// input) depends on the emit pass only, as the rules do: with SCAN, workgroup 0
+// of the fill launch computes it while the others fill, instead of a launch
+// of its own later (masks of up to SCAN1_MAX_ELEMS words).
+struct RankScan {
+  const unsigned long long *bits;
+  unsigned *prefix;
+  size_t n;
+};
+
 // one thread per rule: rules[row * width + q]
-template <int D>
-__global__ void k_rules_fill(GridView in, Geom g, const long long *siteKey,
-                             Count nSites, const long long *outMeta,
-                             const int *invOrd, int *rules) {
-  long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+template <int D, bool SCAN>
+__global__ void __launch_bounds__(256)
+    k_rules_fill(GridView in, Geom g, const long long *siteKey, Count nSites,
+                 const long long *outMeta, const int *invOrd, int *rules,
+                 RankScan rs) {
+  __shared__ uint32_t ldsScan[SCAN1_LDS_WORDS];
+  long long blk = blockIdx.x;
+  if (SCAN) {
+    if (blk == 0) {
+      (void)block_scan_loop<true>(rs.bits, rs.prefix, rs.n, ldsScan);
+      return;
+    }
+    blk -= 1;
+  }
+  long long idx = blk * blockDim.x + threadIdx.x;
   if (outMeta[META_OVERFLOW])
     return;
   long long total = count_now(nSites) * g.width;
@@ -742,11 +762,21 @@ __global__ void k_rules_fill(GridView in, Geom g, const long long *siteKey,
 // axis.  Their input sites are neighbours in the mask, so one mask read serves
 // the whole run (a lane per entry reads a 64-byte line of the mask for every
 // entry, and that line traffic is what bounds the kernel on 3-D batches).
-template <int D>
-__global__ void k_rules_fill_runs(GridView in, Geom g, const long long *siteKey,
-                                  Count nSites, const long long *outMeta,
-                                  int *rules) {
-  long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+template <int D, bool SCAN>
+__global__ void __launch_bounds__(256)
+    k_rules_fill_runs(GridView in, Geom g, const long long *siteKey,
+                      Count nSites, const long long *outMeta, int *rules,
+                      RankScan rs) {
+  __shared__ uint32_t ldsScan[SCAN1_LDS_WORDS];
+  long long blk = blockIdx.x;
+  if (SCAN) {
+    if (blk == 0) {
+      (void)block_scan_loop<true>(rs.bits, rs.prefix, rs.n, ldsScan);
+      return;
+    }
+    blk -= 1;
+  }
+  long long idx = blk * blockDim.x + threadIdx.x;
   if (outMeta[META_OVERFLOW])
     return;
   const int runsPerRow = g.width / g.size;
@@ -1571,46 +1601,44 @@ extern "C" int scn_rules_fill(scn_ctx *ctx, const scn_grids *in,
   SCN_REQUIRE(d_rules, SCN_ERR_ARG, "scn_rules_fill: null rules buffer");
   const bool tri = g.mode == MODE_TRI_NOMIN || g.mode == MODE_TRI_MIN;
   const int *inv = tri ? out->invOrd.p : nullptr;
-  dim3 grid(scn_ceil_div(total, 256)), block(256);
+  // the output mask is final (the emit pass has run): its rank prefix rides
+  // along as one more workgroup when it is short enough for one
+  const bool scan = !out->rankValid && out->nWords + 1 <= SCAN1_MAX_ELEMS;
+  const RankScan rs = {out->bits.p, out->prefix.p, scan ? out->nWords + 1 : 0};
+  const unsigned extra = scan ? 1 : 0;
+  dim3 grid(scn_ceil_div(total, 256) + extra), block(256);
+#define SCN_FILL_DIM(KERNEL, ...)                                              \
+  switch (g.d) {                                                               \
+  case 1:                                                                      \
+    if (scan)                                                                  \
+      hipLaunchKernelGGL((KERNEL<1, true>), __VA_ARGS__);                      \
+    else                                                                       \
+      hipLaunchKernelGGL((KERNEL<1, false>), __VA_ARGS__);                     \
+    break;                                                                     \
+  case 2:                                                                      \
+    if (scan)                                                                  \
+      hipLaunchKernelGGL((KERNEL<2, true>), __VA_ARGS__);                      \
+    else                                                                       \
+      hipLaunchKernelGGL((KERNEL<2, false>), __VA_ARGS__);                     \
+    break;                                                                     \
+  default:                                                                     \
+    if (scan)                                                                  \
+      hipLaunchKernelGGL((KERNEL<3, true>), __VA_ARGS__);                      \
+    else                                                                       \
+      hipLaunchKernelGGL((KERNEL<3, false>), __VA_ARGS__);                     \
+    break;                                                                     \
+  }
   if (!tri && g.size >= 2) {
-    dim3 runs(scn_ceil_div(total / g.size, 256));
-    switch (g.d) {
-    case 1:
-      hipLaunchKernelGGL(k_rules_fill_runs<1>, runs, block, 0, ctx->stream, vin,
-                         g, out->siteKey.p, count_sites(out), out->meta.p,
-                         d_rules);
-      break;
-    case 2:
-      hipLaunchKernelGGL(k_rules_fill_runs<2>, runs, block, 0, ctx->stream, vin,
-                         g, out->siteKey.p, count_sites(out), out->meta.p,
-                         d_rules);
-      break;
-    default:
-      hipLaunchKernelGGL(k_rules_fill_runs<3>, runs, block, 0, ctx->stream, vin,
-                         g, out->siteKey.p, count_sites(out), out->meta.p,
-                         d_rules);
-      break;
-    }
-    SCN_HIP_CHECK(hipGetLastError());
-    return SCN_OK;
+    dim3 runs(scn_ceil_div(total / g.size, 256) + extra);
+    SCN_FILL_DIM(k_rules_fill_runs, runs, block, 0, ctx->stream, vin, g,
+                 out->siteKey.p, count_sites(out), out->meta.p, d_rules, rs)
+  } else {
+    SCN_FILL_DIM(k_rules_fill, grid, block, 0, ctx->stream, vin, g,
+                 out->siteKey.p, count_sites(out), out->meta.p, inv, d_rules, rs)
   }
-  switch (g.d) {
-  case 1:
-    hipLaunchKernelGGL(k_rules_fill<1>, grid, block, 0, ctx->stream, vin, g,
-                       out->siteKey.p, count_sites(out), out->meta.p, inv,
-                       d_rules);
-    break;
-  case 2:
-    hipLaunchKernelGGL(k_rules_fill<2>, grid, block, 0, ctx->stream, vin, g,
-                       out->siteKey.p, count_sites(out), out->meta.p, inv,
-                       d_rules);
-    break;
-  default:
-    hipLaunchKernelGGL(k_rules_fill<3>, grid, block, 0, ctx->stream, vin, g,
-                       out->siteKey.p, count_sites(out), out->meta.p, inv,
-                       d_rules);
-    break;
-  }
+#undef SCN_FILL_DIM
   SCN_HIP_CHECK(hipGetLastError());
+  if (scan)
+    out->rankValid = true;
   return SCN_OK;
 }
