@@ -910,16 +910,26 @@ __global__ void __launch_bounds__(512, NT <= 4 ? 2 : 1)
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int c = lane % ROWS, q = lane / ROWS;
-  const int split = blockIdx.x % nSplits;
-  const int wg = blockIdx.x / nSplits;
-  const int wgs = gridDim.x / nSplits;
-  const int n0 = split * NW;
   const long long nPanels = (M + ROWS - 1) / ROWS;
   const long long nGroups = (nPanels + 7) / 8;    // eight panels, one per wavefront
   const long long nFullGroups = (M / ROWS) / 8;   // ... all of them whole
   const int T = K / KS, nSlabs = T / SA;
-  long long pg = wg;
-  long long panel = pg * 8 + wave; // may lie past the end in the last group
+  // Workgroups are dealt to the 8 XCDs round-robin and every XCD has an L2 of
+  // its own.  A long walk over one column slice (many groups per workgroup)
+  // is therefore cut into eight contiguous ranges, one per XCD, so that
+  // panels which gather the same input rows -- neighbours in the rule book --
+  // meet in one L2; otherwise workgroup w takes groups w, w + wgs, ...
+  const int wgs = gridDim.x / nSplits;
+  const bool ranges = nSplits == 1 && wgs % 8 == 0 && nGroups >= 2ll * wgs;
+  const int split = blockIdx.x % nSplits;
+  const int xcd = blockIdx.x % 8;
+  const long long perXcd = (nGroups + 7) / 8;
+  const int pgStep = ranges ? wgs / 8 : wgs;
+  const long long pgEnd =
+      ranges && (xcd + 1) * perXcd < nGroups ? (xcd + 1) * perXcd : nGroups;
+  const int n0 = split * NW;
+  long long pg = ranges ? xcd * perXcd + blockIdx.x / 8 : blockIdx.x / nSplits;
+  long long panel = pg * 8 + wave; // may lie past the end
 
   int *const sRw = reinterpret_cast<int *>(sW + 2 * SLAB_FLOATS) +
                    wave * (2 * ROWS * gs.fs);
@@ -998,14 +1008,14 @@ __global__ void __launch_bounds__(512, NT <= 4 ? 2 : 1)
   };
 
   Pipe pipe;
-  const bool more = pg + wgs < nGroups; // uniform over the workgroup
+  const bool more = pg + pgStep < pgEnd; // uniform over the workgroup
   if (GATHER) {
     st.bufCur = 0;
     st.bufNext = rulesPerPanel;
     fetch_rules(panel);
     w_load(0);
     keep_rules(0);
-    fetch_rules(panel + 8ll * wgs);
+    fetch_rules(panel + 8ll * pgStep);
     st.ch = 4 * q - (int)__umulhi((unsigned)(4 * q), gs.magic) * gs.nIn;
     st.rule = sRw[c * gs.fs + (int)__umulhi((unsigned)(4 * q), gs.magic)];
     if (!more)
@@ -1032,12 +1042,12 @@ __global__ void __launch_bounds__(512, NT <= 4 ? 2 : 1)
   float *const obase = out + (long long)(4 * q) * N + n0 + NT * c;
 
   auto run_panel = [&](auto guarded) {
-    const long long next = panel + 8ll * wgs;
-    const bool hasNext = pg + wgs < nGroups;
+    const long long next = panel + 8ll * pgStep;
+    const bool hasNext = pg + pgStep < pgEnd;
     if (GATHER) {
       if (hasNext)
         keep_rules(st.bufNext);
-      fetch_rules(next + 8ll * wgs);
+      fetch_rules(next + 8ll * pgStep);
     } else {
       st.nxt = hasNext ? A + row_of(next) * K + 4 * q : st.cur;
       st.wrap = (st.nxt - st.cur) - (long long)KS * T;
@@ -1055,19 +1065,19 @@ __global__ void __launch_bounds__(512, NT <= 4 ? 2 : 1)
     }
     pipe.template store<decltype(guarded)::value>(obase + panel * ROWS * N, N,
                                                   M - panel * ROWS, q, col);
-    pg += wgs;
+    pg += pgStep;
     panel = next;
     if (GATHER) {
       const int b = st.bufCur;
       st.bufCur = st.bufNext;
-      st.bufNext = pg + wgs < nGroups ? b : st.bufCur;
+      st.bufNext = pg + pgStep < pgEnd ? b : st.bufCur;
     } else {
       st.cur = st.nxt;
     }
   };
-  while (pg < nFullGroups)
+  while (pg < pgEnd && pg < nFullGroups)
     run_panel(std::false_type());
-  if (pg < nGroups) // the last group: a ragged panel, panels past the end
+  if (pg < pgEnd) // the last group: a ragged panel, panels past the end
     run_panel(std::true_type());
 }
 
