@@ -623,7 +623,7 @@ __global__ void __launch_bounds__(512)
   const long long nFull = M / ROWS;
   const long long nPanels = (M + ROWS - 1) / ROWS;
   const long long stride = (long long)wgs * 8;
-  long long panel = (long long)wave * wgs + wg;
+  long long panel = (long long)wg * 8 + wave; // a workgroup takes eight neighbouring panels: they gather common rows
   const int T = K / KS;
 
   // Where lane (c, q) finds k-steps of a panel.  Plain: a row of A.  GATHER:
