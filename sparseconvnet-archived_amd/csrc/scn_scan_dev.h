@@ -1,5 +1,5 @@
 // Device-side exclusive prefix sum by ONE workgroup of 256 lanes.  For arrays
-// up to 65536 elements this is one launch instead of the three of the tiled
+// up to SCAN1_MAX_ELEMS elements this is one launch instead of the three of the tiled
 // scan, and launch count is what small batches pay for.
 //
 // The workgroup walks the array in chunks of 8192 elements.  Every lane owns
