@@ -204,6 +204,16 @@ int scn_conv_nin_forward(scn_ctx *ctx, const float *d_in,
                          const float *d_W, const float *d_B,
                          const float *d_prelu, float *d_out, int64_t M, int N,
                          float p, int act);
+/* The same with the operand precision of scn_nin_forward: SCN_FP32, or SCN_BF16
+ * for shapes with nIn a multiple of 8, fs * nIn of 64 and N of 32 (operands
+ * rounded to bf16 on their way to the MFMA, fp32 accumulation); bit-identical to
+ * scn_gather_rows followed by scn_nin_forward with that precision. */
+int scn_conv_nin_supported_p(int fs, int nIn, int N, int precision);
+int scn_conv_nin_forward_p(scn_ctx *ctx, const float *d_in,
+                           const int32_t *d_rules, int fs, int nIn,
+                           const float *d_W, const float *d_B,
+                           const float *d_prelu, float *d_out, int64_t M, int N,
+                           float p, int act, int precision);
 /* maxPool (MaxPoolingLayer.h:6-7; MaxPoolingLayer.cu:9-72): first maximum
  * wins, negative rules skipped, choice = rule * C + channel. */
 int scn_maxpool(scn_ctx *ctx, const float *d_in, float *d_out,

@@ -1192,6 +1192,358 @@ __device__ __forceinline__ void residue8(float *v) {
     v[i] -= __uint_as_float((unsigned)to_bf16(v[i]) << 16);
 }
 
+// ---- W streamed through LDS with bf16 operands --------------------------------
+// k_nin_wstream with v_mfma_f32_16x16x32_bf16: one MFMA consumes 32 k, lane
+// (c, q) supplies the eight consecutive k = 32 t + 8 q .. + 7 of row c (two
+// 16-byte loads of fp32 A, rounded to bf16 in registers: v_cvt_pk_bf16_f32,
+// nearest even) and of its columns of W.  W is rounded on its way into LDS and
+// kept there as [group of 8 k][tile j][lane c][8 bf16] (column NT c + j), so
+// the 16 lanes that read a tile's operands read 256 contiguous bytes.  A slab is 64 k = two steps;
+// the A prefetch ring holds RD steps and the loop body is unrolled over BL
+// steps (a multiple of both), which K / 32 must be a multiple of.  Accumulation
+// and epilogue are fp32 as everywhere.  With GATHER the channels of a rule
+// must come in multiples of 8.
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ unsigned pack_bf16x2(float a, float b) {
+  floatx2 f = {a, b};
+  bf16x2 h = __builtin_convertvector(f, bf16x2);
+  return __builtin_bit_cast(unsigned, h);
+}
+__device__ __forceinline__ bf16x8 pack_bf16x8(const float4 &x, const float4 &y) {
+  uint4 r;
+  r.x = pack_bf16x2(x.x, x.y);
+  r.y = pack_bf16x2(x.z, x.w);
+  r.z = pack_bf16x2(y.x, y.y);
+  r.w = pack_bf16x2(y.z, y.w);
+  return __builtin_bit_cast(bf16x8, r);
+}
+
+template <int NT, int RD, int BL, int GRU>
+__global__ void __launch_bounds__(512, NT <= 4 ? 2 : 1)
+    k_nin_wstream_bf16(const float *__restrict__ A, const float *__restrict__ W,
+                       float *__restrict__ out, long long M, int K, int N,
+                       Epilogue ep, GatherSource gs, int nSplits) {
+  static_assert(BL % 2 == 0 && BL % RD == 0, "body = whole slabs and whole turns of the ring");
+  constexpr int ROWS = 16, KS = 32, NW = ROWS * NT;
+  constexpr bool GATHER = GRU > 0;
+  constexpr int GROUP_BYTES = NW * 16 + 16;   // one group of 8 k: NW columns x 8 bf16, padded
+  constexpr int SLAB_BYTES = 8 * GROUP_BYTES; // 64 k
+  extern __shared__ __attribute__((aligned(16))) unsigned char sWb[]; // [2][SLAB_BYTES], then the rules
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int c = lane % ROWS, q = lane / ROWS;
+  const long long nPanels = (M + ROWS - 1) / ROWS;
+  const long long nGroups = (nPanels + 7) / 8;
+  const long long nFullGroups = (M / ROWS) / 8;
+  const int T = K / KS, nSlabs = T / 2;
+  // the walk over the panel groups: as k_nin_wstream
+  const int wgs = gridDim.x / nSplits;
+  const bool ranges = nSplits == 1 && wgs % 8 == 0 && nGroups >= 2ll * wgs;
+  const int split = blockIdx.x % nSplits;
+  const int xcd = blockIdx.x % 8;
+  const long long perXcd = (nGroups + 7) / 8;
+  const int pgStep = ranges ? wgs / 8 : wgs;
+  const long long pgEnd =
+      ranges && (xcd + 1) * perXcd < nGroups ? (xcd + 1) * perXcd : nGroups;
+  const int n0 = split * NW;
+  long long pg = ranges ? xcd * perXcd + blockIdx.x / 8 : blockIdx.x / nSplits;
+  long long panel = pg * 8 + wave; // may lie past the end
+
+  int *const sRw = reinterpret_cast<int *>(sWb + 2 * SLAB_BYTES) +
+                   wave * (2 * ROWS * gs.fs);
+  const int rulesPerPanel = ROWS * gs.fs;
+  auto row_of = [&](long long pnl) {
+    long long m = pnl * ROWS + c;
+    return m < M ? m : M - 1;
+  };
+  struct {
+    const float *cur, *nxt;
+    long long wrap;
+    int bufCur, bufNext, rule, ch;
+  } st;
+  // where this lane's 8 floats of step tt are; tt >= T: step tt - T of the next panel
+  auto addr = [&](int tt) -> const float * {
+    if (!GATHER)
+      return st.cur + KS * tt + (tt >= T ? st.wrap : 0ll);
+    const float *p =
+        (st.rule >= 0 ? A + (long long)st.rule * gs.nIn : gs.zeros) + st.ch;
+    const int tn = tt + 1;
+    const int kn = KS * (tn >= T ? tn - T : tn) + 8 * q;
+    const int fn = (int)__umulhi((unsigned)kn, gs.magic);
+    st.ch = kn - fn * gs.nIn;
+    st.rule = sRw[(tn >= T ? st.bufNext : st.bufCur) + c * gs.fs + fn];
+    return p;
+  };
+  constexpr int RU = GATHER ? GRU : 1;
+  int rr[RU];
+  auto fetch_rules = [&](long long pnl) {
+    if (pnl >= nPanels)
+      pnl = nPanels - 1;
+    const long long first = pnl * rulesPerPanel, last = M * gs.fs - 1;
+#pragma unroll
+    for (int u = 0; u < RU; ++u) {
+      long long i = first + lane + 64 * u;
+      rr[u] = gs.rules[i < last ? i : last];
+    }
+  };
+  auto keep_rules = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < RU; ++u)
+      if (lane + 64 * u < rulesPerPanel)
+        sRw[buf + lane + 64 * u] = rr[u];
+  };
+
+  // a slab of this workgroup's columns of W: one item = 8 consecutive k of one
+  // column (8 loads, each coalesced across the lanes of a k-row)
+  constexpr int ITEMS = 8 * NW;
+  constexpr int WPER = (ITEMS + 511) / 512;
+  float wv[WPER][8];
+  int dst[WPER];
+  const float *src[WPER];
+#pragma unroll
+  for (int u = 0; u < WPER; ++u) {
+    int x = tid + 512 * u;
+    x = x < ITEMS ? x : ITEMS - 1; // past the end: the last item again (same value, same place)
+    const int kg = x / NW, n = x - kg * NW;
+    // column n = NT c + j is item j * 16 + c of its group: the 16 lanes that
+    // read tile j of a group read 256 contiguous bytes
+    dst[u] = kg * GROUP_BYTES + ((n % NT) * 16 + n / NT) * 16;
+    src[u] = W + (long long)(8 * kg) * N + n0 + n;
+  }
+  auto w_load = [&](int slab) {
+    const long long off = (long long)slab * 64 * N;
+#pragma unroll
+    for (int u = 0; u < WPER; ++u)
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        wv[u][i] = src[u][off + (long long)i * N];
+  };
+  auto w_store = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < WPER; ++u) {
+      asm volatile("" : "+v"(wv[u][0]), "+v"(wv[u][1]), "+v"(wv[u][2]), "+v"(wv[u][3]),
+                        "+v"(wv[u][4]), "+v"(wv[u][5]), "+v"(wv[u][6]), "+v"(wv[u][7]));
+      uint4 r;
+      r.x = pack_bf16x2(wv[u][0], wv[u][1]);
+      r.y = pack_bf16x2(wv[u][2], wv[u][3]);
+      r.z = pack_bf16x2(wv[u][4], wv[u][5]);
+      r.w = pack_bf16x2(wv[u][6], wv[u][7]);
+      *reinterpret_cast<uint4 *>(sWb + buf * SLAB_BYTES + dst[u]) = r;
+    }
+  };
+
+  float4 a[RD][2];
+  bf16x8 b[2][NT];
+  floatx4 acc[NT];
+  // this lane's W operands of step s (0, 1) of the slab in buffer buf
+  const int bLane = q * GROUP_BYTES + c * 16;
+  auto read_b = [&](int buf, int s, int slot) {
+    const unsigned char *p = sWb + buf * SLAB_BYTES + 4 * s * GROUP_BYTES + bLane;
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+      b[slot][j] = *reinterpret_cast<const bf16x8 *>(p + 256 * j);
+  };
+  auto load_a = [&](int slot, int tt) {
+    const float *p = addr(tt);
+    a[slot][0] = *reinterpret_cast<const float4 *>(p);
+    a[slot][1] = *reinterpret_cast<const float4 *>(p + 4);
+  };
+
+  const bool more = pg + pgStep < pgEnd;
+  if (GATHER) {
+    st.bufCur = 0;
+    st.bufNext = rulesPerPanel;
+    fetch_rules(panel);
+    w_load(0);
+    keep_rules(0);
+    fetch_rules(panel + 8ll * pgStep);
+    st.ch = 8 * q - (int)__umulhi((unsigned)(8 * q), gs.magic) * gs.nIn;
+    st.rule = sRw[c * gs.fs + (int)__umulhi((unsigned)(8 * q), gs.magic)];
+    if (!more)
+      st.bufNext = 0;
+  } else {
+    st.cur = A + row_of(panel) * K + 8 * q;
+  }
+  st.wrap = 0;
+#pragma unroll
+  for (int s = 0; s < RD - 1; ++s)
+    load_a(s, s);
+  if (!GATHER)
+    w_load(0);
+  w_store(0);
+  __syncthreads();
+  int cur = 0;
+  read_b(0, 0, 0);
+
+  ColEpilogue col[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+    col[j] = load_col(ep, n0 + NT * c + j);
+  float *const obase = out + (long long)(4 * q) * N + n0 + NT * c;
+
+  auto run_panel = [&](auto guarded) {
+    const long long next = panel + 8ll * pgStep;
+    const bool hasNext = pg + pgStep < pgEnd;
+    if (GATHER) {
+      if (hasNext)
+        keep_rules(st.bufNext);
+      fetch_rules(next + 8ll * pgStep);
+    } else {
+      st.nxt = hasNext ? A + row_of(next) * K + 8 * q : st.cur;
+      st.wrap = (st.nxt - st.cur) - (long long)KS * T;
+    }
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+      acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int t0 = 0; t0 < T; t0 += BL) {
+#pragma unroll
+      for (int s = 0; s < BL; ++s) {
+        const int t = t0 + s;
+        if ((s & 1) == 0) { // first step of a slab: fetch the next slab, read this slab's second step
+          const int slabNext = t / 2 + 1;
+          w_load(slabNext < nSlabs ? slabNext : 0);
+          load_a((s + RD - 1) % RD, t + RD - 1);
+          read_b(cur, 1, 1);
+        } else { // second step: hand the next slab over, read its first step
+          load_a((s + RD - 1) % RD, t + RD - 1);
+          w_store(cur ^ 1);
+          __syncthreads();
+          cur ^= 1;
+          read_b(cur, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        const bf16x8 av = pack_bf16x8(a[s % RD][0], a[s % RD][1]);
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+          acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, b[s & 1][j], acc[j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    // lane (c, q): rows 4 q + v, columns NT c + j
+    float *orow = obase + panel * ROWS * N;
+    const long long rowsLeft = M - panel * ROWS;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      if (decltype(guarded)::value && 4 * q + v >= rowsLeft)
+        continue;
+      float r[NT];
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+        r[j] = finish(acc[j][v], col[j]);
+      float *o = orow + (long long)v * N;
+      if (NT % 4 == 0) {
+#pragma unroll
+        for (int j = 0; j < NT; j += 4)
+          *reinterpret_cast<float4 *>(o + j) = make_float4(r[j], r[j + 1], r[j + 2], r[j + 3]);
+      } else if (NT % 2 == 0) {
+#pragma unroll
+        for (int j = 0; j < NT; j += 2)
+          *reinterpret_cast<float2 *>(o + j) = make_float2(r[j], r[j + 1]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+          o[j] = r[j];
+      }
+    }
+    pg += pgStep;
+    panel = next;
+    if (GATHER) {
+      const int bb = st.bufCur;
+      st.bufCur = st.bufNext;
+      st.bufNext = pg + pgStep < pgEnd ? bb : st.bufCur;
+    } else {
+      st.cur = st.nxt;
+    }
+  };
+  while (pg < pgEnd && pg < nFullGroups)
+    run_panel(std::false_type());
+  if (pg < pgEnd)
+    run_panel(std::true_type());
+}
+
+#define WSTREAM_BF16_LDS_BYTES(nw) (2 * 8 * ((nw) * 16 + 16))
+template <int NT, int RD, int BL>
+static int launch_wstream_bf16(scn_ctx *ctx, const float *A, const float *W,
+                               float *out, long long M, int K, int N,
+                               const Epilogue &ep, const GatherSource *gs) {
+  constexpr int NW = 16 * NT;
+  const int nSplits = N / NW;
+  const size_t lds =
+      WSTREAM_BF16_LDS_BYTES(NW) + (gs ? WRES_RULE_BYTES(gs->fs) : 0);
+  long long wgs = scn_ceil_div(scn_ceil_div(M, 16), 8);
+  const long long cap = (long long)ctx->numCU * (lds * 2 <= WRES_LDS_BYTES ? 2 : 1);
+  if (wgs > cap)
+    wgs = cap;
+  static std::once_flag configured;
+  int rc = SCN_OK;
+  std::call_once(configured, [&]() {
+#define SCN_WSB_LDS(G)                                                         \
+  if (hipFuncSetAttribute(                                                     \
+          reinterpret_cast<const void *>(k_nin_wstream_bf16<NT, RD, BL, G>),   \
+          hipFuncAttributeMaxDynamicSharedMemorySize,                          \
+          WRES_LDS_BYTES) != hipSuccess)                                       \
+    rc = SCN_ERR_HIP;
+    SCN_WSB_LDS(0) SCN_WSB_LDS(1) SCN_WSB_LDS(3) SCN_WSB_LDS(7)
+#undef SCN_WSB_LDS
+  });
+  SCN_REQUIRE(rc == SCN_OK, SCN_ERR_HIP, "hipFuncSetAttribute failed");
+  const dim3 grid((unsigned)(wgs * nSplits));
+#define SCN_WSB_GO(G, src)                                                     \
+  hipLaunchKernelGGL((k_nin_wstream_bf16<NT, RD, BL, G>), grid, dim3(512),     \
+                     lds, ctx->stream, A, W, out, M, K, N, ep, src, nSplits)
+  if (!gs)
+    SCN_WSB_GO(0, GatherSource());
+  else if (gs->fs <= 4)
+    SCN_WSB_GO(1, *gs);
+  else if (gs->fs <= 12)
+    SCN_WSB_GO(3, *gs);
+  else
+    SCN_WSB_GO(7, *gs);
+#undef SCN_WSB_GO
+  return SCN_OK;
+}
+
+// bf16 operands, shapes this kernel takes: K a multiple of 64, N of 32, enough
+// rows; with a gather, channels in multiples of 8.  The choice depends on
+// (M, K, N) only.
+static bool wstream_bf16_shape(long long M, int K, int N) {
+  return K % 64 == 0 && N % 32 == 0 && M >= 256;
+}
+static bool wstream_bf16_forward(scn_ctx *ctx, const float *A, const float *W,
+                                 float *out, long long M, int K, int N,
+                                 const Epilogue &ep, const GatherSource *gs) {
+  if (!wstream_bf16_shape(M, K, N) || (gs && gs->nIn % 8 != 0))
+    return false;
+  const int T = K / 32;
+  static const int widths[] = {6, 4, 2};
+  const long long groups = scn_ceil_div(scn_ceil_div(M, 16), 8);
+  int nt = 0;
+  for (int w : widths) {
+    if (N % (16 * w) != 0)
+      continue;
+    nt = w;
+    if (groups * (N / (16 * w)) >= (long long)ctx->numCU * (w <= 4 ? 2 : 1))
+      break;
+  }
+  if (nt == 0)
+    return false;
+#define SCN_WSB_CASE(NTV)                                                      \
+  case NTV:                                                                    \
+    if (T % 4 == 0)                                                            \
+      return launch_wstream_bf16<NTV, 4, 4>(ctx, A, W, out, M, K, N, ep, gs) == SCN_OK; \
+    if (T % 6 == 0)                                                            \
+      return launch_wstream_bf16<NTV, 3, 6>(ctx, A, W, out, M, K, N, ep, gs) == SCN_OK; \
+    return launch_wstream_bf16<NTV, 2, 2>(ctx, A, W, out, M, K, N, ep, gs) == SCN_OK;
+  switch (nt) {
+    SCN_WSB_CASE(2)
+    SCN_WSB_CASE(4)
+    SCN_WSB_CASE(6)
+  }
+#undef SCN_WSB_CASE
+  return false;
+}
+
 template <int WM, int WN, int NT, bool SPLIT>
 __global__ void __launch_bounds__(256)
     k_nin_mfma_bf16(const float *__restrict__ A, const float *__restrict__ W,
@@ -1397,7 +1749,12 @@ static int nin_forward(scn_ctx *ctx, const float *d_A, const float *d_W,
                    ((uintptr_t)d_W & 15) == 0 && ((uintptr_t)d_out & 15) == 0;
   // bf16 operands only where the contraction is big enough to matter; the
   // classifier head and the thin first layers stay fp32
-  if (vec && K >= 64 && act != SCN_SOFTMAX && precision != SCN_FP32) {
+  if (vec && K >= 64 && act != SCN_SOFTMAX && precision == SCN_BF16 &&
+      wstream_bf16_forward(ctx, d_A, d_W, d_out, M, K, N, ep, gs)) {
+    // W-streaming kernel with bf16 operands took it
+  } else if (vec && K >= 64 && act != SCN_SOFTMAX && precision != SCN_FP32) {
+    SCN_REQUIRE(!gs, SCN_ERR_ARG,
+                "fused convolution: shape outside the bf16 kernel's range");
     const bool split = precision == SCN_BF16X3;
     long long blocksLarge = (long long)scn_ceil_div(M, 128) * scn_ceil_div(N, 64);
     if (N <= 32)
@@ -1474,17 +1831,36 @@ extern "C" int scn_conv_nin_supported(int fs, int nIn, int N) {
   return fs >= 1 && fs <= GF_MAX_FS && nIn >= 4 && nIn % 4 == 0 &&
          nIn <= SCN_ZERO_FLOATS && N % 4 == 0;
 }
+extern "C" int scn_conv_nin_supported_p(int fs, int nIn, int N, int precision) {
+  if (!scn_conv_nin_supported(fs, nIn, N))
+    return 0;
+  if (precision == SCN_FP32)
+    return 1;
+  // bf16 operands: the shapes of the bf16 W-streaming kernel, whatever M
+  return precision == SCN_BF16 && nIn % 8 == 0 &&
+         wstream_bf16_shape(1 << 20, fs * nIn, N);
+}
 
 extern "C" int scn_conv_nin_forward(scn_ctx *ctx, const float *d_in,
                                     const int32_t *d_rules, int fs, int nIn,
                                     const float *d_W, const float *d_B,
                                     const float *d_prelu, float *d_out,
                                     int64_t M, int N, float p, int act) {
+  return scn_conv_nin_forward_p(ctx, d_in, d_rules, fs, nIn, d_W, d_B, d_prelu,
+                                d_out, M, N, p, act, SCN_FP32);
+}
+extern "C" int scn_conv_nin_forward_p(scn_ctx *ctx, const float *d_in,
+                                      const int32_t *d_rules, int fs, int nIn,
+                                      const float *d_W, const float *d_B,
+                                      const float *d_prelu, float *d_out,
+                                      int64_t M, int N, float p, int act,
+                                      int precision) {
   SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_conv_nin_forward: null context");
-  SCN_REQUIRE(scn_conv_nin_supported(fs, nIn, N), SCN_ERR_ARG,
-              "scn_conv_nin_forward: fs %d nIn %d N %d is outside the fused "
-              "kernel's range (fs <= %d, nIn and N multiples of 4)",
-              fs, nIn, N, GF_MAX_FS);
+  SCN_REQUIRE(scn_conv_nin_supported_p(fs, nIn, N, precision), SCN_ERR_ARG,
+              "scn_conv_nin_forward: fs %d nIn %d N %d precision %d is outside "
+              "the fused kernels' range (fs <= %d, nIn and N multiples of 4; "
+              "bf16: nIn of 8, fs nIn of 64, N of 32)",
+              fs, nIn, N, precision, GF_MAX_FS);
   SCN_REQUIRE(d_rules || M == 0, SCN_ERR_ARG,
               "scn_conv_nin_forward: null rules");
   SCN_REQUIRE(((uintptr_t)d_in & 15) == 0 && ((uintptr_t)d_W & 15) == 0,
@@ -1496,5 +1872,5 @@ extern "C" int scn_conv_nin_forward(scn_ctx *ctx, const float *d_in,
   gs.magic = (unsigned)((1ull << 32) / (unsigned)nIn + 1);
   gs.zeros = ctx->d_zeros;
   return nin_forward(ctx, d_in, d_W, d_B, d_prelu, d_out, M, fs * nIn, N, p,
-                     act, SCN_FP32, &gs);
+                     act, precision, &gs);
 }

@@ -231,14 +231,14 @@ static bool nin_fused(cudaMemStream &ms, SpatiallySparseBatchInterface &input,
     return false;
   const int nIn = src->nFeatures;
   const int fs = input.nFeatures / nIn;
-  if (precision != SCN_FP32 || !scn_conv_nin_supported(fs, nIn, nFeaturesOut)) {
+  if (!scn_conv_nin_supported_p(fs, nIn, nFeaturesOut, precision)) {
     gather_now(ms, *src, input);
     return false;
   }
-  SCN_CHECKED(scn_conv_nin_forward(
+  SCN_CHECKED(scn_conv_nin_forward_p(
       ms.ctx, src->sub->features.dPtr(), input.rules.dPtr(), fs, nIn, W.dPtr(),
       B.dPtr(), prelu ? prelu->dPtr() : nullptr, output.sub->features.dPtr(),
-      output.nSpatialSites, nFeaturesOut, p, act));
+      output.nSpatialSites, nFeaturesOut, p, act, precision));
   return true;
 }
 

@@ -181,6 +181,18 @@ def to_bf16(x):
                                    (3000, 1728, 64), (64, 288, 32), (2000, 64, 32)])
 @pytest.mark.parametrize("act", ["RELU", "PRELU", "NOSIGMOID"])
 def test_nin_bf16(scn, ctx, M, K, N, act):
+    check_nin_bf16(scn, ctx, M, K, N, act)
+
+
+# the bf16 W-streaming kernel with wide slices (64 and 96 columns), every depth of its prefetch ring
+# (K / 32 a multiple of 4, of 6, of neither), ragged last groups
+@pytest.mark.parametrize("M,K,N", [(66001, 1728, 64), (33005, 192, 96), (40003, 256, 96), (70001, 320, 128),
+                                   (1, 64, 32), (15, 128, 32)])
+def test_nin_bf16_streamed_w(scn, ctx, M, K, N):
+    check_nin_bf16(scn, ctx, M, K, N, "PRELU", x3=False)
+
+
+def check_nin_bf16(scn, ctx, M, K, N, act, x3=True):
     """bf16 operands, fp32 accumulation: within 2e-2 relative of the fp32
     oracle, and within 1e-4 of the same contraction with operands rounded to
     bf16 on the host (i.e. the rounding is the only difference)."""
@@ -202,11 +214,48 @@ def test_nin_bf16(scn, ctx, M, K, N, act):
     assert np.all(np.abs(got - rounded) <= 1e-4 * scale)
     if K >= 64:  # the rounding is really there: the result differs from fp32
         assert np.abs(got - want).max() > 1e-5
+    if not x3:
+        return
     # hi + lo operand pairs, three MFMAs per tile: back within the fp32 tolerance
     ctx.nin_forward(ctx.array(A), ctx.array(W), ctx.array(B), ctx.array(pr), d_out, M, K, N, 1.0, a, scn.BF16X3)
     got3 = d_out.download()
     assert np.all(np.abs(got3 - want) <= 1e-4 * scale)
     assert np.linalg.norm(got3 - want) / np.linalg.norm(want) <= 1e-4
+
+
+@pytest.mark.parametrize("rows,fs,nIn,N", [(700, 4, 32, 64), (3000, 9, 64, 96), (513, 27, 64, 64), (66001, 27, 64, 64),
+                                           (33005, 8, 24, 96), (1100, 4, 112, 160)])
+def test_fused_gather_nin_bf16_matches_the_two_kernels_bit_for_bit(scn, ctx, rows, fs, nIn, N):
+    """scn_conv_nin_forward_p with bf16 operands: the same bits as gather + bf16 NiN, and the bf16 bar against the
+    oracle."""
+    rng = np.random.default_rng(rows + fs + nIn + N)
+    nInRows = 500
+    inp = rng.uniform(-1, 1, (nInRows, nIn)).astype(np.float32)
+    rules = rng.integers(0, nInRows, (rows, fs)).astype(np.int32)
+    rules[rng.random((rows, fs)) < 0.2] = -1
+    K = fs * nIn
+    W = (rng.standard_normal((K, N)) * np.sqrt(2.0 / K)).astype(np.float32)
+    B = rng.uniform(-0.5, 0.5, N).astype(np.float32)
+    assert scn.lib().scn_conv_nin_supported_p(fs, nIn, N, scn.BF16)
+    d_in, d_rules, d_W, d_B = ctx.array(inp), ctx.array(rules), ctx.array(W), ctx.array(B)
+    fused = ctx.empty((rows, N), np.float32)
+    ctx.conv_nin_forward(d_in, d_rules, fs, nIn, d_W, d_B, None, fused, rows, N, 1.0, scn.RELU, scn.BF16)
+    g = ctx.empty((rows, K), np.float32)
+    two = ctx.empty((rows, N), np.float32)
+    ctx.gather_rows(d_in, g, d_rules, rows * fs, nIn)
+    ctx.nin_forward(g, d_W, d_B, None, two, rows, K, N, 1.0, scn.RELU, scn.BF16)
+    assert np.array_equal(fused.download(), two.download())
+    gathered = np.where(rules[:, :, None] >= 0, inp[np.maximum(rules, 0)], 0).reshape(rows, K).astype(np.float32)
+    scale = np.abs(gathered).astype(np.float64) @ np.abs(W).astype(np.float64) + np.abs(B)
+    want = orc.nin_forward(gathered, W, B, None, 1.0, scn.RELU, f64=True)
+    assert np.all(np.abs(fused.download() - want) <= 2e-2 * scale)
+    rounded = orc.nin_forward(to_bf16(gathered), to_bf16(W), B, None, 1.0, scn.RELU, f64=True)
+    assert np.all(np.abs(fused.download() - rounded) <= 1e-4 * scale)
+    # channels not in multiples of 8, a contraction not of 64, the split mode: not fused with bf16 operands
+    assert not scn.lib().scn_conv_nin_supported_p(4, 20, 64, scn.BF16)
+    assert not scn.lib().scn_conv_nin_supported_p(3, 32, 64, scn.BF16)
+    assert not scn.lib().scn_conv_nin_supported_p(4, 32, 64, scn.BF16X3)
+    assert scn.lib().scn_conv_nin_supported_p(4, 20, 64, scn.FP32)
 
 
 def test_gather_negative_rule_is_zero_row(scn, ctx):

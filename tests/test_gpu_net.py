@@ -168,12 +168,12 @@ def test_fused_convolutions_triangular(scn):
     run_config(scn, cfg, 8, triangular=True, samples=samples, fused=True)
 
 
-@pytest.mark.parametrize("precision", ["FP32", "BF16X3"])
+@pytest.mark.parametrize("precision", ["FP32", "BF16", "BF16X3"])
 def test_fused_convolutions_change_no_bit(scn, precision):
     """The same net, weights and batch with and without fusion: every
     materialised interface and the class probabilities are identical bit for
-    bit, and at least one convolution really was fused.  With bf16 operands
-    the NiN layer gathers first, so nothing may change either."""
+    bit, and the convolutions really were fused (fp32 and bf16 operands).  In
+    the hi + lo mode the NiN layer gathers first, so nothing may change either."""
     from sparseconvnet_archived_amd import hostapi, synthetic
     cfg = synthetic.config(2, batch=12)
     samples = synthetic.make_samples(cfg, 55)
@@ -202,8 +202,8 @@ def test_fused_convolutions_change_no_bit(scn, precision):
             continue
         assert np.array_equal(a["features"], b["features"])
     assert np.array_equal(out0["probabilities"], out1["probabilities"])
-    assert skipped >= (3 if precision == "FP32" else 0)
-    if precision != "FP32":
+    assert skipped >= (3 if precision != "BF16X3" else 0)
+    if precision == "BF16X3":
         assert skipped == 0
 
 
