@@ -1035,10 +1035,6 @@ __global__ void __launch_bounds__(512, NT <= 4 ? 2 : 1)
   pipe.read_w(sW + 4 * q * PITCH + NT * c, 0, 0);
 
   const float *const wl = sW + 4 * q * PITCH + NT * c;
-  ColEpilogue col[NT];
-#pragma unroll
-  for (int j = 0; j < NT; ++j)
-    col[j] = load_col(ep, n0 + NT * c + j);
   float *const obase = out + (long long)(4 * q) * N + n0 + NT * c;
 
   auto run_panel = [&](auto guarded) {
@@ -1063,6 +1059,12 @@ __global__ void __launch_bounds__(512, NT <= 4 ? 2 : 1)
                 wl + (cur ^ 1) * SLAB_FLOATS, handover);
       cur ^= 1;
     }
+    // (the columns' constants are fetched here, once per panel of K / 16
+    // steps, rather than held in registers through the loop)
+    ColEpilogue col[NT];
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+      col[j] = load_col(ep, n0 + NT * c + j);
     pipe.template store<decltype(guarded)::value>(obase + panel * ROWS * N, N,
                                                   M - panel * ROWS, q, col);
     pg += pgStep;
