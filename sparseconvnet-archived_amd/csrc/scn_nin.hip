@@ -5,6 +5,22 @@
 #include <mutex>
 #include <type_traits>
 
+// Kernel attributes (the dynamic LDS limit) are set per device: fn runs once for
+// every device a context of this process lives on, and again if it failed.
+struct OncePerDevice {
+  std::mutex m;
+  unsigned long long done = 0;
+  template <class F> int run(int device, F fn) {
+    std::lock_guard<std::mutex> lock(m);
+    if (device >= 0 && device < 64 && ((done >> device) & 1ull))
+      return SCN_OK;
+    const int rc = fn();
+    if (rc == SCN_OK && device >= 0 && device < 64)
+      done |= 1ull << device;
+    return rc;
+  }
+};
+
 int scn_squash_launch(scn_ctx *ctx, float *d_x, long long n, int logistic);
 int scn_softmax_launch(scn_ctx *ctx, const float *d_in, float *d_out,
                        long long M, int N);
@@ -810,9 +826,9 @@ static int launch_wres(scn_ctx *ctx, const float *A, const float *W, float *out,
   const long long cap = (long long)ctx->numCU * (lds * 2 <= WRES_LDS_BYTES ? 2 : 1);
   if (wgs > cap)
     wgs = cap;
-  static std::once_flag configured; // one set of attribute calls per instantiation
-  int rc = SCN_OK;
-  std::call_once(configured, [&]() {
+  static OncePerDevice configured; // one set of attribute calls per instantiation and device
+  const int rc = configured.run(ctx->device, [&]() {
+    int rc = SCN_OK;
 #define SCN_WRES_LDS(G)                                                        \
   if (hipFuncSetAttribute(                                                     \
           reinterpret_cast<const void *>(k_nin_wres<ROWS, NT, SA, G>),         \
@@ -821,6 +837,7 @@ static int launch_wres(scn_ctx *ctx, const float *A, const float *W, float *out,
     rc = SCN_ERR_HIP;
     SCN_WRES_LDS(0) SCN_WRES_LDS(1) SCN_WRES_LDS(3) SCN_WRES_LDS(7)
 #undef SCN_WRES_LDS
+    return rc;
   });
   SCN_REQUIRE(rc == SCN_OK, SCN_ERR_HIP, "hipFuncSetAttribute failed");
   const dim3 grid((unsigned)(wgs * nSplits));
@@ -1096,9 +1113,9 @@ static int launch_wstream(scn_ctx *ctx, const float *A, const float *W,
   const long long cap = (long long)ctx->numCU * (lds * 2 <= WRES_LDS_BYTES ? 2 : 1);
   if (wgs > cap)
     wgs = cap;
-  static std::once_flag configured; // one set of attribute calls per instantiation
-  int rc = SCN_OK;
-  std::call_once(configured, [&]() {
+  static OncePerDevice configured; // one set of attribute calls per instantiation and device
+  const int rc = configured.run(ctx->device, [&]() {
+    int rc = SCN_OK;
 #define SCN_WSTREAM_LDS(G)                                                     \
   if (hipFuncSetAttribute(                                                     \
           reinterpret_cast<const void *>(k_nin_wstream<NT, SA, G>),            \
@@ -1107,6 +1124,7 @@ static int launch_wstream(scn_ctx *ctx, const float *A, const float *W,
     rc = SCN_ERR_HIP;
     SCN_WSTREAM_LDS(0) SCN_WSTREAM_LDS(1) SCN_WSTREAM_LDS(3) SCN_WSTREAM_LDS(7)
 #undef SCN_WSTREAM_LDS
+    return rc;
   });
   SCN_REQUIRE(rc == SCN_OK, SCN_ERR_HIP, "hipFuncSetAttribute failed");
   const dim3 grid((unsigned)(wgs * nSplits));
@@ -1477,9 +1495,9 @@ static int launch_wstream_bf16(scn_ctx *ctx, const float *A, const float *W,
   const long long cap = (long long)ctx->numCU * (lds * 2 <= WRES_LDS_BYTES ? 2 : 1);
   if (wgs > cap)
     wgs = cap;
-  static std::once_flag configured;
-  int rc = SCN_OK;
-  std::call_once(configured, [&]() {
+  static OncePerDevice configured; // one set of attribute calls per instantiation and device
+  const int rc = configured.run(ctx->device, [&]() {
+    int rc = SCN_OK;
 #define SCN_WSB_LDS(G)                                                         \
   if (hipFuncSetAttribute(                                                     \
           reinterpret_cast<const void *>(k_nin_wstream_bf16<NT, RD, BL, G>),   \
@@ -1488,6 +1506,7 @@ static int launch_wstream_bf16(scn_ctx *ctx, const float *A, const float *W,
     rc = SCN_ERR_HIP;
     SCN_WSB_LDS(0) SCN_WSB_LDS(1) SCN_WSB_LDS(3) SCN_WSB_LDS(7)
 #undef SCN_WSB_LDS
+    return rc;
   });
   SCN_REQUIRE(rc == SCN_OK, SCN_ERR_HIP, "hipFuncSetAttribute failed");
   const dim3 grid((unsigned)(wgs * nSplits));
