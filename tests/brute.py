@@ -109,3 +109,56 @@ def random_samples(rng, batch, d, nIn, density, with_bg=True, shuffle=True):
             row += 1
         samples.append((bg, mp))
     return samples, row
+
+
+def coords_of(key, side, d):
+    c = []
+    for _ in range(d):
+        c.append(key % side)
+        key = key // side
+    return c[::-1]  # most significant axis first
+
+
+def rules_vectorized(d, batch, sIn, sOut, size, stride, gin):
+    """The square rule book with minActive 1 once more, in whole-array numpy, for inputs too large for rules():
+    gridRules (Regions.cu:557-652) under ascending-key iteration.
+    gin = (sample, key, row, background) of the input grids.  Returns (sample, key, row) of the output sites,
+    background row per sample (-1: none), number of rows, and the rules [rows x size^d]."""
+    s, k, r, bg = gin
+    volIn, volOut = sIn ** d, sOut ** d
+    dense = np.repeat(np.asarray(bg, np.int64)[:, None], volIn, 1)  # what a rule says for an empty cell
+    dense[s, k] = r
+    # owner of an output site: the smallest active input key in its window; a site exists iff it has one.
+    # For one window offset, distinct input sites name distinct output sites, so a plain indexed update does.
+    s64, k64 = np.asarray(s, np.int64), np.asarray(k, np.int64)
+    ic = coords_of(k64, sIn, d)
+    owner = np.full(batch * volOut, np.iinfo(np.int64).max, np.int64)
+    offs = np.stack(np.meshgrid(*[np.arange(size)] * d, indexing="ij"), -1).reshape(-1, d)
+    for off in offs:
+        valid, okey = np.ones(len(k64), bool), np.zeros(len(k64), np.int64)
+        for a in range(d):
+            t = ic[a] - off[a]
+            valid &= (t >= 0) & (t % stride == 0) & (t // stride < sOut)
+            okey = okey * sOut + t // stride
+        idx = s64[valid] * volOut + okey[valid]
+        owner[idx] = np.minimum(owner[idx], k64[valid])
+    owner = owner.reshape(batch, volOut)
+    bs, ks = np.nonzero(owner != np.iinfo(np.int64).max)
+    order = np.lexsort((ks, owner[bs, ks], bs))  # by sample, then owner key, then output key
+    bs, ks = bs[order], ks[order]
+    per = np.bincount(bs, minlength=batch)
+    notFull = per < volOut
+    # rows: a sample's sites, then its background row if the sample is not full
+    before = np.concatenate([[0], np.cumsum(per + notFull)[:-1]])
+    rows = before[bs] + (np.arange(len(bs)) - np.concatenate([[0], np.cumsum(per)[:-1]])[bs])
+    bgOut = np.where(notFull, before + per, -1)
+    nRows = int((per + notFull).sum())
+    rules = np.empty((nRows, size ** d), np.int64)
+    oc = coords_of(ks, sOut, d)
+    for q, off in enumerate(offs):
+        kin = np.zeros(len(ks), np.int64)
+        for a in range(d):
+            kin = kin * sIn + (oc[a] * stride + off[a])
+        rules[rows, q] = dense[bs, kin]
+    rules[bgOut[notFull]] = np.asarray(bg, np.int64)[notFull][:, None]
+    return (bs, ks, rows), bgOut, nRows, rules

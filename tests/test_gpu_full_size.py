@@ -1,0 +1,138 @@
+"""The headline configurations at their full batch sizes, checked through properties that do not need the oracle:
+every rule book is rebuilt here with numpy from the grids alone (which sites exist, which rows they get, what each
+rule names), every feature layer is checked against what its definition says of its input (gather = copy through
+the rules, max-pool = first maximum, NiN on a sample of rows in float64, soft-max rows sum to one), and a sample's
+result must not depend on what else is in the batch."""
+import numpy as np
+import pytest
+
+from brute import rules_vectorized
+
+pytestmark = pytest.mark.gpu
+
+
+def layer_geometry(stack):
+    """per net layer: ("conv" | "pool", size, stride), ("nin",) or ("terminal",), in the order the builders add them."""
+    out = []
+    for call in stack:
+        if call[0] == "addLeNetLayerMP":
+            _, nF, fs, fstride, ps, pstride = call[:6]
+            if fs > 1:
+                out.append(("conv", fs, fstride))
+            out.append(("nin",))
+            if ps > 1:
+                out.append(("pool", ps, pstride))
+        elif call[0] == "addTerminalPoolingLayer":
+            out.append(("terminal",))
+        elif call[0] == "addSoftmaxLayer":
+            out.append(("nin",))
+    return out
+
+
+def check_net(scn, number, batch, seed, nin_rows=1500, fused=False, max_rows=1 << 16):
+    from sparseconvnet_archived_amd import hostapi, synthetic
+    cfg = synthetic.config(number, batch=batch)
+    d = cfg.dimension
+    net = hostapi.Net(d, cfg.nInputFeatures, cfg.nClasses, nTop=1, threads=2)
+    cfg.build(net)
+    net.setFusedConvolutions(fused)
+    weights = synthetic.he_normal_weights(net.layers(), seed + 1)
+    for i, (W, B, pr) in weights.items():
+        net.set_weights(i, W, B, pr)
+    samples = synthetic.make_samples(cfg, seed)
+    ds = hostapi.Dataset(cfg.name, cfg.nInputFeatures, max(cfg.nClasses, 1), hostapi.TESTBATCH)
+    for pts, f, label in samples:
+        ds.add_points(d, cfg.lattice, pts, f, label)
+    net.begin(ds, batch)
+    assert net.next_batch()
+    layers = net.layers()
+    geo = layer_geometry(cfg.stack)
+    assert len(geo) == len(layers)
+    rng = np.random.default_rng(seed)
+    prev, before = net.interface(0), None
+    for i, (g, l) in enumerate(zip(geo, layers)):
+        cur = net.interface(i + 1)
+        print("layer", i, l["kind"], g, "rows", cur["nSpatialSites"], flush=True)
+        fin, fout = prev["features"], cur["features"]
+        assert l["kind"].startswith({"conv": "conv", "pool": "maxpool", "nin": "nin", "terminal": "terminal"}[g[0]])
+        if g[0] in ("conv", "pool"):
+            (bs, ks, rows), bgOut, nRows, rules = rules_vectorized(
+                d, batch, prev["spatialSize"], cur["spatialSize"], g[1], g[2], prev["grids"])
+            assert cur["nSpatialSites"] == nRows
+            s2, k2, r2, b2 = cur["grids"]
+            o = np.lexsort((k2, s2))
+            o2 = np.lexsort((ks, bs))
+            assert np.array_equal(s2[o], bs[o2]) and np.array_equal(k2[o], ks[o2])  # the same sites exist
+            assert np.array_equal(r2[o], rows[o2])  # ... and have the same rows
+            assert np.array_equal(b2, bgOut)
+            got = cur["rules"].reshape(nRows, -1)
+            assert np.array_equal(got, rules)
+            pick = np.arange(nRows) if nRows <= max_rows else np.sort(rng.choice(nRows, max_rows, replace=False))
+            if g[0] == "conv":
+                if fout is None:  # the gather runs inside the next NiN kernel
+                    assert fused
+                else:
+                    assert np.array_equal(fout[pick], fin[got[pick]].reshape(len(pick), -1))  # copy through the rules
+            else:
+                cand = fin[got[pick]]  # [rows x window x channels]
+                assert np.array_equal(fout[pick], cand.max(1))
+                C_ = fin.shape[1]
+                ch = cur["choices"].reshape(nRows, C_)[pick]
+                # dMaxPool keeps the first maximum of the window; the choice is its element index in the input
+                assert np.array_equal(ch, np.take_along_axis(got[pick], cand.argmax(1), 1) * C_ + np.arange(C_))
+        elif g[0] == "nin":
+            W, B, pr = weights[i]
+            nR = cur["nSpatialSites"]
+            pick = rng.choice(nR, min(nin_rows, nR), replace=False)
+            if fin is None:  # rows of the convolution's output, gathered here
+                A = before["features"][prev["rules"].reshape(nR, -1)[pick]].reshape(len(pick), -1)
+            else:
+                A = fin[pick]
+            z = A.astype(np.float64) @ W.astype(np.float64) + B
+            act = l["act"]
+            if act == synthetic.SOFTMAX:
+                assert np.allclose(fout.sum(1), 1, atol=1e-4)
+                e = np.exp(z - z.max(1, keepdims=True))
+                want = e / e.sum(1, keepdims=True)
+                assert np.allclose(fout[pick], want, rtol=1e-3, atol=1e-6)
+            else:
+                slope = {synthetic.RELU: 0.0, synthetic.PRELU: None}.get(act, 1.0)
+                want = np.where(z > 0, z, z * (pr if slope is None else slope))
+                scale = np.abs(A).astype(np.float64) @ np.abs(W).astype(np.float64) + np.abs(B)
+                assert np.all(np.abs(fout[pick] - want) <= 1e-4 * scale)
+        else:  # terminal pooling: a sample's row is the mean of its rows (TerminalPoolingLayer.cu:9-30)
+            s, k, r, bg = prev["grids"]
+            assert cur["nSpatialSites"] == batch
+            sums = np.zeros((batch, fin.shape[1]), np.float64)
+            np.add.at(sums, s, fin[r].astype(np.float64))
+            n = np.bincount(s, minlength=batch)
+            want = np.where(n[:, None] > 0, sums / np.maximum(n, 1)[:, None], fin[bg])  # an empty sample: its background
+            assert np.allclose(fout, want, rtol=1e-4, atol=1e-6)
+        before, prev = prev, cur
+    out = net.batch_outputs() if cfg.nClasses > 1 else None
+    net.end()
+    return net, ds, samples, out
+
+
+def test_config2_full_batch_rule_books_and_layers(scn):
+    net, ds, samples, out = check_net(scn, 2, 100, 2015)
+    # a sample's probabilities do not depend on the rest of the batch
+    from sparseconvnet_archived_amd import hostapi
+    for pickOne in (0, 57, 99):
+        one = hostapi.Dataset("one", 3, 100, hostapi.TESTBATCH)
+        pts, f, label = samples[pickOne]
+        one.add_points(2, 96, pts, f, label)
+        net.begin(one, 1)
+        assert net.next_batch()
+        alone = net.batch_outputs()["probabilities"][0]
+        net.end()
+        # (other kernels serve a batch of one: equal to rounding, not to the bit)
+        assert np.allclose(alone, out["probabilities"][pickOne], rtol=1e-3, atol=1e-6)
+    net.close()
+
+
+@pytest.mark.parametrize("number,batch,fused", [(1, 16, False), (3, 32, False), (4, 128, False), (4, 128, True),
+                                                (5, 96, True)])
+def test_full_batch_rule_books_and_layers(scn, number, batch, fused):
+    net, ds, samples, out = check_net(scn, number, batch, 100 * number + 5, fused=fused)
+    net.close()

@@ -91,6 +91,26 @@ def test_square_rules_vs_brute_force(d, size, stride, nOut, minActive):
         assert grids_as_dicts(out) == want_out
 
 
+@pytest.mark.parametrize("d,size,stride,nOut", GEOMS)
+def test_whole_array_rule_book_vs_brute_force(d, size, stride, nOut):
+    """brute.rules_vectorized (what the full-size GPU tests check against) agrees with the per-site brute force."""
+    rng = np.random.default_rng(77 + 1000 * d + 100 * size + 10 * stride + nOut)
+    nIn = size + (nOut - 1) * stride
+    for trial in range(12):
+        density = [0.05, 0.2, 0.5, 0.9, 1.0, 0.0][trial % 6]
+        batch = 1 + trial % 3
+        samples, _ = brute.random_samples(rng, batch, d, nIn, density)
+        want_rules, want_n, want_out = brute.rules(samples, d, nIn, nOut, size, stride, 1)
+        flat = to_grids(samples).flat()
+        (bs, ks, rows), bgOut, n, rules = brute.rules_vectorized(d, batch, nIn, nOut, size, stride, flat)
+        assert n == want_n
+        assert np.array_equal(rules.ravel(), want_rules)
+        for i, (bg, grid) in enumerate(want_out):
+            assert bgOut[i] == bg
+            m = bs == i
+            assert dict(zip(ks[m].tolist(), rows[m].tolist())) == grid
+
+
 def test_square_rules_valid_vs_brute_force():
     rng = np.random.default_rng(7)
     for nOut in (1, 2, 4, 7):
