@@ -227,6 +227,60 @@ int scn_terminal_pool(scn_ctx *ctx, const float *d_in, float *d_out,
 int scn_softmax_rows(scn_ctx *ctx, const float *d_in, float *d_out, int64_t M,
                      int N);
 
+/* ---- backward pass and weight update (training) -------------------------- */
+/* dDerivativeOfCostWRTpreSoftmaxTopLevelWeights (SoftmaxClassifier.cu:7-14):
+ * delta[k][i] = probs[k][i] - (i == labels[k]), the gradient of the negative
+ * log-likelihood with respect to the soft-max layer's input. */
+int scn_softmax_grad(scn_ctx *ctx, const float *d_probs,
+                     const int32_t *d_labels, float *d_delta, int64_t batch,
+                     int N);
+/* What NetworkInNetwork(PReLU)Layer::backwards does to the output gradient
+ * before the two matrix products: applySigmoidBackProp in place
+ * (NetworkInNetworkLayer.cu:222, SigmoidLayer.cu:23-177 and :224-262; the
+ * derivative is written through the layer's output b: ReLU and the leaky
+ * forms test b > 0, tanh is (1 + b)(1 - b), the logistic b(1 - b), soft-max
+ * and none pass the gradient through) or PReLUBackprop
+ * (NetworkInNetworkPReLULayer.cu:25-47: dprelu[c] = sum d * (b > 0 ? 0 :
+ * b / alpha_c), then d *= b > 0 ? 1 : alpha_c), and columnSum of the result
+ * into the bias gradient (NetworkInNetworkLayer.cu:84-105).  d_db[N] and, for
+ * SCN_PRELU, d_dprelu[N] are overwritten. */
+int scn_activation_backward(scn_ctx *ctx, const float *d_out, float *d_delta,
+                            int64_t M, int N, int act, const float *d_prelu,
+                            float *d_db, float *d_dprelu);
+/* d_rowMajorSGEMM_alphaAtB_betaC with alpha 1, beta 0 (utilities.cu:144-152;
+ * call site NetworkInNetworkLayer.cu:225-228): dW[K x N] = A^T D, A [M x K],
+ * D [M x N], all row-major.  fp32 MFMA, fp32 atomics across row ranges. */
+int scn_sgemm_AtB(scn_ctx *ctx, const float *d_A, const float *d_D,
+                  float *d_dW, int64_t M, int K, int N);
+/* d_rowMajorSGEMM_alphaABt_betaC with alpha 1, beta 0 (utilities.cu:153-161;
+ * call site NetworkInNetworkLayer.cu:269-272): dA[M x K] = D[M x N] W^T,
+ * W [K x N].  d_workspace holds scn_sgemm_ABt_workspace(N, K) floats (the
+ * transposed weights, which the forward contraction kernels then stream). */
+int64_t scn_sgemm_ABt_workspace(int N, int K);
+int scn_sgemm_ABt(scn_ctx *ctx, const float *d_D, const float *d_W,
+                  float *d_dA, int64_t M, int N, int K, float *d_workspace);
+/* dGradientDescent / dGradientDescentKeepPositive (NetworkInNetworkLayer.cu:
+ * 27-41, NetworkInNetworkPReLULayer.cu:68-83), "NAG light": w -= m mu;
+ * m = mu m - lr (1 - mu) d; w += m (1 + mu); keepPositive clamps w at 0.001. */
+int scn_nag_update(scn_ctx *ctx, const float *d_delta, float *d_momentum,
+                   float *d_weights, int64_t n, float learningRate,
+                   float momentum, int keepPositive);
+/* propBackwardFromMatrixMultiply (ConvolutionalLayer.cu:42-72):
+ * din[rules[c] * nIn + j] += dconv[c * nIn + j], c < count; the caller zeroes
+ * din first (ConvolutionalLayer.cu:141).  Negative rules are skipped. */
+int scn_gather_rows_backward(scn_ctx *ctx, float *d_din, const float *d_dconv,
+                             const int32_t *d_rules, int64_t count, int nIn);
+/* maxPoolBackProp (MaxPoolingLayer.cu:74-93): din[choice[i]] += dout[i] over
+ * the count x C elements of dout; the caller zeroes din first. */
+int scn_maxpool_backward(scn_ctx *ctx, float *d_din, const float *d_dout,
+                         int64_t count, int C, const int32_t *d_choice);
+/* terminalPoolBackProp (TerminalPoolingLayer.cu:48-73): every row listed for
+ * sample b before the first negative rule is assigned dout[b] / (number of
+ * rows listed); the caller zeroes din first. */
+int scn_terminal_pool_backward(scn_ctx *ctx, float *d_din, const float *d_dout,
+                               const int32_t *d_rules, int64_t count, int C,
+                               int S);
+
 /* ---- per-kernel timing -------------------------------------------------- */
 /* HIP events recorded on the context's stream around every kernel of one
  * family; off by default.  The reference only times whole dataset passes
@@ -241,7 +295,8 @@ enum {
   SCN_K_SOFTMAX = 6,
   SCN_K_CONV_NIN = 7, /* gather fused into the NiN contraction */
   SCN_K_PROBE = 8,    /* scn_prof_probe: what a span costs by itself */
-  SCN_K_COUNT = 9
+  SCN_K_BACKWARD = 9, /* every kernel of the backward pass and the update */
+  SCN_K_COUNT = 10
 };
 int scn_prof_enable(scn_ctx *ctx, int on);
 /* label attached to the spans recorded from now on (e.g. the layer index) */

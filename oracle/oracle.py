@@ -55,6 +55,14 @@ def _load():
         "orc_terminal_pool": (None, [vp, vp, vp, i64, C.c_int, C.c_int]),
         "orc_top_indices": (None, [vp, C.c_int, C.c_int, vp]),
         "orc_softmax_classifier": (C.c_int, [vp, vp, C.c_int, C.c_int, C.c_int, vp, vp]),
+        "orc_softmax_grad": (None, [vp, vp, vp, i64, C.c_int]),
+        "orc_activation_backward": (None, [vp, vp, i64, C.c_int, C.c_int, vp, vp, vp]),
+        "orc_sgemm_AtB": (None, [vp, vp, vp, i64, C.c_int, C.c_int]),
+        "orc_sgemm_ABt": (None, [vp, vp, vp, i64, C.c_int, C.c_int]),
+        "orc_nag_update": (None, [vp, vp, vp, i64, f32, f32, C.c_int]),
+        "orc_gather_rows_backward": (None, [vp, vp, vp, i64, C.c_int]),
+        "orc_maxpool_backward": (None, [vp, vp, i64, C.c_int, vp]),
+        "orc_terminal_pool_backward": (None, [vp, vp, vp, i64, C.c_int, C.c_int]),
         "orc_set_threads": (None, [C.c_int]),
         "orc_get_threads": (C.c_int, []),
     }
@@ -235,3 +243,67 @@ def softmax_classifier(probs, labels, nTop):
     nll = C.c_float(0.0)
     mistakes = lib.orc_softmax_classifier(_p(probs), _p(labels), batch, nClasses, nTop, _p(pred), C.byref(nll))
     return pred, int(mistakes), float(nll.value)
+
+
+# ---- backward pass -------------------------------------------------------
+def softmax_grad(probs, labels):
+    probs, labels = _f32(probs), _i32(labels)
+    out = np.empty_like(probs)
+    lib.orc_softmax_grad(_p(probs), _p(labels), _p(out), probs.shape[0], probs.shape[1])
+    return out
+
+
+def activation_backward(out, delta, act, prelu=None):
+    """(delta multiplied by the activation's derivative, bias gradient, PReLU slope gradient or None)"""
+    out, delta = _f32(out), np.array(delta, np.float32, order="C")
+    M, N = out.shape
+    db = np.empty(N, np.float32)
+    pr = _f32(prelu) if prelu is not None else None
+    dpr = np.empty(N, np.float32) if prelu is not None else None
+    lib.orc_activation_backward(_p(out), _p(delta), M, N, int(act), _p(pr) if pr is not None else None, _p(db),
+                                _p(dpr) if dpr is not None else None)
+    return delta, db, dpr
+
+
+def sgemm_AtB(A, D):
+    A, D = _f32(A), _f32(D)
+    out = np.empty((A.shape[1], D.shape[1]), np.float32)
+    lib.orc_sgemm_AtB(_p(A), _p(D), _p(out), A.shape[0], A.shape[1], D.shape[1])
+    return out
+
+
+def sgemm_ABt(D, W):
+    D, W = _f32(D), _f32(W)
+    out = np.empty((D.shape[0], W.shape[0]), np.float32)
+    lib.orc_sgemm_ABt(_p(D), _p(W), _p(out), D.shape[0], D.shape[1], W.shape[0])
+    return out
+
+
+def nag_update(delta, mom, wts, learningRate, momentum, keepPositive=False):
+    """updates mom and wts (float32 arrays) in place"""
+    delta = _f32(delta)
+    assert mom.dtype == np.float32 and wts.dtype == np.float32 and mom.flags.c_contiguous and wts.flags.c_contiguous
+    lib.orc_nag_update(_p(delta), _p(mom), _p(wts), wts.size, float(learningRate), float(momentum), int(keepPositive))
+
+
+def gather_rows_backward(dconv, rules, nRowsIn, nIn):
+    dconv, rules = _f32(dconv), _i32(rules)
+    din = np.zeros((nRowsIn, nIn), np.float32)
+    lib.orc_gather_rows_backward(_p(din), _p(dconv), _p(rules), rules.size, nIn)
+    return din
+
+
+def maxpool_backward(dout, choice, nRowsIn):
+    dout, choice = _f32(dout), _i32(choice)
+    count, Cn = dout.shape
+    din = np.zeros((nRowsIn, Cn), np.float32)
+    lib.orc_maxpool_backward(_p(din), _p(dout), count, Cn, _p(choice))
+    return din
+
+
+def terminal_pool_backward(dout, rules, S, nRowsIn):
+    dout, rules = _f32(dout), _i32(rules)
+    count, Cn = dout.shape
+    din = np.zeros((nRowsIn, Cn), np.float32)
+    lib.orc_terminal_pool_backward(_p(din), _p(dout), _p(rules), count, Cn, S)
+    return din

@@ -15,6 +15,10 @@
  *   gather / max-pool    brute force on random inputs, tie and negative-rule cases
  *   NiN                  numpy float64 GEMM, W = I, W = 0, single non-zero
  *   softmax / top-k      closed forms
+ *   backward pass        gather / max-pool / terminal: adjoint identity <P x, y> = <x, P^T y>;
+ *                        soft-max gradient, activation derivatives, dW, dB, dA, dPReLU: central finite
+ *                        differences of a float64 numpy loss; weight update: algebraic identities
+ *                        (momentum 0 is plain gradient descent; w' = w + m' + mu (m' - m))
  * Parity unpinned (no reference vector can exist in this build): the row order
  * the reference gets from google::dense_hash_map iteration (its default map),
  * and cuBLAS sgemm's summation order.
@@ -759,4 +763,144 @@ int orc_softmax_classifier(const float *probs, const int32_t *labels,
         mistakes--;
   }
   return mistakes;
+}
+
+/* ---------- backward pass (training) ---------- */
+
+/* dDerivativeOfCostWRTpreSoftmaxTopLevelWeights, SoftmaxClassifier.cu:7-14 */
+void orc_softmax_grad(const float *probs, const int32_t *labels, float *delta,
+                      int64_t batch, int N) {
+  for (int64_t k = 0; k < batch; ++k)
+    for (int i = 0; i < N; ++i)
+      delta[k * N + i] = probs[k * N + i] - (i == labels[k]);
+}
+
+/* applySigmoidBackProp in place as NetworkInNetworkLayer::backwards calls it
+ * (NetworkInNetworkLayer.cu:222; kernels SigmoidLayer.cu:23-177), or
+ * PReLUBackprop (NetworkInNetworkPReLULayer.cu:25-47), followed by columnSum
+ * (NetworkInNetworkLayer.cu:84-105).  The sums are taken in double and
+ * rounded once (the reference's atomics fix no order). */
+void orc_activation_backward(const float *out, float *delta, int64_t M, int N,
+                             int act, const float *prelu, float *db,
+                             float *dprelu) {
+  double *s = (double *)calloc((size_t)N, sizeof(double));
+  double *t = (double *)calloc((size_t)N, sizeof(double));
+  for (int64_t r = 0; r < M; ++r)
+    for (int c = 0; c < N; ++c) {
+      float b = out[r * N + c], d = delta[r * N + c];
+      switch (act) {
+      case A_RELU:
+        d = b > 0 ? d : 0;
+        break;
+      case A_LEAKYRELU:
+        d = b > 0 ? d : d * 0.01f;
+        break;
+      case A_VLEAKYRELU:
+        d = b > 0 ? d : d * 0.333f;
+        break;
+      case A_TANH:
+        d = d * (1 + b) * (1 - b);
+        break;
+      case A_SIGMOID:
+        d = d * b * (1 - b);
+        break;
+      case A_PRELU:
+        t[c] += d * (b > 0 ? 0 : b / prelu[c]);
+        d = b > 0 ? d : d * prelu[c];
+        break;
+      default:
+        break;
+      }
+      delta[r * N + c] = d;
+      s[c] += d;
+    }
+  for (int c = 0; c < N; ++c) {
+    db[c] = (float)s[c];
+    if (act == A_PRELU)
+      dprelu[c] = (float)t[c];
+  }
+  free(s);
+  free(t);
+}
+
+/* d_rowMajorSGEMM_alphaAtB_betaC, alpha 1 beta 0 (utilities.cu:144-152):
+ * dW[K x N] = A^T D, accumulated in double. */
+void orc_sgemm_AtB(const float *A, const float *D, float *dW, int64_t M, int K,
+                   int N) {
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+  for (int k = 0; k < K; ++k) {
+    double *acc = (double *)calloc((size_t)N, sizeof(double));
+    for (int64_t m = 0; m < M; ++m) {
+      double a = A[m * K + k];
+      const float *d = D + m * N;
+      for (int n = 0; n < N; ++n)
+        acc[n] += a * (double)d[n];
+    }
+    for (int n = 0; n < N; ++n)
+      dW[(int64_t)k * N + n] = (float)acc[n];
+    free(acc);
+  }
+}
+
+/* d_rowMajorSGEMM_alphaABt_betaC, alpha 1 beta 0 (utilities.cu:153-161):
+ * dA[M x K] = D W^T, accumulated in double. */
+void orc_sgemm_ABt(const float *D, const float *W, float *dA, int64_t M, int N,
+                   int K) {
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+  for (int64_t m = 0; m < M; ++m)
+    for (int k = 0; k < K; ++k) {
+      double acc = 0;
+      for (int n = 0; n < N; ++n)
+        acc += (double)D[m * N + n] * (double)W[(int64_t)k * N + n];
+      dA[m * K + k] = (float)acc;
+    }
+}
+
+/* dGradientDescent / dGradientDescentKeepPositive
+ * (NetworkInNetworkLayer.cu:27-41, NetworkInNetworkPReLULayer.cu:68-83) */
+void orc_nag_update(const float *delta, float *mom, float *wts, int64_t n,
+                    float learningRate, float momentum, int keepPositive) {
+  for (int64_t j = 0; j < n; ++j) {
+    float w = wts[j], m = mom[j], d = delta[j];
+    w -= m * momentum;
+    m = momentum * m - learningRate * (1 - momentum) * d;
+    w += m * (1 + momentum);
+    if (keepPositive)
+      w = (w > 0.001f) ? w : 0.001f;
+    wts[j] = w;
+    mom[j] = m;
+  }
+}
+
+/* dPropBackwardFromMatrixMultiplyOutput (ConvolutionalLayer.cu:42-63); din is
+ * zeroed by the caller.  Summed in entry order. */
+void orc_gather_rows_backward(float *din, const float *dconv,
+                              const int32_t *rules, int64_t count, int nIn) {
+  for (int64_t c = 0; c < count; ++c)
+    if (rules[c] >= 0)
+      for (int j = 0; j < nIn; ++j)
+        din[(int64_t)rules[c] * nIn + j] += dconv[c * nIn + j];
+}
+
+/* dMaxPoolBackProp (MaxPoolingLayer.cu:74-82) */
+void orc_maxpool_backward(float *din, const float *dout, int64_t count, int C,
+                          const int32_t *choice) {
+  for (int64_t j = 0; j < count * C; ++j)
+    din[choice[j]] += dout[j];
+}
+
+/* dTerminalPoolBackProp (TerminalPoolingLayer.cu:48-62): assignment, not sum */
+void orc_terminal_pool_backward(float *din, const float *dout,
+                                const int32_t *rules, int64_t count, int C,
+                                int S) {
+  for (int64_t b = 0; b < count; ++b) {
+    int maxP = 0;
+    while (maxP < S && rules[b * S + maxP] >= 0)
+      ++maxP;
+    for (int j = 0; j < C; ++j) {
+      float t = dout[b * C + j] / maxP;
+      for (int p = 0; p < maxP; ++p)
+        din[(int64_t)rules[b * S + p] * C + j] = t;
+    }
+  }
 }

@@ -104,6 +104,26 @@ int orc_softmax_classifier(const float *probs, const int32_t *labels,
 void orc_set_threads(int n); /* OpenMP threads for the numeric loops */
 int orc_get_threads(void);
 
+/* ---- backward pass (training); citations in scn_oracle.c ---- */
+void orc_softmax_grad(const float *probs, const int32_t *labels, float *delta,
+                      int64_t batch, int N);
+void orc_activation_backward(const float *out, float *delta, int64_t M, int N,
+                             int act, const float *prelu, float *db,
+                             float *dprelu);
+void orc_sgemm_AtB(const float *A, const float *D, float *dW, int64_t M, int K,
+                   int N);
+void orc_sgemm_ABt(const float *D, const float *W, float *dA, int64_t M, int N,
+                   int K);
+void orc_nag_update(const float *delta, float *mom, float *wts, int64_t n,
+                    float learningRate, float momentum, int keepPositive);
+void orc_gather_rows_backward(float *din, const float *dconv,
+                              const int32_t *rules, int64_t count, int nIn);
+void orc_maxpool_backward(float *din, const float *dout, int64_t count, int C,
+                          const int32_t *choice);
+void orc_terminal_pool_backward(float *din, const float *dout,
+                                const int32_t *rules, int64_t count, int C,
+                                int S);
+
 #ifdef __cplusplus
 }
 #endif

@@ -20,8 +20,9 @@ HEADER = os.path.join(ROOT, "include", "scn_hip.h")
 NOSIGMOID, RELU, VLEAKYRELU, LEAKYRELU, TANH, SOFTMAX, PRELU, SIGMOID = range(8)
 FP32, BF16, BF16X3 = 0, 1, 2
 OK, ERR_ARG, ERR_HIP, ERR_CAPACITY, ERR_STATE = range(5)
-K_GRID_BUILD, K_RULES, K_GATHER, K_NIN, K_MAXPOOL, K_TERMINAL, K_SOFTMAX, K_CONV_NIN, K_PROBE = range(9)
-KERNEL_FAMILIES = ["grid_build", "rules", "gather", "nin", "maxpool", "terminal", "softmax", "conv_nin", "probe"]
+K_GRID_BUILD, K_RULES, K_GATHER, K_NIN, K_MAXPOOL, K_TERMINAL, K_SOFTMAX, K_CONV_NIN, K_PROBE, K_BACKWARD = range(10)
+KERNEL_FAMILIES = ["grid_build", "rules", "gather", "nin", "maxpool", "terminal", "softmax", "conv_nin", "probe",
+                   "backward"]
 
 
 class ScnError(RuntimeError):
@@ -101,6 +102,15 @@ def lib():
         "scn_maxpool": (C.c_int, [vp, vp, vp, vp, i64, C.c_int, C.c_int, vp]),
         "scn_terminal_pool": (C.c_int, [vp, vp, vp, vp, i64, C.c_int, C.c_int]),
         "scn_softmax_rows": (C.c_int, [vp, vp, vp, i64, C.c_int]),
+        "scn_softmax_grad": (C.c_int, [vp, vp, vp, vp, i64, C.c_int]),
+        "scn_activation_backward": (C.c_int, [vp, vp, vp, i64, C.c_int, C.c_int, vp, vp, vp]),
+        "scn_sgemm_AtB": (C.c_int, [vp, vp, vp, vp, i64, C.c_int, C.c_int]),
+        "scn_sgemm_ABt_workspace": (i64, [C.c_int, C.c_int]),
+        "scn_sgemm_ABt": (C.c_int, [vp, vp, vp, vp, i64, C.c_int, C.c_int, vp]),
+        "scn_nag_update": (C.c_int, [vp, vp, vp, vp, i64, f32, f32, C.c_int]),
+        "scn_gather_rows_backward": (C.c_int, [vp, vp, vp, vp, i64, C.c_int]),
+        "scn_maxpool_backward": (C.c_int, [vp, vp, vp, i64, C.c_int, vp]),
+        "scn_terminal_pool_backward": (C.c_int, [vp, vp, vp, vp, i64, C.c_int, C.c_int]),
         "scn_prof_enable": (C.c_int, [vp, C.c_int]),
         "scn_prof_reset": (C.c_int, [vp]),
         "scn_prof_probe": (C.c_int, [vp, C.c_int]),
@@ -242,6 +252,35 @@ class Context:
 
     def softmax_rows(self, d_in, d_out, M, N):
         _check(lib().scn_softmax_rows(self.h, d_in.ptr, d_out.ptr, M, N))
+
+    # ---- backward pass
+    def softmax_grad(self, d_probs, d_labels, d_delta, batch, N):
+        _check(lib().scn_softmax_grad(self.h, d_probs.ptr, d_labels.ptr, d_delta.ptr, batch, N))
+
+    def activation_backward(self, d_out, d_delta, M, N, act, d_prelu, d_db, d_dprelu):
+        _check(lib().scn_activation_backward(self.h, d_out.ptr, d_delta.ptr, M, N, act,
+                                             d_prelu.ptr if d_prelu is not None else None, d_db.ptr,
+                                             d_dprelu.ptr if d_dprelu is not None else None))
+
+    def sgemm_AtB(self, d_A, d_D, d_dW, M, K, N):
+        _check(lib().scn_sgemm_AtB(self.h, d_A.ptr, d_D.ptr, d_dW.ptr, M, K, N))
+
+    def sgemm_ABt(self, d_D, d_W, d_dA, M, N, K, d_workspace):
+        assert d_workspace.size >= lib().scn_sgemm_ABt_workspace(N, K)
+        _check(lib().scn_sgemm_ABt(self.h, d_D.ptr, d_W.ptr, d_dA.ptr, M, N, K, d_workspace.ptr))
+
+    def nag_update(self, d_delta, d_momentum, d_weights, n, learningRate, momentum, keepPositive=False):
+        _check(lib().scn_nag_update(self.h, d_delta.ptr, d_momentum.ptr, d_weights.ptr, n, learningRate, momentum,
+                                    int(keepPositive)))
+
+    def gather_rows_backward(self, d_din, d_dconv, d_rules, count, nIn):
+        _check(lib().scn_gather_rows_backward(self.h, d_din.ptr, d_dconv.ptr, d_rules.ptr, count, nIn))
+
+    def maxpool_backward(self, d_din, d_dout, count, Cn, d_choice):
+        _check(lib().scn_maxpool_backward(self.h, d_din.ptr, d_dout.ptr, count, Cn, d_choice.ptr))
+
+    def terminal_pool_backward(self, d_din, d_dout, d_rules, count, Cn, S):
+        _check(lib().scn_terminal_pool_backward(self.h, d_din.ptr, d_dout.ptr, d_rules.ptr, count, Cn, S))
 
 
 class Grids:

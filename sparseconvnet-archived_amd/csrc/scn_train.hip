@@ -1,0 +1,467 @@
+// The backward pass and the weight update behind the C ABI: what the layers'
+// backwards() call in the reference, one entry point per free function there.
+//   softmax + NLL gradient     SoftmaxClassifier.cu:7-14
+//   activation derivatives     SigmoidLayer.cu:23-177, NetworkInNetworkPReLULayer.cu:25-47
+//   bias gradient              columnSum, NetworkInNetworkLayer.cu:84-105
+//   weight gradient  A^T D     d_rowMajorSGEMM_alphaAtB_betaC, utilities.cu:144-155
+//   input gradient   D W^T     d_rowMajorSGEMM_alphaABt_betaC, utilities.cu:157-168
+//   weight update              dGradientDescent(KeepPositive), NetworkInNetworkLayer.cu:27-41
+//   convolution                dPropBackwardFromMatrixMultiplyOutput, ConvolutionalLayer.cu:42-63
+//   max-pooling                dMaxPoolBackProp, MaxPoolingLayer.cu:74-82
+//   terminal pooling           dTerminalPoolBackProp, TerminalPoolingLayer.cu:48-62
+#include "scn_common.h"
+#include <hip/amd_detail/amd_hip_unsafe_atomics.h>
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+// ---------------------------------------------------------------- softmax
+__global__ void k_softmax_grad(const float *__restrict__ probs,
+                               const int *__restrict__ labels,
+                               float *__restrict__ delta, long long total,
+                               int N) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total)
+    return;
+  long long k = i / N;
+  int c = (int)(i - k * N);
+  delta[i] = probs[i] - (c == labels[k] ? 1.f : 0.f);
+}
+
+extern "C" int scn_softmax_grad(scn_ctx *ctx, const float *d_probs,
+                                const int32_t *d_labels, float *d_delta,
+                                int64_t batch, int N) {
+  SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_softmax_grad: null context");
+  SCN_REQUIRE(batch >= 0 && N >= 1, SCN_ERR_ARG,
+              "scn_softmax_grad: batch %lld N %d", (long long)batch, N);
+  if (batch == 0)
+    return SCN_OK;
+  SCN_REQUIRE(d_probs && d_labels && d_delta, SCN_ERR_ARG,
+              "scn_softmax_grad: null buffer");
+  ProfScope prof(ctx, SCN_K_BACKWARD);
+  long long total = batch * N;
+  hipLaunchKernelGGL(k_softmax_grad, dim3(scn_ceil_div(total, 256)), dim3(256),
+                     0, ctx->stream, d_probs, d_labels, d_delta, total, N);
+  SCN_HIP_CHECK(hipGetLastError());
+  return SCN_OK;
+}
+
+// ------------------------------------------------- activation derivatives
+// One pass over the [M x N] gradient: multiplies it in place by the
+// derivative of the activation (expressed through the layer's output, as the
+// reference does), and leaves the column sums of the result in db (the bias
+// gradient) and, for PReLU, the slope gradient in dprelu.  Lane = column,
+// the four wavefronts of a workgroup interleave rows.
+__global__ __launch_bounds__(256) void k_act_backward(
+    const float *__restrict__ out, float *__restrict__ delta, long long M,
+    int N, int act, const float *__restrict__ prelu, float *__restrict__ db,
+    float *__restrict__ dprelu) {
+  __shared__ float sS[4][64], sT[4][64];
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const int c = blockIdx.x * 64 + tx;
+  float s = 0.f, t = 0.f;
+  if (c < N) {
+    const float alpha = act == SCN_PRELU      ? prelu[c]
+                        : act == SCN_LEAKYRELU ? 0.01f
+                                               : 0.333f;
+    for (long long r = (long long)blockIdx.y * 4 + ty; r < M;
+         r += 4ll * gridDim.y) {
+      const long long i = r * N + c;
+      const float b = out[i];
+      float d = delta[i];
+      switch (act) {
+      case SCN_RELU:
+        d = b > 0 ? d : 0.f;
+        break;
+      case SCN_LEAKYRELU:
+      case SCN_VLEAKYRELU:
+        d = b > 0 ? d : d * alpha;
+        break;
+      case SCN_TANH:
+        d = d * (1 + b) * (1 - b);
+        break;
+      case SCN_SIGMOID:
+        d = d * b * (1 - b);
+        break;
+      case SCN_PRELU:
+        t += d * (b > 0 ? 0.f : b / alpha);
+        d = b > 0 ? d : d * alpha;
+        break;
+      default: // SOFTMAX (folded into the classifier's gradient), NOSIGMOID
+        break;
+      }
+      delta[i] = d;
+      s += d;
+    }
+  }
+  sS[ty][tx] = s;
+  sT[ty][tx] = t;
+  __syncthreads();
+  if (ty == 0 && c < N) {
+    s = sS[0][tx] + sS[1][tx] + sS[2][tx] + sS[3][tx];
+    unsafeAtomicAdd(db + c, s);
+    if (act == SCN_PRELU) {
+      t = sT[0][tx] + sT[1][tx] + sT[2][tx] + sT[3][tx];
+      unsafeAtomicAdd(dprelu + c, t);
+    }
+  }
+}
+
+extern "C" int scn_activation_backward(scn_ctx *ctx, const float *d_out,
+                                       float *d_delta, int64_t M, int N,
+                                       int act, const float *d_prelu,
+                                       float *d_db, float *d_dprelu) {
+  SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_activation_backward: null context");
+  SCN_REQUIRE(M >= 0 && N >= 1, SCN_ERR_ARG,
+              "scn_activation_backward: M %lld N %d", (long long)M, N);
+  SCN_REQUIRE(act >= SCN_NOSIGMOID && act <= SCN_SIGMOID, SCN_ERR_ARG,
+              "scn_activation_backward: activation %d", act);
+  SCN_REQUIRE(d_db, SCN_ERR_ARG, "scn_activation_backward: null d_db");
+  SCN_REQUIRE(act != SCN_PRELU || (d_prelu && d_dprelu), SCN_ERR_ARG,
+              "scn_activation_backward: PReLU needs slopes and their gradient");
+  ProfScope prof(ctx, SCN_K_BACKWARD);
+  SCN_TRY(scn_fill32(ctx, d_db, 0, (size_t)N));
+  if (act == SCN_PRELU)
+    SCN_TRY(scn_fill32(ctx, d_dprelu, 0, (size_t)N));
+  if (M == 0)
+    return SCN_OK;
+  SCN_REQUIRE(d_out && d_delta, SCN_ERR_ARG,
+              "scn_activation_backward: null buffer");
+  int colBlocks = scn_ceil_div(N, 64);
+  int rowBlocks = scn_ceil_div(M, 64); // at least 16 rows per wavefront
+  int cap = (ctx->numCU * 8 + colBlocks - 1) / colBlocks;
+  if (rowBlocks > cap)
+    rowBlocks = cap;
+  hipLaunchKernelGGL(k_act_backward, dim3(colBlocks, rowBlocks), dim3(256), 0,
+                     ctx->stream, d_out, d_delta, (long long)M, N, act,
+                     d_prelu, d_db, d_dprelu);
+  SCN_HIP_CHECK(hipGetLastError());
+  return SCN_OK;
+}
+
+// ------------------------------------------------------- dW = A^T D (MFMA)
+// Output tile 64 (rows of dW = columns of A) x 64 (columns of D) per
+// workgroup, reduction over a range of the M rows; the row ranges of one tile
+// add their partial tiles into dW with float atomics.  A chunk of 32 rows of
+// both operands is staged in LDS (row pitch 80 words: the four row groups
+// that one v_mfma_f32_16x16x4_f32 operand read touches fall on disjoint
+// banks); wavefront w owns columns 16 w .. 16 w + 15 of the tile and all 64 of
+// its rows (four accumulator tiles).
+#define ATB_ROWS 32
+#define ATB_PITCH 80
+__global__ __launch_bounds__(256) void k_gemm_atb(
+    const float *__restrict__ A, const float *__restrict__ D,
+    float *__restrict__ dW, long long M, int K, int N, int nTiles,
+    long long rowsPerSplit) {
+  __shared__ float sA[ATB_ROWS * ATB_PITCH], sD[ATB_ROWS * ATB_PITCH];
+  const int k0 = (blockIdx.x / nTiles) * 64, n0 = (blockIdx.x % nTiles) * 64;
+  const long long m0 = (long long)blockIdx.y * rowsPerSplit;
+  const long long m1 = m0 + rowsPerSplit < M ? m0 + rowsPerSplit : M;
+  const int t = threadIdx.x, col = t & 63, rg = t >> 6;
+  const int lane = t & 63, w = t >> 6, c = lane & 15, q = lane >> 4;
+  const bool aIn = k0 + col < K, dIn = n0 + col < N;
+  floatx4 acc[4];
+  for (int i = 0; i < 4; ++i)
+    acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (long long m = m0; m < m1; m += ATB_ROWS) {
+    for (int i = 0; i < ATB_ROWS / 4; ++i) {
+      const int r = rg + 4 * i;
+      const long long row = m + r;
+      const bool live = row < m1;
+      sA[r * ATB_PITCH + col] = live && aIn ? A[row * K + k0 + col] : 0.f;
+      sD[r * ATB_PITCH + col] = live && dIn ? D[row * N + n0 + col] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int s = 0; s < ATB_ROWS / 4; ++s) {
+      const float *ra = sA + (4 * s + q) * ATB_PITCH + c;
+      const float b = sD[(4 * s + q) * ATB_PITCH + 16 * w + c];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[16 * i], b, acc[i], 0,
+                                                      0, 0);
+    }
+    __syncthreads();
+  }
+  const int n = n0 + 16 * w + c;
+  if (n < N)
+    for (int i = 0; i < 4; ++i)
+      for (int v = 0; v < 4; ++v) {
+        const int k = k0 + 16 * i + 4 * q + v;
+        if (k < K)
+          unsafeAtomicAdd(dW + (long long)k * N + n, acc[i][v]);
+      }
+}
+
+extern "C" int scn_sgemm_AtB(scn_ctx *ctx, const float *d_A, const float *d_D,
+                             float *d_dW, int64_t M, int K, int N) {
+  SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_sgemm_AtB: null context");
+  SCN_REQUIRE(M >= 0 && K >= 1 && N >= 1, SCN_ERR_ARG,
+              "scn_sgemm_AtB: M %lld K %d N %d", (long long)M, K, N);
+  SCN_REQUIRE(d_dW, SCN_ERR_ARG, "scn_sgemm_AtB: null d_dW");
+  ProfScope prof(ctx, SCN_K_BACKWARD);
+  SCN_TRY(scn_fill32(ctx, d_dW, 0, (size_t)K * N));
+  if (M == 0)
+    return SCN_OK;
+  SCN_REQUIRE(d_A && d_D, SCN_ERR_ARG, "scn_sgemm_AtB: null buffer");
+  const int kTiles = scn_ceil_div(K, 64), nTiles = scn_ceil_div(N, 64);
+  const long long tiles = (long long)kTiles * nTiles;
+  SCN_REQUIRE(tiles <= 0x7fffffffll, SCN_ERR_CAPACITY,
+              "scn_sgemm_AtB: %lld tiles", tiles);
+  long long splits = (ctx->numCU * 4 + tiles - 1) / tiles;
+  const long long maxSplits = (M + 8 * ATB_ROWS - 1) / (8 * ATB_ROWS);
+  if (splits > maxSplits)
+    splits = maxSplits;
+  if (splits > 65535)
+    splits = 65535;
+  if (splits < 1)
+    splits = 1;
+  long long rowsPerSplit = (M + splits - 1) / splits;
+  rowsPerSplit = (rowsPerSplit + ATB_ROWS - 1) / ATB_ROWS * ATB_ROWS;
+  splits = (M + rowsPerSplit - 1) / rowsPerSplit;
+  hipLaunchKernelGGL(k_gemm_atb, dim3((unsigned)tiles, (unsigned)splits),
+                     dim3(256), 0, ctx->stream, d_A, d_D, d_dW, (long long)M, K,
+                     N, nTiles, rowsPerSplit);
+  SCN_HIP_CHECK(hipGetLastError());
+  return SCN_OK;
+}
+
+// ------------------------------------------------------------ dA = D W^T
+// The forward contraction with W transposed: the transposed copy (and the
+// zero bias the forward kernels add) live in the caller's workspace.
+__global__ void k_transpose(const float *__restrict__ W, float *__restrict__ Wt,
+                            int K, int N) {
+  __shared__ float tile[32][33];
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5; // 32 x 8
+  const int k0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
+  for (int i = ty; i < 32; i += 8)
+    if (k0 + i < K && n0 + tx < N)
+      tile[i][tx] = W[(long long)(k0 + i) * N + n0 + tx];
+  __syncthreads();
+  for (int i = ty; i < 32; i += 8)
+    if (n0 + i < N && k0 + tx < K)
+      Wt[(long long)(n0 + i) * K + k0 + tx] = tile[tx][i];
+}
+
+extern "C" int64_t scn_sgemm_ABt_workspace(int N, int K) {
+  return (int64_t)N * K + K;
+}
+
+extern "C" int scn_sgemm_ABt(scn_ctx *ctx, const float *d_D, const float *d_W,
+                             float *d_dA, int64_t M, int N, int K,
+                             float *d_workspace) {
+  SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_sgemm_ABt: null context");
+  SCN_REQUIRE(M >= 0 && K >= 1 && N >= 1, SCN_ERR_ARG,
+              "scn_sgemm_ABt: M %lld N %d K %d", (long long)M, N, K);
+  if (M == 0)
+    return SCN_OK;
+  SCN_REQUIRE(d_D && d_W && d_dA && d_workspace, SCN_ERR_ARG,
+              "scn_sgemm_ABt: null buffer");
+  float *Wt = d_workspace, *zeros = d_workspace + (size_t)N * K;
+  {
+    ProfScope prof(ctx, SCN_K_BACKWARD);
+    hipLaunchKernelGGL(k_transpose, dim3(scn_ceil_div(N, 32), scn_ceil_div(K, 32)),
+                       dim3(256), 0, ctx->stream, d_W, Wt, K, N);
+    SCN_HIP_CHECK(hipGetLastError());
+    SCN_TRY(scn_fill32(ctx, zeros, 0, (size_t)K));
+  }
+  return scn_nin_forward(ctx, d_D, Wt, zeros, nullptr, d_dA, M, N, K, 1.0f,
+                         SCN_NOSIGMOID, SCN_FP32);
+}
+
+// ---------------------------------------------------------- weight update
+__global__ void k_nag_update(const float *__restrict__ delta,
+                             float *__restrict__ mom, float *__restrict__ wts,
+                             long long n, float lr, float mu, int keepPositive) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n)
+    return;
+  float w = wts[i], m = mom[i];
+  const float d = delta[i];
+  w -= m * mu;
+  m = mu * m - lr * (1 - mu) * d;
+  w += m * (1 + mu);
+  if (keepPositive)
+    w = w > 0.001f ? w : 0.001f;
+  wts[i] = w;
+  mom[i] = m;
+}
+
+extern "C" int scn_nag_update(scn_ctx *ctx, const float *d_delta,
+                              float *d_momentum, float *d_weights, int64_t n,
+                              float learningRate, float momentum,
+                              int keepPositive) {
+  SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_nag_update: null context");
+  SCN_REQUIRE(n >= 0, SCN_ERR_ARG, "scn_nag_update: n %lld", (long long)n);
+  if (n == 0)
+    return SCN_OK;
+  SCN_REQUIRE(d_delta && d_momentum && d_weights, SCN_ERR_ARG,
+              "scn_nag_update: null buffer");
+  ProfScope prof(ctx, SCN_K_BACKWARD);
+  hipLaunchKernelGGL(k_nag_update, dim3(scn_ceil_div(n, 256)), dim3(256), 0,
+                     ctx->stream, d_delta, d_momentum, d_weights, (long long)n,
+                     learningRate, momentum, keepPositive);
+  SCN_HIP_CHECK(hipGetLastError());
+  return SCN_OK;
+}
+
+// ------------------------------------------------- scatter-add through rules
+// A group of P lanes (P = the power of two that covers min(nIn, 64)) walks a
+// run of consecutive rule entries; lane j of it owns channel j (+ P, + 2P ..).
+// Consecutive entries that name the same input row (a sample's background row
+// fills most of a sparse rule book) are summed in a register and reach memory
+// as one atomic add.
+#define SCATTER_RUN 32
+__global__ __launch_bounds__(256) void k_gather_backward(
+    float *__restrict__ din, const float *__restrict__ dconv,
+    const int *__restrict__ rules, long long count, int nIn, int P) {
+  const long long lane = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long group = lane / P;
+  const int li = (int)(lane - group * P);
+  const long long e0 = group * SCATTER_RUN;
+  if (e0 >= count)
+    return;
+  const long long e1 = e0 + SCATTER_RUN < count ? e0 + SCATTER_RUN : count;
+  for (int j = li; j < nIn; j += P) {
+    int cur = -1;
+    float acc = 0.f;
+    for (long long e = e0; e < e1; ++e) {
+      const int r = rules[e];
+      if (r < 0)
+        continue;
+      if (r != cur) {
+        if (cur >= 0)
+          unsafeAtomicAdd(din + (long long)cur * nIn + j, acc);
+        cur = r;
+        acc = 0.f;
+      }
+      acc += dconv[e * nIn + j];
+    }
+    if (cur >= 0)
+      unsafeAtomicAdd(din + (long long)cur * nIn + j, acc);
+  }
+}
+
+static int group_width(int n) {
+  int P = 1;
+  while (P < n && P < 64)
+    P <<= 1;
+  return P;
+}
+
+extern "C" int scn_gather_rows_backward(scn_ctx *ctx, float *d_din,
+                                        const float *d_dconv,
+                                        const int32_t *d_rules, int64_t count,
+                                        int nIn) {
+  SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_gather_rows_backward: null context");
+  SCN_REQUIRE(count >= 0 && nIn >= 1, SCN_ERR_ARG,
+              "scn_gather_rows_backward: count %lld nIn %d", (long long)count,
+              nIn);
+  if (count == 0)
+    return SCN_OK;
+  SCN_REQUIRE(d_din && d_dconv && d_rules, SCN_ERR_ARG,
+              "scn_gather_rows_backward: null buffer");
+  ProfScope prof(ctx, SCN_K_BACKWARD);
+  const int P = group_width(nIn);
+  const long long groups = (count + SCATTER_RUN - 1) / SCATTER_RUN;
+  const long long blocks = (groups * P + 255) / 256;
+  SCN_REQUIRE(blocks <= 0x7fffffffll, SCN_ERR_CAPACITY,
+              "scn_gather_rows_backward: %lld workgroups", blocks);
+  hipLaunchKernelGGL(k_gather_backward, dim3((unsigned)blocks), dim3(256), 0,
+                     ctx->stream, d_din, d_dconv, d_rules, (long long)count,
+                     nIn, P);
+  SCN_HIP_CHECK(hipGetLastError());
+  return SCN_OK;
+}
+
+// dMaxPoolBackProp: the same walk over output rows, every lane following the
+// choices of its own channel.
+__global__ __launch_bounds__(256) void k_maxpool_backward(
+    float *__restrict__ din, const float *__restrict__ dout, long long count,
+    int C, const int *__restrict__ choice, int P) {
+  const long long lane = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long group = lane / P;
+  const int li = (int)(lane - group * P);
+  const long long r0 = group * SCATTER_RUN;
+  if (r0 >= count)
+    return;
+  const long long r1 = r0 + SCATTER_RUN < count ? r0 + SCATTER_RUN : count;
+  for (int j = li; j < C; j += P) {
+    int cur = -1;
+    float acc = 0.f;
+    for (long long r = r0; r < r1; ++r) {
+      const int tgt = choice[r * C + j];
+      if (tgt != cur) {
+        if (cur >= 0)
+          unsafeAtomicAdd(din + cur, acc);
+        cur = tgt;
+        acc = 0.f;
+      }
+      acc += dout[r * C + j];
+    }
+    if (cur >= 0)
+      unsafeAtomicAdd(din + cur, acc);
+  }
+}
+
+extern "C" int scn_maxpool_backward(scn_ctx *ctx, float *d_din,
+                                    const float *d_dout, int64_t count, int C,
+                                    const int32_t *d_choice) {
+  SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_maxpool_backward: null context");
+  SCN_REQUIRE(count >= 0 && C >= 1, SCN_ERR_ARG,
+              "scn_maxpool_backward: count %lld C %d", (long long)count, C);
+  if (count == 0)
+    return SCN_OK;
+  SCN_REQUIRE(d_din && d_dout && d_choice, SCN_ERR_ARG,
+              "scn_maxpool_backward: null buffer");
+  ProfScope prof(ctx, SCN_K_BACKWARD);
+  const int P = group_width(C);
+  const long long groups = (count + SCATTER_RUN - 1) / SCATTER_RUN;
+  const long long blocks = (groups * P + 255) / 256;
+  SCN_REQUIRE(blocks <= 0x7fffffffll, SCN_ERR_CAPACITY,
+              "scn_maxpool_backward: %lld workgroups", blocks);
+  hipLaunchKernelGGL(k_maxpool_backward, dim3((unsigned)blocks), dim3(256), 0,
+                     ctx->stream, d_din, d_dout, (long long)count, C, d_choice,
+                     P);
+  SCN_HIP_CHECK(hipGetLastError());
+  return SCN_OK;
+}
+
+// dTerminalPoolBackProp: every row listed for a sample receives (not
+// accumulates) the sample's gradient divided by the number of rows listed.
+__global__ void k_terminal_backward(float *__restrict__ din,
+                                    const float *__restrict__ dout,
+                                    const int *__restrict__ rules, int C,
+                                    int S) {
+  const long long b = blockIdx.x;
+  const int *rr = rules + b * S;
+  int maxP = 0;
+  while (maxP < S && rr[maxP] >= 0)
+    ++maxP;
+  for (int j = threadIdx.x; j < C; j += blockDim.x) {
+    const float t = dout[b * C + j] / (float)maxP;
+    for (int p = 0; p < maxP; ++p)
+      din[(long long)rr[p] * C + j] = t;
+  }
+}
+
+extern "C" int scn_terminal_pool_backward(scn_ctx *ctx, float *d_din,
+                                          const float *d_dout,
+                                          const int32_t *d_rules,
+                                          int64_t count, int C, int S) {
+  SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_terminal_pool_backward: null context");
+  SCN_REQUIRE(count >= 0 && C >= 1 && S >= 1, SCN_ERR_ARG,
+              "scn_terminal_pool_backward: count %lld C %d S %d",
+              (long long)count, C, S);
+  if (count == 0)
+    return SCN_OK;
+  SCN_REQUIRE(count <= 0x7fffffffll, SCN_ERR_CAPACITY,
+              "scn_terminal_pool_backward: %lld samples", (long long)count);
+  SCN_REQUIRE(d_din && d_dout && d_rules, SCN_ERR_ARG,
+              "scn_terminal_pool_backward: null buffer");
+  ProfScope prof(ctx, SCN_K_BACKWARD);
+  hipLaunchKernelGGL(k_terminal_backward, dim3((unsigned)count),
+                     dim3(C >= 256 ? 256 : 64), 0, ctx->stream, d_din, d_dout,
+                     d_rules, C, S);
+  SCN_HIP_CHECK(hipGetLastError());
+  return SCN_OK;
+}

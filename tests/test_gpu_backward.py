@@ -1,0 +1,156 @@
+"""The backward pass and the weight update through the C ABI against the oracle.
+Sums that the reference itself leaves to float atomics in no fixed order are held to 1e-4 of the sum of magnitudes;
+assignments and element-wise results are bit-exact."""
+import numpy as np
+import pytest
+
+import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def close(got, want, scale, tol=1e-4):
+    got, want = got.astype(np.float64), want.astype(np.float64)
+    bad = np.abs(got - want) > tol * scale + 1e-30
+    assert not bad.any(), (np.abs(got - want).max(), np.argwhere(bad)[:5])
+
+
+def test_softmax_gradient_bit_exact(scn, ctx):
+    rng = np.random.default_rng(0)
+    for B, N in [(1, 1), (7, 10), (100, 100), (33, 1000)]:
+        probs = orc.softmax_rows(rng.standard_normal((B, N)).astype(np.float32))
+        labels = rng.integers(0, N, B).astype(np.int32)
+        d = ctx.empty((B, N), np.float32)
+        ctx.softmax_grad(ctx.array(probs), ctx.array(labels), d, B, N)
+        assert np.array_equal(d.download(), orc.softmax_grad(probs, labels))
+
+
+@pytest.mark.parametrize("act", [0, 1, 2, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize("M,N", [(1, 32), (77, 100), (5000, 64), (2049, 800), (300, 3)])
+def test_activation_backward(scn, ctx, act, M, N):
+    rng = np.random.default_rng(act * 1000 + M + N)
+    print("activation backward act=%d M=%d N=%d" % (act, M, N), flush=True)
+    out = rng.standard_normal((M, N)).astype(np.float32)
+    if act in (1,):
+        out = np.maximum(out, 0)
+    delta = rng.standard_normal((M, N)).astype(np.float32)
+    pr = rng.uniform(0.05, 0.5, N).astype(np.float32) if act == 6 else None
+    d_delta = ctx.array(delta)
+    d_db = ctx.array(np.full(N, 7, np.float32))  # must be overwritten, not added to
+    d_dpr = ctx.array(np.full(N, 7, np.float32)) if act == 6 else None
+    ctx.activation_backward(ctx.array(out), d_delta, M, N, act, ctx.array(pr) if pr is not None else None, d_db, d_dpr)
+    wd, wdb, wdpr = orc.activation_backward(out, delta, act, pr)
+    assert np.array_equal(d_delta.download(), wd)
+    close(d_db.download(), wdb, np.abs(wd).sum(0))
+    if act == 6:
+        close(d_dpr.download(), wdpr, (np.abs(delta) * np.abs(out) / pr).sum(0))
+
+
+@pytest.mark.parametrize("M,K,N", [(1, 1, 1), (50, 12, 32), (1000, 128, 64), (4097, 288, 64), (333, 100, 100),
+                                   (20000, 256, 96), (2500, 800, 800), (100, 192, 100), (70000, 1728, 64)])
+def test_weight_gradient_AtB(scn, ctx, M, K, N):
+    rng = np.random.default_rng(M + K + N)
+    print("AtB M=%d K=%d N=%d" % (M, K, N), flush=True)
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    D = rng.standard_normal((M, N)).astype(np.float32)
+    d_dW = ctx.array(np.full((K, N), 3, np.float32))
+    ctx.sgemm_AtB(ctx.array(A), ctx.array(D), d_dW, M, K, N)
+    orc.set_threads(8)
+    want = orc.sgemm_AtB(A, D)
+    scale = np.sqrt((A.astype(np.float64) ** 2).sum(0))[:, None] * np.sqrt((D.astype(np.float64) ** 2).sum(0))[None, :]
+    close(d_dW.download(), want, scale + 1e-6)
+    # a one-hot D picks out rows of A exactly
+    if M >= 2 and N >= 2:
+        D[:] = 0
+        D[M // 2, 1] = 1
+        ctx.sgemm_AtB(ctx.array(A), ctx.array(D), d_dW, M, K, N)
+        got = d_dW.download()
+        assert np.array_equal(got[:, 1], A[M // 2]) and not got[:, 0].any()
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1, 1), (50, 32, 12), (1000, 64, 128), (4097, 64, 288), (333, 100, 192),
+                                   (20000, 96, 256), (2500, 800, 800), (100, 100, 192)])
+def test_input_gradient_ABt(scn, ctx, M, N, K):
+    rng = np.random.default_rng(M + K + N + 1)
+    print("ABt M=%d N=%d K=%d" % (M, N, K), flush=True)
+    D = rng.standard_normal((M, N)).astype(np.float32)
+    W = rng.standard_normal((K, N)).astype(np.float32)
+    d_dA = ctx.empty((M, K), np.float32)
+    ws = ctx.empty(scn.lib().scn_sgemm_ABt_workspace(N, K), np.float32)
+    ctx.sgemm_ABt(ctx.array(D), ctx.array(W), d_dA, M, N, K, ws)
+    orc.set_threads(8)
+    want = orc.sgemm_ABt(D, W)
+    scale = np.abs(D).astype(np.float64) @ np.abs(W).astype(np.float64).T
+    close(d_dA.download(), want, scale + 1e-6)
+
+
+def test_weight_update(scn, ctx):
+    rng = np.random.default_rng(3)
+    for n in (1, 100, 12345, 800 * 800):
+        for keep in (False, True):
+            d = rng.standard_normal(n).astype(np.float32)
+            w = rng.standard_normal(n).astype(np.float32)
+            m = (rng.standard_normal(n) * 0.1).astype(np.float32)
+            d_w, d_m = ctx.array(w), ctx.array(m)
+            ctx.nag_update(ctx.array(d), d_m, d_w, n, 0.003, 0.99, keep)
+            orc.nag_update(d, m, w, 0.003, 0.99, keep)
+            # (a fused multiply-add more or less than the host compiler chose: a few ulp of the terms)
+            assert np.allclose(d_w.download(), w, rtol=1e-6, atol=1e-7)
+            assert np.allclose(d_m.download(), m, rtol=1e-6, atol=1e-8)
+
+
+@pytest.mark.parametrize("nIn,rowsIn,count", [(1, 5, 40), (3, 1000, 33333), (32, 5000, 100001), (64, 2000, 54321),
+                                              (96, 300, 9999), (160, 77, 4096), (5, 10, 31)])
+def test_convolution_backward_scatter(scn, ctx, nIn, rowsIn, count):
+    rng = np.random.default_rng(nIn + rowsIn + count)
+    print("scatter nIn=%d rows=%d count=%d" % (nIn, rowsIn, count), flush=True)
+    rules = rng.integers(0, rowsIn, count).astype(np.int32)
+    rules[rng.random(count) < 0.6] = rowsIn // 2  # the background row of a sparse rule book
+    rules[rng.random(count) < 0.01] = -1
+    dconv = rng.standard_normal((count, nIn)).astype(np.float32)
+    d_din = ctx.array(np.zeros((rowsIn, nIn), np.float32))
+    ctx.gather_rows_backward(d_din, ctx.array(dconv), ctx.array(rules), count, nIn)
+    want = orc.gather_rows_backward(dconv, rules, rowsIn, nIn)
+    mag = orc.gather_rows_backward(np.abs(dconv), rules, rowsIn, nIn)
+    close(d_din.download(), want, mag)
+    # integers add exactly in any order
+    dconv = rng.integers(-3, 4, (count, nIn)).astype(np.float32)
+    d_din = ctx.array(np.zeros((rowsIn, nIn), np.float32))
+    ctx.gather_rows_backward(d_din, ctx.array(dconv), ctx.array(rules), count, nIn)
+    assert np.array_equal(d_din.download(), orc.gather_rows_backward(dconv, rules, rowsIn, nIn))
+
+
+@pytest.mark.parametrize("C,rowsIn,nOut,ps", [(1, 6, 10, 4), (32, 3000, 7777, 9), (64, 500, 2001, 8), (96, 100, 333, 27),
+                                              (5, 20, 65, 4)])
+def test_maxpool_backward(scn, ctx, C, rowsIn, nOut, ps):
+    rng = np.random.default_rng(C + rowsIn + nOut)
+    print("maxpool backward C=%d" % C, flush=True)
+    rules = rng.integers(0, rowsIn, (nOut, ps)).astype(np.int32)
+    rules[rng.random((nOut, ps)) < 0.5] = 0
+    x = rng.standard_normal((rowsIn, C)).astype(np.float32)
+    _, choice = orc.maxpool(x, rules, nOut, ps, C)
+    dout = rng.integers(-3, 4, (nOut, C)).astype(np.float32)  # integers: exact in any order
+    d_din = ctx.array(np.zeros((rowsIn, C), np.float32))
+    ctx.maxpool_backward(d_din, ctx.array(dout), nOut, C, ctx.array(choice))
+    assert np.array_equal(d_din.download(), orc.maxpool_backward(dout, choice, rowsIn))
+    dout = rng.standard_normal((nOut, C)).astype(np.float32)
+    d_din = ctx.array(np.zeros((rowsIn, C), np.float32))
+    ctx.maxpool_backward(d_din, ctx.array(dout), nOut, C, ctx.array(choice))
+    close(d_din.download(), orc.maxpool_backward(dout, choice, rowsIn), orc.maxpool_backward(np.abs(dout), choice, rowsIn))
+
+
+def test_terminal_pool_backward_bit_exact(scn, ctx):
+    rng = np.random.default_rng(9)
+    for C in (3, 100, 192, 800):
+        B, S, rows = 37, 9, 400
+        rules = np.full((B, S), -1, np.int32)
+        perm = rng.permutation(rows)
+        at = 0
+        for b in range(B):
+            n = 1 + b % S
+            rules[b, :n] = perm[at:at + n]
+            at += n
+        dout = rng.standard_normal((B, C)).astype(np.float32)
+        d_din = ctx.array(np.zeros((rows, C), np.float32))
+        ctx.terminal_pool_backward(d_din, ctx.array(dout), ctx.array(rules), B, C, S)
+        assert np.array_equal(d_din.download(), orc.terminal_pool_backward(dout, rules, S, rows))
