@@ -137,3 +137,51 @@ class Net:
             else:
                 out["predictions"] = np.stack([orc.top_indices(p, self.nTop) for p in probs])
         return out
+
+    # ---- backward over the batch just forwarded, and the weight update
+    def train_step(self, fwd, labels, learningRate, momentum):
+        """SparseConvNetCUDA::processBatch for a TRAINBATCH without dropout (SparseConvNetCUDA.cu:247-252):
+        SoftmaxClassifier's gradient, then backwards() of every layer, last to first.  Leaves the gradient of each
+        interface in its dict ("dfeatures", where the reference computes one) and updates self.weights and
+        self.momentum in place."""
+        ifaces = fwd["interfaces"]
+        if not hasattr(self, "momentum"):
+            self.momentum = {}
+        backprop = [False]
+        for l in self.layers:  # output.backpropErrors of every layer's preprocess()
+            backprop.append(True if l["kind"] in ("nin", "nin_prelu") else backprop[-1])
+        ifaces[-1]["dfeatures"] = orc.softmax_grad(ifaces[-1]["features"], labels)
+        for i in range(len(self.layers) - 1, -1, -1):
+            l, cur, nxt = self.layers[i], ifaces[i], ifaces[i + 1]
+            k = l["kind"]
+            if k in ("nin", "nin_prelu"):
+                assert l["dropout"] == 0
+                W, B, pr = self.weights[i]
+                W, B = W.copy(), B.copy()
+                pr = None if pr is None else pr.copy()
+                MW, MB, MP = self.momentum.get(i, (np.zeros_like(W), np.zeros_like(B),
+                                                   None if pr is None else np.zeros_like(pr)))
+                dZ, dB, dPr = orc.activation_backward(nxt["features"], nxt["dfeatures"], l["act"], pr)
+                nxt["dfeatures"] = dZ  # in place in the reference
+                Wold = W.copy()
+                if pr is not None:
+                    orc.nag_update(dPr, MP, pr, learningRate, momentum, keepPositive=True)
+                dW = orc.sgemm_AtB(cur["features"], dZ)
+                if backprop[i]:
+                    cur["dfeatures"] = orc.sgemm_ABt(dZ, Wold)
+                orc.nag_update(dW, MW, W, learningRate, momentum)
+                orc.nag_update(dB, MB, B, learningRate, momentum)
+                self.weights[i] = (W, B, pr)
+                self.momentum[i] = (MW, MB, MP)
+                nxt["dW"], nxt["dB"], nxt["dPReLU"] = dW, dB, dPr
+            elif not backprop[i]:
+                continue
+            elif k in ("conv", "conv_tri"):
+                cur["dfeatures"] = orc.gather_rows_backward(nxt["dfeatures"].reshape(-1, cur["nFeatures"]), nxt["rules"],
+                                                            cur["nSpatialSites"], cur["nFeatures"])
+            elif k in ("maxpool", "maxpool_tri"):
+                cur["dfeatures"] = orc.maxpool_backward(nxt["dfeatures"], nxt["choices"], cur["nSpatialSites"])
+            elif k == "terminal":
+                S = nxt["rules"].size // max(nxt["nSpatialSites"], 1)
+                cur["dfeatures"] = orc.terminal_pool_backward(nxt["dfeatures"], nxt["rules"], S, cur["nSpatialSites"])
+        return fwd

@@ -41,7 +41,7 @@ def declared_symbols():
     """Names of every function the C header declares."""
     text = open(HEADER).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(scn_[a-z0-9_]+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(scn_[A-Za-z0-9_]+)\s*\(", text)))
 
 
 _lib = None

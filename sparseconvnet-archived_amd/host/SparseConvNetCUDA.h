@@ -55,6 +55,11 @@ public:
                     int nBatchProducerThreads = 10);
   ~SparseConvNetCUDA();
   void forwardBatch(SpatiallySparseBatch &batch);
+  void backwardBatch(SpatiallySparseBatch &batch, float learningRate,
+                     float momentum);
+  // training batches are drawn in shuffled order (BatchProducer.cu:23-26);
+  // a harness that needs a fixed order turns this off
+  bool shuffleTrainingData = true;
   void finishBatch(SpatiallySparseBatch &batch, std::ofstream &f,
                    std::ofstream &g);
   void processBatch(SpatiallySparseBatch &batch, float learningRate,

@@ -3,9 +3,10 @@
 // preprocess() builds the output interface's grids and rule book, forwards()
 // runs the feature kernels (SpatiallySparseLayer.h:6-27).  In the reference
 // preprocess() is CPU code run by batch-producer threads; here it issues the
-// rule-book kernels on the GPU.  The backward pass is outside this library:
-// backwards() exists so that subclasses written against the reference still
-// compile, and reports an error when called.
+// rule-book kernels on the GPU.  backwards() propagates the gradient of the
+// cost from the output interface's dfeatures to the input's and, in layers
+// with weights, takes one momentum step (dropout during training is not
+// implemented: such a layer stops with a message).
 #pragma once
 #include <fstream>
 #include <iostream>
@@ -63,6 +64,10 @@ public:
   void forwards(SpatiallySparseBatch &batch,
                 SpatiallySparseBatchInterface &input,
                 SpatiallySparseBatchInterface &output);
+  void backwards(SpatiallySparseBatch &batch,
+                 SpatiallySparseBatchInterface &input,
+                 SpatiallySparseBatchInterface &output, float learningRate,
+                 float momentum);
   int calculateInputSpatialSize(int outputSpatialSize);
 };
 
@@ -90,6 +95,10 @@ public:
   void forwards(SpatiallySparseBatch &batch,
                 SpatiallySparseBatchInterface &input,
                 SpatiallySparseBatchInterface &output);
+  void backwards(SpatiallySparseBatch &batch,
+                 SpatiallySparseBatchInterface &input,
+                 SpatiallySparseBatchInterface &output, float learningRate,
+                 float momentum);
   int calculateInputSpatialSize(int outputSpatialSize);
 };
 
@@ -98,10 +107,11 @@ public:
 class NetworkInNetworkLayer : public SpatiallySparseLayer {
 private:
   RNG rng;
+  vectorCUDA<float> dw, db, workspace; // gradients; W transposed for dA
 
 public:
   vectorCUDA<float> W;
-  vectorCUDA<float> MW; // momentum: read and written by the weight files only
+  vectorCUDA<float> MW; // momentum
   vectorCUDA<float> B;
   vectorCUDA<float> MB;
   ActivationFunction fn;
@@ -120,6 +130,10 @@ public:
                 SpatiallySparseBatchInterface &output);
   void loadWeightsFromStream(std::ifstream &f, bool momentum);
   void putWeightsToStream(std::ofstream &f, bool momentum);
+  void backwards(SpatiallySparseBatch &batch,
+                 SpatiallySparseBatchInterface &input,
+                 SpatiallySparseBatchInterface &output, float learningRate,
+                 float momentum);
   int calculateInputSpatialSize(int outputSpatialSize);
 };
 
@@ -127,6 +141,7 @@ public:
 class NetworkInNetworkPReLULayer : public SpatiallySparseLayer {
 private:
   RNG rng;
+  vectorCUDA<float> dw, db, dprelu, workspace;
 
 public:
   vectorCUDA<float> W;
@@ -150,6 +165,10 @@ public:
                 SpatiallySparseBatchInterface &output);
   void loadWeightsFromStream(std::ifstream &f, bool momentum);
   void putWeightsToStream(std::ofstream &f, bool momentum);
+  void backwards(SpatiallySparseBatch &batch,
+                 SpatiallySparseBatchInterface &input,
+                 SpatiallySparseBatchInterface &output, float learningRate,
+                 float momentum);
   int calculateInputSpatialSize(int outputSpatialSize);
 };
 
@@ -170,6 +189,10 @@ public:
   void forwards(SpatiallySparseBatch &batch,
                 SpatiallySparseBatchInterface &input,
                 SpatiallySparseBatchInterface &output);
+  void backwards(SpatiallySparseBatch &batch,
+                 SpatiallySparseBatchInterface &input,
+                 SpatiallySparseBatchInterface &output, float learningRate,
+                 float momentum);
   int calculateInputSpatialSize(int outputSpatialSize);
 };
 
@@ -190,6 +213,10 @@ public:
   void forwards(SpatiallySparseBatch &batch,
                 SpatiallySparseBatchInterface &input,
                 SpatiallySparseBatchInterface &output);
+  void backwards(SpatiallySparseBatch &batch,
+                 SpatiallySparseBatchInterface &input,
+                 SpatiallySparseBatchInterface &output, float learningRate,
+                 float momentum);
   int calculateInputSpatialSize(int outputSpatialSize);
 };
 
@@ -207,6 +234,10 @@ public:
   void forwards(SpatiallySparseBatch &batch,
                 SpatiallySparseBatchInterface &input,
                 SpatiallySparseBatchInterface &output);
+  void backwards(SpatiallySparseBatch &batch,
+                 SpatiallySparseBatchInterface &input,
+                 SpatiallySparseBatchInterface &output, float learningRate,
+                 float momentum);
   int calculateInputSpatialSize(int outputSpatialSize);
 };
 

@@ -1,6 +1,6 @@
-// Layer classes of the forward path.  preprocess() issues the rule-book
-// kernels, forwards() the feature kernels, all through the C ABI of
-// libscn_hip.so on the net's stream.
+// Layer classes.  preprocess() issues the rule-book kernels, forwards() the
+// feature kernels, backwards() the gradient kernels and the weight update, all
+// through the C ABI of libscn_hip.so on the net's stream.
 #include <cassert>
 #include <cmath>
 #include <cstdio>
@@ -8,7 +8,7 @@
 #include "SpatiallySparseLayer.h"
 
 static void unsupported(const char *what) {
-  std::fprintf(stderr, "%s is outside the forward path of this library\n", what);
+  std::fprintf(stderr, "%s is not implemented in this library\n", what);
   std::exit(EXIT_FAILURE);
 }
 
@@ -23,9 +23,7 @@ void SpatiallySparseLayer::scaleWeights(SpatiallySparseBatchInterface &,
 void SpatiallySparseLayer::backwards(SpatiallySparseBatch &,
                                      SpatiallySparseBatchInterface &,
                                      SpatiallySparseBatchInterface &, float,
-                                     float) {
-  unsupported("backwards()");
-}
+                                     float) {}
 
 // preprocess() runs on the batch slot's own stream when it has one, so that
 // rule books of several batches are built side by side
@@ -74,6 +72,23 @@ static void gather_now(cudaMemStream &ms, SpatiallySparseBatchInterface &input,
                               (int64_t)output.nSpatialSites * (width / nIn),
                               (int)nIn));
   output.deferredGatherFrom = nullptr;
+}
+
+// ConvolutionalLayer::backwards (ConvolutionalLayer.cu:134-147): scatter-add of
+// the gathered matrix's gradient through the rules
+static void conv_backwards(SpatiallySparseBatchInterface &input,
+                           SpatiallySparseBatchInterface &output,
+                           cudaMemStream &ms) {
+  if (!input.backpropErrors)
+    return;
+  const size_t nIn = input.featuresPresent.size();
+  const size_t width = output.featuresPresent.size();
+  input.sub->dfeatures.resize64((size_t)input.nSpatialSites * nIn);
+  input.sub->dfeatures.setZero(ms);
+  SCN_CHECKED(scn_gather_rows_backward(
+      ms.ctx, input.sub->dfeatures.dPtr(), output.sub->dfeatures.dPtr(),
+      output.rules.dPtr(), (int64_t)output.nSpatialSites * (width / nIn),
+      (int)nIn));
 }
 
 // featuresPresent of a convolution's output: fs copies of the input's list,
@@ -129,12 +144,19 @@ void ConvolutionalLayer::preprocess(SpatiallySparseBatch &batch,
 void ConvolutionalLayer::forwards(SpatiallySparseBatch &batch,
                                   SpatiallySparseBatchInterface &input,
                                   SpatiallySparseBatchInterface &output) {
-  (void)batch;
-  if (deferGather) { // the following NiN layer reads the input through the rules
-    output.deferredGatherFrom = &input;
+  // (the backward pass needs the gathered matrix: no deferral while training)
+  if (deferGather && batch.type != TRAINBATCH) {
+    output.deferredGatherFrom = &input; // the following NiN layer gathers
     return;
   }
   gather_now(memStream, input, output);
+}
+void ConvolutionalLayer::backwards(SpatiallySparseBatch &batch,
+                                   SpatiallySparseBatchInterface &input,
+                                   SpatiallySparseBatchInterface &output,
+                                   float learningRate, float momentum) {
+  (void)batch, (void)learningRate, (void)momentum;
+  conv_backwards(input, output, memStream);
 }
 int ConvolutionalLayer::calculateInputSpatialSize(int outputSpatialSize) {
   outSpatialSize = outputSpatialSize;
@@ -186,12 +208,17 @@ void ConvolutionalTriangularLayer::preprocess(
 void ConvolutionalTriangularLayer::forwards(
     SpatiallySparseBatch &batch, SpatiallySparseBatchInterface &input,
     SpatiallySparseBatchInterface &output) {
-  (void)batch;
-  if (deferGather) { // the following NiN layer reads the input through the rules
-    output.deferredGatherFrom = &input;
+  if (deferGather && batch.type != TRAINBATCH) {
+    output.deferredGatherFrom = &input; // the following NiN layer gathers
     return;
   }
   gather_now(memStream, input, output);
+}
+void ConvolutionalTriangularLayer::backwards(
+    SpatiallySparseBatch &batch, SpatiallySparseBatchInterface &input,
+    SpatiallySparseBatchInterface &output, float learningRate, float momentum) {
+  (void)batch, (void)learningRate, (void)momentum;
+  conv_backwards(input, output, memStream);
 }
 int ConvolutionalTriangularLayer::calculateInputSpatialSize(
     int outputSpatialSize) {
@@ -242,6 +269,50 @@ static bool nin_fused(cudaMemStream &ms, SpatiallySparseBatchInterface &input,
   return true;
 }
 
+// NetworkInNetwork(PReLU)Layer::backwards without dropout
+// (NetworkInNetworkLayer.cu:219-289, NetworkInNetworkPReLULayer.cu:190-277):
+// activation derivative in place (+ bias and slope gradients), slope update,
+// dW = A^T D, dA = D W^T with the weights of the forward pass, then the
+// momentum step on W and B.
+static void nin_backwards(cudaMemStream &ms,
+                          SpatiallySparseBatchInterface &input,
+                          SpatiallySparseBatchInterface &output, int K, int N,
+                          int act, vectorCUDA<float> &W, vectorCUDA<float> &MW,
+                          vectorCUDA<float> &B, vectorCUDA<float> &MB,
+                          vectorCUDA<float> *PReLU, vectorCUDA<float> *MPReLU,
+                          vectorCUDA<float> &dw, vectorCUDA<float> &db,
+                          vectorCUDA<float> *dprelu,
+                          vectorCUDA<float> &workspace, float learningRate,
+                          float momentum) {
+  const int64_t M = output.nSpatialSites;
+  dw.resize64((size_t)K * N);
+  db.resize64((size_t)N);
+  if (dprelu)
+    dprelu->resize64((size_t)N);
+  SCN_CHECKED(scn_activation_backward(
+      ms.ctx, output.sub->features.dPtr(), output.sub->dfeatures.dPtr(), M, N,
+      act, PReLU ? PReLU->dPtr() : nullptr, db.dPtr(),
+      dprelu ? dprelu->dPtr() : nullptr));
+  if (PReLU)
+    SCN_CHECKED(scn_nag_update(ms.ctx, dprelu->dPtr(), MPReLU->dPtr(),
+                               PReLU->dPtr(), N, learningRate, momentum, 1));
+  SCN_CHECKED(scn_sgemm_AtB(ms.ctx, input.sub->features.dPtr(),
+                            output.sub->dfeatures.dPtr(), dw.dPtr(), M, K, N));
+  multiplyAddCount += (__int128_t)M * K * N;
+  if (input.backpropErrors) {
+    input.sub->dfeatures.resize64((size_t)input.nSpatialSites * K);
+    workspace.resize64((size_t)scn_sgemm_ABt_workspace(N, K));
+    SCN_CHECKED(scn_sgemm_ABt(ms.ctx, output.sub->dfeatures.dPtr(), W.dPtr(),
+                              input.sub->dfeatures.dPtr(), M, N, K,
+                              workspace.dPtr()));
+    multiplyAddCount += (__int128_t)M * K * N;
+  }
+  SCN_CHECKED(scn_nag_update(ms.ctx, dw.dPtr(), MW.dPtr(), W.dPtr(),
+                             (int64_t)K * N, learningRate, momentum, 0));
+  SCN_CHECKED(scn_nag_update(ms.ctx, db.dPtr(), MB.dPtr(), B.dPtr(), N,
+                             learningRate, momentum, 0));
+}
+
 static void read_floats(std::ifstream &f, vectorCUDA<float> &v) {
   std::vector<float> &h = v.hVector();
   f.read((char *)h.data(), sizeof(float) * h.size());
@@ -274,8 +345,8 @@ NetworkInNetworkLayer::NetworkInNetworkLayer(cudaMemStream &memStream,
 void NetworkInNetworkLayer::preprocess(SpatiallySparseBatch &batch,
                                        SpatiallySparseBatchInterface &input,
                                        SpatiallySparseBatchInterface &output) {
-  if (batch.type == TRAINBATCH)
-    unsupported("a TRAINBATCH (dropout and the backward pass)");
+  if (batch.type == TRAINBATCH && dropout > 0)
+    unsupported("dropout during training");
   nin_preprocess(nFeaturesIn, nFeaturesOut, input, output);
 }
 void NetworkInNetworkLayer::forwards(SpatiallySparseBatch &batch,
@@ -293,6 +364,15 @@ void NetworkInNetworkLayer::forwards(SpatiallySparseBatch &batch,
                                 p, (int)fn, precision));
   multiplyAddCount +=
       (__int128_t)output.nSpatialSites * nFeaturesIn * nFeaturesOut;
+}
+void NetworkInNetworkLayer::backwards(SpatiallySparseBatch &batch,
+                                      SpatiallySparseBatchInterface &input,
+                                      SpatiallySparseBatchInterface &output,
+                                      float learningRate, float momentum) {
+  (void)batch;
+  nin_backwards(memStream, input, output, nFeaturesIn, nFeaturesOut, (int)fn, W,
+                MW, B, MB, nullptr, nullptr, dw, db, nullptr, workspace,
+                learningRate, momentum);
 }
 void NetworkInNetworkLayer::loadWeightsFromStream(std::ifstream &f,
                                                   bool momentum) {
@@ -343,8 +423,8 @@ NetworkInNetworkPReLULayer::NetworkInNetworkPReLULayer(
 void NetworkInNetworkPReLULayer::preprocess(
     SpatiallySparseBatch &batch, SpatiallySparseBatchInterface &input,
     SpatiallySparseBatchInterface &output) {
-  if (batch.type == TRAINBATCH)
-    unsupported("a TRAINBATCH (dropout and the backward pass)");
+  if (batch.type == TRAINBATCH && dropout > 0)
+    unsupported("dropout during training");
   nin_preprocess(nFeaturesIn, nFeaturesOut, input, output);
 }
 void NetworkInNetworkPReLULayer::forwards(
@@ -361,6 +441,14 @@ void NetworkInNetworkPReLULayer::forwards(
                                 p, (int)PRELU, precision));
   multiplyAddCount +=
       (__int128_t)output.nSpatialSites * nFeaturesIn * nFeaturesOut;
+}
+void NetworkInNetworkPReLULayer::backwards(
+    SpatiallySparseBatch &batch, SpatiallySparseBatchInterface &input,
+    SpatiallySparseBatchInterface &output, float learningRate, float momentum) {
+  (void)batch;
+  nin_backwards(memStream, input, output, nFeaturesIn, nFeaturesOut,
+                (int)PRELU, W, MW, B, MB, &PReLU, &MPReLU, dw, db, &dprelu,
+                workspace, learningRate, momentum);
 }
 void NetworkInNetworkPReLULayer::loadWeightsFromStream(std::ifstream &f,
                                                        bool momentum) {
@@ -429,6 +517,26 @@ static void pool_forwards(cudaMemStream &ms,
                           output.nSpatialSites, width, (int)nf,
                           output.sub->poolingChoices.dPtr()));
 }
+// MaxPoolingLayer::backwards (MaxPoolingLayer.cu:134-146)
+static void pool_backwards(cudaMemStream &ms,
+                           SpatiallySparseBatchInterface &input,
+                           SpatiallySparseBatchInterface &output) {
+  if (!input.backpropErrors)
+    return;
+  const size_t nf = output.featuresPresent.size();
+  input.sub->dfeatures.resize64((size_t)input.nSpatialSites * nf);
+  input.sub->dfeatures.setZero(ms);
+  SCN_CHECKED(scn_maxpool_backward(
+      ms.ctx, input.sub->dfeatures.dPtr(), output.sub->dfeatures.dPtr(),
+      output.nSpatialSites, (int)nf, output.sub->poolingChoices.dPtr()));
+}
+void MaxPoolingLayer::backwards(SpatiallySparseBatch &batch,
+                                SpatiallySparseBatchInterface &input,
+                                SpatiallySparseBatchInterface &output,
+                                float learningRate, float momentum) {
+  (void)batch, (void)learningRate, (void)momentum;
+  pool_backwards(memStream, input, output);
+}
 void MaxPoolingLayer::forwards(SpatiallySparseBatch &batch,
                                SpatiallySparseBatchInterface &input,
                                SpatiallySparseBatchInterface &output) {
@@ -473,6 +581,12 @@ void MaxPoolingTriangularLayer::preprocess(
                                         &n));
   output.nSpatialSites = (int)n;
   fill_rules(ctx, input, output, n * S);
+}
+void MaxPoolingTriangularLayer::backwards(
+    SpatiallySparseBatch &batch, SpatiallySparseBatchInterface &input,
+    SpatiallySparseBatchInterface &output, float learningRate, float momentum) {
+  (void)batch, (void)learningRate, (void)momentum;
+  pool_backwards(memStream, input, output);
 }
 void MaxPoolingTriangularLayer::forwards(SpatiallySparseBatch &batch,
                                          SpatiallySparseBatchInterface &input,
@@ -524,6 +638,22 @@ void TerminalPoolingLayer::forwards(SpatiallySparseBatch &batch,
       output.rules.dPtr(), output.nSpatialSites,
       (int)(output.rules.size64() / batch.batchSize), (int)nf));
 }
+// TerminalPoolingLayer::backwards (TerminalPoolingLayer.cu:112-125)
+void TerminalPoolingLayer::backwards(SpatiallySparseBatch &batch,
+                                     SpatiallySparseBatchInterface &input,
+                                     SpatiallySparseBatchInterface &output,
+                                     float learningRate, float momentum) {
+  (void)learningRate, (void)momentum;
+  if (!input.backpropErrors)
+    return;
+  const size_t nf = output.featuresPresent.size();
+  input.sub->dfeatures.resize64((size_t)input.nSpatialSites * nf);
+  input.sub->dfeatures.setZero(memStream);
+  SCN_CHECKED(scn_terminal_pool_backward(
+      memStream.ctx, input.sub->dfeatures.dPtr(), output.sub->dfeatures.dPtr(),
+      output.rules.dPtr(), output.nSpatialSites, (int)nf,
+      (int)(output.rules.size64() / batch.batchSize)));
+}
 int TerminalPoolingLayer::calculateInputSpatialSize(int outputSpatialSize) {
   assert(outputSpatialSize == 1);
   (void)outputSpatialSize;
@@ -541,8 +671,16 @@ void SoftmaxClassifierLaunch(SpatiallySparseBatchInterface &input,
                              cudaMemStream &memStream) {
   assert(batch.batchSize == input.nSpatialSites);
   assert(input.nFeatures == (int)input.featuresPresent.size());
-  if (batch.type == TRAINBATCH)
-    unsupported("a TRAINBATCH (dropout and the backward pass)");
+  if (batch.type == TRAINBATCH) {
+    // the backward pass starts here: d cost / d soft-max input
+    // (SoftmaxClassifier.cu:22-31)
+    input.sub->dfeatures.resize64((size_t)input.nSpatialSites *
+                                  input.nFeatures);
+    SCN_CHECKED(scn_softmax_grad(memStream.ctx, input.sub->features.dPtr(),
+                                 batch.labels.dPtr(),
+                                 input.sub->dfeatures.dPtr(), batch.batchSize,
+                                 input.nFeatures));
+  }
   BatchResultStage &r = *batch.result;
   const size_t n = (size_t)batch.batchSize * input.nFeatures;
   if (n > r.capacity) {

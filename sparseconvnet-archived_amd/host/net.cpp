@@ -268,10 +268,21 @@ void SparseConvNetCUDA::setPrecision(int precision) {
 void SparseConvNetCUDA::processBatch(SpatiallySparseBatch &batch,
                                      float learningRate, float momentum,
                                      std::ofstream &f, std::ofstream &g) {
-  (void)learningRate;
-  (void)momentum;
   forwardBatch(batch);
+  if (batch.type == TRAINBATCH)
+    backwardBatch(batch, learningRate, momentum);
   finishBatch(batch, f, g);
+}
+// The training half of processBatch (SparseConvNetCUDA.cu:248-252): the
+// classifier has left d cost / d soft-max input in the top interface; every
+// layer, last to first, hands the gradient down and updates its weights.
+void SparseConvNetCUDA::backwardBatch(SpatiallySparseBatch &batch,
+                                      float learningRate, float momentum) {
+  for (int i = (int)layers.size() - 1; i >= 0; i--) {
+    scn_prof_tag(memStream.ctx, i);
+    layers[i]->backwards(batch, batch.interfaces[i], batch.interfaces[i + 1],
+                         learningRate, momentum);
+  }
 }
 // The two halves of processBatch.  forwardBatch only queues work on the net's
 // stream (every layer, then the copy of the probabilities to the host);
@@ -315,9 +326,9 @@ float SparseConvNetCUDA::processDataset(SpatiallySparseDataset &dataset,
                                         int batchSize, float learningRate,
                                         float momentum) {
   assert(dataset.pictures.size() > 0);
-  if (dataset.type == TRAINBATCH || dataset.type == RESCALEBATCH) {
-    std::fprintf(stderr, "processDataset: %s passes are outside the forward "
-                         "path of this library\n",
+  if (dataset.type == RESCALEBATCH) {
+    std::fprintf(stderr, "processDataset: %s passes are not implemented in "
+                         "this library\n",
                  batchTypeNames[dataset.type]);
     std::exit(EXIT_FAILURE);
   }
@@ -330,8 +341,6 @@ float SparseConvNetCUDA::processDataset(SpatiallySparseDataset &dataset,
     f.open("unlabelledData.predictions");
     g.open("unlabelledData.probabilities");
   }
-  (void)learningRate;
-  (void)momentum;
   bp.keepAlive = nBatchProducerThreads >= 2 ? 1 : 0;
   SpatiallySparseBatch *queued = nullptr; // forward pass queued, not yet read
   auto finish = [&](SpatiallySparseBatch *batch) {
@@ -341,6 +350,8 @@ float SparseConvNetCUDA::processDataset(SpatiallySparseDataset &dataset,
   };
   while (SpatiallySparseBatch *batch = bp.nextBatch()) {
     forwardBatch(*batch);
+    if (batch->type == TRAINBATCH)
+      backwardBatch(*batch, learningRate, momentum);
     if (queued)
       finish(queued);
     queued = batch;
@@ -545,6 +556,10 @@ BatchProducer::BatchProducer(SparseConvNetCUDA &cnn,
   assert(batchSize > 0);
   nBatches = ((int)dataset.pictures.size() + batchSize - 1) / batchSize;
   permutation = range((int)dataset.pictures.size());
+  if (dataset.type == TRAINBATCH && cnn.shuffleTrainingData) {
+    RNG rng; // BatchProducer.cu:23-26
+    rng.vectorShuffle(permutation);
+  }
   start();
 }
 BatchProducer::BatchProducer(SparseConvNetCUDA &cnn,

@@ -18,6 +18,7 @@ struct scnh_net {
   std::unique_ptr<BatchProducer> producer;
   SpatiallySparseBatch *batch = nullptr;
   bool hasClassifier = false;
+  float learningRate = 0, momentum = 0; // of the batches scnh_next_batch runs
 };
 struct scnh_dataset {
   SpatiallySparseDataset ds;
@@ -135,6 +136,28 @@ static void put(vectorCUDA<float> &v, const float *src) {
   std::vector<float> &h = v.hVector();
   std::copy(src, src + h.size(), h.begin());
   v.copyToGPU();
+}
+static void get(vectorCUDA<float> &v, float *out) {
+  if (!out)
+    return;
+  SCN_CHECKED(scn_d2h(scnDefaultContext(), out, v.dPtr(),
+                      v.size64() * sizeof(float)));
+}
+int scnh_get_weights(scnh_net *net, int layer, int momentum, float *W,
+                     float *B, float *prelu) {
+  SpatiallySparseLayer *l = net->cnn->layers.at(layer);
+  if (auto *c = dynamic_cast<NetworkInNetworkLayer *>(l)) {
+    get(momentum ? c->MW : c->W, W);
+    get(momentum ? c->MB : c->B, B);
+    return 0;
+  }
+  if (auto *c = dynamic_cast<NetworkInNetworkPReLULayer *>(l)) {
+    get(momentum ? c->MW : c->W, W);
+    get(momentum ? c->MB : c->B, B);
+    get(momentum ? c->MPReLU : c->PReLU, prelu);
+    return 0;
+  }
+  return -1;
 }
 int scnh_set_weights(scnh_net *net, int layer, const float *W, const float *B,
                      const float *prelu) {
@@ -310,6 +333,17 @@ int64_t scnh_dataset_size(scnh_dataset *ds) {
 float scnh_process_dataset(scnh_net *net, scnh_dataset *ds, int batchSize) {
   return net->cnn->processDataset(ds->ds, batchSize);
 }
+float scnh_process_dataset_train(scnh_net *net, scnh_dataset *ds,
+                                 int batchSize, float learningRate,
+                                 float momentum) {
+  return net->cnn->processDataset(ds->ds, batchSize, learningRate, momentum);
+}
+void scnh_set_training(scnh_net *net, float learningRate, float momentum,
+                       int shuffle) {
+  net->learningRate = learningRate;
+  net->momentum = momentum;
+  net->cnn->shuffleTrainingData = shuffle != 0;
+}
 void scnh_process_dataset_repeat_test(scnh_net *net, scnh_dataset *ds,
                                       int batchSize, int nReps) {
   net->cnn->processDatasetRepeatTest(ds->ds, batchSize, nReps);
@@ -340,7 +374,7 @@ static void forward_layers(scnh_net *net, SpatiallySparseBatch &b) {
   SparseConvNetCUDA *cnn = net->cnn;
   if (net->hasClassifier) {
     std::ofstream f, g;
-    cnn->processBatch(b, 0, 0, f, g);
+    cnn->processBatch(b, net->learningRate, net->momentum, f, g);
   } else {
     for (size_t i = 0; i < cnn->layers.size(); i++) {
       b.interfaces[i + 1].sub->reset();
@@ -406,6 +440,14 @@ void scnh_iface_features(scnh_net *net, int i, float *out) {
   SpatiallySparseBatchInterface &f = net->batch->interfaces.at(i);
   SCN_CHECKED(scn_d2h(net->cnn->memStream.ctx, out, f.sub->features.dPtr(),
                       (size_t)f.nSpatialSites * f.nFeatures * sizeof(float)));
+}
+void scnh_iface_dfeatures(scnh_net *net, int i, float *out) {
+  SpatiallySparseBatchInterface &f = net->batch->interfaces.at(i);
+  SCN_CHECKED(scn_d2h(net->cnn->memStream.ctx, out, f.sub->dfeatures.dPtr(),
+                      f.sub->dfeatures.size64() * sizeof(float)));
+}
+int64_t scnh_iface_dfeatures_size(scnh_net *net, int i) {
+  return (int64_t)net->batch->interfaces.at(i).sub->dfeatures.size64();
 }
 void scnh_iface_choices(scnh_net *net, int i, int32_t *out) {
   SpatiallySparseBatchInterface &f = net->batch->interfaces.at(i);

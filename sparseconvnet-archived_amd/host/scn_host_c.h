@@ -36,6 +36,10 @@ int scnh_layer_info(scnh_net *net, int layer, int *nIn, int *nOut, int *act);
 /* NetworkInNetwork(PReLU)Layer::W, B, PReLU */
 int scnh_set_weights(scnh_net *net, int layer, const float *W, const float *B,
                      const float *prelu);
+/* the same vectors read back (momentum != 0: MW, MB, MPReLU); a null pointer
+ * skips that vector */
+int scnh_get_weights(scnh_net *net, int layer, int momentum, float *W,
+                     float *B, float *prelu);
 void scnh_save_weights(scnh_net *net, const char *baseName, int epoch);
 void scnh_load_weights(scnh_net *net, const char *baseName, int epoch);
 
@@ -100,6 +104,16 @@ int64_t scnh_codify_picture(scnh_dataset *ds, int64_t index, int spatialSize,
 
 /* SparseConvNet::processDataset / processDatasetRepeatTest */
 float scnh_process_dataset(scnh_net *net, scnh_dataset *ds, int batchSize);
+/* the same with processDataset's learningRate and momentum: one pass of
+ * training when the dataset's type is TRAINBATCH */
+float scnh_process_dataset_train(scnh_net *net, scnh_dataset *ds,
+                                 int batchSize, float learningRate,
+                                 float momentum);
+/* learning rate and momentum of the batches that scnh_next_batch processes
+ * (used by TRAINBATCH datasets), and whether training batches are drawn in
+ * shuffled order (the reference always shuffles, BatchProducer.cu:23-26) */
+void scnh_set_training(scnh_net *net, float learningRate, float momentum,
+                       int shuffle);
 void scnh_process_dataset_repeat_test(scnh_net *net, scnh_dataset *ds,
                                       int batchSize, int nReps);
 
@@ -131,6 +145,11 @@ void scnh_iface_info(scnh_net *net, int i, int *nFeatures, int *nSpatialSites,
                      int64_t *nChoices, int64_t *nGridEntries);
 void scnh_iface_rules(scnh_net *net, int i, int32_t *out);
 void scnh_iface_features(scnh_net *net, int i, float *out);
+/* gradient of the cost with respect to that feature matrix after a TRAINBATCH
+ * (SpatiallySparseBatchSubInterface::dfeatures); size in floats, 0 when the
+ * backward pass did not reach the interface */
+int64_t scnh_iface_dfeatures_size(scnh_net *net, int i);
+void scnh_iface_dfeatures(scnh_net *net, int i, float *out);
 void scnh_iface_choices(scnh_net *net, int i, int32_t *out);
 void scnh_iface_grids(scnh_net *net, int i, int32_t *sample, int64_t *key,
                       int32_t *row, int32_t *background);

@@ -62,6 +62,11 @@ def lib():
         "scnh_dataset_add_cifar10_file": (i64, [vp, C.c_char_p]),
         "scnh_codify_picture": (i64, [vp, i64, i32, i64, i64, vp, vp, vp, vp]),
         "scnh_process_dataset": (f32, [vp, vp, i32]),
+        "scnh_process_dataset_train": (f32, [vp, vp, i32, f32, f32]),
+        "scnh_set_training": (None, [vp, f32, f32, i32]),
+        "scnh_get_weights": (i32, [vp, i32, i32, vp, vp, vp]),
+        "scnh_iface_dfeatures_size": (i64, [vp, i32]),
+        "scnh_iface_dfeatures": (None, [vp, i32, vp]),
         "scnh_process_dataset_repeat_test": (None, [vp, vp, i32, i32]),
         "scnh_process_dataset_dump_top_level_features": (None, [vp, vp, i32, i32]),
         "scnh_calculate_input_regularizing_constants": (None, [vp, vp]),
@@ -242,6 +247,31 @@ class Net:
         pr = np.ascontiguousarray(prelu, np.float32) if prelu is not None else None
         rc = lib().scnh_set_weights(self.h, layer, _p(W), _p(B), _p(pr) if pr is not None else None)
         assert rc == 0, "layer %d has no weights" % layer
+
+    def get_weights(self, layer, momentum=False):
+        """(W [K x N], B [N], PReLU slopes [N] or None) of a NiN layer, or their momentum vectors"""
+        l = self.layers()[layer]
+        W = np.empty((l["nIn"], l["nOut"]), np.float32)
+        B = np.empty(l["nOut"], np.float32)
+        pr = np.empty(l["nOut"], np.float32) if l["kind"] == "nin_prelu" else None
+        rc = lib().scnh_get_weights(self.h, layer, int(momentum), _p(W), _p(B), _p(pr) if pr is not None else None)
+        assert rc == 0, "layer %d has no weights" % layer
+        return W, B, pr
+
+    def set_training(self, learningRate, momentum, shuffle=True):
+        """learning rate and momentum of TRAINBATCH batches run by next_batch(); shuffled order or not"""
+        lib().scnh_set_training(self.h, learningRate, momentum, int(shuffle))
+
+    def processDatasetTrain(self, ds, batchSize=100, learningRate=0.0, momentum=0.99):
+        return lib().scnh_process_dataset_train(self.h, ds.h, batchSize, learningRate, momentum)
+
+    def dfeatures(self, i):
+        """gradient left in interface i by the last TRAINBATCH, flat; empty if the backward pass stopped above it"""
+        n = lib().scnh_iface_dfeatures_size(self.h, i)
+        out = np.empty(n, np.float32)
+        if n:
+            lib().scnh_iface_dfeatures(self.h, i, _p(out))
+        return out
 
     def saveWeights(self, base, epoch):
         lib().scnh_save_weights(self.h, base.encode(), epoch)
