@@ -148,6 +148,19 @@ int scn_rules_triangular_plan(scn_ctx *ctx, const scn_grids *in,
                               scn_grids *out, int nIn, int nOut, int size,
                               int stride, int minActive,
                               int64_t *nOutputSpatialSites);
+/* gridRules over FractionalPoolingRegions (Regions.cu:121-156; dispatcher
+ * :782-802), the rule books of the four fractional max-pooling layers
+ * (MaxPoolingLayer.cu:157-420).  The regions of sample b along axis a are
+ * [h_inputL[(b d + a) nOut + j], h_inputR[..]) for output coordinate j: what
+ * the reference's tick constructors draw (Regions.cu:31-119), host arrays of
+ * batch * dimension * nOut ints each.  Region extents lie in 1..poolSize and
+ * both bounds are non-decreasing in j.  Rule rows are poolSize^d wide; offsets
+ * beyond a region's extent hold -1 (Regions.cu:177-178), which scn_maxpool
+ * skips.  Plan, then scn_rules_fill, as for the regular regions. */
+int scn_rules_fmp_plan(scn_ctx *ctx, const scn_grids *in, scn_grids *out,
+                       int nIn, int nOut, int poolSize,
+                       const int32_t *h_inputL, const int32_t *h_inputR,
+                       int64_t *nOutSites);
 /* TerminalPoolingLayer::preprocess + terminalGridPoolingRules
  * (TerminalPoolingLayer.cu:8-20,81-97).  *ruleWidth = S. */
 int scn_rules_terminal_plan(scn_ctx *ctx, const scn_grids *in, scn_grids *out,

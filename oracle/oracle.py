@@ -55,6 +55,12 @@ def _load():
         "orc_terminal_pool": (None, [vp, vp, vp, i64, C.c_int, C.c_int]),
         "orc_top_indices": (None, [vp, C.c_int, C.c_int, vp]),
         "orc_softmax_classifier": (C.c_int, [vp, vp, C.c_int, C.c_int, C.c_int, vp, vp]),
+        "orc_fmp_ticks_po": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_double, vp, vp]),
+        "orc_fmp_ticks_pd": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_double, vp, vp]),
+        "orc_fmp_increments": (C.c_int, [C.c_int, C.c_int, C.c_int, vp]),
+        "orc_fmp_ticks_ro": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, vp]),
+        "orc_fmp_ticks_rd": (C.c_int, [C.c_int, C.c_int, vp, vp, vp]),
+        "orc_rules_fmp": (i64, [vp, vp, C.c_int, C.c_int, C.c_int, C.c_int, vp, vp, C.c_int, vp]),
         "orc_softmax_grad": (None, [vp, vp, vp, i64, C.c_int]),
         "orc_activation_backward": (None, [vp, vp, i64, C.c_int, C.c_int, vp, vp, vp]),
         "orc_sgemm_AtB": (None, [vp, vp, vp, i64, C.c_int, C.c_int]),
@@ -171,6 +177,40 @@ def rules_triangular(grids, dimension, nIn, nOut, size, stride, minActive=1):
     rules = _ivec_take(v)
     if n < 0:
         raise ValueError("orc_rules_triangular: bad arguments")
+    return out, rules, int(n)
+
+
+def fmp_ticks(kind, nIn, nOut, poolSize, draw):
+    """(inputL, inputR) of one axis.  kind: "po" / "pd" (pseudorandom overlapping / disjoint; draw = u in [0, 1))
+    or "ro" / "rd" (random; draw = the shuffled increments, see fmp_increments).  None when the reference asserts."""
+    L, R = np.empty(nOut, np.int32), np.empty(nOut, np.int32)
+    if kind == "po":
+        rc = lib.orc_fmp_ticks_po(nIn, nOut, poolSize, float(draw), _p(L), _p(R))
+    elif kind == "pd":
+        rc = lib.orc_fmp_ticks_pd(nIn, nOut, poolSize, float(draw), _p(L), _p(R))
+    elif kind == "ro":
+        rc = lib.orc_fmp_ticks_ro(nIn, nOut, poolSize, _p(_i32(draw)), _p(L), _p(R))
+    else:
+        rc = lib.orc_fmp_ticks_rd(nIn, nOut, _p(_i32(draw)), _p(L), _p(R))
+    return (L, R) if rc == 0 else None
+
+
+def fmp_increments(nIn, nOut, overlapping):
+    inc = np.empty(nOut, np.int32)
+    n = lib.orc_fmp_increments(nIn, nOut, int(overlapping), _p(inc))
+    return inc[:n].copy()
+
+
+def rules_fmp(grids, dimension, nIn, nOut, poolSize, inputL, inputR, uniform):
+    """inputL / inputR: [batch, dimension, nOut] int32"""
+    inputL, inputR = _i32(inputL), _i32(inputR)
+    assert inputL.shape == (grids.batch, dimension, nOut) == inputR.shape
+    out = Grids(grids.batch)
+    v = lib.orc_ivec_create()
+    n = lib.orc_rules_fmp(grids.h, out.h, dimension, nIn, nOut, poolSize, _p(inputL), _p(inputR), int(uniform), v)
+    rules = _ivec_take(v)
+    if n < 0:
+        raise ValueError("orc_rules_fmp: bad arguments")
     return out, rules, int(n)
 
 

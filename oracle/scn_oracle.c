@@ -12,6 +12,8 @@
  *   triangular NoMin     reference-executed known-answer vector + brute force
  *   triangular Min       brute-force builder                            [no reference vector]
  *   terminal rules       brute force
+ *   fractional regions   tick tables: closed forms at u = 0, partition / coverage invariants, extents in
+ *                        {floor, ceil} of the ratio; rule books: brute-force builder over explicit windows
  *   gather / max-pool    brute force on random inputs, tie and negative-rule cases
  *   NiN                  numpy float64 GEMM, W = I, W = 0, single non-zero
  *   softmax / top-k      closed forms
@@ -373,6 +375,160 @@ static int sq_valid(const vgrid *in, vgrid *out, int d, int nIn, int nOut,
 static void reset_out(orc_grids *out) {
   for (int i = 0; i < out->batch; ++i)
     vg_clear(&out->g[i]);
+}
+
+/* ---------- fractional max-pooling regions (Regions.cu:31-156) ----------
+ * The random draw itself (u, or the shuffled increments) is the caller's: the
+ * reference takes it from a clock-seeded mt19937. */
+
+/* PseudorandomOverlappingFmpTicks, Regions.cu:31-46 */
+int orc_fmp_ticks_po(int nIn, int nOut, int poolSize, double u,
+                     int32_t *inputL, int32_t *inputR) {
+  if (nIn < nOut - 1 + poolSize || nOut < 2)
+    return -1;
+  double alpha = (nIn - poolSize) * 1.0 / (nOut - 1);
+  for (int j = 0; j < nOut; ++j) {
+    int i = (int)((j + u) * alpha) - (int)(u * alpha);
+    inputL[j] = i;
+    inputR[j] = i + poolSize;
+  }
+  return inputR[nOut - 1] == nIn ? 0 : -1;
+}
+/* PseudorandomNonOverlappingFmpTicks, Regions.cu:59-71 */
+int orc_fmp_ticks_pd(int nIn, int nOut, int poolSize, double u,
+                     int32_t *inputL, int32_t *inputR) {
+  double alpha = nIn * 1.0 / nOut;
+  if (nIn < nOut - 1 + poolSize || (int)ceil(alpha) != poolSize)
+    return -1;
+  for (int j = 0; j < nOut; ++j)
+    inputL[j] = (int)((j + u) * alpha) - (int)(u * alpha);
+  for (int j = 1; j <= nOut; ++j)
+    inputR[j - 1] = (int)((j + u) * alpha) - (int)(u * alpha);
+  return inputR[nOut - 1] == nIn ? 0 : -1;
+}
+/* the increments RandomOverlappingFmpTicks / RandomNonOverlappingFmpTicks
+ * shuffle (Regions.cu:87-90, 113-116); returns how many there are */
+int orc_fmp_increments(int nIn, int nOut, int overlapping, int32_t *inc) {
+  int alpha = (int)(nIn * 1.0 / nOut);
+  int first = nOut * (alpha + 1) - nIn;
+  int total = overlapping ? nOut - 1 : nOut;
+  for (int k = 0; k < total; ++k)
+    inc[k] = k < first ? alpha : alpha + 1;
+  return total;
+}
+/* RandomOverlappingFmpTicks from shuffled increments, Regions.cu:91-98 */
+int orc_fmp_ticks_ro(int nIn, int nOut, int poolSize, const int32_t *inc,
+                     int32_t *inputL, int32_t *inputR) {
+  if (nIn <= nOut)
+    return -1;
+  inputL[0] = 0;
+  inputR[0] = poolSize;
+  for (int i = 0; i < nOut - 1; i++) {
+    inputL[i + 1] = inputL[i] + inc[i];
+    inputR[i + 1] = inputL[i + 1] + poolSize;
+  }
+  return inputR[nOut - 1] == nIn ? 0 : -1;
+}
+/* RandomNonOverlappingFmpTicks from shuffled increments, Regions.cu:117-124 */
+int orc_fmp_ticks_rd(int nIn, int nOut, const int32_t *inc, int32_t *inputL,
+                     int32_t *inputR) {
+  if (nIn <= nOut)
+    return -1;
+  inputL[0] = 0;
+  inputR[0] = inc[0];
+  for (int i = 0; i < nOut - 1; i++) {
+    inputL[i + 1] = inputL[i] + inc[i];
+    inputR[i + 1] = inputR[i] + inc[i + 1];
+  }
+  return inputR[nOut - 1] == nIn ? 0 : -1;
+}
+
+/* gridRulesOverlappingNoMin (uniform regions, Regions.cu:528-653) and
+ * gridRulesNonOverlapping (Regions.cu:158-336) over FractionalPoolingRegions:
+ * outputL / outputR from the ticks as Regions.cu:49-56.  inL / inR hold the
+ * regions of this sample, axis after axis (d * nOut ints each). */
+static void fmp_rules(const vgrid *in, vgrid *out, int d, int nIn, int nOut,
+                      int s, const int32_t *inL, const int32_t *inR,
+                      int uniform, int64_t *nSites, orc_ivec *rules) {
+  int sd = orc_ipow(s, d);
+  int32_t *outL = (int32_t *)malloc(sizeof(int32_t) * 2 * d * nIn);
+  int32_t *outR = outL + (size_t)d * nIn;
+  for (int a = 0; a < d; ++a) {
+    for (int i = 0; i < nIn; ++i) {
+      outL[a * nIn + i] = nOut;
+      outR[a * nIn + i] = 0;
+    }
+    for (int j = 0; j < nOut; ++j)
+      for (int i = inL[a * nOut + j]; i < inR[a * nOut + j]; ++i) {
+        if (j < outL[a * nIn + i])
+          outL[a * nIn + i] = j;
+        if (j + 1 > outR[a * nIn + i])
+          outR[a * nIn + i] = j + 1;
+      }
+  }
+  vg_resize(out, orc_ipow(nOut, d));
+  for (int64_t key = 0; key < in->len; ++key) {
+    if (in->vec[key] == VH_EMPTY)
+      continue;
+    int i[4], lo[4], hi[4], j[4];
+    decode(key, nIn, d, i);
+    for (int a = 0; a < d; ++a) {
+      lo[a] = outL[a * nIn + i[a]];
+      hi[a] = outR[a * nIn + i[a]];
+      j[a] = lo[a];
+    }
+    if (!box_nonempty(lo, hi, d))
+      continue;
+    do {
+      int64_t outKey = encode(j, nOut, d);
+      int off = 0;
+      for (int a = 0; a < d; ++a)
+        off = off * s + (i[a] - inL[a * nOut + j[a]]);
+      const int32_t *f = vg_find(out, outKey);
+      if (!f) {
+        int32_t *slot = vg_at(out, outKey);
+        *slot = (int32_t)((*nSites)++);
+        if (uniform) {
+          iv_resize(rules, *nSites * sd, in->backgroundCol);
+        } else { /* -1, then the background row inside the region's extent */
+          iv_resize(rules, *nSites * sd, -1);
+          int ii[4] = {0, 0, 0, 0}, zero[4] = {0, 0, 0, 0}, ext[4];
+          for (int a = 0; a < d; ++a)
+            ext[a] = inR[a * nOut + j[a]] - inL[a * nOut + j[a]];
+          do {
+            int k = 0;
+            for (int a = 0; a < d; ++a)
+              k = k * s + ii[a];
+            rules->d[(*nSites - 1) * sd + k] = in->backgroundCol;
+          } while (odo_next(ii, zero, ext, d));
+        }
+        f = slot;
+      }
+      rules->d[(int64_t)*f * sd + off] = in->vec[key];
+    } while (odo_next(j, lo, hi, d));
+  }
+  free(outL);
+  background_row(in, out, orc_ipow(nOut, d), sd, nSites, rules);
+}
+
+/* one rule book for the batch; inputL / inputR: batch * dimension * nOut ints
+ * (sample-major, then axis), as the layers draw new regions for every sample
+ * (MaxPoolingLayer.cu:181-186) */
+int64_t orc_rules_fmp(const orc_grids *in, orc_grids *out, int dimension,
+                      int nIn, int nOut, int poolSize, const int32_t *inputL,
+                      const int32_t *inputR, int uniform, orc_ivec *rules) {
+  if (in->batch != out->batch || dimension < 1 || dimension > 3)
+    return -1;
+  reset_out(out);
+  rules->n = 0;
+  int64_t nSites = 0;
+  for (int item = 0; item < in->batch; ++item) {
+    const int32_t *l = inputL + (size_t)item * dimension * nOut;
+    const int32_t *r = inputR + (size_t)item * dimension * nOut;
+    fmp_rules(&in->g[item], &out->g[item], dimension, nIn, nOut, poolSize, l,
+              r, uniform, &nSites, rules);
+  }
+  return nSites;
 }
 
 int64_t orc_rules_square(const orc_grids *in, orc_grids *out, int dimension,

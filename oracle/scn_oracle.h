@@ -104,6 +104,20 @@ int orc_softmax_classifier(const float *probs, const int32_t *labels,
 void orc_set_threads(int n); /* OpenMP threads for the numeric loops */
 int orc_get_threads(void);
 
+/* ---- fractional max-pooling regions and their rule books ---- */
+int orc_fmp_ticks_po(int nIn, int nOut, int poolSize, double u,
+                     int32_t *inputL, int32_t *inputR);
+int orc_fmp_ticks_pd(int nIn, int nOut, int poolSize, double u,
+                     int32_t *inputL, int32_t *inputR);
+int orc_fmp_increments(int nIn, int nOut, int overlapping, int32_t *inc);
+int orc_fmp_ticks_ro(int nIn, int nOut, int poolSize, const int32_t *inc,
+                     int32_t *inputL, int32_t *inputR);
+int orc_fmp_ticks_rd(int nIn, int nOut, const int32_t *inc, int32_t *inputL,
+                     int32_t *inputR);
+int64_t orc_rules_fmp(const orc_grids *in, orc_grids *out, int dimension,
+                      int nIn, int nOut, int poolSize, const int32_t *inputL,
+                      const int32_t *inputR, int uniform, orc_ivec *rules);
+
 /* ---- backward pass (training); citations in scn_oracle.c ---- */
 void orc_softmax_grad(const float *probs, const int32_t *labels, float *delta,
                       int64_t batch, int N);

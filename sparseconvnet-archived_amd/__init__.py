@@ -90,6 +90,7 @@ def lib():
         "scn_rules_square_plan": (C.c_int, [vp, vp, vp] + [C.c_int] * 5 + [P(i64)]),
         "scn_rules_triangular_plan": (C.c_int, [vp, vp, vp] + [C.c_int] * 5 + [P(i64)]),
         "scn_rules_terminal_plan": (C.c_int, [vp, vp, vp, P(i64)]),
+        "scn_rules_fmp_plan": (C.c_int, [vp, vp, vp, C.c_int, C.c_int, C.c_int, vp, vp, P(i64)]),
         "scn_rules_width": (C.c_int, [vp, P(i64)]),
         "scn_rules_fill": (C.c_int, [vp, vp, vp, vp, i64]),
         "scn_gather_rows": (C.c_int, [vp, vp, vp, vp, i64, C.c_int]),
@@ -349,6 +350,18 @@ class Grids:
         _check(lib().scn_rules_triangular_plan(self.ctx.h, self.h, out.h, nIn, nOut, size, stride, minActive, C.byref(n)))
         return n.value
 
+    def plan_fmp(self, out, nIn, nOut, poolSize, inputL, inputR):
+        """inputL / inputR: [batch, dimension, nOut] int32 host arrays (fractional max-pooling regions)"""
+        inputL = np.ascontiguousarray(inputL, np.int32)
+        inputR = np.ascontiguousarray(inputR, np.int32)
+        info = self.info()
+        assert inputL.shape == (info["batch"], info["dimension"], nOut) == inputR.shape
+        n = C.c_int64()
+        vp = lambda a: a.ctypes.data_as(C.c_void_p)
+        _check(lib().scn_rules_fmp_plan(self.ctx.h, self.h, out.h, nIn, nOut, poolSize, vp(inputL), vp(inputR),
+                                        C.byref(n)))
+        return n.value
+
     def plan_terminal(self, out):
         S = C.c_int64()
         _check(lib().scn_rules_terminal_plan(self.ctx.h, self.h, out.h, C.byref(S)))
@@ -388,6 +401,16 @@ def rules_square(ctx, grids, nIn, nOut, size, stride, minActive=1, triangular=Fa
     out = out if out is not None else Grids(ctx)
     plan = grids.plan_triangular if triangular else grids.plan_square
     n = plan(out, nIn, nOut, size, stride, minActive)
+    w = out.rules_width()
+    rules = ctx.empty(max(n * w, 1), np.int32)
+    grids.fill(out, rules, n * w)
+    return out, rules, n, w
+
+
+def rules_fmp(ctx, grids, nIn, nOut, poolSize, inputL, inputR, out=None):
+    """plan + fill over fractional max-pooling regions; returns (out grids, device rules, nOutSites, width)."""
+    out = out if out is not None else Grids(ctx)
+    n = grids.plan_fmp(out, nIn, nOut, poolSize, inputL, inputR)
     w = out.rules_width()
     rules = ctx.empty(max(n * w, 1), np.int32)
     grids.fill(out, rules, n * w)

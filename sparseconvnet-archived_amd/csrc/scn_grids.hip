@@ -29,7 +29,7 @@ struct __align__(16) Slot {
 };
 #define SLOT_EMPTY (-1LL)
 
-enum { MODE_SQ_NOMIN = 0, MODE_SQ_MIN, MODE_SQ_VALID, MODE_TRI_NOMIN, MODE_TRI_MIN };
+enum { MODE_SQ_NOMIN = 0, MODE_SQ_MIN, MODE_SQ_VALID, MODE_TRI_NOMIN, MODE_TRI_MIN, MODE_SQ_FMP };
 enum { PLAN_NONE = 0, PLAN_REGIONS = 1, PLAN_TERMINAL = 2 };
 
 struct Geom {
@@ -38,7 +38,18 @@ struct Geom {
   long long volIn, volOut;
   int width; // rule-row width: size^d or triangleSize(size, d)
   int cube;  // size^d
+  // MODE_SQ_FMP: per-sample, per-axis region tables (fractional max-pooling).
+  // inputL at ticks[(b d + a) nOut + j], inputR the same at tInR; outputL and
+  // outputR at tOutL / tOutR + (b d + a) nIn + i.  Null otherwise.
+  const int *ticks;
+  long long tInR, tOutL, tOutR;
 };
+__device__ __forceinline__ int fmp_inputL(const Geom &g, int b, int a, int j) {
+  return g.ticks[((long long)b * g.d + a) * g.nOut + j];
+}
+__device__ __forceinline__ int fmp_inputR(const Geom &g, int b, int a, int j) {
+  return g.ticks[g.tInR + ((long long)b * g.d + a) * g.nOut + j];
+}
 
 struct GridView {
   Slot *table;
@@ -103,6 +114,7 @@ struct scn_grids {
   DevBuf<int> bgBefore;
   DevBuf<unsigned> sampleStart;
   DevBuf<int> invOrd;
+  DevBuf<int> ticks; // region tables of a fractional max-pooling plan
   // scratch for download
   DevBuf<int> dlSample, dlRow;
   DevBuf<long long> dlKey;
@@ -191,30 +203,31 @@ __device__ __forceinline__ long long encode_key(const int *c, int n) {
 }
 
 // Is any site of the window with origin w active at a window offset that
-// precedes offset a (row-major)?  Square window of side `size`.
+// precedes offset a (row-major)?  The window has ext[axis] sites along each
+// axis (all equal for the regular regions).
 template <int D>
 __device__ __forceinline__ bool any_before(const unsigned long long *bits,
                                            long long sampleBase, int nIn,
-                                           int size, const int *w,
+                                           const int *ext, const int *w,
                                            const int *a) {
   if (D == 1) {
     return a[0] > 0 && get_bits(bits, sampleBase + w[0], a[0]) != 0;
   } else if (D == 2) {
     for (int q0 = 0; q0 < a[0]; ++q0)
-      if (get_bits(bits, sampleBase + (long long)(w[0] + q0) * nIn + w[1], size))
+      if (get_bits(bits, sampleBase + (long long)(w[0] + q0) * nIn + w[1], ext[1]))
         return true;
     return a[1] > 0 &&
            get_bits(bits, sampleBase + (long long)(w[0] + a[0]) * nIn + w[1],
                     a[1]) != 0;
   } else {
     for (int q0 = 0; q0 <= a[0]; ++q0) {
-      int q1max = (q0 < a[0]) ? size : a[1];
+      int q1max = (q0 < a[0]) ? ext[1] : a[1];
       for (int q1 = 0; q1 < q1max; ++q1)
         if (get_bits(bits,
                      sampleBase +
                          ((long long)(w[0] + q0) * nIn + (w[1] + q1)) * nIn +
                          w[2],
-                     size))
+                     ext[2]))
           return true;
     }
     return a[2] > 0 &&
@@ -259,9 +272,18 @@ __device__ __forceinline__ int count_active(const unsigned long long *bits,
 // (Regions.cu:13-29), or for valid mode the single site (i0-1, i1-1) when
 // 1 <= i <= nOut on each axis (Regions.cu:693-697).  False when empty.
 template <int D>
-__device__ __forceinline__ bool cand_box(const Geom &g, const int *i, int *lo,
-                                         int *hi) {
-  if (g.mode == MODE_SQ_VALID) {
+__device__ __forceinline__ bool cand_box(const Geom &g, int b, const int *i,
+                                         int *lo, int *hi) {
+  if (g.mode == MODE_SQ_FMP) { // tables (Regions.cu:143-150)
+#pragma unroll
+    for (int a = 0; a < D; ++a) {
+      const long long t = ((long long)b * g.d + a) * g.nIn + i[a];
+      lo[a] = g.ticks[g.tOutL + t];
+      hi[a] = g.ticks[g.tOutR + t];
+      if (lo[a] >= hi[a])
+        return false;
+    }
+  } else if (g.mode == MODE_SQ_VALID) {
 #pragma unroll
     for (int a = 0; a < D; ++a) {
       if (i[a] < 1 || i[a] > g.nOut)
@@ -285,7 +307,7 @@ __device__ __forceinline__ bool cand_box(const Geom &g, const int *i, int *lo,
 // with the smallest key in j's window owns it; Min modes also need enough
 // active inputs; the triangular lattice only has outputs with sum(j) < nOut)
 template <int D>
-__device__ __forceinline__ bool owns(const GridView &in, const Geom &g,
+__device__ __forceinline__ bool owns(const GridView &in, const Geom &g, int b,
                                      long long sampleBase, const int *i,
                                      const int *j) {
   if (g.mode == MODE_TRI_NOMIN || g.mode == MODE_TRI_MIN) {
@@ -298,13 +320,23 @@ __device__ __forceinline__ bool owns(const GridView &in, const Geom &g,
   }
   if (g.mode == MODE_SQ_VALID)
     return true;
-  int w[D], off[D];
+  int w[D], off[D], ext[D];
+  if (g.mode == MODE_SQ_FMP) {
 #pragma unroll
-  for (int a = 0; a < D; ++a) {
-    w[a] = j[a] * g.stride;
-    off[a] = i[a] - w[a];
+    for (int a = 0; a < D; ++a) {
+      w[a] = fmp_inputL(g, b, a, j[a]);
+      ext[a] = fmp_inputR(g, b, a, j[a]) - w[a];
+      off[a] = i[a] - w[a];
+    }
+  } else {
+#pragma unroll
+    for (int a = 0; a < D; ++a) {
+      w[a] = j[a] * g.stride;
+      ext[a] = g.size;
+      off[a] = i[a] - w[a];
+    }
   }
-  if (any_before<D>(in.bits, sampleBase, g.nIn, g.size, w, off))
+  if (any_before<D>(in.bits, sampleBase, g.nIn, ext, w, off))
     return false;
   if (g.mode == MODE_SQ_MIN)
     return count_active<D, false>(in.bits, sampleBase, g.nIn, g.size, w) >=
@@ -323,7 +355,7 @@ __device__ __forceinline__ void for_each_owned(const GridView &in,
                                                const Geom &g, int b,
                                                const int *i, F f) {
   int lo[D], hi[D];
-  if (!cand_box<D>(g, i, lo, hi))
+  if (!cand_box<D>(g, b, i, lo, hi))
     return;
   const long long sampleBase = (long long)b * g.volIn;
   int j[D];
@@ -331,7 +363,7 @@ __device__ __forceinline__ void for_each_owned(const GridView &in,
   for (int a = 0; a < D; ++a)
     j[a] = lo[a];
   for (int c = 0;; ++c) {
-    if (owns<D>(in, g, sampleBase, i, j))
+    if (owns<D>(in, g, b, sampleBase, i, j))
       f(encode_key<D>(j, g.nOut), c);
     // odometer, last axis fastest
     int a = D - 1;
@@ -602,7 +634,7 @@ __global__ void k_plan_emit_masked(GridView in, GridView out, Geom g,
   int b = (int)(p / g.volIn);
   int i[D], lo[D], hi[D], j[D];
   decode_key<D>(p - (long long)b * g.volIn, g.nIn, i);
-  (void)cand_box<D>(g, i, lo, hi);
+  (void)cand_box<D>(g, b, i, lo, hi);
   int rem = c;
 #pragma unroll
   for (int a = D - 1; a >= 0; --a) {
@@ -649,7 +681,7 @@ __global__ void k_plan_emit_walk(GridView in, GridView out, Geom g,
   const int b = (int)(p / g.volIn);
   int i[D], lo[D], hi[D], j[D];
   decode_key<D>(p - (long long)b * g.volIn, g.nIn, i);
-  (void)cand_box<D>(g, i, lo, hi);
+  (void)cand_box<D>(g, b, i, lo, hi);
   unsigned idx = base[r];
   const int shiftRows = bgBefore[b];
   while (mask) { // ascending candidate = ascending output key
@@ -744,10 +776,28 @@ __global__ void __launch_bounds__(256)
   int j[D], c[D];
   decode_key<D>(sk - (long long)b * g.volOut, g.nOut, j);
   int cubeOff = invOrd ? invOrd[q] : q;
+  if (g.mode == MODE_SQ_FMP) {
+    // offsets past a region's extent keep the -1 the reference's rule rows
+    // start from (Regions.cu:177-178)
+    bool outside = false;
 #pragma unroll
-  for (int a = D - 1; a >= 0; --a) {
-    c[a] = j[a] * g.stride + cubeOff % g.size;
-    cubeOff /= g.size;
+    for (int a = D - 1; a >= 0; --a) {
+      const int o = cubeOff % g.size;
+      cubeOff /= g.size;
+      const int l = fmp_inputL(g, b, a, j[a]);
+      outside |= o >= fmp_inputR(g, b, a, j[a]) - l;
+      c[a] = l + o;
+    }
+    if (outside) {
+      rules[idx] = -1;
+      return;
+    }
+  } else {
+#pragma unroll
+    for (int a = D - 1; a >= 0; --a) {
+      c[a] = j[a] * g.stride + cubeOff % g.size;
+      cubeOff /= g.size;
+    }
   }
   long long p = (long long)b * g.volIn + encode_key<D>(c, g.nIn);
   int val;
@@ -1211,6 +1261,7 @@ extern "C" int scn_grids_destroy(scn_ctx *ctx, scn_grids *g) {
   g->bgBefore.release();
   g->sampleStart.release();
   g->invOrd.release();
+  g->ticks.release();
   g->dlSample.release();
   g->dlRow.release();
   g->dlKey.release();
@@ -1315,7 +1366,7 @@ static int triangle_size(int n, int d) { // utilities.cu:27-32
 template <int D>
 static int plan_regions_d(scn_ctx *ctx, scn_grids *in, scn_grids *out,
                           const Geom &g, long long fullSize,
-                          int64_t *nOutSites) {
+                          int64_t *nOutSites, long long fmpCand = 0) {
   // deferred: size by bounds, leave the counts on the device (see scn_rules_settle)
   const bool deferred = ctx->deferCounts && out->seenRows > 0 &&
                         (int)ctx->pendingGrids.size() < SCN_MAX_PENDING;
@@ -1343,6 +1394,8 @@ static int plan_regions_d(scn_ctx *ctx, scn_grids *in, scn_grids *out,
   long long maxCand = 1;
   for (int a = 0; a < D; ++a)
     maxCand *= g.mode == MODE_SQ_VALID ? 1 : (g.size + g.stride - 1) / g.stride;
+  if (g.mode == MODE_SQ_FMP)
+    maxCand = fmpCand; // from the tables themselves
   const bool masked = maxCand <= 64;
   if (masked) {
     SCN_TRY(out->ownMask.reserve((size_t)nE + 2));
@@ -1443,6 +1496,8 @@ static int plan_regions(scn_ctx *ctx, const scn_grids *cin, scn_grids *out,
   g.volIn = in->vol;
   g.volOut = ipow_ll(nOut, in->d);
   g.cube = (int)ipow_ll(size, in->d);
+  g.ticks = nullptr;
+  g.tInR = g.tOutL = g.tOutR = 0;
   SCN_REQUIRE(ipow_ll(size, in->d) <= 32768, SCN_ERR_ARG,
               "rules plan: window of %d^%d sites", size, in->d);
   long long fullSize;
@@ -1506,6 +1561,105 @@ extern "C" int scn_rules_triangular_plan(scn_ctx *ctx, const scn_grids *in,
                                          int64_t *nOutSites) {
   return plan_regions(ctx, in, out, nIn, nOut, size, stride, minActive, true,
                       nOutSites);
+}
+
+// gridRules over FractionalPoolingRegions (Regions.cu:121-156 and the tick
+// constructors :31-119): the caller brings inputL / inputR of every sample and
+// axis; outputL / outputR follow from them as in the tick constructors
+// (:49-56).  The tables are checked on the host so that no kernel indexes
+// outside a grid.
+extern "C" int scn_rules_fmp_plan(scn_ctx *ctx, const scn_grids *cin,
+                                  scn_grids *out, int nIn, int nOut,
+                                  int poolSize, const int32_t *h_inputL,
+                                  const int32_t *h_inputR,
+                                  int64_t *nOutSites) {
+  scn_grids *in = const_cast<scn_grids *>(cin);
+  SCN_REQUIRE(ctx && in && out && nOutSites && h_inputL && h_inputR,
+              SCN_ERR_ARG, "fmp rules plan: null argument");
+  SCN_REQUIRE(in != out, SCN_ERR_ARG,
+              "fmp rules plan: in and out are the same object");
+  SCN_REQUIRE(poolSize >= 1 && poolSize <= 32 && nOut >= 1, SCN_ERR_ARG,
+              "fmp rules plan: poolSize %d nOut %d", poolSize, nOut);
+  SCN_REQUIRE(nIn >= nOut - 1 + poolSize, SCN_ERR_ARG, // Regions.cu:35,131
+              "fmp rules plan: nIn %d < nOut %d - 1 + poolSize %d", nIn, nOut,
+              poolSize);
+  SCN_REQUIRE(in->n == nIn, SCN_ERR_ARG,
+              "fmp rules plan: input grids have spatialSize %d, regions say %d",
+              in->n, nIn);
+  const int d = in->d, B = in->batch;
+  SCN_REQUIRE(ipow_ll(poolSize, d) <= 32768, SCN_ERR_ARG,
+              "fmp rules plan: window of %d^%d sites", poolSize, d);
+  const size_t nT = (size_t)B * d * nOut, nI = (size_t)B * d * nIn;
+  std::vector<int> t(2 * nT + 2 * nI);
+  int *inL = t.data(), *inR = inL + nT, *outL = inR + nT, *outR = outL + nI;
+  long long cand = 1;
+  std::vector<int> widest(d, 0);
+  for (int b = 0; b < B; ++b)
+    for (int a = 0; a < d; ++a) {
+      const size_t o = ((size_t)b * d + a) * nOut, oi = ((size_t)b * d + a) * nIn;
+      for (int i = 0; i < nIn; ++i) {
+        outL[oi + i] = nOut;
+        outR[oi + i] = 0;
+      }
+      for (int j = 0; j < nOut; ++j) {
+        const int l = h_inputL[o + j], r = h_inputR[o + j];
+        SCN_REQUIRE(l >= 0 && r > l && r - l <= poolSize && r <= nIn &&
+                        (j == 0 || (l >= h_inputL[o + j - 1] &&
+                                    r >= h_inputR[o + j - 1])),
+                    SCN_ERR_ARG,
+                    "fmp rules plan: sample %d axis %d region %d = [%d, %d)", b,
+                    a, j, l, r);
+        inL[o + j] = l;
+        inR[o + j] = r;
+        for (int i = l; i < r; ++i) {
+          outL[oi + i] = outL[oi + i] < j ? outL[oi + i] : j;
+          outR[oi + i] = outR[oi + i] > j + 1 ? outR[oi + i] : j + 1;
+        }
+      }
+      for (int i = 0; i < nIn; ++i)
+        if (outR[oi + i] - outL[oi + i] > widest[a])
+          widest[a] = outR[oi + i] - outL[oi + i];
+    }
+  for (int a = 0; a < d; ++a)
+    cand *= widest[a] > 0 ? widest[a] : 1;
+  Geom g;
+  g.d = d;
+  g.nIn = nIn;
+  g.nOut = nOut;
+  g.size = poolSize;
+  g.stride = 1;
+  g.minActive = 1;
+  g.mode = MODE_SQ_FMP;
+  g.volIn = in->vol;
+  g.volOut = ipow_ll(nOut, d);
+  g.cube = (int)ipow_ll(poolSize, d);
+  g.width = g.cube;
+  g.tInR = (long long)nT;
+  g.tOutL = (long long)(2 * nT);
+  g.tOutR = (long long)(2 * nT + nI);
+  ProfScope ps(ctx, SCN_K_RULES);
+  SCN_TRY(out->ticks.reserve(t.size() + 1));
+  // (the copy returns when done: `t` may go out of scope)
+  SCN_TRY(scn_h2d(ctx, out->ticks.p, t.data(), t.size() * sizeof(int)));
+  g.ticks = out->ticks.p;
+  SCN_TRY(ensure_rank(ctx, in));
+  int rc;
+  switch (d) {
+  case 1:
+    rc = plan_regions_d<1>(ctx, in, out, g, g.volOut, nOutSites, cand);
+    break;
+  case 2:
+    rc = plan_regions_d<2>(ctx, in, out, g, g.volOut, nOutSites, cand);
+    break;
+  default:
+    rc = plan_regions_d<3>(ctx, in, out, g, g.volOut, nOutSites, cand);
+    break;
+  }
+  SCN_TRY(rc);
+  out->geom = g;
+  out->planKind = PLAN_REGIONS;
+  out->planIn = in;
+  return SCN_OK;
 }
 
 extern "C" int scn_rules_terminal_plan(scn_ctx *ctx, const scn_grids *cin,
@@ -1628,7 +1782,7 @@ extern "C" int scn_rules_fill(scn_ctx *ctx, const scn_grids *in,
       hipLaunchKernelGGL((KERNEL<3, false>), __VA_ARGS__);                     \
     break;                                                                     \
   }
-  if (!tri && g.size >= 2) {
+  if (!tri && g.size >= 2 && g.mode != MODE_SQ_FMP) {
     dim3 runs(scn_ceil_div(total / g.size, 256) + extra);
     SCN_FILL_DIM(k_rules_fill_runs, runs, block, 0, ctx->stream, vin, g,
                  out->siteKey.p, count_sites(out), out->meta.p, d_rules, rs)

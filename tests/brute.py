@@ -162,3 +162,40 @@ def rules_vectorized(d, batch, sIn, sOut, size, stride, gin):
         rules[rows, q] = dense[bs, kin]
     rules[bgOut[notFull]] = np.asarray(bg, np.int64)[notFull][:, None]
     return (bs, ks, rows), bgOut, nRows, rules
+
+
+def rules_windows(samples, d, nIn, nOut, s, inL, inR, uniform):
+    """Rule book over explicit per-sample windows (fractional max-pooling regions): output site j of sample b looks at
+    the cells [inL[b][a][j_a], inR[b][a][j_a]) along every axis a.  Rows are s^d wide; `uniform` rows start as all
+    background, others as -1 with the background row inside the window's extent.  Same return value as rules()."""
+    out_rules, n, outs = [], 0, []
+    S = s ** d
+    for b, (bg, mp) in enumerate(samples):
+        cands = []
+        for j in itertools.product(range(nOut), repeat=d):
+            ext = [int(inR[b][a][j[a]] - inL[b][a][j[a]]) for a in range(d)]
+            row = [bg if uniform else -1] * S
+            active = []
+            for o in itertools.product(*[range(e) for e in ext]):
+                cell = encode(tuple(int(inL[b][a][j[a]]) + o[a] for a in range(d)), nIn)
+                k = 0
+                for a in range(d):
+                    k = k * s + o[a]
+                row[k] = mp.get(cell, bg)
+                if cell in mp:
+                    active.append(cell)
+            if active:
+                cands.append((min(active), encode(j, nOut), row))
+        cands.sort(key=lambda t: (t[0], t[1]))
+        grid = {}
+        for _, okey, row in cands:
+            grid[okey] = n
+            n += 1
+            out_rules.extend(row)
+        obg = -1
+        if len(grid) < nOut ** d:
+            out_rules.extend([bg] * S)
+            obg = n
+            n += 1
+        outs.append((obg, grid))
+    return np.array(out_rules, np.int32), n, outs
