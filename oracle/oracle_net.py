@@ -56,6 +56,19 @@ class Net:
         if poolSize > 1:
             self.layers.append(dict(kind="maxpool_tri" if tri else "maxpool", size=poolSize, stride=poolStride, nIn=0, nOut=0))
 
+    def addLeNetLayerFMP(self, kind, nFeatures, filterSize, filterStride, poolSize, fmpShrink, activationFn=RELU,
+                         dropout=0.0, minActiveInputs=1):
+        """addLeNetLayerPOFMP / PDFMP / ROFMP / RDFMP (kind 0..3), SparseConvNetCUDA.cu:112-163"""
+        assert not self.triangular
+        if filterSize > 1:
+            fs = filterSize ** self.dimension
+            self.layers.append(dict(kind="conv", size=filterSize, stride=filterStride, minActive=minActiveInputs,
+                                    nIn=self.nOutputFeatures, nOut=self.nOutputFeatures * fs, fs=fs))
+            self.nOutputFeatures *= fs
+        self._learnt(nFeatures, activationFn, dropout)
+        if fmpShrink > 1:
+            self.layers.append(dict(kind="fmp", fmpKind=kind, size=poolSize, shrink=np.float32(fmpShrink), nIn=0, nOut=0))
+
     def addTerminalPoolingLayer(self, poolSize):
         self.layers.append(dict(kind="terminal", size=poolSize, nIn=0, nOut=0))
 
@@ -65,6 +78,9 @@ class Net:
             l["outSize"] = s
             if l["kind"] in ("conv", "conv_tri", "maxpool", "maxpool_tri"):
                 s = l["size"] + (s - 1) * l["stride"]
+            elif l["kind"] == "fmp":  # MaxPoolingLayer.cu:211-217: float product, + 0.5 in double, truncated
+                t = int(np.float64(np.float32(s) * l["shrink"]) + 0.5)
+                s = t + 1 if t == s else t
             elif l["kind"] == "terminal":
                 assert s == 1
                 s = l["size"]
@@ -89,10 +105,11 @@ class Net:
                                None if prelu is None else np.asarray(prelu, np.float32))
 
     # ---- forward over one batch
-    def forward(self, batch, sample, key, row, bg, features, nSpatialSites, labels=None, keep=True):
+    def forward(self, batch, sample, key, row, bg, features, nSpatialSites, labels=None, keep=True, ticks=None):
         """Returns a list of interfaces (dicts with grids, rules, features,
         choices, nSpatialSites, nFeatures, spatialSize) and, when the net ends
-        in the classifier, probabilities / predictions / mistakes / nll."""
+        in the classifier, probabilities / predictions / mistakes / nll.
+        ticks: {layer index: (inputL, inputR)} for fractional max-pooling layers (the random draw is the caller's)."""
         d = self.dimension
         g = orc.Grids.from_flat(batch, sample, key, row, bg)
         feats = np.ascontiguousarray(features, np.float32)
@@ -115,6 +132,14 @@ class Net:
                     width = rules.size // max(n, 1)
                     nxt["features"], ch = orc.maxpool(cur["features"], rules, n, width, cur["nFeatures"])
                     nxt["choices"] = ch.reshape(-1)
+            elif k == "fmp":
+                inL, inR = ticks[i]
+                og, rules, n = orc.rules_fmp(cur["grids"], d, l["inSize"], l["outSize"], l["size"], inL, inR,
+                                             l["fmpKind"] in (0, 2))
+                nxt.update(grids=og, rules=rules, nSpatialSites=n, spatialSize=l["outSize"])
+                width = rules.size // max(n, 1)
+                nxt["features"], ch = orc.maxpool(cur["features"], rules, n, width, cur["nFeatures"])
+                nxt["choices"] = ch.reshape(-1)
             elif k in ("nin", "nin_prelu"):
                 W, B, pr = self.weights[i]
                 p = np.float32(1.0) - np.float32(l["dropout"])
@@ -179,7 +204,7 @@ class Net:
             elif k in ("conv", "conv_tri"):
                 cur["dfeatures"] = orc.gather_rows_backward(nxt["dfeatures"].reshape(-1, cur["nFeatures"]), nxt["rules"],
                                                             cur["nSpatialSites"], cur["nFeatures"])
-            elif k in ("maxpool", "maxpool_tri"):
+            elif k in ("maxpool", "maxpool_tri", "fmp"):
                 cur["dfeatures"] = orc.maxpool_backward(nxt["dfeatures"], nxt["choices"], cur["nSpatialSites"])
             elif k == "terminal":
                 S = nxt["rules"].size // max(nxt["nSpatialSites"], 1)

@@ -42,9 +42,8 @@ class SparseConvNetCUDA;
 
 // Builder and processing calls shared by the square-lattice and the
 // triangular-lattice facade (reference SparseConvNet.h:25-66 and :75-98):
-// same names, argument order and defaults.  Builders for fractional
-// max-pooling and the index-learner head are outside the forward path this
-// library covers and are not declared.
+// same names, argument order and defaults.  The index-learner head is not
+// part of this library and is not declared.
 #define SCN_FACADE_METHODS                                                     \
   void addLeNetLayerMP(int nFeatures, int filterSize, int filterStride,        \
                        int poolSize, int poolStride,                           \
@@ -65,6 +64,10 @@ class SparseConvNetCUDA;
                    int firstNlayers = 1000000);                                \
   void saveWeights(std::string baseName, int epoch, bool momentum = false);
 
+#define SCN_FMP_BUILDER(Name)                                                  \
+  void Name(int nFeatures, int filterSize, int filterStride, int poolSize,     \
+            float fmpShrink, ActivationFunction activationFn = RELU,           \
+            float dropout = 0.0f, int minActiveInputs = 1);
 class SparseConvNet {
 public:
   std::unique_ptr<SparseConvNetCUDA> cnn; // public in the reference too
@@ -72,7 +75,14 @@ public:
                 int pciBusID = -1, int nTop = 1);
   ~SparseConvNet();
   SCN_FACADE_METHODS
+  // convolution + NiN + fractional max-pooling: pseudorandom / random,
+  // overlapping / disjoint regions (SparseConvNet.h:32-47)
+  SCN_FMP_BUILDER(addLeNetLayerPOFMP)
+  SCN_FMP_BUILDER(addLeNetLayerROFMP)
+  SCN_FMP_BUILDER(addLeNetLayerPDFMP)
+  SCN_FMP_BUILDER(addLeNetLayerRDFMP)
 };
+#undef SCN_FMP_BUILDER
 
 class SparseConvTriangLeNet {
   std::unique_ptr<SparseConvNetCUDA> cnn;
@@ -109,3 +119,17 @@ SCN_ARCHITECTURE(DeepC2C2)
 SCN_ARCHITECTURE(DeepC3C3)
 SCN_ARCHITECTURE(DeepC3C3Valid)
 #undef SCN_ARCHITECTURE
+// NetworkArchitectures.h:43-69: l levels of C2 followed by fractional
+// max-pooling with ratio fmpShrink
+#define SCN_FMP_ARCHITECTURE(Name)                                             \
+  class Name : public SparseConvNet {                                         \
+  public:                                                                      \
+    Name(int dimension, int l, int k, float fmpShrink, ActivationFunction fn,  \
+         int nInputFeatures, int nClasses, float p = 0.0f,                     \
+         int cudaDevice = -1, int nTop = 1);                                   \
+  };
+SCN_FMP_ARCHITECTURE(POFMPSparseConvNet)
+SCN_FMP_ARCHITECTURE(ROFMPSparseConvNet)
+SCN_FMP_ARCHITECTURE(PDFMPSparseConvNet)
+SCN_FMP_ARCHITECTURE(RDFMPSparseConvNet)
+#undef SCN_FMP_ARCHITECTURE

@@ -77,6 +77,11 @@ public:
                        int poolSize, int poolStride,
                        ActivationFunction activationFn = RELU,
                        float dropout = 0.0f, int minActiveInputs = 1);
+  // kind: 0 POFMP, 1 PDFMP, 2 ROFMP, 3 RDFMP (SparseConvNetCUDA.cu:112-163)
+  void addLeNetLayerFMP(int kind, int nFeatures, int filterSize,
+                        int filterStride, int poolSize, float fmpShrink,
+                        ActivationFunction activationFn = RELU,
+                        float dropout = 0.0f, int minActiveInputs = 1);
   void addTriangularConvolutionalLayer(int nFeatures, int filterSize,
                                        int filterStride,
                                        ActivationFunction activationFn = RELU,

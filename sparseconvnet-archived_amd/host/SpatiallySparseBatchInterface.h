@@ -30,6 +30,9 @@ public:
   scn_grids *deviceGrids;
   bool ownsDeviceGrids;
   vectorCUDA<int> rules;
+  // Output of a fractional max-pooling layer: the regions drawn for this
+  // batch, inputL then inputR, each [batchSize][dimension][spatialSize].
+  std::vector<int> regionTicks;
   // Set by a convolutional layer that left its gather to the following NiN
   // layer (fused kernel): the interface whose features the rules index.  The
   // feature matrix of THIS interface is then not materialised.

@@ -10,6 +10,7 @@
 #pragma once
 #include <fstream>
 #include <iostream>
+#include <mutex>
 #include "Rng.h"
 #include "SpatiallySparseBatch.h"
 #include "SpatiallySparseBatchInterface.h"
@@ -219,6 +220,64 @@ public:
                  float momentum);
   int calculateInputSpatialSize(int outputSpatialSize);
 };
+
+// MaxPoolingLayer.h:34-143 -- the four fractional max-pooling layers.  Every
+// sample of a batch gets freshly drawn pooling regions along every axis
+// (MaxPoolingLayer.cu:181-186); the draw is host work, the rule book is built
+// on the GPU from the region tables.
+enum FmpKind {
+  FMP_PSEUDORANDOM_OVERLAPPING,
+  FMP_PSEUDORANDOM_NONOVERLAPPING,
+  FMP_RANDOM_OVERLAPPING,
+  FMP_RANDOM_NONOVERLAPPING
+};
+// inputL / inputR of one axis as the reference's tick classes compute them
+// (Regions.cu:31-134); stops the program where the reference asserts
+void fmpTicks(FmpKind kind, int nIn, int nOut, int poolSize, RNG &rng,
+              int *inputL, int *inputR);
+class FractionalMaxPoolingLayer : public SpatiallySparseLayer {
+  int sd;
+  FmpKind kind;
+  std::mutex rngMutex; // preprocess() runs on several producer threads
+
+public:
+  int inSpatialSize;
+  int outSpatialSize;
+  float fmpShrink;
+  int poolSize;
+  int dimension;
+  RNG rng;
+  FractionalMaxPoolingLayer(cudaMemStream &memStream, FmpKind kind,
+                            int poolSize, float fmpShrink, int dimension);
+  void preprocess(SpatiallySparseBatch &batch,
+                  SpatiallySparseBatchInterface &input,
+                  SpatiallySparseBatchInterface &output);
+  void forwards(SpatiallySparseBatch &batch,
+                SpatiallySparseBatchInterface &input,
+                SpatiallySparseBatchInterface &output);
+  void backwards(SpatiallySparseBatch &batch,
+                 SpatiallySparseBatchInterface &input,
+                 SpatiallySparseBatchInterface &output, float learningRate,
+                 float momentum);
+  int calculateInputSpatialSize(int outputSpatialSize);
+};
+#define SCN_FMP_LAYER(Name, Kind)                                              \
+  class Name : public FractionalMaxPoolingLayer {                             \
+  public:                                                                      \
+    Name(cudaMemStream &memStream, int poolSize, float fmpShrink,              \
+         int dimension)                                                        \
+        : FractionalMaxPoolingLayer(memStream, Kind, poolSize, fmpShrink,      \
+                                    dimension) {}                              \
+  };
+SCN_FMP_LAYER(PseudorandomOverlappingFractionalMaxPoolingLayer,
+              FMP_PSEUDORANDOM_OVERLAPPING)
+SCN_FMP_LAYER(PseudorandomNonOverlappingFractionalMaxPoolingLayer,
+              FMP_PSEUDORANDOM_NONOVERLAPPING)
+SCN_FMP_LAYER(RandomOverlappingFractionalMaxPoolingLayer,
+              FMP_RANDOM_OVERLAPPING)
+SCN_FMP_LAYER(RandomNonOverlappingFractionalMaxPoolingLayer,
+              FMP_RANDOM_NONOVERLAPPING)
+#undef SCN_FMP_LAYER
 
 // TerminalPoolingLayer.h:5-25 -- averages every active site of a sample.
 class TerminalPoolingLayer : public SpatiallySparseLayer {

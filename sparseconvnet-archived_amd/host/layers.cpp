@@ -605,6 +605,144 @@ int MaxPoolingTriangularLayer::calculateInputSpatialSize(
   return inSpatialSize;
 }
 
+// ---- fractional max-pooling (Regions.cu:31-134, MaxPoolingLayer.cu:157-420) ----
+static void fmp_stop(const char *what, int nIn, int nOut, int poolSize) {
+  std::fprintf(stderr,
+               "fractional max-pooling regions: %s (nIn %d, nOut %d, "
+               "poolSize %d)\n",
+               what, nIn, nOut, poolSize);
+  std::exit(EXIT_FAILURE);
+}
+void fmpTicks(FmpKind kind, int nIn, int nOut, int poolSize, RNG &rng,
+              int *inputL, int *inputR) {
+  switch (kind) {
+  case FMP_PSEUDORANDOM_OVERLAPPING: { // Regions.cu:31-46
+    if (nIn < nOut - 1 + poolSize)
+      fmp_stop("nIn < nOut - 1 + poolSize", nIn, nOut, poolSize);
+    double alpha = (nIn - poolSize) * 1.0 / (nOut - 1);
+    double u = rng.uniform(0, 1);
+    for (int j = 0; j < nOut; ++j) {
+      int i = (int)((j + u) * alpha) - (int)(u * alpha);
+      inputL[j] = i;
+      inputR[j] = i + poolSize;
+    }
+    break;
+  }
+  case FMP_PSEUDORANDOM_NONOVERLAPPING: { // Regions.cu:59-71
+    double alpha = nIn * 1.0 / nOut;
+    double u = rng.uniform(0, 1);
+    if (nIn < nOut - 1 + poolSize || (int)std::ceil(alpha) != poolSize)
+      fmp_stop("ceil(nIn / nOut) != poolSize", nIn, nOut, poolSize);
+    for (int j = 0; j < nOut; ++j)
+      inputL[j] = (int)((j + u) * alpha) - (int)(u * alpha);
+    for (int j = 1; j <= nOut; ++j)
+      inputR[j - 1] = (int)((j + u) * alpha) - (int)(u * alpha);
+    break;
+  }
+  case FMP_RANDOM_OVERLAPPING: { // Regions.cu:83-98
+    if (nIn <= nOut)
+      fmp_stop("nIn <= nOut", nIn, nOut, poolSize);
+    int alpha = nIn * 1.0 / nOut;
+    std::vector<int> inc;
+    inc.resize(nOut * (alpha + 1) - nIn, alpha);
+    inc.resize(nOut - 1, alpha + 1);
+    rng.vectorShuffle(inc);
+    inputL[0] = 0;
+    inputR[0] = poolSize;
+    for (int i = 0; i < nOut - 1; i++) {
+      inputL[i + 1] = inputL[i] + inc[i];
+      inputR[i + 1] = inputL[i + 1] + poolSize;
+    }
+    break;
+  }
+  case FMP_RANDOM_NONOVERLAPPING: { // Regions.cu:109-124
+    if (nIn <= nOut)
+      fmp_stop("nIn <= nOut", nIn, nOut, poolSize);
+    int alpha = nIn * 1.0 / nOut;
+    std::vector<int> inc;
+    inc.resize(nOut * (alpha + 1) - nIn, alpha);
+    inc.resize(nOut, alpha + 1);
+    rng.vectorShuffle(inc);
+    inputL[0] = 0;
+    inputR[0] = inc[0];
+    for (int i = 0; i < nOut - 1; i++) {
+      inputL[i + 1] = inputL[i] + inc[i];
+      inputR[i + 1] = inputR[i] + inc[i + 1];
+    }
+    break;
+  }
+  }
+  if (inputR[nOut - 1] != nIn) // Regions.cu:47,72,99,125
+    fmp_stop("the last region does not end at nIn", nIn, nOut, poolSize);
+}
+static const char *fmpNames[] = {"Pseudorandom overlapping",
+                                 "Pseudorandom non-overlapping",
+                                 "Random overlapping",
+                                 "Random non-overlapping"};
+static const char *fmpTags[] = {"POFMP", "PDFMP", "ROFMP", "RDFMP"};
+FractionalMaxPoolingLayer::FractionalMaxPoolingLayer(cudaMemStream &memStream,
+                                                     FmpKind kind,
+                                                     int poolSize,
+                                                     float fmpShrink,
+                                                     int dimension)
+    : SpatiallySparseLayer(memStream), kind(kind), inSpatialSize(0),
+      outSpatialSize(0), fmpShrink(fmpShrink), poolSize(poolSize),
+      dimension(dimension) {
+  sd = ipow(poolSize, dimension);
+  std::cout << fmpNames[kind] << " Fractional Max Pooling " << fmpShrink << " "
+            << poolSize << std::endl;
+}
+void FractionalMaxPoolingLayer::preprocess(
+    SpatiallySparseBatch &batch, SpatiallySparseBatchInterface &input,
+    SpatiallySparseBatchInterface &output) {
+  scn_ctx *ctx = pre_ctx(batch, memStream);
+  assert(input.spatialSize == inSpatialSize);
+  output.nFeatures = input.nFeatures;
+  output.featuresPresent.hVector() = input.featuresPresent.hVector();
+  output.spatialSize = outSpatialSize;
+  output.backpropErrors = input.backpropErrors;
+  // new regions for every sample, axis 0 first (Regions.cu:126-127)
+  const size_t per = (size_t)batch.batchSize * dimension * outSpatialSize;
+  std::vector<int> &t = output.regionTicks;
+  t.assign(2 * per, 0);
+  {
+    std::lock_guard<std::mutex> lock(rngMutex);
+    for (int item = 0; item < batch.batchSize; item++)
+      for (int a = 0; a < dimension; ++a) {
+        const size_t o = ((size_t)item * dimension + a) * outSpatialSize;
+        fmpTicks(kind, inSpatialSize, outSpatialSize, poolSize, rng, &t[o],
+                 &t[per + o]);
+      }
+  }
+  int64_t n = 0;
+  SCN_CHECKED(scn_rules_fmp_plan(ctx, input.deviceGrids, own_grids(ctx, output),
+                                 inSpatialSize, outSpatialSize, poolSize,
+                                 t.data(), t.data() + per, &n));
+  output.nSpatialSites = (int)n;
+  fill_rules(ctx, input, output, n * sd);
+}
+void FractionalMaxPoolingLayer::forwards(SpatiallySparseBatch &batch,
+                                         SpatiallySparseBatchInterface &input,
+                                         SpatiallySparseBatchInterface &output) {
+  (void)batch;
+  pool_forwards(memStream, input, output, sd);
+}
+void FractionalMaxPoolingLayer::backwards(
+    SpatiallySparseBatch &batch, SpatiallySparseBatchInterface &input,
+    SpatiallySparseBatchInterface &output, float learningRate, float momentum) {
+  (void)batch, (void)learningRate, (void)momentum;
+  pool_backwards(memStream, input, output);
+}
+int FractionalMaxPoolingLayer::calculateInputSpatialSize(
+    int outputSpatialSize) {
+  outSpatialSize = outputSpatialSize;
+  inSpatialSize = outputSpatialSize * fmpShrink + 0.5; // MaxPoolingLayer.cu:213
+  if (inSpatialSize == outputSpatialSize)
+    inSpatialSize++;
+  std::cout << "-(" << fmpTags[kind] << ")-" << inSpatialSize;
+  return inSpatialSize;
+}
+
 // ---- TerminalPoolingLayer (TerminalPoolingLayer.cu:75-130) --------------------
 TerminalPoolingLayer::TerminalPoolingLayer(cudaMemStream &memStream,
                                            int poolSize, int S)

@@ -89,6 +89,20 @@ void SparseConvNetCUDA::addConvolutionalLayer(int nFeatures, int filterSize,
   addLearntLayer(nFeatures, activationFn, dropout,
                  powf(filterSize * 1.0 / filterStride / poolingToFollow, 2));
 }
+// addLeNetLayerPOFMP / PDFMP / ROFMP / RDFMP (SparseConvNetCUDA.cu:112-163)
+void SparseConvNetCUDA::addLeNetLayerFMP(int kind, int nFeatures,
+                                         int filterSize, int filterStride,
+                                         int poolSize, float fmpShrink,
+                                         ActivationFunction activationFn,
+                                         float dropout, int minActiveInputs) {
+  addConvolutionalLayer(nFeatures, filterSize, filterStride, activationFn,
+                        dropout, minActiveInputs, fmpShrink);
+  if (fmpShrink > 1) {
+    std::cout << layers.size() << ":";
+    layers.push_back(new FractionalMaxPoolingLayer(
+        memStream, (FmpKind)kind, poolSize, fmpShrink, dimension));
+  }
+}
 void SparseConvNetCUDA::addLeNetLayerMP(int nFeatures, int filterSize,
                                         int filterStride, int poolSize,
                                         int poolStride,
@@ -726,6 +740,38 @@ void SparseConvNet::addLeNetLayerMP(int nFeatures, int filterSize,
   cnn->addLeNetLayerMP(nFeatures, filterSize, filterStride, poolSize,
                        poolStride, activationFn, dropout, minActiveInputs);
 }
+void SparseConvNet::addLeNetLayerPOFMP(int nFeatures, int filterSize,
+                                       int filterStride, int poolSize,
+                                       float fmpShrink,
+                                       ActivationFunction activationFn,
+                                       float dropout, int minActiveInputs) {
+  cnn->addLeNetLayerFMP(FMP_PSEUDORANDOM_OVERLAPPING, nFeatures, filterSize, filterStride, poolSize,
+                        fmpShrink, activationFn, dropout, minActiveInputs);
+}
+void SparseConvNet::addLeNetLayerROFMP(int nFeatures, int filterSize,
+                                       int filterStride, int poolSize,
+                                       float fmpShrink,
+                                       ActivationFunction activationFn,
+                                       float dropout, int minActiveInputs) {
+  cnn->addLeNetLayerFMP(FMP_RANDOM_OVERLAPPING, nFeatures, filterSize, filterStride, poolSize,
+                        fmpShrink, activationFn, dropout, minActiveInputs);
+}
+void SparseConvNet::addLeNetLayerPDFMP(int nFeatures, int filterSize,
+                                       int filterStride, int poolSize,
+                                       float fmpShrink,
+                                       ActivationFunction activationFn,
+                                       float dropout, int minActiveInputs) {
+  cnn->addLeNetLayerFMP(FMP_PSEUDORANDOM_NONOVERLAPPING, nFeatures, filterSize, filterStride, poolSize,
+                        fmpShrink, activationFn, dropout, minActiveInputs);
+}
+void SparseConvNet::addLeNetLayerRDFMP(int nFeatures, int filterSize,
+                                       int filterStride, int poolSize,
+                                       float fmpShrink,
+                                       ActivationFunction activationFn,
+                                       float dropout, int minActiveInputs) {
+  cnn->addLeNetLayerFMP(FMP_RANDOM_NONOVERLAPPING, nFeatures, filterSize, filterStride, poolSize,
+                        fmpShrink, activationFn, dropout, minActiveInputs);
+}
 void SparseConvNet::addTerminalPoolingLayer(int poolSize) {
   cnn->addTerminalPoolingLayer(poolSize, ipow(poolSize, cnn->dimension));
 }
@@ -875,3 +921,22 @@ DeepC3C3Valid::DeepC3C3Valid(int dimension, int l, int k,
   addLeNetLayerMP((l + 1) * k, 1, 1, 1, 1, fn, p);
   addSoftmaxLayer();
 }
+
+// NetworkArchitectures.cpp:72-122: l levels of C2 + fractional max-pooling,
+// then C2 and a 1x1 NiN, dropout rising to p
+#define SCN_FMP_ARCHITECTURE(Name, Builder)                                    \
+  Name::Name(int dimension, int l, int k, float fmpShrink,                     \
+             ActivationFunction fn, int nInputFeatures, int nClasses, float p, \
+             int cudaDevice, int nTop)                                         \
+      : SparseConvNet(dimension, nInputFeatures, nClasses, cudaDevice, nTop) { \
+    for (int i = 0; i < l; i++)                                                \
+      Builder(k * (i + 1), 2, 1, 2, fmpShrink, fn, p * i / (l + 1));           \
+    addLeNetLayerMP(k * (l + 1), 2, 1, 1, 1, fn, p * l / (l + 1));             \
+    addLeNetLayerMP(k * (l + 2), 1, 1, 1, 1, fn, p);                           \
+    addSoftmaxLayer();                                                         \
+  }
+SCN_FMP_ARCHITECTURE(POFMPSparseConvNet, addLeNetLayerPOFMP)
+SCN_FMP_ARCHITECTURE(ROFMPSparseConvNet, addLeNetLayerROFMP)
+SCN_FMP_ARCHITECTURE(PDFMPSparseConvNet, addLeNetLayerPDFMP)
+SCN_FMP_ARCHITECTURE(RDFMPSparseConvNet, addLeNetLayerRDFMP)
+#undef SCN_FMP_ARCHITECTURE

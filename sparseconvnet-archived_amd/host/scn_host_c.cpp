@@ -75,6 +75,18 @@ void scnh_add_lenet_layer_mp(scnh_net *net, int nFeatures, int filterSize,
                                  poolStride, (ActivationFunction)activationFn,
                                  dropout, minActiveInputs);
 }
+int scnh_add_lenet_layer_fmp(scnh_net *net, int kind, int nFeatures,
+                             int filterSize, int filterStride, int poolSize,
+                             float fmpShrink, int activationFn, float dropout,
+                             int minActiveInputs) {
+  if (!net->square || kind < 0 || kind > 3)
+    return -1; // the triangular facade has no such builder
+  net->cnn->addLeNetLayerFMP(kind, nFeatures, filterSize, filterStride,
+                             poolSize, fmpShrink,
+                             (ActivationFunction)activationFn, dropout,
+                             minActiveInputs);
+  return 0;
+}
 void scnh_add_terminal_pooling_layer(scnh_net *net, int poolSize) {
   if (net->triangular)
     net->triangular->addTerminalPoolingLayer(poolSize);
@@ -123,6 +135,8 @@ int scnh_layer_info(scnh_net *net, int layer, int *nIn, int *nOut, int *act) {
     kind = 5;
   } else if (dynamic_cast<TerminalPoolingLayer *>(l)) {
     kind = 6;
+  } else if (dynamic_cast<FractionalMaxPoolingLayer *>(l)) {
+    kind = 7;
   }
   if (nIn)
     *nIn = i;
@@ -448,6 +462,13 @@ void scnh_iface_dfeatures(scnh_net *net, int i, float *out) {
 }
 int64_t scnh_iface_dfeatures_size(scnh_net *net, int i) {
   return (int64_t)net->batch->interfaces.at(i).sub->dfeatures.size64();
+}
+int64_t scnh_iface_region_ticks_size(scnh_net *net, int i) {
+  return (int64_t)net->batch->interfaces.at(i).regionTicks.size();
+}
+void scnh_iface_region_ticks(scnh_net *net, int i, int32_t *out) {
+  std::vector<int> &t = net->batch->interfaces.at(i).regionTicks;
+  std::copy(t.begin(), t.end(), out);
 }
 void scnh_iface_choices(scnh_net *net, int i, int32_t *out) {
   SpatiallySparseBatchInterface &f = net->batch->interfaces.at(i);

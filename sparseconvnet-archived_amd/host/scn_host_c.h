@@ -20,6 +20,12 @@ void scnh_add_lenet_layer_mp(scnh_net *net, int nFeatures, int filterSize,
                              int filterStride, int poolSize, int poolStride,
                              int activationFn, float dropout,
                              int minActiveInputs);
+/* addLeNetLayerPOFMP / PDFMP / ROFMP / RDFMP (kind 0..3) of the square
+ * facade: convolution, NiN, fractional max-pooling; -1 on a triangular net */
+int scnh_add_lenet_layer_fmp(scnh_net *net, int kind, int nFeatures,
+                             int filterSize, int filterStride, int poolSize,
+                             float fmpShrink, int activationFn, float dropout,
+                             int minActiveInputs);
 void scnh_add_terminal_pooling_layer(scnh_net *net, int poolSize);
 void scnh_add_softmax_layer(scnh_net *net);
 /* A stack without a classifier: fixes the spatial sizes from the size of the
@@ -148,6 +154,11 @@ void scnh_iface_features(scnh_net *net, int i, float *out);
 /* gradient of the cost with respect to that feature matrix after a TRAINBATCH
  * (SpatiallySparseBatchSubInterface::dfeatures); size in floats, 0 when the
  * backward pass did not reach the interface */
+/* the pooling regions a fractional max-pooling layer drew for the batch:
+ * inputL then inputR, each [batchSize][dimension][spatialSize of the
+ * interface]; size 0 for the output of any other layer */
+int64_t scnh_iface_region_ticks_size(scnh_net *net, int i);
+void scnh_iface_region_ticks(scnh_net *net, int i, int32_t *out);
 int64_t scnh_iface_dfeatures_size(scnh_net *net, int i);
 void scnh_iface_dfeatures(scnh_net *net, int i, float *out);
 void scnh_iface_choices(scnh_net *net, int i, int32_t *out);

@@ -11,7 +11,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libscn_host.so")
 
 TRAINBATCH, TESTBATCH, UNLABELEDBATCH, RESCALEBATCH = range(4)
-LAYER_KINDS = ["conv", "conv_tri", "nin", "nin_prelu", "maxpool", "maxpool_tri", "terminal"]
+LAYER_KINDS = ["conv", "conv_tri", "nin", "nin_prelu", "maxpool", "maxpool_tri", "terminal", "fmp"]
+POFMP, PDFMP, ROFMP, RDFMP = range(4)  # pseudorandom / random, overlapping / disjoint fractional max-pooling
 
 
 def build(force=True):
@@ -62,6 +63,9 @@ def lib():
         "scnh_dataset_add_cifar10_file": (i64, [vp, C.c_char_p]),
         "scnh_codify_picture": (i64, [vp, i64, i32, i64, i64, vp, vp, vp, vp]),
         "scnh_process_dataset": (f32, [vp, vp, i32]),
+        "scnh_add_lenet_layer_fmp": (i32, [vp, i32, i32, i32, i32, i32, f32, i32, f32, i32]),
+        "scnh_iface_region_ticks_size": (i64, [vp, i32]),
+        "scnh_iface_region_ticks": (None, [vp, i32, vp]),
         "scnh_process_dataset_train": (f32, [vp, vp, i32, f32, f32]),
         "scnh_set_training": (None, [vp, f32, f32, i32]),
         "scnh_get_weights": (i32, [vp, i32, i32, vp, vp, vp]),
@@ -214,6 +218,13 @@ class Net:
         lib().scnh_add_lenet_layer_mp(self.h, nFeatures, filterSize, filterStride, poolSize, poolStride, activationFn,
                                       dropout, minActiveInputs)
 
+    def addLeNetLayerFMP(self, kind, nFeatures, filterSize, filterStride, poolSize, fmpShrink, activationFn=1,
+                         dropout=0.0, minActiveInputs=1):
+        """addLeNetLayerPOFMP / PDFMP / ROFMP / RDFMP of the reference (kind = POFMP ...)"""
+        rc = lib().scnh_add_lenet_layer_fmp(self.h, kind, nFeatures, filterSize, filterStride, poolSize, fmpShrink,
+                                            activationFn, dropout, minActiveInputs)
+        assert rc == 0, "fractional max-pooling builders exist on the square-lattice net only"
+
     def addTerminalPoolingLayer(self, poolSize):
         lib().scnh_add_terminal_pooling_layer(self.h, poolSize)
 
@@ -264,6 +275,18 @@ class Net:
 
     def processDatasetTrain(self, ds, batchSize=100, learningRate=0.0, momentum=0.99):
         return lib().scnh_process_dataset_train(self.h, ds.h, batchSize, learningRate, momentum)
+
+    def region_ticks(self, i):
+        """(inputL, inputR), each [batch, dimension, spatialSize of interface i]: the regions a fractional
+        max-pooling layer drew for the current batch; None for any other interface"""
+        n = lib().scnh_iface_region_ticks_size(self.h, i)
+        if n == 0:
+            return None
+        t = np.empty(n, np.int32)
+        lib().scnh_iface_region_ticks(self.h, i, _p(t))
+        b = lib().scnh_batch_size(self.h)
+        t = t.reshape(2, b, self.dimension, -1)
+        return t[0].copy(), t[1].copy()
 
     def dfeatures(self, i):
         """gradient left in interface i by the last TRAINBATCH, flat; empty if the backward pass stopped above it"""

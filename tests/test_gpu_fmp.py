@@ -102,3 +102,111 @@ def test_fmp_bad_tables_are_refused(scn, ctx):
             scn.rules_fmp(ctx, g, 6, 4, 2, bad, bad + 2)
     with pytest.raises(scn.ScnError):  # wider than the pool size
         scn.rules_fmp(ctx, g, 6, 4, 2, L, L + 3)
+
+
+# ---- whole nets with fractional max-pooling layers through the C++ host classes
+def rel_l2(a, b):
+    a, b = a.astype(np.float64).ravel(), b.astype(np.float64).ravel()
+    return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30))
+
+
+@pytest.mark.parametrize("kind", [0, 1, 2, 3])
+@pytest.mark.parametrize("train", [False, True])
+def test_net_with_fractional_max_pooling(scn, kind, train):
+    """addLeNetLayerPOFMP / PDFMP / ROFMP / RDFMP: the regions the layers drew are read back and handed to the oracle;
+    rule books and grids bit-exact, features to 1e-4, and (train) one training step through the pooling choices."""
+    import oracle_net
+    from sparseconvnet_archived_amd import hostapi, synthetic
+    d, nIn, nClasses, batch = 2, 3, 10, 6
+    shrink = 1.5
+    net = hostapi.Net(d, nIn, nClasses, nTop=1, threads=2)
+    ora = oracle_net.Net(d, nIn, nClasses, nTop=1)
+    for n_ in (net, ora):
+        n_.addLeNetLayerFMP(kind, 32, 2, 1, 2, shrink, synthetic.VLEAKYRELU)
+        n_.addLeNetLayerFMP(kind, 64, 2, 1, 2, shrink, synthetic.VLEAKYRELU)
+        n_.addLeNetLayerMP(64, 2, 1, 1, 1, synthetic.VLEAKYRELU)
+        n_.addTerminalPoolingLayer(2)
+        n_.addSoftmaxLayer()
+    assert net.layers() == ora.layer_list()
+    assert net.inputSpatialSize == ora.inputSpatialSize
+    lattice = net.inputSpatialSize
+    for i, (W, B, pr) in synthetic.he_normal_weights(net.layers(), 5).items():
+        net.set_weights(i, W, B, pr)
+        ora.set_weights(i, W, B, pr)
+    rng = np.random.default_rng(40 + kind)
+    samples = []
+    for _ in range(batch):
+        pts = np.array([(a, b) for a in range(lattice) for b in range(lattice) if rng.random() < 0.3], np.int32)
+        samples.append((pts, rng.uniform(-1, 1, (len(pts), nIn)).astype(np.float32), int(rng.integers(0, nClasses))))
+    ds = hostapi.Dataset("fmp", nIn, nClasses, hostapi.TRAINBATCH if train else hostapi.TESTBATCH)
+    for pts, f, label in samples:
+        ds.add_points(d, lattice, pts, f, label)
+    net.set_training(0.01, 0.9, shuffle=False)
+    net.begin(ds, batch)
+    assert net.next_batch()
+    layers = net.layers()
+    ticks = {i: net.region_ticks(i + 1) for i, l in enumerate(layers) if l["kind"] == "fmp"}
+    assert len(ticks) == 2 and all(t is not None for t in ticks.values())
+    S, K, R, bg, feats, n = synthetic.codify(samples, d, lattice, lattice, nIn)
+    labels = np.array([s[2] for s in samples], np.int32)
+    want = ora.forward(batch, S, K, R, bg, feats, n, labels, ticks=ticks)
+    for i, wi in enumerate(want["interfaces"]):
+        gi = net.interface(i)
+        assert gi["nSpatialSites"] == wi["nSpatialSites"] and gi["spatialSize"] == wi["spatialSize"]
+        assert np.array_equal(gi["rules"], wi["rules"])
+        s_, k_, r_, b_ = gi["grids"]
+        os_, ok, or_, ob = wi["grids"].flat()
+        assert np.array_equal(s_, os_) and np.array_equal(k_, ok) and np.array_equal(r_, or_) and np.array_equal(b_, ob)
+        assert rel_l2(gi["features"], wi["features"]) <= 1e-4
+        if i > 0 and layers[i - 1]["kind"] == "fmp":
+            assert np.array_equal(gi["choices"], wi["choices"])
+    out = net.batch_outputs()
+    assert np.allclose(out["probabilities"], want["probabilities"], rtol=1e-3, atol=1e-6)
+    if train:
+        ora.train_step(want, labels, 0.01, 0.9)
+        for i, wi in enumerate(want["interfaces"]):
+            if "dfeatures" in wi:
+                assert rel_l2(net.dfeatures(i), wi["dfeatures"]) <= 1e-4
+        for i, l in enumerate(layers):
+            if l["kind"].startswith("nin"):
+                MW, MB, _ = net.get_weights(i, momentum=True)
+                assert rel_l2(MW, ora.momentum[i][0]) <= 1e-4 and rel_l2(MB, ora.momentum[i][1]) <= 1e-4
+    net.end()
+    net.close()
+
+
+def test_host_ticks_satisfy_the_invariants_and_vary(scn):
+    """The regions drawn by the host library: partition / coverage invariants per kind, new for every sample."""
+    from sparseconvnet_archived_amd import hostapi, synthetic
+    for kind in range(4):
+        net = hostapi.Net(2, 1, 4, nTop=1, threads=1)
+        net.addLeNetLayerFMP(kind, 32, 2, 1, 2, 1.414, synthetic.RELU)
+        net.addLeNetLayerFMP(kind, 32, 2, 1, 2, 1.414, synthetic.RELU)
+        net.addLeNetLayerFMP(kind, 32, 2, 1, 2, 1.414, synthetic.RELU)
+        net.addLeNetLayerMP(32, 2, 1, 1, 1, synthetic.RELU)
+        net.addTerminalPoolingLayer(2)
+        net.addSoftmaxLayer()
+        lattice = net.inputSpatialSize
+        ds = hostapi.Dataset("t", 1, 4, hostapi.TESTBATCH)
+        for b in range(8):
+            ds.add_points(2, lattice, np.array([[b, b], [b + 1, b]], np.int32), np.ones((2, 1), np.float32), 0)
+        net.begin(ds, 8)
+        assert net.next_batch()
+        seen = set()
+        for i, l in enumerate(net.layers()):
+            if l["kind"] != "fmp":
+                continue
+            L, R = net.region_ticks(i + 1)
+            nInAxis = net.interface(i)["spatialSize"]
+            for b in range(8):
+                for a in range(2):
+                    l_, r_ = L[b, a], R[b, a]
+                    assert l_[0] == 0 and r_[-1] == nInAxis and np.all(np.diff(l_) >= 1)
+                    if kind in (0, 2):
+                        assert np.all(r_ - l_ == 2)
+                    else:
+                        assert np.array_equal(r_[:-1], l_[1:])
+                    seen.add((i, tuple(l_)))
+        assert len(seen) > 8  # not one draw repeated everywhere
+        net.end()
+        net.close()
