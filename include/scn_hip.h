@@ -278,6 +278,21 @@ int scn_sgemm_ABt(scn_ctx *ctx, const float *d_D, const float *d_W,
 int scn_nag_update(scn_ctx *ctx, const float *d_delta, float *d_momentum,
                    float *d_weights, int64_t n, float learningRate,
                    float momentum, int keepPositive);
+/* Dropout during training.  dShrinkMatrixForDropout / dShrinkVectorForDropout
+ * (NetworkInNetworkLayer.cu:7-25): w[i][j] = W[inPresent[i]][outPresent[j]],
+ * W with rows of nOut floats; a null d_inPresent keeps the rows (row i of w
+ * is row i of W), so a vector is a matrix of one row.  dGradientDescentShrunkMatrix / ...ShrunkVector
+ * (NetworkInNetworkLayer.cu:43-82): the momentum step of scn_nag_update on
+ * exactly those entries, delta being the gradient of the shrunk matrix. */
+int scn_shrink_matrix(scn_ctx *ctx, const float *d_W, float *d_w,
+                      const int32_t *d_inPresent, const int32_t *d_outPresent,
+                      int nOut, int nInPresent, int nOutPresent);
+int scn_nag_update_shrunk(scn_ctx *ctx, const float *d_delta,
+                          float *d_momentum, float *d_weights,
+                          const int32_t *d_inPresent,
+                          const int32_t *d_outPresent, int nOut,
+                          int nInPresent, int nOutPresent, float learningRate,
+                          float momentum);
 /* propBackwardFromMatrixMultiply (ConvolutionalLayer.cu:42-72):
  * din[rules[c] * nIn + j] += dconv[c * nIn + j], c < count; the caller zeroes
  * din first (ConvolutionalLayer.cu:141).  Negative rules are skipped. */

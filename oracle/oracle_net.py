@@ -105,50 +105,68 @@ class Net:
                                None if prelu is None else np.asarray(prelu, np.float32))
 
     # ---- forward over one batch
-    def forward(self, batch, sample, key, row, bg, features, nSpatialSites, labels=None, keep=True, ticks=None):
+    def forward(self, batch, sample, key, row, bg, features, nSpatialSites, labels=None, keep=True, ticks=None,
+                present=None):
         """Returns a list of interfaces (dicts with grids, rules, features,
         choices, nSpatialSites, nFeatures, spatialSize) and, when the net ends
         in the classifier, probabilities / predictions / mistakes / nll.
-        ticks: {layer index: (inputL, inputR)} for fractional max-pooling layers (the random draw is the caller's)."""
+        ticks: {layer index: (inputL, inputR)} for fractional max-pooling layers (the random draw is the caller's).
+        present: a TRAINBATCH with dropout -- {NiN layer index: the output features kept} (again the caller's draw);
+        feature matrices then hold the kept columns only (featuresPresent of the reference)."""
         d = self.dimension
         g = orc.Grids.from_flat(batch, sample, key, row, bg)
         feats = np.ascontiguousarray(features, np.float32)
         ifaces = [dict(grids=g, rules=np.zeros(0, np.int32), features=feats, choices=np.zeros(0, np.int32),
-                       nSpatialSites=nSpatialSites, nFeatures=self.nInputFeatures, spatialSize=self.inputSpatialSize)]
+                       nSpatialSites=nSpatialSites, nFeatures=self.nInputFeatures, spatialSize=self.inputSpatialSize,
+                       present=np.arange(self.nInputFeatures))]
         for i, l in enumerate(self.layers):
             k = l["kind"]
             cur = ifaces[-1]
             nxt = dict(grids=cur["grids"], rules=np.zeros(0, np.int32), choices=np.zeros(0, np.int32),
-                       nFeatures=cur["nFeatures"], spatialSize=cur["spatialSize"], nSpatialSites=cur["nSpatialSites"])
+                       nFeatures=cur["nFeatures"], spatialSize=cur["spatialSize"], nSpatialSites=cur["nSpatialSites"],
+                       present=cur["present"])
+            width = len(cur["present"])  # columns of the input's feature matrix
             if k in ("conv", "conv_tri", "maxpool", "maxpool_tri"):
                 fn = orc.rules_triangular if k.endswith("_tri") else orc.rules_square
                 minActive = l.get("minActive", 1)
                 og, rules, n = fn(cur["grids"], d, l["inSize"], l["outSize"], l["size"], l["stride"], minActive)
                 nxt.update(grids=og, rules=rules, nSpatialSites=n, spatialSize=l["outSize"])
                 if k.startswith("conv"):
-                    nxt["features"] = orc.gather_rows(cur["features"], rules, cur["nFeatures"]).reshape(n, -1)
+                    nxt["features"] = orc.gather_rows(cur["features"], rules, width).reshape(n, -1)
                     nxt["nFeatures"] = cur["nFeatures"] * l["fs"]
+                    # convolutionFeaturesPresent, ConvolutionalLayer.cu:74-80
+                    nxt["present"] = np.concatenate([cur["present"] + cur["nFeatures"] * q for q in range(l["fs"])])
                 else:
-                    width = rules.size // max(n, 1)
-                    nxt["features"], ch = orc.maxpool(cur["features"], rules, n, width, cur["nFeatures"])
+                    ps = rules.size // max(n, 1)
+                    nxt["features"], ch = orc.maxpool(cur["features"], rules, n, ps, width)
                     nxt["choices"] = ch.reshape(-1)
             elif k == "fmp":
                 inL, inR = ticks[i]
                 og, rules, n = orc.rules_fmp(cur["grids"], d, l["inSize"], l["outSize"], l["size"], inL, inR,
                                              l["fmpKind"] in (0, 2))
                 nxt.update(grids=og, rules=rules, nSpatialSites=n, spatialSize=l["outSize"])
-                width = rules.size // max(n, 1)
-                nxt["features"], ch = orc.maxpool(cur["features"], rules, n, width, cur["nFeatures"])
+                ps = rules.size // max(n, 1)
+                nxt["features"], ch = orc.maxpool(cur["features"], rules, n, ps, width)
                 nxt["choices"] = ch.reshape(-1)
             elif k in ("nin", "nin_prelu"):
                 W, B, pr = self.weights[i]
-                p = np.float32(1.0) - np.float32(l["dropout"])
-                nxt["features"] = orc.nin_forward(cur["features"], W, B, pr, p, l["act"])
+                inP = cur["present"]
+                outP = np.asarray(present[i]) if present is not None and i in present else np.arange(l["nOut"])
+                nxt["present"] = outP
+                if present is not None and len(inP) + len(outP) < l["nIn"] + l["nOut"]:
+                    # the training branch, NetworkInNetworkLayer.cu:162-184: sub-matrix, no scaling
+                    assert pr is None or len(outP) == l["nOut"]
+                    w = np.ascontiguousarray(W[np.ix_(inP, outP)])
+                    nxt["features"] = orc.nin_forward(cur["features"], w, B[outP], pr, 1.0, l["act"])
+                    nxt["shrunk"] = (inP, outP, w)
+                else:
+                    p = np.float32(1.0) - np.float32(l["dropout"])
+                    nxt["features"] = orc.nin_forward(cur["features"], W, B, pr, p, l["act"])
                 nxt["nFeatures"] = l["nOut"]
             elif k == "terminal":
                 og, rules, S = orc.rules_terminal(cur["grids"])
                 nxt.update(grids=og, rules=rules, nSpatialSites=batch, spatialSize=1)
-                nxt["features"] = orc.terminal_pool(cur["features"], rules, batch, S, cur["nFeatures"])
+                nxt["features"] = orc.terminal_pool(cur["features"], rules, batch, S, width)
             if not keep:
                 cur.pop("features", None)
             ifaces.append(nxt)
@@ -180,7 +198,6 @@ class Net:
             l, cur, nxt = self.layers[i], ifaces[i], ifaces[i + 1]
             k = l["kind"]
             if k in ("nin", "nin_prelu"):
-                assert l["dropout"] == 0
                 W, B, pr = self.weights[i]
                 W, B = W.copy(), B.copy()
                 pr = None if pr is None else pr.copy()
@@ -188,22 +205,34 @@ class Net:
                                                    None if pr is None else np.zeros_like(pr)))
                 dZ, dB, dPr = orc.activation_backward(nxt["features"], nxt["dfeatures"], l["act"], pr)
                 nxt["dfeatures"] = dZ  # in place in the reference
-                Wold = W.copy()
                 if pr is not None:
                     orc.nag_update(dPr, MP, pr, learningRate, momentum, keepPositive=True)
                 dW = orc.sgemm_AtB(cur["features"], dZ)
-                if backprop[i]:
-                    cur["dfeatures"] = orc.sgemm_ABt(dZ, Wold)
-                orc.nag_update(dW, MW, W, learningRate, momentum)
-                orc.nag_update(dB, MB, B, learningRate, momentum)
+                if "shrunk" in nxt:  # NetworkInNetworkLayer.cu:235-263: only the entries the batch used move
+                    inP, outP, w = nxt["shrunk"]
+                    if backprop[i]:
+                        cur["dfeatures"] = orc.sgemm_ABt(dZ, w)
+                    ix = np.ix_(inP, outP)
+                    subW, subM = np.ascontiguousarray(W[ix]), np.ascontiguousarray(MW[ix])
+                    orc.nag_update(dW, subM, subW, learningRate, momentum)
+                    W[ix], MW[ix] = subW, subM
+                    subB, subMB = np.ascontiguousarray(B[outP]), np.ascontiguousarray(MB[outP])
+                    orc.nag_update(dB, subMB, subB, learningRate, momentum)
+                    B[outP], MB[outP] = subB, subMB
+                else:
+                    if backprop[i]:
+                        cur["dfeatures"] = orc.sgemm_ABt(dZ, W)
+                    orc.nag_update(dW, MW, W, learningRate, momentum)
+                    orc.nag_update(dB, MB, B, learningRate, momentum)
                 self.weights[i] = (W, B, pr)
                 self.momentum[i] = (MW, MB, MP)
                 nxt["dW"], nxt["dB"], nxt["dPReLU"] = dW, dB, dPr
             elif not backprop[i]:
                 continue
             elif k in ("conv", "conv_tri"):
-                cur["dfeatures"] = orc.gather_rows_backward(nxt["dfeatures"].reshape(-1, cur["nFeatures"]), nxt["rules"],
-                                                            cur["nSpatialSites"], cur["nFeatures"])
+                width = len(cur["present"])
+                cur["dfeatures"] = orc.gather_rows_backward(nxt["dfeatures"].reshape(-1, width), nxt["rules"],
+                                                            cur["nSpatialSites"], width)
             elif k in ("maxpool", "maxpool_tri", "fmp"):
                 cur["dfeatures"] = orc.maxpool_backward(nxt["dfeatures"], nxt["choices"], cur["nSpatialSites"])
             elif k == "terminal":

@@ -109,6 +109,8 @@ def lib():
         "scn_sgemm_ABt_workspace": (i64, [C.c_int, C.c_int]),
         "scn_sgemm_ABt": (C.c_int, [vp, vp, vp, vp, i64, C.c_int, C.c_int, vp]),
         "scn_nag_update": (C.c_int, [vp, vp, vp, vp, i64, f32, f32, C.c_int]),
+        "scn_shrink_matrix": (C.c_int, [vp, vp, vp, vp, vp, C.c_int, C.c_int, C.c_int]),
+        "scn_nag_update_shrunk": (C.c_int, [vp, vp, vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, f32, f32]),
         "scn_gather_rows_backward": (C.c_int, [vp, vp, vp, vp, i64, C.c_int]),
         "scn_maxpool_backward": (C.c_int, [vp, vp, vp, i64, C.c_int, vp]),
         "scn_terminal_pool_backward": (C.c_int, [vp, vp, vp, vp, i64, C.c_int, C.c_int]),
@@ -273,6 +275,13 @@ class Context:
     def nag_update(self, d_delta, d_momentum, d_weights, n, learningRate, momentum, keepPositive=False):
         _check(lib().scn_nag_update(self.h, d_delta.ptr, d_momentum.ptr, d_weights.ptr, n, learningRate, momentum,
                                     int(keepPositive)))
+
+    def shrink_matrix(self, d_W, d_w, d_inPresent, d_outPresent, nOut, nInP, nOutP):
+        _check(lib().scn_shrink_matrix(self.h, d_W.ptr, d_w.ptr, d_inPresent.ptr, d_outPresent.ptr, nOut, nInP, nOutP))
+
+    def nag_update_shrunk(self, d_delta, d_mom, d_wts, d_inPresent, d_outPresent, nOut, nInP, nOutP, lr, momentum):
+        _check(lib().scn_nag_update_shrunk(self.h, d_delta.ptr, d_mom.ptr, d_wts.ptr, d_inPresent.ptr,
+                                           d_outPresent.ptr, nOut, nInP, nOutP, lr, momentum))
 
     def gather_rows_backward(self, d_din, d_dconv, d_rules, count, nIn):
         _check(lib().scn_gather_rows_backward(self.h, d_din.ptr, d_dconv.ptr, d_rules.ptr, count, nIn))

@@ -465,3 +465,93 @@ extern "C" int scn_terminal_pool_backward(scn_ctx *ctx, float *d_din,
   SCN_HIP_CHECK(hipGetLastError());
   return SCN_OK;
 }
+
+// ------------------------------------------------ dropout during training
+// A training batch keeps a random subset of every layer's features
+// (featuresPresent); the layer then works on the sub-matrix of its weights
+// that joins the kept inputs to the kept outputs.
+__global__ void k_shrink_matrix(const float *__restrict__ W,
+                                float *__restrict__ w,
+                                const int *__restrict__ inPresent,
+                                const int *__restrict__ outPresent, int nOut,
+                                long long total, int nOutP) {
+  long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total)
+    return;
+  const long long i = idx / nOutP;
+  const int j = (int)(idx - i * nOutP);
+  const long long row = inPresent ? inPresent[i] : i;
+  w[idx] = W[row * nOut + outPresent[j]];
+}
+
+extern "C" int scn_shrink_matrix(scn_ctx *ctx, const float *d_W, float *d_w,
+                                 const int32_t *d_inPresent,
+                                 const int32_t *d_outPresent, int nOut,
+                                 int nInPresent, int nOutPresent) {
+  SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_shrink_matrix: null context");
+  SCN_REQUIRE(nOut >= 1 && nInPresent >= 0 && nOutPresent >= 0 &&
+                  nOutPresent <= nOut,
+              SCN_ERR_ARG, "scn_shrink_matrix: nOut %d present %d x %d", nOut,
+              nInPresent, nOutPresent);
+  const long long total = (long long)nInPresent * nOutPresent;
+  if (total == 0)
+    return SCN_OK;
+  SCN_REQUIRE(d_W && d_w && d_outPresent, SCN_ERR_ARG,
+              "scn_shrink_matrix: null buffer");
+  ProfScope prof(ctx, SCN_K_BACKWARD);
+  hipLaunchKernelGGL(k_shrink_matrix, dim3(scn_ceil_div(total, 256)), dim3(256),
+                     0, ctx->stream, d_W, d_w, d_inPresent, d_outPresent, nOut,
+                     total, nOutPresent);
+  SCN_HIP_CHECK(hipGetLastError());
+  return SCN_OK;
+}
+
+// dGradientDescentShrunkMatrix: the momentum step on the entries of W (and MW)
+// that the batch used; delta is the gradient of the shrunk matrix.
+__global__ void k_nag_update_shrunk(const float *__restrict__ delta,
+                                    float *__restrict__ mom,
+                                    float *__restrict__ wts,
+                                    const int *__restrict__ inPresent,
+                                    const int *__restrict__ outPresent,
+                                    int nOut, long long total, int nOutP,
+                                    float lr, float mu) {
+  long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total)
+    return;
+  const long long i = idx / nOutP;
+  const int j = (int)(idx - i * nOutP);
+  const long long row = inPresent ? inPresent[i] : i;
+  const long long at = row * nOut + outPresent[j];
+  float w = wts[at], m = mom[at];
+  const float d = delta[idx];
+  w -= m * mu;
+  m = mu * m - lr * (1 - mu) * d;
+  w += m * (1 + mu);
+  wts[at] = w;
+  mom[at] = m;
+}
+
+extern "C" int scn_nag_update_shrunk(scn_ctx *ctx, const float *d_delta,
+                                     float *d_momentum, float *d_weights,
+                                     const int32_t *d_inPresent,
+                                     const int32_t *d_outPresent, int nOut,
+                                     int nInPresent, int nOutPresent,
+                                     float learningRate, float momentum) {
+  SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_nag_update_shrunk: null context");
+  SCN_REQUIRE(nOut >= 1 && nInPresent >= 0 && nOutPresent >= 0 &&
+                  nOutPresent <= nOut,
+              SCN_ERR_ARG, "scn_nag_update_shrunk: nOut %d present %d x %d",
+              nOut, nInPresent, nOutPresent);
+  const long long total = (long long)nInPresent * nOutPresent;
+  if (total == 0)
+    return SCN_OK;
+  SCN_REQUIRE(d_delta && d_momentum && d_weights && d_outPresent, SCN_ERR_ARG,
+              "scn_nag_update_shrunk: null buffer");
+  ProfScope prof(ctx, SCN_K_BACKWARD);
+  hipLaunchKernelGGL(k_nag_update_shrunk, dim3(scn_ceil_div(total, 256)),
+                     dim3(256), 0, ctx->stream, d_delta, d_momentum, d_weights,
+                     d_inPresent, d_outPresent, nOut, total, nOutPresent,
+                     learningRate, momentum);
+  SCN_HIP_CHECK(hipGetLastError());
+  return SCN_OK;
+}

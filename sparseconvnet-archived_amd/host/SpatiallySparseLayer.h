@@ -108,7 +108,9 @@ public:
 class NetworkInNetworkLayer : public SpatiallySparseLayer {
 private:
   RNG rng;
+  std::mutex rngMutex; // preprocess() runs on several producer threads
   vectorCUDA<float> dw, db, workspace; // gradients; W transposed for dA
+  vectorCUDA<float> w, b; // sub-matrix of a training batch with dropout
 
 public:
   vectorCUDA<float> W;
@@ -142,7 +144,9 @@ public:
 class NetworkInNetworkPReLULayer : public SpatiallySparseLayer {
 private:
   RNG rng;
+  std::mutex rngMutex;
   vectorCUDA<float> dw, db, dprelu, workspace;
+  vectorCUDA<float> w, b;
 
 public:
   vectorCUDA<float> W;

@@ -233,6 +233,8 @@ int ConvolutionalTriangularLayer::calculateInputSpatialSize(
 
 // ---- NetworkInNetworkLayer (NetworkInNetworkLayer.cu:125-202,290-331) ---------
 static void nin_preprocess(int nFeaturesIn, int nFeaturesOut,
+                           SpatiallySparseBatch &batch, float dropout,
+                           RNG &rng, std::mutex &rngMutex,
                            SpatiallySparseBatchInterface &input,
                            SpatiallySparseBatchInterface &output) {
   assert(input.nFeatures == nFeaturesIn);
@@ -241,9 +243,52 @@ static void nin_preprocess(int nFeaturesIn, int nFeaturesOut,
   output.spatialSize = input.spatialSize;
   output.nSpatialSites = input.nSpatialSites;
   share_grids(input, output);
-  // no dropout outside training: every output feature is present
-  output.featuresPresent.hVector() = range(nFeaturesOut);
+  // a training batch keeps a random subset of the output features
+  // (NetworkInNetworkLayer.cu:153-154); every other batch keeps them all
+  int o = nFeaturesOut * (batch.type == TRAINBATCH ? (1.0f - dropout) : 1.0f);
+  if (o == nFeaturesOut) {
+    output.featuresPresent.hVector() = range(nFeaturesOut);
+  } else {
+    std::lock_guard<std::mutex> lock(rngMutex);
+    output.featuresPresent.hVector() = rng.NchooseM(nFeaturesOut, o);
+  }
   output.backpropErrors = true;
+}
+// Does this training batch use a sub-matrix of the layer's weights
+// (NetworkInNetworkLayer.cu:162-164)?
+static bool nin_shrunk(SpatiallySparseBatch &batch, int nFeaturesIn,
+                       int nFeaturesOut, SpatiallySparseBatchInterface &input,
+                       SpatiallySparseBatchInterface &output) {
+  return batch.type == TRAINBATCH &&
+         (size_t)nFeaturesIn + nFeaturesOut >
+             input.featuresPresent.size() + output.featuresPresent.size();
+}
+// the training branch of forwards() (NetworkInNetworkLayer.cu:165-184): no
+// scaling by the kept fraction, weights and bias of the features present
+static void nin_forwards_shrunk(cudaMemStream &ms,
+                                SpatiallySparseBatchInterface &input,
+                                SpatiallySparseBatchInterface &output,
+                                vectorCUDA<float> &W, vectorCUDA<float> &B,
+                                vectorCUDA<float> *PReLU, vectorCUDA<float> &w,
+                                vectorCUDA<float> &b, int nFeaturesOut,
+                                int act, int precision) {
+  const int Kp = (int)input.featuresPresent.size();
+  const int Np = (int)output.featuresPresent.size();
+  w.resize64((size_t)Kp * Np);
+  b.resize64((size_t)Np);
+  SCN_CHECKED(scn_shrink_matrix(ms.ctx, W.dPtr(), w.dPtr(),
+                                input.featuresPresent.dPtr(),
+                                output.featuresPresent.dPtr(), nFeaturesOut, Kp,
+                                Np));
+  // a vector is a matrix of one row
+  SCN_CHECKED(scn_shrink_matrix(ms.ctx, B.dPtr(), b.dPtr(), nullptr,
+                                output.featuresPresent.dPtr(), nFeaturesOut, 1,
+                                Np));
+  SCN_CHECKED(scn_nin_forward(ms.ctx, input.sub->features.dPtr(), w.dPtr(),
+                              b.dPtr(), PReLU ? PReLU->dPtr() : nullptr,
+                              output.sub->features.dPtr(), output.nSpatialSites,
+                              Kp, Np, 1.0f, act, precision));
+  multiplyAddCount += (__int128_t)output.nSpatialSites * Kp * Np;
 }
 // When the preceding convolutional layer deferred its gather: run the fused
 // kernel (fp32 operands), or gather now if this layer wants bf16 operands.
@@ -276,7 +321,8 @@ static bool nin_fused(cudaMemStream &ms, SpatiallySparseBatchInterface &input,
 // momentum step on W and B.
 static void nin_backwards(cudaMemStream &ms,
                           SpatiallySparseBatchInterface &input,
-                          SpatiallySparseBatchInterface &output, int K, int N,
+                          SpatiallySparseBatchInterface &output, int nFeaturesIn,
+                          int nFeaturesOut, vectorCUDA<float> *shrunkW,
                           int act, vectorCUDA<float> &W, vectorCUDA<float> &MW,
                           vectorCUDA<float> &B, vectorCUDA<float> &MB,
                           vectorCUDA<float> *PReLU, vectorCUDA<float> *MPReLU,
@@ -284,7 +330,11 @@ static void nin_backwards(cudaMemStream &ms,
                           vectorCUDA<float> *dprelu,
                           vectorCUDA<float> &workspace, float learningRate,
                           float momentum) {
+  // with dropout: the features present, and the sub-matrix forwards() left
+  // in shrunkW (NetworkInNetworkLayer.cu:235-263)
   const int64_t M = output.nSpatialSites;
+  const int K = (int)input.featuresPresent.size();
+  const int N = (int)output.featuresPresent.size();
   dw.resize64((size_t)K * N);
   db.resize64((size_t)N);
   if (dprelu)
@@ -302,15 +352,28 @@ static void nin_backwards(cudaMemStream &ms,
   if (input.backpropErrors) {
     input.sub->dfeatures.resize64((size_t)input.nSpatialSites * K);
     workspace.resize64((size_t)scn_sgemm_ABt_workspace(N, K));
-    SCN_CHECKED(scn_sgemm_ABt(ms.ctx, output.sub->dfeatures.dPtr(), W.dPtr(),
+    SCN_CHECKED(scn_sgemm_ABt(ms.ctx, output.sub->dfeatures.dPtr(),
+                              shrunkW ? shrunkW->dPtr() : W.dPtr(),
                               input.sub->dfeatures.dPtr(), M, N, K,
                               workspace.dPtr()));
     multiplyAddCount += (__int128_t)M * K * N;
   }
-  SCN_CHECKED(scn_nag_update(ms.ctx, dw.dPtr(), MW.dPtr(), W.dPtr(),
-                             (int64_t)K * N, learningRate, momentum, 0));
-  SCN_CHECKED(scn_nag_update(ms.ctx, db.dPtr(), MB.dPtr(), B.dPtr(), N,
-                             learningRate, momentum, 0));
+  if (shrunkW) {
+    SCN_CHECKED(scn_nag_update_shrunk(
+        ms.ctx, dw.dPtr(), MW.dPtr(), W.dPtr(), input.featuresPresent.dPtr(),
+        output.featuresPresent.dPtr(), nFeaturesOut, K, N, learningRate,
+        momentum));
+    SCN_CHECKED(scn_nag_update_shrunk(
+        ms.ctx, db.dPtr(), MB.dPtr(), B.dPtr(), nullptr,
+        output.featuresPresent.dPtr(), nFeaturesOut, 1, N, learningRate,
+        momentum));
+  } else {
+    SCN_CHECKED(scn_nag_update(ms.ctx, dw.dPtr(), MW.dPtr(), W.dPtr(),
+                               (int64_t)K * N, learningRate, momentum, 0));
+    SCN_CHECKED(scn_nag_update(ms.ctx, db.dPtr(), MB.dPtr(), B.dPtr(), N,
+                               learningRate, momentum, 0));
+  }
+  (void)nFeaturesIn;
 }
 
 static void read_floats(std::ifstream &f, vectorCUDA<float> &v) {
@@ -345,14 +408,19 @@ NetworkInNetworkLayer::NetworkInNetworkLayer(cudaMemStream &memStream,
 void NetworkInNetworkLayer::preprocess(SpatiallySparseBatch &batch,
                                        SpatiallySparseBatchInterface &input,
                                        SpatiallySparseBatchInterface &output) {
-  if (batch.type == TRAINBATCH && dropout > 0)
-    unsupported("dropout during training");
-  nin_preprocess(nFeaturesIn, nFeaturesOut, input, output);
+  nin_preprocess(nFeaturesIn, nFeaturesOut, batch, dropout, rng, rngMutex,
+                 input, output);
 }
 void NetworkInNetworkLayer::forwards(SpatiallySparseBatch &batch,
                                      SpatiallySparseBatchInterface &input,
                                      SpatiallySparseBatchInterface &output) {
-  output.sub->features.resize64((size_t)output.nSpatialSites * nFeaturesOut);
+  output.sub->features.resize64((size_t)output.nSpatialSites *
+                                output.featuresPresent.size());
+  if (nin_shrunk(batch, nFeaturesIn, nFeaturesOut, input, output)) {
+    nin_forwards_shrunk(memStream, input, output, W, B, nullptr, w, b,
+                        nFeaturesOut, (int)fn, precision);
+    return;
+  }
   // test-time scaling by the kept fraction (NetworkInNetworkLayer.cu:188)
   float p = 1.0f - (batch.type != RESCALEBATCH ? dropout : 0.0f);
   if (!nin_fused(memStream, input, output, W, B, nullptr, nFeaturesOut, p,
@@ -369,10 +437,12 @@ void NetworkInNetworkLayer::backwards(SpatiallySparseBatch &batch,
                                       SpatiallySparseBatchInterface &input,
                                       SpatiallySparseBatchInterface &output,
                                       float learningRate, float momentum) {
-  (void)batch;
-  nin_backwards(memStream, input, output, nFeaturesIn, nFeaturesOut, (int)fn, W,
-                MW, B, MB, nullptr, nullptr, dw, db, nullptr, workspace,
-                learningRate, momentum);
+  nin_backwards(memStream, input, output, nFeaturesIn, nFeaturesOut,
+                nin_shrunk(batch, nFeaturesIn, nFeaturesOut, input, output)
+                    ? &w
+                    : nullptr,
+                (int)fn, W, MW, B, MB, nullptr, nullptr, dw, db, nullptr,
+                workspace, learningRate, momentum);
 }
 void NetworkInNetworkLayer::loadWeightsFromStream(std::ifstream &f,
                                                   bool momentum) {
@@ -424,13 +494,22 @@ void NetworkInNetworkPReLULayer::preprocess(
     SpatiallySparseBatch &batch, SpatiallySparseBatchInterface &input,
     SpatiallySparseBatchInterface &output) {
   if (batch.type == TRAINBATCH && dropout > 0)
-    unsupported("dropout during training");
-  nin_preprocess(nFeaturesIn, nFeaturesOut, input, output);
+    // NetworkInNetworkPReLULayer.cu:195: the reference's backward pass then
+    // pairs the slopes with the wrong columns and reads past their gradient
+    unsupported("training a PReLU layer with dropout of its own");
+  nin_preprocess(nFeaturesIn, nFeaturesOut, batch, dropout, rng, rngMutex,
+                 input, output);
 }
 void NetworkInNetworkPReLULayer::forwards(
     SpatiallySparseBatch &batch, SpatiallySparseBatchInterface &input,
     SpatiallySparseBatchInterface &output) {
-  output.sub->features.resize64((size_t)output.nSpatialSites * nFeaturesOut);
+  output.sub->features.resize64((size_t)output.nSpatialSites *
+                                output.featuresPresent.size());
+  if (nin_shrunk(batch, nFeaturesIn, nFeaturesOut, input, output)) {
+    nin_forwards_shrunk(memStream, input, output, W, B, &PReLU, w, b,
+                        nFeaturesOut, (int)PRELU, precision);
+    return;
+  }
   float p = 1.0f - (batch.type != RESCALEBATCH ? dropout : 0.0f);
   if (!nin_fused(memStream, input, output, W, B, &PReLU, nFeaturesOut, p,
                  (int)PRELU, precision))
@@ -445,8 +524,10 @@ void NetworkInNetworkPReLULayer::forwards(
 void NetworkInNetworkPReLULayer::backwards(
     SpatiallySparseBatch &batch, SpatiallySparseBatchInterface &input,
     SpatiallySparseBatchInterface &output, float learningRate, float momentum) {
-  (void)batch;
   nin_backwards(memStream, input, output, nFeaturesIn, nFeaturesOut,
+                nin_shrunk(batch, nFeaturesIn, nFeaturesOut, input, output)
+                    ? &w
+                    : nullptr,
                 (int)PRELU, W, MW, B, MB, &PReLU, &MPReLU, dw, db, &dprelu,
                 workspace, learningRate, momentum);
 }

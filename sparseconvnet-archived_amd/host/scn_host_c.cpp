@@ -432,12 +432,16 @@ void scnh_iface_info(scnh_net *net, int i, int *nFeatures, int *nSpatialSites,
                      int *spatialSize, int64_t *nRules, int64_t *nFeatureElems,
                      int64_t *nChoices, int64_t *nGridEntries) {
   SpatiallySparseBatchInterface &f = net->batch->interfaces.at(i);
-  *nFeatures = f.nFeatures;
+  // the width of the feature matrix: all features, or during a training
+  // batch with dropout the ones present
+  *nFeatures = (int)f.featuresPresent.size();
   *nSpatialSites = f.nSpatialSites;
   *spatialSize = f.spatialSize;
   *nRules = (int64_t)f.rules.size64();
   *nFeatureElems =
-      f.deferredGatherFrom ? 0 : (int64_t)f.nSpatialSites * f.nFeatures;
+      f.deferredGatherFrom
+          ? 0
+          : (int64_t)f.nSpatialSites * (int64_t)f.featuresPresent.size();
   *nChoices = (int64_t)f.sub->poolingChoices.size64();
   int64_t n = 0;
   if (f.deviceGrids)
@@ -453,7 +457,15 @@ void scnh_iface_rules(scnh_net *net, int i, int32_t *out) {
 void scnh_iface_features(scnh_net *net, int i, float *out) {
   SpatiallySparseBatchInterface &f = net->batch->interfaces.at(i);
   SCN_CHECKED(scn_d2h(net->cnn->memStream.ctx, out, f.sub->features.dPtr(),
-                      (size_t)f.nSpatialSites * f.nFeatures * sizeof(float)));
+                      (size_t)f.nSpatialSites * f.featuresPresent.size() *
+                          sizeof(float)));
+}
+int scnh_iface_features_present(scnh_net *net, int i, int32_t *out) {
+  SpatiallySparseBatchInterface &f = net->batch->interfaces.at(i);
+  std::vector<int> &v = f.featuresPresent.hVector();
+  if (out)
+    std::copy(v.begin(), v.end(), out);
+  return (int)v.size();
 }
 void scnh_iface_dfeatures(scnh_net *net, int i, float *out) {
   SpatiallySparseBatchInterface &f = net->batch->interfaces.at(i);

@@ -151,6 +151,10 @@ void scnh_iface_info(scnh_net *net, int i, int *nFeatures, int *nSpatialSites,
                      int64_t *nChoices, int64_t *nGridEntries);
 void scnh_iface_rules(scnh_net *net, int i, int32_t *out);
 void scnh_iface_features(scnh_net *net, int i, float *out);
+/* SpatiallySparseBatchInterface::featuresPresent: which of the interface's
+ * nFeatures the columns of its feature matrix are (all of them except in a
+ * training batch with dropout).  Returns their number; out may be null. */
+int scnh_iface_features_present(scnh_net *net, int i, int32_t *out);
 /* gradient of the cost with respect to that feature matrix after a TRAINBATCH
  * (SpatiallySparseBatchSubInterface::dfeatures); size in floats, 0 when the
  * backward pass did not reach the interface */

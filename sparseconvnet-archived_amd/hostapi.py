@@ -64,6 +64,7 @@ def lib():
         "scnh_codify_picture": (i64, [vp, i64, i32, i64, i64, vp, vp, vp, vp]),
         "scnh_process_dataset": (f32, [vp, vp, i32]),
         "scnh_add_lenet_layer_fmp": (i32, [vp, i32, i32, i32, i32, i32, f32, i32, f32, i32]),
+        "scnh_iface_features_present": (i32, [vp, i32, vp]),
         "scnh_iface_region_ticks_size": (i64, [vp, i32]),
         "scnh_iface_region_ticks": (None, [vp, i32, vp]),
         "scnh_process_dataset_train": (f32, [vp, vp, i32, f32, f32]),
@@ -275,6 +276,13 @@ class Net:
 
     def processDatasetTrain(self, ds, batchSize=100, learningRate=0.0, momentum=0.99):
         return lib().scnh_process_dataset_train(self.h, ds.h, batchSize, learningRate, momentum)
+
+    def features_present(self, i):
+        """featuresPresent of interface i: which features the columns of its feature matrix are"""
+        n = lib().scnh_iface_features_present(self.h, i, None)
+        out = np.empty(n, np.int32)
+        lib().scnh_iface_features_present(self.h, i, _p(out))
+        return out
 
     def region_ticks(self, i):
         """(inputL, inputR), each [batch, dimension, spatialSize of interface i]: the regions a fractional

@@ -154,3 +154,34 @@ def test_terminal_pool_backward_bit_exact(scn, ctx):
         d_din = ctx.array(np.zeros((rows, C), np.float32))
         ctx.terminal_pool_backward(d_din, ctx.array(dout), ctx.array(rules), B, C, S)
         assert np.array_equal(d_din.download(), orc.terminal_pool_backward(dout, rules, S, rows))
+
+
+def test_dropout_sub_matrix_and_its_update(scn, ctx):
+    """scn_shrink_matrix picks W[inPresent][outPresent]; scn_nag_update_shrunk moves exactly those entries."""
+    rng = np.random.default_rng(21)
+    for K, N, Kp, Np in [(12, 32, 12, 16), (256, 64, 128, 32), (100, 100, 37, 100), (1, 800, 1, 123)]:
+        W = rng.standard_normal((K, N)).astype(np.float32)
+        M = (rng.standard_normal((K, N)) * 0.1).astype(np.float32)
+        inP = np.sort(rng.choice(K, Kp, replace=False)).astype(np.int32)
+        outP = np.sort(rng.choice(N, Np, replace=False)).astype(np.int32)
+        d_w = ctx.empty((Kp, Np), np.float32)
+        d_W, d_M = ctx.array(W), ctx.array(M)
+        ctx.shrink_matrix(d_W, d_w, ctx.array(inP), ctx.array(outP), N, Kp, Np)
+        assert np.array_equal(d_w.download(), W[np.ix_(inP, outP)])
+        delta = rng.standard_normal((Kp, Np)).astype(np.float32)
+        ctx.nag_update_shrunk(ctx.array(delta), d_M, d_W, ctx.array(inP), ctx.array(outP), N, Kp, Np, 0.01, 0.9)
+        subW, subM = np.ascontiguousarray(W[np.ix_(inP, outP)]), np.ascontiguousarray(M[np.ix_(inP, outP)])
+        orc.nag_update(delta, subM, subW, 0.01, 0.9)
+        wantW, wantM = W.copy(), M.copy()
+        wantW[np.ix_(inP, outP)], wantM[np.ix_(inP, outP)] = subW, subM
+        gotW, gotM = d_W.download(), d_M.download()
+        untouched = np.ones((K, N), bool)
+        untouched[np.ix_(inP, outP)] = False
+        assert np.array_equal(gotW[untouched], W[untouched]) and np.array_equal(gotM[untouched], M[untouched])
+        assert np.allclose(gotW, wantW, rtol=1e-6, atol=1e-7) and np.allclose(gotM, wantM, rtol=1e-6, atol=1e-8)
+    # a vector is a matrix of one row: null row list
+    B = rng.standard_normal(64).astype(np.float32)
+    outP = np.array([3, 9, 63], np.int32)
+    d_b = ctx.empty(3, np.float32)
+    scn._check(scn.lib().scn_shrink_matrix(ctx.h, ctx.array(B).ptr, d_b.ptr, None, ctx.array(outP).ptr, 64, 1, 3))
+    assert np.array_equal(d_b.download(), B[outP])

@@ -147,3 +147,85 @@ def test_training_lowers_the_cost(scn):
     print("NLL before %.4f after %.4f" % (before, after), flush=True)
     assert after < 0.5 * before
     net.close()
+
+
+def test_training_with_dropout(scn):
+    """NiN layers with dropout: a training batch keeps a random subset of their output features (read back from the
+    host library and handed to the oracle), the layers run on the sub-matrices of their weights, and only the entries
+    used take the momentum step.  A PReLU layer without dropout of its own sits above dropped inputs."""
+    from sparseconvnet_archived_amd import hostapi, synthetic
+    stack = [("addLeNetLayerMP", 64, 2, 1, 3, 2, synthetic.VLEAKYRELU, 0.5),
+             ("addLeNetLayerMP", 64, 2, 1, 2, 2, synthetic.RELU, 0.5),
+             ("addLeNetLayerMP", 96, 2, 1, 1, 1, synthetic.PRELU, 0.0),
+             ("addLeNetLayerMP", 64, 1, 1, 1, 1, synthetic.TANH, 0.5),
+             ("addTerminalPoolingLayer", 2), ("addSoftmaxLayer",)]
+    cfg = synthetic.Config("dropout", 2, 3, 10, 8, 14, stack)
+    cfg.number = 2
+    net, ora = pair(cfg, hostapi, 91)
+    assert net.inputSpatialSize == ora.inputSpatialSize
+    lattice = net.inputSpatialSize
+    rng = np.random.default_rng(12)
+    samples = []
+    for _ in range(16):
+        pts = np.array([(a, b) for a in range(lattice) for b in range(lattice) if rng.random() < 0.3], np.int32)
+        samples.append((pts, rng.uniform(-1, 1, (len(pts), 3)).astype(np.float32), int(rng.integers(0, 10))))
+    ds = hostapi.Dataset("dropout", 3, 10, hostapi.TRAINBATCH)
+    for pts, f, label in samples:
+        ds.add_points(2, lattice, pts, f, label)
+    lr, mu = 0.01, 0.9
+    net.set_training(lr, mu, shuffle=False)
+    net.begin(ds, 8)
+    layers = net.layers()
+    before = {i: net.get_weights(i) for i, l in enumerate(layers) if l["kind"].startswith("nin")}
+    drawn = []
+    for b in range(2):
+        assert net.next_batch()
+        mine = samples[b * 8:(b + 1) * 8]
+        present = {i: net.features_present(i + 1) for i, l in enumerate(layers) if l["kind"].startswith("nin")}
+        drawn.append(present)
+        kept = {i: len(p) for i, p in present.items()}
+        print("batch", b, "features kept per NiN layer:", kept, flush=True)
+        for i, p in present.items():
+            assert np.all(np.diff(p) > 0) and p[0] >= 0 and p[-1] < layers[i]["nOut"]
+        # (the builder rounds the kept features to a multiple of 32, SparseConvNetCUDA.cu:55-58)
+        assert kept == {1: 32, 4: 32, 7: 96, 8: 32, 10: 10}
+        S, K, R, bg, feats, n = synthetic.codify(mine, 2, lattice, lattice, 3)
+        labels = np.array([s[2] for s in mine], np.int32)
+        fwd = ora.forward(len(mine), S, K, R, bg, feats, n, labels, present=present)
+        ora.train_step(fwd, labels, lr, mu)
+        for i, wi in enumerate(fwd["interfaces"]):
+            gi = net.interface(i)
+            assert gi["features"].shape == wi["features"].shape
+            assert rel_l2(gi["features"], wi["features"]) <= 1e-4
+            if "dfeatures" in wi:
+                assert rel_l2(net.dfeatures(i), wi["dfeatures"]) <= 1e-4
+        for i in present:
+            W, B, pr = net.get_weights(i)
+            MW, MB, MP = net.get_weights(i, momentum=True)
+            oW, oB, opr = ora.weights[i]
+            assert rel_l2(MW, ora.momentum[i][0]) <= 1e-4 and rel_l2(MB, ora.momentum[i][1]) <= 1e-4
+            assert np.allclose(W, oW, rtol=1e-4, atol=1e-6) and np.allclose(B, oB, rtol=1e-4, atol=1e-6)
+    # weights that joined no kept pair in either batch have not moved at all
+    i = 4
+    W0 = before[i][0]
+    W1 = net.get_weights(i)[0]
+    used = np.zeros_like(W0, bool)
+    for present in drawn:
+        used[np.ix_(net_in_present(layers, present, i), present[i])] = True
+    assert np.array_equal(W1[~used], W0[~used]) and (~used).any() and not np.array_equal(W1[used], W0[used])
+    assert drawn[0][4].tolist() != drawn[1][4].tolist()  # a new draw for every batch
+    net.close()
+
+
+def net_in_present(layers, present, i):
+    """features present at the input of NiN layer i: the kept outputs of the NiN below, replicated by the
+    convolution in between (ConvolutionalLayer.cu:74-80); pooling layers pass them on"""
+    below = [j for j in present if j < i]
+    if not below:
+        return np.arange(layers[i]["nIn"])
+    p, nf = present[max(below)], layers[max(below)]["nOut"]
+    conv = [l for l in layers[max(below) + 1:i] if l["kind"] == "conv"]
+    if not conv:
+        return p
+    fs = conv[0]["nOut"] // conv[0]["nIn"]
+    return np.concatenate([p + nf * q for q in range(fs)])
