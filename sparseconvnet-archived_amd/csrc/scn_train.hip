@@ -309,8 +309,9 @@ extern "C" int scn_nag_update(scn_ctx *ctx, const float *d_delta,
 // run of consecutive rule entries; lane j of it owns channel j (+ P, + 2P ..).
 // Consecutive entries that name the same input row (a sample's background row
 // fills most of a sparse rule book) are summed in a register and reach memory
-// as one atomic add.
-#define SCATTER_RUN 32
+// as one atomic add.  Runs of 8: measured on the 2-D benchmark net, one atomic
+// per entry and runs of 32 both cost 10 % more of a training step.
+#define SCATTER_RUN 8
 __global__ __launch_bounds__(256) void k_gather_backward(
     float *__restrict__ din, const float *__restrict__ dconv,
     const int *__restrict__ rules, long long count, int nIn, int P) {
