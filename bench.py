@@ -34,21 +34,21 @@ BALANCE_FLOP_PER_BYTE = {k: v * 1e12 / 8e12 for k, v in MFMA_PEAK_TFLOPS.items()
 # Only valid for the default batch and seed of the config with fused convolutions (the default).
 MEASURED_TRAFFIC = {
     ("c2_sparse_net_2d", "gather", 0): 2.66e6 + 4.01e6,
-    ("c2_sparse_net_2d", "nin", 1): 4.07e6 + 10.70e6,
+    ("c2_sparse_net_2d", "nin", 1): 4.06e6 + 10.70e6,
     ("c2_sparse_net_2d", "maxpool", 2): 14.57e6 + 10.77e6,
-    ("c2_sparse_net_2d", "conv_nin", 4): 7.59e6 + 15.48e6,
-    ("c2_sparse_net_2d", "maxpool", 5): 22.67e6 + 11.76e6,
-    ("c2_sparse_net_2d", "conv_nin", 7): 8.11e6 + 11.45e6,
+    ("c2_sparse_net_2d", "conv_nin", 4): 7.56e6 + 15.48e6,
+    ("c2_sparse_net_2d", "maxpool", 5): 22.66e6 + 11.76e6,
+    ("c2_sparse_net_2d", "conv_nin", 7): 8.12e6 + 11.45e6,
     ("c2_sparse_net_2d", "maxpool", 8): 17.42e6 + 8.01e6,
-    ("c2_sparse_net_2d", "conv_nin", 10): 10.10e6 + 5.98e6,
+    ("c2_sparse_net_2d", "conv_nin", 10): 10.07e6 + 5.98e6,
     ("c2_sparse_net_2d", "maxpool", 11): 8.42e6 + 3.35e6,
-    ("c2_sparse_net_2d", "conv_nin", 13): 16.47e6 + 1.58e6,
+    ("c2_sparse_net_2d", "conv_nin", 13): 16.48e6 + 1.58e6,
     ("c2_sparse_net_2d", "maxpool", 14): 1.79e6 + 0.51e6,
-    ("c2_sparse_net_2d", "nin", 15): 2.63e6 + 0.31e6,
-    ("c2_sparse_net_2d", "nin", 17): 0.87e6 + 0.04e6,
-    ("c5_spatiotemporal_3d", "conv_nin", 1): 696.17e6 + 845.62e6,
-    ("c5_spatiotemporal_3d", "conv_nin", 3): 1762.18e6 + 1614.81e6,
-    ("c5_spatiotemporal_3d", "maxpool", 4): 1651.07e6 + 522.02e6,
+    ("c2_sparse_net_2d", "nin", 15): 2.66e6 + 0.31e6,
+    ("c2_sparse_net_2d", "nin", 17): 0.89e6 + 0.04e6,
+    ("c5_spatiotemporal_3d", "conv_nin", 1): 717.18e6 + 845.62e6,
+    ("c5_spatiotemporal_3d", "conv_nin", 3): 1816.42e6 + 1614.81e6,
+    ("c5_spatiotemporal_3d", "maxpool", 4): 1651.12e6 + 522.02e6,
 }
 
 
@@ -72,6 +72,9 @@ def parse():
                          "spreads streams over 4 hardware queues, and kernels of streams that share a queue run "
                          "in order: with 5 producer streams the forward pass's stream (created first) still has "
                          "its queue to itself (measured: 0.30 ms per batch of config 2, 0.35 with 6 or 4)")
+    ap.add_argument("--train", action="store_true",
+                    help="time training batches instead (forward, backward pass, momentum step; Pictures on the host, "
+                         "processDataset on a TRAINBATCH dataset): an auxiliary line, not the headline metric")
     ap.add_argument("--fused", type=int, choices=[0, 1], default=1,
                     help="1: setFusedConvolutions, a convolution's gather runs inside the next NiN kernel (same "
                          "results bit for bit); 0: the reference's two steps, gather then NiN")
@@ -141,6 +144,9 @@ def main():
     for i, (W, Bv, pr) in weights.items():
         net.set_weights(i, W, Bv, pr)
     samples = synthetic.make_samples(cfg, args.seed)
+    if args.train:
+        train_leg(args, cfg, net, hostapi, samples, saved_stdout)
+        return
     S, K, R, bg, feats, nSites = synthetic.codify(samples, cfg.dimension, cfg.lattice, net.inputSpatialSize,
                                                   cfg.nInputFeatures)
     active = int(len(K))
@@ -338,6 +344,38 @@ def main():
     sys.stdout.flush()
     os.dup2(saved_stdout, 1)
     print(json.dumps(out))
+
+
+def train_leg(args, cfg, net, hostapi, samples, saved_stdout):
+    """--train: `warmup` untimed training batches, then `steps` timed ones, through processDataset on a TRAINBATCH
+    dataset of the same synthetic samples (learning rate 1e-4, momentum 0.9)."""
+    assert cfg.nClasses > 1, "training needs a net that ends in the classifier (configs 2, 3, 4)"
+    B = cfg.batch
+
+    def dataset(nBatches):
+        ds = hostapi.Dataset("train", cfg.nInputFeatures, cfg.nClasses, hostapi.TRAINBATCH)
+        for _ in range(nBatches):
+            for pts, f, label in samples:
+                ds.add_points(cfg.dimension, cfg.lattice, pts, f, label)
+        return ds
+
+    net.processDatasetTrain(dataset(max(1, args.warmup)), B, 1e-4, 0.9)
+    timed = dataset(args.steps)
+    t0 = time.perf_counter()
+    nll = net.processDatasetTrain(timed, B, 1e-4, 0.9)
+    dt = time.perf_counter() - t0
+    line = {
+        "metric": "training samples/s (forward + backward + momentum step, 1 GPU)", "value": B * args.steps / dt,
+        "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": 1e3 * dt / args.steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "%s, batch %d, training batches from host-resident Pictures" % (cfg.name, B),
+                   "mode": "train", "learning_rate": 1e-4, "momentum": 0.9, "nll_of_the_timed_pass": nll},
+        "roofline": None, "cpu_baseline": None,
+    }
+    sys.stdout.flush()
+    os.dup2(saved_stdout, 1)
+    print(json.dumps(line))
 
 
 def cpu_leg(cfg, layers, weights, samples, spatialSize, budget_s):
