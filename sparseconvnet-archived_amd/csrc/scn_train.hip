@@ -192,6 +192,151 @@ __global__ __launch_bounds__(256) void k_gemm_atb(
       }
 }
 
+// The same product for shapes that fill wider tiles (K and N multiples of 4,
+// 16-byte aligned operands).  WK x WN wavefronts per workgroup, 64 x 64 of
+// the output each: 16 accumulator tiles per wavefront fed by ONE 128-bit LDS
+// read per operand and k-step (lane (c, q) reads columns 4c..4c+3 of row
+// 4s + q, so MFMA tile i covers the output rows 4 * (its A-operand index) + i
+// and tile j the output columns 4c + j: 0.125 LDS reads per MFMA instead of
+// 1.25).  Chunks of 16 rows, double-buffered: the global loads of the next
+// chunk are in flight under the MFMAs of this one, one barrier per chunk.
+#define ATBW_ROWS 16
+template <int WK, int WN>
+__global__ __launch_bounds__(64 * WK * WN) void k_gemm_atb_wide(
+    const float *__restrict__ A, const float *__restrict__ D,
+    float *__restrict__ dW, long long M, int K, int N, int nTiles,
+    long long rowsPerSplit) {
+  constexpr int TK = 64 * WK, TN = 64 * WN, PA = TK + 16, PD = TN + 16;
+  constexpr int NT = 64 * WK * WN;
+  constexpr int LA = ATBW_ROWS * TK / 4 / NT; // float4 loads per lane, A
+  constexpr int LD = ATBW_ROWS * TN / 4 / NT; // ... and D
+  static_assert(LA * NT * 4 == ATBW_ROWS * TK && LD * NT * 4 == ATBW_ROWS * TN &&
+                    LD >= 1,
+                "chunk loads divide evenly");
+  __shared__ __align__(16) float sA[2][ATBW_ROWS * PA];
+  __shared__ __align__(16) float sD[2][ATBW_ROWS * PD];
+  const int k0 = (blockIdx.x / nTiles) * TK, n0 = (blockIdx.x % nTiles) * TN;
+  const long long m0 = (long long)blockIdx.y * rowsPerSplit;
+  const long long m1 = m0 + rowsPerSplit < M ? m0 + rowsPerSplit : M;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int wk = wave / WN, wn = wave % WN, c = lane & 15, q = lane >> 4;
+  floatx4 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float4 ra[LA], rd[LD];
+  auto fetch = [&](long long m) {
+#pragma unroll
+    for (int u = 0; u < LA; ++u) {
+      const int f = t + u * NT, r = f / (TK / 4), col = (f % (TK / 4)) * 4;
+      const long long row = m + r;
+      ra[u] = row < m1 && k0 + col < K
+                  ? *(const float4 *)(A + row * K + k0 + col)
+                  : float4{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int u = 0; u < LD; ++u) {
+      const int f = t + u * NT, r = f / (TN / 4), col = (f % (TN / 4)) * 4;
+      const long long row = m + r;
+      rd[u] = row < m1 && n0 + col < N
+                  ? *(const float4 *)(D + row * N + n0 + col)
+                  : float4{0.f, 0.f, 0.f, 0.f};
+    }
+  };
+  auto stage = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < LA; ++u) {
+      const int f = t + u * NT, r = f / (TK / 4), col = (f % (TK / 4)) * 4;
+      *(float4 *)(&sA[buf][r * PA + col]) = ra[u];
+    }
+#pragma unroll
+    for (int u = 0; u < LD; ++u) {
+      const int f = t + u * NT, r = f / (TN / 4), col = (f % (TN / 4)) * 4;
+      *(float4 *)(&sD[buf][r * PD + col]) = rd[u];
+    }
+  };
+  fetch(m0);
+  stage(0);
+  __syncthreads();
+  int buf = 0;
+  for (long long m = m0; m < m1; m += ATBW_ROWS, buf ^= 1) {
+    const bool more = m + ATBW_ROWS < m1;
+    if (more)
+      fetch(m + ATBW_ROWS);
+    const float *pa = &sA[buf][q * PA + wk * 64 + 4 * c];
+    const float *pd = &sD[buf][q * PD + wn * 64 + 4 * c];
+#pragma unroll
+    for (int s4 = 0; s4 < ATBW_ROWS / 4; ++s4) {
+      const float4 a = *(const float4 *)(pa + 4 * s4 * PA);
+      const float4 d = *(const float4 *)(pd + 4 * s4 * PD);
+      const float av[4] = {a.x, a.y, a.z, a.w}, dv[4] = {d.x, d.y, d.z, d.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[i], dv[j],
+                                                           acc[i][j], 0, 0, 0);
+    }
+    if (more)
+      stage(buf ^ 1);
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int k = k0 + wk * 64 + 4 * (4 * q + v) + i;
+      if (k >= K)
+        continue;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int n = n0 + wn * 64 + 4 * c + j;
+        if (n < N)
+          unsafeAtomicAdd(dW + (long long)k * N + n, acc[i][j][v]);
+      }
+    }
+}
+
+template <int WK, int WN>
+static int launch_atb_wide(scn_ctx *ctx, const float *d_A, const float *d_D,
+                           float *d_dW, int64_t M, int K, int N) {
+  constexpr int TK = 64 * WK, TN = 64 * WN;
+  const int kTiles = scn_ceil_div(K, TK), nTiles = scn_ceil_div(N, TN);
+  const long long tiles = (long long)kTiles * nTiles;
+  // Row ranges: more of them shorten every workgroup's walk, but each adds
+  // one more tile of float atomics onto the same K x N addresses, and those
+  // serialise.  Measured on MI355X: a workgroup walks a row in about 60 ns
+  // (it waits for memory more than for the matrix cores; four of them share a
+  // compute unit), the part retires about 45 contended atomics per ns.  Take
+  // the count that minimises the sum.
+  const long long maxSplits = (M + 8 * ATBW_ROWS - 1) / (8 * ATBW_ROWS);
+  const double flushNs = (double)K * N / (double)tiles / 45.0;
+  long long splits = 1;
+  double best = 1e300;
+  for (long long cand = 1; cand <= maxSplits && cand <= 4096;
+       cand += cand < 16 ? 1 : cand / 8) {
+    const long long wgs = tiles * cand;
+    const long long rounds = (wgs + 4 * ctx->numCU - 1) / (4 * ctx->numCU);
+    const double cost = (double)rounds * ((double)M / cand) * 60.0 +
+                        (double)wgs * flushNs;
+    if (cost < best) {
+      best = cost;
+      splits = cand;
+    }
+  }
+  long long rowsPerSplit = (M + splits - 1) / splits;
+  rowsPerSplit = (rowsPerSplit + ATBW_ROWS - 1) / ATBW_ROWS * ATBW_ROWS;
+  splits = (M + rowsPerSplit - 1) / rowsPerSplit;
+  hipLaunchKernelGGL((k_gemm_atb_wide<WK, WN>),
+                     dim3((unsigned)tiles, (unsigned)splits),
+                     dim3(64 * WK * WN), 0, ctx->stream, d_A, d_D, d_dW,
+                     (long long)M, K, N, nTiles, rowsPerSplit);
+  SCN_HIP_CHECK(hipGetLastError());
+  return SCN_OK;
+}
+
 extern "C" int scn_sgemm_AtB(scn_ctx *ctx, const float *d_A, const float *d_D,
                              float *d_dW, int64_t M, int K, int N) {
   SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_sgemm_AtB: null context");
@@ -203,6 +348,19 @@ extern "C" int scn_sgemm_AtB(scn_ctx *ctx, const float *d_A, const float *d_D,
   if (M == 0)
     return SCN_OK;
   SCN_REQUIRE(d_A && d_D, SCN_ERR_ARG, "scn_sgemm_AtB: null buffer");
+  // (outputs of a few tiles only are bound by the atomics either way: the
+  // narrow kernel below does as well on them)
+  if (K % 4 == 0 && N % 4 == 0 && N >= 48 && M >= 1024 &&
+      ((long long)K * N >= 160 * 1024 || (K >= 1024 && N >= 64)) &&
+      ((uintptr_t)d_A & 15) == 0 && ((uintptr_t)d_D & 15) == 0) {
+    // 256 x 64 or 128 x 128 tiles: whichever pads the output less
+    const long long pad41 = (long long)scn_ceil_div(K, 256) * 256 *
+                            scn_ceil_div(N, 64) * 64;
+    const long long pad22 = (long long)scn_ceil_div(K, 128) * 128 *
+                            scn_ceil_div(N, 128) * 128;
+    return pad41 < pad22 ? launch_atb_wide<4, 1>(ctx, d_A, d_D, d_dW, M, K, N)
+                         : launch_atb_wide<2, 2>(ctx, d_A, d_D, d_dW, M, K, N);
+  }
   const int kTiles = scn_ceil_div(K, 64), nTiles = scn_ceil_div(N, 64);
   const long long tiles = (long long)kTiles * nTiles;
   SCN_REQUIRE(tiles <= 0x7fffffffll, SCN_ERR_CAPACITY,

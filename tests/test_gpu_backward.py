@@ -47,7 +47,8 @@ def test_activation_backward(scn, ctx, act, M, N):
 
 
 @pytest.mark.parametrize("M,K,N", [(1, 1, 1), (50, 12, 32), (1000, 128, 64), (4097, 288, 64), (333, 100, 100),
-                                   (20000, 256, 96), (2500, 800, 800), (100, 192, 100), (70000, 1728, 64)])
+                                   (20000, 256, 96), (2500, 800, 800), (100, 192, 100), (70000, 1728, 64),
+                                   (5000, 64, 48), (3000, 132, 52), (1024, 260, 132), (9999, 1280, 480)])
 def test_weight_gradient_AtB(scn, ctx, M, K, N):
     rng = np.random.default_rng(M + K + N)
     print("AtB M=%d K=%d N=%d" % (M, K, N), flush=True)
