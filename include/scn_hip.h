@@ -293,6 +293,12 @@ int scn_nag_update_shrunk(scn_ctx *ctx, const float *d_delta,
                           const int32_t *d_outPresent, int nOut,
                           int nInPresent, int nOutPresent, float learningRate,
                           float momentum);
+/* What a RESCALEBATCH pass (scaleWeights, NetworkInNetworkLayer.cu:203-218)
+ * needs of vectorCUDA<float>: meanAbs (vectorCUDA.cu:121-155; here the sum of
+ * |x[i]| in double, returned to the host: the call waits for the stream) and
+ * multiplicativeRescale (vectorCUDA.cu:156-170). */
+int scn_sum_abs(scn_ctx *ctx, const float *d_x, int64_t n, double *h_sum);
+int scn_scale(scn_ctx *ctx, float *d_x, int64_t n, float multiplier);
 /* propBackwardFromMatrixMultiply (ConvolutionalLayer.cu:42-72):
  * din[rules[c] * nIn + j] += dconv[c * nIn + j], c < count; the caller zeroes
  * din first (ConvolutionalLayer.cu:141).  Negative rules are skipped. */

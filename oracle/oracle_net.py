@@ -106,13 +106,16 @@ class Net:
 
     # ---- forward over one batch
     def forward(self, batch, sample, key, row, bg, features, nSpatialSites, labels=None, keep=True, ticks=None,
-                present=None):
+                present=None, rescale=False):
         """Returns a list of interfaces (dicts with grids, rules, features,
         choices, nSpatialSites, nFeatures, spatialSize) and, when the net ends
         in the classifier, probabilities / predictions / mistakes / nll.
         ticks: {layer index: (inputL, inputR)} for fractional max-pooling layers (the random draw is the caller's).
         present: a TRAINBATCH with dropout -- {NiN layer index: the output features kept} (again the caller's draw);
-        feature matrices then hold the kept columns only (featuresPresent of the reference)."""
+        feature matrices then hold the kept columns only (featuresPresent of the reference).
+        rescale: a RESCALEBATCH -- no dropout scaling, and every NiN layer's weights are rescaled right after its
+        forward pass (SparseConvNetCUDA.cu:230-241, NetworkInNetworkLayer.cu:203-218); self.weights changes."""
+        scalingUnderneath = np.float32(1)
         d = self.dimension
         g = orc.Grids.from_flat(batch, sample, key, row, bg)
         feats = np.ascontiguousarray(features, np.float32)
@@ -160,9 +163,18 @@ class Net:
                     nxt["features"] = orc.nin_forward(cur["features"], w, B[outP], pr, 1.0, l["act"])
                     nxt["shrunk"] = (inP, outP, w)
                 else:
-                    p = np.float32(1.0) - np.float32(l["dropout"])
+                    p = np.float32(1.0) - (np.float32(0) if rescale else np.float32(l["dropout"]))
                     nxt["features"] = orc.nin_forward(cur["features"], W, B, pr, p, l["act"])
                 nxt["nFeatures"] = l["nOut"]
+                if rescale:
+                    scale = np.float32(np.abs(nxt["features"].astype(np.float64)).sum() / nxt["features"].size)
+                    nxt["featureScale"] = scale
+                    scale = np.float32(1) if i == len(self.layers) - 1 else np.float32(np.power(scale, np.float32(-0.1)))
+                    MW, MB, MP = getattr(self, "momentum", {}).get(i, (None, None, None))
+                    self.weights[i] = (W * (scale / scalingUnderneath), B * scale, pr)
+                    if MW is not None:
+                        self.momentum[i] = (MW * (scale / scalingUnderneath), MB * scale, MP)
+                    scalingUnderneath = scale
             elif k == "terminal":
                 og, rules, S = orc.rules_terminal(cur["grids"])
                 nxt.update(grids=og, rules=rules, nSpatialSites=batch, spatialSize=1)

@@ -111,6 +111,8 @@ def lib():
         "scn_nag_update": (C.c_int, [vp, vp, vp, vp, i64, f32, f32, C.c_int]),
         "scn_shrink_matrix": (C.c_int, [vp, vp, vp, vp, vp, C.c_int, C.c_int, C.c_int]),
         "scn_nag_update_shrunk": (C.c_int, [vp, vp, vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, f32, f32]),
+        "scn_sum_abs": (C.c_int, [vp, vp, i64, P(C.c_double)]),
+        "scn_scale": (C.c_int, [vp, vp, i64, f32]),
         "scn_gather_rows_backward": (C.c_int, [vp, vp, vp, vp, i64, C.c_int]),
         "scn_maxpool_backward": (C.c_int, [vp, vp, vp, i64, C.c_int, vp]),
         "scn_terminal_pool_backward": (C.c_int, [vp, vp, vp, vp, i64, C.c_int, C.c_int]),
@@ -282,6 +284,14 @@ class Context:
     def nag_update_shrunk(self, d_delta, d_mom, d_wts, d_inPresent, d_outPresent, nOut, nInP, nOutP, lr, momentum):
         _check(lib().scn_nag_update_shrunk(self.h, d_delta.ptr, d_mom.ptr, d_wts.ptr, d_inPresent.ptr,
                                            d_outPresent.ptr, nOut, nInP, nOutP, lr, momentum))
+
+    def sum_abs(self, d_x, n):
+        out = C.c_double()
+        _check(lib().scn_sum_abs(self.h, d_x.ptr, n, C.byref(out)))
+        return out.value
+
+    def scale(self, d_x, n, multiplier):
+        _check(lib().scn_scale(self.h, d_x.ptr, n, multiplier))
 
     def gather_rows_backward(self, d_din, d_dconv, d_rules, count, nIn):
         _check(lib().scn_gather_rows_backward(self.h, d_din.ptr, d_dconv.ptr, d_rules.ptr, count, nIn))

@@ -714,3 +714,60 @@ extern "C" int scn_nag_update_shrunk(scn_ctx *ctx, const float *d_delta,
   SCN_HIP_CHECK(hipGetLastError());
   return SCN_OK;
 }
+
+// ------------------------------------------------ weight rescaling passes
+// What a RESCALEBATCH needs of vectorCUDA<float>: meanAbs() and
+// multiplicativeRescale() (vectorCUDA.cu:121-170).
+__global__ __launch_bounds__(256) void k_sum_abs(const float *__restrict__ x,
+                                                 long long n, double *out) {
+  __shared__ double part[4];
+  double s = 0;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (long long)gridDim.x * blockDim.x)
+    s += fabsf(x[i]);
+  for (int o = 32; o > 0; o >>= 1)
+    s += __shfl_down(s, o, 64);
+  if ((threadIdx.x & 63) == 0)
+    part[threadIdx.x >> 6] = s;
+  __syncthreads();
+  if (threadIdx.x == 0)
+    unsafeAtomicAdd(out, part[0] + part[1] + part[2] + part[3]);
+}
+
+extern "C" int scn_sum_abs(scn_ctx *ctx, const float *d_x, int64_t n,
+                           double *h_sum) {
+  SCN_REQUIRE(ctx && h_sum, SCN_ERR_ARG, "scn_sum_abs: null argument");
+  SCN_REQUIRE(n >= 0, SCN_ERR_ARG, "scn_sum_abs: n %lld", (long long)n);
+  *h_sum = 0;
+  if (n == 0)
+    return SCN_OK;
+  SCN_REQUIRE(d_x, SCN_ERR_ARG, "scn_sum_abs: null buffer");
+  double *acc = (double *)(ctx->d_scalars + 8); // words 8..9: free for this
+  SCN_TRY(scn_fill32(ctx, acc, 0u, 2));
+  int blocks = scn_ceil_div(n, 256 * 16);
+  if (blocks > ctx->numCU * 8)
+    blocks = ctx->numCU * 8;
+  hipLaunchKernelGGL(k_sum_abs, dim3(blocks), dim3(256), 0, ctx->stream, d_x,
+                     (long long)n, acc);
+  SCN_HIP_CHECK(hipGetLastError());
+  return scn_d2h(ctx, h_sum, acc, sizeof(double));
+}
+
+__global__ void k_scale(float *__restrict__ x, long long n, float m) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n)
+    x[i] *= m;
+}
+
+extern "C" int scn_scale(scn_ctx *ctx, float *d_x, int64_t n,
+                         float multiplier) {
+  SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_scale: null context");
+  SCN_REQUIRE(n >= 0, SCN_ERR_ARG, "scn_scale: n %lld", (long long)n);
+  if (n == 0)
+    return SCN_OK;
+  SCN_REQUIRE(d_x, SCN_ERR_ARG, "scn_scale: null buffer");
+  hipLaunchKernelGGL(k_scale, dim3(scn_ceil_div(n, 256)), dim3(256), 0,
+                     ctx->stream, d_x, (long long)n, multiplier);
+  SCN_HIP_CHECK(hipGetLastError());
+  return SCN_OK;
+}

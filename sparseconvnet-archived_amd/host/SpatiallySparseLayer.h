@@ -131,6 +131,9 @@ public:
   void forwards(SpatiallySparseBatch &batch,
                 SpatiallySparseBatchInterface &input,
                 SpatiallySparseBatchInterface &output);
+  void scaleWeights(SpatiallySparseBatchInterface &input,
+                    SpatiallySparseBatchInterface &output,
+                    float &scalingUnderneath, bool topLayer);
   void loadWeightsFromStream(std::ifstream &f, bool momentum);
   void putWeightsToStream(std::ofstream &f, bool momentum);
   void backwards(SpatiallySparseBatch &batch,
@@ -168,6 +171,9 @@ public:
   void forwards(SpatiallySparseBatch &batch,
                 SpatiallySparseBatchInterface &input,
                 SpatiallySparseBatchInterface &output);
+  void scaleWeights(SpatiallySparseBatchInterface &input,
+                    SpatiallySparseBatchInterface &output,
+                    float &scalingUnderneath, bool topLayer);
   void loadWeightsFromStream(std::ifstream &f, bool momentum);
   void putWeightsToStream(std::ofstream &f, bool momentum);
   void backwards(SpatiallySparseBatch &batch,

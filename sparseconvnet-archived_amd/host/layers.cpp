@@ -444,6 +444,49 @@ void NetworkInNetworkLayer::backwards(SpatiallySparseBatch &batch,
                 (int)fn, W, MW, B, MB, nullptr, nullptr, dw, db, nullptr,
                 workspace, learningRate, momentum);
 }
+// scaleWeights (NetworkInNetworkLayer.cu:203-218; the PReLU layer's is the
+// same, NetworkInNetworkPReLULayer.cu:175-189): bring the mean magnitude of
+// the layer's output towards one, undoing what the layer below was scaled by
+static void nin_scale_weights(cudaMemStream &ms,
+                              SpatiallySparseBatchInterface &output,
+                              vectorCUDA<float> &W, vectorCUDA<float> &MW,
+                              vectorCUDA<float> &B, vectorCUDA<float> &MB,
+                              float &scalingUnderneath, bool topLayer) {
+  const size_t n = output.sub->features.size64();
+  assert(n > 0 && "call after forwards(...)");
+  double total = 0;
+  SCN_CHECKED(scn_sum_abs(ms.ctx, output.sub->features.dPtr(), (int64_t)n,
+                          &total));
+  if (total != total) {
+    std::cout << "NaN in vectorCUDA<t>::meanAbs()\n";
+    std::exit(1);
+  }
+  float scale = (float)(total / (double)n);
+  std::cout << "featureScale:" << scale << std::endl;
+  scale = topLayer ? 1 : powf(scale, -0.1);
+  SCN_CHECKED(scn_scale(ms.ctx, W.dPtr(), (int64_t)W.size64(),
+                        scale / scalingUnderneath));
+  SCN_CHECKED(scn_scale(ms.ctx, B.dPtr(), (int64_t)B.size64(), scale));
+  SCN_CHECKED(scn_scale(ms.ctx, MW.dPtr(), (int64_t)MW.size64(),
+                        scale / scalingUnderneath));
+  SCN_CHECKED(scn_scale(ms.ctx, MB.dPtr(), (int64_t)MB.size64(), scale));
+  scalingUnderneath = scale;
+}
+void NetworkInNetworkLayer::scaleWeights(SpatiallySparseBatchInterface &input,
+                                         SpatiallySparseBatchInterface &output,
+                                         float &scalingUnderneath,
+                                         bool topLayer) {
+  (void)input;
+  nin_scale_weights(memStream, output, W, MW, B, MB, scalingUnderneath,
+                    topLayer);
+}
+void NetworkInNetworkPReLULayer::scaleWeights(
+    SpatiallySparseBatchInterface &input, SpatiallySparseBatchInterface &output,
+    float &scalingUnderneath, bool topLayer) {
+  (void)input;
+  nin_scale_weights(memStream, output, W, MW, B, MB, scalingUnderneath,
+                    topLayer);
+}
 void NetworkInNetworkLayer::loadWeightsFromStream(std::ifstream &f,
                                                   bool momentum) {
   read_floats(f, W);

@@ -304,10 +304,21 @@ void SparseConvNetCUDA::backwardBatch(SpatiallySparseBatch &batch,
 // dataset loops queue batch i + 1 before finishing batch i, so the stream never
 // runs dry while the host is busy.
 void SparseConvNetCUDA::forwardBatch(SpatiallySparseBatch &batch) {
+  // a RESCALEBATCH rescales every layer's weights right after its forward
+  // pass (SparseConvNetCUDA.cu:230-241)
+  float scalingUnderneath = 1;
   for (size_t i = 0; i < layers.size(); i++) {
     batch.interfaces[i + 1].sub->reset();
     scn_prof_tag(memStream.ctx, (int)i);
     layers[i]->forwards(batch, batch.interfaces[i], batch.interfaces[i + 1]);
+    if (batch.type == RESCALEBATCH) {
+      std::cout << i << ":"
+                << batch.interfaces[i].sub->features.size64() * sizeof(float) /
+                       (1 << 20)
+                << "MB ";
+      layers[i]->scaleWeights(batch.interfaces[i], batch.interfaces[i + 1],
+                              scalingUnderneath, i == layers.size() - 1);
+    }
   }
   SoftmaxClassifierLaunch(batch.interfaces.back(), batch, memStream);
 }
@@ -340,12 +351,6 @@ float SparseConvNetCUDA::processDataset(SpatiallySparseDataset &dataset,
                                         int batchSize, float learningRate,
                                         float momentum) {
   assert(dataset.pictures.size() > 0);
-  if (dataset.type == RESCALEBATCH) {
-    std::fprintf(stderr, "processDataset: %s passes are not implemented in "
-                         "this library\n",
-                 batchTypeNames[dataset.type]);
-    std::exit(EXIT_FAILURE);
-  }
   float errorRate = 0, nll = 0;
   multiplyAddCount = 0;
   auto start = std::chrono::system_clock::now();
@@ -379,10 +384,12 @@ float SparseConvNetCUDA::processDataset(SpatiallySparseDataset &dataset,
   auto end = std::chrono::system_clock::now();
   auto diff =
       std::chrono::duration_cast<std::chrono::nanoseconds>(end - start).count();
-  std::cout << dataset.name;
-  if (dataset.type != UNLABELEDBATCH)
-    std::cout << " Mistakes:" << 100.0 * errorRate << "% NLL:" << nll;
-  printThroughput(diff, dataset.pictures.size());
+  if (dataset.type != RESCALEBATCH) { // SparseConvNetCUDA.cu:311
+    std::cout << dataset.name;
+    if (dataset.type != UNLABELEDBATCH)
+      std::cout << " Mistakes:" << 100.0 * errorRate << "% NLL:" << nll;
+    printThroughput(diff, dataset.pictures.size());
+  }
   return nll;
 }
 // SparseConvNetCUDA.cu:507-538

@@ -229,3 +229,33 @@ def net_in_present(layers, present, i):
         return p
     fs = conv[0]["nOut"] // conv[0]["nIn"]
     return np.concatenate([p + nf * q for q in range(fs)])
+
+
+def test_rescale_batches(scn):
+    """RESCALEBATCH passes (scaleWeights after every layer's forward pass): the weights after two passes against
+    the oracle's, and the effect they are for: the mean magnitude of every hidden layer's output moves towards 1."""
+    from sparseconvnet_archived_amd import hostapi, synthetic
+    cfg = synthetic.config(2, batch=12)
+    net, ora = pair(cfg, hostapi, 31)
+    samples = synthetic.make_samples(cfg, 32)
+    ds = hostapi.Dataset("rescale", cfg.nInputFeatures, cfg.nClasses, hostapi.RESCALEBATCH)
+    for pts, f, label in samples:
+        ds.add_points(cfg.dimension, cfg.lattice, pts, f, label)
+    S, K, R, bg, feats, n = synthetic.codify(samples, cfg.dimension, cfg.lattice, net.inputSpatialSize, cfg.nInputFeatures)
+    labels = np.array([s[2] for s in samples], np.int32)
+    layers = net.layers()
+    scales = []
+    for rep in range(3):
+        net.processDataset(ds, len(samples))
+        fwd = ora.forward(len(samples), S, K, R, bg, feats, n, labels, rescale=True)
+        scales.append([wi["featureScale"] for wi in fwd["interfaces"] if "featureScale" in wi])
+        for i, l in enumerate(layers):
+            if l["kind"].startswith("nin"):
+                W, B, pr = net.get_weights(i)
+                oW, oB, opr = ora.weights[i]
+                assert np.allclose(W, oW, rtol=2e-4, atol=1e-7), (rep, i)
+                assert np.allclose(B, oB, rtol=2e-4, atol=1e-7)
+    first, last = np.array(scales[0][:-1]), np.array(scales[-1][:-1])
+    print("feature scales of the hidden layers, first pass:", first, "third pass:", last, flush=True)
+    assert np.all(np.abs(np.log(last)) <= np.abs(np.log(first)) + 1e-3)
+    net.close()
