@@ -16,9 +16,11 @@ class StrokePicture : public Picture {
   int size;
 
 public:
-  StrokePicture(int size, int nSites, unsigned seed, int label)
+  // shapeSeed fixes where the strokes go, seed the features along them
+  StrokePicture(int size, int nSites, unsigned seed, int label,
+                unsigned shapeSeed = 0)
       : Picture(label), size(size) {
-    RNG rng(seed);
+    RNG rng(shapeSeed ? shapeSeed : seed), featureRng(seed);
     float x = rng.uniform(0.2f * size, 0.8f * size);
     float y = rng.uniform(0.2f * size, 0.8f * size);
     float angle = rng.uniform(0, 6.2831853f);
@@ -33,7 +35,8 @@ public:
       xs.push_back((int)std::lround(x));
       ys.push_back((int)std::lround(y));
       for (int c = 0; c < 3; ++c)
-        feats.push_back(rng.uniform(-1, 1));
+        feats.push_back(shapeSeed ? featureRng.uniform(0.5f, 1)
+                                  : rng.uniform(-1, 1));
     }
   }
   // the contract of Picture::codifyInputData: background row first, then one
@@ -82,6 +85,36 @@ int main(int argc, char **argv) {
               << std::endl;
     return 1;
   }
-  std::cout << "example driver ok, NLL " << nll << std::endl;
+  // Training, the way the reference's drivers loop over epochs: ten classes,
+  // each a fixed set of strokes with varying features; a small net with
+  // dropout learns to tell them apart.
+  SpatiallySparseDataset trainSet;
+  trainSet.name = "Synthetic strokes (train)";
+  trainSet.type = TRAINBATCH;
+  trainSet.nFeatures = 3;
+  trainSet.nClasses = 10;
+  for (int i = 0; i < 200; ++i)
+    trainSet.pictures.push_back(
+        new StrokePicture(28, 80, 5000u + i, i % 10, 77u + i % 10));
+  SpatiallySparseDataset validationSet = trainSet; // same pictures, test mode
+  validationSet.name = "Synthetic strokes (validation)";
+  validationSet.type = TESTBATCH;
+  DeepC2 small(2, 3, 16, VLEAKYRELU, trainSet.nFeatures, trainSet.nClasses,
+               0.2f);
+  float before = small.processDataset(validationSet, 100);
+  for (int epoch = 1; epoch <= 20; epoch++) {
+    std::cout << "epoch: " << epoch << " " << std::flush;
+    small.processDataset(trainSet, 100, 0.003 * exp(-0.01 * epoch));
+  }
+  float after = small.processDataset(validationSet, 100);
+  for (auto *p : trainSet.pictures)
+    delete p;
+  if (!(after < 0.5f * before)) {
+    std::cout << "training did not lower the cost: " << before << " -> "
+              << after << std::endl;
+    return 1;
+  }
+  std::cout << "example driver ok, NLL " << nll << ", trained " << before
+            << " -> " << after << std::endl;
   return 0;
 }
