@@ -107,18 +107,25 @@ static scn_ctx *g_defaultCtx = nullptr;
 static std::vector<scn_ctx *> g_liveCtx; // oldest first
 static std::mutex g_ctxMutex;
 
+// Ends the process the way the reference's error paths do (print, exit),
+// but without running static destructors: other threads (batch producers)
+// may still be inside the library.
+void scnExit(int code) {
+  std::fflush(nullptr);
+  std::_Exit(code);
+}
 void scnCheck(int rc, const char *file, int line) {
   if (rc == SCN_OK)
     return;
   // the reference prints the CUDA error and exits (utilities.h:36-67)
   std::fprintf(stderr, "%s:%d: libscn_hip error %d: %s\n", file, line, rc,
                scn_last_error());
-  std::exit(EXIT_FAILURE);
+  scnExit(EXIT_FAILURE);
 }
 scn_ctx *scnDefaultContext() {
   if (!g_defaultCtx) {
     std::fprintf(stderr, "no SparseConvNet context: construct the net first\n");
-    std::exit(EXIT_FAILURE);
+    scnExit(EXIT_FAILURE);
   }
   return g_defaultCtx;
 }

@@ -9,7 +9,7 @@
 
 static void unsupported(const char *what) {
   std::fprintf(stderr, "%s is not implemented in this library\n", what);
-  std::exit(EXIT_FAILURE);
+  scnExit(EXIT_FAILURE);
 }
 
 SpatiallySparseLayer::SpatiallySparseLayer(cudaMemStream &memStream)
@@ -459,7 +459,7 @@ static void nin_scale_weights(cudaMemStream &ms,
                           &total));
   if (total != total) {
     std::cout << "NaN in vectorCUDA<t>::meanAbs()\n";
-    std::exit(1);
+    scnExit(1);
   }
   float scale = (float)(total / (double)n);
   std::cout << "featureScale:" << scale << std::endl;
@@ -735,7 +735,7 @@ static void fmp_stop(const char *what, int nIn, int nOut, int poolSize) {
                "fractional max-pooling regions: %s (nIn %d, nOut %d, "
                "poolSize %d)\n",
                what, nIn, nOut, poolSize);
-  std::exit(EXIT_FAILURE);
+  scnExit(EXIT_FAILURE);
 }
 void fmpTicks(FmpKind kind, int nIn, int nOut, int poolSize, RNG &rng,
               int *inputL, int *inputR) {

@@ -542,7 +542,7 @@ void SparseConvNetCUDA::loadWeights(std::string baseName, int epoch,
   std::ifstream f(filename.c_str(), std::ios::in | std::ios::binary);
   if (!f) {
     std::cout << "Cannot find " << filename << std::endl;
-    std::exit(EXIT_FAILURE);
+    scnExit(EXIT_FAILURE);
   }
   std::cout << "Loading network parameters from " << filename << std::endl;
   for (int i = 0; i < std::min((int)layers.size(), firstNlayers); i++)
@@ -557,7 +557,7 @@ void SparseConvNetCUDA::saveWeights(std::string baseName, int epoch,
   std::ofstream f(filename.c_str(), std::ios::binary);
   if (!f) {
     std::cout << "Cannot write " << filename << std::endl;
-    std::exit(EXIT_FAILURE);
+    scnExit(EXIT_FAILURE);
   }
   for (auto *l : layers)
     l->putWeightsToStream(f, momentum);

@@ -25,6 +25,7 @@ public:
 // oldest live cudaMemStream (the net's own memStream)
 scn_ctx *scnDefaultContext();
 void scnCheck(int rc, const char *file, int line);
+void scnExit(int code); // flush, then leave without static destructors
 #define SCN_CHECKED(expr) scnCheck((expr), __FILE__, __LINE__)
 
 template <typename t> class vectorCUDA {
