@@ -121,7 +121,7 @@ def main():
     args = parse()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus %d is not supported (the forward path shards by sample "
-              "with no exchange, see DESIGN.md)" % args.gpus, file=sys.stderr)
+              "with no exchange between the GPUs)" % args.gpus, file=sys.stderr)
         sys.exit(2)
     # the host classes announce every layer on stdout like the reference does;
     # keep stdout for the one JSON line and send that chatter to stderr
