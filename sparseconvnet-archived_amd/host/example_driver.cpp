@@ -107,8 +107,19 @@ int main(int argc, char **argv) {
     small.processDataset(trainSet, 100, 0.003 * exp(-0.01 * epoch));
   }
   float after = small.processDataset(validationSet, 100);
+  // a net with fractional max-pooling: every pass draws new pooling regions,
+  // so two passes over the same pictures give slightly different costs
+  POFMPSparseConvNet fmp(2, 5, 8, 1.5f, VLEAKYRELU, trainSet.nFeatures,
+                         trainSet.nClasses);
+  float fmp1 = fmp.processDataset(validationSet, 100);
+  float fmp2 = fmp.processDataset(validationSet, 100);
   for (auto *p : trainSet.pictures)
     delete p;
+  if (!(fmp1 > 0 && fmp2 > 0 && fmp1 < 50 && fmp2 < 50)) {
+    std::cout << "fractional max-pooling net: NLL " << fmp1 << " " << fmp2
+              << std::endl;
+    return 1;
+  }
   if (!(after < 0.5f * before)) {
     std::cout << "training did not lower the cost: " << before << " -> "
               << after << std::endl;
