@@ -162,22 +162,35 @@ __global__ __launch_bounds__(256) void k_gemm_atb(
   floatx4 acc[4];
   for (int i = 0; i < 4; ++i)
     acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+  // the next chunk's loads are in flight under this chunk's MFMAs
+  float ra[ATB_ROWS / 4], rd[ATB_ROWS / 4];
+  auto fetch = [&](long long m) {
+#pragma unroll
+    for (int i = 0; i < ATB_ROWS / 4; ++i) {
+      const long long row = m + rg + 4 * i;
+      const bool live = row < m1;
+      ra[i] = live && aIn ? A[row * K + k0 + col] : 0.f;
+      rd[i] = live && dIn ? D[row * N + n0 + col] : 0.f;
+    }
+  };
+  fetch(m0);
   for (long long m = m0; m < m1; m += ATB_ROWS) {
+#pragma unroll
     for (int i = 0; i < ATB_ROWS / 4; ++i) {
       const int r = rg + 4 * i;
-      const long long row = m + r;
-      const bool live = row < m1;
-      sA[r * ATB_PITCH + col] = live && aIn ? A[row * K + k0 + col] : 0.f;
-      sD[r * ATB_PITCH + col] = live && dIn ? D[row * N + n0 + col] : 0.f;
+      sA[r * ATB_PITCH + col] = ra[i];
+      sD[r * ATB_PITCH + col] = rd[i];
     }
     __syncthreads();
+    if (m + ATB_ROWS < m1)
+      fetch(m + ATB_ROWS);
 #pragma unroll
     for (int s = 0; s < ATB_ROWS / 4; ++s) {
-      const float *ra = sA + (4 * s + q) * ATB_PITCH + c;
+      const float *pa = sA + (4 * s + q) * ATB_PITCH + c;
       const float b = sD[(4 * s + q) * ATB_PITCH + 16 * w + c];
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[16 * i], b, acc[i], 0,
+        acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[16 * i], b, acc[i], 0,
                                                       0, 0);
     }
     __syncthreads();
@@ -348,9 +361,10 @@ extern "C" int scn_sgemm_AtB(scn_ctx *ctx, const float *d_A, const float *d_D,
   if (M == 0)
     return SCN_OK;
   SCN_REQUIRE(d_A && d_D, SCN_ERR_ARG, "scn_sgemm_AtB: null buffer");
-  // (outputs of a few tiles only are bound by the atomics either way: the
-  // narrow kernel below does as well on them)
-  if (K % 4 == 0 && N % 4 == 0 && N >= 48 && M >= 1024 &&
+  // The wide tiles pay on long walks over the rows (measured: 200000 x 1728 x
+  // 64 and 100000 x 800 x 800 gain 20 %); up to some ten thousand rows, or with
+  // an output of a few tiles only, the narrow kernel's many short walks win.
+  if (K % 4 == 0 && N % 4 == 0 && N >= 48 && M >= 65536 &&
       ((long long)K * N >= 160 * 1024 || (K >= 1024 && N >= 64)) &&
       ((uintptr_t)d_A & 15) == 0 && ((uintptr_t)d_D & 15) == 0) {
     // 256 x 64 or 128 x 128 tiles: whichever pads the output less
