@@ -428,13 +428,17 @@ extern "C" int scn_sgemm_ABt(scn_ctx *ctx, const float *d_D, const float *d_W,
     return SCN_OK;
   SCN_REQUIRE(d_D && d_W && d_dA && d_workspace, SCN_ERR_ARG,
               "scn_sgemm_ABt: null buffer");
+  // the zero bias: the context's own zeros when they are enough of them
   float *Wt = d_workspace, *zeros = d_workspace + (size_t)N * K;
   {
     ProfScope prof(ctx, SCN_K_BACKWARD);
     hipLaunchKernelGGL(k_transpose, dim3(scn_ceil_div(N, 32), scn_ceil_div(K, 32)),
                        dim3(256), 0, ctx->stream, d_W, Wt, K, N);
     SCN_HIP_CHECK(hipGetLastError());
-    SCN_TRY(scn_fill32(ctx, zeros, 0, (size_t)K));
+    if (K <= SCN_ZERO_FLOATS)
+      zeros = ctx->d_zeros;
+    else
+      SCN_TRY(scn_fill32(ctx, zeros, 0, (size_t)K));
   }
   return scn_nin_forward(ctx, d_D, Wt, zeros, nullptr, d_dA, M, N, K, 1.0f,
                          SCN_NOSIGMOID, SCN_FP32);
@@ -494,11 +498,21 @@ __global__ __launch_bounds__(256) void k_gather_backward(
   if (e0 >= count)
     return;
   const long long e1 = e0 + SCATTER_RUN < count ? e0 + SCATTER_RUN : count;
+  // the run's rules and values are all requested before the first is used
+  int rl[SCATTER_RUN];
+#pragma unroll
+  for (int u = 0; u < SCATTER_RUN; ++u)
+    rl[u] = e0 + u < e1 ? rules[e0 + u] : -1;
   for (int j = li; j < nIn; j += P) {
+    float dv[SCATTER_RUN];
+#pragma unroll
+    for (int u = 0; u < SCATTER_RUN; ++u)
+      dv[u] = e0 + u < e1 ? dconv[(e0 + u) * nIn + j] : 0.f;
     int cur = -1;
     float acc = 0.f;
-    for (long long e = e0; e < e1; ++e) {
-      const int r = rules[e];
+#pragma unroll
+    for (int u = 0; u < SCATTER_RUN; ++u) {
+      const int r = rl[u];
       if (r < 0)
         continue;
       if (r != cur) {
@@ -507,7 +521,7 @@ __global__ __launch_bounds__(256) void k_gather_backward(
         cur = r;
         acc = 0.f;
       }
-      acc += dconv[e * nIn + j];
+      acc += dv[u];
     }
     if (cur >= 0)
       unsafeAtomicAdd(din + (long long)cur * nIn + j, acc);
@@ -559,17 +573,27 @@ __global__ __launch_bounds__(256) void k_maxpool_backward(
     return;
   const long long r1 = r0 + SCATTER_RUN < count ? r0 + SCATTER_RUN : count;
   for (int j = li; j < C; j += P) {
+    int tg[SCATTER_RUN];
+    float dv[SCATTER_RUN];
+#pragma unroll
+    for (int u = 0; u < SCATTER_RUN; ++u) {
+      const bool live = r0 + u < r1;
+      tg[u] = live ? choice[(r0 + u) * C + j] : -1;
+      dv[u] = live ? dout[(r0 + u) * C + j] : 0.f;
+    }
     int cur = -1;
     float acc = 0.f;
-    for (long long r = r0; r < r1; ++r) {
-      const int tgt = choice[r * C + j];
-      if (tgt != cur) {
+#pragma unroll
+    for (int u = 0; u < SCATTER_RUN; ++u) {
+      if (tg[u] < 0)
+        continue;
+      if (tg[u] != cur) {
         if (cur >= 0)
           unsafeAtomicAdd(din + cur, acc);
-        cur = tgt;
+        cur = tg[u];
         acc = 0.f;
       }
-      acc += dout[r * C + j];
+      acc += dv[u];
     }
     if (cur >= 0)
       unsafeAtomicAdd(din + cur, acc);
