@@ -13,6 +13,7 @@
 #include "SpatiallySparseLayer.h"
 
 #define N_MAX_BATCH_PRODUCER_THREADS 20
+#define N_PRODUCER_STREAMS 5
 
 // A batch whose input is already in HBM: active sites (sample, key, row),
 // backgroundCol per sample, and the feature matrix [nSpatialSites x
@@ -45,7 +46,19 @@ public:
   // upload and the rule-book kernels of its batch there, while the forward
   // pass of another batch runs on memStream (the reference declares the same
   // array, SparseConvNetCUDA.h:38, and leaves it unused)
+  // The streams the batch slots issue their grid and rule-book kernels on:
+  // at most N_PRODUCER_STREAMS of them, slot c uses stream c % their number
+  // (HIP spreads streams over four hardware queues; with more than five
+  // producer streams the forward pass's stream has to share its queue).  Two
+  // slots that share a stream take turns for the GPU half of batch production
+  // (batchStreamLocks); their CPU halves run side by side.
   std::vector<std::unique_ptr<cudaMemStream>> batchMemStreams;
+  std::vector<std::unique_ptr<std::mutex>> batchStreamLocks;
+  std::mutex &streamLockOfSlot(int slot) {
+    return *batchStreamLocks[slot % batchStreamLocks.size()];
+  }
+  // fewer producer threads than the net was constructed with
+  void limitBatchProducerThreads(int n);
   std::mutex batchLock[N_MAX_BATCH_PRODUCER_THREADS];
   std::vector<SpatiallySparseBatch> batchPool;
   std::vector<SpatiallySparseBatchSubInterface *> initialSubInterfaces;

@@ -27,12 +27,30 @@ SparseConvNetCUDA::SparseConvNetCUDA(int dimension, int nInputFeatures,
             << " nInputFeatures=" << nInputFeatures << " nClasses=" << nClasses
             << std::endl;
   batchPool.reserve(nBatchProducerThreads);
+  const int nStreams = std::min(nBatchProducerThreads, N_PRODUCER_STREAMS);
+  for (int c = 0; c < nStreams; c++) {
+    batchMemStreams.emplace_back(new cudaMemStream());
+    batchStreamLocks.emplace_back(new std::mutex());
+  }
   for (int c = 0; c < nBatchProducerThreads; c++) {
     initialSubInterfaces.push_back(new SpatiallySparseBatchSubInterface());
     batchPool.emplace_back(initialSubInterfaces.back());
-    batchMemStreams.emplace_back(new cudaMemStream());
-    batchPool.back().preprocessStream = batchMemStreams.back().get();
+    batchPool.back().preprocessStream = batchMemStreams[c % nStreams].get();
   }
+}
+void SparseConvNetCUDA::limitBatchProducerThreads(int n) {
+  if (n < 1 || n >= nBatchProducerThreads)
+    return;
+  nBatchProducerThreads = n;
+  while ((int)batchPool.size() > n)
+    batchPool.pop_back();
+  const int nStreams = std::min(n, N_PRODUCER_STREAMS);
+  while ((int)batchMemStreams.size() > nStreams) {
+    batchMemStreams.pop_back();
+    batchStreamLocks.pop_back();
+  }
+  for (int c = 0; c < n; c++)
+    batchPool[c].preprocessStream = batchMemStreams[c % nStreams].get();
 }
 SparseConvNetCUDA::~SparseConvNetCUDA() {
   for (auto &s : batchMemStreams)
@@ -695,10 +713,12 @@ void BatchProducer::batchProducerThread(int nThread) {
     {
       std::lock_guard<std::mutex> slot(cnn.batchLock[nThread]);
       if (resident) {
+        std::lock_guard<std::mutex> stream(cnn.streamLockOfSlot(nThread));
         cnn.preprocessResident(nThread, *resident);
       } else {
-        preprocessBatch(c, nThread, rng);
-        preprocessBatchOnDevice(nThread);
+        preprocessBatch(c, nThread, rng); // CPU half
+        std::lock_guard<std::mutex> stream(cnn.streamLockOfSlot(nThread));
+        preprocessBatchOnDevice(nThread); // GPU half, on the slot's stream
       }
     }
     {

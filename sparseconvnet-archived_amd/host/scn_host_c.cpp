@@ -45,14 +45,7 @@ scnh_net *scnh_net_create(int dimension, int nInputFeatures, int nClasses,
   }
   // the thread count is fixed at construction in the reference (default 10);
   // a smaller pool is allowed here because every slot owns device tables
-  if (nBatchProducerThreads >= 1 &&
-      nBatchProducerThreads < n->cnn->nBatchProducerThreads) {
-    n->cnn->nBatchProducerThreads = nBatchProducerThreads;
-    while ((int)n->cnn->batchPool.size() > nBatchProducerThreads) {
-      n->cnn->batchPool.pop_back();
-      n->cnn->batchMemStreams.pop_back();
-    }
-  }
+  n->cnn->limitBatchProducerThreads(nBatchProducerThreads);
   return n;
 }
 void scnh_net_destroy(scnh_net *net) {

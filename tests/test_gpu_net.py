@@ -207,7 +207,7 @@ def test_fused_convolutions_change_no_bit(scn, precision):
         assert skipped == 0
 
 
-@pytest.mark.parametrize("threads", [1, 3])
+@pytest.mark.parametrize("threads", [1, 3, 8])
 def test_batches_of_changing_size_through_one_slot(scn, threads):
     """Rule books are planned with counts deferred and sized by what the slot
     has seen before: sparse batches, then one several times denser (outgrows
@@ -390,3 +390,31 @@ def test_reference_style_cpp_driver(scn):
     print(out.stdout[-1500:], out.stderr[-500:], flush=True)
     assert out.returncode == 0
     assert "example driver ok" in out.stdout and "rate:" in out.stdout
+
+
+def test_ten_producer_threads_share_five_streams(scn):
+    """The reference's default of 10 batch-producer threads: the slots share five streams for the GPU half of batch
+    production.  Thirty batches of changing size give, sample for sample, what one producer thread gives."""
+    from sparseconvnet_archived_amd import hostapi, synthetic
+    cfg = synthetic.config(2, batch=7)
+    samples = synthetic.make_samples(cfg, 77, batch=7 * 30 - 3)
+    results = []
+    for threads in (1, 10):
+        net = hostapi.Net(cfg.dimension, cfg.nInputFeatures, cfg.nClasses, nTop=1, threads=threads)
+        cfg.build(net)
+        net.setFusedConvolutions(True)
+        for i, (W, B, pr) in synthetic.he_normal_weights(net.layers(), 78).items():
+            net.set_weights(i, W, B, pr)
+        ds = hostapi.Dataset("many", 3, 100, hostapi.TESTBATCH)
+        for pts, f, label in samples:
+            ds.add_points(2, cfg.lattice, pts, f, label)
+        probs = []
+        net.begin(ds, 7)
+        while net.next_batch():
+            out = net.batch_outputs()
+            assert out["sampleNumbers"].tolist() == list(range(len(probs), len(probs) + out["batchSize"]))
+            probs.extend(out["probabilities"])
+        net.close()
+        results.append(np.array(probs))
+    assert results[0].shape == (len(samples), 100)
+    assert np.array_equal(results[0], results[1])
