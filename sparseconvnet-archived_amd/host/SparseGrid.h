@@ -22,16 +22,18 @@ public:
   SparseGridMap() : live_(0), sorted_(true) {}
 
   int &operator[](int64_t key) {
-    int at = lookup(key);
+    size_t slot = 0;
+    int at = lookup(key, &slot);
     if (at < 0)
-      at = append(key, 0);
+      at = append(key, 0, slot);
     return entries_[at].second;
   }
   std::pair<iterator, bool> insert(const value_type &kv) {
-    int at = lookup(kv.first);
+    size_t slot = 0;
+    int at = lookup(kv.first, &slot);
     bool fresh = at < 0;
     if (fresh)
-      at = append(kv.first, kv.second);
+      at = append(kv.first, kv.second, slot);
     return std::make_pair(entries_.begin() + at, fresh);
   }
   iterator find(int64_t key) {
@@ -50,6 +52,18 @@ public:
     reindex();
   }
   size_t size() const { return entries_.size(); }
+  // room for n sites without growing on the way (optional)
+  void reserve(size_t n) {
+    entries_.reserve(n);
+    size_t cap = 16;
+    while (cap < 2 * n + 2)
+      cap *= 2;
+    if (cap > index_.size()) {
+      index_.assign(cap, -1);
+      for (size_t i = 0; i < entries_.size(); ++i)
+        place((int)i);
+    }
+  }
   void clear() {
     entries_.clear();
     index_.clear();
@@ -68,14 +82,18 @@ private:
     uint64_t x = (uint64_t)k * 0x9E3779B97F4A7C15ull;
     return (size_t)(x ^ (x >> 29));
   }
-  int lookup(int64_t key) const {
+  // the entry of `key`, or -1 and (if asked) the empty slot its probe ended at
+  int lookup(int64_t key, size_t *emptySlot = nullptr) const {
     if (index_.empty())
       return -1;
     size_t mask = index_.size() - 1, s = mix(key) & mask;
     for (;;) {
       int at = index_[s];
-      if (at < 0)
+      if (at < 0) {
+        if (emptySlot)
+          *emptySlot = s;
         return -1;
+      }
       if (entries_[at].first == key)
         return at;
       s = (s + 1) & mask;
@@ -95,14 +113,15 @@ private:
     for (size_t i = 0; i < entries_.size(); ++i)
       place((int)i);
   }
-  int append(int64_t key, int row) {
+  // slot: where lookup(key) gave up (valid unless the index has to grow)
+  int append(int64_t key, int row, size_t slot) {
     if (!entries_.empty() && key < entries_.back().first)
       sorted_ = false;
     entries_.push_back(value_type(key, row));
     if (index_.size() < 2 * entries_.size() + 2)
       reindex();
     else
-      place((int)entries_.size() - 1);
+      index_[slot] = (int)entries_.size() - 1;
     return (int)entries_.size() - 1;
   }
   void order() {

@@ -388,6 +388,7 @@ void SparsePointsPicture::codifyInputData(SparseGrid &grid,
   grid.backgroundCol = nSpatialSites++;
   const int shift = (spatialSize - latticeSize) / 2;
   const size_t nSites = coords.size() / dimension;
+  grid.mp.reserve(nSites);
   for (size_t s = 0; s < nSites; ++s) {
     int64_t key = 0;
     bool inside = true;
@@ -396,9 +397,10 @@ void SparsePointsPicture::codifyInputData(SparseGrid &grid,
       inside = inside && c >= 0 && c < spatialSize;
       key = key * spatialSize + c;
     }
-    if (!inside || grid.mp.find(key) != grid.mp.end())
+    // the first point of a site makes its row; later ones change nothing
+    if (!inside || !grid.mp.insert(std::make_pair(key, nSpatialSites)).second)
       continue;
-    grid.mp[key] = nSpatialSites++;
+    nSpatialSites++;
     out.insert(out.end(), features.begin() + s * nFeatures,
                features.begin() + (s + 1) * nFeatures);
   }
