@@ -190,13 +190,17 @@ def test_fused_convolutions_change_no_bit(scn, precision):
         net.begin(ds, len(samples))
         assert net.next_batch()
         ifaces = [net.interface(i) for i in range(len(net.layers()) + 1)]
+        hostapi_layers = net.layers()
         runs.append((ifaces, net.batch_outputs()))
         net.end()
         net.close()
     (plain, out0), (fusedrun, out1) = runs
     skipped = 0
-    for a, b in zip(plain, fusedrun):
-        assert np.array_equal(a["rules"], b["rules"]) and np.array_equal(a["choices"], b["choices"])
+    kinds = [None] + [l["kind"] for l in hostapi_layers]
+    for i, (a, b) in enumerate(zip(plain, fusedrun)):
+        assert np.array_equal(a["rules"], b["rules"])
+        if kinds[i] and kinds[i].startswith("maxpool"):  # (other layers size the choices buffer but never write it)
+            assert np.array_equal(a["choices"], b["choices"])
         if b["features"] is None:
             skipped += 1
             continue
