@@ -186,3 +186,34 @@ def test_dropout_sub_matrix_and_its_update(scn, ctx):
     d_b = ctx.empty(3, np.float32)
     scn._check(scn.lib().scn_shrink_matrix(ctx.h, ctx.array(B).ptr, d_b.ptr, None, ctx.array(outP).ptr, 64, 1, 3))
     assert np.array_equal(d_b.download(), B[outP])
+
+
+def test_empty_inputs_and_bad_arguments(scn, ctx):
+    """M = 0 is legal everywhere (gradients of nothing are zero); null buffers and bad sizes are refused."""
+    K, N = 8, 16
+    one = ctx.array(np.ones(4, np.float32))
+    d_db = ctx.array(np.full(N, 5, np.float32))
+    ctx.activation_backward(one, one, 0, N, scn.RELU, None, d_db, None)
+    assert not d_db.download().any()
+    d_dW = ctx.array(np.full((K, N), 5, np.float32))
+    ctx.sgemm_AtB(one, one, d_dW, 0, K, N)
+    assert not d_dW.download().any()
+    ws = ctx.empty(scn.lib().scn_sgemm_ABt_workspace(N, K), np.float32)
+    ctx.sgemm_ABt(one, one, one, 0, N, K, ws)
+    ctx.softmax_grad(one, ctx.array(np.zeros(1, np.int32)), one, 0, 4)
+    ctx.gather_rows_backward(one, one, ctx.array(np.zeros(1, np.int32)), 0, 4)
+    ctx.maxpool_backward(one, one, 0, 4, ctx.array(np.zeros(1, np.int32)))
+    ctx.terminal_pool_backward(one, one, ctx.array(np.zeros(1, np.int32)), 0, 4, 1)
+    ctx.nag_update(one, one, one, 0, 0.1, 0.9)
+    assert ctx.sum_abs(one, 0) == 0.0 and ctx.sum_abs(one, 4) == 4.0
+    ctx.scale(one, 4, 0.5)
+    assert one.download().tolist() == [0.5] * 4
+    L = scn.lib()
+    assert L.scn_activation_backward(ctx.h, one.ptr, one.ptr, 1, 4, 99, None, one.ptr, None) == scn.ERR_ARG
+    assert L.scn_activation_backward(ctx.h, one.ptr, one.ptr, 1, 4, scn.PRELU, None, one.ptr, None) == scn.ERR_ARG
+    assert L.scn_sgemm_AtB(ctx.h, None, one.ptr, one.ptr, 4, 1, 1) == scn.ERR_ARG
+    assert L.scn_sgemm_ABt(ctx.h, one.ptr, one.ptr, one.ptr, 4, 1, 1, None) == scn.ERR_ARG
+    assert L.scn_nag_update(ctx.h, one.ptr, None, one.ptr, 4, 0.1, 0.9, 0) == scn.ERR_ARG
+    assert L.scn_gather_rows_backward(ctx.h, one.ptr, one.ptr, None, 4, 1) == scn.ERR_ARG
+    assert L.scn_terminal_pool_backward(ctx.h, one.ptr, one.ptr, one.ptr, 1, 4, 0) == scn.ERR_ARG
+    assert b"scn_terminal_pool_backward" in L.scn_last_error()

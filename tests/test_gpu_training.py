@@ -259,3 +259,22 @@ def test_rescale_batches(scn):
     print("feature scales of the hidden layers, first pass:", first, "third pass:", last, flush=True)
     assert np.all(np.abs(np.log(last)) <= np.abs(np.log(first)) + 1e-3)
     net.close()
+
+
+def test_train_config4_wide_layers(scn):
+    """The wide net (contractions of 640..3200 by 160..800): other kernels serve the backward products here."""
+    from sparseconvnet_archived_amd import synthetic
+    cfg = synthetic.config(4, batch=3)
+    train_and_compare(scn, cfg, synthetic.make_samples(cfg, 304), 1)
+
+
+def test_train_batch_of_one_and_empty_sample(scn):
+    """Edge cases: a batch of one sample, then a batch whose second sample has no active site at all."""
+    from sparseconvnet_archived_amd import synthetic
+    cfg = synthetic.config(2, batch=1)
+    train_and_compare(scn, cfg, synthetic.make_samples(cfg, 305), 1)
+    cfg = synthetic.config(2, batch=3)
+    samples = synthetic.make_samples(cfg, 306)
+    pts, f, label = samples[1]
+    samples[1] = (pts[:0], f[:0], label)
+    train_and_compare(scn, cfg, samples, 1)
