@@ -49,60 +49,75 @@ extern "C" int scn_softmax_grad(scn_ctx *ctx, const float *d_probs,
 // One pass over the [M x N] gradient: multiplies it in place by the
 // derivative of the activation (expressed through the layer's output, as the
 // reference does), and leaves the column sums of the result in db (the bias
-// gradient) and, for PReLU, the slope gradient in dprelu.  Lane = column,
-// the four wavefronts of a workgroup interleave rows.
+// gradient) and, for PReLU, the slope gradient in dprelu.  A workgroup covers
+// P columns (the power of two that covers min(N, 64)) with 256 / P lanes per
+// column, which interleave rows and take four of them per trip so that eight
+// loads are in flight per lane.
+__device__ __forceinline__ float act_derivative(int act, float b, float d,
+                                                float alpha, float &t) {
+  switch (act) {
+  case SCN_RELU:
+    return b > 0 ? d : 0.f;
+  case SCN_LEAKYRELU:
+  case SCN_VLEAKYRELU:
+    return b > 0 ? d : d * alpha;
+  case SCN_TANH:
+    return d * (1 + b) * (1 - b);
+  case SCN_SIGMOID:
+    return d * b * (1 - b);
+  case SCN_PRELU:
+    t += d * (b > 0 ? 0.f : b / alpha);
+    return b > 0 ? d : d * alpha;
+  default: // SOFTMAX (folded into the classifier's gradient), NOSIGMOID
+    return d;
+  }
+}
 __global__ __launch_bounds__(256) void k_act_backward(
     const float *__restrict__ out, float *__restrict__ delta, long long M,
     int N, int act, const float *__restrict__ prelu, float *__restrict__ db,
-    float *__restrict__ dprelu) {
-  __shared__ float sS[4][64], sT[4][64];
-  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-  const int c = blockIdx.x * 64 + tx;
+    float *__restrict__ dprelu, int P) {
+  __shared__ float sS[256], sT[256];
+  const int tx = threadIdx.x % P, ty = threadIdx.x / P, lanesPerCol = 256 / P;
+  const int c = blockIdx.x * P + tx;
   float s = 0.f, t = 0.f;
   if (c < N) {
     const float alpha = act == SCN_PRELU      ? prelu[c]
                         : act == SCN_LEAKYRELU ? 0.01f
                                                : 0.333f;
-    for (long long r = (long long)blockIdx.y * 4 + ty; r < M;
-         r += 4ll * gridDim.y) {
-      const long long i = r * N + c;
-      const float b = out[i];
-      float d = delta[i];
-      switch (act) {
-      case SCN_RELU:
-        d = b > 0 ? d : 0.f;
-        break;
-      case SCN_LEAKYRELU:
-      case SCN_VLEAKYRELU:
-        d = b > 0 ? d : d * alpha;
-        break;
-      case SCN_TANH:
-        d = d * (1 + b) * (1 - b);
-        break;
-      case SCN_SIGMOID:
-        d = d * b * (1 - b);
-        break;
-      case SCN_PRELU:
-        t += d * (b > 0 ? 0.f : b / alpha);
-        d = b > 0 ? d : d * alpha;
-        break;
-      default: // SOFTMAX (folded into the classifier's gradient), NOSIGMOID
-        break;
+    const long long step = (long long)lanesPerCol * gridDim.y;
+    long long r = (long long)blockIdx.y * lanesPerCol + ty;
+    for (; r + 3 * step < M; r += 4 * step) {
+      float b[4], d[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        b[u] = out[(r + u * step) * N + c];
+        d[u] = delta[(r + u * step) * N + c];
       }
-      delta[i] = d;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        d[u] = act_derivative(act, b[u], d[u], alpha, t);
+        delta[(r + u * step) * N + c] = d[u];
+        s += d[u];
+      }
+    }
+    for (; r < M; r += step) {
+      const float d = act_derivative(act, out[r * N + c], delta[r * N + c], alpha, t);
+      delta[r * N + c] = d;
       s += d;
     }
   }
-  sS[ty][tx] = s;
-  sT[ty][tx] = t;
+  sS[threadIdx.x] = s;
+  sT[threadIdx.x] = t;
   __syncthreads();
   if (ty == 0 && c < N) {
-    s = sS[0][tx] + sS[1][tx] + sS[2][tx] + sS[3][tx];
-    unsafeAtomicAdd(db + c, s);
-    if (act == SCN_PRELU) {
-      t = sT[0][tx] + sT[1][tx] + sT[2][tx] + sT[3][tx];
-      unsafeAtomicAdd(dprelu + c, t);
+    s = 0.f, t = 0.f;
+    for (int k = 0; k < lanesPerCol; ++k) {
+      s += sS[k * P + tx];
+      t += sT[k * P + tx];
     }
+    unsafeAtomicAdd(db + c, s);
+    if (act == SCN_PRELU)
+      unsafeAtomicAdd(dprelu + c, t);
   }
 }
 
@@ -126,14 +141,23 @@ extern "C" int scn_activation_backward(scn_ctx *ctx, const float *d_out,
     return SCN_OK;
   SCN_REQUIRE(d_out && d_delta, SCN_ERR_ARG,
               "scn_activation_backward: null buffer");
-  int colBlocks = scn_ceil_div(N, 64);
-  int rowBlocks = scn_ceil_div(M, 64); // at least 16 rows per wavefront
-  int cap = (ctx->numCU * 8 + colBlocks - 1) / colBlocks;
+  int P = 1;
+  while (P < N && P < 64)
+    P <<= 1;
+  const int lanesPerCol = 256 / P;
+  int colBlocks = scn_ceil_div(N, P);
+  // every workgroup ends with one atomic per column onto the same N
+  // addresses, and those serialise (about 25 ns each): few, long-lived
+  // workgroups, two per compute unit
+  int rowBlocks = scn_ceil_div(M, 8 * lanesPerCol); // at least eight rows per lane
+  int cap = (ctx->numCU * 2 + colBlocks - 1) / colBlocks;
   if (rowBlocks > cap)
     rowBlocks = cap;
+  if (rowBlocks < 1)
+    rowBlocks = 1;
   hipLaunchKernelGGL(k_act_backward, dim3(colBlocks, rowBlocks), dim3(256), 0,
                      ctx->stream, d_out, d_delta, (long long)M, N, act,
-                     d_prelu, d_db, d_dprelu);
+                     d_prelu, d_db, d_dprelu, P);
   SCN_HIP_CHECK(hipGetLastError());
   return SCN_OK;
 }
