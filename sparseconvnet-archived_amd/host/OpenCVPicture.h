@@ -72,3 +72,6 @@ int loadMnist(const char *imagesFile, const char *labelsFile,
 // CIFAR-10 binary batches (SpatiallySparseDatasetCIFAR10.cpp:6-28): 32 x 32
 // pictures of 3 channels stored blue, green, red, background 128.
 int readCIFAR10File(std::vector<Picture *> &characters, const char *filename);
+// CIFAR-100 (SpatiallySparseDatasetCIFAR100.cpp:6-29): a coarse and a fine
+// label byte per record, the fine one is the class.
+int readCIFAR100File(std::vector<Picture *> &characters, const char *filename);

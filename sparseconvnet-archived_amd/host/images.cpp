@@ -124,13 +124,18 @@ int loadMnist(const char *imagesFile, const char *labelsFile,
   return n1;
 }
 
-int readCIFAR10File(std::vector<Picture *> &characters, const char *filename) {
+// A record is `labelBytes` label bytes, the last of which is the class, then
+// the three colour planes: CIFAR-10 has one label byte, CIFAR-100 a coarse
+// and a fine one (SpatiallySparseDatasetCIFAR100.cpp:13-15 keeps the fine).
+static int read_cifar_file(std::vector<Picture *> &characters,
+                           const char *filename, int labelBytes) {
   std::ifstream file(filename, std::ios::in | std::ios::binary);
   if (!file)
     return -1;
-  unsigned char label;
+  unsigned char labels[2];
   int added = 0;
-  while (file.read((char *)&label, 1)) {
+  while (file.read((char *)labels, labelBytes)) {
+    const unsigned char label = labels[labelBytes - 1];
     unsigned char bitmap[3072];
     if (!file.read((char *)bitmap, 3072))
       break; // a truncated record is dropped
@@ -144,4 +149,10 @@ int readCIFAR10File(std::vector<Picture *> &characters, const char *filename) {
     ++added;
   }
   return added;
+}
+int readCIFAR10File(std::vector<Picture *> &characters, const char *filename) {
+  return read_cifar_file(characters, filename, 1);
+}
+int readCIFAR100File(std::vector<Picture *> &characters, const char *filename) {
+  return read_cifar_file(characters, filename, 2);
 }

@@ -295,6 +295,11 @@ int64_t scnh_dataset_add_cifar10_file(scnh_dataset *ds, const char *path) {
     return -1;
   return readCIFAR10File(ds->ds.pictures, path);
 }
+int64_t scnh_dataset_add_cifar100_file(scnh_dataset *ds, const char *path) {
+  if (ds->ds.nFeatures != 3)
+    return -1;
+  return readCIFAR100File(ds->ds.pictures, path);
+}
 int64_t scnh_constant_speed(const double *xy, int nPoints, float density,
                             int multiplier, double *out, int64_t capacity) {
   if (nPoints <= 0)
@@ -335,6 +340,11 @@ int64_t scnh_codify_picture(scnh_dataset *ds, int64_t index, int spatialSize,
 }
 int64_t scnh_dataset_size(scnh_dataset *ds) {
   return (int64_t)ds->ds.pictures.size();
+}
+int scnh_dataset_label(scnh_dataset *ds, int64_t index) {
+  if (index < 0 || index >= (int64_t)ds->ds.pictures.size())
+    return -1;
+  return ds->ds.pictures[(size_t)index]->label;
 }
 
 float scnh_process_dataset(scnh_net *net, scnh_dataset *ds, int batchSize) {

@@ -57,6 +57,8 @@ void scnh_dataset_add_points(scnh_dataset *ds, int dimension, int latticeSize,
                              int64_t nSites, const int32_t *coords,
                              const float *features, int label);
 int64_t scnh_dataset_size(scnh_dataset *ds);
+/* Picture::label of picture `index` (-1 when there is no such picture) */
+int scnh_dataset_label(scnh_dataset *ds, int64_t index);
 /* OffSurfaceModelPicture (Off3DFormatPicture.h): from an OFF file (returns -1
  * when it cannot be read) or from arrays (points: nPoints x 3 doubles,
  * triangles: nTriangles x 3 vertex indices).  The dataset needs nFeatures 1. */
@@ -94,6 +96,7 @@ int scnh_dataset_add_image(scnh_dataset *ds, int xSize, int ySize, int channels,
 int64_t scnh_dataset_add_mnist_files(scnh_dataset *ds, const char *imagesPath,
                                      const char *labelsPath);
 int64_t scnh_dataset_add_cifar10_file(scnh_dataset *ds, const char *path);
+int64_t scnh_dataset_add_cifar100_file(scnh_dataset *ds, const char *path);
 /* constantSpeed (OnlineHandwritingPicture.cpp:27-53) of one stroke: returns the
  * number of points and, when that fits capacity, writes them to out. */
 int64_t scnh_constant_speed(const double *xy, int nPoints, float density,

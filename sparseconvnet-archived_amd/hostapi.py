@@ -53,6 +53,7 @@ def lib():
         "scnh_dataset_destroy": (None, [vp]),
         "scnh_dataset_add_points": (None, [vp, i32, i32, i64, vp, vp, i32]),
         "scnh_dataset_size": (i64, [vp]),
+        "scnh_dataset_label": (i32, [vp, i64]),
         "scnh_dataset_add_off_file": (i32, [vp, C.c_char_p, i32, i32]),
         "scnh_dataset_add_mesh": (None, [vp, i64, vp, i64, vp, i32, i32]),
         "scnh_dataset_add_strokes": (i32, [vp, i32, vp, vp, i32, i32, i32, i32]),
@@ -61,6 +62,7 @@ def lib():
         "scnh_dataset_add_image": (i32, [vp, i32, i32, i32, vp, i32, i32, i32]),
         "scnh_dataset_add_mnist_files": (i64, [vp, C.c_char_p, C.c_char_p]),
         "scnh_dataset_add_cifar10_file": (i64, [vp, C.c_char_p]),
+        "scnh_dataset_add_cifar100_file": (i64, [vp, C.c_char_p]),
         "scnh_codify_picture": (i64, [vp, i64, i32, i64, i64, vp, vp, vp, vp]),
         "scnh_process_dataset": (f32, [vp, vp, i32]),
         "scnh_add_lenet_layer_fmp": (i32, [vp, i32, i32, i32, i32, i32, f32, i32, f32, i32]),
@@ -159,6 +161,12 @@ class Dataset:
             raise IOError("%s: not a readable CIFAR-10 batch (or nFeatures != 3)" % path)
         return int(n)
 
+    def add_cifar100_file(self, path):
+        n = lib().scnh_dataset_add_cifar100_file(self.h, str(path).encode())
+        if n < 0:
+            raise IOError("%s: not a readable CIFAR-100 file (or nFeatures != 3)" % path)
+        return int(n)
+
     def add_pendigits_file(self, path, renderSize, encoding):
         """every character of a UCI pen-digits file; returns how many."""
         n = lib().scnh_dataset_add_pendigits_file(self.h, str(path).encode(), renderSize, encoding)
@@ -182,6 +190,9 @@ class Dataset:
 
     def __len__(self):
         return lib().scnh_dataset_size(self.h)
+
+    def label(self, index):
+        return lib().scnh_dataset_label(self.h, index)
 
     def close(self):
         if getattr(self, "h", None):

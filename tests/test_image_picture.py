@@ -132,6 +132,14 @@ def test_mnist_and_cifar_files(tmp_path):
     with pytest.raises(IOError):
         ds.add_cifar10_file(tmp_path / "batch.bin")  # three channels into one feature
     ds.close()
+    # CIFAR-100: a coarse and a fine label byte, the fine one is the class
+    (tmp_path / "c100.bin").write_bytes(b"".join(bytes([3, 40 + k]) + planes[k].tobytes() for k in range(2)))
+    ds = h.Dataset("cifar100", 3, 100)
+    assert ds.add_cifar100_file(tmp_path / "c100.bin") == 2
+    assert [ds.label(k) for k in range(2)] == [40, 41]
+    keys, rows, bg, feats = ds.codify(1, 36)
+    assert list(keys) == list(want[0]) and np.array_equal(feats, want[3])
+    ds.close()
 
 
 @pytest.mark.gpu
