@@ -1,5 +1,5 @@
-"""Net-level CPU oracle: the reference's layer builders and per-batch forward
-restated over the C oracle.  TEST INFRASTRUCTURE ONLY.
+"""Net-level CPU oracle: the reference's layer builders, per-batch forward pass and
+training step restated over the C oracle.  TEST INFRASTRUCTURE ONLY.
 
 Builders follow SparseConvNetCUDA.cu:50-111 (addLearntLayer rounding to 32,
 filterSize 1 adds no gather layer, poolSize 1 adds no pooling layer),
@@ -7,7 +7,10 @@ filterSize 1 adds no gather layer, poolSize 1 adds no pooling layer),
 convolution's minActiveInputs equal to the pool size) and :198-210 (spatial
 sizes worked out from the top).  forward() follows BatchProducer.cu:40-87
 (every layer's preprocess) and SparseConvNetCUDA.cu:227-247 (forwards loop,
-then SoftmaxClassifier).
+then SoftmaxClassifier); train_step() follows :247-252 and every layer's
+backwards().  What the reference draws from its clock-seeded RNG (dropout
+subsets, fractional max-pooling regions) is an argument here: parity unpinned
+for the draw itself, pinned for everything computed from it.
 """
 import numpy as np
 

@@ -1,5 +1,6 @@
 /*
- * CPU oracle for the spatially-sparse forward path.  TEST INFRASTRUCTURE ONLY:
+ * CPU oracle for the spatially-sparse forward path (and the training pass
+ * behind it).  TEST INFRASTRUCTURE ONLY:
  * the product never links this file.  See scn_oracle.h for the contract and
  * the reference citations of every entry point.
  *
@@ -23,7 +24,9 @@
  *                        (momentum 0 is plain gradient descent; w' = w + m' + mu (m' - m))
  * Parity unpinned (no reference vector can exist in this build): the row order
  * the reference gets from google::dense_hash_map iteration (its default map),
- * and cuBLAS sgemm's summation order.
+ * cuBLAS sgemm's and the atomics' summation order, and every draw of the
+ * reference's clock-seeded RNG (dropout subsets, fractional pooling regions,
+ * the order of training batches): those are arguments of the functions here.
  *
  * Dimension 4 is refused: the reference's own d == 4 NoMin loop starts axis 0
  * at outputL(0, i1) (Regions.cu:614) and writes outside its rule row.

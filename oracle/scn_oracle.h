@@ -1,5 +1,6 @@
 /*
- * CPU oracle for the spatially-sparse forward path.  TEST INFRASTRUCTURE ONLY.
+ * CPU oracle for the spatially-sparse forward path, and for the backward pass
+ * and weight update that follow it in a training batch.  TEST INFRASTRUCTURE ONLY.
  *
  * Nothing in the product (the HIP library, the C++ host classes, the Python
  * binding) may include, link or call anything declared here; only tests, the
