@@ -26,7 +26,7 @@ public:
   std::vector<Picture *> pictures;
   int nFeatures; // channels per site
   int nClasses;
-  batchType type; // TESTBATCH or UNLABELEDBATCH on the forward path
+  batchType type; // TRAINBATCH, TESTBATCH, UNLABELEDBATCH or RESCALEBATCH
 
   void summary();
   void shuffle();

@@ -9,7 +9,7 @@
 class SpatiallySparseBatchSubInterface {
 public:
   vectorCUDA<float> features;
-  vectorCUDA<float> dfeatures; // backward pass only; never filled here
+  vectorCUDA<float> dfeatures; // gradient of the cost, training batches only
   vectorCUDA<int> poolingChoices;
   SpatiallySparseBatchSubInterface();
   void reset();
@@ -19,7 +19,7 @@ class SpatiallySparseBatchInterface {
 public:
   SpatiallySparseBatchSubInterface *sub;
   int nFeatures;                   // features per spatial location
-  vectorCUDA<int> featuresPresent; // identity at test time
+  vectorCUDA<int> featuresPresent; // all of them, except under dropout in a training batch
   int nSpatialSites; // active rows of the whole batch, background rows included
   int spatialSize;
   bool backpropErrors;

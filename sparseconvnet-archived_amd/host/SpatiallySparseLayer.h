@@ -1,12 +1,13 @@
-// The layer interface and every layer class of the forward path.
+// The layer interface and every layer class.
 //
 // preprocess() builds the output interface's grids and rule book, forwards()
 // runs the feature kernels (SpatiallySparseLayer.h:6-27).  In the reference
 // preprocess() is CPU code run by batch-producer threads; here it issues the
 // rule-book kernels on the GPU.  backwards() propagates the gradient of the
 // cost from the output interface's dfeatures to the input's and, in layers
-// with weights, takes one momentum step (dropout during training is not
-// implemented: such a layer stops with a message).
+// with weights, takes one momentum step on the weights the batch used (all of
+// them, or with dropout the sub-matrix of the features present); scaleWeights()
+// is the per-layer step of a RESCALEBATCH pass.
 #pragma once
 #include <fstream>
 #include <iostream>
