@@ -1,10 +1,11 @@
 /*
  * libscn_hip.so -- C ABI of the MI355X (gfx950) implementation of
- * SparseConvNet's spatially-sparse forward path.
+ * SparseConvNet's spatially-sparse forward path, and of the backward pass
+ * and weight update that follow it in a training batch.
  *
  * The reference has no plugin interface; its seam is the set of free functions
- * that the layer classes' preprocess()/forwards() call with raw device
- * pointers and a stream.  Each entry point below names the reference function
+ * that the layer classes' preprocess()/forwards()/backwards() call with raw
+ * device pointers and a stream.  Each entry point below names the reference function
  * it stands in for (paths relative to the reference's SparseConvNet/ folder).
  *
  * Conventions
