@@ -5,7 +5,9 @@
 #include <fstream>
 #include <iostream>
 #include <memory>
+#include <condition_variable>
 #include <mutex>
+#include <set>
 #include <string>
 #include <vector>
 #include "SpatiallySparseBatch.h"
@@ -46,19 +48,26 @@ public:
   // upload and the rule-book kernels of its batch there, while the forward
   // pass of another batch runs on memStream (the reference declares the same
   // array, SparseConvNetCUDA.h:38, and leaves it unused)
-  // The streams the batch slots issue their grid and rule-book kernels on:
-  // at most N_PRODUCER_STREAMS of them, slot c uses stream c % their number
-  // (HIP spreads streams over four hardware queues; with more than five
-  // producer streams the forward pass's stream has to share its queue).  Two
-  // slots that share a stream take turns for the GPU half of batch production
-  // (batchStreamLocks); their CPU halves run side by side.
+  // The streams the batch slots issue their grid and rule-book kernels on: at
+  // most N_PRODUCER_STREAMS (HIP spreads streams over four hardware queues;
+  // with more than five producer streams the forward pass's stream has to
+  // share its queue).  A producer thread borrows one for the GPU half of batch
+  // production (acquireProducerStream: the waiting batch with the lowest
+  // number goes first, so the consumer's next batch is never behind a later
+  // one); the CPU halves of all threads run side by side.
   std::vector<std::unique_ptr<cudaMemStream>> batchMemStreams;
-  std::vector<std::unique_ptr<std::mutex>> batchStreamLocks;
-  std::mutex &streamLockOfSlot(int slot) {
-    return *batchStreamLocks[slot % batchStreamLocks.size()];
-  }
+  cudaMemStream *acquireProducerStream(int batchNumber);
+  void releaseProducerStream(cudaMemStream *stream);
   // fewer producer threads than the net was constructed with
   void limitBatchProducerThreads(int n);
+
+private:
+  std::mutex streamPoolMutex;
+  std::condition_variable streamPoolChanged;
+  std::vector<cudaMemStream *> freeProducerStreams;
+  std::multiset<int> waitingBatches;
+
+public:
   std::mutex batchLock[N_MAX_BATCH_PRODUCER_THREADS];
   std::vector<SpatiallySparseBatch> batchPool;
   std::vector<SpatiallySparseBatchSubInterface *> initialSubInterfaces;

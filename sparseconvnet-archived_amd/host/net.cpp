@@ -30,13 +30,33 @@ SparseConvNetCUDA::SparseConvNetCUDA(int dimension, int nInputFeatures,
   const int nStreams = std::min(nBatchProducerThreads, N_PRODUCER_STREAMS);
   for (int c = 0; c < nStreams; c++) {
     batchMemStreams.emplace_back(new cudaMemStream());
-    batchStreamLocks.emplace_back(new std::mutex());
+    freeProducerStreams.push_back(batchMemStreams.back().get());
   }
   for (int c = 0; c < nBatchProducerThreads; c++) {
     initialSubInterfaces.push_back(new SpatiallySparseBatchSubInterface());
     batchPool.emplace_back(initialSubInterfaces.back());
     batchPool.back().preprocessStream = batchMemStreams[c % nStreams].get();
   }
+}
+cudaMemStream *SparseConvNetCUDA::acquireProducerStream(int batchNumber) {
+  std::unique_lock<std::mutex> lock(streamPoolMutex);
+  auto mine = waitingBatches.insert(batchNumber);
+  streamPoolChanged.wait(lock, [&] {
+    return !freeProducerStreams.empty() && *waitingBatches.begin() == batchNumber;
+  });
+  waitingBatches.erase(mine);
+  cudaMemStream *s = freeProducerStreams.front(); // the longest idle one
+  freeProducerStreams.erase(freeProducerStreams.begin());
+  if (!freeProducerStreams.empty() && !waitingBatches.empty())
+    streamPoolChanged.notify_all(); // the next waiter may go too
+  return s;
+}
+void SparseConvNetCUDA::releaseProducerStream(cudaMemStream *stream) {
+  {
+    std::lock_guard<std::mutex> lock(streamPoolMutex);
+    freeProducerStreams.push_back(stream);
+  }
+  streamPoolChanged.notify_all();
 }
 void SparseConvNetCUDA::limitBatchProducerThreads(int n) {
   if (n < 1 || n >= nBatchProducerThreads)
@@ -45,10 +65,11 @@ void SparseConvNetCUDA::limitBatchProducerThreads(int n) {
   while ((int)batchPool.size() > n)
     batchPool.pop_back();
   const int nStreams = std::min(n, N_PRODUCER_STREAMS);
-  while ((int)batchMemStreams.size() > nStreams) {
+  while ((int)batchMemStreams.size() > nStreams)
     batchMemStreams.pop_back();
-    batchStreamLocks.pop_back();
-  }
+  freeProducerStreams.clear();
+  for (auto &s : batchMemStreams)
+    freeProducerStreams.push_back(s.get());
   for (int c = 0; c < n; c++)
     batchPool[c].preprocessStream = batchMemStreams[c % nStreams].get();
 }
@@ -712,14 +733,16 @@ void BatchProducer::batchProducerThread(int nThread) {
     }
     {
       std::lock_guard<std::mutex> slot(cnn.batchLock[nThread]);
-      if (resident) {
-        std::lock_guard<std::mutex> stream(cnn.streamLockOfSlot(nThread));
-        cnn.preprocessResident(nThread, *resident);
-      } else {
+      if (!resident)
         preprocessBatch(c, nThread, rng); // CPU half
-        std::lock_guard<std::mutex> stream(cnn.streamLockOfSlot(nThread));
-        preprocessBatchOnDevice(nThread); // GPU half, on the slot's stream
-      }
+      // GPU half, on a stream borrowed for it
+      cudaMemStream *stream = cnn.acquireProducerStream(c);
+      cnn.batchPool[nThread].preprocessStream = stream;
+      if (resident)
+        cnn.preprocessResident(nThread, *resident);
+      else
+        preprocessBatchOnDevice(nThread);
+      cnn.releaseProducerStream(stream);
     }
     {
       std::lock_guard<std::mutex> lock(slotMutex);
