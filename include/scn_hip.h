@@ -279,6 +279,32 @@ int scn_sgemm_ABt(scn_ctx *ctx, const float *d_D, const float *d_W,
 int scn_nag_update(scn_ctx *ctx, const float *d_delta, float *d_momentum,
                    float *d_weights, int64_t n, float learningRate,
                    float momentum, int keepPositive);
+/* The same step on up to SCN_NAG_MAX tensors in one launch (what backwards()
+ * applies to W, B and the PReLU slopes one after the other,
+ * NetworkInNetworkLayer.cu:274-287, NetworkInNetworkPReLULayer.cu:211-214 and
+ * :262-275).  With clearGradients the gradients are left zero, which is what
+ * the accumulating products below expect of the next batch. */
+#define SCN_NAG_MAX 4
+typedef struct scn_nag_item {
+  float *d_delta;
+  float *d_momentum;
+  float *d_weights;
+  int64_t n;
+  int keepPositive;
+} scn_nag_item;
+int scn_nag_update_many(scn_ctx *ctx, const scn_nag_item *items, int nItems,
+                        float learningRate, float momentum,
+                        int clearGradients);
+/* scn_activation_backward and scn_sgemm_AtB with beta 1: they add to d_db,
+ * d_dprelu and d_dW instead of overwriting them (the reference's products are
+ * all beta 0; a caller that keeps its gradient buffers zero between batches,
+ * as scn_nag_update_many leaves them, saves the clearing launches). */
+int scn_activation_backward_acc(scn_ctx *ctx, const float *d_out,
+                                float *d_delta, int64_t M, int N, int act,
+                                const float *d_prelu, float *d_db,
+                                float *d_dprelu);
+int scn_sgemm_AtB_acc(scn_ctx *ctx, const float *d_A, const float *d_D,
+                      float *d_dW, int64_t M, int K, int N);
 /* Dropout during training.  dShrinkMatrixForDropout / dShrinkVectorForDropout
  * (NetworkInNetworkLayer.cu:7-25): w[i][j] = W[inPresent[i]][outPresent[j]],
  * W with rows of nOut floats; a null d_inPresent keeps the rows (row i of w

@@ -29,6 +29,15 @@ class ScnError(RuntimeError):
     pass
 
 
+NAG_MAX = 4
+
+
+class NagItem(C.Structure):
+    """scn_nag_item of the C header."""
+    _fields_ = [("d_delta", C.c_void_p), ("d_momentum", C.c_void_p), ("d_weights", C.c_void_p),
+                ("n", C.c_int64), ("keepPositive", C.c_int)]
+
+
 def build(force=True):
     """Compile the HIP library for gfx950 (works without a GPU)."""
     args = ["make", "-C", os.path.join(_HERE, "csrc"), "-s", "-j8"]
@@ -109,6 +118,9 @@ def lib():
         "scn_sgemm_ABt_workspace": (i64, [C.c_int, C.c_int]),
         "scn_sgemm_ABt": (C.c_int, [vp, vp, vp, vp, i64, C.c_int, C.c_int, vp]),
         "scn_nag_update": (C.c_int, [vp, vp, vp, vp, i64, f32, f32, C.c_int]),
+        "scn_nag_update_many": (C.c_int, [vp, P(NagItem), C.c_int, f32, f32, C.c_int]),
+        "scn_activation_backward_acc": (C.c_int, [vp, vp, vp, i64, C.c_int, C.c_int, vp, vp, vp]),
+        "scn_sgemm_AtB_acc": (C.c_int, [vp, vp, vp, vp, i64, C.c_int, C.c_int]),
         "scn_shrink_matrix": (C.c_int, [vp, vp, vp, vp, vp, C.c_int, C.c_int, C.c_int]),
         "scn_nag_update_shrunk": (C.c_int, [vp, vp, vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, f32, f32]),
         "scn_sum_abs": (C.c_int, [vp, vp, i64, P(C.c_double)]),
@@ -262,13 +274,22 @@ class Context:
     def softmax_grad(self, d_probs, d_labels, d_delta, batch, N):
         _check(lib().scn_softmax_grad(self.h, d_probs.ptr, d_labels.ptr, d_delta.ptr, batch, N))
 
-    def activation_backward(self, d_out, d_delta, M, N, act, d_prelu, d_db, d_dprelu):
-        _check(lib().scn_activation_backward(self.h, d_out.ptr, d_delta.ptr, M, N, act,
-                                             d_prelu.ptr if d_prelu is not None else None, d_db.ptr,
-                                             d_dprelu.ptr if d_dprelu is not None else None))
+    def activation_backward(self, d_out, d_delta, M, N, act, d_prelu, d_db, d_dprelu, accumulate=False):
+        f = lib().scn_activation_backward_acc if accumulate else lib().scn_activation_backward
+        _check(f(self.h, d_out.ptr, d_delta.ptr, M, N, act,
+                 d_prelu.ptr if d_prelu is not None else None, d_db.ptr,
+                 d_dprelu.ptr if d_dprelu is not None else None))
 
-    def sgemm_AtB(self, d_A, d_D, d_dW, M, K, N):
-        _check(lib().scn_sgemm_AtB(self.h, d_A.ptr, d_D.ptr, d_dW.ptr, M, K, N))
+    def sgemm_AtB(self, d_A, d_D, d_dW, M, K, N, accumulate=False):
+        f = lib().scn_sgemm_AtB_acc if accumulate else lib().scn_sgemm_AtB
+        _check(f(self.h, d_A.ptr, d_D.ptr, d_dW.ptr, M, K, N))
+
+    def nag_update_many(self, items, learningRate, momentum, clearGradients=False):
+        """items: (d_delta, d_momentum, d_weights, n, keepPositive) tuples, at most NAG_MAX of them."""
+        arr = (NagItem * max(1, len(items)))()
+        for k, (d, m, w, n, kp) in enumerate(items):
+            arr[k] = NagItem(d.ptr, m.ptr, w.ptr, n, int(kp))
+        _check(lib().scn_nag_update_many(self.h, arr, len(items), learningRate, momentum, int(clearGradients)))
 
     def sgemm_ABt(self, d_D, d_W, d_dA, M, N, K, d_workspace):
         assert d_workspace.size >= lib().scn_sgemm_ABt_workspace(N, K)

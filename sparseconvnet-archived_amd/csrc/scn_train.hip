@@ -121,10 +121,10 @@ __global__ __launch_bounds__(256) void k_act_backward(
   }
 }
 
-extern "C" int scn_activation_backward(scn_ctx *ctx, const float *d_out,
-                                       float *d_delta, int64_t M, int N,
-                                       int act, const float *d_prelu,
-                                       float *d_db, float *d_dprelu) {
+static int activation_backward(scn_ctx *ctx, const float *d_out,
+                               float *d_delta, int64_t M, int N, int act,
+                               const float *d_prelu, float *d_db,
+                               float *d_dprelu, bool clear) {
   SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_activation_backward: null context");
   SCN_REQUIRE(M >= 0 && N >= 1, SCN_ERR_ARG,
               "scn_activation_backward: M %lld N %d", (long long)M, N);
@@ -134,9 +134,11 @@ extern "C" int scn_activation_backward(scn_ctx *ctx, const float *d_out,
   SCN_REQUIRE(act != SCN_PRELU || (d_prelu && d_dprelu), SCN_ERR_ARG,
               "scn_activation_backward: PReLU needs slopes and their gradient");
   ProfScope prof(ctx, SCN_K_BACKWARD);
-  SCN_TRY(scn_fill32(ctx, d_db, 0, (size_t)N));
-  if (act == SCN_PRELU)
-    SCN_TRY(scn_fill32(ctx, d_dprelu, 0, (size_t)N));
+  if (clear) {
+    SCN_TRY(scn_fill32(ctx, d_db, 0, (size_t)N));
+    if (act == SCN_PRELU)
+      SCN_TRY(scn_fill32(ctx, d_dprelu, 0, (size_t)N));
+  }
   if (M == 0)
     return SCN_OK;
   SCN_REQUIRE(d_out && d_delta, SCN_ERR_ARG,
@@ -160,6 +162,22 @@ extern "C" int scn_activation_backward(scn_ctx *ctx, const float *d_out,
                      d_prelu, d_db, d_dprelu, P);
   SCN_HIP_CHECK(hipGetLastError());
   return SCN_OK;
+}
+
+extern "C" int scn_activation_backward(scn_ctx *ctx, const float *d_out,
+                                       float *d_delta, int64_t M, int N,
+                                       int act, const float *d_prelu,
+                                       float *d_db, float *d_dprelu) {
+  return activation_backward(ctx, d_out, d_delta, M, N, act, d_prelu, d_db,
+                             d_dprelu, true);
+}
+
+extern "C" int scn_activation_backward_acc(scn_ctx *ctx, const float *d_out,
+                                           float *d_delta, int64_t M, int N,
+                                           int act, const float *d_prelu,
+                                           float *d_db, float *d_dprelu) {
+  return activation_backward(ctx, d_out, d_delta, M, N, act, d_prelu, d_db,
+                             d_dprelu, false);
 }
 
 // ------------------------------------------------------- dW = A^T D (MFMA)
@@ -374,14 +392,15 @@ static int launch_atb_wide(scn_ctx *ctx, const float *d_A, const float *d_D,
   return SCN_OK;
 }
 
-extern "C" int scn_sgemm_AtB(scn_ctx *ctx, const float *d_A, const float *d_D,
-                             float *d_dW, int64_t M, int K, int N) {
+static int sgemm_AtB(scn_ctx *ctx, const float *d_A, const float *d_D,
+                     float *d_dW, int64_t M, int K, int N, bool clear) {
   SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_sgemm_AtB: null context");
   SCN_REQUIRE(M >= 0 && K >= 1 && N >= 1, SCN_ERR_ARG,
               "scn_sgemm_AtB: M %lld K %d N %d", (long long)M, K, N);
   SCN_REQUIRE(d_dW, SCN_ERR_ARG, "scn_sgemm_AtB: null d_dW");
   ProfScope prof(ctx, SCN_K_BACKWARD);
-  SCN_TRY(scn_fill32(ctx, d_dW, 0, (size_t)K * N));
+  if (clear)
+    SCN_TRY(scn_fill32(ctx, d_dW, 0, (size_t)K * N));
   if (M == 0)
     return SCN_OK;
   SCN_REQUIRE(d_A && d_D, SCN_ERR_ARG, "scn_sgemm_AtB: null buffer");
@@ -419,6 +438,19 @@ extern "C" int scn_sgemm_AtB(scn_ctx *ctx, const float *d_A, const float *d_D,
                      N, nTiles, rowsPerSplit);
   SCN_HIP_CHECK(hipGetLastError());
   return SCN_OK;
+}
+
+extern "C" int scn_sgemm_AtB(scn_ctx *ctx, const float *d_A, const float *d_D,
+                             float *d_dW, int64_t M, int K, int N) {
+  return sgemm_AtB(ctx, d_A, d_D, d_dW, M, K, N, true);
+}
+
+// the kernels only ever add to dW, so beta = 1 is the same launch without the
+// clearing one before it
+extern "C" int scn_sgemm_AtB_acc(scn_ctx *ctx, const float *d_A,
+                                 const float *d_D, float *d_dW, int64_t M,
+                                 int K, int N) {
+  return sgemm_AtB(ctx, d_A, d_D, d_dW, M, K, N, false);
 }
 
 // ------------------------------------------------------------ dA = D W^T
@@ -500,6 +532,81 @@ extern "C" int scn_nag_update(scn_ctx *ctx, const float *d_delta,
   hipLaunchKernelGGL(k_nag_update, dim3(scn_ceil_div(n, 256)), dim3(256), 0,
                      ctx->stream, d_delta, d_momentum, d_weights, (long long)n,
                      learningRate, momentum, keepPositive);
+  SCN_HIP_CHECK(hipGetLastError());
+  return SCN_OK;
+}
+
+// The momentum step of several tensors (a layer's W, B and PReLU slopes) in
+// one launch: a workgroup finds its tensor from the running workgroup counts.
+// With `clear` the gradient is left zero, so the next batch's accumulating
+// products need no clearing launch.
+struct NagList {
+  float *delta[SCN_NAG_MAX];
+  float *mom[SCN_NAG_MAX];
+  float *wts[SCN_NAG_MAX];
+  long long n[SCN_NAG_MAX];
+  unsigned firstBlock[SCN_NAG_MAX + 1];
+  int keepPositive[SCN_NAG_MAX];
+  int count;
+};
+
+__global__ __launch_bounds__(256) void k_nag_update_many(NagList l, float lr,
+                                                         float mu, int clear) {
+  int t = 0;
+  while (t + 1 < l.count && blockIdx.x >= l.firstBlock[t + 1])
+    ++t;
+  const long long i =
+      (long long)(blockIdx.x - l.firstBlock[t]) * blockDim.x + threadIdx.x;
+  if (i >= l.n[t])
+    return;
+  float w = l.wts[t][i], m = l.mom[t][i];
+  const float d = l.delta[t][i];
+  w -= m * mu;
+  m = mu * m - lr * (1 - mu) * d;
+  w += m * (1 + mu);
+  if (l.keepPositive[t])
+    w = w > 0.001f ? w : 0.001f;
+  l.wts[t][i] = w;
+  l.mom[t][i] = m;
+  if (clear)
+    l.delta[t][i] = 0.f;
+}
+
+extern "C" int scn_nag_update_many(scn_ctx *ctx, const scn_nag_item *items,
+                                   int nItems, float learningRate,
+                                   float momentum, int clearGradients) {
+  SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_nag_update_many: null context");
+  SCN_REQUIRE(nItems >= 0 && nItems <= SCN_NAG_MAX && (items || nItems == 0),
+              SCN_ERR_ARG, "scn_nag_update_many: %d items (at most %d)",
+              nItems, SCN_NAG_MAX);
+  NagList l;
+  l.count = 0;
+  long long blocks = 0;
+  for (int k = 0; k < nItems; ++k) {
+    const scn_nag_item &it = items[k];
+    SCN_REQUIRE(it.n >= 0, SCN_ERR_ARG, "scn_nag_update_many: item %d n %lld",
+                k, (long long)it.n);
+    if (it.n == 0)
+      continue;
+    SCN_REQUIRE(it.d_delta && it.d_momentum && it.d_weights, SCN_ERR_ARG,
+                "scn_nag_update_many: item %d null buffer", k);
+    const int c = l.count++;
+    l.delta[c] = it.d_delta;
+    l.mom[c] = it.d_momentum;
+    l.wts[c] = it.d_weights;
+    l.n[c] = it.n;
+    l.keepPositive[c] = it.keepPositive;
+    l.firstBlock[c] = (unsigned)blocks;
+    blocks += scn_ceil_div(it.n, 256);
+    SCN_REQUIRE(blocks <= 0x7fffffffll, SCN_ERR_CAPACITY,
+                "scn_nag_update_many: %lld workgroups", blocks);
+  }
+  if (l.count == 0)
+    return SCN_OK;
+  l.firstBlock[l.count] = (unsigned)blocks;
+  ProfScope prof(ctx, SCN_K_BACKWARD);
+  hipLaunchKernelGGL(k_nag_update_many, dim3((unsigned)blocks), dim3(256), 0,
+                     ctx->stream, l, learningRate, momentum, clearGradients);
   SCN_HIP_CHECK(hipGetLastError());
   return SCN_OK;
 }

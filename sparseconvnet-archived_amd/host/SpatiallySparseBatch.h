@@ -14,6 +14,9 @@ struct BatchResultStage {
   size_t capacity; // floats
   scn_event *arrived;
   bool pending;
+  // the labels as the statistics need them, on the host, while batch.labels
+  // is in device memory for the gradient of a training batch
+  std::vector<int> labels;
   BatchResultStage();
   ~BatchResultStage();
   BatchResultStage(const BatchResultStage &) = delete;

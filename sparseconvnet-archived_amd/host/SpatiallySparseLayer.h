@@ -111,6 +111,7 @@ private:
   RNG rng;
   std::mutex rngMutex; // preprocess() runs on several producer threads
   vectorCUDA<float> dw, db, workspace; // gradients; W transposed for dA
+  bool gradsClean = false; // dw and db hold zeros (the momentum step left them so)
   vectorCUDA<float> w, b; // sub-matrix of a training batch with dropout
 
 public:
@@ -150,6 +151,7 @@ private:
   RNG rng;
   std::mutex rngMutex;
   vectorCUDA<float> dw, db, dprelu, workspace;
+  bool gradsClean = false; // as NetworkInNetworkLayer's
   vectorCUDA<float> w, b;
 
 public:

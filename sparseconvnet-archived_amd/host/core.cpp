@@ -361,6 +361,7 @@ void SpatiallySparseBatch::reset() {
   interfaces[0].sub->features.copyToCPU();
   labels.resize(0);
   labels.copyToCPU();
+  result->labels.clear();
   predictions.resize(0);
   probabilities.resize(0);
   negativeLogLikelihood = 0;

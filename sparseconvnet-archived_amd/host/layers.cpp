@@ -314,11 +314,14 @@ static bool nin_fused(cudaMemStream &ms, SpatiallySparseBatchInterface &input,
   return true;
 }
 
-// NetworkInNetwork(PReLU)Layer::backwards without dropout
+// NetworkInNetwork(PReLU)Layer::backwards
 // (NetworkInNetworkLayer.cu:219-289, NetworkInNetworkPReLULayer.cu:190-277):
-// activation derivative in place (+ bias and slope gradients), slope update,
-// dW = A^T D, dA = D W^T with the weights of the forward pass, then the
-// momentum step on W and B.
+// activation derivative in place (+ bias and slope gradients), dW = A^T D,
+// dA = D W^T with the weights of the forward pass, then the momentum step on
+// the slopes, W and B.  Without dropout that step is one launch which also
+// leaves the gradients zero (gradsClean), so the next batch's products add to
+// them without clearing launches of their own; the reference updates the
+// slopes before the products, which nothing after that point reads.
 static void nin_backwards(cudaMemStream &ms,
                           SpatiallySparseBatchInterface &input,
                           SpatiallySparseBatchInterface &output, int nFeaturesIn,
@@ -328,26 +331,28 @@ static void nin_backwards(cudaMemStream &ms,
                           vectorCUDA<float> *PReLU, vectorCUDA<float> *MPReLU,
                           vectorCUDA<float> &dw, vectorCUDA<float> &db,
                           vectorCUDA<float> *dprelu,
-                          vectorCUDA<float> &workspace, float learningRate,
-                          float momentum) {
+                          vectorCUDA<float> &workspace, bool &gradsClean,
+                          float learningRate, float momentum) {
   // with dropout: the features present, and the sub-matrix forwards() left
   // in shrunkW (NetworkInNetworkLayer.cu:235-263)
   const int64_t M = output.nSpatialSites;
   const int K = (int)input.featuresPresent.size();
   const int N = (int)output.featuresPresent.size();
+  const bool clean = gradsClean && dw.size64() == (size_t)K * N &&
+                     db.size64() == (size_t)N &&
+                     (!dprelu || dprelu->size64() == (size_t)N);
+  gradsClean = false;
   dw.resize64((size_t)K * N);
   db.resize64((size_t)N);
   if (dprelu)
     dprelu->resize64((size_t)N);
-  SCN_CHECKED(scn_activation_backward(
+  SCN_CHECKED((clean ? scn_activation_backward_acc : scn_activation_backward)(
       ms.ctx, output.sub->features.dPtr(), output.sub->dfeatures.dPtr(), M, N,
       act, PReLU ? PReLU->dPtr() : nullptr, db.dPtr(),
       dprelu ? dprelu->dPtr() : nullptr));
-  if (PReLU)
-    SCN_CHECKED(scn_nag_update(ms.ctx, dprelu->dPtr(), MPReLU->dPtr(),
-                               PReLU->dPtr(), N, learningRate, momentum, 1));
-  SCN_CHECKED(scn_sgemm_AtB(ms.ctx, input.sub->features.dPtr(),
-                            output.sub->dfeatures.dPtr(), dw.dPtr(), M, K, N));
+  SCN_CHECKED((clean ? scn_sgemm_AtB_acc : scn_sgemm_AtB)(
+      ms.ctx, input.sub->features.dPtr(), output.sub->dfeatures.dPtr(),
+      dw.dPtr(), M, K, N));
   multiplyAddCount += (__int128_t)M * K * N;
   if (input.backpropErrors) {
     input.sub->dfeatures.resize64((size_t)input.nSpatialSites * K);
@@ -359,6 +364,9 @@ static void nin_backwards(cudaMemStream &ms,
     multiplyAddCount += (__int128_t)M * K * N;
   }
   if (shrunkW) {
+    if (PReLU)
+      SCN_CHECKED(scn_nag_update(ms.ctx, dprelu->dPtr(), MPReLU->dPtr(),
+                                 PReLU->dPtr(), N, learningRate, momentum, 1));
     SCN_CHECKED(scn_nag_update_shrunk(
         ms.ctx, dw.dPtr(), MW.dPtr(), W.dPtr(), input.featuresPresent.dPtr(),
         output.featuresPresent.dPtr(), nFeaturesOut, K, N, learningRate,
@@ -368,10 +376,15 @@ static void nin_backwards(cudaMemStream &ms,
         output.featuresPresent.dPtr(), nFeaturesOut, 1, N, learningRate,
         momentum));
   } else {
-    SCN_CHECKED(scn_nag_update(ms.ctx, dw.dPtr(), MW.dPtr(), W.dPtr(),
-                               (int64_t)K * N, learningRate, momentum, 0));
-    SCN_CHECKED(scn_nag_update(ms.ctx, db.dPtr(), MB.dPtr(), B.dPtr(), N,
-                               learningRate, momentum, 0));
+    scn_nag_item items[3];
+    int n = 0;
+    if (PReLU)
+      items[n++] = {dprelu->dPtr(), MPReLU->dPtr(), PReLU->dPtr(), N, 1};
+    items[n++] = {dw.dPtr(), MW.dPtr(), W.dPtr(), (int64_t)K * N, 0};
+    items[n++] = {db.dPtr(), MB.dPtr(), B.dPtr(), N, 0};
+    SCN_CHECKED(
+        scn_nag_update_many(ms.ctx, items, n, learningRate, momentum, 1));
+    gradsClean = true;
   }
   (void)nFeaturesIn;
 }
@@ -442,7 +455,7 @@ void NetworkInNetworkLayer::backwards(SpatiallySparseBatch &batch,
                     ? &w
                     : nullptr,
                 (int)fn, W, MW, B, MB, nullptr, nullptr, dw, db, nullptr,
-                workspace, learningRate, momentum);
+                workspace, gradsClean, learningRate, momentum);
 }
 // scaleWeights (NetworkInNetworkLayer.cu:203-218; the PReLU layer's is the
 // same, NetworkInNetworkPReLULayer.cu:175-189): bring the mean magnitude of
@@ -572,7 +585,7 @@ void NetworkInNetworkPReLULayer::backwards(
                     ? &w
                     : nullptr,
                 (int)PRELU, W, MW, B, MB, &PReLU, &MPReLU, dw, db, &dprelu,
-                workspace, learningRate, momentum);
+                workspace, gradsClean, learningRate, momentum);
 }
 void NetworkInNetworkPReLULayer::loadWeightsFromStream(std::ifstream &f,
                                                        bool momentum) {
@@ -933,6 +946,10 @@ void SoftmaxClassifierLaunch(SpatiallySparseBatchInterface &input,
                              cudaMemStream &memStream) {
   assert(batch.batchSize == input.nSpatialSites);
   assert(input.nFeatures == (int)input.featuresPresent.size());
+  // (a batch that did not come from a BatchProducer has its labels on the host still)
+  if (batch.type != UNLABELEDBATCH &&
+      (int)batch.result->labels.size() != batch.batchSize)
+    batch.result->labels = batch.labels.hVector();
   if (batch.type == TRAINBATCH) {
     // the backward pass starts here: d cost / d soft-max input
     // (SoftmaxClassifier.cu:22-31)
@@ -974,7 +991,7 @@ void SoftmaxClassifierCollect(SpatiallySparseBatchInterface &input,
   for (int i = 0; i < batch.batchSize; i++)
     batch.predictions.push_back(vectorTopIndices(batch.probabilities[i], nTop));
   if (batch.type != UNLABELEDBATCH) {
-    std::vector<int> &labels = batch.labels.hVector();
+    const std::vector<int> &labels = r.labels;
     batch.mistakes += batch.batchSize;
     for (int i = 0; i < batch.batchSize; i++) {
       double pr = batch.probabilities[i][labels[i]];

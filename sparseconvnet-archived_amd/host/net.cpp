@@ -719,6 +719,12 @@ void BatchProducer::preprocessBatchOnDevice(int cc) {
                               b.stagingRow.dPtr(), (int64_t)n,
                               b.stagingBackground.dPtr(), in.nSpatialSites));
   in.sub->features.copyToGPUAsync(ms);
+  if (b.type == TRAINBATCH) {
+    // the classifier's gradient reads the labels on the device: uploaded here,
+    // on this slot's stream, so that the net's stream is never waited for
+    b.result->labels = b.labels.hVector();
+    b.labels.copyToGPUAsync(ms);
+  }
   buildRuleBooks(cnn, ctx, b);
   SCN_CHECKED(scn_sync(ctx));
 }

@@ -100,6 +100,67 @@ def test_weight_update(scn, ctx):
             assert np.allclose(d_m.download(), m, rtol=1e-6, atol=1e-8)
 
 
+def test_weight_update_of_several_tensors_in_one_launch(scn, ctx):
+    """scn_nag_update_many = scn_nag_update on each tensor (bit for bit: the same arithmetic), gradients left zero
+    when asked; sizes chosen so that tensors end inside, at the end of and one past a workgroup of 256."""
+    rng = np.random.default_rng(4)
+    for sizes, clear in [((100,), True), ((96, 256 * 96, 96), True), ((257, 1, 256, 511), False),
+                         ((0, 800 * 800, 800), True), ((5, 0, 7), False), ((), True)]:
+        print("nag_update_many sizes", sizes, flush=True)
+        items, single = [], []
+        for k, n in enumerate(sizes):
+            d = rng.standard_normal(n).astype(np.float32)
+            w = rng.standard_normal(n).astype(np.float32)
+            m = (rng.standard_normal(n) * 0.1).astype(np.float32)
+            keep = k == 0
+            d_d, d_m, d_w = ctx.array(d), ctx.array(m), ctx.array(w)
+            items.append((d_d, d_m, d_w, n, keep))
+            s_m, s_w = ctx.array(m), ctx.array(w)
+            if n:
+                ctx.nag_update(ctx.array(d), s_m, s_w, n, 0.003, 0.99, keep)
+            single.append((d, s_m, s_w))
+        ctx.nag_update_many(items, 0.003, 0.99, clear)
+        for (d_d, d_m, d_w, n, keep), (d, s_m, s_w) in zip(items, single):
+            if n == 0:
+                continue
+            assert np.array_equal(d_w.download(), s_w.download())
+            assert np.array_equal(d_m.download(), s_m.download())
+            assert np.array_equal(d_d.download(), np.zeros(n, np.float32) if clear else d)
+    with pytest.raises(scn.ScnError):
+        z = ctx.array(np.zeros(4, np.float32))
+        ctx.nag_update_many([(z, z, z, 4, False)] * (scn.NAG_MAX + 1), 0.1, 0.9)
+
+
+def test_accumulating_products_add_to_what_is_there(scn, ctx):
+    """The beta = 1 variants: on zeroed buffers they are the plain entry points, on others they add."""
+    rng = np.random.default_rng(5)
+    for M, K, N in [(50, 12, 32), (4097, 288, 64), (70000, 256, 96), (0, 8, 8)]:
+        print("accumulating products M=%d K=%d N=%d" % (M, K, N), flush=True)
+        A = rng.standard_normal((M, K)).astype(np.float32)
+        D = rng.standard_normal((M, N)).astype(np.float32)
+        base = rng.standard_normal((K, N)).astype(np.float32)
+        plain, acc = ctx.empty((K, N), np.float32), ctx.array(base)
+        ctx.sgemm_AtB(ctx.array(A), ctx.array(D), plain, M, K, N)
+        ctx.sgemm_AtB(ctx.array(A), ctx.array(D), acc, M, K, N, accumulate=True)
+        scale = np.sqrt((A.astype(np.float64) ** 2).sum(0))[:, None] * np.sqrt((D.astype(np.float64) ** 2).sum(0))[None]
+        close(acc.download(), base.astype(np.float64) + plain.download(), scale + np.abs(base) + 1e-6)
+        for act in (1, 6):
+            out = rng.standard_normal((M, N)).astype(np.float32)
+            pr = ctx.array(rng.uniform(0.05, 0.5, N).astype(np.float32)) if act == 6 else None
+            b0 = rng.standard_normal(N).astype(np.float32)
+            p_d, a_d = ctx.array(D), ctx.array(D)
+            p_db, a_db = ctx.empty(N, np.float32), ctx.array(b0)
+            p_dp, a_dp = (ctx.empty(N, np.float32), ctx.array(b0)) if act == 6 else (None, None)
+            ctx.activation_backward(ctx.array(out), p_d, M, N, act, pr, p_db, p_dp)
+            ctx.activation_backward(ctx.array(out), a_d, M, N, act, pr, a_db, a_dp, accumulate=True)
+            assert np.array_equal(p_d.download(), a_d.download())
+            mag = np.abs(p_d.download()).sum(0) + np.abs(b0)
+            close(a_db.download(), b0.astype(np.float64) + p_db.download(), mag + 1e-6)
+            if act == 6:
+                close(a_dp.download(), b0.astype(np.float64) + p_dp.download(),
+                      (np.abs(D) * np.abs(out)).sum(0) / 0.05 + np.abs(b0) + 1e-6)
+
+
 @pytest.mark.parametrize("nIn,rowsIn,count", [(1, 5, 40), (3, 1000, 33333), (32, 5000, 100001), (64, 2000, 54321),
                                               (96, 300, 9999), (160, 77, 4096), (5, 10, 31)])
 def test_convolution_backward_scatter(scn, ctx, nIn, rowsIn, count):
