@@ -273,6 +273,17 @@ int scn_sgemm_AtB(scn_ctx *ctx, const float *d_A, const float *d_D,
 int64_t scn_sgemm_ABt_workspace(int N, int K);
 int scn_sgemm_ABt(scn_ctx *ctx, const float *d_D, const float *d_W,
                   float *d_dA, int64_t M, int N, int K, float *d_workspace);
+/* scn_sgemm_ABt for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): no
+ * counterpart in the reference.  The transposed weights go to a static device
+ * array of scn_sgemm_ABt_static_limit() floats (4 MiB, held by every device
+ * the library runs on until the process ends) instead of a workspace; the call
+ * allocates and frees nothing.  scn_sgemm_ABt_workspace(N, K) beyond the limit
+ * is refused with SCN_ERR_CAPACITY.  All calls on one device share the array:
+ * calls that overlap on one device (two contexts, two streams) race. */
+int64_t scn_sgemm_ABt_static_limit(void);
+int scn_sgemm_ABt_static(scn_ctx *ctx, const float *d_D, const float *d_W,
+                         float *d_dA, int64_t M, int N, int K);
 /* dGradientDescent / dGradientDescentKeepPositive (NetworkInNetworkLayer.cu:
  * 27-41, NetworkInNetworkPReLULayer.cu:68-83), "NAG light": w -= m mu;
  * m = mu m - lr (1 - mu) d; w += m (1 + mu); keepPositive clamps w at 0.001. */

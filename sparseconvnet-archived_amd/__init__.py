@@ -117,6 +117,8 @@ def lib():
         "scn_sgemm_AtB": (C.c_int, [vp, vp, vp, vp, i64, C.c_int, C.c_int]),
         "scn_sgemm_ABt_workspace": (i64, [C.c_int, C.c_int]),
         "scn_sgemm_ABt": (C.c_int, [vp, vp, vp, vp, i64, C.c_int, C.c_int, vp]),
+        "scn_sgemm_ABt_static_limit": (i64, []),
+        "scn_sgemm_ABt_static": (C.c_int, [vp, vp, vp, vp, i64, C.c_int, C.c_int]),
         "scn_nag_update": (C.c_int, [vp, vp, vp, vp, i64, f32, f32, C.c_int]),
         "scn_nag_update_many": (C.c_int, [vp, P(NagItem), C.c_int, f32, f32, C.c_int]),
         "scn_activation_backward_acc": (C.c_int, [vp, vp, vp, i64, C.c_int, C.c_int, vp, vp, vp]),
@@ -294,6 +296,9 @@ class Context:
     def sgemm_ABt(self, d_D, d_W, d_dA, M, N, K, d_workspace):
         assert d_workspace.size >= lib().scn_sgemm_ABt_workspace(N, K)
         _check(lib().scn_sgemm_ABt(self.h, d_D.ptr, d_W.ptr, d_dA.ptr, M, N, K, d_workspace.ptr))
+
+    def sgemm_ABt_static(self, d_D, d_W, d_dA, M, N, K):
+        _check(lib().scn_sgemm_ABt_static(self.h, d_D.ptr, d_W.ptr, d_dA.ptr, M, N, K))
 
     def nag_update(self, d_delta, d_momentum, d_weights, n, learningRate, momentum, keepPositive=False):
         _check(lib().scn_nag_update(self.h, d_delta.ptr, d_momentum.ptr, d_weights.ptr, n, learningRate, momentum,

@@ -108,6 +108,9 @@ static inline int scn_ceil_div(int64_t a, int64_t b) {
   return (int)((a + b - 1) / b);
 }
 
+// address of the static scratch of scn_sgemm_ABt_static on `device` (scn_train.hip)
+int scn_abt_static_setup(int device);
+
 // exclusive prefix sum of n uint32 values; out has n + 1 elements (out[n] =
 // total).  `tmp` must hold scn_scan_tmp_elems(n) uint32.
 size_t scn_scan_tmp_elems(size_t n);

@@ -25,6 +25,7 @@ extern "C" int scn_ctx_create(int device, scn_ctx **out) {
   SCN_REQUIRE(device < n, SCN_ERR_ARG, "scn_ctx_create: device %d of %d",
               device, n);
   SCN_HIP_CHECK(hipSetDevice(device));
+  SCN_TRY(scn_abt_static_setup(device));
   scn_ctx *c = new scn_ctx();
   c->device = device;
   c->prof = false;

@@ -500,6 +500,56 @@ extern "C" int scn_sgemm_ABt(scn_ctx *ctx, const float *d_D, const float *d_W,
                          SCN_NOSIGMOID, SCN_FP32);
 }
 
+// dA = D W^T for callers that may not allocate (code under HIP graph capture,
+// serving loops, harnesses that forbid hipMalloc): the transposed weights and
+// the zero bias live in a file-scope device array instead of a caller's
+// workspace.  Every device the library runs on holds its own copy of the array
+// at its own address; host code reaches it only through the pointer that
+// hipGetSymbolAddress returned for that device.
+#define ABT_STATIC_FLOATS (1 << 20) // 4 MiB per device
+static __device__ __align__(256) float scratch[ABT_STATIC_FLOATS];
+#define ABT_MAX_DEVICES 64
+static float *g_abtScratch[ABT_MAX_DEVICES]; // per device, set once by scn_ctx_create
+
+int scn_abt_static_setup(int device) {
+  SCN_REQUIRE(device >= 0 && device < ABT_MAX_DEVICES, SCN_ERR_ARG,
+              "device %d: at most %d devices", device, ABT_MAX_DEVICES);
+  if (g_abtScratch[device])
+    return SCN_OK;
+  float *ptr = nullptr;
+  SCN_HIP_CHECK(hipSetDevice(device));
+  SCN_HIP_CHECK(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
+  SCN_REQUIRE(ptr != nullptr, SCN_ERR_HIP,
+              "hipGetSymbolAddress returned no address for the static scratch");
+  g_abtScratch[device] = ptr;
+  return SCN_OK;
+}
+
+extern "C" int64_t scn_sgemm_ABt_static_limit(void) { return ABT_STATIC_FLOATS; }
+
+extern "C" int scn_sgemm_ABt_static(scn_ctx *ctx, const float *d_D,
+                                    const float *d_W, float *d_dA, int64_t M,
+                                    int N, int K) {
+  SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_sgemm_ABt_static: null context");
+  SCN_REQUIRE(M >= 0 && K >= 1 && N >= 1, SCN_ERR_ARG,
+              "scn_sgemm_ABt_static: M %lld N %d K %d", (long long)M, N, K);
+  SCN_REQUIRE(scn_sgemm_ABt_workspace(N, K) <= ABT_STATIC_FLOATS,
+              SCN_ERR_CAPACITY,
+              "scn_sgemm_ABt_static: N %d x K %d weights need %lld floats of "
+              "scratch, the static array holds %d; use scn_sgemm_ABt with a "
+              "workspace",
+              N, K, (long long)scn_sgemm_ABt_workspace(N, K), ABT_STATIC_FLOATS);
+  float *ptr = ctx->device >= 0 && ctx->device < ABT_MAX_DEVICES
+                   ? g_abtScratch[ctx->device]
+                   : nullptr;
+  SCN_REQUIRE(ptr, SCN_ERR_STATE,
+              "scn_sgemm_ABt_static: no scratch address for device %d",
+              ctx->device);
+  // (the kernels clear and fill what they use of the array: nothing of an
+  // earlier call is read)
+  return scn_sgemm_ABt(ctx, d_D, d_W, d_dA, M, N, K, ptr);
+}
+
 // ---------------------------------------------------------- weight update
 __global__ void k_nag_update(const float *__restrict__ delta,
                              float *__restrict__ mom, float *__restrict__ wts,
