@@ -180,6 +180,24 @@ int scn_rules_terminal_plan(scn_ctx *ctx, const scn_grids *in, scn_grids *out,
  * plans the batch again with deferral off (that also raises the bounds). */
 int scn_ctx_defer_counts(scn_ctx *ctx, int on);
 int scn_rules_settle(scn_ctx *ctx);
+/* Recorded plans.  gridRules runs per sample (ConvolutionalLayer.cu:114-118,
+ * MaxPoolingLayer.cu:116-118) and the layers' preprocess() calls follow one
+ * another without anything else in between (BatchProducer.cu:79-81).  With
+ * recording on (and deferred counts on), scn_rules_square_plan,
+ * scn_rules_triangular_plan, scn_rules_terminal_plan and scn_rules_fill calls
+ * that continue from one another -- each plan's `in` being the `out` of the
+ * plan before -- are only noted, provided every `out` has held a plan before
+ * and a sample's grids fit the LDS of a compute unit (2-D and small 3-D
+ * fields); scn_ctx_chain_rules(ctx, 0), scn_rules_settle or any call that
+ * cannot join then runs all of them in two launches, one workgroup carrying
+ * one sample through every layer.  Results (rules, counts, grids as seen
+ * through scn_grids_download / scn_grids_find) are those of the calls made one
+ * by one; a sample too large for the LDS is reported by scn_rules_settle as
+ * SCN_ERR_CAPACITY like any outgrown bound. */
+int scn_ctx_chain_rules(scn_ctx *ctx, int on);
+/* how many chains of recorded plans the context has run, and how many plans
+ * they held in all (a plan that could not join is not counted) */
+int scn_ctx_chain_count(scn_ctx *ctx, int64_t *chains, int64_t *plans);
 int scn_rules_width(const scn_grids *out, int64_t *width);
 /* Writes nOutputSpatialSites * width int32 rules; capacity in int32s. */
 int scn_rules_fill(scn_ctx *ctx, const scn_grids *in, scn_grids *out,

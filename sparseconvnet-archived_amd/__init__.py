@@ -90,6 +90,8 @@ def lib():
         "scn_grids_create": (C.c_int, [vp, P(vp)]),
         "scn_grids_clear_many": (C.c_int, [vp, C.POINTER(vp), C.c_int]),
         "scn_ctx_defer_counts": (C.c_int, [vp, C.c_int]),
+        "scn_ctx_chain_rules": (C.c_int, [vp, C.c_int]),
+        "scn_ctx_chain_count": (C.c_int, [vp, P(i64), P(i64)]),
         "scn_rules_settle": (C.c_int, [vp]),
         "scn_grids_destroy": (C.c_int, [vp, vp]),
         "scn_grids_build": (C.c_int, [vp, vp, C.c_int, C.c_int, C.c_int, vp, vp, vp, i64, vp, i32]),
@@ -424,6 +426,18 @@ class Grids:
 
 def defer_counts(ctx, on):
     _check(lib().scn_ctx_defer_counts(ctx.h, int(on)))
+
+
+def chain_rules(ctx, on):
+    """Record plan / fill calls that continue from one another and run them together (needs deferred counts)."""
+    _check(lib().scn_ctx_chain_rules(ctx.h, int(on)))
+
+
+def chain_count(ctx):
+    """(chains run, plans they held) so far on this context"""
+    a, b = C.c_int64(), C.c_int64()
+    _check(lib().scn_ctx_chain_count(ctx.h, C.byref(a), C.byref(b)))
+    return a.value, b.value
 
 
 def settle(ctx):

@@ -1,0 +1,945 @@
+// Rule books of every layer of a net in two launches (small fields).
+//
+// BatchProducer::preprocessBatch (BatchProducer.cu:40-87) calls preprocess()
+// of every layer back to back, and gridRules runs per sample
+// (ConvolutionalLayer.cu:114-118, MaxPoolingLayer.cu:116-118): the samples of
+// a batch never meet until their rows are numbered.  scn_grids.hip builds one
+// layer at a time over the whole batch through tables in HBM, four launches
+// per layer; for a 2-D net that is some fifty dependent launches of a few
+// microseconds each.  Here the plan and fill calls of consecutive layers are
+// only recorded (scn_ctx_chain_rules) and then run together:
+//
+//   k_chain_sample  one workgroup per sample carries the sample's grid --
+//                   occupancy mask, rank prefix, (key, row) by rank -- in LDS
+//                   through all recorded layers: owner test and counts, prefix
+//                   sum, output sites, rule rows, with rows numbered from zero
+//                   within the sample; rule rows and site keys go to a staging
+//                   area at sample-local positions;
+//   k_chain_place   one workgroup per (sample, layer) adds up the counts of
+//                   the samples before it and copies the staged rows to their
+//                   batch-global place, adding the row offsets of the sample.
+//
+// Row numbers are the reference's: first touch while the input map is
+// iterated in ascending key (Regions.cu:557-576), background row last
+// (:647-652), samples concatenated in batch order.  The grids objects of the
+// recorded layers get their entry lists, backgroundCol and counts; their hash
+// tables and masks are only built if somebody asks (ensure_index).
+#include "scn_grids_dev.h"
+#include <string.h>
+#include <mutex>
+
+#define CHAIN_MAX_LEVELS 24
+#define CHAIN_THREADS 256
+#define CHAIN_WAVES (CHAIN_THREADS / 64)
+#define CHAIN_LDS_MAX (152 * 1024)
+#define CHAIN_HEADER_BYTES 512
+#define CHAIN_MIN_ARENA (16 * 1024)
+// bytes of arena per entry of the input grid (key, row, ownership mask, base)
+// and of the output grid (key, row)
+#define CHAIN_IN_BYTES 16
+#define CHAIN_OUT_BYTES 8
+
+enum { CH_REGIONS = 0, CH_TERMINAL = 1 };
+
+struct ChainLevel {
+  int kind;
+  int mode, nIn, nOut, size, stride, minActive, width, cube;
+  int capRows; // rows of one sample the staging area holds
+  int slot;    // pinned slot of the deferred counts
+  int pad;
+  long long fullSize; // sites of a full output grid
+  // staging, in ints: rule rows of sample b at stRules + b capRows width,
+  // site keys at stKeys + b capRows
+  long long stRules, stKeys;
+  int *rules; // the caller's buffer (null: no rules wanted)
+  long long capacity;
+  long long *ekey;
+  int *erow;
+  int *bg;
+  long long *meta;
+  long long boundRows, boundActive; // terminal: boundRows bounds the width
+};
+
+struct ChainArgs {
+  int nLevels, batch, d, n0;
+  const Slot *table; // the source grids
+  unsigned shift, mask;
+  const unsigned long long *bits;
+  const int *bg;
+  long long vol0;
+  int maskOff[3], prefOff[2], arenaOff, arenaBytes; // LDS layout, bytes
+  int maskWords[3]; // capacity of the three mask buffers, 64-bit words
+  int *counts; // [nLevels][batch][2]
+  unsigned long long *flag;
+  unsigned long long ticket;
+  int *staging;
+  long long *scalars;
+  const long long *badSites;
+  ChainLevel lv[CHAIN_MAX_LEVELS];
+};
+static_assert(sizeof(ChainArgs) <= 4096, "kernel arguments");
+
+struct ChainRec {
+  scn_grids *in, *out;
+  ChainLevel lv;
+  Geom geom;
+  bool filled;
+};
+struct ChainState {
+  bool on = false;
+  bool wide = false; // a sample has outgrown a tight arena: use the largest
+  long long nChains = 0, nPlans = 0; // run so far
+  std::vector<ChainRec> recs;
+  DevBuf<int> staging, counts;
+  DevBuf<unsigned long long> flag;
+};
+
+// ------------------------------------------------------------------ device
+
+__device__ __forceinline__ unsigned wave_scan_incl(unsigned v, int lane) {
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    unsigned up = __shfl_up(v, off, 64);
+    if (lane >= off)
+      v += up;
+  }
+  return v;
+}
+
+// Exclusive prefix sum over n values held in LDS, by the whole workgroup:
+// put(i, sum of get(0..i)); returns the total to every lane.  Every lane takes
+// a run of consecutive values.  ws: CHAIN_WAVES words.
+template <typename Get, typename Put>
+__device__ __forceinline__ unsigned chain_scan(int n, Get get, Put put,
+                                               unsigned *ws) {
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int per = (n + CHAIN_THREADS - 1) / CHAIN_THREADS;
+  const int i0 = t * per < n ? t * per : n;
+  const int i1 = i0 + per < n ? i0 + per : n;
+  unsigned s = 0;
+  for (int i = i0; i < i1; ++i)
+    s += get(i);
+  const unsigned incl = wave_scan_incl(s, lane);
+  if (lane == 63)
+    ws[wave] = incl;
+  __syncthreads();
+  unsigned before = 0, total = 0;
+#pragma unroll
+  for (int w = 0; w < CHAIN_WAVES; ++w) {
+    const unsigned x = ws[w];
+    before += w < wave ? x : 0u;
+    total += x;
+  }
+  unsigned run = before + incl - s;
+  for (int i = i0; i < i1; ++i) {
+    const unsigned v = get(i);
+    put(i, run);
+    run += v;
+  }
+  __syncthreads();
+  return total;
+}
+
+__device__ __forceinline__ unsigned lds_rank(const unsigned long long *bits,
+                                             const unsigned short *pref,
+                                             unsigned p) {
+  const unsigned w = p >> 6, sh = p & 63;
+  const unsigned long long below = sh ? (bits[w] & ((1ull << sh) - 1ull)) : 0ull;
+  return pref[w] + (unsigned)__popcll(below);
+}
+
+// The sample could not be carried (LDS or staging too small): every plan of
+// the chain is reported as outgrown, and the caller plans the batch again
+// layer by layer.
+__device__ __forceinline__ void chain_give_up(const ChainArgs &a) {
+  if (threadIdx.x == 0)
+    atomicMax(a.flag, a.ticket);
+}
+
+template <int D>
+__global__ void __launch_bounds__(CHAIN_THREADS) k_chain_sample(ChainArgs a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  const int b = blockIdx.x, t = threadIdx.x;
+  unsigned *ws = reinterpret_cast<unsigned *>(lds); // CHAIN_WAVES words
+  int *invOrd = reinterpret_cast<int *>(lds + 64);  // up to 64 offsets
+  auto M = [&](int x) {
+    return reinterpret_cast<unsigned long long *>(lds + a.maskOff[x]);
+  };
+  auto P = [&](int x) {
+    return reinterpret_cast<unsigned short *>(lds + a.prefOff[x]);
+  };
+  unsigned *arena = reinterpret_cast<unsigned *>(lds + a.arenaOff);
+  const int arenaWords = a.arenaBytes / 4;
+
+  // ---- the source grid of this sample: its slice of the batch's mask
+  long long vol = a.vol0;
+  int words = (int)((vol + 63) >> 6);
+  {
+    unsigned long long *bitsA = M(0);
+    const long long p0 = (long long)b * vol;
+    for (int w = t; w <= words; w += CHAIN_THREADS) {
+      unsigned long long v = 0;
+      const long long left = vol - 64ll * w;
+      if (left > 0) {
+        const long long p = p0 + 64ll * w;
+        const long long gw = p >> 6;
+        const int sh = (int)(p & 63);
+        v = a.bits[gw] >> sh;
+        if (sh)
+          v |= a.bits[gw + 1] << (64 - sh);
+        if (left < 64)
+          v &= (1ull << left) - 1ull;
+      }
+      bitsA[w] = v;
+    }
+    // the mask of the first output grid starts empty
+    for (int w = t; w < a.maskWords[1]; w += CHAIN_THREADS)
+      M(1)[w] = 0ull;
+  }
+  __syncthreads();
+  unsigned nA;
+  {
+    const unsigned long long *bitsA = M(0);
+    unsigned short *prefA = P(0);
+    nA = chain_scan(
+        words, [&](int i) { return (unsigned)__popcll(bitsA[i]); },
+        [&](int i, unsigned v) { prefA[i] = (unsigned short)v; }, ws);
+  }
+  if ((long long)nA * CHAIN_IN_BYTES > a.arenaBytes) {
+    chain_give_up(a);
+    return;
+  }
+  // entries by rank at the bottom of the arena: key[nA], row[nA]
+  unsigned *keyA = arena, *rowA = arena + nA;
+  {
+    const unsigned long long *bitsA = M(0);
+    const unsigned short *prefA = P(0);
+    const long long p0 = (long long)b * vol;
+    for (int w = t; w < words; w += CHAIN_THREADS) {
+      unsigned long long v = bitsA[w];
+      unsigned r = prefA[w];
+      while (v) {
+        const unsigned key = 64u * w + (unsigned)(__ffsll((long long)v) - 1);
+        v &= v - 1;
+        keyA[r] = key;
+        rowA[r] = (unsigned)hash_find(a.table, a.shift, a.mask, p0 + key);
+        ++r;
+      }
+    }
+  }
+  int bgA = a.bg[b];
+  __syncthreads();
+
+  for (int l = 0; l < a.nLevels; ++l) {
+    const ChainLevel &L = a.lv[l];
+    const unsigned long long *bitsA = M(l % 3);
+    const unsigned short *prefA = P(l & 1);
+    int *st = a.staging + L.stRules + (long long)b * L.capRows * L.width;
+    if (L.kind == CH_TERMINAL) {
+      // terminalGridPoolingRules (TerminalPoolingLayer.cu:8-20): the rows in
+      // iteration order, or the background row of a sample without sites
+      if (nA == 0) {
+        if (t == 0)
+          st[0] = bgA;
+      } else {
+        for (unsigned r = t; r < nA; r += CHAIN_THREADS)
+          st[r] = (int)rowA[r];
+      }
+      if (t == 0) {
+        a.counts[((long long)l * a.batch + b) * 2] = (int)nA;
+        a.counts[((long long)l * a.batch + b) * 2 + 1] = 0;
+      }
+      return; // nothing is recorded behind a terminal layer
+    }
+    if ((long long)nA * CHAIN_IN_BYTES > a.arenaBytes) {
+      chain_give_up(a);
+      return;
+    }
+    Geom g;
+    g.d = D;
+    g.nIn = L.nIn;
+    g.nOut = L.nOut;
+    g.size = L.size;
+    g.stride = L.stride;
+    g.minActive = L.minActive;
+    g.mode = L.mode;
+    g.volIn = vol;
+    long long volOut = 1;
+#pragma unroll
+    for (int q = 0; q < D; ++q)
+      volOut *= L.nOut;
+    g.volOut = volOut;
+    g.width = L.width;
+    g.cube = L.cube;
+    g.ticks = nullptr;
+    g.tInR = g.tOutL = g.tOutR = 0;
+    const bool tri = L.mode == MODE_TRI_NOMIN || L.mode == MODE_TRI_MIN;
+    unsigned long long *bitsB = M((l + 1) % 3);
+    unsigned short *prefB = P((l + 1) & 1);
+    const int wordsB = (int)((volOut + 63) >> 6);
+    // ownership masks and bases beside the input's entries: above them when
+    // those sit at the bottom of the arena (even layers), below them otherwise
+    unsigned *maskS, *keyB, *rowB;
+    unsigned short *baseS;
+    const unsigned halfA = (nA + 1) / 2; // words of nA 16-bit bases
+    if (l & 1) {
+      maskS = keyA - nA - halfA;
+      baseS = reinterpret_cast<unsigned short *>(keyA - halfA);
+    } else {
+      maskS = rowA + nA;
+      baseS = reinterpret_cast<unsigned short *>(maskS + nA);
+    }
+    GridView vin;
+    vin.bits = const_cast<unsigned long long *>(bitsA);
+
+    // -- which candidates each input owns; the output mask
+    for (unsigned r = t; r < nA; r += CHAIN_THREADS) {
+      int i[D], lo[D], hi[D], j[D];
+      decode_key<D>((long long)keyA[r], L.nIn, i);
+      unsigned m = 0;
+      if (cand_box<D>(g, b, i, lo, hi)) {
+#pragma unroll
+        for (int q = 0; q < D; ++q)
+          j[q] = lo[q];
+        for (int c = 0;; ++c) {
+          if (owns<D>(vin, g, b, 0ll, i, j)) {
+            m |= 1u << c;
+            const unsigned ok = (unsigned)encode_key<D>(j, L.nOut);
+            atomicOr(&bitsB[ok >> 6], 1ull << (ok & 63));
+          }
+          int q = D - 1;
+          for (; q >= 0; --q) {
+            if (++j[q] < hi[q])
+              break;
+            j[q] = lo[q];
+          }
+          if (q < 0)
+            break;
+        }
+      }
+      maskS[r] = m;
+    }
+    { // the mask of the grid after the next starts empty (its buffer held
+      // the grid before this layer's input, which nothing reads any more)
+      unsigned long long *z = M((l + 2) % 3);
+      const int nz = a.maskWords[(l + 2) % 3];
+      for (int w = t; w < nz; w += CHAIN_THREADS)
+        z[w] = 0ull;
+    }
+    if (tri && t == 0) { // inverse of RegularTriangularRegions::ord (Regions.cu:810-826)
+      int S = 0;
+      for (int q = 0; q < L.cube; ++q) {
+        int x = q, sum = 0;
+        while (x > 0) {
+          sum += x % L.size;
+          x /= L.size;
+        }
+        if (sum < L.size)
+          invOrd[S++] = q;
+      }
+    }
+    __syncthreads();
+
+    // -- rows of the outputs: prefix sum of the owned counts, and the rank
+    //    prefix of the output mask
+    const unsigned nB = chain_scan(
+        (int)nA, [&](int i) { return (unsigned)__popc(maskS[i]); },
+        [&](int i, unsigned v) { baseS[i] = (unsigned short)v; }, ws);
+    (void)chain_scan(
+        wordsB, [&](int i) { return (unsigned)__popcll(bitsB[i]); },
+        [&](int i, unsigned v) { prefB[i] = (unsigned short)v; }, ws);
+    const int hasBg = (long long)nB < L.fullSize;
+    if ((long long)nA * CHAIN_IN_BYTES + (long long)nB * CHAIN_OUT_BYTES >
+            a.arenaBytes ||
+        (long long)nB + 1 > L.capRows) {
+      chain_give_up(a);
+      return;
+    }
+    if (t == 0) {
+      a.counts[((long long)l * a.batch + b) * 2] = (int)nB;
+      a.counts[((long long)l * a.batch + b) * 2 + 1] = hasBg;
+    }
+    if (l & 1) {
+      keyB = arena;
+      rowB = arena + nB;
+    } else {
+      keyB = arena + arenaWords - 2 * nB;
+      rowB = keyB + nB;
+    }
+    int *stKey = a.staging + L.stKeys + (long long)b * L.capRows;
+
+    // -- the output grid's entries by rank; site keys by row to the staging area
+    for (unsigned r = t; r < nA; r += CHAIN_THREADS) {
+      unsigned m = maskS[r];
+      if (!m)
+        continue;
+      unsigned row = baseS[r];
+      int i[D], lo[D], hi[D], j[D];
+      decode_key<D>((long long)keyA[r], L.nIn, i);
+      (void)cand_box<D>(g, b, i, lo, hi);
+      while (m) { // ascending candidate = ascending output key
+        int rem = __ffs((int)m) - 1;
+        m &= m - 1;
+#pragma unroll
+        for (int q = D - 1; q >= 0; --q) {
+          const int ext = hi[q] - lo[q];
+          j[q] = lo[q] + rem % ext;
+          rem /= ext;
+        }
+        const unsigned ok = (unsigned)encode_key<D>(j, L.nOut);
+        const unsigned rk = lds_rank(bitsB, prefB, ok);
+        keyB[rk] = ok;
+        rowB[rk] = row;
+        stKey[row] = (int)ok;
+        ++row;
+      }
+    }
+    __syncthreads();
+
+    // -- rule rows (sample-local row numbers) to the staging area
+    if (L.rules) {
+      if (!tri && L.size >= 2) {
+        // one lane per run of `size` entries along the innermost axis: their
+        // input sites are neighbours in the mask and in rank
+        const int runsPerRow = L.width / L.size;
+        const unsigned items = nB * (unsigned)runsPerRow;
+        for (unsigned it = t; it < items; it += CHAIN_THREADS) {
+          const unsigned rk = it / runsPerRow;
+          const int run0 = (int)(it - rk * runsPerRow);
+          int run = run0;
+          int j[D], c[D];
+          decode_key<D>((long long)keyB[rk], L.nOut, j);
+          c[D - 1] = j[D - 1] * L.stride;
+#pragma unroll
+          for (int q = D - 2; q >= 0; --q) {
+            c[q] = j[q] * L.stride + run % L.size;
+            run /= L.size;
+          }
+          const unsigned p0 = (unsigned)encode_key<D>(c, L.nIn);
+          const unsigned present = get_bits(bitsA, (long long)p0, L.size);
+          const unsigned rank0 = lds_rank(bitsA, prefA, p0);
+          int *dst = st + (long long)rowB[rk] * L.width + run0 * L.size;
+          for (int q = 0; q < L.size; ++q)
+            dst[q] = (present >> q) & 1u
+                         ? (int)rowA[rank0 + __popc(present & ((1u << q) - 1u))]
+                         : bgA;
+        }
+      } else {
+        const unsigned items = nB * (unsigned)L.width;
+        for (unsigned it = t; it < items; it += CHAIN_THREADS) {
+          const unsigned rk = it / L.width;
+          const int q = (int)(it - rk * L.width);
+          int off = tri ? invOrd[q] : q;
+          int j[D], c[D];
+          decode_key<D>((long long)keyB[rk], L.nOut, j);
+#pragma unroll
+          for (int x = D - 1; x >= 0; --x) {
+            c[x] = j[x] * L.stride + off % L.size;
+            off /= L.size;
+          }
+          const unsigned p = (unsigned)encode_key<D>(c, L.nIn);
+          const bool present = (bitsA[p >> 6] >> (p & 63)) & 1ull;
+          st[(long long)rowB[rk] * L.width + q] =
+              present ? (int)rowA[lds_rank(bitsA, prefA, p)] : bgA;
+        }
+      }
+      if (hasBg) // the all-background row (Regions.cu:647-652)
+        for (int q = t; q < L.width; q += CHAIN_THREADS)
+          st[(long long)nB * L.width + q] = bgA;
+    }
+    __syncthreads();
+    // the output grid is the next layer's input
+    keyA = keyB;
+    rowA = rowB;
+    nA = nB;
+    bgA = hasBg ? (int)nB : -1;
+    vol = volOut;
+  }
+}
+
+// Sums over the samples of a layer's counts: what lies before sample b, the
+// totals, and the largest sample.
+struct PlaceSums {
+  long long actBefore, bgBefore, actAll, bgAll, maxAct;
+};
+__device__ __forceinline__ PlaceSums place_sums(const int *cnt, int batch, int b,
+                                                long long *red) {
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  long long v[5] = {0, 0, 0, 0, 0};
+  for (int s = t; s < batch; s += CHAIN_THREADS) {
+    const int n = cnt[2 * s], h = cnt[2 * s + 1];
+    if (s < b) {
+      v[0] += n;
+      v[1] += h;
+    }
+    v[2] += n;
+    v[3] += h;
+    v[4] = n > v[4] ? n : v[4];
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      v[k] += __shfl_xor(v[k], off, 64);
+    const long long o = __shfl_xor(v[4], off, 64);
+    v[4] = o > v[4] ? o : v[4];
+  }
+  __syncthreads(); // (red may still be read from an earlier call)
+  if (lane == 0)
+#pragma unroll
+    for (int k = 0; k < 5; ++k)
+      red[wave * 5 + k] = v[k];
+  __syncthreads();
+  PlaceSums r = {0, 0, 0, 0, 0};
+#pragma unroll
+  for (int w = 0; w < CHAIN_WAVES; ++w) {
+    r.actBefore += red[w * 5 + 0];
+    r.bgBefore += red[w * 5 + 1];
+    r.actAll += red[w * 5 + 2];
+    r.bgAll += red[w * 5 + 3];
+    r.maxAct = red[w * 5 + 4] > r.maxAct ? red[w * 5 + 4] : r.maxAct;
+  }
+  return r;
+}
+
+__global__ void __launch_bounds__(CHAIN_THREADS) k_chain_place(ChainArgs a) {
+  __shared__ long long red[CHAIN_WAVES * 5];
+  const int b = blockIdx.x, l = blockIdx.y, t = threadIdx.x;
+  const ChainLevel &L = a.lv[l];
+  const int *cnt = a.counts + (long long)l * a.batch * 2;
+  const bool gaveUp = *reinterpret_cast<volatile unsigned long long *>(a.flag) == a.ticket;
+  const PlaceSums me = place_sums(cnt, a.batch, b, red);
+  long long inBase = 0; // first row of this sample in the layer's input
+  if (l > 0) {
+    const PlaceSums in = place_sums(cnt - (long long)a.batch * 2, a.batch, b, red);
+    inBase = in.actBefore + in.bgBefore;
+  }
+  const bool terminal = L.kind == CH_TERMINAL;
+  long long nSites, nActive, width;
+  bool over = gaveUp;
+  if (terminal) {
+    width = me.maxAct > 1 ? me.maxAct : 1; // TerminalPoolingLayer.cu:90-96
+    nSites = nActive = a.batch;
+    over = over || width > L.boundRows ||
+           (L.rules && width * a.batch > L.capacity);
+  } else {
+    width = L.width;
+    nSites = me.actAll + me.bgAll;
+    nActive = me.actAll;
+    over = over || nSites > L.boundRows || nActive > L.boundActive ||
+           (L.rules && nSites * width > L.capacity);
+  }
+  if (b == 0 && t == 0) {
+    L.meta[META_SITES] = over ? 0 : nSites;
+    L.meta[META_ACTIVE] = over ? 0 : nActive;
+    L.meta[META_OVERFLOW] = over;
+    L.meta[META_WIDTH] = terminal ? width : 0;
+    volatile long long *slot = a.scalars + 16 + 4 * L.slot;
+    slot[0] = nSites;
+    slot[1] = nActive;
+    slot[2] = over;
+    slot[3] = terminal ? width : me.maxAct;
+    if (l == 0)
+      a.scalars[15] = *a.badSites;
+  }
+  if (over)
+    return;
+  const int n = cnt[2 * b], hasBg = cnt[2 * b + 1];
+  const int *st = a.staging + L.stRules + (long long)b * L.capRows * L.width;
+  if (terminal) {
+    if (L.rules) {
+      const int have = n > 1 ? n : 1;
+      int *dst = L.rules + (long long)b * width;
+      for (long long i = t; i < width; i += CHAIN_THREADS) {
+        int v = -1;
+        if (i < have) {
+          v = st[i];
+          v = v < 0 ? v : v + (int)inBase;
+        }
+        dst[i] = v;
+      }
+    }
+    if (t == 0) { // the output grid: site 0 of sample b is row b
+      L.ekey[b] = b;
+      L.erow[b] = b;
+      L.bg[b] = -1;
+    }
+    return;
+  }
+  const long long rowBase = me.actBefore + me.bgBefore;
+  if (L.rules) {
+    const long long total = (long long)(n + hasBg) * L.width;
+    int *dst = L.rules + rowBase * L.width;
+    for (long long i = t; i < total; i += CHAIN_THREADS) {
+      const int v = st[i];
+      dst[i] = v < 0 ? v : v + (int)inBase;
+    }
+  }
+  const int *stKey = a.staging + L.stKeys + (long long)b * L.capRows;
+  long long volOut = 1;
+  for (int q = 0; q < a.d; ++q)
+    volOut *= L.nOut;
+  for (int i = t; i < n; i += CHAIN_THREADS) {
+    L.ekey[me.actBefore + i] = (long long)b * volOut + stKey[i];
+    L.erow[me.actBefore + i] = (int)(rowBase + i);
+  }
+  if (t == 0)
+    L.bg[b] = hasBg ? (int)(rowBase + n) : -1;
+}
+
+// -------------------------------------------------------------------- host
+
+static ChainState *chain_state(scn_ctx *ctx) {
+  if (!ctx->chain)
+    ctx->chain = new ChainState();
+  return ctx->chain;
+}
+
+void scn_chain_release(scn_ctx *ctx) {
+  if (!ctx->chain)
+    return;
+  ctx->chain->staging.release();
+  ctx->chain->counts.release();
+  ctx->chain->flag.release();
+  delete ctx->chain;
+  ctx->chain = nullptr;
+}
+
+extern "C" int scn_ctx_chain_rules(scn_ctx *ctx, int on) {
+  SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_ctx_chain_rules: null context");
+  if (!on)
+    SCN_TRY(scn_chain_flush(ctx));
+  chain_state(ctx)->on = on != 0;
+  return SCN_OK;
+}
+
+extern "C" int scn_ctx_chain_count(scn_ctx *ctx, int64_t *chains, int64_t *plans) {
+  SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_ctx_chain_count: null context");
+  if (chains)
+    *chains = ctx->chain ? ctx->chain->nChains : 0;
+  if (plans)
+    *plans = ctx->chain ? ctx->chain->nPlans : 0;
+  return SCN_OK;
+}
+
+// LDS bytes of everything but the arena for a chain over grids of these
+// volumes (the source first); fills the layout when `a` is given
+static long long chain_fixed_lds(const std::vector<long long> &vols, ChainArgs *a) {
+  long long mw[3] = {1, 1, 1}, pw[2] = {1, 1};
+  for (size_t k = 0; k < vols.size(); ++k) {
+    const long long w = (vols[k] + 63) / 64 + 1;
+    mw[k % 3] = w > mw[k % 3] ? w : mw[k % 3];
+    pw[k & 1] = w > pw[k & 1] ? w : pw[k & 1];
+  }
+  long long off = CHAIN_HEADER_BYTES;
+  for (int x = 0; x < 3; ++x) {
+    if (a) {
+      a->maskOff[x] = (int)off;
+      a->maskWords[x] = (int)mw[x];
+    }
+    off += 8 * mw[x];
+  }
+  for (int x = 0; x < 2; ++x) {
+    if (a)
+      a->prefOff[x] = (int)off;
+    off += (2 * pw[x] + 15) / 16 * 16;
+  }
+  if (a)
+    a->arenaOff = (int)off;
+  return off;
+}
+
+static std::vector<long long> chain_volumes(const ChainState *cs) {
+  std::vector<long long> vols;
+  if (cs->recs.empty())
+    return vols;
+  vols.push_back(cs->recs[0].in->vol);
+  for (const ChainRec &r : cs->recs)
+    if (r.lv.kind == CH_REGIONS)
+      vols.push_back(r.geom.volOut);
+  return vols;
+}
+
+// Can a plan from `in` into `out` join the chain being recorded?
+static bool chain_accepts(scn_ctx *ctx, const scn_grids *in, const scn_grids *out,
+                          long long volOut) {
+  ChainState *cs = ctx->chain;
+  if (!cs || !cs->on || !ctx->deferCounts)
+    return false;
+  if ((int)ctx->pendingGrids.size() >= SCN_MAX_PENDING ||
+      (int)cs->recs.size() >= CHAIN_MAX_LEVELS)
+    return false;
+  if (in->batch < 1 || in->d < 1 || in->d > 3 || in->vol >= (1ll << 31))
+    return false;
+  if (cs->recs.empty()) {
+    // the source: grids with a table and a mask, counts known
+    if (in->pending || !in->indexValid)
+      return false;
+  } else {
+    const ChainRec &last = cs->recs.back();
+    if (last.out != in || last.lv.kind == CH_TERMINAL)
+      return false;
+  }
+  for (const ChainRec &r : cs->recs)
+    if (r.out == out || r.in == out)
+      return false;
+  std::vector<long long> vols = chain_volumes(cs);
+  if (vols.empty())
+    vols.push_back(in->vol);
+  vols.push_back(volOut);
+  return chain_fixed_lds(vols, nullptr) + CHAIN_MIN_ARENA <= CHAIN_LDS_MAX;
+}
+
+static void chain_mark_output(scn_ctx *ctx, scn_grids *in, scn_grids *out,
+                              int n, long long vol, long long boundActive,
+                              long long boundRows, int slot) {
+  out->batch = in->batch;
+  out->d = in->d;
+  out->n = n;
+  out->vol = vol;
+  out->nActive = boundActive;
+  out->nSites = (int)boundRows;
+  out->rankValid = false;
+  out->indexValid = false;
+  out->chained = true;
+  out->planIn = in;
+  mark_pending(ctx, out, slot);
+}
+
+int scn_chain_record_regions(scn_ctx *ctx, scn_grids *in, scn_grids *out,
+                             const Geom &g, long long fullSize,
+                             long long maxCand, int64_t *nOutSites,
+                             bool *taken) {
+  *taken = false;
+  if (g.mode == MODE_SQ_FMP || maxCand > 32 || g.cube > 64 || out->seenRows <= 0 ||
+      !chain_accepts(ctx, in, out, g.volOut))
+    return SCN_OK;
+  ChainState *cs = ctx->chain;
+  const long long volOutAll = (long long)in->batch * g.volOut;
+  const long long boundActive = grow_bound(out->seenActive, 64, volOutAll);
+  const long long boundRows = grow_bound(out->seenRows, 64, boundActive + in->batch);
+  if (boundRows >= 2147483647ll)
+    return SCN_OK;
+  SCN_TRY(out->meta.reserve(8));
+  SCN_TRY(out->ekey.reserve((size_t)boundActive + 1));
+  SCN_TRY(out->erow.reserve((size_t)boundActive + 1));
+  SCN_TRY(out->bg.reserve((size_t)in->batch + 1));
+  ChainRec r;
+  r.in = in;
+  r.out = out;
+  r.geom = g;
+  r.filled = false;
+  ChainLevel &L = r.lv;
+  memset(&L, 0, sizeof(L));
+  L.kind = CH_REGIONS;
+  L.mode = g.mode;
+  L.nIn = g.nIn;
+  L.nOut = g.nOut;
+  L.size = g.size;
+  L.stride = g.stride;
+  L.minActive = g.minActive;
+  L.width = g.width;
+  L.cube = g.cube;
+  L.fullSize = fullSize;
+  L.slot = (int)ctx->pendingGrids.size();
+  L.ekey = out->ekey.p;
+  L.erow = out->erow.p;
+  L.bg = out->bg.p;
+  L.meta = out->meta.p;
+  L.boundRows = boundRows;
+  L.boundActive = boundActive;
+  cs->recs.push_back(r);
+  chain_mark_output(ctx, in, out, g.nOut, g.volOut, boundActive, boundRows, L.slot);
+  out->geom = g;
+  out->planKind = PLAN_REGIONS;
+  *nOutSites = boundRows;
+  *taken = true;
+  return SCN_OK;
+}
+
+int scn_chain_record_terminal(scn_ctx *ctx, scn_grids *in, scn_grids *out,
+                              int64_t *ruleWidth, bool *taken) {
+  *taken = false;
+  if (out->seenWidth <= 0 || !chain_accepts(ctx, in, out, 1))
+    return SCN_OK;
+  ChainState *cs = ctx->chain;
+  const long long boundWidth = grow_bound(out->seenWidth, 8, in->vol);
+  SCN_TRY(out->meta.reserve(8));
+  SCN_TRY(out->ekey.reserve((size_t)in->batch + 1));
+  SCN_TRY(out->erow.reserve((size_t)in->batch + 1));
+  SCN_TRY(out->bg.reserve((size_t)in->batch + 1));
+  ChainRec r;
+  r.in = in;
+  r.out = out;
+  memset(&r.geom, 0, sizeof(r.geom));
+  r.geom.volOut = 1;
+  r.filled = false;
+  ChainLevel &L = r.lv;
+  memset(&L, 0, sizeof(L));
+  L.kind = CH_TERMINAL;
+  L.nOut = 1;
+  L.width = 1;
+  L.fullSize = 1;
+  L.slot = (int)ctx->pendingGrids.size();
+  L.ekey = out->ekey.p;
+  L.erow = out->erow.p;
+  L.bg = out->bg.p;
+  L.meta = out->meta.p;
+  L.boundRows = boundWidth;
+  L.boundActive = in->batch;
+  cs->recs.push_back(r);
+  chain_mark_output(ctx, in, out, 1, 1, in->batch, in->batch, L.slot);
+  out->termS = boundWidth;
+  out->planKind = PLAN_TERMINAL;
+  *ruleWidth = boundWidth;
+  *taken = true;
+  return SCN_OK;
+}
+
+int scn_chain_record_fill(scn_ctx *ctx, const scn_grids *in, scn_grids *out,
+                          int32_t *d_rules, int64_t capacity, bool *taken) {
+  *taken = false;
+  ChainState *cs = ctx->chain;
+  if (!cs || cs->recs.empty())
+    return SCN_OK;
+  ChainRec &r = cs->recs.back();
+  if (r.out != out || r.in != in || r.filled)
+    return SCN_OK;
+  const long long total = r.lv.kind == CH_TERMINAL
+                              ? (long long)in->batch * out->termS
+                              : (long long)out->nSites * r.lv.width;
+  SCN_REQUIRE(capacity >= total, SCN_ERR_CAPACITY,
+              "scn_rules_fill: %lld rules, capacity %lld", total,
+              (long long)capacity);
+  SCN_REQUIRE(d_rules || total == 0, SCN_ERR_ARG,
+              "scn_rules_fill: null rules buffer");
+  r.lv.rules = d_rules;
+  r.lv.capacity = capacity;
+  r.filled = true;
+  *taken = true;
+  return SCN_OK;
+}
+
+int scn_chain_flush(scn_ctx *ctx) {
+  ChainState *cs = ctx->chain;
+  if (!cs || cs->recs.empty())
+    return SCN_OK;
+  std::vector<ChainRec> recs;
+  recs.swap(cs->recs);
+  cs->nChains += 1;
+  cs->nPlans += (long long)recs.size();
+  ProfScope ps(ctx, SCN_K_RULES);
+  scn_grids *src = recs[0].in;
+  ChainArgs a;
+  memset(&a, 0, sizeof(a));
+  a.nLevels = (int)recs.size();
+  a.batch = src->batch;
+  a.d = src->d;
+  a.n0 = src->n;
+  a.table = src->table.p;
+  a.shift = 64 - src->log2cap;
+  a.mask = (1u << src->log2cap) - 1u;
+  a.bits = src->bits.p;
+  a.bg = src->bg.p;
+  a.vol0 = src->vol;
+  std::vector<long long> vols;
+  vols.push_back(src->vol);
+  for (const ChainRec &r : recs)
+    if (r.lv.kind == CH_REGIONS)
+      vols.push_back(r.geom.volOut);
+  const long long fixed = chain_fixed_lds(vols, &a);
+  // the arena: sized from the largest sample seen at any layer, or as large
+  // as the LDS allows while that is unknown or has proved too tight
+  long long arena = CHAIN_LDS_MAX - fixed;
+  long long sampleBound = 0;
+  bool known = !cs->wide;
+  for (const ChainRec &r : recs)
+    if (r.lv.kind == CH_REGIONS) {
+      known = known && r.out->seenSample > 0;
+      sampleBound = r.out->seenSample > sampleBound ? r.out->seenSample : sampleBound;
+    }
+  if (known) {
+    sampleBound += sampleBound / 2 + 64;
+    long long want = (CHAIN_IN_BYTES + CHAIN_OUT_BYTES) * sampleBound;
+    want = want < CHAIN_MIN_ARENA ? CHAIN_MIN_ARENA : want;
+    arena = want < arena ? want : arena;
+  }
+  arena = arena / 16 * 16;
+  a.arenaBytes = (int)arena;
+  const long long entriesMax = arena / CHAIN_OUT_BYTES;
+  long long stagingInts = 0;
+  for (int l = 0; l < a.nLevels; ++l) {
+    ChainLevel &L = recs[l].lv;
+    long long cap = entriesMax < L.fullSize ? entriesMax : L.fullSize;
+    if (L.kind == CH_TERMINAL)
+      cap = entriesMax; // rows of the input that one sample may list
+    else if (known) {
+      const long long tight = 2 * recs[l].out->seenSample + 64;
+      cap = tight < cap ? tight : cap;
+    }
+    L.capRows = (int)cap + 1;
+    L.stRules = stagingInts;
+    stagingInts += (long long)a.batch * L.capRows * L.width;
+    stagingInts = (stagingInts + 3) / 4 * 4;
+    L.stKeys = stagingInts;
+    stagingInts += (long long)a.batch * L.capRows;
+    stagingInts = (stagingInts + 3) / 4 * 4;
+    a.lv[l] = L;
+  }
+  SCN_TRY(cs->staging.reserve((size_t)stagingInts + 4));
+  SCN_TRY(cs->counts.reserve((size_t)a.nLevels * a.batch * 2 + 2));
+  if (!cs->flag.p) {
+    SCN_TRY(cs->flag.reserve(2));
+    SCN_TRY(scn_fill32(ctx, cs->flag.p, 0u, 4));
+  }
+  a.staging = cs->staging.p;
+  a.counts = cs->counts.p;
+  a.flag = cs->flag.p;
+  a.ticket = (unsigned long long)++ctx->ticket;
+  a.scalars = (long long *)ctx->d_pinned;
+  a.badSites = (const long long *)(ctx->d_scalars + 15);
+  const size_t ldsBytes = (size_t)(fixed + arena);
+  {
+    // (above 64 KB of LDS a kernel has to be told so once)
+    static std::once_flag once;
+    static hipError_t attr = hipSuccess;
+    std::call_once(once, [] {
+      const void *k[3] = {reinterpret_cast<const void *>(&k_chain_sample<1>),
+                          reinterpret_cast<const void *>(&k_chain_sample<2>),
+                          reinterpret_cast<const void *>(&k_chain_sample<3>)};
+      for (int i = 0; i < 3 && attr == hipSuccess; ++i)
+        attr = hipFuncSetAttribute(k[i], hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   CHAIN_LDS_MAX);
+    });
+    SCN_HIP_CHECK(attr);
+  }
+  const dim3 grid((unsigned)a.batch), block(CHAIN_THREADS);
+  switch (a.d) {
+  case 1:
+    hipLaunchKernelGGL(k_chain_sample<1>, grid, block, ldsBytes, ctx->stream, a);
+    break;
+  case 2:
+    hipLaunchKernelGGL(k_chain_sample<2>, grid, block, ldsBytes, ctx->stream, a);
+    break;
+  default:
+    hipLaunchKernelGGL(k_chain_sample<3>, grid, block, ldsBytes, ctx->stream, a);
+    break;
+  }
+  SCN_HIP_CHECK(hipGetLastError());
+  hipLaunchKernelGGL(k_chain_place, dim3((unsigned)a.batch, (unsigned)a.nLevels),
+                     dim3(CHAIN_THREADS), 0, ctx->stream, a);
+  SCN_HIP_CHECK(hipGetLastError());
+  return SCN_OK;
+}
+
+// what scn_rules_settle learns about a chained plan from its pinned slot
+void scn_chain_settled(scn_ctx *ctx, scn_grids *g, long long sampleMax,
+                       bool overflowed) {
+  if (overflowed) {
+    if (ctx->chain)
+      ctx->chain->wide = true;
+    return;
+  }
+  if (g->planKind == PLAN_REGIONS)
+    g->seenSample = sampleMax > g->seenSample ? sampleMax : g->seenSample;
+}

@@ -57,6 +57,7 @@ struct scn_ctx {
   bool deferCounts;
   bool wstream; // NiN: W-streaming kernel allowed (SCN_NIN_WSTREAM=0 turns it off)
   std::vector<struct scn_grids *> pendingGrids;
+  struct ChainState *chain; // recorded rule-book plans (scn_chain.hip)
   // profiling
   bool prof;
   int profTag;
@@ -110,6 +111,10 @@ static inline int scn_ceil_div(int64_t a, int64_t b) {
 
 // address of the static scratch of scn_sgemm_ABt_static on `device` (scn_train.hip)
 int scn_abt_static_setup(int device);
+
+// runs the recorded rule-book plans of the context, if any (scn_chain.hip)
+int scn_chain_flush(scn_ctx *ctx);
+void scn_chain_release(scn_ctx *ctx);
 
 // exclusive prefix sum of n uint32 values; out has n + 1 elements (out[n] =
 // total).  `tmp` must hold scn_scan_tmp_elems(n) uint32.

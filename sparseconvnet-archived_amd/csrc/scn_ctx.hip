@@ -32,6 +32,7 @@ extern "C" int scn_ctx_create(int device, scn_ctx **out) {
   c->profTag = 0;
   c->ticket = 0;
   c->deferCounts = false;
+  c->chain = nullptr;
   {
     const char *e = getenv("SCN_NIN_WSTREAM");
     c->wstream = !(e && e[0] == '0');
@@ -57,7 +58,9 @@ extern "C" int scn_ctx_create(int device, scn_ctx **out) {
 extern "C" int scn_ctx_destroy(scn_ctx *c) {
   if (!c)
     return SCN_OK;
+  (void)scn_chain_flush(c);
   (void)hipStreamSynchronize(c->stream);
+  scn_chain_release(c);
   for (auto &s : c->spans) {
     (void)hipEventDestroy(s.a);
     (void)hipEventDestroy(s.b);

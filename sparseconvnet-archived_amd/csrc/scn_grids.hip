@@ -22,360 +22,7 @@
 #include <atomic>
 #include "scn_scan_dev.h"
 
-struct __align__(16) Slot {
-  long long key;
-  int row;
-  int pad;
-};
-#define SLOT_EMPTY (-1LL)
-
-enum { MODE_SQ_NOMIN = 0, MODE_SQ_MIN, MODE_SQ_VALID, MODE_TRI_NOMIN, MODE_TRI_MIN, MODE_SQ_FMP };
-enum { PLAN_NONE = 0, PLAN_REGIONS = 1, PLAN_TERMINAL = 2 };
-
-struct Geom {
-  int d;
-  int nIn, nOut, size, stride, minActive, mode;
-  long long volIn, volOut;
-  int width; // rule-row width: size^d or triangleSize(size, d)
-  int cube;  // size^d
-  // MODE_SQ_FMP: per-sample, per-axis region tables (fractional max-pooling).
-  // inputL at ticks[(b d + a) nOut + j], inputR the same at tInR; outputL and
-  // outputR at tOutL / tOutR + (b d + a) nIn + i.  Null otherwise.
-  const int *ticks;
-  long long tInR, tOutL, tOutR;
-};
-__device__ __forceinline__ int fmp_inputL(const Geom &g, int b, int a, int j) {
-  return g.ticks[((long long)b * g.d + a) * g.nOut + j];
-}
-__device__ __forceinline__ int fmp_inputR(const Geom &g, int b, int a, int j) {
-  return g.ticks[g.tInR + ((long long)b * g.d + a) * g.nOut + j];
-}
-
-struct GridView {
-  Slot *table;
-  unsigned shift, mask;
-  unsigned long long *bits;
-  const unsigned *prefix;
-  const int *bg;
-  long long vol;
-  int n, d, batch;
-};
-
-// A count the host may not know yet: an upper bound, and where the real value
-// is (device memory written by an earlier kernel of the same stream); live ==
-// null means the bound is exact.
-struct Count {
-  long long bound;
-  const long long *live;
-};
-__device__ __forceinline__ long long count_now(const Count &c) {
-  if (!c.live)
-    return c.bound;
-  const long long v = *c.live;
-  return v < c.bound ? v : c.bound;
-}
-// per-grids device record
-enum { META_SITES = 0, META_ACTIVE = 1, META_OVERFLOW = 2, META_WIDTH = 3 };
-
-struct scn_grids {
-  int batch = 0, d = 0, n = 0;
-  long long vol = 0;
-  long long nActive = 0;
-  int nSites = 0;
-  unsigned log2cap = 0;
-  size_t nWords = 0;
-  bool rankValid = false;
-  // how much of table / bits is known to be empty right now (scn_grids_clear_many)
-  size_t cleanSlots = 0, cleanWords = 0;
-  // Deferred counts: while pending, nActive / nSites / termS hold upper bounds
-  // and the real values are in meta (device) and on their way to the pinned
-  // slot; seen* are the largest values this object has ever held, from which
-  // the next bounds are derived.
-  bool pending = false;
-  int pinnedSlot = -1;
-  long long seenRows = 0, seenActive = 0, seenWidth = 0;
-  DevBuf<long long> meta; // META_* words
-  DevBuf<Slot> table;
-  DevBuf<unsigned long long> bits;
-  DevBuf<unsigned> prefix;
-  DevBuf<long long> ekey;
-  DevBuf<int> erow;
-  DevBuf<int> bg;
-  DevBuf<unsigned> scanTmp;
-  // state of the plan that produced this object
-  int planKind = PLAN_NONE;
-  const scn_grids *planIn = nullptr;
-  Geom geom;
-  long long termS = 0;
-  DevBuf<long long> siteKey; // per output row: packed key, or -1 - sample for a background row
-  DevBuf<unsigned> cnt, base;
-  DevBuf<unsigned long long> ownMask;
-  DevBuf<unsigned> rankOf;
-  DevBuf<int> bgBefore;
-  DevBuf<unsigned> sampleStart;
-  DevBuf<int> invOrd;
-  DevBuf<int> ticks; // region tables of a fractional max-pooling plan
-  // scratch for download
-  DevBuf<int> dlSample, dlRow;
-  DevBuf<long long> dlKey;
-};
-
-// ---------------------------------------------------------------- device
-
-__device__ __forceinline__ unsigned hash_slot(long long p, unsigned shift) {
-  return (unsigned)(((unsigned long long)p * 0x9E3779B97F4A7C15ull) >> shift);
-}
-
-__device__ __forceinline__ void hash_insert(Slot *t, unsigned shift,
-                                            unsigned mask, long long p,
-                                            int row) {
-  unsigned s = hash_slot(p, shift);
-  for (;;) {
-    unsigned long long prev =
-        atomicCAS((unsigned long long *)&t[s].key,
-                  (unsigned long long)SLOT_EMPTY, (unsigned long long)p);
-    if (prev == (unsigned long long)SLOT_EMPTY ||
-        prev == (unsigned long long)p) {
-      t[s].row = row;
-      return;
-    }
-    s = (s + 1) & mask;
-  }
-}
-
-__device__ __forceinline__ int hash_find(const Slot *t, unsigned shift,
-                                         unsigned mask, long long p) {
-  unsigned s = hash_slot(p, shift);
-  for (;;) {
-    const int4 v = *reinterpret_cast<const int4 *>(&t[s]); // one 128-bit load
-    long long k = ((long long)v.y << 32) | (unsigned)v.x;
-    if (k == p)
-      return v.z;
-    if (k == SLOT_EMPTY)
-      return -1;
-    s = (s + 1) & mask;
-  }
-}
-
-// `len` (1..32) mask bits starting at bit position p
-__device__ __forceinline__ unsigned get_bits(const unsigned long long *bits,
-                                             long long p, int len) {
-  long long w = p >> 6;
-  int sh = (int)(p & 63);
-  unsigned long long lo = bits[w] >> sh;
-  if (sh + len > 64)
-    lo |= bits[w + 1] << (64 - sh);
-  unsigned m = (len >= 32) ? 0xFFFFFFFFu : ((1u << len) - 1u);
-  return (unsigned)lo & m;
-}
-
-__device__ __forceinline__ unsigned rank_of(const GridView &g, long long p) {
-  long long w = p >> 6;
-  int sh = (int)(p & 63);
-  unsigned long long below = sh ? (g.bits[w] & ((1ull << sh) - 1ull)) : 0ull;
-  return g.prefix[w] + (unsigned)__popcll(below);
-}
-
-__device__ __forceinline__ int sq_outputL(int size, int stride, int i) {
-  int v = (i - size + stride) / stride; // truncation toward zero, as in C
-  return v > 0 ? v : 0;
-}
-__device__ __forceinline__ int sq_outputR(int stride, int nOut, int i) {
-  int v = i / stride + 1;
-  return v < nOut ? v : nOut;
-}
-
-template <int D>
-__device__ __forceinline__ void decode_key(long long key, int n, int *c) {
-#pragma unroll
-  for (int a = D - 1; a >= 0; --a) {
-    c[a] = (int)(key % n);
-    key /= n;
-  }
-}
-template <int D>
-__device__ __forceinline__ long long encode_key(const int *c, int n) {
-  long long k = 0;
-#pragma unroll
-  for (int a = 0; a < D; ++a)
-    k = k * n + c[a];
-  return k;
-}
-
-// Is any site of the window with origin w active at a window offset that
-// precedes offset a (row-major)?  The window has ext[axis] sites along each
-// axis (all equal for the regular regions).
-template <int D>
-__device__ __forceinline__ bool any_before(const unsigned long long *bits,
-                                           long long sampleBase, int nIn,
-                                           const int *ext, const int *w,
-                                           const int *a) {
-  if (D == 1) {
-    return a[0] > 0 && get_bits(bits, sampleBase + w[0], a[0]) != 0;
-  } else if (D == 2) {
-    for (int q0 = 0; q0 < a[0]; ++q0)
-      if (get_bits(bits, sampleBase + (long long)(w[0] + q0) * nIn + w[1], ext[1]))
-        return true;
-    return a[1] > 0 &&
-           get_bits(bits, sampleBase + (long long)(w[0] + a[0]) * nIn + w[1],
-                    a[1]) != 0;
-  } else {
-    for (int q0 = 0; q0 <= a[0]; ++q0) {
-      int q1max = (q0 < a[0]) ? ext[1] : a[1];
-      for (int q1 = 0; q1 < q1max; ++q1)
-        if (get_bits(bits,
-                     sampleBase +
-                         ((long long)(w[0] + q0) * nIn + (w[1] + q1)) * nIn +
-                         w[2],
-                     ext[2]))
-          return true;
-    }
-    return a[2] > 0 &&
-           get_bits(bits,
-                    sampleBase +
-                        ((long long)(w[0] + a[0]) * nIn + (w[1] + a[1])) * nIn +
-                        w[2],
-                    a[2]) != 0;
-  }
-}
-
-// number of active sites in the window; TRI counts only offsets with
-// coordinate sum < size
-template <int D, bool TRI>
-__device__ __forceinline__ int count_active(const unsigned long long *bits,
-                                            long long sampleBase, int nIn,
-                                            int size, const int *w) {
-  int c = 0;
-  if (D == 1) {
-    c = __popc(get_bits(bits, sampleBase + w[0], size));
-  } else if (D == 2) {
-    for (int q0 = 0; q0 < size; ++q0) {
-      int len = TRI ? size - q0 : size;
-      c += __popc(get_bits(bits, sampleBase + (long long)(w[0] + q0) * nIn + w[1], len));
-    }
-  } else {
-    for (int q0 = 0; q0 < size; ++q0) {
-      int q1n = TRI ? size - q0 : size;
-      for (int q1 = 0; q1 < q1n; ++q1) {
-        int len = TRI ? size - q0 - q1 : size;
-        c += __popc(get_bits(
-            bits,
-            sampleBase + ((long long)(w[0] + q0) * nIn + (w[1] + q1)) * nIn + w[2],
-            len));
-      }
-    }
-  }
-  return c;
-}
-
-// The box [lo, hi) of output sites whose window holds the input site i
-// (Regions.cu:13-29), or for valid mode the single site (i0-1, i1-1) when
-// 1 <= i <= nOut on each axis (Regions.cu:693-697).  False when empty.
-template <int D>
-__device__ __forceinline__ bool cand_box(const Geom &g, int b, const int *i,
-                                         int *lo, int *hi) {
-  if (g.mode == MODE_SQ_FMP) { // tables (Regions.cu:143-150)
-#pragma unroll
-    for (int a = 0; a < D; ++a) {
-      const long long t = ((long long)b * g.d + a) * g.nIn + i[a];
-      lo[a] = g.ticks[g.tOutL + t];
-      hi[a] = g.ticks[g.tOutR + t];
-      if (lo[a] >= hi[a])
-        return false;
-    }
-  } else if (g.mode == MODE_SQ_VALID) {
-#pragma unroll
-    for (int a = 0; a < D; ++a) {
-      if (i[a] < 1 || i[a] > g.nOut)
-        return false;
-      lo[a] = i[a] - 1;
-      hi[a] = i[a];
-    }
-  } else {
-#pragma unroll
-    for (int a = 0; a < D; ++a) {
-      lo[a] = sq_outputL(g.size, g.stride, i[a]);
-      hi[a] = sq_outputR(g.stride, g.nOut, i[a]);
-      if (lo[a] >= hi[a])
-        return false;
-    }
-  }
-  return true;
-}
-
-// Does input site i of sample b own candidate output j?  (the active input
-// with the smallest key in j's window owns it; Min modes also need enough
-// active inputs; the triangular lattice only has outputs with sum(j) < nOut)
-template <int D>
-__device__ __forceinline__ bool owns(const GridView &in, const Geom &g, int b,
-                                     long long sampleBase, const int *i,
-                                     const int *j) {
-  if (g.mode == MODE_TRI_NOMIN || g.mode == MODE_TRI_MIN) {
-    int sum = 0;
-#pragma unroll
-    for (int a = 0; a < D; ++a)
-      sum += j[a];
-    if (sum >= g.nOut) // Regions.cu:874,900
-      return false;
-  }
-  if (g.mode == MODE_SQ_VALID)
-    return true;
-  int w[D], off[D], ext[D];
-  if (g.mode == MODE_SQ_FMP) {
-#pragma unroll
-    for (int a = 0; a < D; ++a) {
-      w[a] = fmp_inputL(g, b, a, j[a]);
-      ext[a] = fmp_inputR(g, b, a, j[a]) - w[a];
-      off[a] = i[a] - w[a];
-    }
-  } else {
-#pragma unroll
-    for (int a = 0; a < D; ++a) {
-      w[a] = j[a] * g.stride;
-      ext[a] = g.size;
-      off[a] = i[a] - w[a];
-    }
-  }
-  if (any_before<D>(in.bits, sampleBase, g.nIn, ext, w, off))
-    return false;
-  if (g.mode == MODE_SQ_MIN)
-    return count_active<D, false>(in.bits, sampleBase, g.nIn, g.size, w) >=
-           g.minActive;
-  if (g.mode == MODE_TRI_MIN)
-    return count_active<D, true>(in.bits, sampleBase, g.nIn, g.size, w) >=
-           g.minActive;
-  return true;
-}
-
-// Visits, in ascending output key, the output sites owned by the input site
-// with coordinates i of sample b; f(outKey, c) is called for each, c being the
-// position of the site among the candidates of the box.
-template <int D, typename F>
-__device__ __forceinline__ void for_each_owned(const GridView &in,
-                                               const Geom &g, int b,
-                                               const int *i, F f) {
-  int lo[D], hi[D];
-  if (!cand_box<D>(g, b, i, lo, hi))
-    return;
-  const long long sampleBase = (long long)b * g.volIn;
-  int j[D];
-#pragma unroll
-  for (int a = 0; a < D; ++a)
-    j[a] = lo[a];
-  for (int c = 0;; ++c) {
-    if (owns<D>(in, g, b, sampleBase, i, j))
-      f(encode_key<D>(j, g.nOut), c);
-    // odometer, last axis fastest
-    int a = D - 1;
-    for (; a >= 0; --a) {
-      if (++j[a] < hi[a])
-        break;
-      j[a] = lo[a];
-    }
-    if (a < 0)
-      break;
-  }
-}
+#include "scn_grids_dev.h"
 
 __global__ void k_grid_build(GridView g, const int *sample,
                              const long long *key, const int *row, long long n,
@@ -979,7 +626,7 @@ __global__ void k_find(GridView g, const int *sample, const long long *key,
 
 // ------------------------------------------------------------------ host
 
-static GridView view_of(const scn_grids *g) {
+GridView view_of(const scn_grids *g) {
   GridView v;
   v.table = g->table.p;
   v.shift = 64 - g->log2cap;
@@ -1019,6 +666,8 @@ static int grids_prepare(scn_ctx *ctx, scn_grids *g, int batch, int d, int n,
   g->vol = vol;
   g->nActive = nActive;
   g->rankValid = false;
+  g->indexValid = true;
+  g->chained = false;
   g->planKind = PLAN_NONE;
   g->planIn = nullptr;
   g->pending = false;
@@ -1075,6 +724,7 @@ __global__ void k_clear_many(ClearList l) {
 extern "C" int scn_grids_clear_many(scn_ctx *ctx, scn_grids **grids, int n) {
   SCN_REQUIRE(ctx && (grids || n == 0) && n >= 0, SCN_ERR_ARG,
               "scn_grids_clear_many: bad argument");
+  SCN_TRY(scn_chain_flush(ctx));
   for (int first = 0; first < n; first += CLEAR_MANY) {
     ClearList l;
     int m = 0;
@@ -1082,6 +732,11 @@ extern "C" int scn_grids_clear_many(scn_ctx *ctx, scn_grids **grids, int n) {
     for (int i = first; i < n && i < first + CLEAR_MANY; ++i) {
       scn_grids *g = grids[i];
       if (!g || (!g->table.p && !g->bits.p))
+        continue;
+      // nothing to do for grids whose table and mask are not in use (a chain
+      // of recorded plans fills the entry list only) or are empty already
+      if (!g->indexValid || ((!g->table.p || g->cleanSlots >= g->table.cap) &&
+                             (!g->bits.p || g->cleanWords >= g->bits.cap)))
         continue;
       l.slots[m] = (uint4 *)g->table.p;
       l.nSlots[m] = g->table.p ? g->table.cap : 0;
@@ -1105,7 +760,44 @@ extern "C" int scn_grids_clear_many(scn_ctx *ctx, scn_grids **grids, int n) {
   return SCN_OK;
 }
 
+// table and mask of grids that only hold their entry list
+__global__ void k_grid_index(GridView g, const long long *ekey, const int *erow,
+                             Count n, const long long *meta) {
+  long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= n.bound || (meta && meta[META_OVERFLOW]) || e >= count_now(n))
+    return;
+  const long long p = ekey[e];
+  hash_insert(g.table, g.shift, g.mask, p, erow[e]);
+  atomicOr(&g.bits[p >> 6], 1ull << (p & 63));
+}
+static Count count_active(const scn_grids *g);
+static int ensure_index(scn_ctx *ctx, scn_grids *g) {
+  if (g->indexValid)
+    return SCN_OK;
+  SCN_TRY(scn_chain_flush(ctx));
+  // (grids_prepare forgets the plan and the deferral: they are put back)
+  const int planKind = g->planKind, nSites = g->nSites, pinnedSlot = g->pinnedSlot;
+  const scn_grids *planIn = g->planIn;
+  const bool pending = g->pending, chained = g->chained;
+  const long long nActive = g->nActive;
+  SCN_TRY(grids_prepare(ctx, g, g->batch, g->d, g->n, nActive));
+  g->planKind = planKind;
+  g->planIn = planIn;
+  g->nSites = nSites;
+  g->pending = pending;
+  g->pinnedSlot = pinnedSlot;
+  g->chained = chained;
+  if (nActive > 0) {
+    hipLaunchKernelGGL(k_grid_index, dim3(scn_ceil_div(nActive, 256)), dim3(256),
+                       0, ctx->stream, view_of(g), g->ekey.p, g->erow.p,
+                       count_active(g), pending ? g->meta.p : nullptr);
+    SCN_HIP_CHECK(hipGetLastError());
+  }
+  return SCN_OK;
+}
+
 static int ensure_rank(scn_ctx *ctx, scn_grids *g) {
+  SCN_TRY(ensure_index(ctx, g));
   if (g->rankValid)
     return SCN_OK;
   SCN_TRY(g->scanTmp.reserve(scn_scan_tmp_elems(g->nWords + 1)));
@@ -1166,7 +858,7 @@ static Count count_width(const scn_grids *g) {
   c.live = g->pending ? g->meta.p + META_WIDTH : nullptr;
   return c;
 }
-static long long grow_bound(long long seen, long long slack, long long cap) {
+long long grow_bound(long long seen, long long slack, long long cap) {
   long long b = seen + seen / 4 + slack;
   return b < cap ? b : cap;
 }
@@ -1183,6 +875,7 @@ extern "C" int scn_ctx_defer_counts(scn_ctx *ctx, int on) {
 }
 extern "C" int scn_rules_settle(scn_ctx *ctx) {
   SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_rules_settle: null context");
+  SCN_TRY(scn_chain_flush(ctx));
   if (ctx->pendingGrids.empty())
     return SCN_OK;
   SCN_HIP_CHECK(hipStreamSynchronize(ctx->stream));
@@ -1190,6 +883,8 @@ extern "C" int scn_rules_settle(scn_ctx *ctx) {
   bool overflowed = false;
   for (scn_grids *g : ctx->pendingGrids) {
     const volatile int64_t *slot = ctx->h_pinned + 16 + 4 * g->pinnedSlot;
+    if (g->chained)
+      scn_chain_settled(ctx, g, slot[3], slot[2] != 0);
     if (slot[2]) {
       overflowed = true;
       g->planKind = PLAN_NONE; // nothing was emitted
@@ -1221,7 +916,7 @@ extern "C" int scn_rules_settle(scn_ctx *ctx) {
               "plans; plan it again with deferral off");
   return SCN_OK;
 }
-static void mark_pending(scn_ctx *ctx, scn_grids *g, int slot) {
+void mark_pending(scn_ctx *ctx, scn_grids *g, int slot) {
   g->pending = true;
   g->pinnedSlot = slot;
   ctx->pendingGrids.push_back(g);
@@ -1237,6 +932,7 @@ extern "C" int scn_grids_destroy(scn_ctx *ctx, scn_grids *g) {
   if (!g)
     return SCN_OK;
   if (ctx) {
+    (void)scn_chain_flush(ctx);
     (void)hipStreamSynchronize(ctx->stream);
     auto &pl = ctx->pendingGrids;
     for (size_t i = 0; i < pl.size(); ++i)
@@ -1280,6 +976,7 @@ extern "C" int scn_grids_build(scn_ctx *ctx, scn_grids *g, int batch,
               "scn_grids_build: null site arrays");
   SCN_REQUIRE(batch == 0 || d_background, SCN_ERR_ARG,
               "scn_grids_build: null background array");
+  SCN_TRY(scn_chain_flush(ctx));
   ProfScope ps(ctx, SCN_K_GRID_BUILD);
   SCN_TRY(grids_prepare(ctx, g, batch, dimension, spatialSize, n));
   g->nSites = nSpatialSites;
@@ -1349,6 +1046,7 @@ extern "C" int scn_grids_find(scn_ctx *ctx, const scn_grids *g,
   SCN_REQUIRE(ctx && g, SCN_ERR_ARG, "scn_grids_find: null argument");
   if (n <= 0)
     return SCN_OK;
+  SCN_TRY(ensure_index(ctx, const_cast<scn_grids *>(g)));
   hipLaunchKernelGGL(k_find, dim3(scn_ceil_div(n, 256)), dim3(256), 0,
                      ctx->stream, view_of(g), d_sample,
                      (const long long *)d_key, (long long)n, d_row);
@@ -1520,6 +1218,18 @@ static int plan_regions(scn_ctx *ctx, const scn_grids *cin, scn_grids *out,
     g.width = g.cube;
     fullSize = g.volOut;
   }
+  {
+    // a plan that can wait joins the chain of recorded plans
+    long long maxCand = 1;
+    for (int a = 0; a < in->d; ++a)
+      maxCand *= g.mode == MODE_SQ_VALID ? 1 : (size + stride - 1) / stride;
+    bool taken = false;
+    SCN_TRY(scn_chain_record_regions(ctx, in, out, g, fullSize, maxCand,
+                                     nOutSites, &taken));
+    if (taken)
+      return SCN_OK;
+    SCN_TRY(scn_chain_flush(ctx));
+  }
   ProfScope ps(ctx, SCN_K_RULES);
   SCN_TRY(ensure_rank(ctx, in));
   int rc;
@@ -1637,6 +1347,7 @@ extern "C" int scn_rules_fmp_plan(scn_ctx *ctx, const scn_grids *cin,
   g.tInR = (long long)nT;
   g.tOutL = (long long)(2 * nT);
   g.tOutR = (long long)(2 * nT + nI);
+  SCN_TRY(scn_chain_flush(ctx));
   ProfScope ps(ctx, SCN_K_RULES);
   SCN_TRY(out->ticks.reserve(t.size() + 1));
   // (the copy returns when done: `t` may go out of scope)
@@ -1669,6 +1380,13 @@ extern "C" int scn_rules_terminal_plan(scn_ctx *ctx, const scn_grids *cin,
               "terminal rules plan: null argument");
   SCN_REQUIRE(in != out, SCN_ERR_ARG,
               "terminal rules plan: in and out are the same object");
+  {
+    bool taken = false;
+    SCN_TRY(scn_chain_record_terminal(ctx, in, out, ruleWidth, &taken));
+    if (taken)
+      return SCN_OK;
+    SCN_TRY(scn_chain_flush(ctx));
+  }
   ProfScope ps(ctx, SCN_K_RULES);
   const bool deferred = ctx->deferCounts && out->seenWidth > 0 &&
                         (int)ctx->pendingGrids.size() < SCN_MAX_PENDING;
@@ -1721,6 +1439,17 @@ extern "C" int scn_rules_fill(scn_ctx *ctx, const scn_grids *in,
   SCN_REQUIRE(ctx && in && out, SCN_ERR_ARG, "scn_rules_fill: null argument");
   SCN_REQUIRE(out->planKind != PLAN_NONE && out->planIn == in, SCN_ERR_STATE,
               "scn_rules_fill: `out` does not hold a plan made from `in`");
+  {
+    bool taken = false;
+    SCN_TRY(scn_chain_record_fill(ctx, in, out, d_rules, capacity, &taken));
+    if (taken)
+      return SCN_OK;
+    SCN_TRY(scn_chain_flush(ctx));
+  }
+  SCN_REQUIRE(!out->chained, SCN_ERR_STATE,
+              "scn_rules_fill: the rules of a recorded plan are written when "
+              "the chain runs; plan again to fill another buffer");
+  SCN_TRY(ensure_index(ctx, const_cast<scn_grids *>(in)));
   ProfScope ps(ctx, SCN_K_RULES);
   GridView vin = view_of(in);
   if (out->planKind == PLAN_TERMINAL) {

@@ -1,0 +1,387 @@
+// Types and device helpers shared by the translation units that build sparse
+// grids and rule books (scn_grids.hip: one layer at a time through tables in
+// HBM; scn_chain.hip: all layers of a net at once, one workgroup per sample).
+#pragma once
+#include "scn_common.h"
+#include "scn_scan_dev.h"
+
+struct __align__(16) Slot {
+  long long key;
+  int row;
+  int pad;
+};
+#define SLOT_EMPTY (-1LL)
+
+enum { MODE_SQ_NOMIN = 0, MODE_SQ_MIN, MODE_SQ_VALID, MODE_TRI_NOMIN, MODE_TRI_MIN, MODE_SQ_FMP };
+enum { PLAN_NONE = 0, PLAN_REGIONS = 1, PLAN_TERMINAL = 2 };
+
+struct Geom {
+  int d;
+  int nIn, nOut, size, stride, minActive, mode;
+  long long volIn, volOut;
+  int width; // rule-row width: size^d or triangleSize(size, d)
+  int cube;  // size^d
+  // MODE_SQ_FMP: per-sample, per-axis region tables (fractional max-pooling).
+  // inputL at ticks[(b d + a) nOut + j], inputR the same at tInR; outputL and
+  // outputR at tOutL / tOutR + (b d + a) nIn + i.  Null otherwise.
+  const int *ticks;
+  long long tInR, tOutL, tOutR;
+};
+__device__ __forceinline__ int fmp_inputL(const Geom &g, int b, int a, int j) {
+  return g.ticks[((long long)b * g.d + a) * g.nOut + j];
+}
+__device__ __forceinline__ int fmp_inputR(const Geom &g, int b, int a, int j) {
+  return g.ticks[g.tInR + ((long long)b * g.d + a) * g.nOut + j];
+}
+
+struct GridView {
+  Slot *table;
+  unsigned shift, mask;
+  unsigned long long *bits;
+  const unsigned *prefix;
+  const int *bg;
+  long long vol;
+  int n, d, batch;
+};
+
+// A count the host may not know yet: an upper bound, and where the real value
+// is (device memory written by an earlier kernel of the same stream); live ==
+// null means the bound is exact.
+struct Count {
+  long long bound;
+  const long long *live;
+};
+__device__ __forceinline__ long long count_now(const Count &c) {
+  if (!c.live)
+    return c.bound;
+  const long long v = *c.live;
+  return v < c.bound ? v : c.bound;
+}
+// per-grids device record
+enum { META_SITES = 0, META_ACTIVE = 1, META_OVERFLOW = 2, META_WIDTH = 3 };
+
+struct scn_grids {
+  int batch = 0, d = 0, n = 0;
+  long long vol = 0;
+  long long nActive = 0;
+  int nSites = 0;
+  unsigned log2cap = 0;
+  size_t nWords = 0;
+  bool rankValid = false;
+  // table, mask and prefix describe the entries (false for grids a chain of
+  // recorded plans produced: those hold the entry list, backgroundCol and the
+  // counts, and the rest is built from them on demand)
+  bool indexValid = true;
+  bool chained = false; // plan and rules came from a chain of recorded plans
+  long long seenSample = 0; // most active sites one sample has had (chained plans)
+  // how much of table / bits is known to be empty right now (scn_grids_clear_many)
+  size_t cleanSlots = 0, cleanWords = 0;
+  // Deferred counts: while pending, nActive / nSites / termS hold upper bounds
+  // and the real values are in meta (device) and on their way to the pinned
+  // slot; seen* are the largest values this object has ever held, from which
+  // the next bounds are derived.
+  bool pending = false;
+  int pinnedSlot = -1;
+  long long seenRows = 0, seenActive = 0, seenWidth = 0;
+  DevBuf<long long> meta; // META_* words
+  DevBuf<Slot> table;
+  DevBuf<unsigned long long> bits;
+  DevBuf<unsigned> prefix;
+  DevBuf<long long> ekey;
+  DevBuf<int> erow;
+  DevBuf<int> bg;
+  DevBuf<unsigned> scanTmp;
+  // state of the plan that produced this object
+  int planKind = PLAN_NONE;
+  const scn_grids *planIn = nullptr;
+  Geom geom;
+  long long termS = 0;
+  DevBuf<long long> siteKey; // per output row: packed key, or -1 - sample for a background row
+  DevBuf<unsigned> cnt, base;
+  DevBuf<unsigned long long> ownMask;
+  DevBuf<unsigned> rankOf;
+  DevBuf<int> bgBefore;
+  DevBuf<unsigned> sampleStart;
+  DevBuf<int> invOrd;
+  DevBuf<int> ticks; // region tables of a fractional max-pooling plan
+  // scratch for download
+  DevBuf<int> dlSample, dlRow;
+  DevBuf<long long> dlKey;
+};
+
+// ---------------------------------------------------------------- device
+
+__device__ __forceinline__ unsigned hash_slot(long long p, unsigned shift) {
+  return (unsigned)(((unsigned long long)p * 0x9E3779B97F4A7C15ull) >> shift);
+}
+
+__device__ __forceinline__ void hash_insert(Slot *t, unsigned shift,
+                                            unsigned mask, long long p,
+                                            int row) {
+  unsigned s = hash_slot(p, shift);
+  for (;;) {
+    unsigned long long prev =
+        atomicCAS((unsigned long long *)&t[s].key,
+                  (unsigned long long)SLOT_EMPTY, (unsigned long long)p);
+    if (prev == (unsigned long long)SLOT_EMPTY ||
+        prev == (unsigned long long)p) {
+      t[s].row = row;
+      return;
+    }
+    s = (s + 1) & mask;
+  }
+}
+
+__device__ __forceinline__ int hash_find(const Slot *t, unsigned shift,
+                                         unsigned mask, long long p) {
+  unsigned s = hash_slot(p, shift);
+  for (;;) {
+    const int4 v = *reinterpret_cast<const int4 *>(&t[s]); // one 128-bit load
+    long long k = ((long long)v.y << 32) | (unsigned)v.x;
+    if (k == p)
+      return v.z;
+    if (k == SLOT_EMPTY)
+      return -1;
+    s = (s + 1) & mask;
+  }
+}
+
+// `len` (1..32) mask bits starting at bit position p
+__device__ __forceinline__ unsigned get_bits(const unsigned long long *bits,
+                                             long long p, int len) {
+  long long w = p >> 6;
+  int sh = (int)(p & 63);
+  unsigned long long lo = bits[w] >> sh;
+  if (sh + len > 64)
+    lo |= bits[w + 1] << (64 - sh);
+  unsigned m = (len >= 32) ? 0xFFFFFFFFu : ((1u << len) - 1u);
+  return (unsigned)lo & m;
+}
+
+__device__ __forceinline__ unsigned rank_of(const GridView &g, long long p) {
+  long long w = p >> 6;
+  int sh = (int)(p & 63);
+  unsigned long long below = sh ? (g.bits[w] & ((1ull << sh) - 1ull)) : 0ull;
+  return g.prefix[w] + (unsigned)__popcll(below);
+}
+
+__device__ __forceinline__ int sq_outputL(int size, int stride, int i) {
+  int v = (i - size + stride) / stride; // truncation toward zero, as in C
+  return v > 0 ? v : 0;
+}
+__device__ __forceinline__ int sq_outputR(int stride, int nOut, int i) {
+  int v = i / stride + 1;
+  return v < nOut ? v : nOut;
+}
+
+template <int D>
+__device__ __forceinline__ void decode_key(long long key, int n, int *c) {
+#pragma unroll
+  for (int a = D - 1; a >= 0; --a) {
+    c[a] = (int)(key % n);
+    key /= n;
+  }
+}
+template <int D>
+__device__ __forceinline__ long long encode_key(const int *c, int n) {
+  long long k = 0;
+#pragma unroll
+  for (int a = 0; a < D; ++a)
+    k = k * n + c[a];
+  return k;
+}
+
+// Is any site of the window with origin w active at a window offset that
+// precedes offset a (row-major)?  The window has ext[axis] sites along each
+// axis (all equal for the regular regions).
+template <int D>
+__device__ __forceinline__ bool any_before(const unsigned long long *bits,
+                                           long long sampleBase, int nIn,
+                                           const int *ext, const int *w,
+                                           const int *a) {
+  if (D == 1) {
+    return a[0] > 0 && get_bits(bits, sampleBase + w[0], a[0]) != 0;
+  } else if (D == 2) {
+    for (int q0 = 0; q0 < a[0]; ++q0)
+      if (get_bits(bits, sampleBase + (long long)(w[0] + q0) * nIn + w[1], ext[1]))
+        return true;
+    return a[1] > 0 &&
+           get_bits(bits, sampleBase + (long long)(w[0] + a[0]) * nIn + w[1],
+                    a[1]) != 0;
+  } else {
+    for (int q0 = 0; q0 <= a[0]; ++q0) {
+      int q1max = (q0 < a[0]) ? ext[1] : a[1];
+      for (int q1 = 0; q1 < q1max; ++q1)
+        if (get_bits(bits,
+                     sampleBase +
+                         ((long long)(w[0] + q0) * nIn + (w[1] + q1)) * nIn +
+                         w[2],
+                     ext[2]))
+          return true;
+    }
+    return a[2] > 0 &&
+           get_bits(bits,
+                    sampleBase +
+                        ((long long)(w[0] + a[0]) * nIn + (w[1] + a[1])) * nIn +
+                        w[2],
+                    a[2]) != 0;
+  }
+}
+
+// number of active sites in the window; TRI counts only offsets with
+// coordinate sum < size
+template <int D, bool TRI>
+__device__ __forceinline__ int count_active(const unsigned long long *bits,
+                                            long long sampleBase, int nIn,
+                                            int size, const int *w) {
+  int c = 0;
+  if (D == 1) {
+    c = __popc(get_bits(bits, sampleBase + w[0], size));
+  } else if (D == 2) {
+    for (int q0 = 0; q0 < size; ++q0) {
+      int len = TRI ? size - q0 : size;
+      c += __popc(get_bits(bits, sampleBase + (long long)(w[0] + q0) * nIn + w[1], len));
+    }
+  } else {
+    for (int q0 = 0; q0 < size; ++q0) {
+      int q1n = TRI ? size - q0 : size;
+      for (int q1 = 0; q1 < q1n; ++q1) {
+        int len = TRI ? size - q0 - q1 : size;
+        c += __popc(get_bits(
+            bits,
+            sampleBase + ((long long)(w[0] + q0) * nIn + (w[1] + q1)) * nIn + w[2],
+            len));
+      }
+    }
+  }
+  return c;
+}
+
+// The box [lo, hi) of output sites whose window holds the input site i
+// (Regions.cu:13-29), or for valid mode the single site (i0-1, i1-1) when
+// 1 <= i <= nOut on each axis (Regions.cu:693-697).  False when empty.
+template <int D>
+__device__ __forceinline__ bool cand_box(const Geom &g, int b, const int *i,
+                                         int *lo, int *hi) {
+  if (g.mode == MODE_SQ_FMP) { // tables (Regions.cu:143-150)
+#pragma unroll
+    for (int a = 0; a < D; ++a) {
+      const long long t = ((long long)b * g.d + a) * g.nIn + i[a];
+      lo[a] = g.ticks[g.tOutL + t];
+      hi[a] = g.ticks[g.tOutR + t];
+      if (lo[a] >= hi[a])
+        return false;
+    }
+  } else if (g.mode == MODE_SQ_VALID) {
+#pragma unroll
+    for (int a = 0; a < D; ++a) {
+      if (i[a] < 1 || i[a] > g.nOut)
+        return false;
+      lo[a] = i[a] - 1;
+      hi[a] = i[a];
+    }
+  } else {
+#pragma unroll
+    for (int a = 0; a < D; ++a) {
+      lo[a] = sq_outputL(g.size, g.stride, i[a]);
+      hi[a] = sq_outputR(g.stride, g.nOut, i[a]);
+      if (lo[a] >= hi[a])
+        return false;
+    }
+  }
+  return true;
+}
+
+// Does input site i of sample b own candidate output j?  (the active input
+// with the smallest key in j's window owns it; Min modes also need enough
+// active inputs; the triangular lattice only has outputs with sum(j) < nOut)
+template <int D>
+__device__ __forceinline__ bool owns(const GridView &in, const Geom &g, int b,
+                                     long long sampleBase, const int *i,
+                                     const int *j) {
+  if (g.mode == MODE_TRI_NOMIN || g.mode == MODE_TRI_MIN) {
+    int sum = 0;
+#pragma unroll
+    for (int a = 0; a < D; ++a)
+      sum += j[a];
+    if (sum >= g.nOut) // Regions.cu:874,900
+      return false;
+  }
+  if (g.mode == MODE_SQ_VALID)
+    return true;
+  int w[D], off[D], ext[D];
+  if (g.mode == MODE_SQ_FMP) {
+#pragma unroll
+    for (int a = 0; a < D; ++a) {
+      w[a] = fmp_inputL(g, b, a, j[a]);
+      ext[a] = fmp_inputR(g, b, a, j[a]) - w[a];
+      off[a] = i[a] - w[a];
+    }
+  } else {
+#pragma unroll
+    for (int a = 0; a < D; ++a) {
+      w[a] = j[a] * g.stride;
+      ext[a] = g.size;
+      off[a] = i[a] - w[a];
+    }
+  }
+  if (any_before<D>(in.bits, sampleBase, g.nIn, ext, w, off))
+    return false;
+  if (g.mode == MODE_SQ_MIN)
+    return count_active<D, false>(in.bits, sampleBase, g.nIn, g.size, w) >=
+           g.minActive;
+  if (g.mode == MODE_TRI_MIN)
+    return count_active<D, true>(in.bits, sampleBase, g.nIn, g.size, w) >=
+           g.minActive;
+  return true;
+}
+
+// Visits, in ascending output key, the output sites owned by the input site
+// with coordinates i of sample b; f(outKey, c) is called for each, c being the
+// position of the site among the candidates of the box.
+template <int D, typename F>
+__device__ __forceinline__ void for_each_owned(const GridView &in,
+                                               const Geom &g, int b,
+                                               const int *i, F f) {
+  int lo[D], hi[D];
+  if (!cand_box<D>(g, b, i, lo, hi))
+    return;
+  const long long sampleBase = (long long)b * g.volIn;
+  int j[D];
+#pragma unroll
+  for (int a = 0; a < D; ++a)
+    j[a] = lo[a];
+  for (int c = 0;; ++c) {
+    if (owns<D>(in, g, b, sampleBase, i, j))
+      f(encode_key<D>(j, g.nOut), c);
+    // odometer, last axis fastest
+    int a = D - 1;
+    for (; a >= 0; --a) {
+      if (++j[a] < hi[a])
+        break;
+      j[a] = lo[a];
+    }
+    if (a < 0)
+      break;
+  }
+}
+
+
+// ---- host helpers shared by scn_grids.hip and scn_chain.hip
+GridView view_of(const scn_grids *g);
+long long grow_bound(long long seen, long long slack, long long cap);
+void mark_pending(scn_ctx *ctx, scn_grids *g, int slot);
+
+// Chains of recorded plans (scn_chain.hip).  The record functions set *taken
+// when the call joined the chain being recorded; otherwise the caller runs it
+// the ordinary way (after scn_chain_flush).
+int scn_chain_record_regions(scn_ctx *ctx, scn_grids *in, scn_grids *out,
+                             const Geom &g, long long fullSize,
+                             long long maxCand, int64_t *nOutSites,
+                             bool *taken);
+int scn_chain_record_terminal(scn_ctx *ctx, scn_grids *in, scn_grids *out,
+                              int64_t *ruleWidth, bool *taken);
+int scn_chain_record_fill(scn_ctx *ctx, const scn_grids *in, scn_grids *out,
+                          int32_t *d_rules, int64_t capacity, bool *taken);
+void scn_chain_settled(scn_ctx *ctx, scn_grids *g, long long sampleMax,
+                       bool overflowed);

@@ -82,6 +82,9 @@ public:
   // training batches are drawn in shuffled order (BatchProducer.cu:23-26);
   // a harness that needs a fixed order turns this off
   bool shuffleTrainingData = true;
+  // rule books of consecutive layers are built together, one workgroup per
+  // sample, where the library can (scn_ctx_chain_rules); off: layer by layer
+  bool chainRuleBooks = true;
   void finishBatch(SpatiallySparseBatch &batch, std::ofstream &f,
                    std::ofstream &g);
   void processBatch(SpatiallySparseBatch &batch, float learningRate,

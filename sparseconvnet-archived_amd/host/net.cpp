@@ -255,8 +255,11 @@ static void buildRuleBooks(SparseConvNetCUDA &cnn, scn_ctx *ctx,
       cnn.layers[i]->preprocess(b, b.interfaces[i], b.interfaces[i + 1]);
     }
   };
+  // (plans that continue from one another are recorded and run together)
   SCN_CHECKED(scn_ctx_defer_counts(ctx, 1));
+  SCN_CHECKED(scn_ctx_chain_rules(ctx, cnn.chainRuleBooks ? 1 : 0));
   all();
+  SCN_CHECKED(scn_ctx_chain_rules(ctx, 0));
   SCN_CHECKED(scn_ctx_defer_counts(ctx, 0));
   const int rc = scn_rules_settle(ctx);
   if (rc == SCN_ERR_CAPACITY) {

@@ -106,6 +106,9 @@ int scnh_finish_headless(scnh_net *net, int topSpatialSize) {
 void scnh_set_fused_convolutions(scnh_net *net, int on) {
   net->cnn->setFusedConvolutions(on != 0);
 }
+void scnh_set_chained_rule_books(scnh_net *net, int on) {
+  net->cnn->chainRuleBooks = on != 0;
+}
 void scnh_set_precision(scnh_net *net, int precision) {
   net->cnn->setPrecision(precision);
 }

@@ -34,6 +34,8 @@ int scnh_finish_headless(scnh_net *net, int topSpatialSize);
 void scnh_set_precision(scnh_net *net, int precision);
 /* SparseConvNetCUDA::setFusedConvolutions */
 void scnh_set_fused_convolutions(scnh_net *net, int on);
+/* rule books of consecutive layers built together (default) or layer by layer */
+void scnh_set_chained_rule_books(scnh_net *net, int on);
 int scnh_input_spatial_size(scnh_net *net);
 int scnh_n_layers(scnh_net *net);
 /* kind: 0 conv, 1 triangular conv, 2 NiN, 3 NiN PReLU, 4 max-pool,

@@ -43,6 +43,7 @@ def lib():
         "scnh_finish_headless": (i32, [vp, i32]),
         "scnh_set_precision": (None, [vp, i32]),
         "scnh_set_fused_convolutions": (None, [vp, i32]),
+        "scnh_set_chained_rule_books": (None, [vp, i32]),
         "scnh_input_spatial_size": (i32, [vp]),
         "scnh_n_layers": (i32, [vp]),
         "scnh_layer_info": (i32, [vp, i32, P(i32), P(i32), P(i32)]),
@@ -248,6 +249,9 @@ class Net:
 
     def setFusedConvolutions(self, on=True):
         lib().scnh_set_fused_convolutions(self.h, int(on))
+
+    def setChainedRuleBooks(self, on=True):
+        lib().scnh_set_chained_rule_books(self.h, int(on))
 
     def setPrecision(self, precision):
         lib().scnh_set_precision(self.h, precision)
