@@ -4,12 +4,17 @@
 A step is one forward pass of one synthetic batch through the C++ host classes
 (SparseConvNet) on top of libscn_hip.so: grid hash build, every rule book,
 gather / NiN / max-pool / terminal pool / softmax kernels, and the copy of the
-class probabilities back to the host.  The batch's active sites and input
-features are already in HBM when the timed region starts.
+class probabilities back to the host.  `value` is measured with the batch's
+active sites and input features already in HBM when the timed region starts;
+`with_input_upload` is the same pass with sites and features in pinned host
+memory, uploaded for every batch (the forward time that also counts the H2D of
+the inputs).  Warm-up and timed batches are one pass: the producer threads are
+not restarted in between.
 
 Prints ONE JSON line: active sites/s (value) and samples/s, the roofline of the
-kernel family that takes the most time, a per-kernel table, and the CPU oracle
-timed on this host's cores beside it.
+kernel -- or the rule-book construction as a whole -- that takes the most GPU
+time, the busiest NiN contraction beside it, a per-kernel table, and the CPU
+oracle timed on this host's cores.
 """
 import argparse
 import json
@@ -29,27 +34,20 @@ MFMA_PEAK_TFLOPS = {"fp32": 157.3, "bf16": 2500.0, "bf16x3": 2500.0 / 3}
 BALANCE_FLOP_PER_BYTE = {k: v * 1e12 / 8e12 for k, v in MFMA_PEAK_TFLOPS.items()}
 
 
-# HBM bytes per launch (read + written) measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by
-# a copy kernel of known size; the runs are summarised in profiles/hbm_traffic_c2.txt and hbm_traffic_c5.txt.
-# Only valid for the default batch and seed of the config with fused convolutions (the default).
-MEASURED_TRAFFIC = {
-    ("c2_sparse_net_2d", "gather", 0): 2.66e6 + 4.01e6,
-    ("c2_sparse_net_2d", "nin", 1): 4.06e6 + 10.70e6,
-    ("c2_sparse_net_2d", "maxpool", 2): 14.57e6 + 10.77e6,
-    ("c2_sparse_net_2d", "conv_nin", 4): 7.56e6 + 15.48e6,
-    ("c2_sparse_net_2d", "maxpool", 5): 22.66e6 + 11.76e6,
-    ("c2_sparse_net_2d", "conv_nin", 7): 8.12e6 + 11.45e6,
-    ("c2_sparse_net_2d", "maxpool", 8): 17.42e6 + 8.01e6,
-    ("c2_sparse_net_2d", "conv_nin", 10): 10.07e6 + 5.98e6,
-    ("c2_sparse_net_2d", "maxpool", 11): 8.42e6 + 3.35e6,
-    ("c2_sparse_net_2d", "conv_nin", 13): 16.48e6 + 1.58e6,
-    ("c2_sparse_net_2d", "maxpool", 14): 1.79e6 + 0.51e6,
-    ("c2_sparse_net_2d", "nin", 15): 2.66e6 + 0.31e6,
-    ("c2_sparse_net_2d", "nin", 17): 0.89e6 + 0.04e6,
-    ("c5_spatiotemporal_3d", "conv_nin", 1): 717.18e6 + 845.62e6,
-    ("c5_spatiotemporal_3d", "conv_nin", 3): 1816.42e6 + 1614.81e6,
-    ("c5_spatiotemporal_3d", "maxpool", 4): 1651.12e6 + 522.02e6,
-}
+# HBM bytes per launch (read + written) measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by a
+# copy kernel of known size: kept in a file beside the profiles it was taken from, with the commit it was measured at.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic_bench.json")
+
+
+def measured_traffic():
+    """{(workload, kernel family, layer): bytes per launch}, the commit of the measurement (or {} and None)."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            t = json.load(f)
+    except (OSError, ValueError):
+        return {}, None
+    table = {(e["workload"], e["kernel"], e["layer"]): e["read_bytes"] + e["written_bytes"] for e in t["entries"]}
+    return table, t.get("measured_at_commit")
 
 
 def parse():
@@ -171,20 +169,27 @@ def main():
               file=sys.stderr)
         del src, dst, ident
 
-    def run(n):
-        # n batches the way processDataset runs them: producer threads build
-        # grids and rule books on their own streams while this thread runs the
-        # forward pass of the previous batch
-        done = net.forward_resident_stream(n, B, dS.ptr, dK.ptr, dR.ptr, dBg.ptr, active, nSites, dF.ptr, probs)
-        assert done == n
+    # pinned host copies of the inputs, for the pass that uploads them with every batch
+    def pinned(a):
+        h = ctx.host_alloc(a.nbytes)
+        np.frombuffer(h.buffer(), a.dtype, a.size)[:] = a.reshape(-1)
+        return h
 
-    run(args.warmup)
+    hS, hK, hR, hBg, hF = (pinned(np.ascontiguousarray(x)) for x in
+                           (S.astype(np.int32), K.astype(np.int64), R.astype(np.int32), bg.astype(np.int32),
+                            feats.astype(np.float32)))
+    # warm-up and timed batches the way processDataset runs them, in ONE pass: producer threads build grids and
+    # rule books on their own streams while this thread runs the forward pass of the previous batch; the clock
+    # starts when the last warm-up batch is finished and the net's stream is idle, and the producers meanwhile
+    # hold the next batches ready, as in the middle of any dataset pass
+    dt = net.forward_stream_timed(args.warmup, args.steps, B, dS.ptr, dK.ptr, dR.ptr, dBg.ptr, active, nSites, dF.ptr,
+                                  inputs_on_host=False, h_probs=probs)
     ctx.sync()
-    t0 = time.perf_counter()
-    run(args.steps)
-    ctx.sync()
-    dt = time.perf_counter() - t0
     ms_per_step = 1e3 * dt / args.steps
+    dt_up = net.forward_stream_timed(args.warmup, args.steps, B, hS.ptr, hK.ptr, hR.ptr, hBg.ptr, active, nSites,
+                                     hF.ptr, inputs_on_host=True, h_probs=probs)
+    ctx.sync()
+    upload_bytes = int(S.size * 4 + K.size * 8 + R.size * 4 + bg.size * 4 + feats.size * 4)
     # one batch at a time on one stream, nothing overlapped: the latency of a batch
     for _ in range(3):
         step()
@@ -269,20 +274,53 @@ def main():
     fam_ms = {}
     for e in kernels:
         fam_ms[e["kernel"]] = fam_ms.get(e["kernel"], 0.0) + e["ms_per_step"]
+    # Rule-book construction as a whole (every layer's plan and fill, recorded and run together as two kernels, or
+    # layer by layer): a span of it covers several launches, so it is priced as one family against the algorithmic
+    # bytes of all rule books of a step
+    rule_spans = [e for e in kernels if e["kernel"] == "rules"]
+    rules_entry = None
+    if rule_spans:
+        r_ms = sum(e["ms_per_step"] for e in rule_spans)
+        r_launches = sum(e["launches_per_step"] for e in rule_spans)
+        r_ms_k = max(r_ms - span_floor_ms * r_launches, 1e-6)
+        r_bytes = sum(b_ for (fam, _), (b_, _f) in work.items() if fam == "rules")
+        a = r_bytes / (r_ms_k * 1e-3) / 1e9
+        rules_entry = dict(kernel="rules", layer="all", ms_per_step=round(r_ms, 5), ms_kernel=round(r_ms_k, 5),
+                           launches_per_step=r_launches, bound="hbm", achieved=round(a, 3), peak=HBM_PEAK_GBS,
+                           unit="GB/s", frac=round(a / HBM_PEAK_GBS, 5), algorithmic_bytes=int(r_bytes), traffic=None,
+                           note="latency-bound integer work: one workgroup per sample walks the layers in turn; "
+                                "the HBM roofline is far from binding")
+    traffic_table, traffic_commit = measured_traffic()
     default_input = args.batch is None and args.seed == 2015 and args.precision == "fp32" and args.fused == 1
     fused_layers = {e["layer"] for e in kernels if e["kernel"] == "conv_nin"}
     for e in kernels:
-        e["traffic"] = MEASURED_TRAFFIC.get((cfg.name, e["kernel"], e["layer"])) if default_input else None
-    # the dominant kernel: the single-kernel span that takes the most time (a "rules" or "grid_build" span covers
-    # several small kernels and a host round trip, so it has no one roofline)
-    dominant = next((e for e in kernels if "achieved" in e and e["kernel"] in ("gather", "nin", "conv_nin", "maxpool", "terminal")), None)
-    roofline = None
-    if dominant:
-        roofline = dict(kernel="%s[layer %d]" % (dominant["kernel"], dominant["layer"]), bound=dominant["bound"],
-                        achieved=dominant["achieved"], peak=dominant["peak"], unit=dominant["unit"], frac=dominant["frac"],
-                        traffic=dominant["traffic"])
-        if "shape" in dominant:
-            roofline["shape_MKN"] = dominant["shape"]
+        e["traffic"] = traffic_table.get((cfg.name, e["kernel"], e["layer"])) if default_input else None
+    if rules_entry and default_input:
+        rules_entry["traffic"] = traffic_table.get((cfg.name, "rules", "all"))
+
+    def as_roofline(e):
+        r = dict(kernel="%s[layer %s]" % (e["kernel"], e["layer"]), bound=e["bound"], achieved=e["achieved"],
+                 peak=e["peak"], unit=e["unit"], frac=e["frac"], traffic=e["traffic"],
+                 us_per_step=round(1e3 * e.get("ms_kernel", e["ms_per_step"]), 2))
+        if "shape" in e:
+            r["shape_MKN"] = e["shape"]
+        if "note" in e:
+            r["note"] = e["note"]
+        return r
+
+    # the dominant entry: whatever takes the most GPU time per step, a single kernel or the rule books as a whole
+    single = [e for e in kernels if "achieved" in e and e["kernel"] in ("gather", "nin", "conv_nin", "maxpool", "terminal")]
+    candidates = single + ([rules_entry] if rules_entry else [])
+    dominant = max(candidates, key=lambda e: e.get("ms_kernel", e["ms_per_step"])) if candidates else None
+    roofline = as_roofline(dominant) if dominant else None
+    nin_only = [e for e in single if e["kernel"] in ("nin", "conv_nin") and e.get("bound") == "mfma"]
+    roofline_nin = as_roofline(max(nin_only, key=lambda e: e["ms_kernel"])) if nin_only else None
+    nin_flops = sum(work[(e["kernel"], e["layer"])][1] for e in nin_only)
+    nin_ms = sum(e["ms_kernel"] for e in nin_only)
+    if roofline_nin and nin_ms > 0:
+        roofline_nin["all_mfma_bound_layers"] = dict(
+            layers=sorted(e["layer"] for e in nin_only), tflops=round(nin_flops / (nin_ms * 1e-3) / 1e12, 2),
+            frac=round(nin_flops / (nin_ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS[args.precision], 4))
 
     from_host = None
     if args.from_host:
@@ -312,6 +350,10 @@ def main():
         "value": active * args.steps / dt,
         "unit": "active sites/s",
         "samples_per_s": B * args.steps / dt,
+        "with_input_upload": {"active_sites_per_s": active * args.steps / dt_up, "samples_per_s": B * args.steps / dt_up,
+                              "ms_per_step": 1e3 * dt_up / args.steps, "bytes_uploaded_per_step": upload_bytes,
+                              "note": "sites and features in pinned host memory, uploaded on the producer streams for "
+                                      "every batch: forward time = rule build + H2D of inputs + kernels + D2H"},
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
@@ -334,6 +376,9 @@ def main():
         "mega_multiply_adds_per_sample": mac / B / 1e6,
         "giga_multiply_adds_per_s": mac / (ms_per_step * 1e-3) / 1e9,
         "roofline": roofline,
+        "roofline_nin": roofline_nin,
+        "rules": rules_entry,
+        "traffic_measured_at_commit": traffic_commit,
         "kernel_family_ms_per_step": {k: round(v, 5) for k, v in fam_ms.items()},
         "kernels": kernels,
         "cpu_baseline": cpu_baseline,
@@ -383,7 +428,9 @@ def cpu_leg(cfg, layers, weights, samples, spatialSize, budget_s):
     import oracle as orc
     import oracle_net
     from sparseconvnet_archived_amd import synthetic
-    cores = min(os.cpu_count() or 1, 16)
+    # threads used: the host's cores, at most 16 (a one-GPU box's share of its machine)
+    nproc = os.cpu_count() or 1
+    cores = min(nproc, 16)
     ora = oracle_net.Net(cfg.dimension, cfg.nInputFeatures, max(cfg.nClasses, 1))
     cfg.build(ora)
     for i, (W, Bv, pr) in weights.items():
@@ -433,7 +480,15 @@ def cpu_leg(cfg, layers, weights, samples, spatialSize, budget_s):
     for th in threads:
         th.join()
     rules_T = time.perf_counter() - t0
-    return {"value": len(K) / full, "unit": "active sites/s", "cores": cores, "kind": "port",
+    flags = ""
+    try:
+        for line in open(os.path.join(ROOT, "oracle", "Makefile")):
+            if line.startswith("CFLAGS"):
+                flags = line.split("=", 1)[1].strip()
+    except OSError:
+        pass
+    return {"value": len(K) / full, "unit": "active sites/s", "cores": cores, "host_nproc": nproc, "kind": "port",
+            "oracle_cflags": flags,
             "sample": "%s, %d of %d samples, %d passes, median" % (cfg.name, len(sub), len(samples), len(times)),
             "ms_per_batch": 1e3 * full, "samples_per_s": len(sub) / full,
             "rulebooks_only_1_thread_ms": 1e3 * rules_only,

@@ -73,6 +73,7 @@ int scn_sync(scn_ctx *ctx);
  * blocking copies / fill. */
 int scn_malloc(scn_ctx *ctx, size_t bytes, void **d_ptr);
 int scn_free(scn_ctx *ctx, void *d_ptr);
+/* (a null ctx names no stream: the copy waits for every stream of the device) */
 int scn_h2d(scn_ctx *ctx, void *d_dst, const void *h_src, size_t bytes);
 int scn_d2h(scn_ctx *ctx, void *h_dst, const void *d_src, size_t bytes);
 /* The asynchronous half of the same interface (vectorCUDA<T>::copyToCPUAsync,
@@ -84,6 +85,11 @@ typedef struct scn_event scn_event;
 int scn_host_alloc(scn_ctx *ctx, size_t bytes, void **h_ptr);
 int scn_host_free(scn_ctx *ctx, void *h_ptr);
 int scn_d2h_async(scn_ctx *ctx, void *h_pinned_dst, const void *d_src, size_t bytes);
+/* the upload of the same interface (vectorCUDA<T>::copyToGPUAsync,
+ * vectorCUDA.cu:58-87, as BatchProducer::nextBatch uses it for the input
+ * features, BatchProducer.cu:127-134): queued on the context's stream; the
+ * source must stay untouched until the stream has passed the copy */
+int scn_h2d_async(scn_ctx *ctx, void *d_dst, const void *h_pinned_src, size_t bytes);
 int scn_event_create(scn_ctx *ctx, scn_event **event);
 int scn_event_destroy(scn_event *event);
 /* marks the point the stream has reached */

@@ -80,6 +80,7 @@ def lib():
         "scn_d2h": (C.c_int, [vp, vp, vp, sz]),
         "scn_host_alloc": (C.c_int, [vp, sz, C.POINTER(vp)]),
         "scn_host_free": (C.c_int, [vp, vp]),
+        "scn_h2d_async": (C.c_int, [vp, vp, vp, C.c_size_t]),
         "scn_d2h_async": (C.c_int, [vp, vp, vp, sz]),
         "scn_event_create": (C.c_int, [vp, C.POINTER(vp)]),
         "scn_event_destroy": (C.c_int, [vp]),
@@ -153,6 +154,28 @@ def _check(rc):
         raise ScnError("scn error %d: %s" % (rc, lib().scn_last_error().decode()))
 
 
+class PinnedBuf:
+    def __init__(self, ctx, nbytes):
+        self.ctx, self.nbytes = ctx, int(nbytes)
+        p = C.c_void_p()
+        _check(lib().scn_host_alloc(ctx.h, max(self.nbytes, 16), C.byref(p)))
+        self.ptr = p.value
+
+    def buffer(self):
+        return (C.c_char * self.nbytes).from_address(self.ptr)
+
+    def free(self):
+        if self.ptr:
+            lib().scn_host_free(self.ctx.h, C.c_void_p(self.ptr))
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
 class DevArray:
     """A typed device buffer allocated through the C ABI."""
 
@@ -222,6 +245,10 @@ class Context:
 
     def empty(self, shape, dtype):
         return DevArray(self, shape, dtype)
+
+    def host_alloc(self, nbytes):
+        """Pinned host memory (scn_host_alloc), freed with the object."""
+        return PinnedBuf(self, nbytes)
 
     # ---- profiling
     def prof_enable(self, on=True):

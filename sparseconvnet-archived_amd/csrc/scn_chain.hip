@@ -29,7 +29,9 @@
 #include <mutex>
 
 #define CHAIN_MAX_LEVELS 24
-#define CHAIN_THREADS 256
+#ifndef CHAIN_THREADS
+#define CHAIN_THREADS 512
+#endif
 #define CHAIN_WAVES (CHAIN_THREADS / 64)
 #define CHAIN_LDS_MAX (152 * 1024)
 #define CHAIN_HEADER_BYTES 512
@@ -46,7 +48,8 @@ struct ChainLevel {
   int mode, nIn, nOut, size, stride, minActive, width, cube;
   int capRows; // rows of one sample the staging area holds
   int slot;    // pinned slot of the deferred counts
-  int pad;
+  // floor(2^32 / d) + 1 for d = width / size, width and size: x / d without a division
+  unsigned magicRuns, magicWidth, magicSize, magicStride;
   long long fullSize; // sites of a full output grid
   // staging, in ints: rule rows of sample b at stRules + b capRows width,
   // site keys at stKeys + b capRows
@@ -95,6 +98,26 @@ struct ChainState {
 };
 
 // ------------------------------------------------------------------ device
+#ifdef CHAIN_TIMING
+__device__ long long g_chainT[512];
+#define CT(i)                                                                  \
+  if (blockIdx.x == 0 && threadIdx.x == 0)                                     \
+  g_chainT[i] = wall_clock64()
+extern "C" int scn_debug_chain_times(long long *out, int n) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_chainT), n * sizeof(long long));
+}
+#else
+#define CT(i)
+#endif
+
+// A barrier that orders LDS traffic only.  __syncthreads() also waits for the
+// global stores in flight (the staged rule rows), a microsecond or two each
+// time; nothing a workgroup stores to global memory is read back by it.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
 
 __device__ __forceinline__ unsigned wave_scan_incl(unsigned v, int lane) {
 #pragma unroll
@@ -106,38 +129,56 @@ __device__ __forceinline__ unsigned wave_scan_incl(unsigned v, int lane) {
   return v;
 }
 
-// Exclusive prefix sum over n values held in LDS, by the whole workgroup:
-// put(i, sum of get(0..i)); returns the total to every lane.  Every lane takes
-// a run of consecutive values.  ws: CHAIN_WAVES words.
-template <typename Get, typename Put>
-__device__ __forceinline__ unsigned chain_scan(int n, Get get, Put put,
-                                               unsigned *ws) {
+// Exclusive prefix sums over two sequences held in LDS at once, by the whole
+// workgroup: putX(i, sum of getX(0..i)); the totals come back to every lane.
+// Every lane takes a run of consecutive values.  ws: 2 * CHAIN_WAVES words.
+template <typename GetA, typename PutA, typename GetB, typename PutB>
+__device__ __forceinline__ void chain_scan2(int nA, GetA getA, PutA putA,
+                                            unsigned &totalA, int nB, GetB getB,
+                                            PutB putB, unsigned &totalB,
+                                            unsigned *ws) {
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-  const int per = (n + CHAIN_THREADS - 1) / CHAIN_THREADS;
-  const int i0 = t * per < n ? t * per : n;
-  const int i1 = i0 + per < n ? i0 + per : n;
-  unsigned s = 0;
-  for (int i = i0; i < i1; ++i)
-    s += get(i);
-  const unsigned incl = wave_scan_incl(s, lane);
-  if (lane == 63)
-    ws[wave] = incl;
-  __syncthreads();
-  unsigned before = 0, total = 0;
+  const int perA = (nA + CHAIN_THREADS - 1) / CHAIN_THREADS;
+  const int a0 = t * perA < nA ? t * perA : nA;
+  const int a1 = a0 + perA < nA ? a0 + perA : nA;
+  const int perB = (nB + CHAIN_THREADS - 1) / CHAIN_THREADS;
+  const int b0 = t * perB < nB ? t * perB : nB;
+  const int b1 = b0 + perB < nB ? b0 + perB : nB;
+  unsigned sA = 0, sB = 0;
+  for (int i = a0; i < a1; ++i)
+    sA += getA(i);
+  for (int i = b0; i < b1; ++i)
+    sB += getB(i);
+  const unsigned inclA = wave_scan_incl(sA, lane);
+  const unsigned inclB = wave_scan_incl(sB, lane);
+  if (lane == 63) {
+    ws[wave] = inclA;
+    ws[CHAIN_WAVES + wave] = inclB;
+  }
+  lds_barrier();
+  unsigned beforeA = 0, beforeB = 0;
+  totalA = totalB = 0;
 #pragma unroll
   for (int w = 0; w < CHAIN_WAVES; ++w) {
-    const unsigned x = ws[w];
-    before += w < wave ? x : 0u;
-    total += x;
+    const unsigned x = ws[w], y = ws[CHAIN_WAVES + w];
+    beforeA += w < wave ? x : 0u;
+    beforeB += w < wave ? y : 0u;
+    totalA += x;
+    totalB += y;
   }
-  unsigned run = before + incl - s;
-  for (int i = i0; i < i1; ++i) {
-    const unsigned v = get(i);
-    put(i, run);
+  unsigned run = beforeA + inclA - sA;
+  for (int i = a0; i < a1; ++i) {
+    const unsigned v = getA(i);
+    putA(i, run);
     run += v;
   }
-  __syncthreads();
-  return total;
+  run = beforeB + inclB - sB;
+  for (int i = b0; i < b1; ++i) {
+    const unsigned v = getB(i);
+    putB(i, run);
+    run += v;
+  }
+  lds_barrier();
 }
 
 __device__ __forceinline__ unsigned lds_rank(const unsigned long long *bits,
@@ -146,6 +187,164 @@ __device__ __forceinline__ unsigned lds_rank(const unsigned long long *bits,
   const unsigned w = p >> 6, sh = p & 63;
   const unsigned long long below = sh ? (bits[w] & ((1ull << sh) - 1ull)) : 0ull;
   return pref[w] + (unsigned)__popcll(below);
+}
+
+// Entries carry their site as packed coordinates, so that no lane divides:
+// 30 bits in one dimension, 15 bits an axis in two, 10 in three.
+template <int D> struct Packed {
+  static constexpr int BITS = D == 1 ? 30 : (D == 2 ? 15 : 10);
+  static constexpr unsigned MASK = (1u << BITS) - 1u;
+};
+template <int D> __device__ __forceinline__ unsigned pack_site(const int *c) {
+  unsigned v = 0;
+#pragma unroll
+  for (int q = 0; q < D; ++q)
+    v |= (unsigned)c[q] << (q * Packed<D>::BITS);
+  return v;
+}
+template <int D> __device__ __forceinline__ void unpack_site(unsigned v, int *c) {
+#pragma unroll
+  for (int q = 0; q < D; ++q)
+    c[q] = (int)((v >> (q * Packed<D>::BITS)) & Packed<D>::MASK);
+}
+template <int D> __device__ __forceinline__ unsigned site_key(const int *c, int n) {
+  unsigned k = 0;
+#pragma unroll
+  for (int q = 0; q < D; ++q)
+    k = k * (unsigned)n + (unsigned)c[q];
+  return k;
+}
+// x / d for x d < 2^32, magic = floor(2^32 / d) + 1 (d >= 2)
+__device__ __forceinline__ unsigned div_magic(unsigned x, unsigned d, unsigned magic) {
+  return d == 1 ? x : __umulhi(x, magic);
+}
+
+
+// `len` (<= 32) mask bits of the row with leading coordinates lead[0 .. D-2],
+// columns c0 .. c0 + len - 1; sites outside the field read as inactive.  Both
+// words are always fetched (the mask has a spare word), so that a lane's reads
+// do not wait for one another.
+template <int D>
+__device__ __forceinline__ unsigned row_bits(const unsigned long long *bits,
+                                             const int *lead, int c0, int len,
+                                             int n) {
+  bool inside = true;
+  unsigned p = 0;
+#pragma unroll
+  for (int q = 0; q < D - 1; ++q) {
+    inside = inside && (unsigned)lead[q] < (unsigned)n;
+    p = p * (unsigned)n + (unsigned)lead[q];
+  }
+  const int lo = c0 > 0 ? c0 : 0;
+  const int hi = c0 + len < n ? c0 + len : n;
+  p = p * (unsigned)n + (unsigned)lo;
+  if (!inside || hi <= lo)
+    p = 0; // any valid address; the result is masked away
+  const unsigned w = p >> 6, sh = p & 63;
+  const unsigned long long a = bits[w], b = bits[w + 1];
+  unsigned long long v = a >> sh;
+  if (sh)
+    v |= b << (64 - sh);
+  const int m = hi - lo;
+  unsigned r = (unsigned)v & (m >= 32 ? 0xFFFFFFFFu : ((1u << (m > 0 ? m : 0)) - 1u));
+  r = (!inside || hi <= lo) ? 0u : r;
+  return r << (lo - c0 > 0 ? lo - c0 : 0);
+}
+
+// Square regions without a minimum (Regions.cu:528-653), window side S: which
+// of the outputs whose window holds input site i is first touched by i, i.e.
+// has no active site before i in its window (row-major).  All mask reads of a
+// site are issued together -- the S rows (2-D) or S (2S - 1) rows (3-D) of its
+// neighbourhood -- and every candidate is then decided in registers.  Bit c of
+// the result stands for candidate c of the box [lo, hi) in ascending key;
+// f(j) is called for the owned ones.
+template <int D, int S, typename F>
+__device__ __forceinline__ unsigned
+owned_nomin(const unsigned long long *bits, const int *i, const int *lo,
+            const int *hi, int nIn, int stride, unsigned magicStride, F f) {
+  static_assert(D == 2 || D == 3, "two or three dimensions");
+  constexpr int W = 2 * S - 1;
+  constexpr unsigned FULL = (1u << S) - 1u;
+  unsigned m = 0;
+  if (D == 2) {
+    unsigned nb[S];
+#pragma unroll
+    for (int r = 0; r < S; ++r) {
+      const int lead[1] = {i[0] - (S - 1) + r};
+      nb[r] = row_bits<2>(bits, lead, i[1] - (S - 1), W, nIn);
+    }
+#pragma unroll
+    for (int a0 = 0; a0 < S; ++a0) {
+      const int d0 = i[0] - a0;
+      const int j0 = (int)div_magic((unsigned)(d0 > 0 ? d0 : 0), (unsigned)stride, magicStride);
+      const bool ok0 = d0 >= 0 && j0 * stride == d0 && j0 >= lo[0] && j0 < hi[0];
+      unsigned above = 0;
+#pragma unroll
+      for (int r = S - 1 - a0; r < S - 1; ++r)
+        above |= nb[r];
+#pragma unroll
+      for (int a1 = 0; a1 < S; ++a1) {
+        const int d1 = i[1] - a1;
+        const int j1 = (int)div_magic((unsigned)(d1 > 0 ? d1 : 0), (unsigned)stride, magicStride);
+        const bool ok1 = d1 >= 0 && j1 * stride == d1 && j1 >= lo[1] && j1 < hi[1];
+        const unsigned before = (above & (FULL << (S - 1 - a1))) |
+                                (nb[S - 1] & (((1u << a1) - 1u) << (S - 1 - a1)));
+        if (ok0 && ok1 && before == 0) {
+          const int j[2] = {j0, j1};
+          m |= 1u << ((j0 - lo[0]) * (hi[1] - lo[1]) + (j1 - lo[1]));
+          f(j);
+        }
+      }
+    }
+  } else {
+    unsigned nb[S][W];
+#pragma unroll
+    for (int pl = 0; pl < S; ++pl)
+#pragma unroll
+      for (int r = 0; r < W; ++r) {
+        const int lead[2] = {i[0] - (S - 1) + pl, i[1] - (S - 1) + r};
+        nb[pl][r] = row_bits<3>(bits, lead, i[2] - (S - 1), W, nIn);
+      }
+#pragma unroll
+    for (int a0 = 0; a0 < S; ++a0) {
+      const int d0 = i[0] - a0;
+      const int j0 = (int)div_magic((unsigned)(d0 > 0 ? d0 : 0), (unsigned)stride, magicStride);
+      const bool ok0 = d0 >= 0 && j0 * stride == d0 && j0 >= lo[0] && j0 < hi[0];
+#pragma unroll
+      for (int a1 = 0; a1 < S; ++a1) {
+        const int d1 = i[1] - a1;
+        const int j1 = (int)div_magic((unsigned)(d1 > 0 ? d1 : 0), (unsigned)stride, magicStride);
+        const bool ok1 = d1 >= 0 && j1 * stride == d1 && j1 >= lo[1] && j1 < hi[1];
+        // whole planes before the site's, then whole rows of its plane
+        unsigned above = 0;
+#pragma unroll
+        for (int pl = S - 1 - a0; pl < S - 1; ++pl)
+#pragma unroll
+          for (int q1 = 0; q1 < S; ++q1)
+            above |= nb[pl][S - 1 - a1 + q1];
+#pragma unroll
+        for (int q1 = 0; q1 < a1; ++q1)
+          above |= nb[S - 1][S - 1 - a1 + q1];
+#pragma unroll
+        for (int a2 = 0; a2 < S; ++a2) {
+          const int d2 = i[2] - a2;
+          const int j2 = (int)div_magic((unsigned)(d2 > 0 ? d2 : 0), (unsigned)stride, magicStride);
+          const bool ok2 = d2 >= 0 && j2 * stride == d2 && j2 >= lo[2] && j2 < hi[2];
+          const unsigned before =
+              (above & (FULL << (S - 1 - a2))) |
+              (nb[S - 1][S - 1] & (((1u << a2) - 1u) << (S - 1 - a2)));
+          if (ok0 && ok1 && ok2 && before == 0) {
+            const int j[3] = {j0, j1, j2};
+            m |= 1u << (((j0 - lo[0]) * (hi[1] - lo[1]) + (j1 - lo[1])) *
+                            (hi[2] - lo[2]) +
+                        (j2 - lo[2]));
+            f(j);
+          }
+        }
+      }
+    }
+  }
+  return m;
 }
 
 // The sample could not be carried (LDS or staging too small): every plan of
@@ -160,8 +359,8 @@ template <int D>
 __global__ void __launch_bounds__(CHAIN_THREADS) k_chain_sample(ChainArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   const int b = blockIdx.x, t = threadIdx.x;
-  unsigned *ws = reinterpret_cast<unsigned *>(lds); // CHAIN_WAVES words
-  int *invOrd = reinterpret_cast<int *>(lds + 64);  // up to 64 offsets
+  unsigned *ws = reinterpret_cast<unsigned *>(lds); // 2 * CHAIN_WAVES words
+  int *invOrd = reinterpret_cast<int *>(lds + 128); // up to 64 offsets
   auto M = [&](int x) {
     return reinterpret_cast<unsigned long long *>(lds + a.maskOff[x]);
   };
@@ -171,6 +370,7 @@ __global__ void __launch_bounds__(CHAIN_THREADS) k_chain_sample(ChainArgs a) {
   unsigned *arena = reinterpret_cast<unsigned *>(lds + a.arenaOff);
   const int arenaWords = a.arenaBytes / 4;
 
+  CT(0);
   // ---- the source grid of this sample: its slice of the batch's mask
   long long vol = a.vol0;
   int words = (int)((vol + 63) >> 6);
@@ -192,43 +392,60 @@ __global__ void __launch_bounds__(CHAIN_THREADS) k_chain_sample(ChainArgs a) {
       }
       bitsA[w] = v;
     }
-    // the mask of the first output grid starts empty
+    // the masks of the first two output grids start empty
     for (int w = t; w < a.maskWords[1]; w += CHAIN_THREADS)
       M(1)[w] = 0ull;
+    for (int w = t; w < a.maskWords[2]; w += CHAIN_THREADS)
+      M(2)[w] = 0ull;
   }
-  __syncthreads();
+  lds_barrier();
+  CT(1);
   unsigned nA;
   {
     const unsigned long long *bitsA = M(0);
     unsigned short *prefA = P(0);
-    nA = chain_scan(
+    unsigned none;
+    chain_scan2(
         words, [&](int i) { return (unsigned)__popcll(bitsA[i]); },
-        [&](int i, unsigned v) { prefA[i] = (unsigned short)v; }, ws);
+        [&](int i, unsigned v) { prefA[i] = (unsigned short)v; }, nA, 0,
+        [&](int) { return 0u; }, [&](int, unsigned) {}, none, ws);
   }
+  CT(2);
   if ((long long)nA * CHAIN_IN_BYTES > a.arenaBytes) {
     chain_give_up(a);
     return;
   }
-  // entries by rank at the bottom of the arena: key[nA], row[nA]
+  // entries by rank at the bottom of the arena: site[nA], row[nA]
   unsigned *keyA = arena, *rowA = arena + nA;
   {
     const unsigned long long *bitsA = M(0);
     const unsigned short *prefA = P(0);
-    const long long p0 = (long long)b * vol;
     for (int w = t; w < words; w += CHAIN_THREADS) {
       unsigned long long v = bitsA[w];
       unsigned r = prefA[w];
       while (v) {
-        const unsigned key = 64u * w + (unsigned)(__ffsll((long long)v) - 1);
+        keyA[r++] = 64u * w + (unsigned)(__ffsll((long long)v) - 1);
         v &= v - 1;
-        keyA[r] = key;
-        rowA[r] = (unsigned)hash_find(a.table, a.shift, a.mask, p0 + key);
-        ++r;
       }
+    }
+    lds_barrier();
+    // (one lane per entry: the table look-ups of a sample are all in flight together)
+    const long long p0 = (long long)b * vol;
+    for (unsigned r = t; r < nA; r += CHAIN_THREADS) {
+      unsigned key = keyA[r];
+      rowA[r] = (unsigned)hash_find(a.table, a.shift, a.mask, p0 + key);
+      int c[D];
+#pragma unroll
+      for (int q = D - 1; q >= 0; --q) {
+        c[q] = (int)(key % (unsigned)a.n0);
+        key /= (unsigned)a.n0;
+      }
+      keyA[r] = pack_site<D>(c);
     }
   }
   int bgA = a.bg[b];
-  __syncthreads();
+  lds_barrier();
+  CT(3);
 
   for (int l = 0; l < a.nLevels; ++l) {
     const ChainLevel &L = a.lv[l];
@@ -293,19 +510,32 @@ __global__ void __launch_bounds__(CHAIN_THREADS) k_chain_sample(ChainArgs a) {
     vin.bits = const_cast<unsigned long long *>(bitsA);
 
     // -- which candidates each input owns; the output mask
+    const bool fast = D >= 2 && L.mode == MODE_SQ_NOMIN && (L.size == 2 || L.size == 3);
     for (unsigned r = t; r < nA; r += CHAIN_THREADS) {
       int i[D], lo[D], hi[D], j[D];
-      decode_key<D>((long long)keyA[r], L.nIn, i);
+      unpack_site<D>(keyA[r], i);
       unsigned m = 0;
-      if (cand_box<D>(g, b, i, lo, hi)) {
+      auto mark = [&](const int *jj) {
+        const unsigned ok = site_key<D>(jj, L.nOut);
+        atomicOr(&bitsB[ok >> 6], 1ull << (ok & 63));
+      };
+      if (!cand_box<D>(g, b, i, lo, hi)) {
+        m = 0;
+      } else if (fast) {
+        if constexpr (D >= 2) {
+          if (L.size == 2)
+            m = owned_nomin<D, 2>(bitsA, i, lo, hi, L.nIn, L.stride, L.magicStride, mark);
+          else
+            m = owned_nomin<D, 3>(bitsA, i, lo, hi, L.nIn, L.stride, L.magicStride, mark);
+        }
+      } else {
 #pragma unroll
         for (int q = 0; q < D; ++q)
           j[q] = lo[q];
         for (int c = 0;; ++c) {
           if (owns<D>(vin, g, b, 0ll, i, j)) {
             m |= 1u << c;
-            const unsigned ok = (unsigned)encode_key<D>(j, L.nOut);
-            atomicOr(&bitsB[ok >> 6], 1ull << (ok & 63));
+            mark(j);
           }
           int q = D - 1;
           for (; q >= 0; --q) {
@@ -319,13 +549,6 @@ __global__ void __launch_bounds__(CHAIN_THREADS) k_chain_sample(ChainArgs a) {
       }
       maskS[r] = m;
     }
-    { // the mask of the grid after the next starts empty (its buffer held
-      // the grid before this layer's input, which nothing reads any more)
-      unsigned long long *z = M((l + 2) % 3);
-      const int nz = a.maskWords[(l + 2) % 3];
-      for (int w = t; w < nz; w += CHAIN_THREADS)
-        z[w] = 0ull;
-    }
     if (tri && t == 0) { // inverse of RegularTriangularRegions::ord (Regions.cu:810-826)
       int S = 0;
       for (int q = 0; q < L.cube; ++q) {
@@ -338,16 +561,18 @@ __global__ void __launch_bounds__(CHAIN_THREADS) k_chain_sample(ChainArgs a) {
           invOrd[S++] = q;
       }
     }
-    __syncthreads();
+    lds_barrier();
+    CT(4 + 4 * l);
 
     // -- rows of the outputs: prefix sum of the owned counts, and the rank
     //    prefix of the output mask
-    const unsigned nB = chain_scan(
+    unsigned nB, nBits;
+    chain_scan2(
         (int)nA, [&](int i) { return (unsigned)__popc(maskS[i]); },
-        [&](int i, unsigned v) { baseS[i] = (unsigned short)v; }, ws);
-    (void)chain_scan(
-        wordsB, [&](int i) { return (unsigned)__popcll(bitsB[i]); },
-        [&](int i, unsigned v) { prefB[i] = (unsigned short)v; }, ws);
+        [&](int i, unsigned v) { baseS[i] = (unsigned short)v; }, nB, wordsB,
+        [&](int i) { return (unsigned)__popcll(bitsB[i]); },
+        [&](int i, unsigned v) { prefB[i] = (unsigned short)v; }, nBits, ws);
+    CT(5 + 4 * l);
     const int hasBg = (long long)nB < L.fullSize;
     if ((long long)nA * CHAIN_IN_BYTES + (long long)nB * CHAIN_OUT_BYTES >
             a.arenaBytes ||
@@ -375,47 +600,57 @@ __global__ void __launch_bounds__(CHAIN_THREADS) k_chain_sample(ChainArgs a) {
         continue;
       unsigned row = baseS[r];
       int i[D], lo[D], hi[D], j[D];
-      decode_key<D>((long long)keyA[r], L.nIn, i);
+      unpack_site<D>(keyA[r], i);
       (void)cand_box<D>(g, b, i, lo, hi);
       while (m) { // ascending candidate = ascending output key
         int rem = __ffs((int)m) - 1;
         m &= m - 1;
 #pragma unroll
         for (int q = D - 1; q >= 0; --q) {
-          const int ext = hi[q] - lo[q];
-          j[q] = lo[q] + rem % ext;
-          rem /= ext;
+          const unsigned ext = (unsigned)(hi[q] - lo[q]);
+          const unsigned up = (unsigned)rem / ext;
+          j[q] = lo[q] + (int)((unsigned)rem - up * ext);
+          rem = (int)up;
         }
-        const unsigned ok = (unsigned)encode_key<D>(j, L.nOut);
+        const unsigned ok = site_key<D>(j, L.nOut);
         const unsigned rk = lds_rank(bitsB, prefB, ok);
-        keyB[rk] = ok;
+        keyB[rk] = pack_site<D>(j);
         rowB[rk] = row;
         stKey[row] = (int)ok;
         ++row;
       }
     }
-    __syncthreads();
+    { // the mask of the grid after the next starts empty (its buffer held
+      // the grid before this layer's input, which nothing reads any more)
+      unsigned long long *z = M((l + 2) % 3);
+      const int nz = l == 0 ? 0 : a.maskWords[(l + 2) % 3];
+      for (int w = t; w < nz; w += CHAIN_THREADS)
+        z[w] = 0ull;
+    }
+    lds_barrier();
+    CT(6 + 4 * l);
 
     // -- rule rows (sample-local row numbers) to the staging area
     if (L.rules) {
       if (!tri && L.size >= 2) {
         // one lane per run of `size` entries along the innermost axis: their
         // input sites are neighbours in the mask and in rank
-        const int runsPerRow = L.width / L.size;
-        const unsigned items = nB * (unsigned)runsPerRow;
+        const unsigned runsPerRow = (unsigned)(L.width / L.size);
+        const unsigned items = nB * runsPerRow;
         for (unsigned it = t; it < items; it += CHAIN_THREADS) {
-          const unsigned rk = it / runsPerRow;
+          const unsigned rk = div_magic(it, runsPerRow, L.magicRuns);
           const int run0 = (int)(it - rk * runsPerRow);
-          int run = run0;
           int j[D], c[D];
-          decode_key<D>((long long)keyB[rk], L.nOut, j);
+          unpack_site<D>(keyB[rk], j);
           c[D - 1] = j[D - 1] * L.stride;
-#pragma unroll
-          for (int q = D - 2; q >= 0; --q) {
-            c[q] = j[q] * L.stride + run % L.size;
-            run /= L.size;
+          if (D == 2) {
+            c[0] = j[0] * L.stride + run0;
+          } else if (D == 3) {
+            const int hiRun = (int)div_magic((unsigned)run0, (unsigned)L.size, L.magicSize);
+            c[1] = j[1] * L.stride + (run0 - hiRun * L.size);
+            c[0] = j[0] * L.stride + hiRun;
           }
-          const unsigned p0 = (unsigned)encode_key<D>(c, L.nIn);
+          const unsigned p0 = site_key<D>(c, L.nIn);
           const unsigned present = get_bits(bitsA, (long long)p0, L.size);
           const unsigned rank0 = lds_rank(bitsA, prefA, p0);
           int *dst = st + (long long)rowB[rk] * L.width + run0 * L.size;
@@ -427,17 +662,18 @@ __global__ void __launch_bounds__(CHAIN_THREADS) k_chain_sample(ChainArgs a) {
       } else {
         const unsigned items = nB * (unsigned)L.width;
         for (unsigned it = t; it < items; it += CHAIN_THREADS) {
-          const unsigned rk = it / L.width;
+          const unsigned rk = div_magic(it, (unsigned)L.width, L.magicWidth);
           const int q = (int)(it - rk * L.width);
           int off = tri ? invOrd[q] : q;
           int j[D], c[D];
-          decode_key<D>((long long)keyB[rk], L.nOut, j);
+          unpack_site<D>(keyB[rk], j);
 #pragma unroll
           for (int x = D - 1; x >= 0; --x) {
-            c[x] = j[x] * L.stride + off % L.size;
-            off /= L.size;
+            const int hiOff = (int)div_magic((unsigned)off, (unsigned)L.size, L.magicSize);
+            c[x] = j[x] * L.stride + (off - hiOff * L.size);
+            off = hiOff;
           }
-          const unsigned p = (unsigned)encode_key<D>(c, L.nIn);
+          const unsigned p = site_key<D>(c, L.nIn);
           const bool present = (bitsA[p >> 6] >> (p & 63)) & 1ull;
           st[(long long)rowB[rk] * L.width + q] =
               present ? (int)rowA[lds_rank(bitsA, prefA, p)] : bgA;
@@ -447,7 +683,8 @@ __global__ void __launch_bounds__(CHAIN_THREADS) k_chain_sample(ChainArgs a) {
         for (int q = t; q < L.width; q += CHAIN_THREADS)
           st[(long long)nB * L.width + q] = bgA;
     }
-    __syncthreads();
+    lds_barrier();
+    CT(7 + 4 * l);
     // the output grid is the next layer's input
     keyA = keyB;
     rowA = rowB;
@@ -671,6 +908,9 @@ static bool chain_accepts(scn_ctx *ctx, const scn_grids *in, const scn_grids *ou
     return false;
   if (in->batch < 1 || in->d < 1 || in->d > 3 || in->vol >= (1ll << 31))
     return false;
+  // sites travel as packed coordinates: 30, 15 or 10 bits an axis
+  if (in->n >= (in->d == 1 ? (1 << 30) : (in->d == 2 ? (1 << 15) : (1 << 10))))
+    return false;
   if (cs->recs.empty()) {
     // the source: grids with a table and a mask, counts known
     if (in->pending || !in->indexValid)
@@ -741,6 +981,10 @@ int scn_chain_record_regions(scn_ctx *ctx, scn_grids *in, scn_grids *out,
   L.width = g.width;
   L.cube = g.cube;
   L.fullSize = fullSize;
+  L.magicRuns = (unsigned)((1ull << 32) / (unsigned)(g.width / g.size > 0 ? g.width / g.size : 1) + 1);
+  L.magicWidth = (unsigned)((1ull << 32) / (unsigned)g.width + 1);
+  L.magicSize = (unsigned)((1ull << 32) / (unsigned)g.size + 1);
+  L.magicStride = (unsigned)((1ull << 32) / (unsigned)g.stride + 1);
   L.slot = (int)ctx->pendingGrids.size();
   L.ekey = out->ekey.p;
   L.erow = out->erow.p;

@@ -102,6 +102,10 @@ extern "C" int scn_h2d(scn_ctx *c, void *d_dst, const void *h_src,
                        size_t bytes) {
   if (bytes == 0)
     return SCN_OK;
+  if (!c) { // no stream named: ordered after the work of every stream
+    SCN_HIP_CHECK(hipMemcpy(d_dst, h_src, bytes, hipMemcpyHostToDevice));
+    return SCN_OK;
+  }
   SCN_HIP_CHECK(
       hipMemcpyAsync(d_dst, h_src, bytes, hipMemcpyHostToDevice, c->stream));
   SCN_HIP_CHECK(hipStreamSynchronize(c->stream));
@@ -112,6 +116,10 @@ extern "C" int scn_d2h(scn_ctx *c, void *h_dst, const void *d_src,
                        size_t bytes) {
   if (bytes == 0)
     return SCN_OK;
+  if (!c) {
+    SCN_HIP_CHECK(hipMemcpy(h_dst, d_src, bytes, hipMemcpyDeviceToHost));
+    return SCN_OK;
+  }
   SCN_HIP_CHECK(
       hipMemcpyAsync(h_dst, d_src, bytes, hipMemcpyDeviceToHost, c->stream));
   SCN_HIP_CHECK(hipStreamSynchronize(c->stream));
@@ -134,6 +142,16 @@ extern "C" int scn_host_free(scn_ctx *c, void *h_ptr) {
   (void)c;
   if (h_ptr)
     SCN_HIP_CHECK(hipHostFree(h_ptr));
+  return SCN_OK;
+}
+extern "C" int scn_h2d_async(scn_ctx *c, void *d_dst, const void *h_src,
+                             size_t bytes) {
+  SCN_REQUIRE(c, SCN_ERR_ARG, "scn_h2d_async: null context");
+  if (bytes == 0)
+    return SCN_OK;
+  SCN_REQUIRE(d_dst && h_src, SCN_ERR_ARG, "scn_h2d_async: null buffer");
+  SCN_HIP_CHECK(
+      hipMemcpyAsync(d_dst, h_src, bytes, hipMemcpyHostToDevice, c->stream));
   return SCN_OK;
 }
 extern "C" int scn_d2h_async(scn_ctx *c, void *h_dst, const void *d_src,

@@ -29,6 +29,8 @@ struct ResidentBatch {
   int64_t nActive;
   int nSpatialSites;
   const float *d_features;
+  // the pointers name pinned host memory instead: every batch uploads them
+  bool onHost = false;
 };
 
 class SparseConvNetCUDA {

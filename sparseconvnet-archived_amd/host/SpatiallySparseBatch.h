@@ -14,6 +14,11 @@ struct BatchResultStage {
   size_t capacity; // floats
   scn_event *arrived;
   bool pending;
+  // a training batch: the point of the net's stream behind the backward pass,
+  // the last reader of the slot's rule books and features.  The slot goes
+  // back to its producer only after this point has been passed.
+  scn_event *consumed;
+  bool consumedPending;
   // the labels as the statistics need them, on the host, while batch.labels
   // is in device memory for the gradient of a training batch
   std::vector<int> labels;

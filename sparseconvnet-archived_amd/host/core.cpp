@@ -167,15 +167,18 @@ template <typename t> vectorCUDA<t>::~vectorCUDA() {
   if (d_vec)
     scn_free(nullptr, d_vec);
 }
+// No stream named (vectorCUDA.cu:26-57, blocking cudaMemcpy): a copy with a
+// null context waits for the work of every stream of the device first, so the
+// data is complete whichever net's stream produced it.
 template <typename t> void vectorCUDA<t>::copyToCPU() {
   if (!onGPU)
     return;
-  toCPU(scnDefaultContext());
+  toCPU(nullptr);
 }
 template <typename t> void vectorCUDA<t>::copyToGPU() {
   if (onGPU)
     return;
-  toGPU(scnDefaultContext());
+  toGPU(nullptr);
 }
 template <typename t> void vectorCUDA<t>::toCPU(scn_ctx *ctx) {
   onGPU = false;
@@ -220,14 +223,21 @@ template <typename t> size_t vectorCUDA<t>::size64() {
 template <typename t> void vectorCUDA<t>::setZero() {
   if (onGPU) {
     static_assert(sizeof(t) == 4, "32-bit elements");
+    // no stream named: done before the call returns, whatever stream uses
+    // the memory next
     SCN_CHECKED(scn_fill32(scnDefaultContext(), d_vec, 0u, dsize));
+    SCN_CHECKED(scn_sync(scnDefaultContext()));
   } else {
     std::fill(vec.begin(), vec.end(), (t)0);
   }
 }
 template <typename t> void vectorCUDA<t>::setZero(cudaMemStream &memStream) {
-  (void)memStream;
-  setZero();
+  if (onGPU) {
+    static_assert(sizeof(t) == 4, "32-bit elements");
+    SCN_CHECKED(scn_fill32(memStream.ctx, d_vec, 0u, dsize));
+  } else {
+    std::fill(vec.begin(), vec.end(), (t)0);
+  }
 }
 template <typename t> void vectorCUDA<t>::setConstant(float a) {
   bool wasOnGPU = onGPU;
@@ -335,10 +345,13 @@ void SpatiallySparseBatchInterface::summary() {
 }
 
 BatchResultStage::BatchResultStage()
-    : pinned(nullptr), capacity(0), arrived(nullptr), pending(false) {}
+    : pinned(nullptr), capacity(0), arrived(nullptr), pending(false),
+      consumed(nullptr), consumedPending(false) {}
 BatchResultStage::~BatchResultStage() {
   if (arrived)
     scn_event_destroy(arrived);
+  if (consumed)
+    scn_event_destroy(consumed);
   if (pinned)
     scn_host_free(scnDefaultContext(), pinned);
 }

@@ -300,15 +300,44 @@ void SparseConvNetCUDA::preprocessResident(int cc, const ResidentBatch &input) {
   }
   scn_prof_tag(ctx, -1);
   clearDeviceGrids(ctx, b);
+  const int32_t *d_sample = input.d_sample, *d_row = input.d_row,
+                *d_background = input.d_background;
+  const int64_t *d_key = input.d_key;
+  const size_t n = (size_t)input.nActive;
+  if (input.onHost) {
+    // sites in pinned host memory: uploaded on this slot's stream first
+    // (BatchProducer.cu:127-134 uploads a batch's inputs the same way)
+    b.stagingSample.copyToGPU();
+    b.stagingKey.copyToGPU();
+    b.stagingRow.copyToGPU();
+    b.stagingBackground.copyToGPU();
+    b.stagingSample.resize64(n);
+    b.stagingKey.resize64(2 * n);
+    b.stagingRow.resize64(n);
+    b.stagingBackground.resize64((size_t)input.batchSize);
+    SCN_CHECKED(scn_h2d_async(ctx, b.stagingSample.dPtr(), input.d_sample, n * 4));
+    SCN_CHECKED(scn_h2d_async(ctx, b.stagingKey.dPtr(), input.d_key, n * 8));
+    SCN_CHECKED(scn_h2d_async(ctx, b.stagingRow.dPtr(), input.d_row, n * 4));
+    SCN_CHECKED(scn_h2d_async(ctx, b.stagingBackground.dPtr(), input.d_background,
+                              (size_t)input.batchSize * 4));
+    d_sample = b.stagingSample.dPtr();
+    d_key = (const int64_t *)b.stagingKey.dPtr();
+    d_row = b.stagingRow.dPtr();
+    d_background = b.stagingBackground.dPtr();
+  }
   SCN_CHECKED(scn_grids_build(ctx, in.deviceGrids, input.batchSize, dimension,
-                              in.spatialSize, input.d_sample, input.d_key,
-                              input.d_row, input.nActive, input.d_background,
+                              in.spatialSize, d_sample, d_key, d_row,
+                              input.nActive, d_background,
                               input.nSpatialSites));
   in.sub->features.copyToGPU();
   size_t nElems = (size_t)input.nSpatialSites * nInputFeatures;
   in.sub->features.resize64(nElems);
-  SCN_CHECKED(scn_d2d(ctx, in.sub->features.dPtr(), input.d_features,
-                      nElems * sizeof(float)));
+  if (input.onHost)
+    SCN_CHECKED(scn_h2d_async(ctx, in.sub->features.dPtr(), input.d_features,
+                              nElems * sizeof(float)));
+  else
+    SCN_CHECKED(scn_d2d(ctx, in.sub->features.dPtr(), input.d_features,
+                        nElems * sizeof(float)));
   buildRuleBooks(*this, ctx, b);
   SCN_CHECKED(scn_sync(ctx));
 }
@@ -339,6 +368,13 @@ void SparseConvNetCUDA::backwardBatch(SpatiallySparseBatch &batch,
     layers[i]->backwards(batch, batch.interfaces[i], batch.interfaces[i + 1],
                          learningRate, momentum);
   }
+  // the backward kernels read the slot's rule books and features: the slot
+  // stays with the consumer until the stream has passed this point
+  BatchResultStage &r = *batch.result;
+  if (!r.consumed)
+    SCN_CHECKED(scn_event_create(memStream.ctx, &r.consumed));
+  SCN_CHECKED(scn_event_record(memStream.ctx, r.consumed));
+  r.consumedPending = true;
 }
 // The two halves of processBatch.  forwardBatch only queues work on the net's
 // stream (every layer, then the copy of the probabilities to the host);
@@ -367,6 +403,10 @@ void SparseConvNetCUDA::forwardBatch(SpatiallySparseBatch &batch) {
 void SparseConvNetCUDA::finishBatch(SpatiallySparseBatch &batch,
                                     std::ofstream &f, std::ofstream &g) {
   SoftmaxClassifierCollect(batch.interfaces.back(), batch, nTop);
+  if (batch.result->consumedPending) {
+    SCN_CHECKED(scn_event_wait(batch.result->consumed));
+    batch.result->consumedPending = false;
+  }
   if (f.is_open())
     for (auto &p : batch.predictions) {
       for (size_t k = 0; k < p.size(); k++)
@@ -763,6 +803,12 @@ void BatchProducer::batchProducerThread(int nThread) {
 SpatiallySparseBatch *BatchProducer::nextBatch() {
   if (batchCounter - keepAlive >= 0) { // hand a finished slot back to its worker
     int cc = (batchCounter - keepAlive) % cnn.nBatchProducerThreads;
+    const BatchResultStage &r = *cnn.batchPool[cc].result;
+    if (r.pending || r.consumedPending) {
+      std::fprintf(stderr, "BatchProducer: slot %d handed back while the net's "
+                           "stream may still read it\n", cc);
+      scnExit(EXIT_FAILURE);
+    }
     cnn.batchPool[cc].batchSize = 0;
     {
       std::lock_guard<std::mutex> lock(slotMutex);

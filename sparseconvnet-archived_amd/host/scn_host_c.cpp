@@ -1,4 +1,5 @@
 // C view of the host classes (see scn_host_c.h).
+#include <chrono>
 #include "scn_host_c.h"
 #include "Off3DFormatPicture.h"
 #include "OnlineHandwritingPicture.h"
@@ -514,6 +515,7 @@ static ResidentBatch resident_of(int batch, const int32_t *d_sample,
   r.nActive = nActive;
   r.nSpatialSites = nSpatialSites;
   r.d_features = d_features;
+  r.onHost = false;
   return r;
 }
 
@@ -579,6 +581,65 @@ int scnh_forward_resident_stream(scnh_net *net, int nBatches, int batch,
   if (queued)
     finish(queued);
   cnn->memStream.synchronize();
+  net->batch = nullptr;
+  return done;
+}
+// nWarmup + nTimed batches through one BatchProducer, as one dataset pass runs
+// them; *seconds is the wall time of the last nTimed, taken between two points
+// at which the net's stream is idle and every earlier batch is finished.  The
+// producers are not stopped in between: at the first point they hold the next
+// batches ready, as they do in the middle of any pass.
+int scnh_forward_stream_timed(scnh_net *net, int nWarmup, int nTimed, int batch,
+                              const int32_t *sample, const int64_t *key,
+                              const int32_t *row, const int32_t *background,
+                              int64_t nActive, int nSpatialSites,
+                              const float *features, int inputsOnHost,
+                              float *h_probs, double *seconds) {
+  SparseConvNetCUDA *cnn = net->cnn;
+  ResidentBatch r = resident_of(batch, sample, key, row, background, nActive,
+                                nSpatialSites, features);
+  r.onHost = inputsOnHost != 0;
+  BatchProducer bp(*cnn, r, nWarmup + nTimed);
+  bp.keepAlive = cnn->nBatchProducerThreads >= 2 ? 1 : 0;
+  int done = 0, started = 0;
+  SpatiallySparseBatch *queued = nullptr;
+  auto finish = [&](SpatiallySparseBatch *b) {
+    if (net->hasClassifier) {
+      std::ofstream f, g;
+      cnn->finishBatch(*b, f, g);
+      net->batch = b;
+      if (h_probs)
+        scnh_batch_probabilities(net, h_probs);
+    }
+    ++done;
+  };
+  auto t0 = std::chrono::steady_clock::now();
+  while (SpatiallySparseBatch *b = bp.nextBatch()) {
+    if (started == nWarmup) { // every warm-up batch done before the clock starts
+      if (queued)
+        finish(queued);
+      queued = nullptr;
+      cnn->memStream.synchronize();
+      t0 = std::chrono::steady_clock::now();
+    }
+    ++started;
+    if (net->hasClassifier)
+      cnn->forwardBatch(*b);
+    else
+      forward_layers(net, *b);
+    if (queued)
+      finish(queued);
+    queued = b;
+    if (!bp.keepAlive) {
+      finish(queued);
+      queued = nullptr;
+    }
+  }
+  if (queued)
+    finish(queued);
+  cnn->memStream.synchronize();
+  if (seconds)
+    *seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
   net->batch = nullptr;
   return done;
 }

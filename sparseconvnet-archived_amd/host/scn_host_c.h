@@ -195,6 +195,16 @@ int scnh_forward_resident_stream(scnh_net *net, int nBatches, int batch,
                                  const int32_t *d_background, int64_t nActive,
                                  int nSpatialSites, const float *d_features,
                                  float *h_probs);
+/* nWarmup untimed and nTimed timed batches in one pass (the producers keep
+ * running across the boundary); inputsOnHost: the five arrays are pinned host
+ * memory and every batch uploads them on its producer's stream, otherwise
+ * device memory.  *seconds: wall time of the timed batches. */
+int scnh_forward_stream_timed(scnh_net *net, int nWarmup, int nTimed, int batch,
+                              const int32_t *sample, const int64_t *key,
+                              const int32_t *row, const int32_t *background,
+                              int64_t nActive, int nSpatialSites,
+                              const float *features, int inputsOnHost,
+                              float *h_probs, double *seconds);
 /* the library context of the net (scn_ctx *), for timing and raw buffers */
 void *scnh_context(scnh_net *net);
 /* multiply-accumulates of the NiN layers since the last call */

@@ -95,6 +95,7 @@ def lib():
         "scnh_iface_grids": (None, [vp, i32, vp, vp, vp, vp]),
         "scnh_forward_resident": (i32, [vp, i32, vp, vp, vp, vp, i64, i32, vp, vp]),
         "scnh_forward_resident_stream": (i32, [vp, i32, i32, vp, vp, vp, vp, i64, i32, vp, vp]),
+        "scnh_forward_stream_timed": (i32, [vp, i32, i32, i32, vp, vp, vp, vp, i64, i32, vp, i32, vp, P(C.c_double)]),
         "scnh_context": (vp, [vp]),
         "scnh_take_multiply_add_count": (C.c_double, []),
     }
@@ -402,6 +403,17 @@ class Net:
                                 h_probs=None):
         return lib().scnh_forward_resident_stream(self.h, nBatches, batch, d_sample, d_key, d_row, d_bg, nActive,
                                                   nSpatialSites, d_features, _p(h_probs) if h_probs is not None else None)
+
+    def forward_stream_timed(self, nWarmup, nTimed, batch, sample, key, row, bg, nActive, nSpatialSites, features,
+                             inputs_on_host=False, h_probs=None):
+        """nWarmup + nTimed batches in one pass; returns the wall time of the timed ones in seconds.  The five
+        arrays are device pointers, or pinned host pointers with inputs_on_host (uploaded for every batch)."""
+        sec = C.c_double()
+        done = lib().scnh_forward_stream_timed(self.h, nWarmup, nTimed, batch, sample, key, row, bg, nActive,
+                                               nSpatialSites, features, int(inputs_on_host),
+                                               _p(h_probs) if h_probs is not None else None, C.byref(sec))
+        assert done == nWarmup + nTimed
+        return sec.value
 
     def context_handle(self):
         return lib().scnh_context(self.h)
