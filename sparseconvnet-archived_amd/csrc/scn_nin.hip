@@ -1525,11 +1525,12 @@ static int launch_wstream_bf16(scn_ctx *ctx, const float *A, const float *W,
   return SCN_OK;
 }
 
-// bf16 operands, shapes this kernel takes: K a multiple of 64, N of 32, enough
-// rows; with a gather, channels in multiples of 8.  The choice depends on
-// (M, K, N) only.
+// bf16 operands, shapes this kernel takes: K a multiple of 64, N of 32, any
+// number of rows (a fused convolution has no other bf16 kernel to fall back
+// on, and the short last batch of a dataset has few rows); with a gather,
+// channels in multiples of 8.  The choice depends on (K, N) only.
 static bool wstream_bf16_shape(long long M, int K, int N) {
-  return K % 64 == 0 && N % 32 == 0 && M >= 256;
+  return K % 64 == 0 && N % 32 == 0 && M >= 1;
 }
 static bool wstream_bf16_forward(scn_ctx *ctx, const float *A, const float *W,
                                  float *out, long long M, int K, int N,

@@ -186,8 +186,9 @@ def test_nin_bf16(scn, ctx, M, K, N, act):
 
 # the bf16 W-streaming kernel with wide slices (64 and 96 columns), every depth of its prefetch ring
 # (K / 32 a multiple of 4, of 6, of neither), ragged last groups
+# ... and the wide contractions of the GEMM-bound 2-D net (K up to 2560, N up to 800)
 @pytest.mark.parametrize("M,K,N", [(66001, 1728, 64), (33005, 192, 96), (40003, 256, 96), (70001, 320, 128),
-                                   (1, 64, 32), (15, 128, 32)])
+                                   (1, 64, 32), (15, 128, 32), (255, 512, 160), (1025, 3200, 320), (2600, 2560, 800)])
 def test_nin_bf16_streamed_w(scn, ctx, M, K, N):
     check_nin_bf16(scn, ctx, M, K, N, "PRELU", x3=False)
 
@@ -223,8 +224,10 @@ def check_nin_bf16(scn, ctx, M, K, N, act, x3=True):
     assert np.linalg.norm(got3 - want) / np.linalg.norm(want) <= 1e-4
 
 
+# (a few rows: the deepest convolutions of a batch of one to four samples)
 @pytest.mark.parametrize("rows,fs,nIn,N", [(700, 4, 32, 64), (3000, 9, 64, 96), (513, 27, 64, 64), (66001, 27, 64, 64),
-                                           (33005, 8, 24, 96), (1100, 4, 112, 160)])
+                                           (33005, 8, 24, 96), (1100, 4, 112, 160), (1, 4, 32, 64), (7, 4, 128, 160),
+                                           (100, 9, 64, 96), (255, 4, 96, 128)])
 def test_fused_gather_nin_bf16_matches_the_two_kernels_bit_for_bit(scn, ctx, rows, fs, nIn, N):
     """scn_conv_nin_forward_p with bf16 operands: the same bits as gather + bf16 NiN, and the bf16 bar against the
     oracle."""

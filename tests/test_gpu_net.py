@@ -344,16 +344,22 @@ def test_dump_top_level_features_and_input_regularizing_constants(scn, tmp_path,
     net2.end()
 
 
+def top2_margin(probs):
+    """(p1 - p2) / p1 of every row: how far the arg-max is from changing"""
+    srt = np.sort(probs.astype(np.float64), axis=1)
+    return (srt[:, -1] - srt[:, -2]) / srt[:, -1]
+
+
 @pytest.mark.parametrize("mode", ["BF16", "BF16X3"])
 def test_bf16_mode_net(scn, mode):
-    """bf16 NiN contractions against the fp32 oracle on 200 samples.
+    """bf16 NiN contractions against the fp32 oracle on 200 samples of the 2-D net with random He-normal weights.
 
-    Plain bf16 operands: class probabilities within 2e-2 relative.  The
-    synthetic nets have random He-normal weights, so their 100-class softmax is
-    nearly flat and a 1e-2 relative change of the logits moves the arg-max of
-    2-3 % of the samples; top-1 agreement with plain bf16 is therefore checked
-    at 95 % here.  The hi + lo mode (three MFMAs per tile) has to meet the full
-    bar: 1e-4 relative and at least 99.5 % top-1 agreement."""
+    Class probabilities within 2e-2 relative (plain bf16 operands) or 1e-4 (hi + lo pairs, three MFMAs per tile).
+    A net with random weights has a nearly flat 100-class soft-max: the printed margins show the two largest
+    probabilities of many samples within a few per cent of each other, closer than the 2e-2 the mode is allowed
+    to move them.  So for plain bf16 the arg-max is required to agree wherever the oracle's own margin exceeds
+    twice that tolerance, and the plain count is printed; the 99.5 % bar itself is met on a trained, peaked
+    classifier in test_bf16_trained_net_meets_the_bar.  The hi + lo mode has to meet 99.5 % here too."""
     from sparseconvnet_archived_amd import hostapi, synthetic
     cfg = synthetic.config(2, batch=200)
     net, ora = build_pair(cfg, hostapi)
@@ -371,17 +377,142 @@ def test_bf16_mode_net(scn, mode):
     assert net.next_batch()
     out = net.batch_outputs()
     err = rel_l2(out["probabilities"], want["probabilities"])
-    agree = np.mean(out["predictions"][:, 0] == want["predictions"][:, 0])
-    print("%s probabilities rel-L2 %.3g, top-1 agreement %.4f" % (mode, err, agree), flush=True)
+    same = out["predictions"][:, 0] == want["predictions"][:, 0]
+    margin = top2_margin(want["probabilities"])
+    print("%s probabilities rel-L2 %.3g, top-1 agreement %.4f; oracle top-2 margins: 5%% %.4f, 25%% %.4f, median %.4f; "
+          "margins of the samples that disagree: %s" % (mode, err, same.mean(), *np.percentile(margin, [5, 25, 50]),
+                                                       np.round(margin[~same], 4).tolist()), flush=True)
     if mode == "BF16":
-        assert err <= 2e-2 and agree >= 0.95
+        assert err <= 2e-2
+        assert np.all(same[margin > 2 * 2e-2])
     else:
-        assert err <= 1e-4 and agree >= 0.995
+        assert err <= 1e-4 and same.mean() >= 0.995
     # rule books do not depend on the precision
     for i, wi in enumerate(want["interfaces"]):
         assert np.array_equal(net.interface(i, want_features=False)["rules"], wi["rules"])
     net.end()
     net.close()
+
+
+def test_bf16_trained_net_meets_the_bar(scn):
+    """The stated bar for bf16 operands -- 2e-2 relative, top-1 agreement of at least 99.5 % -- on a classifier that
+    has something to say: the 2-D net trained by this library's own processDataset(TRAINBATCH) on a separable
+    labelling (ten classes told apart by the mean colour of the strokes) until its soft-max is peaked, then 200
+    fresh samples forwarded with bf16 operands and compared with the fp32 oracle holding the trained weights."""
+    from sparseconvnet_archived_amd import hostapi, synthetic
+    cfg = synthetic.config(2, batch=100)
+    colours = np.random.default_rng(5).standard_normal((10, 3))
+    colours /= np.linalg.norm(colours, axis=1, keepdims=True)
+
+    def coloured(seed, n):
+        rng = np.random.default_rng(seed)
+        out = []
+        for i, (pts, f, _) in enumerate(synthetic.make_samples(cfg, seed, batch=n)):
+            out.append((pts, (colours[i % 10] + 0.3 * rng.uniform(-1, 1, f.shape)).astype(np.float32), i % 10))
+        return out
+
+    net, ora = build_pair(cfg, hostapi)
+    net.setFusedConvolutions(True)
+    for i, (W, B, pr) in synthetic.he_normal_weights(net.layers(), 9).items():
+        net.set_weights(i, W, B, pr)
+    train = hostapi.Dataset("train", 3, 100, hostapi.TRAINBATCH)
+    for pts, f, label in coloured(1, 400):
+        train.add_points(2, cfg.lattice, pts, f, label)
+    for epoch in range(30):
+        nll = net.processDatasetTrain(train, 100, 0.003, 0.9)
+    print("training NLL after 120 batches: %.5f" % nll, flush=True)
+    assert nll < 0.05
+    for i, l in enumerate(net.layers()):
+        if l["kind"].startswith("nin"):
+            ora.set_weights(i, *net.get_weights(i))
+    test = coloured(2, 200)
+    ds = hostapi.Dataset("test", 3, 100, hostapi.TESTBATCH)
+    for pts, f, label in test:
+        ds.add_points(2, cfg.lattice, pts, f, label)
+    S, K, R, bg, feats, n = synthetic.codify(test, 2, cfg.lattice, net.inputSpatialSize, 3)
+    want = ora.forward(200, S, K, R, bg, feats, n, np.array([s[2] for s in test], np.int32))
+    net.setPrecision(scn.BF16)
+    net.begin(ds, 200)
+    assert net.next_batch()
+    out = net.batch_outputs()
+    hidden = len(net.layers()) - 1  # input of the classifier: the last activations before the soft-max
+    errHidden = rel_l2(net.interface(hidden)["features"], want["interfaces"][hidden]["features"])
+    err = rel_l2(out["probabilities"], want["probabilities"])
+    agree = np.mean(out["predictions"][:, 0] == want["predictions"][:, 0])
+    margin = top2_margin(want["probabilities"])
+    print("trained net, bf16 operands: probabilities rel-L2 %.3g, classifier input rel-L2 %.3g, top-1 agreement %.4f, "
+          "oracle mistakes %d of 200, smallest top-2 margin %.4f" % (err, errHidden, agree, want["mistakes"], margin.min()),
+          flush=True)
+    assert want["mistakes"] <= 10  # the classifier did learn the labelling
+    assert err <= 2e-2 and errHidden <= 2e-2 and agree >= 0.995
+    assert errHidden > 1e-5  # ... and the operands really were rounded
+    net.end()
+    net.close()
+
+
+def test_bf16_wide_net(scn):
+    """The GEMM-bound 2-D net (contractions up to 2560 x 800) with bf16 operands, 8 samples against the fp32 oracle:
+    every materialised interface within 2e-2 relative, rule books and pooling choices of identical inputs exact."""
+    from sparseconvnet_archived_amd import hostapi, synthetic
+    cfg = synthetic.config(4, batch=8)
+    for fused in (False, True):
+        net, ora = build_pair(cfg, hostapi)
+        net.setPrecision(scn.BF16)
+        net.setFusedConvolutions(fused)
+        for i, (W, B, pr) in synthetic.he_normal_weights(net.layers(), 41).items():
+            net.set_weights(i, W, B, pr)
+            ora.set_weights(i, W, B, pr)
+        samples = synthetic.make_samples(cfg, 42)
+        ds = hostapi.Dataset("wide", 3, 100, hostapi.TESTBATCH)
+        for pts, f, label in samples:
+            ds.add_points(2, cfg.lattice, pts, f, label)
+        S, K, R, bg, feats, n = synthetic.codify(samples, 2, cfg.lattice, net.inputSpatialSize, 3)
+        want = ora.forward(len(samples), S, K, R, bg, feats, n, np.array([s[2] for s in samples], np.int32))
+        net.begin(ds, len(samples))
+        assert net.next_batch()
+        worst = 0.0
+        for i, wi in enumerate(want["interfaces"]):
+            gi = net.interface(i)
+            assert np.array_equal(gi["rules"], wi["rules"])
+            if gi["features"] is None:
+                assert fused
+                continue
+            worst = max(worst, rel_l2(gi["features"], wi["features"]))
+        out = net.batch_outputs()
+        err = rel_l2(out["probabilities"], want["probabilities"])
+        print("wide net, bf16 operands, fused %s: worst interface rel-L2 %.3g, probabilities %.3g" % (fused, worst, err),
+              flush=True)
+        assert worst <= 2e-2 and err <= 2e-2 and worst > 1e-5
+        net.end()
+        net.close()
+
+
+def test_bf16_fused_short_batches(scn):
+    """bf16 operands with fused convolutions on batches of one to four samples, as the last batch of a dataset may
+    be: the deepest convolutions then have a handful of rows.  Same bits as the unfused run."""
+    from sparseconvnet_archived_amd import hostapi, synthetic
+    cfg = synthetic.config(2, batch=10)
+    samples = synthetic.make_samples(cfg, 91)
+    runs = []
+    for fused in (False, True):
+        net, _ = build_pair(cfg, hostapi)
+        net.setPrecision(scn.BF16)
+        net.setFusedConvolutions(fused)
+        for i, (W, B, pr) in synthetic.he_normal_weights(net.layers(), 92).items():
+            net.set_weights(i, W, B, pr)
+        ds = hostapi.Dataset("short", 3, 100, hostapi.TESTBATCH)
+        for pts, f, label in samples:
+            ds.add_points(2, cfg.lattice, pts, f, label)
+        probs = []
+        for batch in (4, 3, 1):  # 4 + 4 + 2, 3 + 3 + 3 + 1, ten batches of one
+            net.begin(ds, batch)
+            while net.next_batch():
+                probs.append(net.batch_outputs()["probabilities"].copy())
+            net.end()
+        runs.append(np.concatenate(probs))
+        net.close()
+    assert runs[0].shape == (30, 100)
+    assert np.array_equal(runs[0], runs[1])
 
 
 def test_reference_style_cpp_driver(scn):
