@@ -257,6 +257,13 @@ int scn_conv_nin_forward_p(scn_ctx *ctx, const float *d_in,
 int scn_maxpool(scn_ctx *ctx, const float *d_in, float *d_out,
                 const int32_t *d_rules, int64_t nOutSites, int ps, int C,
                 int32_t *d_choice);
+/* The same for a caller that knows how many rows d_in has: the choices are
+ * 32-bit element indices into d_in, as the reference's poolingChoices are
+ * (MaxPoolingLayer.cu:9-35), so an input of more than 2^31 - 1 elements is
+ * refused with SCN_ERR_CAPACITY instead of being indexed modulo 2^32. */
+int scn_maxpool_checked(scn_ctx *ctx, const float *d_in, int64_t nInRows,
+                        float *d_out, const int32_t *d_rules,
+                        int64_t nOutSites, int ps, int C, int32_t *d_choice);
 /* terminalPool (TerminalPoolingLayer.cu:22-46): mean over the rows listed
  * before the first negative rule, summed in rule order. */
 int scn_terminal_pool(scn_ctx *ctx, const float *d_in, float *d_out,

@@ -113,6 +113,7 @@ def lib():
         "scn_conv_nin_forward_p": (C.c_int, [vp, vp, vp, C.c_int, C.c_int, vp, vp, vp, vp, i64, C.c_int, f32, C.c_int,
                                              C.c_int]),
         "scn_maxpool": (C.c_int, [vp, vp, vp, vp, i64, C.c_int, C.c_int, vp]),
+        "scn_maxpool_checked": (C.c_int, [vp, vp, i64, vp, vp, i64, C.c_int, C.c_int, vp]),
         "scn_terminal_pool": (C.c_int, [vp, vp, vp, vp, i64, C.c_int, C.c_int]),
         "scn_softmax_rows": (C.c_int, [vp, vp, vp, i64, C.c_int]),
         "scn_softmax_grad": (C.c_int, [vp, vp, vp, vp, i64, C.c_int]),

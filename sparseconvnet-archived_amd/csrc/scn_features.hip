@@ -133,7 +133,9 @@ __global__ void __launch_bounds__(256)
     } else {
       v[0] = src[0];
     }
-    int flat = rule * C + c0; // 32-bit, as the reference's poolingChoices
+    // 32-bit, as the reference's poolingChoices (the entry points refuse
+    // inputs of 2^31 elements and more where they know the input's size)
+    const int flat = (int)((unsigned)rule * (unsigned)C + (unsigned)c0);
 #pragma unroll
     for (int k = 0; k < VEC; ++k)
       if (none || best[k] < v[k]) {
@@ -179,6 +181,19 @@ extern "C" int scn_maxpool(scn_ctx *ctx, const float *d_in, float *d_out,
   }
   SCN_HIP_CHECK(hipGetLastError());
   return SCN_OK;
+}
+
+extern "C" int scn_maxpool_checked(scn_ctx *ctx, const float *d_in,
+                                   int64_t nInRows, float *d_out,
+                                   const int32_t *d_rules, int64_t nOutSites,
+                                   int ps, int C, int32_t *d_choice) {
+  SCN_REQUIRE(nInRows >= 0 && C >= 1, SCN_ERR_ARG,
+              "scn_maxpool_checked: nInRows %lld C %d", (long long)nInRows, C);
+  SCN_REQUIRE(nInRows * (int64_t)C <= 2147483647ll, SCN_ERR_CAPACITY,
+              "scn_maxpool: %lld input rows of %d features are %lld elements; "
+              "the 32-bit pooling choices index at most 2^31 - 1",
+              (long long)nInRows, C, (long long)(nInRows * (int64_t)C));
+  return scn_maxpool(ctx, d_in, d_out, d_rules, nOutSites, ps, C, d_choice);
 }
 
 // dTerminalPool (TerminalPoolingLayer.cu:22-34): sequential fp32 sum in rule

@@ -649,10 +649,12 @@ static void pool_forwards(cudaMemStream &ms,
   const size_t nf = output.featuresPresent.size();
   output.sub->poolingChoices.resize64((size_t)output.nSpatialSites * nf);
   output.sub->features.resize64((size_t)output.nSpatialSites * nf);
-  SCN_CHECKED(scn_maxpool(ms.ctx, input.sub->features.dPtr(),
-                          output.sub->features.dPtr(), output.rules.dPtr(),
-                          output.nSpatialSites, width, (int)nf,
-                          output.sub->poolingChoices.dPtr()));
+  SCN_CHECKED(scn_maxpool_checked(ms.ctx, input.sub->features.dPtr(),
+                                  input.nSpatialSites,
+                                  output.sub->features.dPtr(),
+                                  output.rules.dPtr(), output.nSpatialSites,
+                                  width, (int)nf,
+                                  output.sub->poolingChoices.dPtr()));
 }
 // MaxPoolingLayer::backwards (MaxPoolingLayer.cu:134-146)
 static void pool_backwards(cudaMemStream &ms,

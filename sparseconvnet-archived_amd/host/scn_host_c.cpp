@@ -187,11 +187,11 @@ int scnh_set_weights(scnh_net *net, int layer, const float *W, const float *B,
   }
   return -1;
 }
-void scnh_save_weights(scnh_net *net, const char *baseName, int epoch) {
-  net->cnn->saveWeights(baseName, epoch, false);
+void scnh_save_weights(scnh_net *net, const char *baseName, int epoch, int momentum) {
+  net->cnn->saveWeights(baseName, epoch, momentum != 0);
 }
-void scnh_load_weights(scnh_net *net, const char *baseName, int epoch) {
-  net->cnn->loadWeights(baseName, epoch, false);
+void scnh_load_weights(scnh_net *net, const char *baseName, int epoch, int momentum) {
+  net->cnn->loadWeights(baseName, epoch, momentum != 0);
 }
 
 scnh_dataset *scnh_dataset_create(const char *name, int nFeatures,

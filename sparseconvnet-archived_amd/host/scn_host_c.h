@@ -48,8 +48,9 @@ int scnh_set_weights(scnh_net *net, int layer, const float *W, const float *B,
  * skips that vector */
 int scnh_get_weights(scnh_net *net, int layer, int momentum, float *W,
                      float *B, float *prelu);
-void scnh_save_weights(scnh_net *net, const char *baseName, int epoch);
-void scnh_load_weights(scnh_net *net, const char *baseName, int epoch);
+/* momentum != 0: the momentum arrays follow each layer's parameters */
+void scnh_save_weights(scnh_net *net, const char *baseName, int epoch, int momentum);
+void scnh_load_weights(scnh_net *net, const char *baseName, int epoch, int momentum);
 
 scnh_dataset *scnh_dataset_create(const char *name, int nFeatures,
                                   int nClasses, int type);

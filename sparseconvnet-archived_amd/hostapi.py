@@ -48,8 +48,8 @@ def lib():
         "scnh_n_layers": (i32, [vp]),
         "scnh_layer_info": (i32, [vp, i32, P(i32), P(i32), P(i32)]),
         "scnh_set_weights": (i32, [vp, i32, vp, vp, vp]),
-        "scnh_save_weights": (None, [vp, C.c_char_p, i32]),
-        "scnh_load_weights": (None, [vp, C.c_char_p, i32]),
+        "scnh_save_weights": (None, [vp, C.c_char_p, i32, i32]),
+        "scnh_load_weights": (None, [vp, C.c_char_p, i32, i32]),
         "scnh_dataset_create": (vp, [C.c_char_p, i32, i32, i32]),
         "scnh_dataset_destroy": (None, [vp]),
         "scnh_dataset_add_points": (None, [vp, i32, i32, i64, vp, vp, i32]),
@@ -320,11 +320,11 @@ class Net:
             lib().scnh_iface_dfeatures(self.h, i, _p(out))
         return out
 
-    def saveWeights(self, base, epoch):
-        lib().scnh_save_weights(self.h, base.encode(), epoch)
+    def saveWeights(self, base, epoch, momentum=False):
+        lib().scnh_save_weights(self.h, base.encode(), epoch, int(momentum))
 
-    def loadWeights(self, base, epoch):
-        lib().scnh_load_weights(self.h, base.encode(), epoch)
+    def loadWeights(self, base, epoch, momentum=False):
+        lib().scnh_load_weights(self.h, base.encode(), epoch, int(momentum))
 
     def processDataset(self, ds, batchSize=100):
         return lib().scnh_process_dataset(self.h, ds.h, batchSize)

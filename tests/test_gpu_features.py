@@ -323,3 +323,26 @@ def test_fused_gather_nin_matches_the_two_kernels_bit_for_bit(scn, ctx, rows, fs
     assert np.all(np.abs(fused.download() - want) <= 1e-4 * scale)
     assert not scn.lib().scn_conv_nin_supported(64, 32, 64)  # window too large for the staged rules
     assert not scn.lib().scn_conv_nin_supported(4, 3, 32)  # channels not a multiple of 4
+
+
+def test_maxpool_refuses_inputs_beyond_32_bit_choices(scn, ctx):
+    """poolingChoices are 32-bit element indices into the input (MaxPoolingLayer.cu:9-35): the entry point that is told
+    the input's row count refuses 2^31 elements and more.  An argument check: nothing is launched, no such buffer
+    is needed."""
+    L = scn.lib()
+    one = ctx.empty(4, np.float32)
+    rows = (1 << 31) // 64
+    assert L.scn_maxpool_checked(ctx.h, one.ptr, rows, one.ptr, one.ptr, 1, 1, 64, one.ptr) == scn.ERR_CAPACITY
+    assert "32-bit" in L.scn_last_error().decode()
+    assert L.scn_maxpool_checked(ctx.h, one.ptr, -1, one.ptr, one.ptr, 1, 1, 64, one.ptr) == scn.ERR_ARG
+    # the largest input that fits, with no output rows asked for: accepted
+    assert L.scn_maxpool_checked(ctx.h, one.ptr, rows - 1, one.ptr, one.ptr, 0, 1, 64, one.ptr) == scn.OK
+    # ... and an ordinary call gives what scn_maxpool gives
+    rng = np.random.default_rng(1)
+    feats = rng.standard_normal((50, 8)).astype(np.float32)
+    rules = rng.integers(0, 50, (20, 4)).astype(np.int32)
+    d_f, d_r = ctx.array(feats), ctx.array(rules)
+    a, ca, b, cb = ctx.empty((20, 8), np.float32), ctx.empty((20, 8), np.int32), ctx.empty((20, 8), np.float32), ctx.empty((20, 8), np.int32)
+    ctx.maxpool(d_f, a, d_r, 20, 4, 8, ca)
+    assert L.scn_maxpool_checked(ctx.h, d_f.ptr, 50, b.ptr, d_r.ptr, 20, 4, 8, cb.ptr) == scn.OK
+    assert np.array_equal(a.download(), b.download()) and np.array_equal(ca.download(), cb.download())

@@ -290,6 +290,84 @@ def test_process_dataset_and_weight_files(scn, tmp_path):
     net2.processDatasetRepeatTest(ds, 10, 2)
 
 
+def test_weight_file_layout_byte_for_byte(scn, tmp_path):
+    """The .cnn format is raw little-endian fp32 with no header (SparseConvNetCUDA.cu:406-442): for every layer in
+    order W[nIn x nOut] row-major, B[nOut], for a PReLU layer its slopes (NetworkInNetworkLayer.cu:311-328,
+    NetworkInNetworkPReLULayer.cu:308-331), with `momentum` the layer's own momentum arrays in the same order right
+    behind them, and after the last layer inputNormalizingConstants.  Known values in, the file read back with
+    numpy.fromfile, every field at its place; then a file assembled here by hand is loaded."""
+    from sparseconvnet_archived_amd import hostapi, synthetic
+    stack = [("addLeNetLayerMP", 32, 2, 1, 2, 2, synthetic.RELU), ("addLeNetLayerMP", 32, 1, 1, 1, 1, synthetic.PRELU),
+             ("addTerminalPoolingLayer", 2), ("addSoftmaxLayer",)]
+    cfg = synthetic.Config("layout", 2, 3, 10, 4, 4, stack)
+    cfg.number = 2
+    net = hostapi.Net(2, 3, 10, nTop=1, threads=1)
+    cfg.build(net)
+    nin = [i for i, l in enumerate(net.layers()) if l["kind"].startswith("nin")]
+    assert [net.layers()[i]["kind"] for i in nin] == ["nin", "nin_prelu", "nin"]
+    assert [(net.layers()[i]["nIn"], net.layers()[i]["nOut"]) for i in nin] == [(12, 32), (32, 32), (32, 10)]
+    for n, i in enumerate(nin):  # every number in the file is different, and says where it belongs
+        l = net.layers()[i]
+        W = (1000 * (n + 1) + np.arange(l["nIn"] * l["nOut"]).reshape(l["nIn"], l["nOut"]) / 1024).astype(np.float32)
+        B = (2000 * (n + 1) + np.arange(l["nOut"]) / 64).astype(np.float32)
+        pr = (3000 * (n + 1) + np.arange(l["nOut"]) / 64).astype(np.float32) if l["kind"] == "nin_prelu" else None
+        net.set_weights(i, W * 1e-4, B * 1e-4, None if pr is None else pr * 1e-4)
+    rng = np.random.default_rng(3)
+    ds = hostapi.Dataset("layout", 3, 10, hostapi.TRAINBATCH)
+    for k in range(4):
+        pts = np.array([(a, b) for a in range(4) for b in range(4) if rng.random() < 0.6], np.int32)
+        ds.add_points(2, 4, pts, rng.uniform(-1, 1, (len(pts), 3)).astype(np.float32), k)
+    consts = net.calculateInputRegularizingConstants(ds)
+    assert len(consts) == 3
+    net.processDatasetTrain(ds, 4, 0.01, 0.9)  # one training batch: the momentum arrays are no longer zero
+    fields, moment = [], []
+    for i in nin:
+        W, B, pr = net.get_weights(i)
+        MW, MB, Mpr = net.get_weights(i, momentum=True)
+        assert np.abs(MW).max() > 0
+        fields.append([W.ravel(), B] + ([pr] if pr is not None else []))
+        moment.append([MW.ravel(), MB] + ([Mpr] if Mpr is not None else []))
+    base = str(tmp_path / "net")
+    net.saveWeights(base, 7)
+    net.saveWeights(base, 8, momentum=True)
+    plain = np.fromfile(base + "_epoch-7.cnn", "<f4")
+    full = np.fromfile(base + "_epoch-8.cnn", "<f4")
+    want_plain = np.concatenate([x for f in fields for x in f] + [np.asarray(consts, np.float32)])
+    want_full = np.concatenate([x for f, m in zip(fields, moment) for x in f + m] + [np.asarray(consts, np.float32)])
+    assert plain.size == want_plain.size and np.array_equal(plain, want_plain)
+    assert full.size == want_full.size and np.array_equal(full, want_full)
+    # W is row-major [nIn x nOut]: element (k, n) of the first layer sits at k * 32 + n
+    W0 = net.get_weights(nin[0])[0]
+    assert plain[5 * 32 + 7] == W0[5, 7]
+    # a file written by hand, momentum included, read by a fresh net
+    hand = [np.full(12 * 32, 0.5, np.float32), np.full(32, 0.25, np.float32),        # layer 1: W, B
+            np.full(12 * 32, -1.0, np.float32), np.full(32, -2.0, np.float32),       #          MW, MB
+            np.full(32 * 32, 0.125, np.float32), np.full(32, 0.75, np.float32), np.full(32, 0.3, np.float32),  # W, B, PReLU
+            np.full(32 * 32, -3.0, np.float32), np.full(32, -4.0, np.float32), np.full(32, -5.0, np.float32),  # momenta
+            np.full(32 * 10, 2.0, np.float32), np.full(10, 3.0, np.float32),         # classifier: W, B
+            np.full(32 * 10, -6.0, np.float32), np.full(10, -7.0, np.float32),
+            np.array([9.0, 8.0, 7.0], np.float32)]                                   # inputNormalizingConstants
+    np.concatenate(hand).astype("<f4").tofile(base + "_epoch-9.cnn")
+    net2 = hostapi.Net(2, 3, 10, nTop=1, threads=1)
+    cfg.build(net2)
+    net2.calculateInputRegularizingConstants(ds)  # sizes the vector, as the reference's drivers do before loading
+    net2.loadWeights(base, 9, momentum=True)
+    for i, (w, b, pr, mw, mb, mpr) in zip(nin, [(0.5, 0.25, None, -1.0, -2.0, None), (0.125, 0.75, 0.3, -3.0, -4.0, -5.0),
+                                                  (2.0, 3.0, None, -6.0, -7.0, None)]):
+        W, B, P = net2.get_weights(i)
+        MW, MB, MP = net2.get_weights(i, momentum=True)
+        assert np.all(W == w) and np.all(B == b) and np.all(MW == mw) and np.all(MB == mb)
+        assert (P is None and pr is None) or (np.all(P == np.float32(pr)) and np.all(MP == mpr))
+    assert net2.inputNormalizingConstants().tolist() == [9.0, 8.0, 7.0]
+    # without the flag the momentum arrays are not in the file: the same bytes then mean something else, and the
+    # loader zeroes the momenta (NetworkInNetworkLayer.cu:301-304)
+    net2.loadWeights(base, 7)
+    assert np.array_equal(net2.get_weights(nin[1])[0].ravel(), fields[1][0])
+    assert not net2.get_weights(nin[1], momentum=True)[0].any()
+    net.close()
+    net2.close()
+
+
 def test_dump_top_level_features_and_input_regularizing_constants(scn, tmp_path, monkeypatch):
     """processDatasetDumpTopLevelFeatures (every layer but the last, one text line per sample) and
     calculateInputRegularizingConstants (1 / max |x| per input feature, applied to every later batch and
@@ -418,10 +496,13 @@ def test_bf16_trained_net_meets_the_bar(scn):
     train = hostapi.Dataset("train", 3, 100, hostapi.TRAINBATCH)
     for pts, f, label in coloured(1, 400):
         train.add_points(2, cfg.lattice, pts, f, label)
-    for epoch in range(30):
+    net.set_training(0.003, 0.9, shuffle=False)  # (a fixed order of the batches: the same run every time)
+    for epoch in range(150):
         nll = net.processDatasetTrain(train, 100, 0.003, 0.9)
-    print("training NLL after 120 batches: %.5f" % nll, flush=True)
-    assert nll < 0.05
+        if nll < 0.01:
+            break
+    print("training NLL after %d batches: %.5f" % (4 * (epoch + 1), nll), flush=True)
+    assert nll < 0.01
     for i, l in enumerate(net.layers()):
         if l["kind"].startswith("nin"):
             ora.set_weights(i, *net.get_weights(i))
