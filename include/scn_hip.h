@@ -98,6 +98,10 @@ int scn_event_record(scn_ctx *ctx, scn_event *event);
 int scn_event_wait(scn_event *event);
 /* device-to-device, asynchronous on the context's stream */
 int scn_d2d(scn_ctx *ctx, void *d_dst, const void *d_src, size_t bytes);
+/* The same copy made by a kernel, for which either side may also be pinned
+ * host memory (scn_host_alloc) that the device reaches over the bus: an
+ * upload or download that costs the host one kernel launch. */
+int scn_copy(scn_ctx *ctx, void *dst, const void *src, size_t bytes);
 int scn_fill32(scn_ctx *ctx, void *d_dst, uint32_t word, size_t nWords);
 
 /* ---- sparse grids ----------------------------------------------------- */

@@ -81,6 +81,7 @@ def lib():
         "scn_host_alloc": (C.c_int, [vp, sz, C.POINTER(vp)]),
         "scn_host_free": (C.c_int, [vp, vp]),
         "scn_h2d_async": (C.c_int, [vp, vp, vp, C.c_size_t]),
+        "scn_copy": (C.c_int, [vp, vp, vp, C.c_size_t]),
         "scn_d2h_async": (C.c_int, [vp, vp, vp, sz]),
         "scn_event_create": (C.c_int, [vp, C.POINTER(vp)]),
         "scn_event_destroy": (C.c_int, [vp]),

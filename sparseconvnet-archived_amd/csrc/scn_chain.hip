@@ -98,17 +98,6 @@ struct ChainState {
 };
 
 // ------------------------------------------------------------------ device
-#ifdef CHAIN_TIMING
-__device__ long long g_chainT[512];
-#define CT(i)                                                                  \
-  if (blockIdx.x == 0 && threadIdx.x == 0)                                     \
-  g_chainT[i] = wall_clock64()
-extern "C" int scn_debug_chain_times(long long *out, int n) {
-  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_chainT), n * sizeof(long long));
-}
-#else
-#define CT(i)
-#endif
 
 // A barrier that orders LDS traffic only.  __syncthreads() also waits for the
 // global stores in flight (the staged rule rows), a microsecond or two each
@@ -369,8 +358,6 @@ __global__ void __launch_bounds__(CHAIN_THREADS) k_chain_sample(ChainArgs a) {
   };
   unsigned *arena = reinterpret_cast<unsigned *>(lds + a.arenaOff);
   const int arenaWords = a.arenaBytes / 4;
-
-  CT(0);
   // ---- the source grid of this sample: its slice of the batch's mask
   long long vol = a.vol0;
   int words = (int)((vol + 63) >> 6);
@@ -399,7 +386,6 @@ __global__ void __launch_bounds__(CHAIN_THREADS) k_chain_sample(ChainArgs a) {
       M(2)[w] = 0ull;
   }
   lds_barrier();
-  CT(1);
   unsigned nA;
   {
     const unsigned long long *bitsA = M(0);
@@ -410,7 +396,6 @@ __global__ void __launch_bounds__(CHAIN_THREADS) k_chain_sample(ChainArgs a) {
         [&](int i, unsigned v) { prefA[i] = (unsigned short)v; }, nA, 0,
         [&](int) { return 0u; }, [&](int, unsigned) {}, none, ws);
   }
-  CT(2);
   if ((long long)nA * CHAIN_IN_BYTES > a.arenaBytes) {
     chain_give_up(a);
     return;
@@ -445,7 +430,6 @@ __global__ void __launch_bounds__(CHAIN_THREADS) k_chain_sample(ChainArgs a) {
   }
   int bgA = a.bg[b];
   lds_barrier();
-  CT(3);
 
   for (int l = 0; l < a.nLevels; ++l) {
     const ChainLevel &L = a.lv[l];
@@ -562,7 +546,6 @@ __global__ void __launch_bounds__(CHAIN_THREADS) k_chain_sample(ChainArgs a) {
       }
     }
     lds_barrier();
-    CT(4 + 4 * l);
 
     // -- rows of the outputs: prefix sum of the owned counts, and the rank
     //    prefix of the output mask
@@ -572,7 +555,6 @@ __global__ void __launch_bounds__(CHAIN_THREADS) k_chain_sample(ChainArgs a) {
         [&](int i, unsigned v) { baseS[i] = (unsigned short)v; }, nB, wordsB,
         [&](int i) { return (unsigned)__popcll(bitsB[i]); },
         [&](int i, unsigned v) { prefB[i] = (unsigned short)v; }, nBits, ws);
-    CT(5 + 4 * l);
     const int hasBg = (long long)nB < L.fullSize;
     if ((long long)nA * CHAIN_IN_BYTES + (long long)nB * CHAIN_OUT_BYTES >
             a.arenaBytes ||
@@ -628,7 +610,6 @@ __global__ void __launch_bounds__(CHAIN_THREADS) k_chain_sample(ChainArgs a) {
         z[w] = 0ull;
     }
     lds_barrier();
-    CT(6 + 4 * l);
 
     // -- rule rows (sample-local row numbers) to the staging area
     if (L.rules) {
@@ -684,7 +665,6 @@ __global__ void __launch_bounds__(CHAIN_THREADS) k_chain_sample(ChainArgs a) {
           st[(long long)nB * L.width + q] = bgA;
     }
     lds_barrier();
-    CT(7 + 4 * l);
     // the output grid is the next layer's input
     keyA = keyB;
     rowA = rowB;

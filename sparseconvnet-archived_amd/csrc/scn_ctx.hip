@@ -194,13 +194,44 @@ extern "C" int scn_event_wait(scn_event *event) {
   return SCN_OK;
 }
 
-extern "C" int scn_d2d(scn_ctx *c, void *d_dst, const void *d_src,
-                       size_t bytes) {
+// A copy made by a kernel: either side may be device memory or pinned host
+// memory (which the device reads and writes over the bus).  Queueing it costs
+// the host one kernel launch, where an asynchronous memcpy of a few hundred
+// kilobytes costs many times that.
+__global__ void k_copy(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
+                       size_t bytes, int vec) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t step = (size_t)gridDim.x * blockDim.x;
+  if (vec) {
+    const size_t n16 = bytes / 16;
+    const uint4 *s = reinterpret_cast<const uint4 *>(src);
+    uint4 *d = reinterpret_cast<uint4 *>(dst);
+    for (size_t k = i; k < n16; k += step)
+      d[k] = s[k];
+    for (size_t k = n16 * 16 + i; k < bytes; k += step)
+      dst[k] = src[k];
+  } else {
+    for (size_t k = i; k < bytes; k += step)
+      dst[k] = src[k];
+  }
+}
+extern "C" int scn_copy(scn_ctx *c, void *dst, const void *src, size_t bytes) {
+  SCN_REQUIRE(c, SCN_ERR_ARG, "scn_copy: null context");
   if (bytes == 0)
     return SCN_OK;
-  SCN_HIP_CHECK(
-      hipMemcpyAsync(d_dst, d_src, bytes, hipMemcpyDeviceToDevice, c->stream));
+  SCN_REQUIRE(dst && src, SCN_ERR_ARG, "scn_copy: null buffer");
+  const int vec = (((uintptr_t)dst | (uintptr_t)src) & 15) == 0;
+  size_t blocks = (bytes / (vec ? 16 : 1) + 255) / 256;
+  blocks = blocks < 1 ? 1 : (blocks > 4096 ? 4096 : blocks);
+  hipLaunchKernelGGL(k_copy, dim3((unsigned)blocks), dim3(256), 0, c->stream,
+                     (const uint8_t *)src, (uint8_t *)dst, bytes, vec);
+  SCN_HIP_CHECK(hipGetLastError());
   return SCN_OK;
+}
+
+extern "C" int scn_d2d(scn_ctx *c, void *d_dst, const void *d_src,
+                       size_t bytes) {
+  return scn_copy(c, d_dst, d_src, bytes);
 }
 
 __global__ void k_fill32(uint32_t *dst, uint32_t w, size_t n) {

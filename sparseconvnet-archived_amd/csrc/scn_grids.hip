@@ -27,8 +27,11 @@
 __global__ void k_grid_build(GridView g, const int *sample,
                              const long long *key, const int *row, long long n,
                              long long *ekey, int *erow,
-                             unsigned long long *badSites) {
+                             unsigned long long *badSites,
+                             const int *bgIn, int *bgOut) {
   long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e < g.batch)
+    bgOut[e] = bgIn[e];
   if (e >= n)
     return;
   const int b = sample[e];
@@ -980,14 +983,14 @@ extern "C" int scn_grids_build(scn_ctx *ctx, scn_grids *g, int batch,
   ProfScope ps(ctx, SCN_K_GRID_BUILD);
   SCN_TRY(grids_prepare(ctx, g, batch, dimension, spatialSize, n));
   g->nSites = nSpatialSites;
-  if (batch > 0)
-    SCN_HIP_CHECK(hipMemcpyAsync(g->bg.p, d_background, batch * sizeof(int),
-                                 hipMemcpyDeviceToDevice, ctx->stream));
-  if (n > 0) {
-    hipLaunchKernelGGL(k_grid_build, dim3(scn_ceil_div(n, 256)), dim3(256), 0,
+  // (backgroundCol is copied by the same launch: lane e < batch takes entry e)
+  const long long lanes = n > batch ? n : batch;
+  if (lanes > 0) {
+    hipLaunchKernelGGL(k_grid_build, dim3(scn_ceil_div(lanes, 256)), dim3(256), 0,
                        ctx->stream, view_of(g), d_sample,
                        (const long long *)d_key, d_row, (long long)n, g->ekey.p,
-                       g->erow.p, (unsigned long long *)(ctx->d_scalars + 15));
+                       g->erow.p, (unsigned long long *)(ctx->d_scalars + 15),
+                       d_background, g->bg.p);
     SCN_HIP_CHECK(hipGetLastError());
   }
   return SCN_OK;

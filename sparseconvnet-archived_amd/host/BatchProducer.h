@@ -6,12 +6,49 @@
 // caller in order, so rule books of the next batches are built while the
 // forward pass of the current one runs on the net's stream.
 #pragma once
+#include <mutex>
+#include <memory>
 #include <condition_variable>
 #include <thread>
 #include <vector>
 #include "SparseConvNetCUDA.h"
 #include "SpatiallySparseBatch.h"
 #include "SpatiallySparseDataset.h"
+
+class BatchProducer;
+
+// The dataset loops' way through the batches of a BatchProducer: the forward
+// pass of a batch is only queued, on the next forward lane in turn, and a batch
+// is finished (probabilities read, statistics taken) when as many younger
+// ones are queued behind it as the net has lanes -- so the GPU never waits for
+// the host between batches.  Training batches run one after the other.
+class ForwardQueue {
+public:
+  ForwardQueue(SparseConvNetCUDA &cnn, BatchProducer &bp, bool training);
+  ~ForwardQueue();
+  // queues b; returns the batch that has to be finished now, or null
+  SpatiallySparseBatch *push(SpatiallySparseBatch *b);
+  // the oldest batch still queued, or null when there is none (call until null)
+  SpatiallySparseBatch *pop();
+  int depth;
+
+private:
+  SparseConvNetCUDA &cnn;
+  std::vector<SpatiallySparseBatch *> inFlight;
+  int lanes, count;
+  // With several lanes the kernel launches of a forward pass are made by a
+  // thread per lane: queueing a pass costs the host about as long as the GPU
+  // needs to run it, and one thread cannot feed two lanes.
+  struct Worker {
+    std::thread thread;
+    std::mutex m;
+    std::condition_variable cv;
+    std::vector<SpatiallySparseBatch *> todo;
+    bool stop = false;
+  };
+  std::vector<std::unique_ptr<Worker>> workers;
+  void work(int lane);
+};
 
 class BatchProducer {
 public:

@@ -58,6 +58,19 @@ public:
   // number goes first, so the consumer's next batch is never behind a later
   // one); the CPU halves of all threads run side by side.
   std::vector<std::unique_ptr<cudaMemStream>> batchMemStreams;
+  // Forward lanes.  The kernels of one forward pass follow one another on one
+  // stream, and most of them are too short to fill the GPU: with two lanes
+  // the dataset loops keep the forward passes of two consecutive test batches
+  // in flight, each on a stream and a set of feature buffers of its own (the
+  // reference shares one set between all batches because it runs one batch at
+  // a time, BatchProducer.cu:28-33).  Lane 0 is memStream and the shared
+  // buffers.  Results do not depend on the number of lanes.  Training batches
+  // always use lane 0: they update the weights.
+  int nForwardLanes;
+  std::vector<std::unique_ptr<cudaMemStream>> laneStreams; // lanes 1, 2, ..
+  std::vector<std::vector<SpatiallySparseBatchSubInterface *>> laneSubInterfaces;
+  cudaMemStream &laneStream(int lane);
+  void synchronizeLanes();
   cudaMemStream *acquireProducerStream(int batchNumber);
   void releaseProducerStream(cudaMemStream *stream);
   // fewer producer threads than the net was constructed with
@@ -78,7 +91,7 @@ public:
                     int pciBusID = -1, int nTop = 1,
                     int nBatchProducerThreads = 10);
   ~SparseConvNetCUDA();
-  void forwardBatch(SpatiallySparseBatch &batch);
+  void forwardBatch(SpatiallySparseBatch &batch, int lane = 0);
   void backwardBatch(SpatiallySparseBatch &batch, float learningRate,
                      float momentum);
   // training batches are drawn in shuffled order (BatchProducer.cu:23-26);

@@ -1,5 +1,6 @@
 // One batch travelling through the net (SpatiallySparseBatch.h:7-22).
 #pragma once
+#include <atomic>
 #include <memory>
 #include <vector>
 #include "SpatiallySparseBatchInterface.h"
@@ -19,6 +20,9 @@ struct BatchResultStage {
   // back to its producer only after this point has been passed.
   scn_event *consumed;
   bool consumedPending;
+  // set by the thread that queued the batch's forward pass once all of it is
+  // queued (the dataset loops may leave that to a thread per forward lane)
+  std::atomic<bool> enqueued;
   // the labels as the statistics need them, on the host, while batch.labels
   // is in device memory for the gradient of a training batch
   std::vector<int> labels;
@@ -37,6 +41,9 @@ public:
   // The stream this slot's preprocess() -- grid upload and rule-book kernels
   // -- is issued on (one of the net's batchMemStreams); null: the layer's own.
   cudaMemStream *preprocessStream;
+  // The stream this batch's forward pass is issued on when that is not the
+  // layers' own (a net with several forward lanes); null: the layers' own.
+  cudaMemStream *forwardStream;
   batchType type;
   int batchSize;
   std::vector<int> sampleNumbers;

@@ -20,6 +20,11 @@ const char *batchTypeNames[] = {"TRAINBATCH", "TESTBATCH", "UNLABELEDBATCH",
 const char *sigmoidNames[] = {"", "ReLU", "VeryLeakyReLU", "LeakyReLU", "tanh",
                               "Softmax Classification", "PReLU", "Sigmoid"};
 __int128_t multiplyAddCount;
+static std::mutex g_macMutex;
+void addMultiplyAdds(__int128_t n) {
+  std::lock_guard<std::mutex> lock(g_macMutex);
+  multiplyAddCount += n;
+}
 
 // ---- utilities (utilities.cu:5-56,102-103) -----------------------------------
 std::vector<int> range(int n) {
@@ -346,7 +351,7 @@ void SpatiallySparseBatchInterface::summary() {
 
 BatchResultStage::BatchResultStage()
     : pinned(nullptr), capacity(0), arrived(nullptr), pending(false),
-      consumed(nullptr), consumedPending(false) {}
+      consumed(nullptr), consumedPending(false), enqueued(true) {}
 BatchResultStage::~BatchResultStage() {
   if (arrived)
     scn_event_destroy(arrived);
@@ -358,7 +363,8 @@ BatchResultStage::~BatchResultStage() {
 
 SpatiallySparseBatch::SpatiallySparseBatch(
     SpatiallySparseBatchSubInterface *inputSub)
-    : inputSub(inputSub), preprocessStream(nullptr), labels(false, 0),
+    : inputSub(inputSub), preprocessStream(nullptr), forwardStream(nullptr),
+      labels(false, 0),
       stagingSample(true, 0), stagingKey(true, 0), stagingRow(true, 0),
       stagingBackground(true, 0), result(new BatchResultStage()) {
   interfaces.emplace_back(inputSub);

@@ -30,6 +30,10 @@ void SpatiallySparseLayer::backwards(SpatiallySparseBatch &,
 static scn_ctx *pre_ctx(SpatiallySparseBatch &batch, cudaMemStream &ms) {
   return batch.preprocessStream ? batch.preprocessStream->ctx : ms.ctx;
 }
+// forwards() runs on the batch's forward lane when the net has given it one
+static cudaMemStream &fwd_stream(SpatiallySparseBatch &batch, cudaMemStream &ms) {
+  return batch.forwardStream ? *batch.forwardStream : ms;
+}
 
 // the output interface's own grids object, created on first use and kept for
 // later batches (its tables only grow)
@@ -149,7 +153,7 @@ void ConvolutionalLayer::forwards(SpatiallySparseBatch &batch,
     output.deferredGatherFrom = &input; // the following NiN layer gathers
     return;
   }
-  gather_now(memStream, input, output);
+  gather_now(fwd_stream(batch, memStream), input, output);
 }
 void ConvolutionalLayer::backwards(SpatiallySparseBatch &batch,
                                    SpatiallySparseBatchInterface &input,
@@ -212,7 +216,7 @@ void ConvolutionalTriangularLayer::forwards(
     output.deferredGatherFrom = &input; // the following NiN layer gathers
     return;
   }
-  gather_now(memStream, input, output);
+  gather_now(fwd_stream(batch, memStream), input, output);
 }
 void ConvolutionalTriangularLayer::backwards(
     SpatiallySparseBatch &batch, SpatiallySparseBatchInterface &input,
@@ -288,7 +292,7 @@ static void nin_forwards_shrunk(cudaMemStream &ms,
                               b.dPtr(), PReLU ? PReLU->dPtr() : nullptr,
                               output.sub->features.dPtr(), output.nSpatialSites,
                               Kp, Np, 1.0f, act, precision));
-  multiplyAddCount += (__int128_t)output.nSpatialSites * Kp * Np;
+  addMultiplyAdds((__int128_t)output.nSpatialSites * Kp * Np);
 }
 // When the preceding convolutional layer deferred its gather: run the fused
 // kernel (fp32 operands), or gather now if this layer wants bf16 operands.
@@ -353,7 +357,7 @@ static void nin_backwards(cudaMemStream &ms,
   SCN_CHECKED((clean ? scn_sgemm_AtB_acc : scn_sgemm_AtB)(
       ms.ctx, input.sub->features.dPtr(), output.sub->dfeatures.dPtr(),
       dw.dPtr(), M, K, N));
-  multiplyAddCount += (__int128_t)M * K * N;
+  addMultiplyAdds((__int128_t)M * K * N);
   if (input.backpropErrors) {
     input.sub->dfeatures.resize64((size_t)input.nSpatialSites * K);
     workspace.resize64((size_t)scn_sgemm_ABt_workspace(N, K));
@@ -361,7 +365,7 @@ static void nin_backwards(cudaMemStream &ms,
                               shrunkW ? shrunkW->dPtr() : W.dPtr(),
                               input.sub->dfeatures.dPtr(), M, N, K,
                               workspace.dPtr()));
-    multiplyAddCount += (__int128_t)M * K * N;
+    addMultiplyAdds((__int128_t)M * K * N);
   }
   if (shrunkW) {
     if (PReLU)
@@ -436,15 +440,15 @@ void NetworkInNetworkLayer::forwards(SpatiallySparseBatch &batch,
   }
   // test-time scaling by the kept fraction (NetworkInNetworkLayer.cu:188)
   float p = 1.0f - (batch.type != RESCALEBATCH ? dropout : 0.0f);
-  if (!nin_fused(memStream, input, output, W, B, nullptr, nFeaturesOut, p,
+  cudaMemStream &ms = fwd_stream(batch, memStream);
+  if (!nin_fused(ms, input, output, W, B, nullptr, nFeaturesOut, p,
                  (int)fn, precision))
-    SCN_CHECKED(scn_nin_forward(memStream.ctx, input.sub->features.dPtr(),
+    SCN_CHECKED(scn_nin_forward(ms.ctx, input.sub->features.dPtr(),
                                 W.dPtr(), B.dPtr(), nullptr,
                                 output.sub->features.dPtr(),
                                 output.nSpatialSites, nFeaturesIn, nFeaturesOut,
                                 p, (int)fn, precision));
-  multiplyAddCount +=
-      (__int128_t)output.nSpatialSites * nFeaturesIn * nFeaturesOut;
+  addMultiplyAdds((__int128_t)output.nSpatialSites * nFeaturesIn * nFeaturesOut);
 }
 void NetworkInNetworkLayer::backwards(SpatiallySparseBatch &batch,
                                       SpatiallySparseBatchInterface &input,
@@ -567,15 +571,15 @@ void NetworkInNetworkPReLULayer::forwards(
     return;
   }
   float p = 1.0f - (batch.type != RESCALEBATCH ? dropout : 0.0f);
-  if (!nin_fused(memStream, input, output, W, B, &PReLU, nFeaturesOut, p,
+  cudaMemStream &ms = fwd_stream(batch, memStream);
+  if (!nin_fused(ms, input, output, W, B, &PReLU, nFeaturesOut, p,
                  (int)PRELU, precision))
-    SCN_CHECKED(scn_nin_forward(memStream.ctx, input.sub->features.dPtr(),
+    SCN_CHECKED(scn_nin_forward(ms.ctx, input.sub->features.dPtr(),
                                 W.dPtr(), B.dPtr(), PReLU.dPtr(),
                                 output.sub->features.dPtr(),
                                 output.nSpatialSites, nFeaturesIn, nFeaturesOut,
                                 p, (int)PRELU, precision));
-  multiplyAddCount +=
-      (__int128_t)output.nSpatialSites * nFeaturesIn * nFeaturesOut;
+  addMultiplyAdds((__int128_t)output.nSpatialSites * nFeaturesIn * nFeaturesOut);
 }
 void NetworkInNetworkPReLULayer::backwards(
     SpatiallySparseBatch &batch, SpatiallySparseBatchInterface &input,
@@ -679,8 +683,7 @@ void MaxPoolingLayer::backwards(SpatiallySparseBatch &batch,
 void MaxPoolingLayer::forwards(SpatiallySparseBatch &batch,
                                SpatiallySparseBatchInterface &input,
                                SpatiallySparseBatchInterface &output) {
-  (void)batch;
-  pool_forwards(memStream, input, output, sd);
+  pool_forwards(fwd_stream(batch, memStream), input, output, sd);
 }
 int MaxPoolingLayer::calculateInputSpatialSize(int outputSpatialSize) {
   outSpatialSize = outputSpatialSize;
@@ -730,8 +733,7 @@ void MaxPoolingTriangularLayer::backwards(
 void MaxPoolingTriangularLayer::forwards(SpatiallySparseBatch &batch,
                                          SpatiallySparseBatchInterface &input,
                                          SpatiallySparseBatchInterface &output) {
-  (void)batch;
-  pool_forwards(memStream, input, output, S);
+  pool_forwards(fwd_stream(batch, memStream), input, output, S);
 }
 int MaxPoolingTriangularLayer::calculateInputSpatialSize(
     int outputSpatialSize) {
@@ -863,8 +865,7 @@ void FractionalMaxPoolingLayer::preprocess(
 void FractionalMaxPoolingLayer::forwards(SpatiallySparseBatch &batch,
                                          SpatiallySparseBatchInterface &input,
                                          SpatiallySparseBatchInterface &output) {
-  (void)batch;
-  pool_forwards(memStream, input, output, sd);
+  pool_forwards(fwd_stream(batch, memStream), input, output, sd);
 }
 void FractionalMaxPoolingLayer::backwards(
     SpatiallySparseBatch &batch, SpatiallySparseBatchInterface &input,
@@ -911,7 +912,8 @@ void TerminalPoolingLayer::forwards(SpatiallySparseBatch &batch,
   output.sub->poolingChoices.resize64((size_t)output.nSpatialSites * nf);
   output.sub->features.resize64((size_t)output.nSpatialSites * nf);
   SCN_CHECKED(scn_terminal_pool(
-      memStream.ctx, input.sub->features.dPtr(), output.sub->features.dPtr(),
+      fwd_stream(batch, memStream).ctx, input.sub->features.dPtr(),
+      output.sub->features.dPtr(),
       output.rules.dPtr(), output.nSpatialSites,
       (int)(output.rules.size64() / batch.batchSize), (int)nf));
 }

@@ -1,10 +1,12 @@
 // Net runtime, batch production, public facades and canned architectures.
 #include <algorithm>
+#include <atomic>
 #include <cassert>
 #include <chrono>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
+#include <thread>
 #include "BatchProducer.h"
 #include "NetworkArchitectures.h"
 #include "SparseConvNet.h"
@@ -26,6 +28,11 @@ SparseConvNetCUDA::SparseConvNetCUDA(int dimension, int nInputFeatures,
   std::cout << "Sparse CNN - dimension=" << dimension
             << " nInputFeatures=" << nInputFeatures << " nClasses=" << nClasses
             << std::endl;
+  // (lane streams first: streams take hardware queues in order of creation,
+  // and the forward passes should not share theirs with producer streams)
+  nForwardLanes = nBatchProducerThreads >= 4 ? 2 : 1;
+  for (int lane = 1; lane < nForwardLanes; ++lane)
+    laneStreams.emplace_back(new cudaMemStream());
   batchPool.reserve(nBatchProducerThreads);
   const int nStreams = std::min(nBatchProducerThreads, N_PRODUCER_STREAMS);
   for (int c = 0; c < nStreams; c++) {
@@ -58,10 +65,20 @@ void SparseConvNetCUDA::releaseProducerStream(cudaMemStream *stream) {
   }
   streamPoolChanged.notify_all();
 }
+cudaMemStream &SparseConvNetCUDA::laneStream(int lane) {
+  return lane == 0 ? memStream : *laneStreams[lane - 1];
+}
+void SparseConvNetCUDA::synchronizeLanes() {
+  memStream.synchronize();
+  for (auto &s : laneStreams)
+    s->synchronize();
+}
 void SparseConvNetCUDA::limitBatchProducerThreads(int n) {
   if (n < 1 || n >= nBatchProducerThreads)
     return;
   nBatchProducerThreads = n;
+  if (n < 4)
+    nForwardLanes = 1;
   while ((int)batchPool.size() > n)
     batchPool.pop_back();
   const int nStreams = std::min(n, N_PRODUCER_STREAMS);
@@ -76,7 +93,7 @@ void SparseConvNetCUDA::limitBatchProducerThreads(int n) {
 SparseConvNetCUDA::~SparseConvNetCUDA() {
   for (auto &s : batchMemStreams)
     s->synchronize();
-  memStream.synchronize();
+  synchronizeLanes();
   batchPool.clear();
   for (auto p : layers)
     delete p;
@@ -84,6 +101,9 @@ SparseConvNetCUDA::~SparseConvNetCUDA() {
     delete p;
   for (auto p : sharedSubInterfaces)
     delete p;
+  for (auto &lane : laneSubInterfaces)
+    for (auto p : lane)
+      delete p;
 }
 // SparseConvNetCUDA.cu:50-70
 void SparseConvNetCUDA::addLearntLayer(int nFeatures,
@@ -232,6 +252,11 @@ void SparseConvNetCUDA::ensureInterfaces() {
     for (auto &slot : batchPool)
       slot.interfaces.emplace_back(sharedSubInterfaces.back());
   }
+  // ... and one more set per forward lane beyond the first
+  laneSubInterfaces.resize(laneStreams.size());
+  for (auto &lane : laneSubInterfaces)
+    while (lane.size() < sharedSubInterfaces.size())
+      lane.push_back(new SpatiallySparseBatchSubInterface());
 }
 // every grids object the slot owns, emptied in one launch at the start of a batch
 static void clearDeviceGrids(scn_ctx *ctx, SpatiallySparseBatch &b) {
@@ -303,28 +328,9 @@ void SparseConvNetCUDA::preprocessResident(int cc, const ResidentBatch &input) {
   const int32_t *d_sample = input.d_sample, *d_row = input.d_row,
                 *d_background = input.d_background;
   const int64_t *d_key = input.d_key;
-  const size_t n = (size_t)input.nActive;
-  if (input.onHost) {
-    // sites in pinned host memory: uploaded on this slot's stream first
-    // (BatchProducer.cu:127-134 uploads a batch's inputs the same way)
-    b.stagingSample.copyToGPU();
-    b.stagingKey.copyToGPU();
-    b.stagingRow.copyToGPU();
-    b.stagingBackground.copyToGPU();
-    b.stagingSample.resize64(n);
-    b.stagingKey.resize64(2 * n);
-    b.stagingRow.resize64(n);
-    b.stagingBackground.resize64((size_t)input.batchSize);
-    SCN_CHECKED(scn_h2d_async(ctx, b.stagingSample.dPtr(), input.d_sample, n * 4));
-    SCN_CHECKED(scn_h2d_async(ctx, b.stagingKey.dPtr(), input.d_key, n * 8));
-    SCN_CHECKED(scn_h2d_async(ctx, b.stagingRow.dPtr(), input.d_row, n * 4));
-    SCN_CHECKED(scn_h2d_async(ctx, b.stagingBackground.dPtr(), input.d_background,
-                              (size_t)input.batchSize * 4));
-    d_sample = b.stagingSample.dPtr();
-    d_key = (const int64_t *)b.stagingKey.dPtr();
-    d_row = b.stagingRow.dPtr();
-    d_background = b.stagingBackground.dPtr();
-  }
+  // (input.onHost: the arrays are pinned host memory, which the device reads
+  // over the bus -- the grid-building kernel and the copy below are the upload,
+  // BatchProducer.cu:127-134, on this slot's stream)
   SCN_CHECKED(scn_grids_build(ctx, in.deviceGrids, input.batchSize, dimension,
                               in.spatialSize, d_sample, d_key, d_row,
                               input.nActive, d_background,
@@ -332,12 +338,8 @@ void SparseConvNetCUDA::preprocessResident(int cc, const ResidentBatch &input) {
   in.sub->features.copyToGPU();
   size_t nElems = (size_t)input.nSpatialSites * nInputFeatures;
   in.sub->features.resize64(nElems);
-  if (input.onHost)
-    SCN_CHECKED(scn_h2d_async(ctx, in.sub->features.dPtr(), input.d_features,
-                              nElems * sizeof(float)));
-  else
-    SCN_CHECKED(scn_d2d(ctx, in.sub->features.dPtr(), input.d_features,
-                        nElems * sizeof(float)));
+  SCN_CHECKED(scn_copy(ctx, in.sub->features.dPtr(), input.d_features,
+                       nElems * sizeof(float)));
   buildRuleBooks(*this, ctx, b);
   SCN_CHECKED(scn_sync(ctx));
 }
@@ -381,13 +383,21 @@ void SparseConvNetCUDA::backwardBatch(SpatiallySparseBatch &batch,
 // finishBatch waits for that copy and does the host-side statistics.  The
 // dataset loops queue batch i + 1 before finishing batch i, so the stream never
 // runs dry while the host is busy.
-void SparseConvNetCUDA::forwardBatch(SpatiallySparseBatch &batch) {
+void SparseConvNetCUDA::forwardBatch(SpatiallySparseBatch &batch, int lane) {
+  assert(lane >= 0 && lane < nForwardLanes);
+  assert(lane == 0 || (batch.type != TRAINBATCH && batch.type != RESCALEBATCH));
+  // the lane's stream and feature buffers
+  cudaMemStream &ms = laneStream(lane);
+  batch.forwardStream = lane == 0 ? nullptr : &ms;
+  for (size_t i = 0; i < layers.size(); i++)
+    batch.interfaces[i + 1].sub =
+        lane == 0 ? sharedSubInterfaces[i] : laneSubInterfaces[lane - 1][i];
   // a RESCALEBATCH rescales every layer's weights right after its forward
   // pass (SparseConvNetCUDA.cu:230-241)
   float scalingUnderneath = 1;
   for (size_t i = 0; i < layers.size(); i++) {
     batch.interfaces[i + 1].sub->reset();
-    scn_prof_tag(memStream.ctx, (int)i);
+    scn_prof_tag(ms.ctx, (int)i);
     layers[i]->forwards(batch, batch.interfaces[i], batch.interfaces[i + 1]);
     if (batch.type == RESCALEBATCH) {
       std::cout << i << ":"
@@ -398,7 +408,7 @@ void SparseConvNetCUDA::forwardBatch(SpatiallySparseBatch &batch) {
                               scalingUnderneath, i == layers.size() - 1);
     }
   }
-  SoftmaxClassifierLaunch(batch.interfaces.back(), batch, memStream);
+  SoftmaxClassifierLaunch(batch.interfaces.back(), batch, ms);
 }
 void SparseConvNetCUDA::finishBatch(SpatiallySparseBatch &batch,
                                     std::ofstream &f, std::ofstream &g) {
@@ -428,6 +438,76 @@ static void printThroughput(long long nanoseconds, size_t nPictures) {
             << " rate:" << roundf(nPictures * 1000000000.0f / nanoseconds)
             << "/s" << std::endl;
 }
+ForwardQueue::ForwardQueue(SparseConvNetCUDA &cnn, BatchProducer &bp,
+                           bool training)
+    : cnn(cnn), count(0) {
+  lanes = training ? 1 : cnn.nForwardLanes;
+  // a batch stays queued while up to `depth` younger ones are queued behind
+  // it; each of them holds a slot, and the producers need one to work in
+  depth = std::min(lanes, cnn.nBatchProducerThreads - 1);
+  if (depth < lanes)
+    lanes = std::max(1, depth);
+  bp.keepAlive = depth;
+  if (lanes > 1)
+    for (int lane = 0; lane < lanes; ++lane) {
+      workers.emplace_back(new Worker());
+      workers.back()->thread = std::thread(&ForwardQueue::work, this, lane);
+    }
+}
+ForwardQueue::~ForwardQueue() {
+  for (auto &w : workers) {
+    {
+      std::lock_guard<std::mutex> lock(w->m);
+      w->stop = true;
+    }
+    w->cv.notify_all();
+    w->thread.join();
+  }
+}
+void ForwardQueue::work(int lane) {
+  Worker &w = *workers[lane];
+  for (;;) {
+    SpatiallySparseBatch *b = nullptr;
+    {
+      std::unique_lock<std::mutex> lock(w.m);
+      w.cv.wait(lock, [&] { return w.stop || !w.todo.empty(); });
+      if (w.todo.empty())
+        return; // (stop is only set once everything queued has been popped)
+      b = w.todo.front();
+      w.todo.erase(w.todo.begin());
+    }
+    cnn.forwardBatch(*b, lane);
+    b->result->enqueued.store(true, std::memory_order_release);
+  }
+}
+SpatiallySparseBatch *ForwardQueue::push(SpatiallySparseBatch *b) {
+  const int lane = count++ % lanes;
+  if (workers.empty()) {
+    cnn.forwardBatch(*b, lane);
+  } else {
+    b->result->enqueued.store(false, std::memory_order_relaxed);
+    Worker &w = *workers[lane];
+    {
+      std::lock_guard<std::mutex> lock(w.m);
+      w.todo.push_back(b);
+    }
+    w.cv.notify_one();
+  }
+  inFlight.push_back(b);
+  if ((int)inFlight.size() > depth)
+    return pop();
+  return nullptr;
+}
+SpatiallySparseBatch *ForwardQueue::pop() {
+  if (inFlight.empty())
+    return nullptr;
+  SpatiallySparseBatch *b = inFlight.front();
+  inFlight.erase(inFlight.begin());
+  // its forward pass may still be on its way into the lane's stream
+  while (!b->result->enqueued.load(std::memory_order_acquire))
+    std::this_thread::yield();
+  return b;
+}
 // SparseConvNetCUDA.cu:272-326
 float SparseConvNetCUDA::processDataset(SpatiallySparseDataset &dataset,
                                         int batchSize, float learningRate,
@@ -442,27 +522,36 @@ float SparseConvNetCUDA::processDataset(SpatiallySparseDataset &dataset,
     f.open("unlabelledData.predictions");
     g.open("unlabelledData.probabilities");
   }
-  bp.keepAlive = nBatchProducerThreads >= 2 ? 1 : 0;
-  SpatiallySparseBatch *queued = nullptr; // forward pass queued, not yet read
+  const bool oneLane = dataset.type == TRAINBATCH || dataset.type == RESCALEBATCH;
+  ForwardQueue queue(*this, bp, oneLane);
+  SpatiallySparseBatch *trainQueued = nullptr; // training batch queued, not yet read
   auto finish = [&](SpatiallySparseBatch *batch) {
     finishBatch(*batch, f, g);
     errorRate += batch->mistakes * 1.0 / dataset.pictures.size();
     nll += batch->negativeLogLikelihood * 1.0 / dataset.pictures.size();
   };
   while (SpatiallySparseBatch *batch = bp.nextBatch()) {
-    forwardBatch(*batch);
-    if (batch->type == TRAINBATCH)
+    SpatiallySparseBatch *due = nullptr;
+    if (batch->type == TRAINBATCH) {
+      forwardBatch(*batch);
       backwardBatch(*batch, learningRate, momentum);
-    if (queued)
-      finish(queued);
-    queued = batch;
-    if (!bp.keepAlive) {
-      finish(queued);
-      queued = nullptr;
+      // (one training batch may stay queued while the next is produced)
+      due = trainQueued;
+      trainQueued = batch;
+      if (!bp.keepAlive) {
+        due = batch;
+        trainQueued = nullptr;
+      }
+    } else {
+      due = queue.push(batch);
     }
+    if (due)
+      finish(due);
   }
-  if (queued)
-    finish(queued);
+  if (trainQueued)
+    finish(trainQueued);
+  while (SpatiallySparseBatch *batch = queue.pop())
+    finish(batch);
   auto end = std::chrono::system_clock::now();
   auto diff =
       std::chrono::duration_cast<std::chrono::nanoseconds>(end - start).count();
@@ -544,8 +633,7 @@ void SparseConvNetCUDA::processDatasetRepeatTest(
   for (int rep = 1; rep <= nReps; ++rep) {
     {
       BatchProducer bp(*this, dataset, inputSpatialSize, batchSize);
-      bp.keepAlive = nBatchProducerThreads >= 2 ? 1 : 0;
-      SpatiallySparseBatch *queued = nullptr;
+      ForwardQueue queue(*this, bp, false);
       auto finish = [&](SpatiallySparseBatch *batch) {
         std::ofstream f, g;
         finishBatch(*batch, f, g);
@@ -556,18 +644,11 @@ void SparseConvNetCUDA::processDatasetRepeatTest(
             probs[ii][j] += batch->probabilities[i][j];
         }
       };
-      while (SpatiallySparseBatch *batch = bp.nextBatch()) {
-        forwardBatch(*batch);
-        if (queued)
-          finish(queued);
-        queued = batch;
-        if (!bp.keepAlive) {
-          finish(queued);
-          queued = nullptr;
-        }
-      }
-      if (queued)
-        finish(queued);
+      while (SpatiallySparseBatch *batch = bp.nextBatch())
+        if (SpatiallySparseBatch *due = queue.push(batch))
+          finish(due);
+      while (SpatiallySparseBatch *batch = queue.pop())
+        finish(batch);
     }
     int errors = (int)nPictures;
     float nll = 0;

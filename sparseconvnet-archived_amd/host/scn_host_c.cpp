@@ -548,42 +548,12 @@ int scnh_forward_resident_stream(scnh_net *net, int nBatches, int batch,
                                  const int32_t *d_background, int64_t nActive,
                                  int nSpatialSites, const float *d_features,
                                  float *h_probs) {
-  SparseConvNetCUDA *cnn = net->cnn;
-  ResidentBatch r = resident_of(batch, d_sample, d_key, d_row, d_background,
-                                nActive, nSpatialSites, d_features);
-  BatchProducer bp(*cnn, r, nBatches);
-  bp.keepAlive = cnn->nBatchProducerThreads >= 2 ? 1 : 0;
-  int done = 0;
-  SpatiallySparseBatch *queued = nullptr; // forward pass queued, not yet read
-  auto finish = [&](SpatiallySparseBatch *b) {
-    if (net->hasClassifier) {
-      std::ofstream f, g;
-      cnn->finishBatch(*b, f, g);
-      net->batch = b;
-      if (h_probs)
-        scnh_batch_probabilities(net, h_probs);
-    }
-    ++done;
-  };
-  while (SpatiallySparseBatch *b = bp.nextBatch()) {
-    if (net->hasClassifier)
-      cnn->forwardBatch(*b);
-    else
-      forward_layers(net, *b);
-    if (queued)
-      finish(queued);
-    queued = b;
-    if (!bp.keepAlive) {
-      finish(queued);
-      queued = nullptr;
-    }
-  }
-  if (queued)
-    finish(queued);
-  cnn->memStream.synchronize();
-  net->batch = nullptr;
-  return done;
+  double seconds = 0;
+  return scnh_forward_stream_timed(net, 0, nBatches, batch, d_sample, d_key,
+                                   d_row, d_background, nActive, nSpatialSites,
+                                   d_features, 0, h_probs, &seconds);
 }
+
 // nWarmup + nTimed batches through one BatchProducer, as one dataset pass runs
 // them; *seconds is the wall time of the last nTimed, taken between two points
 // at which the net's stream is idle and every earlier batch is finished.  The
@@ -600,9 +570,8 @@ int scnh_forward_stream_timed(scnh_net *net, int nWarmup, int nTimed, int batch,
                                 nSpatialSites, features);
   r.onHost = inputsOnHost != 0;
   BatchProducer bp(*cnn, r, nWarmup + nTimed);
-  bp.keepAlive = cnn->nBatchProducerThreads >= 2 ? 1 : 0;
+  ForwardQueue queue(*cnn, bp, !net->hasClassifier); // (a headless net: layer by layer on lane 0)
   int done = 0, started = 0;
-  SpatiallySparseBatch *queued = nullptr;
   auto finish = [&](SpatiallySparseBatch *b) {
     if (net->hasClassifier) {
       std::ofstream f, g;
@@ -614,30 +583,37 @@ int scnh_forward_stream_timed(scnh_net *net, int nWarmup, int nTimed, int batch,
     ++done;
   };
   auto t0 = std::chrono::steady_clock::now();
+  SpatiallySparseBatch *headless = nullptr;
   while (SpatiallySparseBatch *b = bp.nextBatch()) {
     if (started == nWarmup) { // every warm-up batch done before the clock starts
-      if (queued)
-        finish(queued);
-      queued = nullptr;
-      cnn->memStream.synchronize();
+      while (SpatiallySparseBatch *q = queue.pop())
+        finish(q);
+      if (headless)
+        finish(headless);
+      headless = nullptr;
+      cnn->synchronizeLanes();
       t0 = std::chrono::steady_clock::now();
     }
     ++started;
-    if (net->hasClassifier)
-      cnn->forwardBatch(*b);
-    else
+    if (net->hasClassifier) {
+      if (SpatiallySparseBatch *due = queue.push(b))
+        finish(due);
+    } else {
       forward_layers(net, *b);
-    if (queued)
-      finish(queued);
-    queued = b;
-    if (!bp.keepAlive) {
-      finish(queued);
-      queued = nullptr;
+      if (headless)
+        finish(headless);
+      headless = b;
+      if (!bp.keepAlive) {
+        finish(headless);
+        headless = nullptr;
+      }
     }
   }
-  if (queued)
-    finish(queued);
-  cnn->memStream.synchronize();
+  while (SpatiallySparseBatch *q = queue.pop())
+    finish(q);
+  if (headless)
+    finish(headless);
+  cnn->synchronizeLanes();
   if (seconds)
     *seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
   net->batch = nullptr;

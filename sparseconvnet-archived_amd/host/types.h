@@ -22,3 +22,5 @@ extern const char *sigmoidNames[];
 // multiply-accumulate operations of the NiN contractions since the last reset
 // (types.h:46-52); processDataset prints it.
 extern __int128_t multiplyAddCount;
+// (forward passes may be queued from more than one host thread)
+void addMultiplyAdds(__int128_t n);
