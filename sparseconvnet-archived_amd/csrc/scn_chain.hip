@@ -203,139 +203,6 @@ template <int D> __device__ __forceinline__ unsigned site_key(const int *c, int 
     k = k * (unsigned)n + (unsigned)c[q];
   return k;
 }
-// x / d for x d < 2^32, magic = floor(2^32 / d) + 1 (d >= 2)
-__device__ __forceinline__ unsigned div_magic(unsigned x, unsigned d, unsigned magic) {
-  return d == 1 ? x : __umulhi(x, magic);
-}
-
-
-// `len` (<= 32) mask bits of the row with leading coordinates lead[0 .. D-2],
-// columns c0 .. c0 + len - 1; sites outside the field read as inactive.  Both
-// words are always fetched (the mask has a spare word), so that a lane's reads
-// do not wait for one another.
-template <int D>
-__device__ __forceinline__ unsigned row_bits(const unsigned long long *bits,
-                                             const int *lead, int c0, int len,
-                                             int n) {
-  bool inside = true;
-  unsigned p = 0;
-#pragma unroll
-  for (int q = 0; q < D - 1; ++q) {
-    inside = inside && (unsigned)lead[q] < (unsigned)n;
-    p = p * (unsigned)n + (unsigned)lead[q];
-  }
-  const int lo = c0 > 0 ? c0 : 0;
-  const int hi = c0 + len < n ? c0 + len : n;
-  p = p * (unsigned)n + (unsigned)lo;
-  if (!inside || hi <= lo)
-    p = 0; // any valid address; the result is masked away
-  const unsigned w = p >> 6, sh = p & 63;
-  const unsigned long long a = bits[w], b = bits[w + 1];
-  unsigned long long v = a >> sh;
-  if (sh)
-    v |= b << (64 - sh);
-  const int m = hi - lo;
-  unsigned r = (unsigned)v & (m >= 32 ? 0xFFFFFFFFu : ((1u << (m > 0 ? m : 0)) - 1u));
-  r = (!inside || hi <= lo) ? 0u : r;
-  return r << (lo - c0 > 0 ? lo - c0 : 0);
-}
-
-// Square regions without a minimum (Regions.cu:528-653), window side S: which
-// of the outputs whose window holds input site i is first touched by i, i.e.
-// has no active site before i in its window (row-major).  All mask reads of a
-// site are issued together -- the S rows (2-D) or S (2S - 1) rows (3-D) of its
-// neighbourhood -- and every candidate is then decided in registers.  Bit c of
-// the result stands for candidate c of the box [lo, hi) in ascending key;
-// f(j) is called for the owned ones.
-template <int D, int S, typename F>
-__device__ __forceinline__ unsigned
-owned_nomin(const unsigned long long *bits, const int *i, const int *lo,
-            const int *hi, int nIn, int stride, unsigned magicStride, F f) {
-  static_assert(D == 2 || D == 3, "two or three dimensions");
-  constexpr int W = 2 * S - 1;
-  constexpr unsigned FULL = (1u << S) - 1u;
-  unsigned m = 0;
-  if (D == 2) {
-    unsigned nb[S];
-#pragma unroll
-    for (int r = 0; r < S; ++r) {
-      const int lead[1] = {i[0] - (S - 1) + r};
-      nb[r] = row_bits<2>(bits, lead, i[1] - (S - 1), W, nIn);
-    }
-#pragma unroll
-    for (int a0 = 0; a0 < S; ++a0) {
-      const int d0 = i[0] - a0;
-      const int j0 = (int)div_magic((unsigned)(d0 > 0 ? d0 : 0), (unsigned)stride, magicStride);
-      const bool ok0 = d0 >= 0 && j0 * stride == d0 && j0 >= lo[0] && j0 < hi[0];
-      unsigned above = 0;
-#pragma unroll
-      for (int r = S - 1 - a0; r < S - 1; ++r)
-        above |= nb[r];
-#pragma unroll
-      for (int a1 = 0; a1 < S; ++a1) {
-        const int d1 = i[1] - a1;
-        const int j1 = (int)div_magic((unsigned)(d1 > 0 ? d1 : 0), (unsigned)stride, magicStride);
-        const bool ok1 = d1 >= 0 && j1 * stride == d1 && j1 >= lo[1] && j1 < hi[1];
-        const unsigned before = (above & (FULL << (S - 1 - a1))) |
-                                (nb[S - 1] & (((1u << a1) - 1u) << (S - 1 - a1)));
-        if (ok0 && ok1 && before == 0) {
-          const int j[2] = {j0, j1};
-          m |= 1u << ((j0 - lo[0]) * (hi[1] - lo[1]) + (j1 - lo[1]));
-          f(j);
-        }
-      }
-    }
-  } else {
-    unsigned nb[S][W];
-#pragma unroll
-    for (int pl = 0; pl < S; ++pl)
-#pragma unroll
-      for (int r = 0; r < W; ++r) {
-        const int lead[2] = {i[0] - (S - 1) + pl, i[1] - (S - 1) + r};
-        nb[pl][r] = row_bits<3>(bits, lead, i[2] - (S - 1), W, nIn);
-      }
-#pragma unroll
-    for (int a0 = 0; a0 < S; ++a0) {
-      const int d0 = i[0] - a0;
-      const int j0 = (int)div_magic((unsigned)(d0 > 0 ? d0 : 0), (unsigned)stride, magicStride);
-      const bool ok0 = d0 >= 0 && j0 * stride == d0 && j0 >= lo[0] && j0 < hi[0];
-#pragma unroll
-      for (int a1 = 0; a1 < S; ++a1) {
-        const int d1 = i[1] - a1;
-        const int j1 = (int)div_magic((unsigned)(d1 > 0 ? d1 : 0), (unsigned)stride, magicStride);
-        const bool ok1 = d1 >= 0 && j1 * stride == d1 && j1 >= lo[1] && j1 < hi[1];
-        // whole planes before the site's, then whole rows of its plane
-        unsigned above = 0;
-#pragma unroll
-        for (int pl = S - 1 - a0; pl < S - 1; ++pl)
-#pragma unroll
-          for (int q1 = 0; q1 < S; ++q1)
-            above |= nb[pl][S - 1 - a1 + q1];
-#pragma unroll
-        for (int q1 = 0; q1 < a1; ++q1)
-          above |= nb[S - 1][S - 1 - a1 + q1];
-#pragma unroll
-        for (int a2 = 0; a2 < S; ++a2) {
-          const int d2 = i[2] - a2;
-          const int j2 = (int)div_magic((unsigned)(d2 > 0 ? d2 : 0), (unsigned)stride, magicStride);
-          const bool ok2 = d2 >= 0 && j2 * stride == d2 && j2 >= lo[2] && j2 < hi[2];
-          const unsigned before =
-              (above & (FULL << (S - 1 - a2))) |
-              (nb[S - 1][S - 1] & (((1u << a2) - 1u) << (S - 1 - a2)));
-          if (ok0 && ok1 && ok2 && before == 0) {
-            const int j[3] = {j0, j1, j2};
-            m |= 1u << (((j0 - lo[0]) * (hi[1] - lo[1]) + (j1 - lo[1])) *
-                            (hi[2] - lo[2]) +
-                        (j2 - lo[2]));
-            f(j);
-          }
-        }
-      }
-    }
-  }
-  return m;
-}
-
 // The sample could not be carried (LDS or staging too small): every plan of
 // the chain is reported as outgrown, and the caller plans the batch again
 // layer by layer.
@@ -508,9 +375,9 @@ __global__ void __launch_bounds__(CHAIN_THREADS) k_chain_sample(ChainArgs a) {
       } else if (fast) {
         if constexpr (D >= 2) {
           if (L.size == 2)
-            m = owned_nomin<D, 2>(bitsA, i, lo, hi, L.nIn, L.stride, L.magicStride, mark);
+            m = owned_nomin<D, 2>(bitsA, 0u, i, lo, hi, L.nIn, L.stride, L.magicStride, mark);
           else
-            m = owned_nomin<D, 3>(bitsA, i, lo, hi, L.nIn, L.stride, L.magicStride, mark);
+            m = owned_nomin<D, 3>(bitsA, 0u, i, lo, hi, L.nIn, L.stride, L.magicStride, mark);
         }
       } else {
 #pragma unroll
@@ -920,6 +787,8 @@ static void chain_mark_output(scn_ctx *ctx, scn_grids *in, scn_grids *out,
   out->nActive = boundActive;
   out->nSites = (int)boundRows;
   out->rankValid = false;
+  out->rankRowValid = false;
+  out->tableValid = false;
   out->indexValid = false;
   out->chained = true;
   out->planIn = in;
@@ -1054,6 +923,7 @@ int scn_chain_flush(scn_ctx *ctx) {
   cs->nPlans += (long long)recs.size();
   ProfScope ps(ctx, SCN_K_RULES);
   scn_grids *src = recs[0].in;
+  SCN_TRY(scn_grids_ensure_table(ctx, src)); // the kernel reads the source's rows through it
   ChainArgs a;
   memset(&a, 0, sizeof(a));
   a.nLevels = (int)recs.size();

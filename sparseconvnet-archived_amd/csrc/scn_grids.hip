@@ -1,13 +1,19 @@
 // Sparse grids in HBM and rule-book construction.
 //
 // A batch of SparseGrids (SparseGrid.h:26-37) is kept as
-//   * an open-addressing hash table, linear probing, 16-byte slots
-//     {int64 packed coordinate, int32 row}, load factor <= 1/2;
-//     packed coordinate = sample * spatialSize^d + key;
-//   * an occupancy bit mask over the packed coordinates, with an exclusive
-//     popcount prefix per 64-bit word, so that the position of a site in map
-//     iteration order (sample, then ascending key) is prefix + popcount;
-//   * the list of entries (packed coordinate, row) in no particular order.
+//   * an occupancy bit mask over the packed coordinates (packed coordinate =
+//     sample * spatialSize^d + key), with an exclusive popcount prefix per
+//     64-bit word, so that the position of a site in map iteration order
+//     (sample, then ascending key) -- its rank -- is prefix + popcount;
+//   * the rows by rank: the row of the site at every position of iteration
+//     order.  "Which row has site p" is one mask word, one prefix word and one
+//     element of this array, and sites that are neighbours along the innermost
+//     axis are neighbours in it: a run of a rule row reads consecutive words;
+//   * the list of entries (packed coordinate, row) in no particular order;
+//   * on demand, an open-addressing hash table, linear probing, 16-byte slots
+//     {int64 packed coordinate, int32 row}, load factor <= 1/2, for look-ups by
+//     coordinate (scn_grids_find) and for the source of a chain of recorded
+//     plans.
 //
 // Rule books (Regions.cu gridRules*) number output sites in first-touch order
 // while the input map is iterated in ascending key.  An output site is first
@@ -46,7 +52,8 @@ __global__ void k_grid_build(GridView g, const int *sample,
   }
   long long p = (long long)b * g.vol + k;
   int r = row[e];
-  hash_insert(g.table, g.shift, g.mask, p, r);
+  if (g.table)
+    hash_insert(g.table, g.shift, g.mask, p, r);
   atomicOr(&g.bits[p >> 6], 1ull << (p & 63));
   ekey[e] = p;
   erow[e] = r;
@@ -71,15 +78,35 @@ __global__ void k_plan_count(GridView in, Geom g, const long long *ekey,
     return;
   }
   long long p = ekey[e];
-  int b = (int)(p / g.volIn);
   int i[D];
-  decode_key<D>(p - (long long)b * g.volIn, g.nIn, i);
+  const int b = split_site<D>(p, g.volIn, g.nIn, i);
   unsigned n = 0;
   unsigned long long mask = 0;
-  for_each_owned<D>(in, g, b, i, [&](long long, int c) {
-    ++n;
-    mask |= 1ull << (c & 63);
-  });
+  bool done = false;
+  if constexpr (D >= 2) {
+    // square windows of side 2 or 3 without a minimum: every mask word of the
+    // site's neighbourhood is requested at once and the candidates are decided
+    // in registers
+    if (g.mode == MODE_SQ_NOMIN && (g.size == 2 || g.size == 3)) {
+      int lo[D], hi[D];
+      if (cand_box<D>(g, b, i, lo, hi)) {
+        const long long sampleBase = (long long)b * g.volIn;
+        auto none = [](const int *) {};
+        mask = g.size == 2
+                   ? owned_nomin<D, 2>(in.bits, sampleBase, i, lo, hi, g.nIn,
+                                       g.stride, g.magicStride, none)
+                   : owned_nomin<D, 3>(in.bits, sampleBase, i, lo, hi, g.nIn,
+                                       g.stride, g.magicStride, none);
+        n = (unsigned)__popcll(mask);
+      }
+      done = true;
+    }
+  }
+  if (!done)
+    for_each_owned<D>(in, g, b, i, [&](long long, int c) {
+      ++n;
+      mask |= 1ull << (c & 63);
+    });
   unsigned r = rank_of(in, p);
   cntByRank[r] = n;
   if (ownMask) { // only when a box never has more than 64 candidates
@@ -234,19 +261,19 @@ __global__ void k_plan_emit(GridView in, GridView out, Geom g,
   if (e >= count_now(nEntries))
     return;
   long long p = ekey[e];
-  int b = (int)(p / g.volIn);
   int i[D];
-  decode_key<D>(p - (long long)b * g.volIn, g.nIn, i);
+  const int b = split_site<D>(p, g.volIn, g.nIn, i);
   unsigned idx = base[rank_of(in, p)];
   const int shiftRows = bgBefore[b];
   for_each_owned<D>(in, g, b, i, [&](long long outKey, int) {
     long long po = (long long)b * g.volOut + outKey;
     int row = (int)idx + shiftRows;
-    hash_insert(out.table, out.shift, out.mask, po, row);
+    int j[D];
+    decode_key<D>(outKey, g.nOut, j);
     atomicOr(&out.bits[po >> 6], 1ull << (po & 63));
     okey[idx] = po;
     orow[idx] = row;
-    siteKey[row] = po;
+    siteKey[row] = pack_row_site<D>(b, j);
     ++idx;
   });
 }
@@ -281,9 +308,8 @@ __global__ void k_plan_emit_masked(GridView in, GridView out, Geom g,
   const unsigned r = rankOf[e];
   if (!((mask >> c) & 1ull))
     return;
-  int b = (int)(p / g.volIn);
   int i[D], lo[D], hi[D], j[D];
-  decode_key<D>(p - (long long)b * g.volIn, g.nIn, i);
+  const int b = split_site<D>(p, g.volIn, g.nIn, i);
   (void)cand_box<D>(g, b, i, lo, hi);
   int rem = c;
 #pragma unroll
@@ -295,11 +321,10 @@ __global__ void k_plan_emit_masked(GridView in, GridView out, Geom g,
   unsigned idx = base[r] + (unsigned)__popcll(mask & ((1ull << c) - 1ull));
   long long po = (long long)b * g.volOut + encode_key<D>(j, g.nOut);
   int row = (int)idx + bgBefore[b];
-  hash_insert(out.table, out.shift, out.mask, po, row);
   atomicOr(&out.bits[po >> 6], 1ull << (po & 63));
   okey[idx] = po;
   orow[idx] = row;
-  siteKey[row] = po;
+  siteKey[row] = pack_row_site<D>(b, j);
 }
 
 // The same with one lane per input walking the set bits of its ownership
@@ -328,28 +353,34 @@ __global__ void k_plan_emit_walk(GridView in, GridView out, Geom g,
   const unsigned r = rankOf[e];
   if (mask == 0)
     return;
-  const int b = (int)(p / g.volIn);
   int i[D], lo[D], hi[D], j[D];
-  decode_key<D>(p - (long long)b * g.volIn, g.nIn, i);
+  const int b = split_site<D>(p, g.volIn, g.nIn, i);
   (void)cand_box<D>(g, b, i, lo, hi);
+  // a box is at most 64 candidates, so its sides are small: x / ext by a
+  // multiplication (exact for x < 64: the error of the factor stays below 1 / 64 ext)
+  unsigned ext[D], inv[D];
+#pragma unroll
+  for (int a = 0; a < D; ++a) {
+    ext[a] = (unsigned)(hi[a] - lo[a]);
+    inv[a] = 65536u / ext[a] + 1u;
+  }
   unsigned idx = base[r];
   const int shiftRows = bgBefore[b];
   while (mask) { // ascending candidate = ascending output key
-    int rem = __ffsll((long long)mask) - 1;
+    unsigned rem = (unsigned)(__ffsll((long long)mask) - 1);
     mask &= mask - 1;
 #pragma unroll
     for (int a = D - 1; a >= 0; --a) {
-      int ext = hi[a] - lo[a];
-      j[a] = lo[a] + rem % ext;
-      rem /= ext;
+      const unsigned up = (rem * inv[a]) >> 16;
+      j[a] = lo[a] + (int)(rem - up * ext[a]);
+      rem = up;
     }
     const long long po = (long long)b * g.volOut + encode_key<D>(j, g.nOut);
     const int row = (int)idx + shiftRows;
-    hash_insert(out.table, out.shift, out.mask, po, row);
     atomicOr(&out.bits[po >> 6], 1ull << (po & 63));
     okey[idx] = po;
     orow[idx] = row;
-    siteKey[row] = po;
+    siteKey[row] = pack_row_site<D>(b, j);
     ++idx;
   }
 }
@@ -394,6 +425,11 @@ struct RankScan {
   size_t n;
 };
 
+// row of the active site at packed position p
+__device__ __forceinline__ int row_at(const GridView &g, long long p) {
+  return g.rankRow[rank_of(g, p)];
+}
+
 // one thread per rule: rules[row * width + q]
 template <int D, bool SCAN>
 __global__ void __launch_bounds__(256)
@@ -422,9 +458,8 @@ __global__ void __launch_bounds__(256)
     rules[idx] = in.bg[-1 - sk];
     return;
   }
-  int b = (int)(sk / g.volOut);
   int j[D], c[D];
-  decode_key<D>(sk - (long long)b * g.volOut, g.nOut, j);
+  const int b = unpack_row_site<D>(sk, j);
   int cubeOff = invOrd ? invOrd[q] : q;
   if (g.mode == MODE_SQ_FMP) {
     // offsets past a region's extent keep the -1 the reference's rule rows
@@ -452,22 +487,33 @@ __global__ void __launch_bounds__(256)
   long long p = (long long)b * g.volIn + encode_key<D>(c, g.nIn);
   int val;
   if ((in.bits[p >> 6] >> (p & 63)) & 1ull)
-    val = hash_find(in.table, in.shift, in.mask, p);
+    val = row_at(in, p);
   else
     val = in.bg[b];
   rules[idx] = val;
 }
 
-// Square windows: one lane per run of `size` rule entries along the innermost
-// axis.  Their input sites are neighbours in the mask, so one mask read serves
-// the whole run (a lane per entry reads a 64-byte line of the mask for every
-// entry, and that line traffic is what bounds the kernel on 3-D batches).
-template <int D, bool SCAN>
+// Square windows.  A workgroup takes `rowsPerBlock` consecutive rule rows -- a
+// contiguous piece of the rule book -- one lane per row.  A lane decodes its
+// output site once and walks the runs of `size` entries along the innermost
+// axis: the input sites of a run are neighbours in the mask and in rank, so a
+// run costs one mask word (two when it straddles), one prefix word and
+// consecutive words of the rows by rank; and since consecutive rows are mostly
+// neighbouring sites, the lanes of a wavefront read the same few lines in
+// every step.  FILL_UNROLL runs are in flight per lane (all loads
+// unconditional, results selected afterwards).  The rows are collected in LDS
+// (odd pitch: no bank conflicts) and leave as whole 16-byte stores, lane after
+// lane.  S: the window's side when it is 2 or 3, else 0 (read from g).
+#define FILL_LDS_INTS 8192
+#define FILL_UNROLL 3
+template <int D, bool SCAN, int S>
 __global__ void __launch_bounds__(256)
     k_rules_fill_runs(GridView in, Geom g, const long long *siteKey,
                       Count nSites, const long long *outMeta, int *rules,
-                      RankScan rs) {
+                      RankScan rs, int rowsPerBlock, int pitch,
+                      unsigned magicWidth, unsigned magicSize) {
   __shared__ uint32_t ldsScan[SCAN1_LDS_WORDS];
+  __shared__ __attribute__((aligned(16))) int staged[FILL_LDS_INTS + 256];
   long long blk = blockIdx.x;
   if (SCAN) {
     if (blk == 0) {
@@ -476,37 +522,116 @@ __global__ void __launch_bounds__(256)
     }
     blk -= 1;
   }
-  long long idx = blk * blockDim.x + threadIdx.x;
   if (outMeta[META_OVERFLOW])
     return;
-  const int runsPerRow = g.width / g.size;
-  if (idx >= count_now(nSites) * runsPerRow)
+  const int t = threadIdx.x;
+  const long long row0 = blk * rowsPerBlock;
+  const long long left = count_now(nSites) - row0;
+  if (left <= 0)
     return;
-  const long long r = idx / runsPerRow;
-  int run = (int)(idx - r * runsPerRow);
-  int *dst = rules + r * g.width + (long long)run * g.size;
-  const long long sk = siteKey[r];
-  if (sk < 0) { // all-background row (Regions.cu:647-652)
-    const int v = in.bg[-1 - sk];
-    for (int t = 0; t < g.size; ++t)
-      dst[t] = v;
-    return;
-  }
-  const int b = (int)(sk / g.volOut);
-  int j[D], c[D];
-  decode_key<D>(sk - (long long)b * g.volOut, g.nOut, j);
-  c[D - 1] = j[D - 1] * g.stride;
+  const int nRows = left < rowsPerBlock ? (int)left : rowsPerBlock;
+  const int size = S ? S : g.size;
+  const int runsPerRow = g.width / size;
+  if (t < nRows) {
+    const long long sk = siteKey[row0 + t];
+    int *dst = staged + t * pitch;
+    if (sk < 0) { // all-background row (Regions.cu:647-652)
+      const int v = in.bg[-1 - sk];
+      for (int q = 0; q < g.width; ++q)
+        dst[q] = v;
+    } else {
+      int j[D];
+      const int b = unpack_row_site<D>(sk, j);
+      const int bgRow = in.bg[b];
+      // packed position of the window's origin
+      long long origin = 0;
 #pragma unroll
-  for (int a = D - 2; a >= 0; --a) {
-    c[a] = j[a] * g.stride + run % g.size;
-    run /= g.size;
+      for (int a = 0; a < D; ++a)
+        origin = origin * g.nIn + (long long)j[a] * g.stride;
+      origin += (long long)b * g.volIn;
+      const long long plane = D == 3 ? (long long)g.nIn * g.nIn : 0;
+      for (int k0 = 0; k0 < runsPerRow; k0 += FILL_UNROLL) {
+        unsigned long long w0[FILL_UNROLL], w1[FILL_UNROLL];
+        unsigned pre[FILL_UNROLL];
+        int sh[FILL_UNROLL];
+#pragma unroll
+        for (int u = 0; u < FILL_UNROLL; ++u) {
+          const int k = k0 + u < runsPerRow ? k0 + u : runsPerRow - 1;
+          long long p0 = origin;
+          if (D == 2) {
+            p0 += (long long)k * g.nIn;
+          } else if (D == 3) {
+            const int hiRun = (int)div_magic((unsigned)k, (unsigned)size, magicSize);
+            p0 += hiRun * plane + (long long)(k - hiRun * size) * g.nIn;
+          }
+          const long long w = p0 >> 6;
+          sh[u] = (int)(p0 & 63);
+          w0[u] = in.bits[w];
+          w1[u] = in.bits[w + 1];
+          pre[u] = in.prefix[w];
+        }
+        if (S) {
+          int val[FILL_UNROLL][S ? S : 1];
+          unsigned present[FILL_UNROLL];
+#pragma unroll
+          for (int u = 0; u < FILL_UNROLL; ++u) {
+            unsigned long long lo = w0[u] >> sh[u];
+            if (sh[u])
+              lo |= w1[u] << (64 - sh[u]);
+            present[u] = (unsigned)lo & ((1u << S) - 1u);
+            const unsigned rank0 =
+                pre[u] + (unsigned)__popcll(sh[u] ? (w0[u] & ((1ull << sh[u]) - 1ull)) : 0ull);
+#pragma unroll
+            for (int q = 0; q < S; ++q) {
+              const bool on = (present[u] >> q) & 1u;
+              val[u][q] = in.rankRow[on ? rank0 + __popc(present[u] & ((1u << q) - 1u)) : 0u];
+            }
+          }
+#pragma unroll
+          for (int u = 0; u < FILL_UNROLL; ++u)
+            if (k0 + u < runsPerRow) {
+#pragma unroll
+              for (int q = 0; q < S; ++q)
+                dst[(k0 + u) * S + q] = (present[u] >> q) & 1u ? val[u][q] : bgRow;
+            }
+        } else {
+#pragma unroll
+          for (int u = 0; u < FILL_UNROLL; ++u) {
+            if (k0 + u >= runsPerRow)
+              break;
+            unsigned long long lo = w0[u] >> sh[u];
+            if (sh[u])
+              lo |= w1[u] << (64 - sh[u]);
+            const unsigned present =
+                (unsigned)lo & (size >= 32 ? 0xFFFFFFFFu : ((1u << size) - 1u));
+            const unsigned rank0 =
+                pre[u] + (unsigned)__popcll(sh[u] ? (w0[u] & ((1ull << sh[u]) - 1ull)) : 0ull);
+            for (int q = 0; q < size; ++q)
+              dst[(k0 + u) * size + q] =
+                  (present >> q) & 1u
+                      ? in.rankRow[rank0 + __popc(present & ((1u << q) - 1u))]
+                      : bgRow;
+          }
+        }
+      }
+    }
   }
-  const long long p0 = (long long)b * g.volIn + encode_key<D>(c, g.nIn);
-  const unsigned present = get_bits(in.bits, p0, g.size);
-  const int bgRow = in.bg[b];
-  for (int t = 0; t < g.size; ++t)
-    dst[t] = (present >> t) & 1u ? hash_find(in.table, in.shift, in.mask, p0 + t)
-                                 : bgRow;
+  __syncthreads();
+  const unsigned total = (unsigned)nRows * (unsigned)g.width;
+  int *out = rules + row0 * g.width;
+  if (pitch == g.width && (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
+    const int4 *src = reinterpret_cast<const int4 *>(staged);
+    for (unsigned v = t; 4 * v + 4 <= total; v += 256)
+      reinterpret_cast<int4 *>(out)[v] = src[v];
+    const unsigned tail = total & ~3u;
+    if (t < (int)(total - tail))
+      out[tail + t] = staged[tail + t];
+  } else {
+    for (unsigned v = t; v < total; v += 256) {
+      const unsigned r = div_magic(v, (unsigned)g.width, magicWidth);
+      out[v] = staged[r * pitch + (v - r * g.width)];
+    }
+  }
 }
 
 // terminal pooling: sample sizes and their maximum.  One block.
@@ -561,7 +686,6 @@ __global__ void k_terminal_out(GridView out, long long *okey, int *orow,
   if (b >= out.batch)
     return;
   long long p = (long long)b * out.vol;
-  hash_insert(out.table, out.shift, out.mask, p, b);
   atomicOr(&out.bits[p >> 6], 1ull << (p & 63));
   okey[b] = p;
   orow[b] = b;
@@ -629,13 +753,18 @@ __global__ void k_find(GridView g, const int *sample, const long long *key,
 
 // ------------------------------------------------------------------ host
 
+// largest field (sites of one sample) whose source grids get a hash table as
+// they are built: about what a workgroup's LDS can hold as masks
+#define SCN_EAGER_TABLE_VOL (1ll << 20)
+
 GridView view_of(const scn_grids *g) {
   GridView v;
-  v.table = g->table.p;
+  v.table = g->tableValid ? g->table.p : nullptr;
   v.shift = 64 - g->log2cap;
   v.mask = (1u << g->log2cap) - 1u;
   v.bits = g->bits.p;
   v.prefix = g->prefix.p;
+  v.rankRow = g->rankRow.p;
   v.bg = g->bg.p;
   v.vol = g->vol;
   v.n = g->n;
@@ -652,9 +781,10 @@ static long long ipow_ll(long long b, int e) {
 }
 
 // (re)shape a grids object for `batch` samples of an n^d field holding up to
-// nActive sites; clears the table and the mask
+// nActive sites; clears the mask, and the hash table when the caller is about
+// to fill it (withTable)
 static int grids_prepare(scn_ctx *ctx, scn_grids *g, int batch, int d, int n,
-                         long long nActive) {
+                         long long nActive, bool withTable = false) {
   SCN_REQUIRE(batch >= 0 && d >= 1 && d <= 3 && n >= 1, SCN_ERR_ARG,
               "grids: batch %d dimension %d spatialSize %d (dimension must be 1..3)",
               batch, d, n);
@@ -663,12 +793,17 @@ static int grids_prepare(scn_ctx *ctx, scn_grids *g, int batch, int d, int n,
               SCN_ERR_CAPACITY,
               "grids: %d samples of %lld sites exceed the occupancy-mask limit",
               batch, vol);
+  // (the rows of a rule-book plan carry their sample above 40 bits of coordinates)
+  SCN_REQUIRE(batch < (1 << 22) && (d == 1 || n < (d == 3 ? (1 << 13) : (1 << 20))),
+              SCN_ERR_CAPACITY, "grids: %d samples of side %d", batch, n);
   g->batch = batch;
   g->d = d;
   g->n = n;
   g->vol = vol;
   g->nActive = nActive;
   g->rankValid = false;
+  g->rankRowValid = false;
+  g->tableValid = withTable;
   g->indexValid = true;
   g->chained = false;
   g->planKind = PLAN_NONE;
@@ -679,27 +814,33 @@ static int grids_prepare(scn_ctx *ctx, scn_grids *g, int batch, int d, int n,
     ++lg;
   SCN_REQUIRE(lg <= 31, SCN_ERR_CAPACITY, "grids: %lld active sites", nActive);
   g->log2cap = lg;
-  size_t cap = (size_t)1 << lg;
+  const size_t cap = (size_t)1 << lg;
   g->nWords = (size_t)(((long long)batch * vol + 63) / 64);
   const void *hadTable = g->table.p, *hadBits = g->bits.p;
-  SCN_TRY(g->table.reserve(cap));
+  if (withTable)
+    SCN_TRY(g->table.reserve(cap));
   SCN_TRY(g->bits.reserve(g->nWords + 8)); // the scan reads whole 32-byte groups
-  if (g->table.p != hadTable || g->bits.p != hadBits)
-    g->cleanSlots = g->cleanWords = 0; // fresh memory
+  if (g->table.p != hadTable)
+    g->cleanSlots = 0; // fresh memory
+  if (g->bits.p != hadBits)
+    g->cleanWords = 0;
   SCN_TRY(g->prefix.reserve(g->nWords + 2));
   SCN_TRY(g->ekey.reserve((size_t)nActive + 1));
   SCN_TRY(g->erow.reserve((size_t)nActive + 1));
   SCN_TRY(g->bg.reserve((size_t)batch + 1));
-  const bool clean = cap <= g->cleanSlots && g->nWords + 2 <= g->cleanWords;
-  g->cleanSlots = g->cleanWords = 0; // about to be written
-  if (!clean) {
-    size_t most = cap > g->nWords + 2 ? cap : g->nWords + 2;
+  const size_t clearSlots = withTable && cap > g->cleanSlots ? cap : 0;
+  const size_t clearWords = g->nWords + 2 > g->cleanWords ? g->nWords + 2 : 0;
+  if (withTable)
+    g->cleanSlots = 0; // about to be written
+  g->cleanWords = 0;
+  if (clearSlots || clearWords) {
+    size_t most = clearSlots > clearWords ? clearSlots : clearWords;
     size_t blocks = (most + 255) / 256;
     if (blocks > 16384)
       blocks = 16384;
     hipLaunchKernelGGL(k_clear_grid, dim3((unsigned)blocks), dim3(256), 0,
-                       ctx->stream, (uint4 *)g->table.p, cap, g->bits.p,
-                       g->nWords + 2);
+                       ctx->stream, (uint4 *)g->table.p, clearSlots, g->bits.p,
+                       clearWords);
     SCN_HIP_CHECK(hipGetLastError());
   }
   return SCN_OK;
@@ -750,6 +891,8 @@ extern "C" int scn_grids_clear_many(scn_ctx *ctx, scn_grids **grids, int n) {
       g->cleanSlots = l.nSlots[m];
       g->cleanWords = l.nWords[m];
       g->rankValid = false;
+      g->rankRowValid = false;
+      g->tableValid = false;
       ++m;
     }
     if (m == 0)
@@ -763,17 +906,33 @@ extern "C" int scn_grids_clear_many(scn_ctx *ctx, scn_grids **grids, int n) {
   return SCN_OK;
 }
 
-// table and mask of grids that only hold their entry list
+// mask of grids that only hold their entry list
 __global__ void k_grid_index(GridView g, const long long *ekey, const int *erow,
                              Count n, const long long *meta) {
   long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (e >= n.bound || (meta && meta[META_OVERFLOW]) || e >= count_now(n))
     return;
   const long long p = ekey[e];
-  hash_insert(g.table, g.shift, g.mask, p, erow[e]);
   atomicOr(&g.bits[p >> 6], 1ull << (p & 63));
 }
+// the rows by rank from the entry list
+__global__ void k_rank_rows(GridView g, const long long *ekey, const int *erow,
+                            Count n, const long long *meta, int *rankRow) {
+  long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= n.bound || (meta && meta[META_OVERFLOW]) || e >= count_now(n))
+    return;
+  rankRow[rank_of(g, ekey[e])] = erow[e];
+}
+// the hash table from the entry list
+__global__ void k_grid_table(GridView g, const long long *ekey, const int *erow,
+                             Count n, const long long *meta) {
+  long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= n.bound || (meta && meta[META_OVERFLOW]) || e >= count_now(n))
+    return;
+  hash_insert(g.table, g.shift, g.mask, ekey[e], erow[e]);
+}
 static Count count_active(const scn_grids *g);
+// the occupancy mask of grids that only hold their entry list
 static int ensure_index(scn_ctx *ctx, scn_grids *g) {
   if (g->indexValid)
     return SCN_OK;
@@ -799,16 +958,59 @@ static int ensure_index(scn_ctx *ctx, scn_grids *g) {
   return SCN_OK;
 }
 
+// mask, rank prefix and rows by rank: what a rule book needs of its input
 static int ensure_rank(scn_ctx *ctx, scn_grids *g) {
   SCN_TRY(ensure_index(ctx, g));
-  if (g->rankValid)
+  if (!g->rankValid) {
+    SCN_TRY(g->scanTmp.reserve(scn_scan_tmp_elems(g->nWords + 1)));
+    // one word past the mask so that the rank of the end position is defined
+    SCN_TRY(scn_scan_exclusive_popc64(ctx->stream,
+                                      (const uint64_t *)g->bits.p, g->prefix.p,
+                                      g->nWords + 1, g->scanTmp.p));
+    g->rankValid = true;
+  }
+  if (!g->rankRowValid) {
+    SCN_TRY(g->rankRow.reserve((size_t)g->nActive + 4));
+    if (g->nActive > 0) {
+      hipLaunchKernelGGL(k_rank_rows, dim3(scn_ceil_div(g->nActive, 256)),
+                         dim3(256), 0, ctx->stream, view_of(g), g->ekey.p,
+                         g->erow.p, count_active(g),
+                         g->pending ? g->meta.p : nullptr, g->rankRow.p);
+      SCN_HIP_CHECK(hipGetLastError());
+    }
+    g->rankRowValid = true;
+  }
+  return SCN_OK;
+}
+
+// the hash table, for look-ups by coordinate
+int scn_grids_ensure_table(scn_ctx *ctx, scn_grids *g) {
+  SCN_TRY(ensure_index(ctx, g));
+  if (g->tableValid)
     return SCN_OK;
-  SCN_TRY(g->scanTmp.reserve(scn_scan_tmp_elems(g->nWords + 1)));
-  // one word past the mask so that the rank of the end position is defined
-  SCN_TRY(scn_scan_exclusive_popc64(ctx->stream,
-                                    (const uint64_t *)g->bits.p, g->prefix.p,
-                                    g->nWords + 1, g->scanTmp.p));
-  g->rankValid = true;
+  const size_t cap = (size_t)1 << g->log2cap;
+  const void *had = g->table.p;
+  SCN_TRY(g->table.reserve(cap));
+  if (g->table.p != had)
+    g->cleanSlots = 0;
+  if (g->cleanSlots < cap) {
+    size_t blocks = (cap + 255) / 256;
+    if (blocks > 16384)
+      blocks = 16384;
+    hipLaunchKernelGGL(k_clear_grid, dim3((unsigned)blocks), dim3(256), 0,
+                       ctx->stream, (uint4 *)g->table.p, cap,
+                       (unsigned long long *)nullptr, (size_t)0);
+    SCN_HIP_CHECK(hipGetLastError());
+  }
+  g->cleanSlots = 0;
+  g->tableValid = true; // (view_of hands the table out from here on)
+  if (g->nActive > 0) {
+    hipLaunchKernelGGL(k_grid_table, dim3(scn_ceil_div(g->nActive, 256)),
+                       dim3(256), 0, ctx->stream, view_of(g), g->ekey.p,
+                       g->erow.p, count_active(g),
+                       g->pending ? g->meta.p : nullptr);
+    SCN_HIP_CHECK(hipGetLastError());
+  }
   return SCN_OK;
 }
 
@@ -948,6 +1150,7 @@ extern "C" int scn_grids_destroy(scn_ctx *ctx, scn_grids *g) {
   g->table.release();
   g->bits.release();
   g->prefix.release();
+  g->rankRow.release();
   g->ekey.release();
   g->erow.release();
   g->bg.release();
@@ -981,7 +1184,13 @@ extern "C" int scn_grids_build(scn_ctx *ctx, scn_grids *g, int batch,
               "scn_grids_build: null background array");
   SCN_TRY(scn_chain_flush(ctx));
   ProfScope ps(ctx, SCN_K_GRID_BUILD);
-  SCN_TRY(grids_prepare(ctx, g, batch, dimension, spatialSize, n));
+  // fields small enough for a chain of recorded plans get their table now
+  // (the chain reads its source through it); larger ones when somebody asks
+  long long vol = 1;
+  for (int a = 0; a < dimension && a < 3; ++a)
+    vol *= spatialSize > 0 ? spatialSize : 1;
+  SCN_TRY(grids_prepare(ctx, g, batch, dimension, spatialSize, n,
+                        vol <= SCN_EAGER_TABLE_VOL));
   g->nSites = nSpatialSites;
   // (backgroundCol is copied by the same launch: lane e < batch takes entry e)
   const long long lanes = n > batch ? n : batch;
@@ -1049,7 +1258,7 @@ extern "C" int scn_grids_find(scn_ctx *ctx, const scn_grids *g,
   SCN_REQUIRE(ctx && g, SCN_ERR_ARG, "scn_grids_find: null argument");
   if (n <= 0)
     return SCN_OK;
-  SCN_TRY(ensure_index(ctx, const_cast<scn_grids *>(g)));
+  SCN_TRY(scn_grids_ensure_table(ctx, const_cast<scn_grids *>(g)));
   hipLaunchKernelGGL(k_find, dim3(scn_ceil_div(n, 256)), dim3(256), 0,
                      ctx->stream, view_of(g), d_sample,
                      (const long long *)d_key, (long long)n, d_row);
@@ -1197,6 +1406,7 @@ static int plan_regions(scn_ctx *ctx, const scn_grids *cin, scn_grids *out,
   g.volIn = in->vol;
   g.volOut = ipow_ll(nOut, in->d);
   g.cube = (int)ipow_ll(size, in->d);
+  g.magicStride = (unsigned)((1ull << 32) / (unsigned)stride + 1);
   g.ticks = nullptr;
   g.tInR = g.tOutL = g.tOutR = 0;
   SCN_REQUIRE(ipow_ll(size, in->d) <= 32768, SCN_ERR_ARG,
@@ -1346,6 +1556,7 @@ extern "C" int scn_rules_fmp_plan(scn_ctx *ctx, const scn_grids *cin,
   g.volIn = in->vol;
   g.volOut = ipow_ll(nOut, d);
   g.cube = (int)ipow_ll(poolSize, d);
+  g.magicStride = 0; // (stride 1: div_magic leaves x as it is)
   g.width = g.cube;
   g.tInR = (long long)nT;
   g.tOutL = (long long)(2 * nT);
@@ -1452,8 +1663,8 @@ extern "C" int scn_rules_fill(scn_ctx *ctx, const scn_grids *in,
   SCN_REQUIRE(!out->chained, SCN_ERR_STATE,
               "scn_rules_fill: the rules of a recorded plan are written when "
               "the chain runs; plan again to fill another buffer");
-  SCN_TRY(ensure_index(ctx, const_cast<scn_grids *>(in)));
   ProfScope ps(ctx, SCN_K_RULES);
+  SCN_TRY(ensure_rank(ctx, const_cast<scn_grids *>(in)));
   GridView vin = view_of(in);
   if (out->planKind == PLAN_TERMINAL) {
     long long total = (long long)in->batch * out->termS;
@@ -1514,10 +1725,42 @@ extern "C" int scn_rules_fill(scn_ctx *ctx, const scn_grids *in,
       hipLaunchKernelGGL((KERNEL<3, false>), __VA_ARGS__);                     \
     break;                                                                     \
   }
-  if (!tri && g.size >= 2 && g.mode != MODE_SQ_FMP) {
-    dim3 runs(scn_ceil_div(total / g.size, 256) + extra);
-    SCN_FILL_DIM(k_rules_fill_runs, runs, block, 0, ctx->stream, vin, g,
-                 out->siteKey.p, count_sites(out), out->meta.p, d_rules, rs)
+  // rule rows a workgroup of the run kernel collects in LDS
+  const int rowsPerBlock =
+      g.width > 0 && FILL_LDS_INTS / g.width < 256 ? FILL_LDS_INTS / g.width : 256;
+  if (!tri && g.size >= 2 && g.mode != MODE_SQ_FMP && rowsPerBlock >= 1) {
+    const int pitch = g.width | 1;
+    const unsigned magicWidth = (unsigned)((1ull << 32) / (unsigned)g.width + 1);
+    const unsigned magicSize = (unsigned)((1ull << 32) / (unsigned)g.size + 1);
+    dim3 runs(scn_ceil_div(out->nSites, rowsPerBlock) + extra);
+#define SCN_FILL_RUNS(D, SC)                                                   \
+  if (g.size == 2)                                                             \
+    hipLaunchKernelGGL((k_rules_fill_runs<D, SC, 2>), runs, block, 0,          \
+                       ctx->stream, vin, g, out->siteKey.p, count_sites(out),  \
+                       out->meta.p, d_rules, rs, rowsPerBlock, pitch,          \
+                       magicWidth, magicSize);                                 \
+  else if (g.size == 3)                                                        \
+    hipLaunchKernelGGL((k_rules_fill_runs<D, SC, 3>), runs, block, 0,          \
+                       ctx->stream, vin, g, out->siteKey.p, count_sites(out),  \
+                       out->meta.p, d_rules, rs, rowsPerBlock, pitch,          \
+                       magicWidth, magicSize);                                 \
+  else                                                                         \
+    hipLaunchKernelGGL((k_rules_fill_runs<D, SC, 0>), runs, block, 0,          \
+                       ctx->stream, vin, g, out->siteKey.p, count_sites(out),  \
+                       out->meta.p, d_rules, rs, rowsPerBlock, pitch,          \
+                       magicWidth, magicSize);
+    switch (g.d) {
+    case 1:
+      if (scan) { SCN_FILL_RUNS(1, true) } else { SCN_FILL_RUNS(1, false) }
+      break;
+    case 2:
+      if (scan) { SCN_FILL_RUNS(2, true) } else { SCN_FILL_RUNS(2, false) }
+      break;
+    default:
+      if (scan) { SCN_FILL_RUNS(3, true) } else { SCN_FILL_RUNS(3, false) }
+      break;
+    }
+#undef SCN_FILL_RUNS
   } else {
     SCN_FILL_DIM(k_rules_fill, grid, block, 0, ctx->stream, vin, g,
                  out->siteKey.p, count_sites(out), out->meta.p, inv, d_rules, rs)

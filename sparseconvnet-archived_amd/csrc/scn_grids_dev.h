@@ -21,6 +21,7 @@ struct Geom {
   long long volIn, volOut;
   int width; // rule-row width: size^d or triangleSize(size, d)
   int cube;  // size^d
+  unsigned magicStride; // floor(2^32 / stride) + 1 (div_magic)
   // MODE_SQ_FMP: per-sample, per-axis region tables (fractional max-pooling).
   // inputL at ticks[(b d + a) nOut + j], inputR the same at tInR; outputL and
   // outputR at tOutL / tOutR + (b d + a) nIn + i.  Null otherwise.
@@ -39,6 +40,7 @@ struct GridView {
   unsigned shift, mask;
   unsigned long long *bits;
   const unsigned *prefix;
+  const int *rankRow; // row of the site at each position of iteration order
   const int *bg;
   long long vol;
   int n, d, batch;
@@ -67,10 +69,17 @@ struct scn_grids {
   int nSites = 0;
   unsigned log2cap = 0;
   size_t nWords = 0;
+  // What is current beside the entry list: the occupancy mask (indexValid;
+  // false for grids a chain of recorded plans produced: those hold the entry
+  // list, backgroundCol and the counts, and the rest is built from them on
+  // demand), its rank prefix (rankValid), the rows by rank (rankRowValid) and
+  // the hash table (tableValid).  Rule books are built from mask, prefix and
+  // rows by rank; the table serves scn_grids_find and the source of a chain
+  // of recorded plans, and is filled by scn_grids_build only for fields small
+  // enough for such a chain.
   bool rankValid = false;
-  // table, mask and prefix describe the entries (false for grids a chain of
-  // recorded plans produced: those hold the entry list, backgroundCol and the
-  // counts, and the rest is built from them on demand)
+  bool rankRowValid = false;
+  bool tableValid = false;
   bool indexValid = true;
   bool chained = false; // plan and rules came from a chain of recorded plans
   long long seenSample = 0; // most active sites one sample has had (chained plans)
@@ -87,6 +96,7 @@ struct scn_grids {
   DevBuf<Slot> table;
   DevBuf<unsigned long long> bits;
   DevBuf<unsigned> prefix;
+  DevBuf<int> rankRow;
   DevBuf<long long> ekey;
   DevBuf<int> erow;
   DevBuf<int> bg;
@@ -96,7 +106,7 @@ struct scn_grids {
   const scn_grids *planIn = nullptr;
   Geom geom;
   long long termS = 0;
-  DevBuf<long long> siteKey; // per output row: packed key, or -1 - sample for a background row
+  DevBuf<long long> siteKey; // per output row: sample and coordinates (pack_row_site), or -1 - sample for a background row
   DevBuf<unsigned> cnt, base;
   DevBuf<unsigned long long> ownMask;
   DevBuf<unsigned> rankOf;
@@ -367,10 +377,196 @@ __device__ __forceinline__ void for_each_owned(const GridView &in,
 }
 
 
+// x / d for x d < 2^32, magic = floor(2^32 / d) + 1 (d >= 2)
+__device__ __forceinline__ unsigned div_magic(unsigned x, unsigned d, unsigned magic) {
+  return d == 1 ? x : __umulhi(x, magic);
+}
+
+
+// `len` (<= 32) mask bits of the row with leading coordinates lead[0 .. D-2],
+// columns c0 .. c0 + len - 1; sites outside the field read as inactive.  Both
+// words are always fetched (the mask has a spare word), so that a lane's reads
+// do not wait for one another.  The field starts at bit `base` of the mask
+// (Pos: unsigned for a sample's mask in LDS, long long for a batch's in HBM).
+template <int D, typename Pos>
+__device__ __forceinline__ unsigned row_bits(const unsigned long long *bits,
+                                             Pos base, const int *lead, int c0,
+                                             int len, int n) {
+  bool inside = true;
+  Pos p = 0;
+#pragma unroll
+  for (int q = 0; q < D - 1; ++q) {
+    inside = inside && (unsigned)lead[q] < (unsigned)n;
+    p = p * (Pos)n + (Pos)lead[q];
+  }
+  const int lo = c0 > 0 ? c0 : 0;
+  const int hi = c0 + len < n ? c0 + len : n;
+  p = p * (Pos)n + (Pos)lo;
+  if (!inside || hi <= lo)
+    p = 0; // any valid address; the result is masked away
+  p += base;
+  const Pos w = p >> 6;
+  const unsigned sh = (unsigned)(p & 63);
+  const unsigned long long a = bits[w], b = bits[w + 1];
+  unsigned long long v = a >> sh;
+  if (sh)
+    v |= b << (64 - sh);
+  const int m = hi - lo;
+  unsigned r = (unsigned)v & (m >= 32 ? 0xFFFFFFFFu : ((1u << (m > 0 ? m : 0)) - 1u));
+  r = (!inside || hi <= lo) ? 0u : r;
+  return r << (lo - c0 > 0 ? lo - c0 : 0);
+}
+
+// Square regions without a minimum (Regions.cu:528-653), window side S: which
+// of the outputs whose window holds input site i is first touched by i, i.e.
+// has no active site before i in its window (row-major).  All mask reads of a
+// site are issued together -- the S rows (2-D) or S (2S - 1) rows (3-D) of its
+// neighbourhood -- and every candidate is then decided in registers.  Bit c of
+// the result stands for candidate c of the box [lo, hi) in ascending key;
+// f(j) is called for the owned ones.
+template <int D, int S, typename Pos, typename F>
+__device__ __forceinline__ unsigned
+owned_nomin(const unsigned long long *bits, Pos base, const int *i,
+            const int *lo, const int *hi, int nIn, int stride,
+            unsigned magicStride, F f) {
+  static_assert(D == 2 || D == 3, "two or three dimensions");
+  constexpr int W = 2 * S - 1;
+  constexpr unsigned FULL = (1u << S) - 1u;
+  unsigned m = 0;
+  if (D == 2) {
+    unsigned nb[S];
+#pragma unroll
+    for (int r = 0; r < S; ++r) {
+      const int lead[1] = {i[0] - (S - 1) + r};
+      nb[r] = row_bits<2>(bits, base, lead, i[1] - (S - 1), W, nIn);
+    }
+#pragma unroll
+    for (int a0 = 0; a0 < S; ++a0) {
+      const int d0 = i[0] - a0;
+      const int j0 = (int)div_magic((unsigned)(d0 > 0 ? d0 : 0), (unsigned)stride, magicStride);
+      const bool ok0 = d0 >= 0 && j0 * stride == d0 && j0 >= lo[0] && j0 < hi[0];
+      unsigned above = 0;
+#pragma unroll
+      for (int r = S - 1 - a0; r < S - 1; ++r)
+        above |= nb[r];
+#pragma unroll
+      for (int a1 = 0; a1 < S; ++a1) {
+        const int d1 = i[1] - a1;
+        const int j1 = (int)div_magic((unsigned)(d1 > 0 ? d1 : 0), (unsigned)stride, magicStride);
+        const bool ok1 = d1 >= 0 && j1 * stride == d1 && j1 >= lo[1] && j1 < hi[1];
+        const unsigned before = (above & (FULL << (S - 1 - a1))) |
+                                (nb[S - 1] & (((1u << a1) - 1u) << (S - 1 - a1)));
+        if (ok0 && ok1 && before == 0) {
+          const int j[2] = {j0, j1};
+          m |= 1u << ((j0 - lo[0]) * (hi[1] - lo[1]) + (j1 - lo[1]));
+          f(j);
+        }
+      }
+    }
+  } else {
+    unsigned nb[S][W];
+#pragma unroll
+    for (int pl = 0; pl < S; ++pl)
+#pragma unroll
+      for (int r = 0; r < W; ++r) {
+        const int lead[2] = {i[0] - (S - 1) + pl, i[1] - (S - 1) + r};
+        nb[pl][r] = row_bits<3>(bits, base, lead, i[2] - (S - 1), W, nIn);
+      }
+#pragma unroll
+    for (int a0 = 0; a0 < S; ++a0) {
+      const int d0 = i[0] - a0;
+      const int j0 = (int)div_magic((unsigned)(d0 > 0 ? d0 : 0), (unsigned)stride, magicStride);
+      const bool ok0 = d0 >= 0 && j0 * stride == d0 && j0 >= lo[0] && j0 < hi[0];
+#pragma unroll
+      for (int a1 = 0; a1 < S; ++a1) {
+        const int d1 = i[1] - a1;
+        const int j1 = (int)div_magic((unsigned)(d1 > 0 ? d1 : 0), (unsigned)stride, magicStride);
+        const bool ok1 = d1 >= 0 && j1 * stride == d1 && j1 >= lo[1] && j1 < hi[1];
+        // whole planes before the site's, then whole rows of its plane
+        unsigned above = 0;
+#pragma unroll
+        for (int pl = S - 1 - a0; pl < S - 1; ++pl)
+#pragma unroll
+          for (int q1 = 0; q1 < S; ++q1)
+            above |= nb[pl][S - 1 - a1 + q1];
+#pragma unroll
+        for (int q1 = 0; q1 < a1; ++q1)
+          above |= nb[S - 1][S - 1 - a1 + q1];
+#pragma unroll
+        for (int a2 = 0; a2 < S; ++a2) {
+          const int d2 = i[2] - a2;
+          const int j2 = (int)div_magic((unsigned)(d2 > 0 ? d2 : 0), (unsigned)stride, magicStride);
+          const bool ok2 = d2 >= 0 && j2 * stride == d2 && j2 >= lo[2] && j2 < hi[2];
+          const unsigned before =
+              (above & (FULL << (S - 1 - a2))) |
+              (nb[S - 1][S - 1] & (((1u << a2) - 1u) << (S - 1 - a2)));
+          if (ok0 && ok1 && ok2 && before == 0) {
+            const int j[3] = {j0, j1, j2};
+            m |= 1u << (((j0 - lo[0]) * (hi[1] - lo[1]) + (j1 - lo[1])) *
+                            (hi[2] - lo[2]) +
+                        (j2 - lo[2]));
+            f(j);
+          }
+        }
+      }
+    }
+  }
+  return m;
+}
+
+
+// What a rule-book plan keeps per output row: sample and coordinates in fixed
+// bit fields, so that the lanes that fill the rule rows shift instead of
+// dividing.  40 bits of coordinates (40, 20 or 13 an axis), the sample above.
+template <int D> struct RowSite {
+  static constexpr int AX = D == 1 ? 40 : (D == 2 ? 20 : 13);
+};
+template <int D>
+__device__ __forceinline__ long long pack_row_site(int b, const int *j) {
+  unsigned long long v = (unsigned long long)b;
+#pragma unroll
+  for (int a = 0; a < D; ++a)
+    v = (v << RowSite<D>::AX) | (unsigned long long)(unsigned)j[a];
+  return (long long)v;
+}
+template <int D>
+__device__ __forceinline__ int unpack_row_site(long long sk, int *j) {
+  unsigned long long v = (unsigned long long)sk;
+#pragma unroll
+  for (int a = D - 1; a >= 0; --a) {
+    j[a] = (int)(v & ((1ull << RowSite<D>::AX) - 1ull));
+    v >>= RowSite<D>::AX;
+  }
+  return (int)v;
+}
+
+// sample and coordinates of the packed position p = sample * vol + key; the
+// key is taken apart in 32-bit arithmetic when the field allows it
+template <int D>
+__device__ __forceinline__ int split_site(long long p, long long vol, int n,
+                                          int *c) {
+  const int b = (int)(p / vol);
+  const long long key = p - (long long)b * vol;
+  if (vol < (1ll << 31)) {
+    unsigned k = (unsigned)key;
+#pragma unroll
+    for (int a = D - 1; a >= 0; --a) {
+      const unsigned up = k / (unsigned)n;
+      c[a] = (int)(k - up * (unsigned)n);
+      k = up;
+    }
+  } else {
+    decode_key<D>(key, n, c);
+  }
+  return b;
+}
+
 // ---- host helpers shared by scn_grids.hip and scn_chain.hip
 GridView view_of(const scn_grids *g);
 long long grow_bound(long long seen, long long slack, long long cap);
 void mark_pending(scn_ctx *ctx, scn_grids *g, int slot);
+// fills the hash table of grids that do not have it yet (scn_grids.hip)
+int scn_grids_ensure_table(scn_ctx *ctx, scn_grids *g);
 
 // Chains of recorded plans (scn_chain.hip).  The record functions set *taken
 // when the call joined the chain being recorded; otherwise the caller runs it
