@@ -270,7 +270,8 @@ __global__ void k_plan_emit(GridView in, GridView out, Geom g,
     int row = (int)idx + shiftRows;
     int j[D];
     decode_key<D>(outKey, g.nOut, j);
-    atomicOr(&out.bits[po >> 6], 1ull << (po & 63));
+    if (out.bits)
+      atomicOr(&out.bits[po >> 6], 1ull << (po & 63));
     okey[idx] = po;
     orow[idx] = row;
     siteKey[row] = pack_row_site<D>(b, j);
@@ -321,7 +322,8 @@ __global__ void k_plan_emit_masked(GridView in, GridView out, Geom g,
   unsigned idx = base[r] + (unsigned)__popcll(mask & ((1ull << c) - 1ull));
   long long po = (long long)b * g.volOut + encode_key<D>(j, g.nOut);
   int row = (int)idx + bgBefore[b];
-  atomicOr(&out.bits[po >> 6], 1ull << (po & 63));
+  if (out.bits)
+    atomicOr(&out.bits[po >> 6], 1ull << (po & 63));
   okey[idx] = po;
   orow[idx] = row;
   siteKey[row] = pack_row_site<D>(b, j);
@@ -377,12 +379,136 @@ __global__ void k_plan_emit_walk(GridView in, GridView out, Geom g,
     }
     const long long po = (long long)b * g.volOut + encode_key<D>(j, g.nOut);
     const int row = (int)idx + shiftRows;
-    atomicOr(&out.bits[po >> 6], 1ull << (po & 63));
+    if (out.bits)
+      atomicOr(&out.bits[po >> 6], 1ull << (po & 63));
     okey[idx] = po;
     orow[idx] = row;
     siteKey[row] = pack_row_site<D>(b, j);
     ++idx;
   }
+}
+
+// Square windows without a minimum: an output site is active when any site of
+// its window is, so the output mask is the input mask OR-ed over the window
+// and thinned by the stride -- whole words at a time, every word of the
+// output mask written once (no atomics, no clearing).  One lane per output
+// word; a word is cut into the pieces that lie in one row of the output field.
+struct Bits128 {
+  unsigned long long lo, hi;
+};
+__device__ __forceinline__ Bits128 get_bits128(const unsigned long long *bits,
+                                               long long p) {
+  const long long w = p >> 6;
+  const int sh = (int)(p & 63);
+  Words3 ww;
+  __builtin_memcpy(&ww, bits + w, sizeof(ww));
+  const unsigned long long a = ww.a, b = ww.b, c = ww.c;
+  Bits128 r;
+  r.lo = sh ? (a >> sh) | (b << (64 - sh)) : a;
+  r.hi = sh ? (b >> sh) | (c << (64 - sh)) : b;
+  return r;
+}
+// the even bits of x, packed
+__device__ __forceinline__ unsigned long long even_bits(unsigned long long x) {
+  x &= 0x5555555555555555ull;
+  x = (x | (x >> 1)) & 0x3333333333333333ull;
+  x = (x | (x >> 2)) & 0x0F0F0F0F0F0F0F0Full;
+  x = (x | (x >> 4)) & 0x00FF00FF00FF00FFull;
+  x = (x | (x >> 8)) & 0x0000FFFF0000FFFFull;
+  x = (x | (x >> 16)) & 0x00000000FFFFFFFFull;
+  return x;
+}
+template <int D>
+__global__ void __launch_bounds__(256)
+    k_mask_dilate(GridView in, Geom g, unsigned long long *outBits,
+                  long long nWords, long long totalBits) {
+  const long long w = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (w >= nWords)
+    return;
+  unsigned long long res = 0;
+  long long pos = 64 * w;
+  const long long end = pos + 64 < totalBits ? pos + 64 : totalBits;
+  // a piece reads (len - 1) stride + size input bits: at most 128
+  const int lenMax = g.stride == 1 ? 64 : (128 - g.size) / g.stride + 1;
+  int j[D];
+  int b = split_site<D>(pos, g.volOut, g.nOut, j);
+  while (pos < end) {
+    long long len = g.nOut - j[D - 1];
+    len = len < end - pos ? len : end - pos;
+    len = len < lenMax ? len : lenMax;
+    const int L = ((int)len - 1) * g.stride + g.size;
+    const long long sampleBase = (long long)b * g.volIn;
+    unsigned long long lo = 0, hi = 0;
+    if (D == 1) {
+      const Bits128 x = get_bits128(in.bits, sampleBase + (long long)j[0] * g.stride);
+      lo = x.lo;
+      hi = x.hi;
+    } else if (D == 2) {
+      for (int q0 = 0; q0 < g.size; ++q0) {
+        const Bits128 x = get_bits128(
+            in.bits, sampleBase + (long long)(j[0] * g.stride + q0) * g.nIn +
+                         (long long)j[1] * g.stride);
+        lo |= x.lo;
+        hi |= x.hi;
+      }
+    } else {
+      for (int q0 = 0; q0 < g.size; ++q0)
+        for (int q1 = 0; q1 < g.size; ++q1) {
+          const Bits128 x = get_bits128(
+              in.bits,
+              sampleBase +
+                  ((long long)(j[0] * g.stride + q0) * g.nIn +
+                   (j[D > 1 ? 1 : 0] * g.stride + q1)) * g.nIn +
+                  (long long)j[D - 1] * g.stride);
+          lo |= x.lo;
+          hi |= x.hi;
+        }
+    }
+    // only the L bits of this piece's windows
+    if (L < 64) {
+      lo &= (1ull << L) - 1ull;
+      hi = 0;
+    } else if (L < 128) {
+      hi &= L == 64 ? 0ull : (1ull << (L - 64)) - 1ull;
+    }
+    // bit t: any of the `size` sites from t on
+    unsigned long long ylo = lo, yhi = hi;
+    for (int q = 1; q < g.size; ++q) {
+      lo = (lo >> 1) | (hi << 63);
+      hi >>= 1;
+      ylo |= lo;
+      yhi |= hi;
+    }
+    unsigned long long r;
+    if (g.stride == 1) {
+      r = ylo;
+    } else if (g.stride == 2) {
+      r = even_bits(ylo) | (even_bits(yhi) << 32);
+    } else {
+      r = 0;
+      for (int t = 0; t < (int)len; ++t) {
+        const int at = t * g.stride;
+        const unsigned long long bit = at < 64 ? (ylo >> at) : (yhi >> (at - 64));
+        r |= (bit & 1ull) << t;
+      }
+    }
+    if (len < 64)
+      r &= (1ull << len) - 1ull;
+    res |= r << (pos - 64 * w);
+    pos += len;
+    // the next piece starts where this one ended: carry through the axes
+    j[D - 1] += (int)len;
+#pragma unroll
+    for (int a = D - 1; a >= 0; --a)
+      if (j[a] >= g.nOut) {
+        j[a] = 0;
+        if (a > 0)
+          ++j[a - 1];
+        else
+          ++b;
+      }
+  }
+  outBits[w] = res;
 }
 
 // clears a hash table (all-ones = empty slots) and an occupancy mask at once
@@ -500,12 +626,15 @@ __global__ void __launch_bounds__(256)
 // run costs one mask word (two when it straddles), one prefix word and
 // consecutive words of the rows by rank; and since consecutive rows are mostly
 // neighbouring sites, the lanes of a wavefront read the same few lines in
-// every step.  FILL_UNROLL runs are in flight per lane (all loads
-// unconditional, results selected afterwards).  The rows are collected in LDS
+// every step.  All runs of a row are in flight at once when the side is 2 or
+// 3, else three at a time (all loads unconditional, results selected
+// afterwards).  The rows are collected in LDS
 // (odd pitch: no bank conflicts) and leave as whole 16-byte stores, lane after
 // lane.  S: the window's side when it is 2 or 3, else 0 (read from g).
 #define FILL_LDS_INTS 8192
-#define FILL_UNROLL 3
+struct __attribute__((packed, aligned(4))) Rows4 {
+  int r[4];
+};
 template <int D, bool SCAN, int S>
 __global__ void __launch_bounds__(256)
     k_rules_fill_runs(GridView in, Geom g, const long long *siteKey,
@@ -524,6 +653,8 @@ __global__ void __launch_bounds__(256)
   }
   if (outMeta[META_OVERFLOW])
     return;
+  // runs in flight per lane: a whole row when the side is known
+  constexpr int U = S == 0 ? 3 : (D == 1 ? 1 : (D == 2 ? S : S * S));
   const int t = threadIdx.x;
   const long long row0 = blk * rowsPerBlock;
   const long long left = count_now(nSites) - row0;
@@ -550,12 +681,12 @@ __global__ void __launch_bounds__(256)
         origin = origin * g.nIn + (long long)j[a] * g.stride;
       origin += (long long)b * g.volIn;
       const long long plane = D == 3 ? (long long)g.nIn * g.nIn : 0;
-      for (int k0 = 0; k0 < runsPerRow; k0 += FILL_UNROLL) {
-        unsigned long long w0[FILL_UNROLL], w1[FILL_UNROLL];
-        unsigned pre[FILL_UNROLL];
-        int sh[FILL_UNROLL];
+      for (int k0 = 0; k0 < runsPerRow; k0 += U) {
+        unsigned long long w0[U], w1[U];
+        unsigned pre[U];
+        int sh[U];
 #pragma unroll
-        for (int u = 0; u < FILL_UNROLL; ++u) {
+        for (int u = 0; u < U; ++u) {
           const int k = k0 + u < runsPerRow ? k0 + u : runsPerRow - 1;
           long long p0 = origin;
           if (D == 2) {
@@ -566,37 +697,41 @@ __global__ void __launch_bounds__(256)
           }
           const long long w = p0 >> 6;
           sh[u] = (int)(p0 & 63);
-          w0[u] = in.bits[w];
-          w1[u] = in.bits[w + 1];
+          // both words in one request (the mask has spare words at its end)
+          Words2 ww;
+          __builtin_memcpy(&ww, in.bits + w, sizeof(ww));
+          w0[u] = ww.a;
+          w1[u] = ww.b;
           pre[u] = in.prefix[w];
         }
         if (S) {
-          int val[FILL_UNROLL][S ? S : 1];
-          unsigned present[FILL_UNROLL];
+          Rows4 val[U];
+          unsigned present[U];
 #pragma unroll
-          for (int u = 0; u < FILL_UNROLL; ++u) {
+          for (int u = 0; u < U; ++u) {
             unsigned long long lo = w0[u] >> sh[u];
             if (sh[u])
               lo |= w1[u] << (64 - sh[u]);
             present[u] = (unsigned)lo & ((1u << S) - 1u);
             const unsigned rank0 =
                 pre[u] + (unsigned)__popcll(sh[u] ? (w0[u] & ((1ull << sh[u]) - 1ull)) : 0ull);
-#pragma unroll
-            for (int q = 0; q < S; ++q) {
-              const bool on = (present[u] >> q) & 1u;
-              val[u][q] = in.rankRow[on ? rank0 + __popc(present[u] & ((1u << q) - 1u)) : 0u];
-            }
+            // the rows of the run's active sites are consecutive words: one
+            // request (the array has spare words at its end)
+            __builtin_memcpy(&val[u], in.rankRow + (present[u] ? rank0 : 0u), sizeof(Rows4));
           }
 #pragma unroll
-          for (int u = 0; u < FILL_UNROLL; ++u)
+          for (int u = 0; u < U; ++u)
             if (k0 + u < runsPerRow) {
 #pragma unroll
-              for (int q = 0; q < S; ++q)
-                dst[(k0 + u) * S + q] = (present[u] >> q) & 1u ? val[u][q] : bgRow;
+              for (int q = 0; q < S; ++q) {
+                const int at = __popc(present[u] & ((1u << q) - 1u));
+                const int v = at == 0 ? val[u].r[0] : (at == 1 ? val[u].r[1] : val[u].r[2]);
+                dst[(k0 + u) * S + q] = (present[u] >> q) & 1u ? v : bgRow;
+              }
             }
         } else {
 #pragma unroll
-          for (int u = 0; u < FILL_UNROLL; ++u) {
+          for (int u = 0; u < U; ++u) {
             if (k0 + u >= runsPerRow)
               break;
             unsigned long long lo = w0[u] >> sh[u];
@@ -1352,9 +1487,20 @@ static int plan_regions_d(scn_ctx *ctx, scn_grids *in, scn_grids *out,
     mark_pending(ctx, out, slot);
   SCN_TRY(out->siteKey.reserve((size_t)nSites + 1));
   long long nThreads = nE > in->batch ? nE : in->batch;
+  // the output mask: word by word from the input mask where the mode allows
+  // it, else bit by bit as the emit pass finds the sites
+  GridView vout = view_of(out);
+  if (g.mode == MODE_SQ_NOMIN && g.size <= 64) {
+    const long long words = (long long)out->nWords + 2;
+    hipLaunchKernelGGL(k_mask_dilate<D>, dim3(scn_ceil_div(words, 256)), dim3(256),
+                       0, ctx->stream, vin, g, out->bits.p, words,
+                       (long long)in->batch * g.volOut);
+    SCN_HIP_CHECK(hipGetLastError());
+    vout.bits = nullptr;
+  }
   if (nThreads > 0 && masked && maxCand > 9) {
     hipLaunchKernelGGL(k_plan_emit_walk<D>, dim3(scn_ceil_div(nThreads, 256)),
-                       dim3(256), 0, ctx->stream, vin, view_of(out), g,
+                       dim3(256), 0, ctx->stream, vin, vout, g,
                        in->ekey.p, nEc, out->meta.p, out->base.p, out->ownMask.p,
                        out->rankOf.p, out->bgBefore.p, out->bg.p, out->ekey.p,
                        out->erow.p, out->siteKey.p);
@@ -1362,14 +1508,14 @@ static int plan_regions_d(scn_ctx *ctx, scn_grids *in, scn_grids *out,
   } else if (nThreads > 0 && masked) {
     hipLaunchKernelGGL(k_plan_emit_masked<D>,
                        dim3(scn_ceil_div(nThreads, 256), (unsigned)maxCand),
-                       dim3(256), 0, ctx->stream, vin, view_of(out), g,
+                       dim3(256), 0, ctx->stream, vin, vout, g,
                        in->ekey.p, nEc, out->meta.p, out->base.p, out->ownMask.p,
                        out->rankOf.p, out->bgBefore.p, out->bg.p, out->ekey.p,
                        out->erow.p, out->siteKey.p);
     SCN_HIP_CHECK(hipGetLastError());
   } else if (nThreads > 0) {
     hipLaunchKernelGGL(k_plan_emit<D>, dim3(scn_ceil_div(nThreads, 256)),
-                       dim3(256), 0, ctx->stream, vin, view_of(out), g,
+                       dim3(256), 0, ctx->stream, vin, vout, g,
                        in->ekey.p, nEc, out->meta.p, out->base.p, out->bgBefore.p,
                        out->bg.p,
                        out->ekey.p, out->erow.p, out->siteKey.p);

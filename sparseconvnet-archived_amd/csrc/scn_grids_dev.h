@@ -156,6 +156,15 @@ __device__ __forceinline__ int hash_find(const Slot *t, unsigned shift,
   }
 }
 
+// two or three consecutive mask words fetched as one request (global memory
+// takes 16-byte loads at any 4-byte boundary)
+struct __attribute__((packed, aligned(8))) Words2 {
+  unsigned long long a, b;
+};
+struct __attribute__((packed, aligned(8))) Words3 {
+  unsigned long long a, b, c;
+};
+
 // `len` (1..32) mask bits starting at bit position p
 __device__ __forceinline__ unsigned get_bits(const unsigned long long *bits,
                                              long long p, int len) {
@@ -407,7 +416,16 @@ __device__ __forceinline__ unsigned row_bits(const unsigned long long *bits,
   p += base;
   const Pos w = p >> 6;
   const unsigned sh = (unsigned)(p & 63);
-  const unsigned long long a = bits[w], b = bits[w + 1];
+  unsigned long long a, b;
+  if constexpr (sizeof(Pos) == 8) { // global memory: one 16-byte request
+    Words2 ww;
+    __builtin_memcpy(&ww, bits + w, sizeof(ww));
+    a = ww.a;
+    b = ww.b;
+  } else {
+    a = bits[w];
+    b = bits[w + 1];
+  }
   unsigned long long v = a >> sh;
   if (sh)
     v |= b << (64 - sh);
