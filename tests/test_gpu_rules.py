@@ -61,6 +61,54 @@ def test_square_rules(scn, ctx, d, size, stride, nOut, minActive):
         run_both(scn, ctx, samples, d, nIn, nOut, size, stride, minActive, False, nSites)
 
 
+WIDE_GEOMS = [(1, 3, 1, 300), (1, 3, 2, 150), (1, 5, 3, 90), (2, 2, 1, 100), (2, 3, 2, 70), (2, 4, 3, 45), (3, 3, 1, 70),
+              (3, 2, 2, 40)]
+
+
+@pytest.mark.parametrize("d,size,stride,nOut", WIDE_GEOMS)
+def test_square_rules_rows_longer_than_a_mask_word(scn, ctx, d, size, stride, nOut):
+    """Fields whose rows span several 64-bit mask words and do not start on word boundaries (the output mask of these
+    rule books is derived from the input mask a word at a time)."""
+    rng = np.random.default_rng(1000 * d + 100 * size + 10 * stride + nOut)
+    nIn = size + (nOut - 1) * stride
+    for density in (0.002, 0.03, 0.6):
+        samples, nSites = brute.random_samples(rng, 3, d, nIn, density)
+        run_both(scn, ctx, samples, d, nIn, nOut, size, stride, 1, False, nSites)
+
+
+def test_find_on_grids_without_a_table(scn, ctx):
+    """Look-ups by coordinate on grids whose hash table is only built when asked for: input grids of a field too large
+    for one, and the output grids of a rule-book plan."""
+    rng = np.random.default_rng(21)
+    d, nIn = 3, 110  # 110^3 sites: beyond the fields that get a table as they are built
+    samples = []
+    row = 0
+    for b in range(2):
+        keys = rng.choice(nIn ** d, size=500, replace=False)
+        samples.append((-1, {int(k): row + i for i, k in enumerate(keys)}))
+        row += 500
+    samples = [(row + b, mp) for b, (_, mp) in enumerate(samples)]
+    g = device_grids(scn, ctx, samples, d, nIn, row + 2)
+    qs = [0] * 300 + [1] * 300
+    qk = [int(k) for k in list(samples[0][1])[:150]] + [int(k) for k in rng.integers(0, nIn ** d, 150)] + \
+         [int(k) for k in list(samples[1][1])[:150]] + [int(k) for k in rng.integers(0, nIn ** d, 150)]
+    want = [samples[b][1].get(k, -1) for b, k in zip(qs, qk)]
+    assert g.find(qs, qk).tolist() == want
+    # the outputs of a plan, before and after their rules are filled
+    o_out, o_rules, o_n = orc.rules_square(oracle_grids(samples), d, nIn, nIn - 2, 3, 1, 1)
+    out = scn.Grids(ctx)
+    n = g.plan_square(out, nIn, nIn - 2, 3, 1)
+    assert n == o_n
+    os_, ok, or_, _ = o_out.flat()
+    omap = {(int(a), int(b)): int(c) for a, b, c in zip(os_, ok, or_)}
+    pick = rng.choice(len(ok), size=200, replace=False)
+    assert out.find(os_[pick], ok[pick]).tolist() == or_[pick].tolist()
+    rules = ctx.empty(n * 27, np.int32)
+    g.fill(out, rules, n * 27)
+    assert np.array_equal(rules.download()[: n * 27], o_rules)
+    assert out.find([1] * 3, [0, 1, 2]).tolist() == [omap.get((1, k), -1) for k in (0, 1, 2)]
+
+
 def test_valid_rules(scn, ctx):
     rng = np.random.default_rng(8)
     for nOut in (1, 2, 4, 7, 20):
