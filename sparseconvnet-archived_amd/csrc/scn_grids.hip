@@ -755,9 +755,11 @@ __global__ void __launch_bounds__(256)
   const unsigned total = (unsigned)nRows * (unsigned)g.width;
   int *out = rules + row0 * g.width;
   if (pitch == g.width && (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
-    const int4 *src = reinterpret_cast<const int4 *>(staged);
+    typedef int v4i __attribute__((ext_vector_type(4)));
+    const v4i *src = reinterpret_cast<const v4i *>(staged);
+    // (written once, read by a later kernel: streamed past the caches)
     for (unsigned v = t; 4 * v + 4 <= total; v += 256)
-      reinterpret_cast<int4 *>(out)[v] = src[v];
+      __builtin_nontemporal_store(src[v], reinterpret_cast<v4i *>(out) + v);
     const unsigned tail = total & ~3u;
     if (t < (int)(total - tail))
       out[tail + t] = staged[tail + t];
