@@ -542,62 +542,77 @@ __global__ void __launch_bounds__(CHAIN_THREADS) k_chain_sample(ChainArgs a) {
 }
 
 // Sums over the samples of a layer's counts: what lies before sample b, the
-// totals, and the largest sample.
+// totals, and the largest sample; and the first row of sample b in the layer's
+// input (the same sums of the layer before).  Every lane adds up its samples,
+// the lane sums meet in LDS and are folded in two short steps (a shuffle tree
+// over six 64-bit values would cost this short kernel more than its copy).
+#define PLACE_THREADS 256
 struct PlaceSums {
-  long long actBefore, bgBefore, actAll, bgAll, maxAct;
+  long long actBefore, bgBefore, actAll, bgAll, maxAct, inBase;
 };
-__device__ __forceinline__ PlaceSums place_sums(const int *cnt, int batch, int b,
-                                                long long *red) {
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-  long long v[5] = {0, 0, 0, 0, 0};
-  for (int s = t; s < batch; s += CHAIN_THREADS) {
+__device__ __forceinline__ PlaceSums place_sums(const int *cnt, const int *cntIn,
+                                                int batch, int b,
+                                                long long (*part)[PLACE_THREADS],
+                                                long long (*fold)[8]) {
+  const int t = threadIdx.x;
+  long long v[6] = {0, 0, 0, 0, 0, 0};
+  for (int s = t; s < batch; s += PLACE_THREADS) {
     const int n = cnt[2 * s], h = cnt[2 * s + 1];
     if (s < b) {
       v[0] += n;
       v[1] += h;
+      if (cntIn)
+        v[5] += cntIn[2 * s] + cntIn[2 * s + 1];
     }
     v[2] += n;
     v[3] += h;
     v[4] = n > v[4] ? n : v[4];
   }
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-#pragma unroll
-    for (int k = 0; k < 4; ++k)
-      v[k] += __shfl_xor(v[k], off, 64);
-    const long long o = __shfl_xor(v[4], off, 64);
-    v[4] = o > v[4] ? o : v[4];
-  }
-  __syncthreads(); // (red may still be read from an earlier call)
-  if (lane == 0)
-#pragma unroll
-    for (int k = 0; k < 5; ++k)
-      red[wave * 5 + k] = v[k];
+  for (int k = 0; k < 6; ++k)
+    part[k][t] = v[k];
   __syncthreads();
-  PlaceSums r = {0, 0, 0, 0, 0};
-#pragma unroll
-  for (int w = 0; w < CHAIN_WAVES; ++w) {
-    r.actBefore += red[w * 5 + 0];
-    r.bgBefore += red[w * 5 + 1];
-    r.actAll += red[w * 5 + 2];
-    r.bgAll += red[w * 5 + 3];
-    r.maxAct = red[w * 5 + 4] > r.maxAct ? red[w * 5 + 4] : r.maxAct;
+  if (t < 48) { // eight lanes a value, 32 lane sums each
+    const int k = t >> 3, seg = t & 7;
+    long long x = 0;
+    for (int i = 0; i < PLACE_THREADS / 8; ++i) {
+      const long long y = part[k][seg * (PLACE_THREADS / 8) + i];
+      x = k == 4 ? (y > x ? y : x) : x + y;
+    }
+    fold[k][seg] = x;
   }
-  return r;
+  __syncthreads();
+  long long r[6];
+#pragma unroll
+  for (int k = 0; k < 6; ++k) {
+    long long x = 0;
+#pragma unroll
+    for (int seg = 0; seg < 8; ++seg) {
+      const long long y = fold[k][seg];
+      x = k == 4 ? (y > x ? y : x) : x + y;
+    }
+    r[k] = x;
+  }
+  PlaceSums out;
+  out.actBefore = r[0];
+  out.bgBefore = r[1];
+  out.actAll = r[2];
+  out.bgAll = r[3];
+  out.maxAct = r[4];
+  out.inBase = r[5];
+  return out;
 }
 
-__global__ void __launch_bounds__(CHAIN_THREADS) k_chain_place(ChainArgs a) {
-  __shared__ long long red[CHAIN_WAVES * 5];
+__global__ void __launch_bounds__(PLACE_THREADS) k_chain_place(ChainArgs a) {
+  __shared__ long long part[6][PLACE_THREADS];
+  __shared__ long long fold[6][8];
   const int b = blockIdx.x, l = blockIdx.y, t = threadIdx.x;
   const ChainLevel &L = a.lv[l];
   const int *cnt = a.counts + (long long)l * a.batch * 2;
   const bool gaveUp = *reinterpret_cast<volatile unsigned long long *>(a.flag) == a.ticket;
-  const PlaceSums me = place_sums(cnt, a.batch, b, red);
-  long long inBase = 0; // first row of this sample in the layer's input
-  if (l > 0) {
-    const PlaceSums in = place_sums(cnt - (long long)a.batch * 2, a.batch, b, red);
-    inBase = in.actBefore + in.bgBefore;
-  }
+  const PlaceSums me = place_sums(cnt, l > 0 ? cnt - (long long)a.batch * 2 : nullptr,
+                                  a.batch, b, part, fold);
+  const long long inBase = me.inBase; // first row of this sample in the layer's input
   const bool terminal = L.kind == CH_TERMINAL;
   long long nSites, nActive, width;
   bool over = gaveUp;
@@ -634,7 +649,7 @@ __global__ void __launch_bounds__(CHAIN_THREADS) k_chain_place(ChainArgs a) {
     if (L.rules) {
       const int have = n > 1 ? n : 1;
       int *dst = L.rules + (long long)b * width;
-      for (long long i = t; i < width; i += CHAIN_THREADS) {
+      for (long long i = t; i < width; i += PLACE_THREADS) {
         int v = -1;
         if (i < have) {
           v = st[i];
@@ -654,7 +669,21 @@ __global__ void __launch_bounds__(CHAIN_THREADS) k_chain_place(ChainArgs a) {
   if (L.rules) {
     const long long total = (long long)(n + hasBg) * L.width;
     int *dst = L.rules + rowBase * L.width;
-    for (long long i = t; i < total; i += CHAIN_THREADS) {
+    // eight loads in flight per lane (the staged rows were written by the
+    // kernel before this one: every load is a trip to the L2 at least)
+    constexpr int PU = 8;
+    const int total32 = (int)total; // capRows * width fits 31 bits
+    int i = t;
+    for (; i + (PU - 1) * PLACE_THREADS < total32; i += PU * PLACE_THREADS) {
+      int v[PU];
+#pragma unroll
+      for (int u = 0; u < PU; ++u)
+        v[u] = st[i + u * PLACE_THREADS];
+#pragma unroll
+      for (int u = 0; u < PU; ++u)
+        dst[i + u * PLACE_THREADS] = v[u] < 0 ? v[u] : v[u] + (int)inBase;
+    }
+    for (; i < total32; i += PLACE_THREADS) {
       const int v = st[i];
       dst[i] = v < 0 ? v : v + (int)inBase;
     }
@@ -663,7 +692,7 @@ __global__ void __launch_bounds__(CHAIN_THREADS) k_chain_place(ChainArgs a) {
   long long volOut = 1;
   for (int q = 0; q < a.d; ++q)
     volOut *= L.nOut;
-  for (int i = t; i < n; i += CHAIN_THREADS) {
+  for (int i = t; i < n; i += PLACE_THREADS) {
     L.ekey[me.actBefore + i] = (long long)b * volOut + stKey[i];
     L.erow[me.actBefore + i] = (int)(rowBase + i);
   }
@@ -1021,7 +1050,7 @@ int scn_chain_flush(scn_ctx *ctx) {
   }
   SCN_HIP_CHECK(hipGetLastError());
   hipLaunchKernelGGL(k_chain_place, dim3((unsigned)a.batch, (unsigned)a.nLevels),
-                     dim3(CHAIN_THREADS), 0, ctx->stream, a);
+                     dim3(PLACE_THREADS), 0, ctx->stream, a);
   SCN_HIP_CHECK(hipGetLastError());
   return SCN_OK;
 }
