@@ -106,15 +106,19 @@ int scn_fill32(scn_ctx *ctx, void *d_dst, uint32_t word, size_t nWords);
 
 /* ---- sparse grids ----------------------------------------------------- */
 /* A scn_grids holds, for one depth of the net, the SparseGrid of every sample
- * of the batch (SparseGrid.h:26-37, SpatiallySparseBatchInterface.h:36):
- * an open-addressing hash table in HBM from the packed coordinate
- * sample * spatialSize^dimension + key to the batch-global row, an occupancy
- * bit mask over the same packed coordinates, and backgroundCol per sample. */
+ * of the batch (SparseGrid.h:26-37, SpatiallySparseBatchInterface.h:36), over
+ * packed coordinates sample * spatialSize^dimension + key: an occupancy bit
+ * mask with a rank prefix per word, the batch-global rows of the active sites
+ * in map iteration order (sample, then ascending key), the entry list, and
+ * backgroundCol per sample.  An open-addressing hash table in HBM from packed
+ * coordinate to row serves look-ups by coordinate (scn_grids_find); it is
+ * filled as the grids are built for fields of up to 2^20 sites and on the
+ * first look-up otherwise. */
 int scn_grids_create(scn_ctx *ctx, scn_grids **grids);
 int scn_grids_destroy(scn_ctx *ctx, scn_grids *grids);
 /* Start of a batch (SpatiallySparseBatch::reset, SpatiallySparseBatch.cu:14-27,
- * which empties every interface's grids): empties the hash tables and masks
- * of all n objects in one launch, so that the build / plan calls of the batch
+ * which empties every interface's grids): empties the masks (and the hash
+ * tables that are in use) of all n objects in one launch, so that the build / plan calls of the batch
  * need not do it one by one.  Optional; objects it has not seen are emptied
  * by the call that fills them. */
 int scn_grids_clear_many(scn_ctx *ctx, scn_grids **grids, int n);
