@@ -164,77 +164,152 @@ struct GatherSource {
 // The classifier head and the deepest layers of small batches have a few
 // hundred rows: tiles would leave most of the chip idle and run a long k-loop
 // in a handful of workgroups.  Here a workgroup owns FR_ROWS rows x 64 columns
-// and its four wavefronts split K between them: a lane owns one column, loads
-// its quarter of that column of W with FR_DEPTH loads in flight (W is small
+// and its eight wavefronts split K between them: a lane owns one column, loads
+// its share of that column of W with FR_DEPTH loads in flight (W is small
 // and served by the caches) and multiplies it with the rows of A staged in LDS
-// (gathered through the rules if asked); the four partial sums meet in LDS.
+// (gathered through the rules if asked); the eight partial sums meet in LDS.
 #define FR_ROWS 8
-#define FR_DEPTH 24
+#define FR_DEPTH 32
+#define FR_WAVES 8
+#define FR_THREADS (64 * FR_WAVES)
 #define FR_MAX_M 512
 #define FR_MAX_K 1024
-__global__ void __launch_bounds__(256)
+// NB: columns a lane owns (n, n + 64, ...), i.e. a workgroup covers 64 NB
+// columns.  SOFTMAX (the classifier: N <= 64 NB, one workgroup per group of
+// rows holds whole rows): the soft-max of a row is taken by the wavefront
+// that sums it, with the arithmetic of the kernel that does it as a pass of
+// its own (running maximum from -10000, lanes striding over the classes).
+template <int NB, bool SOFTMAX>
+__global__ void __launch_bounds__(FR_THREADS)
     k_nin_fewrows(const float *__restrict__ A, const float *__restrict__ W,
                   float *__restrict__ out, long long M, int K, int N,
                   Epilogue ep, GatherSource gs, bool gather) {
   __shared__ float sA[FR_ROWS * FR_MAX_K];
-  __shared__ float part[4][FR_ROWS][64];
+  __shared__ float part[FR_WAVES][FR_ROWS][64 * NB];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const long long m0 = (long long)blockIdx.x * FR_ROWS;
-  const int n = blockIdx.y * 64 + lane;
-  for (int x = tid; x < FR_ROWS * K; x += 256) {
-    const int r = x / K, k = x - r * K;
+  const int nBase = blockIdx.y * 64 * NB;
+  // this wavefront's share of K, and the first batch of its columns of W on
+  // its way before the rows of A are staged
+  constexpr int DEPTH = FR_DEPTH / NB;
+  const int per = (K + FR_WAVES - 1) / FR_WAVES;
+  const int k0 = wave * per < K ? wave * per : K, k1 = min(K, k0 + per);
+  const float *w[NB];
+#pragma unroll
+  for (int j = 0; j < NB; ++j) {
+    const int n = nBase + 64 * j + lane;
+    w[j] = W + (n < N ? n : 0);
+  }
+  float wv[NB][DEPTH];
+#pragma unroll
+  for (int i = 0; i < DEPTH; ++i) {
+    const int kk = k0 + i < k1 ? k0 + i : (k1 > 0 ? k1 - 1 : 0); // clamped, the product is dropped below
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+      wv[j][i] = w[j][(long long)kk * N];
+  }
+  for (int r = 0; r < FR_ROWS; ++r) {
     const long long m = m0 + r;
-    float v = 0.f;
-    if (m < M) {
-      if (gather) {
-        const int f = k / gs.nIn;
-        const int rule = gs.rules[m * gs.fs + f];
-        if (rule >= 0)
-          v = A[(long long)rule * gs.nIn + (k - f * gs.nIn)];
-      } else {
-        v = A[m * K + k];
+    for (int k = tid; k < K; k += FR_THREADS) {
+      float v = 0.f;
+      if (m < M) {
+        if (gather) {
+          const int f = (int)__umulhi((unsigned)k, gs.magic);
+          const int rule = gs.rules[m * gs.fs + f];
+          if (rule >= 0)
+            v = A[(long long)rule * gs.nIn + (k - f * gs.nIn)];
+        } else {
+          v = A[m * K + k];
+        }
       }
+      sA[r * K + k] = v;
     }
-    sA[x] = v;
   }
   __syncthreads();
-  // this wavefront's share of K
-  const int per = (K + 3) / 4;
-  const int k0 = wave * per, k1 = min(K, k0 + per);
-  float acc[FR_ROWS];
+  float acc[NB][FR_ROWS];
 #pragma unroll
-  for (int r = 0; r < FR_ROWS; ++r)
-    acc[r] = 0.f;
-  const bool col = n < N;
-  const float *w = W + (col ? n : 0);
-  for (int k = k0; k < k1; k += FR_DEPTH) {
-    float wv[FR_DEPTH];
+  for (int j = 0; j < NB; ++j)
 #pragma unroll
-    for (int i = 0; i < FR_DEPTH; ++i) {
-      const int kk = k + i < k1 ? k + i : k1 - 1; // clamped, the product is dropped below
-      wv[i] = w[(long long)kk * N];
+    for (int r = 0; r < FR_ROWS; ++r)
+      acc[j][r] = 0.f;
+  for (int k = k0; k < k1; k += DEPTH) {
+    if (k > k0) {
+#pragma unroll
+      for (int i = 0; i < DEPTH; ++i) {
+        const int kk = k + i < k1 ? k + i : k1 - 1;
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+          wv[j][i] = w[j][(long long)kk * N];
+      }
     }
 #pragma unroll
-    for (int i = 0; i < FR_DEPTH; ++i)
+    for (int i = 0; i < DEPTH; ++i)
       if (k + i < k1) {
 #pragma unroll
-        for (int r = 0; r < FR_ROWS; ++r)
-          acc[r] = fmaf(sA[r * K + k + i], wv[i], acc[r]);
+        for (int r = 0; r < FR_ROWS; ++r) {
+          const float a = sA[r * K + k + i];
+#pragma unroll
+          for (int j = 0; j < NB; ++j)
+            acc[j][r] = fmaf(a, wv[j][i], acc[j][r]);
+        }
       }
   }
 #pragma unroll
-  for (int r = 0; r < FR_ROWS; ++r)
-    part[wave][r][lane] = acc[r];
+  for (int j = 0; j < NB; ++j)
+#pragma unroll
+    for (int r = 0; r < FR_ROWS; ++r)
+      part[wave][r][64 * j + lane] = acc[j][r];
   __syncthreads();
-  // 512 sums, two per lane, always added in wavefront order
-  for (int x = tid; x < FR_ROWS * 64; x += 256) {
-    const int r = x >> 6, c = x & 63;
-    const long long m = m0 + r;
-    const int nn = blockIdx.y * 64 + c;
-    if (m < M && nn < N) {
-      const float v = ((part[0][r][c] + part[1][r][c]) + part[2][r][c]) + part[3][r][c];
-      out[m * N + nn] = apply_act(v, nn, ep);
+  // the partial sums are always added in wavefront order
+  if (!SOFTMAX) {
+    for (int x = tid; x < FR_ROWS * 64 * NB; x += FR_THREADS) {
+      const int r = x / (64 * NB), c = x - r * (64 * NB);
+      const long long m = m0 + r;
+      const int nn = nBase + c;
+      if (m < M && nn < N) {
+        float v = part[0][r][c];
+#pragma unroll
+        for (int u = 1; u < FR_WAVES; ++u)
+          v += part[u][r][c];
+        out[m * N + nn] = apply_act(v, nn, ep);
+      }
     }
+  } else {
+    static_assert(FR_WAVES == FR_ROWS, "one wavefront per row");
+    const int r = wave;
+    const long long m = m0 + r;
+    if (m >= M)
+      return;
+    float z[NB];
+    float mx = -10000.0f;
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+      const int c = 64 * j + lane;
+      float v = part[0][r][c];
+#pragma unroll
+      for (int u = 1; u < FR_WAVES; ++u)
+        v += part[u][r][c];
+      z[j] = 0.f;
+      if (c < N) {
+        z[j] = apply_act(v, c, ep); // bias and scale; the activation itself is the soft-max below
+        mx = fmaxf(mx, z[j]);
+      }
+    }
+    for (int off = 32; off > 0; off >>= 1)
+      mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+      if (64 * j + lane < N) {
+        z[j] = expf(z[j] - mx);
+        sum += z[j];
+      }
+    for (int off = 32; off > 0; off >>= 1)
+      sum += __shfl_xor(sum, off, 64);
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+      if (64 * j + lane < N)
+        out[m * N + 64 * j + lane] = z[j] / sum;
   }
 }
 
@@ -1785,6 +1860,7 @@ static int nin_forward(scn_ctx *ctx, const float *d_A, const float *d_W,
   ep.slope = act == SCN_LEAKYRELU ? 0.01f : (act == SCN_VLEAKYRELU ? 0.333f : 0.f);
   ep.act = act;
   ProfScope prof(ctx, gs ? SCN_K_CONV_NIN : SCN_K_NIN);
+  bool softmaxDone = false;
   const bool vec = K % 4 == 0 && N % 4 == 0 && ((uintptr_t)d_A & 15) == 0 &&
                    ((uintptr_t)d_W & 15) == 0 && ((uintptr_t)d_out & 15) == 0;
   // bf16 operands only where the contraction is big enough to matter; the
@@ -1806,10 +1882,18 @@ static int nin_forward(scn_ctx *ctx, const float *d_A, const float *d_W,
   } else if (M <= FR_MAX_M && K <= FR_MAX_K && !(vec && K % 32 == 0 && N % 16 == 0)) {
     // (shapes the W-resident kernel takes are faster there)
     GatherSource none = GatherSource();
-    hipLaunchKernelGGL(k_nin_fewrows,
-                       dim3(scn_ceil_div(M, FR_ROWS), scn_ceil_div(N, 64)),
-                       dim3(256), 0, ctx->stream, d_A, d_W, d_out, (long long)M,
-                       K, N, ep, gs ? *gs : none, gs != nullptr);
+    if (act == SCN_SOFTMAX && N <= 128) {
+      // whole rows in one workgroup: the soft-max rides along
+      softmaxDone = true;
+      hipLaunchKernelGGL((k_nin_fewrows<2, true>), dim3(scn_ceil_div(M, FR_ROWS), 1),
+                         dim3(FR_THREADS), 0, ctx->stream, d_A, d_W, d_out,
+                         (long long)M, K, N, ep, gs ? *gs : none, gs != nullptr);
+    } else {
+      hipLaunchKernelGGL((k_nin_fewrows<1, false>),
+                         dim3(scn_ceil_div(M, FR_ROWS), scn_ceil_div(N, 64)),
+                         dim3(FR_THREADS), 0, ctx->stream, d_A, d_W, d_out,
+                         (long long)M, K, N, ep, gs ? *gs : none, gs != nullptr);
+    }
   } else if (vec && !gs && K <= TK_MAX_K) {
     hipLaunchKernelGGL(k_nin_thin, dim3(scn_ceil_div(M, 32), scn_ceil_div(N, 32)),
                        dim3(256), 0, ctx->stream, d_A, d_W, d_out, (long long)M,
@@ -1852,7 +1936,7 @@ static int nin_forward(scn_ctx *ctx, const float *d_A, const float *d_W,
   // softmax, tanh and the logistic function are a pass of their own over the
   // layer's output, as in the reference (the kernels above treat them as
   // "no activation")
-  if (act == SCN_SOFTMAX)
+  if (act == SCN_SOFTMAX && !softmaxDone)
     SCN_TRY(scn_softmax_launch(ctx, d_out, d_out, (long long)M, N));
   if (act == SCN_TANH || act == SCN_SIGMOID)
     SCN_TRY(scn_squash_launch(ctx, d_out, (long long)M * N, act == SCN_SIGMOID));
