@@ -442,12 +442,57 @@ __device__ __forceinline__ unsigned row_bits(const unsigned long long *bits,
 // neighbourhood -- and every candidate is then decided in registers.  Bit c of
 // the result stands for candidate c of the box [lo, hi) in ascending key;
 // f(j) is called for the owned ones.
+// The same for windows that do not overlap (stride == S, the usual max-pooling
+// geometry): the one output whose window holds site i is owned by i when no
+// site of that window before i is active.  The window's S^(D-1) rows are
+// requested together.
+template <int D, int S, typename Pos, typename F>
+__device__ __forceinline__ unsigned
+owned_disjoint(const unsigned long long *bits, Pos base, const int *i,
+               const int *lo, const int *hi, int nIn, unsigned magicStride,
+               F f) {
+  int j[D], a[D];
+  bool ok = true;
+#pragma unroll
+  for (int q = 0; q < D; ++q) {
+    j[q] = (int)div_magic((unsigned)i[q], (unsigned)S, magicStride);
+    a[q] = i[q] - j[q] * S;
+    ok = ok && j[q] >= lo[q] && j[q] < hi[q];
+  }
+  unsigned before = 0;
+  if (D == 2) {
+#pragma unroll
+    for (int r = 0; r < S; ++r) {
+      const int lead[1] = {j[0] * S + r};
+      const unsigned row = row_bits<2>(bits, base, lead, j[1] * S, S, nIn);
+      before |= r < a[0] ? row : (r == a[0] ? row & ((1u << a[1]) - 1u) : 0u);
+    }
+  } else {
+#pragma unroll
+    for (int pl = 0; pl < S; ++pl)
+#pragma unroll
+      for (int r = 0; r < S; ++r) {
+        const int lead[2] = {j[0] * S + pl, j[1] * S + r};
+        const unsigned row = row_bits<3>(bits, base, lead, j[D - 1] * S, S, nIn);
+        const bool whole = pl < a[0] || (pl == a[0] && r < a[1]);
+        const bool part = pl == a[0] && r == a[1];
+        before |= whole ? row : (part ? row & ((1u << a[D - 1]) - 1u) : 0u);
+      }
+  }
+  if (!ok || before != 0)
+    return 0u;
+  f(j);
+  return 1u; // the box has this one candidate
+}
+
 template <int D, int S, typename Pos, typename F>
 __device__ __forceinline__ unsigned
 owned_nomin(const unsigned long long *bits, Pos base, const int *i,
             const int *lo, const int *hi, int nIn, int stride,
             unsigned magicStride, F f) {
   static_assert(D == 2 || D == 3, "two or three dimensions");
+  if (stride == S)
+    return owned_disjoint<D, S>(bits, base, i, lo, hi, nIn, magicStride, f);
   constexpr int W = 2 * S - 1;
   constexpr unsigned FULL = (1u << S) - 1u;
   unsigned m = 0;
