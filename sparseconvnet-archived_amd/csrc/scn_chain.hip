@@ -281,18 +281,47 @@ __global__ void __launch_bounds__(CHAIN_THREADS) k_chain_sample(ChainArgs a) {
       }
     }
     lds_barrier();
-    // (one lane per entry: the table look-ups of a sample are all in flight together)
+    // One lane per entry, eight entries a lane at a time: their first probes
+    // of the table are requested together (a probe is a trip to HBM, and at
+    // load factor 1/2 three look-ups in four end with the first).
     const long long p0 = (long long)b * vol;
-    for (unsigned r = t; r < nA; r += CHAIN_THREADS) {
-      unsigned key = keyA[r];
-      rowA[r] = (unsigned)hash_find(a.table, a.shift, a.mask, p0 + key);
-      int c[D];
+    constexpr int EU = 8;
+    for (unsigned r0 = t; r0 < nA; r0 += EU * CHAIN_THREADS) {
+      unsigned key[EU], slot[EU];
+      int4 first[EU];
 #pragma unroll
-      for (int q = D - 1; q >= 0; --q) {
-        c[q] = (int)(key % (unsigned)a.n0);
-        key /= (unsigned)a.n0;
+      for (int u = 0; u < EU; ++u) {
+        const unsigned r = r0 + u * CHAIN_THREADS;
+        key[u] = keyA[r < nA ? r : t];
+        slot[u] = hash_slot(p0 + key[u], a.shift);
+        first[u] = *reinterpret_cast<const int4 *>(&a.table[slot[u]]);
       }
-      keyA[r] = pack_site<D>(c);
+#pragma unroll
+      for (int u = 0; u < EU; ++u) {
+        const unsigned r = r0 + u * CHAIN_THREADS;
+        if (r >= nA)
+          continue;
+        const long long p = p0 + key[u];
+        long long k = ((long long)first[u].y << 32) | (unsigned)first[u].x;
+        int row = first[u].z;
+        unsigned sl = slot[u];
+        while (k != p && k != SLOT_EMPTY) { // the rest of the probe sequence
+          sl = (sl + 1) & a.mask;
+          const int4 v = *reinterpret_cast<const int4 *>(&a.table[sl]);
+          k = ((long long)v.y << 32) | (unsigned)v.x;
+          row = v.z;
+        }
+        rowA[r] = (unsigned)(k == p ? row : -1);
+        unsigned kk = key[u];
+        int c[D];
+#pragma unroll
+        for (int q = D - 1; q >= 0; --q) {
+          const unsigned up = kk / (unsigned)a.n0;
+          c[q] = (int)(kk - up * (unsigned)a.n0);
+          kk = up;
+        }
+        keyA[r] = pack_site<D>(c);
+      }
     }
   }
   int bgA = a.bg[b];

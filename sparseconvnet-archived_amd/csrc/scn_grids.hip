@@ -1030,6 +1030,7 @@ extern "C" int scn_grids_clear_many(scn_ctx *ctx, scn_grids **grids, int n) {
       g->rankValid = false;
       g->rankRowValid = false;
       g->tableValid = false;
+      g->nActive = 0; // (the entry list goes with the mask: an emptied object holds no sites)
       ++m;
     }
     if (m == 0)
