@@ -1191,13 +1191,7 @@ static int launch_wstream(scn_ctx *ctx, const float *A, const float *W,
   const size_t lds =
       WSTREAM_LDS_BYTES(NW, SA) + (gs ? WRES_RULE_BYTES(gs->fs) : 0);
   long long wgs = scn_ceil_div(scn_ceil_div(M, 16), 8);
-  // Two workgroups per compute unit where LDS allows, except when that would
-  // leave every wavefront a single panel: then one workgroup per compute unit,
-  // whose wavefronts fetch their second panel under the first one's MFMAs
-  // (measured on 60478 x 128 x 64: 17.8 us against 19.1).
-  long long cap = (long long)ctx->numCU * (lds * 2 <= WRES_LDS_BYTES ? 2 : 1);
-  if (wgs <= cap && wgs > ctx->numCU)
-    cap = ctx->numCU;
+  const long long cap = (long long)ctx->numCU * (lds * 2 <= WRES_LDS_BYTES ? 2 : 1);
   if (wgs > cap)
     wgs = cap;
   static OncePerDevice configured; // one set of attribute calls per instantiation and device
@@ -1579,13 +1573,7 @@ static int launch_wstream_bf16(scn_ctx *ctx, const float *A, const float *W,
   const size_t lds =
       WSTREAM_BF16_LDS_BYTES(NW) + (gs ? WRES_RULE_BYTES(gs->fs) : 0);
   long long wgs = scn_ceil_div(scn_ceil_div(M, 16), 8);
-  // Two workgroups per compute unit where LDS allows, except when that would
-  // leave every wavefront a single panel: then one workgroup per compute unit,
-  // whose wavefronts fetch their second panel under the first one's MFMAs
-  // (measured on 60478 x 128 x 64: 17.8 us against 19.1).
-  long long cap = (long long)ctx->numCU * (lds * 2 <= WRES_LDS_BYTES ? 2 : 1);
-  if (wgs <= cap && wgs > ctx->numCU)
-    cap = ctx->numCU;
+  const long long cap = (long long)ctx->numCU * (lds * 2 <= WRES_LDS_BYTES ? 2 : 1);
   if (wgs > cap)
     wgs = cap;
   static OncePerDevice configured; // one set of attribute calls per instantiation and device
