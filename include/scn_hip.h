@@ -110,10 +110,10 @@ int scn_fill32(scn_ctx *ctx, void *d_dst, uint32_t word, size_t nWords);
  * packed coordinates sample * spatialSize^dimension + key: an occupancy bit
  * mask with a rank prefix per word, the batch-global rows of the active sites
  * in map iteration order (sample, then ascending key), the entry list, and
- * backgroundCol per sample.  An open-addressing hash table in HBM from packed
- * coordinate to row serves look-ups by coordinate (scn_grids_find); it is
- * filled as the grids are built for fields of up to 2^20 sites and on the
- * first look-up otherwise. */
+ * backgroundCol per sample.  Look-ups by coordinate (scn_grids_find) go
+ * through a dense table of rows, filled as the grids are built, for batches
+ * of up to 2^24 lattice sites, and otherwise through an open-addressing hash
+ * table in HBM from packed coordinate to row that the first look-up fills. */
 int scn_grids_create(scn_ctx *ctx, scn_grids **grids);
 int scn_grids_destroy(scn_ctx *ctx, scn_grids *grids);
 /* Start of a batch (SpatiallySparseBatch::reset, SpatiallySparseBatch.cu:14-27,

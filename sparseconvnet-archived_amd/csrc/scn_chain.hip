@@ -65,7 +65,8 @@ struct ChainLevel {
 
 struct ChainArgs {
   int nLevels, batch, d, n0;
-  const Slot *table; // the source grids
+  const Slot *table; // the source grids: hash table,
+  const int *dense;  // or dense row table
   unsigned shift, mask;
   const unsigned long long *bits;
   const int *bg;
@@ -286,6 +287,20 @@ __global__ void __launch_bounds__(CHAIN_THREADS) k_chain_sample(ChainArgs a) {
     // load factor 1/2 three look-ups in four end with the first).
     const long long p0 = (long long)b * vol;
     constexpr int EU = 8;
+    if (a.dense) { // the row of every site of the field: one load an entry
+      for (unsigned r = t; r < nA; r += CHAIN_THREADS) {
+        unsigned kk = keyA[r];
+        rowA[r] = (unsigned)a.dense[p0 + kk];
+        int c[D];
+#pragma unroll
+        for (int q = D - 1; q >= 0; --q) {
+          const unsigned up = kk / (unsigned)a.n0;
+          c[q] = (int)(kk - up * (unsigned)a.n0);
+          kk = up;
+        }
+        keyA[r] = pack_site<D>(c);
+      }
+    } else
     for (unsigned r0 = t; r0 < nA; r0 += EU * CHAIN_THREADS) {
       unsigned key[EU], slot[EU];
       int4 first[EU];
@@ -989,6 +1004,7 @@ int scn_chain_flush(scn_ctx *ctx) {
   a.d = src->d;
   a.n0 = src->n;
   a.table = src->table.p;
+  a.dense = (long long)src->batch * src->vol <= SCN_DENSE_MAX_SITES ? src->dense.p : nullptr;
   a.shift = 64 - src->log2cap;
   a.mask = (1u << src->log2cap) - 1u;
   a.bits = src->bits.p;

@@ -10,10 +10,11 @@
 //     element of this array, and sites that are neighbours along the innermost
 //     axis are neighbours in it: a run of a rule row reads consecutive words;
 //   * the list of entries (packed coordinate, row) in no particular order;
-//   * on demand, an open-addressing hash table, linear probing, 16-byte slots
-//     {int64 packed coordinate, int32 row}, load factor <= 1/2, for look-ups by
-//     coordinate (scn_grids_find) and for the source of a chain of recorded
-//     plans.
+//   * for look-ups by coordinate (scn_grids_find, the source of a chain of
+//     recorded plans) a dense table of rows, one int per site of the field and
+//     valid where the mask is set, while the batch's fields are small enough;
+//     else, on demand, an open-addressing hash table, linear probing, 16-byte
+//     slots {int64 packed coordinate, int32 row}, load factor <= 1/2.
 //
 // Rule books (Regions.cu gridRules*) number output sites in first-touch order
 // while the input map is iterated in ascending key.  An output site is first
@@ -52,7 +53,9 @@ __global__ void k_grid_build(GridView g, const int *sample,
   }
   long long p = (long long)b * g.vol + k;
   int r = row[e];
-  if (g.table)
+  if (g.dense)
+    g.dense[p] = r;
+  else if (g.table)
     hash_insert(g.table, g.shift, g.mask, p, r);
   atomicOr(&g.bits[p >> 6], 1ull << (p & 63));
   ekey[e] = p;
@@ -884,19 +887,20 @@ __global__ void k_find(GridView g, const int *sample, const long long *key,
   int b = sample[e];
   int r = -1;
   if (b >= 0 && b < g.batch && k >= 0 && k < g.vol)
-    r = hash_find(g.table, g.shift, g.mask, (long long)b * g.vol + k);
+    r = grid_row(g, (long long)b * g.vol + k);
   row[e] = r;
 }
 
 // ------------------------------------------------------------------ host
 
-// largest field (sites of one sample) whose source grids get a hash table as
-// they are built: about what a workgroup's LDS can hold as masks
-#define SCN_EAGER_TABLE_VOL (1ll << 20)
+static bool dense_rows(const scn_grids *g) {
+  return (long long)(g->batch > 0 ? g->batch : 1) * g->vol <= SCN_DENSE_MAX_SITES;
+}
 
 GridView view_of(const scn_grids *g) {
   GridView v;
-  v.table = g->tableValid ? g->table.p : nullptr;
+  v.table = g->tableValid && !dense_rows(g) ? g->table.p : nullptr;
+  v.dense = g->tableValid && dense_rows(g) ? g->dense.p : nullptr;
   v.shift = 64 - g->log2cap;
   v.mask = (1u << g->log2cap) - 1u;
   v.bits = g->bits.p;
@@ -954,7 +958,10 @@ static int grids_prepare(scn_ctx *ctx, scn_grids *g, int batch, int d, int n,
   const size_t cap = (size_t)1 << lg;
   g->nWords = (size_t)(((long long)batch * vol + 63) / 64);
   const void *hadTable = g->table.p, *hadBits = g->bits.p;
-  if (withTable)
+  const bool dense = dense_rows(g);
+  if (withTable && dense)
+    SCN_TRY(g->dense.reserve((size_t)((long long)batch * vol) + 1));
+  else if (withTable)
     SCN_TRY(g->table.reserve(cap));
   SCN_TRY(g->bits.reserve(g->nWords + 8)); // the scan reads whole 32-byte groups
   if (g->table.p != hadTable)
@@ -965,9 +972,10 @@ static int grids_prepare(scn_ctx *ctx, scn_grids *g, int batch, int d, int n,
   SCN_TRY(g->ekey.reserve((size_t)nActive + 1));
   SCN_TRY(g->erow.reserve((size_t)nActive + 1));
   SCN_TRY(g->bg.reserve((size_t)batch + 1));
-  const size_t clearSlots = withTable && cap > g->cleanSlots ? cap : 0;
+  // (a dense row table needs no clearing: it is read where the mask is set)
+  const size_t clearSlots = withTable && !dense && cap > g->cleanSlots ? cap : 0;
   const size_t clearWords = g->nWords + 2 > g->cleanWords ? g->nWords + 2 : 0;
-  if (withTable)
+  if (withTable && !dense)
     g->cleanSlots = 0; // about to be written
   g->cleanWords = 0;
   if (clearSlots || clearWords) {
@@ -1061,13 +1069,16 @@ __global__ void k_rank_rows(GridView g, const long long *ekey, const int *erow,
     return;
   rankRow[rank_of(g, ekey[e])] = erow[e];
 }
-// the hash table from the entry list
+// the look-up table (dense rows or hash) from the entry list
 __global__ void k_grid_table(GridView g, const long long *ekey, const int *erow,
                              Count n, const long long *meta) {
   long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (e >= n.bound || (meta && meta[META_OVERFLOW]) || e >= count_now(n))
     return;
-  hash_insert(g.table, g.shift, g.mask, ekey[e], erow[e]);
+  if (g.dense)
+    g.dense[ekey[e]] = erow[e];
+  else
+    hash_insert(g.table, g.shift, g.mask, ekey[e], erow[e]);
 }
 static Count count_active(const scn_grids *g);
 // the occupancy mask of grids that only hold their entry list
@@ -1121,26 +1132,30 @@ static int ensure_rank(scn_ctx *ctx, scn_grids *g) {
   return SCN_OK;
 }
 
-// the hash table, for look-ups by coordinate
+// the table for look-ups by coordinate
 int scn_grids_ensure_table(scn_ctx *ctx, scn_grids *g) {
   SCN_TRY(ensure_index(ctx, g));
   if (g->tableValid)
     return SCN_OK;
-  const size_t cap = (size_t)1 << g->log2cap;
-  const void *had = g->table.p;
-  SCN_TRY(g->table.reserve(cap));
-  if (g->table.p != had)
+  if (dense_rows(g)) {
+    SCN_TRY(g->dense.reserve((size_t)((long long)g->batch * g->vol) + 1));
+  } else {
+    const size_t cap = (size_t)1 << g->log2cap;
+    const void *had = g->table.p;
+    SCN_TRY(g->table.reserve(cap));
+    if (g->table.p != had)
+      g->cleanSlots = 0;
+    if (g->cleanSlots < cap) {
+      size_t blocks = (cap + 255) / 256;
+      if (blocks > 16384)
+        blocks = 16384;
+      hipLaunchKernelGGL(k_clear_grid, dim3((unsigned)blocks), dim3(256), 0,
+                         ctx->stream, (uint4 *)g->table.p, cap,
+                         (unsigned long long *)nullptr, (size_t)0);
+      SCN_HIP_CHECK(hipGetLastError());
+    }
     g->cleanSlots = 0;
-  if (g->cleanSlots < cap) {
-    size_t blocks = (cap + 255) / 256;
-    if (blocks > 16384)
-      blocks = 16384;
-    hipLaunchKernelGGL(k_clear_grid, dim3((unsigned)blocks), dim3(256), 0,
-                       ctx->stream, (uint4 *)g->table.p, cap,
-                       (unsigned long long *)nullptr, (size_t)0);
-    SCN_HIP_CHECK(hipGetLastError());
   }
-  g->cleanSlots = 0;
   g->tableValid = true; // (view_of hands the table out from here on)
   if (g->nActive > 0) {
     hipLaunchKernelGGL(k_grid_table, dim3(scn_ceil_div(g->nActive, 256)),
@@ -1286,6 +1301,7 @@ extern "C" int scn_grids_destroy(scn_ctx *ctx, scn_grids *g) {
   }
   g->meta.release();
   g->table.release();
+  g->dense.release();
   g->bits.release();
   g->prefix.release();
   g->rankRow.release();
@@ -1322,13 +1338,14 @@ extern "C" int scn_grids_build(scn_ctx *ctx, scn_grids *g, int batch,
               "scn_grids_build: null background array");
   SCN_TRY(scn_chain_flush(ctx));
   ProfScope ps(ctx, SCN_K_GRID_BUILD);
-  // fields small enough for a chain of recorded plans get their table now
-  // (the chain reads its source through it); larger ones when somebody asks
-  long long vol = 1;
+  // batches small enough for a dense row table get it as they are built (a
+  // chain of recorded plans reads its source through it); larger ones get
+  // their hash table when somebody asks
+  long long sites = batch > 0 ? batch : 1;
   for (int a = 0; a < dimension && a < 3; ++a)
-    vol *= spatialSize > 0 ? spatialSize : 1;
+    sites *= spatialSize > 0 ? spatialSize : 1;
   SCN_TRY(grids_prepare(ctx, g, batch, dimension, spatialSize, n,
-                        vol <= SCN_EAGER_TABLE_VOL));
+                        sites <= SCN_DENSE_MAX_SITES));
   g->nSites = nSpatialSites;
   // (backgroundCol is copied by the same launch: lane e < batch takes entry e)
   const long long lanes = n > batch ? n : batch;

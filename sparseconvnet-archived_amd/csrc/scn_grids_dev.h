@@ -36,7 +36,8 @@ __device__ __forceinline__ int fmp_inputR(const Geom &g, int b, int a, int j) {
 }
 
 struct GridView {
-  Slot *table;
+  Slot *table; // look-ups by coordinate: a hash table, or for small batches
+  int *dense;  // the row of every site of the field (valid where the mask is set)
   unsigned shift, mask;
   unsigned long long *bits;
   const unsigned *prefix;
@@ -74,9 +75,10 @@ struct scn_grids {
   // list, backgroundCol and the counts, and the rest is built from them on
   // demand), its rank prefix (rankValid), the rows by rank (rankRowValid) and
   // the hash table (tableValid).  Rule books are built from mask, prefix and
-  // rows by rank; the table serves scn_grids_find and the source of a chain
-  // of recorded plans, and is filled by scn_grids_build only for fields small
-  // enough for such a chain.
+  // rows by rank; look-ups by coordinate (scn_grids_find, the source of a
+  // chain of recorded plans) go through a dense row table when the batch's
+  // fields are small enough for one (SCN_DENSE_MAX_SITES, filled as the grids
+  // are built) and through a hash table otherwise (filled on demand).
   bool rankValid = false;
   bool rankRowValid = false;
   bool tableValid = false;
@@ -94,6 +96,7 @@ struct scn_grids {
   long long seenRows = 0, seenActive = 0, seenWidth = 0;
   DevBuf<long long> meta; // META_* words
   DevBuf<Slot> table;
+  DevBuf<int> dense;
   DevBuf<unsigned long long> bits;
   DevBuf<unsigned> prefix;
   DevBuf<int> rankRow;
@@ -142,6 +145,10 @@ __device__ __forceinline__ void hash_insert(Slot *t, unsigned shift,
   }
 }
 
+// sites of a batch (batch * spatialSize^d) up to which look-ups by coordinate
+// use a dense row table instead of a hash table
+#define SCN_DENSE_MAX_SITES (1ll << 24)
+
 __device__ __forceinline__ int hash_find(const Slot *t, unsigned shift,
                                          unsigned mask, long long p) {
   unsigned s = hash_slot(p, shift);
@@ -164,6 +171,13 @@ struct __attribute__((packed, aligned(8))) Words2 {
 struct __attribute__((packed, aligned(8))) Words3 {
   unsigned long long a, b, c;
 };
+
+// row of the site at packed position p, -1 when it is not active
+__device__ __forceinline__ int grid_row(const GridView &g, long long p) {
+  if (g.dense)
+    return (g.bits[p >> 6] >> (p & 63)) & 1ull ? g.dense[p] : -1;
+  return hash_find(g.table, g.shift, g.mask, p);
+}
 
 // `len` (1..32) mask bits starting at bit position p
 __device__ __forceinline__ unsigned get_bits(const unsigned long long *bits,

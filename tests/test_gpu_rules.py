@@ -77,10 +77,10 @@ def test_square_rules_rows_longer_than_a_mask_word(scn, ctx, d, size, stride, nO
 
 
 def test_find_on_grids_without_a_table(scn, ctx):
-    """Look-ups by coordinate on grids whose hash table is only built when asked for: input grids of a field too large
-    for one, and the output grids of a rule-book plan."""
+    """Look-ups by coordinate on grids whose hash table is only built when asked for: input grids of a batch too large
+    for a dense row table, and the output grids of a rule-book plan (which never get either as they are built)."""
     rng = np.random.default_rng(21)
-    d, nIn = 3, 110  # 110^3 sites: beyond the fields that get a table as they are built
+    d, nIn = 3, 210  # 2 x 210^3 sites: beyond the batches that get a dense row table as they are built
     samples = []
     row = 0
     for b in range(2):
