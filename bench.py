@@ -63,6 +63,10 @@ def parse():
     ap.add_argument("--calibration-copy-mb", type=int, default=0,
                     help="first launch a plain row copy (gather with identity rules) of this many MB, so that "
                          "hardware byte counters collected over the run can be scaled by a kernel of known traffic")
+    ap.add_argument("--distinct-batches", type=int, default=8,
+                    help="also time a pass over this many DIFFERENT synthetic batches taken in turn (other seeds, same "
+                         "batch size): their site counts differ, so the bounds of the deferred counts are exercised; "
+                         "reported beside the headline figure (0 disables it)")
     ap.add_argument("--from-host", action="store_true",
                     help="also time processDataset() on host-resident Pictures (CPU codify + PCIe upload included)")
     ap.add_argument("--producers", type=int, default=5,
@@ -196,6 +200,28 @@ def main():
                                      hF.ptr, inputs_on_host=True, h_probs=probs)
     ctx.sync()
     upload_bytes = int(S.size * 4 + K.size * 8 + R.size * 4 + bg.size * 4 + feats.size * 4)
+    # the same pass over several different batches taken in turn
+    varied = None
+    if args.distinct_batches > 1:
+        keep, descr, actives = [], [], []
+        for i in range(args.distinct_batches):
+            Si, Ki, Ri, bgi, fi, ni = synthetic.codify(synthetic.make_samples(cfg, args.seed + 100 + i), cfg.dimension,
+                                                       cfg.lattice, net.inputSpatialSize, cfg.nInputFeatures)
+            arrs = (ctx.array(Si, np.int32), ctx.array(Ki, np.int64), ctx.array(Ri, np.int32), ctx.array(bgi, np.int32),
+                    ctx.array(fi, np.float32))
+            keep.append(arrs)
+            descr.append((B, arrs[0].ptr, arrs[1].ptr, arrs[2].ptr, arrs[3].ptr, int(len(Ki)), int(ni), arrs[4].ptr))
+            actives.append(int(len(Ki)))
+        net.forward_stream_timed_many(0, priming + args.distinct_batches, descr, h_probs=probs)
+        dt_var = net.forward_stream_timed_many(args.warmup, args.steps, descr, h_probs=probs)
+        ctx.sync()
+        timed_sites = sum(actives[(args.warmup + i) % len(actives)] for i in range(args.steps))
+        varied = {"distinct_batches": args.distinct_batches, "ms_per_step": 1e3 * dt_var / args.steps,
+                  "active_sites_per_s": timed_sites / dt_var, "samples_per_s": B * args.steps / dt_var,
+                  "active_sites_min_max": [min(actives), max(actives)],
+                  "note": "different batches in turn (seeds %d..%d), inputs resident" % (args.seed + 100,
+                                                                                        args.seed + 99 + len(actives))}
+        del keep
     # one batch at a time on one stream, nothing overlapped: the latency of a batch
     for _ in range(3):
         step()
@@ -364,6 +390,7 @@ def main():
                               "ms_per_step": 1e3 * dt_up / args.steps, "bytes_uploaded_per_step": upload_bytes,
                               "note": "sites and features in pinned host memory, uploaded on the producer streams for "
                                       "every batch: forward time = rule build + H2D of inputs + kernels + D2H"},
+        "varied_batches": varied,
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,

@@ -62,9 +62,12 @@ public:
   std::vector<int> permutation;
   BatchProducer(SparseConvNetCUDA &cnn, SpatiallySparseDataset &dataset,
                 int spatialSize, int batchSize);
-  // nBatches passes over one batch that is resident in HBM (benchmarking)
+  // nBatches passes over one batch that is resident in HBM (benchmarking), or
+  // over several taken in turn
   BatchProducer(SparseConvNetCUDA &cnn, const ResidentBatch &resident,
                 int nBatches);
+  BatchProducer(SparseConvNetCUDA &cnn,
+                const std::vector<ResidentBatch> &residents, int nBatches);
   ~BatchProducer();
   // nextBatch() hands the slot of the batch it returned keepAlive + 1 calls
   // ago back to the workers: 0 is the reference's behaviour; 1 lets the caller
@@ -79,8 +82,7 @@ public:
 
 private:
   static SpatiallySparseDataset emptyDataset;
-  const ResidentBatch *resident;
-  ResidentBatch residentCopy;
+  std::vector<ResidentBatch> residents; // empty: batches come from the dataset
   void start();
   std::vector<char> slotFull;
   std::condition_variable slotChanged;

@@ -736,7 +736,7 @@ BatchProducer::BatchProducer(SparseConvNetCUDA &cnn,
                              SpatiallySparseDataset &dataset, int spatialSize,
                              int batchSize)
     : cnn(cnn), batchCounter(-1), dataset(dataset), batchSize(batchSize),
-      spatialSize(spatialSize), resident(nullptr), stopping(false) {
+      spatialSize(spatialSize), stopping(false) {
   assert(batchSize > 0);
   nBatches = ((int)dataset.pictures.size() + batchSize - 1) / batchSize;
   permutation = range((int)dataset.pictures.size());
@@ -748,9 +748,14 @@ BatchProducer::BatchProducer(SparseConvNetCUDA &cnn,
 }
 BatchProducer::BatchProducer(SparseConvNetCUDA &cnn,
                              const ResidentBatch &residentBatch, int nBatches)
+    : BatchProducer(cnn, std::vector<ResidentBatch>(1, residentBatch), nBatches) {}
+BatchProducer::BatchProducer(SparseConvNetCUDA &cnn,
+                             const std::vector<ResidentBatch> &residentBatches,
+                             int nBatches)
     : cnn(cnn), batchCounter(-1), nBatches(nBatches), dataset(emptyDataset),
-      batchSize(residentBatch.batchSize), spatialSize(cnn.inputSpatialSize),
-      resident(&residentCopy), residentCopy(residentBatch), stopping(false) {
+      batchSize(residentBatches.at(0).batchSize),
+      spatialSize(cnn.inputSpatialSize), residents(residentBatches),
+      stopping(false) {
   start();
 }
 void BatchProducer::start() {
@@ -863,13 +868,14 @@ void BatchProducer::batchProducerThread(int nThread) {
     }
     {
       std::lock_guard<std::mutex> slot(cnn.batchLock[nThread]);
+      const bool resident = !residents.empty();
       if (!resident)
         preprocessBatch(c, nThread, rng); // CPU half
       // GPU half, on a stream borrowed for it
       cudaMemStream *stream = cnn.acquireProducerStream(c);
       cnn.batchPool[nThread].preprocessStream = stream;
       if (resident)
-        cnn.preprocessResident(nThread, *resident);
+        cnn.preprocessResident(nThread, residents[c % residents.size()]);
       else
         preprocessBatchOnDevice(nThread);
       cnn.releaseProducerStream(stream);

@@ -565,11 +565,31 @@ int scnh_forward_stream_timed(scnh_net *net, int nWarmup, int nTimed, int batch,
                               int64_t nActive, int nSpatialSites,
                               const float *features, int inputsOnHost,
                               float *h_probs, double *seconds) {
+  const int32_t *samples[1] = {sample};
+  const int64_t *keys[1] = {key};
+  const int32_t *rows[1] = {row};
+  const int32_t *backgrounds[1] = {background};
+  const float *feats[1] = {features};
+  return scnh_forward_stream_timed_many(net, nWarmup, nTimed, 1, &batch, samples,
+                                        keys, rows, backgrounds, &nActive,
+                                        &nSpatialSites, feats, inputsOnHost,
+                                        h_probs, seconds);
+}
+int scnh_forward_stream_timed_many(
+    scnh_net *net, int nWarmup, int nTimed, int nDistinct, const int *batch,
+    const int32_t *const *sample, const int64_t *const *key,
+    const int32_t *const *row, const int32_t *const *background,
+    const int64_t *nActive, const int *nSpatialSites,
+    const float *const *features, int inputsOnHost, float *h_probs,
+    double *seconds) {
   SparseConvNetCUDA *cnn = net->cnn;
-  ResidentBatch r = resident_of(batch, sample, key, row, background, nActive,
-                                nSpatialSites, features);
-  r.onHost = inputsOnHost != 0;
-  BatchProducer bp(*cnn, r, nWarmup + nTimed);
+  std::vector<ResidentBatch> rs;
+  for (int i = 0; i < nDistinct; ++i) {
+    rs.push_back(resident_of(batch[i], sample[i], key[i], row[i], background[i],
+                             nActive[i], nSpatialSites[i], features[i]));
+    rs.back().onHost = inputsOnHost != 0;
+  }
+  BatchProducer bp(*cnn, rs, nWarmup + nTimed);
   ForwardQueue queue(*cnn, bp, !net->hasClassifier); // (a headless net: layer by layer on lane 0)
   int done = 0, started = 0;
   auto finish = [&](SpatiallySparseBatch *b) {

@@ -206,6 +206,16 @@ int scnh_forward_stream_timed(scnh_net *net, int nWarmup, int nTimed, int batch,
                               int64_t nActive, int nSpatialSites,
                               const float *features, int inputsOnHost,
                               float *h_probs, double *seconds);
+/* The same over nDistinct different batches taken in turn (batch i of the pass
+ * is number i % nDistinct): every argument that describes a batch is an array
+ * of nDistinct.  h_probs must hold the largest batch. */
+int scnh_forward_stream_timed_many(
+    scnh_net *net, int nWarmup, int nTimed, int nDistinct, const int *batch,
+    const int32_t *const *sample, const int64_t *const *key,
+    const int32_t *const *row, const int32_t *const *background,
+    const int64_t *nActive, const int *nSpatialSites,
+    const float *const *features, int inputsOnHost, float *h_probs,
+    double *seconds);
 /* the library context of the net (scn_ctx *), for timing and raw buffers */
 void *scnh_context(scnh_net *net);
 /* multiply-accumulates of the NiN layers since the last call */

@@ -96,6 +96,7 @@ def lib():
         "scnh_forward_resident": (i32, [vp, i32, vp, vp, vp, vp, i64, i32, vp, vp]),
         "scnh_forward_resident_stream": (i32, [vp, i32, i32, vp, vp, vp, vp, i64, i32, vp, vp]),
         "scnh_forward_stream_timed": (i32, [vp, i32, i32, i32, vp, vp, vp, vp, i64, i32, vp, i32, vp, P(C.c_double)]),
+        "scnh_forward_stream_timed_many": (i32, [vp, i32, i32, i32, vp, vp, vp, vp, vp, vp, vp, vp, i32, vp, P(C.c_double)]),
         "scnh_context": (vp, [vp]),
         "scnh_take_multiply_add_count": (C.c_double, []),
     }
@@ -412,6 +413,22 @@ class Net:
         done = lib().scnh_forward_stream_timed(self.h, nWarmup, nTimed, batch, sample, key, row, bg, nActive,
                                                nSpatialSites, features, int(inputs_on_host),
                                                _p(h_probs) if h_probs is not None else None, C.byref(sec))
+        assert done == nWarmup + nTimed
+        return sec.value
+
+    def forward_stream_timed_many(self, nWarmup, nTimed, batches, inputs_on_host=False, h_probs=None):
+        """The same over several different batches taken in turn; batches: list of (batch, sample, key, row, bg,
+        nActive, nSpatialSites, features) with pointers as integers."""
+        n = len(batches)
+        vpa = C.c_void_p * n
+        col = lambda i: vpa(*[b[i] for b in batches])
+        sizes = (C.c_int * n)(*[b[0] for b in batches])
+        act = (C.c_int64 * n)(*[b[5] for b in batches])
+        sites = (C.c_int * n)(*[b[6] for b in batches])
+        sec = C.c_double()
+        done = lib().scnh_forward_stream_timed_many(self.h, nWarmup, nTimed, n, sizes, col(1), col(2), col(3), col(4),
+                                                    act, sites, col(7), int(inputs_on_host),
+                                                    _p(h_probs) if h_probs is not None else None, C.byref(sec))
         assert done == nWarmup + nTimed
         return sec.value
 

@@ -636,3 +636,34 @@ def test_ten_producer_threads_share_five_streams(scn):
         results.append(np.array(probs))
     assert results[0].shape == (len(samples), 100)
     assert np.array_equal(results[0], results[1])
+
+
+def test_resident_batches_taken_in_turn(scn):
+    """scnh_forward_stream_timed_many: three different resident batches of different sizes taken in turn through five
+    producer threads and two forward lanes; the probabilities left behind are those of the pass's last batch, bit for
+    bit what one batch alone on one stream gives."""
+    from sparseconvnet_archived_amd import hostapi, synthetic
+    cfg = synthetic.config(2, batch=24)
+    net = hostapi.Net(cfg.dimension, cfg.nInputFeatures, cfg.nClasses, nTop=1, threads=5)
+    cfg.build(net)
+    net.setFusedConvolutions(True)
+    for i, (W, B, pr) in synthetic.he_normal_weights(net.layers(), 5).items():
+        net.set_weights(i, W, B, pr)
+    ctx = scn.Context(handle=net.context_handle())
+    keep, descr, alone = [], [], []
+    for i, b in enumerate((24, 9, 17)):
+        samples = synthetic.make_samples(cfg, 300 + i, batch=b)
+        S, K, R, bg, feats, n = synthetic.codify(samples, 2, cfg.lattice, net.inputSpatialSize, 3)
+        arrs = (ctx.array(S, np.int32), ctx.array(K, np.int64), ctx.array(R, np.int32), ctx.array(bg, np.int32),
+                ctx.array(feats, np.float32))
+        keep.append(arrs)
+        descr.append((b, arrs[0].ptr, arrs[1].ptr, arrs[2].ptr, arrs[3].ptr, len(K), n, arrs[4].ptr))
+        p = np.zeros((b, 100), np.float32)
+        net.forward_resident(b, arrs[0].ptr, arrs[1].ptr, arrs[2].ptr, arrs[3].ptr, len(K), n, arrs[4].ptr, p)
+        alone.append(p)
+    for nBatches in (7, 12, 14):  # ends on batch (nBatches - 1) % 3
+        probs = np.zeros((24, 100), np.float32)
+        assert net.forward_stream_timed_many(2, nBatches - 2, descr, h_probs=probs) > 0
+        last = (nBatches - 1) % 3
+        assert np.array_equal(probs[: descr[last][0]], alone[last])
+    net.close()
