@@ -158,6 +158,11 @@ struct GatherSource {
   unsigned magic;     // floor(2^32 / nIn) + 1: k / nIn == mulhi(k, magic) for k nIn < 2^32
   const float *zeros; // at least nIn zeros: the row a negative rule stands for
 };
+// k / nIn for the kernels that take any number of channels (the factor does
+// not fit 32 bits for a single channel)
+__device__ __forceinline__ int gather_rule_of(const GatherSource &gs, int k) {
+  return gs.nIn == 1 ? k : (int)__umulhi((unsigned)k, gs.magic);
+}
 
 
 // ---- few rows: split-k FMA kernel --------------------------------------------
@@ -214,7 +219,7 @@ __global__ void __launch_bounds__(FR_THREADS)
       float v = 0.f;
       if (m < M) {
         if (gather) {
-          const int f = (int)__umulhi((unsigned)k, gs.magic);
+          const int f = gather_rule_of(gs, k);
           const int rule = gs.rules[m * gs.fs + f];
           if (rule >= 0)
             v = A[(long long)rule * gs.nIn + (k - f * gs.nIn)];
@@ -356,6 +361,80 @@ __global__ void __launch_bounds__(256)
     r.z = apply_act(acc.z, n + 2, ep);
     r.w = apply_act(acc.w, n + 3, ep);
     *reinterpret_cast<float4 *>(out + m * N + n) = r;
+  }
+}
+
+// The same with the row of A read through the rules (the receptive field of
+// output site m) -- any number of channels, so a convolution over one to three
+// input channels, the first layer of most nets, needs no matrix either.  A
+// workgroup gathers its rows into LDS once (eight lanes a row, up to four
+// values a lane) and walks all of its columns, CT_COLS at most, in blocks of
+// 32; the products of an output are those of the plain kernel on the gathered
+// matrix, in the same order.
+#define CT_COLS 256
+#define CT_GROUPS 2 // groups of 32 rows a workgroup takes: all their loads are in flight together
+__global__ void __launch_bounds__(256)
+    k_conv_thin(const float *__restrict__ A, const float *__restrict__ W,
+                float *__restrict__ out, long long M, int K, int N, Epilogue ep,
+                GatherSource gs) {
+  // LDS: the gathered rows, then this workgroup's columns of W at pitch wp
+  extern __shared__ __attribute__((aligned(16))) float ctLds[];
+  float *const sA = ctLds;
+  float *const sW = ctLds + CT_GROUPS * 32 * TK_MAX_K;
+  const int wp = N < CT_COLS ? N : CT_COLS;
+  const int tid = threadIdx.x;
+  const int n0 = blockIdx.y * CT_COLS;
+  const int cols = N - n0 < CT_COLS ? N - n0 : CT_COLS; // a multiple of 4
+  const int r = tid >> 3;
+  const long long mFirst = (long long)blockIdx.x * (32 * CT_GROUPS) + r;
+  int rule[CT_GROUPS][TK_MAX_K / 8];
+#pragma unroll
+  for (int g = 0; g < CT_GROUPS; ++g)
+#pragma unroll
+    for (int j = 0; j < TK_MAX_K / 8; ++j) {
+      const int k = (tid & 7) + 8 * j;
+      const long long m = mFirst + 32 * g;
+      rule[g][j] = k < K && m < M ? gs.rules[m * gs.fs + gather_rule_of(gs, k)] : -1;
+    }
+  for (int k = tid >> 6; k < K; k += 4) // a wavefront a row of W
+    for (int c = 4 * (tid & 63); c < cols; c += 256)
+      *reinterpret_cast<float4 *>(&sW[k * wp + c]) =
+          *reinterpret_cast<const float4 *>(W + (long long)k * N + n0 + c);
+#pragma unroll
+  for (int g = 0; g < CT_GROUPS; ++g)
+#pragma unroll
+    for (int j = 0; j < TK_MAX_K / 8; ++j) {
+      const int k = (tid & 7) + 8 * j;
+      float v = 0.f;
+      if (rule[g][j] >= 0)
+        v = A[(long long)rule[g][j] * gs.nIn + (k - gather_rule_of(gs, k) * gs.nIn)];
+      sA[(32 * g + r) * TK_MAX_K + k] = v;
+    }
+  __syncthreads();
+#pragma unroll
+  for (int g = 0; g < CT_GROUPS; ++g) {
+    const long long m = mFirst + 32 * g;
+    if (m >= M)
+      break;
+    const float *arow = sA + (32 * g + r) * TK_MAX_K;
+    for (int c4 = (tid & 7) * 4; c4 < cols; c4 += 32) {
+      float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+      for (int k = 0; k < K; ++k) {
+        const float a = arow[k];
+        const float4 wv = *reinterpret_cast<const float4 *>(&sW[k * wp + c4]);
+        acc.x = fmaf(a, wv.x, acc.x);
+        acc.y = fmaf(a, wv.y, acc.y);
+        acc.z = fmaf(a, wv.z, acc.z);
+        acc.w = fmaf(a, wv.w, acc.w);
+      }
+      const int n = n0 + c4;
+      float4 o;
+      o.x = apply_act(acc.x, n, ep);
+      o.y = apply_act(acc.y, n + 1, ep);
+      o.z = apply_act(acc.z, n + 2, ep);
+      o.w = apply_act(acc.w, n + 3, ep);
+      *reinterpret_cast<float4 *>(out + m * N + n) = o;
+    }
   }
 }
 
@@ -1882,6 +1961,12 @@ static int nin_forward(scn_ctx *ctx, const float *d_A, const float *d_W,
                          dim3(FR_THREADS), 0, ctx->stream, d_A, d_W, d_out,
                          (long long)M, K, N, ep, gs ? *gs : none, gs != nullptr);
     }
+  } else if (vec && gs && gs->nIn % 4 != 0) {
+    // channels in other than fours: K <= TK_MAX_K (scn_conv_nin_supported)
+    const size_t lds = (size_t)(CT_GROUPS * 32 * TK_MAX_K + K * (N < CT_COLS ? N : CT_COLS)) * sizeof(float);
+    hipLaunchKernelGGL(k_conv_thin, dim3(scn_ceil_div(M, 32 * CT_GROUPS), scn_ceil_div(N, CT_COLS)),
+                       dim3(256), lds, ctx->stream, d_A, d_W, d_out, (long long)M,
+                       K, N, ep, *gs);
   } else if (vec && !gs && K <= TK_MAX_K) {
     hipLaunchKernelGGL(k_nin_thin, dim3(scn_ceil_div(M, 32), scn_ceil_div(N, 32)),
                        dim3(256), 0, ctx->stream, d_A, d_W, d_out, (long long)M,
@@ -1939,14 +2024,21 @@ extern "C" int scn_nin_forward(scn_ctx *ctx, const float *d_A,
                      precision, nullptr);
 }
 
+// few channels (any number of them) times a small window: the thin kernel
+static bool conv_thin_shape(int fs, int nIn, int N) {
+  return fs >= 1 && fs <= GF_MAX_FS && nIn >= 1 && nIn % 4 != 0 &&
+         fs * nIn <= TK_MAX_K && (fs * nIn) % 4 == 0 && N % 4 == 0;
+}
 extern "C" int scn_conv_nin_supported(int fs, int nIn, int N) {
-  return fs >= 1 && fs <= GF_MAX_FS && nIn >= 4 && nIn % 4 == 0 &&
-         nIn <= SCN_ZERO_FLOATS && N % 4 == 0;
+  return (fs >= 1 && fs <= GF_MAX_FS && nIn >= 4 && nIn % 4 == 0 &&
+          nIn <= SCN_ZERO_FLOATS && N % 4 == 0) ||
+         conv_thin_shape(fs, nIn, N);
 }
 extern "C" int scn_conv_nin_supported_p(int fs, int nIn, int N, int precision) {
   if (!scn_conv_nin_supported(fs, nIn, N))
     return 0;
-  if (precision == SCN_FP32)
+  // (contractions this short stay fp32 in every mode)
+  if (precision == SCN_FP32 || conv_thin_shape(fs, nIn, N))
     return 1;
   // bf16 operands: the shapes of the bf16 W-streaming kernel, whatever M
   return precision == SCN_BF16 && nIn % 8 == 0 &&
@@ -1970,7 +2062,7 @@ extern "C" int scn_conv_nin_forward_p(scn_ctx *ctx, const float *d_in,
   SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_conv_nin_forward: null context");
   SCN_REQUIRE(scn_conv_nin_supported_p(fs, nIn, N, precision), SCN_ERR_ARG,
               "scn_conv_nin_forward: fs %d nIn %d N %d precision %d is outside "
-              "the fused kernels' range (fs <= %d, nIn and N multiples of 4; "
+              "the fused kernels' range (fs <= %d, nIn and N multiples of 4, or fs nIn <= 32 and a multiple of 4; "
               "bf16: nIn of 8, fs nIn of 64, N of 32)",
               fs, nIn, N, precision, GF_MAX_FS);
   SCN_REQUIRE(d_rules || M == 0, SCN_ERR_ARG,

@@ -293,7 +293,10 @@ def test_argument_errors(scn, ctx):
                                            (5000, 4, 128, 160), (64, 1, 4, 32), (300, 25, 8, 100),
                                            # W-streaming kernel: every width of slice, every size of rule load
                                            (1500, 27, 64, 64), (66001, 27, 64, 64), (33005, 9, 192, 96),
-                                           (1100, 4, 504, 48)])
+                                           (1100, 4, 504, 48),
+                                           # few channels: the thin kernel (and the few-rows kernel) through the rules
+                                           (83597, 4, 3, 32), (20000, 8, 1, 32), (300, 4, 3, 32), (400, 16, 2, 32),
+                                           (9000, 16, 2, 64), (2500, 4, 2, 160), (5000, 2, 6, 36)])
 @pytest.mark.parametrize("act", ["RELU", "PRELU"])
 def test_fused_gather_nin_matches_the_two_kernels_bit_for_bit(scn, ctx, rows, fs, nIn, N, act):
     a = getattr(scn, act)
@@ -322,7 +325,9 @@ def test_fused_gather_nin_matches_the_two_kernels_bit_for_bit(scn, ctx, rows, fs
     scale = np.abs(gathered).astype(np.float64) @ np.abs(W).astype(np.float64) + np.abs(B)
     assert np.all(np.abs(fused.download() - want) <= 1e-4 * scale)
     assert not scn.lib().scn_conv_nin_supported(64, 32, 64)  # window too large for the staged rules
-    assert not scn.lib().scn_conv_nin_supported(4, 3, 32)  # channels not a multiple of 4
+    assert scn.lib().scn_conv_nin_supported(4, 3, 32)  # few channels, contraction of 12: the thin kernel
+    assert not scn.lib().scn_conv_nin_supported(9, 3, 32)  # channels not a multiple of 4 and a contraction beyond it
+    assert not scn.lib().scn_conv_nin_supported(5, 3, 32)  # ... or not a multiple of 4
 
 
 def test_maxpool_refuses_inputs_beyond_32_bit_choices(scn, ctx):
