@@ -243,7 +243,10 @@ int scn_nin_forward(scn_ctx *ctx, const float *d_A, const float *d_W,
  * what it replaces on the live path is ConvolutionalLayer::forwards +
  * NetworkInNetwork(PReLU)Layer::forwards (ConvolutionalLayer.cu:125-133,
  * NetworkInNetworkLayer.cu:187-200).  W is [fs * nIn x N].
- * scn_conv_nin_supported tells whether (fs, nIn, N) is in the kernel's range. */
+ * scn_conv_nin_supported tells whether (fs, nIn, N) is in the kernels' range:
+ * windows of up to 27 sites over channels in multiples of 4 with N a multiple
+ * of 4, or any number of channels when fs * nIn is at most 32 and a multiple
+ * of 4 (the first layer of a net: one to three input channels). */
 int scn_conv_nin_supported(int fs, int nIn, int N);
 int scn_conv_nin_forward(scn_ctx *ctx, const float *d_in,
                          const int32_t *d_rules, int fs, int nIn,
@@ -253,7 +256,8 @@ int scn_conv_nin_forward(scn_ctx *ctx, const float *d_in,
 /* The same with the operand precision of scn_nin_forward: SCN_FP32, or SCN_BF16
  * for shapes with nIn a multiple of 8, fs * nIn of 64 and N of 32 (operands
  * rounded to bf16 on their way to the MFMA, fp32 accumulation); bit-identical to
- * scn_gather_rows followed by scn_nin_forward with that precision. */
+ * scn_gather_rows followed by scn_nin_forward with that precision.  (Contractions
+ * of up to 32 stay fp32 in every precision, fused or not.) */
 int scn_conv_nin_supported_p(int fs, int nIn, int N, int precision);
 int scn_conv_nin_forward_p(scn_ctx *ctx, const float *d_in,
                            const int32_t *d_rules, int fs, int nIn,
