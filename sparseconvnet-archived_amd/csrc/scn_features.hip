@@ -118,31 +118,45 @@ __global__ void __launch_bounds__(256)
     arg[k] = 0;
   }
   bool none = true;
-  for (int p = 0; p < ps; ++p) {
-    int rule = rr[p];
-    if (rule < 0)
-      continue;
-    const float *src = in + (long long)rule * C + c0;
-    float v[VEC];
-    if (VEC == 4) {
-      float4 t = *reinterpret_cast<const float4 *>(src);
-      v[0] = t.x;
-      v[1] = t.y;
-      v[2] = t.z;
-      v[3] = t.w;
-    } else {
-      v[0] = src[0];
-    }
-    // 32-bit, as the reference's poolingChoices (the entry points refuse
-    // inputs of 2^31 elements and more where they know the input's size)
-    const int flat = (int)((unsigned)rule * (unsigned)C + (unsigned)c0);
+  // Nine candidates at a time: their rules are requested together, then
+  // their values (a skipped rule reads row 0 and is dropped below), so that a
+  // window costs two trips to memory rather than two per candidate; they
+  // are compared in rule order.
+  constexpr int MP = 9;
+  for (int p0 = 0; p0 < ps; p0 += MP) {
+    int rule[MP];
 #pragma unroll
-    for (int k = 0; k < VEC; ++k)
-      if (none || best[k] < v[k]) {
-        best[k] = v[k];
-        arg[k] = flat + k;
+    for (int u = 0; u < MP; ++u)
+      rule[u] = rr[p0 + u < ps ? p0 + u : ps - 1];
+    float v[MP][VEC];
+#pragma unroll
+    for (int u = 0; u < MP; ++u) {
+      const float *src = in + (long long)(rule[u] > 0 ? rule[u] : 0) * C + c0;
+      if (VEC == 4) {
+        float4 t = *reinterpret_cast<const float4 *>(src);
+        v[u][0] = t.x;
+        v[u][1] = t.y;
+        v[u][2] = t.z;
+        v[u][3] = t.w;
+      } else {
+        v[u][0] = src[0];
       }
-    none = false;
+    }
+#pragma unroll
+    for (int u = 0; u < MP; ++u) {
+      if (p0 + u >= ps || rule[u] < 0)
+        continue;
+      // 32-bit, as the reference's poolingChoices (the entry points refuse
+      // inputs of 2^31 elements and more where they know the input's size)
+      const int flat = (int)((unsigned)rule[u] * (unsigned)C + (unsigned)c0);
+#pragma unroll
+      for (int k = 0; k < VEC; ++k)
+        if (none || best[k] < v[u][k]) {
+          best[k] = v[u][k];
+          arg[k] = flat + k;
+        }
+      none = false;
+    }
   }
   long long o = r * C + c0;
   if (VEC == 4) {
