@@ -213,22 +213,27 @@ __global__ void __launch_bounds__(FR_THREADS)
     for (int j = 0; j < NB; ++j)
       wv[j][i] = w[j][(long long)kk * N];
   }
-  for (int r = 0; r < FR_ROWS; ++r) {
-    const long long m = m0 + r;
-    for (int k = tid; k < K; k += FR_THREADS) {
-      float v = 0.f;
-      if (m < M) {
-        if (gather) {
-          const int f = gather_rule_of(gs, k);
-          const int rule = gs.rules[m * gs.fs + f];
-          if (rule >= 0)
-            v = A[(long long)rule * gs.nIn + (k - f * gs.nIn)];
-        } else {
-          v = A[m * K + k];
-        }
-      }
-      sA[r * K + k] = v;
+  // the rows of A: all FR_ROWS values of a lane's column requested together
+  // (through the rules: the rules together, then the values)
+  for (int k = tid; k < K; k += FR_THREADS) {
+    float v[FR_ROWS];
+    if (gather) {
+      const int f = gather_rule_of(gs, k);
+      int rule[FR_ROWS];
+#pragma unroll
+      for (int r = 0; r < FR_ROWS; ++r)
+        rule[r] = m0 + r < M ? gs.rules[(m0 + r) * gs.fs + f] : -1;
+#pragma unroll
+      for (int r = 0; r < FR_ROWS; ++r)
+        v[r] = rule[r] >= 0 ? A[(long long)rule[r] * gs.nIn + (k - f * gs.nIn)] : 0.f;
+    } else {
+#pragma unroll
+      for (int r = 0; r < FR_ROWS; ++r)
+        v[r] = m0 + r < M ? A[(m0 + r) * K + k] : 0.f;
     }
+#pragma unroll
+    for (int r = 0; r < FR_ROWS; ++r)
+      sA[r * K + k] = v[r];
   }
   __syncthreads();
   float acc[NB][FR_ROWS];
