@@ -224,11 +224,27 @@ __global__ void k_terminal_pool(const float *__restrict__ in,
   const int *rr = rules + b * S;
   float t = 0.f;
   int p = 0;
-  for (; p < S; ++p) {
-    int rule = rr[p];
-    if (rule < 0)
-      break;
-    t += in[(long long)rule * C + j];
+  // four rows at a time: their rules requested together, then their values
+  // (a rule past the sample's last reads row 0 and ends the sum); added in
+  // rule order
+  bool more = true;
+  for (int p0 = 0; p0 < S && more; p0 += 4) {
+    int rule[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      rule[u] = p0 + u < S ? rr[p0 + u] : -1;
+    float v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      v[u] = in[(long long)(rule[u] > 0 ? rule[u] : 0) * C + j];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      more = more && rule[u] >= 0;
+      if (more) {
+        t += v[u];
+        ++p;
+      }
+    }
   }
   out[idx] = t / (float)p;
 }
