@@ -308,6 +308,9 @@ static void buildRuleBooks(SparseConvNetCUDA &cnn, scn_ctx *ctx,
     }
   }
 }
+// Host-resident input of at least this many bytes is uploaded by the copy
+// engine rather than read over the bus by the kernels that use it.
+static const size_t kCopyEngineBytes = 4u << 20;
 void SparseConvNetCUDA::preprocessResident(int cc, const ResidentBatch &input) {
   SpatiallySparseBatch &b = batchPool[cc];
   scn_ctx *ctx = b.preprocessStream ? b.preprocessStream->ctx : memStream.ctx;
@@ -328,18 +331,41 @@ void SparseConvNetCUDA::preprocessResident(int cc, const ResidentBatch &input) {
   const int32_t *d_sample = input.d_sample, *d_row = input.d_row,
                 *d_background = input.d_background;
   const int64_t *d_key = input.d_key;
-  // (input.onHost: the arrays are pinned host memory, which the device reads
-  // over the bus -- the grid-building kernel and the copy below are the upload,
-  // BatchProducer.cu:127-134, on this slot's stream)
+  // input.onHost: the arrays are pinned host memory (the upload of
+  // BatchProducer.cu:127-134, on this slot's stream).  A small batch is read
+  // over the bus by the grid-building kernel and the copy below themselves,
+  // which costs no launch of its own.  A large one goes through the copy
+  // engine into this slot's staging first: kernels that wait for the bus
+  // would hold the wavefront slots that the other batches' layers need for as
+  // long as the transfer takes.
+  size_t nElems = (size_t)input.nSpatialSites * nInputFeatures;
+  const bool byCopyEngine =
+      input.onHost &&
+      (size_t)input.nActive * 16 + nElems * sizeof(float) >= kCopyEngineBytes;
+  if (byCopyEngine) {
+    const size_t n = (size_t)input.nActive;
+    b.stagingSample.resize64(n);
+    b.stagingKey.resize64(2 * n);
+    b.stagingRow.resize64(n);
+    SCN_CHECKED(scn_h2d_async(ctx, b.stagingSample.dPtr(), d_sample, n * 4));
+    SCN_CHECKED(scn_h2d_async(ctx, b.stagingKey.dPtr(), d_key, n * 8));
+    SCN_CHECKED(scn_h2d_async(ctx, b.stagingRow.dPtr(), d_row, n * 4));
+    d_sample = b.stagingSample.dPtr();
+    d_key = (const int64_t *)b.stagingKey.dPtr();
+    d_row = b.stagingRow.dPtr();
+  }
   SCN_CHECKED(scn_grids_build(ctx, in.deviceGrids, input.batchSize, dimension,
                               in.spatialSize, d_sample, d_key, d_row,
                               input.nActive, d_background,
                               input.nSpatialSites));
   in.sub->features.copyToGPU();
-  size_t nElems = (size_t)input.nSpatialSites * nInputFeatures;
   in.sub->features.resize64(nElems);
-  SCN_CHECKED(scn_copy(ctx, in.sub->features.dPtr(), input.d_features,
-                       nElems * sizeof(float)));
+  if (byCopyEngine)
+    SCN_CHECKED(scn_h2d_async(ctx, in.sub->features.dPtr(), input.d_features,
+                              nElems * sizeof(float)));
+  else
+    SCN_CHECKED(scn_copy(ctx, in.sub->features.dPtr(), input.d_features,
+                         nElems * sizeof(float)));
   buildRuleBooks(*this, ctx, b);
   SCN_CHECKED(scn_sync(ctx));
 }
