@@ -1077,7 +1077,12 @@ static bool wres_forward(scn_ctx *ctx, const float *A, const float *W,
 // of the next slab at the start of a slab and puts it into the other buffer
 // at the end; the slab after a panel's last is the next panel's first, so the
 // stream never drains.
-template <int NT, int SA, int GRU>
+//
+// ONE (gathered A only): the input has a multiple of the slab's k channels, so
+// a slab lies within one filter position and its k-steps are consecutive
+// pieces of one input row.  The rule look-up and the 64-bit address then cost
+// once per slab, not once per step; the steps and their order are the same.
+template <int NT, int SA, int GRU, bool ONE>
 __global__ void __launch_bounds__(512, NT <= 4 ? 2 : 1)
     k_nin_wstream(const float *__restrict__ A, const float *__restrict__ W,
                   float *__restrict__ out, long long M, int K, int N,
@@ -1085,6 +1090,7 @@ __global__ void __launch_bounds__(512, NT <= 4 ? 2 : 1)
   constexpr int ROWS = 16;
   typedef WresPipe<ROWS, NT, SA> Pipe;
   constexpr bool GATHER = GRU > 0;
+  static_assert(GATHER || !ONE, "ONE is a way of gathering");
   constexpr int KS = Pipe::KS, NW = Pipe::NW, PITCH = Pipe::PITCH;
   constexpr int SLAB = KS * SA;            // k per slab
   constexpr int SLAB_FLOATS = SLAB * PITCH;
@@ -1125,10 +1131,37 @@ __global__ void __launch_bounds__(512, NT <= 4 ? 2 : 1)
     long long wrap;
     int bufCur, bufNext, rule, ch; // gather
   } st;
+  // ONE: p walks the slab in hand; the second request of a slab is the first
+  // step of the next slab, which starts at pn.  The rule behind pn's successor
+  // is read from LDS a slab before it is turned into an address.
+  struct {
+    const float *p, *pn;
+    int ruleNext, chNext, cnt;
+  } one;
+  // slab G of this panel (G >= nSlabs: slab G - nSlabs of the next panel):
+  // the rule it gathers through and its first channel
+  auto slab_rule = [&](int G, int &ch) -> int {
+    const bool wrap = G >= nSlabs;
+    const int k = SLAB * (wrap ? G - nSlabs : G);
+    const int f = (int)__umulhi((unsigned)k, gs.magic);
+    ch = k - f * gs.nIn;
+    return sRw[(wrap ? st.bufNext : st.bufCur) + c * gs.fs + f];
+  };
+  auto row_ptr = [&](int rule, int ch) -> const float * {
+    return (rule >= 0 ? A + (long long)rule * gs.nIn : gs.zeros) + ch + 4 * q;
+  };
   // as in the W-resident kernel: tt >= T means step tt - T of the next panel
   auto addr = [&](int tt) -> const float * {
     if (!GATHER)
       return st.cur + KS * tt + (tt >= T ? st.wrap : 0ll);
+    if (ONE) {
+      if (one.cnt == 1)
+        one.p = one.pn;
+      ++one.cnt;
+      const float *p = one.p;
+      one.p += KS;
+      return p;
+    }
     const float *p =
         (st.rule >= 0 ? A + (long long)st.rule * gs.nIn : gs.zeros) + st.ch;
     const int tn = tt + 1;
@@ -1198,10 +1231,18 @@ __global__ void __launch_bounds__(512, NT <= 4 ? 2 : 1)
     w_load(0);
     keep_rules(0);
     fetch_rules(panel + 8ll * pgStep);
-    st.ch = 4 * q - (int)__umulhi((unsigned)(4 * q), gs.magic) * gs.nIn;
-    st.rule = sRw[c * gs.fs + (int)__umulhi((unsigned)(4 * q), gs.magic)];
     if (!more)
       st.bufNext = 0; // no next panel: the prefetch past the end re-reads this one
+    if (ONE) {
+      int ch0;
+      const int r0 = slab_rule(0, ch0);
+      one.p = row_ptr(r0, ch0);
+      one.ruleNext = slab_rule(1, one.chNext);
+      one.cnt = 2;
+    } else {
+      st.ch = 4 * q - (int)__umulhi((unsigned)(4 * q), gs.magic) * gs.nIn;
+      st.rule = sRw[c * gs.fs + (int)__umulhi((unsigned)(4 * q), gs.magic)];
+    }
   } else {
     st.cur = A + row_of(panel) * K + 4 * q;
   }
@@ -1233,6 +1274,11 @@ __global__ void __launch_bounds__(512, NT <= 4 ? 2 : 1)
     pipe.clear();
     for (int g = 0; g < nSlabs; ++g) {
       w_load(g + 1 < nSlabs ? g + 1 : 0);
+      if (ONE) {
+        one.pn = row_ptr(one.ruleNext, one.chNext);
+        one.ruleNext = slab_rule(g + 2, one.chNext);
+        one.cnt = 0;
+      }
       auto handover = [&]() {
         w_store(cur ^ 1);
         __syncthreads();
@@ -1281,29 +1327,41 @@ static int launch_wstream(scn_ctx *ctx, const float *A, const float *W,
   static OncePerDevice configured; // one set of attribute calls per instantiation and device
   const int rc = configured.run(ctx->device, [&]() {
     int rc = SCN_OK;
-#define SCN_WSTREAM_LDS(G)                                                     \
+#define SCN_WSTREAM_LDS(G, ONE)                                                \
   if (hipFuncSetAttribute(                                                     \
-          reinterpret_cast<const void *>(k_nin_wstream<NT, SA, G>),            \
+          reinterpret_cast<const void *>(k_nin_wstream<NT, SA, G, ONE>),       \
           hipFuncAttributeMaxDynamicSharedMemorySize,                          \
           WRES_LDS_BYTES) != hipSuccess)                                       \
     rc = SCN_ERR_HIP;
-    SCN_WSTREAM_LDS(0) SCN_WSTREAM_LDS(1) SCN_WSTREAM_LDS(3) SCN_WSTREAM_LDS(7)
+    SCN_WSTREAM_LDS(0, false)
+    SCN_WSTREAM_LDS(1, false) SCN_WSTREAM_LDS(3, false) SCN_WSTREAM_LDS(7, false)
+    SCN_WSTREAM_LDS(1, true) SCN_WSTREAM_LDS(3, true) SCN_WSTREAM_LDS(7, true)
 #undef SCN_WSTREAM_LDS
     return rc;
   });
   SCN_REQUIRE(rc == SCN_OK, SCN_ERR_HIP, "hipFuncSetAttribute failed");
   const dim3 grid((unsigned)(wgs * nSplits));
-#define SCN_WSTREAM_GO(G, src)                                                 \
-  hipLaunchKernelGGL((k_nin_wstream<NT, SA, G>), grid, dim3(512), lds,         \
+#define SCN_WSTREAM_GO(G, ONE, src)                                            \
+  hipLaunchKernelGGL((k_nin_wstream<NT, SA, G, ONE>), grid, dim3(512), lds,    \
                      ctx->stream, A, W, out, M, K, N, ep, src, nSplits)
+#define SCN_WSTREAM_EITHER(G)                                                  \
+  do {                                                                         \
+    if (one)                                                                   \
+      SCN_WSTREAM_GO(G, true, *gs);                                            \
+    else                                                                       \
+      SCN_WSTREAM_GO(G, false, *gs);                                           \
+  } while (0)
+  // a slab within one filter position, and at least two slabs to a panel
+  const bool one = gs && gs->nIn % (16 * SA) == 0 && K >= 2 * 16 * SA;
   if (!gs)
-    SCN_WSTREAM_GO(0, GatherSource());
+    SCN_WSTREAM_GO(0, false, GatherSource());
   else if (gs->fs <= 4)
-    SCN_WSTREAM_GO(1, *gs);
+    SCN_WSTREAM_EITHER(1);
   else if (gs->fs <= 12)
-    SCN_WSTREAM_GO(3, *gs);
+    SCN_WSTREAM_EITHER(3);
   else
-    SCN_WSTREAM_GO(7, *gs);
+    SCN_WSTREAM_EITHER(7);
+#undef SCN_WSTREAM_EITHER
 #undef SCN_WSTREAM_GO
   return SCN_OK;
 }
