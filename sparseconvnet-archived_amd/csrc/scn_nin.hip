@@ -706,43 +706,64 @@ template <int ROWS, int NT, int SA> struct WresPipe {
       a[(s + SA - 1) % SA] =
           *reinterpret_cast<const float4 *>(addr(t + SA - 1));
       read_w(wl, t + 1 < T ? t + 1 : 0, (s + 1) & 1);
-      // keep this step's prefetches ahead of its MFMAs and inside the step
-      __builtin_amdgcn_sched_barrier(0);
       const float av[4] = {a[s].x, a[s].y, a[s].z, a[s].w};
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int j = 0; j < NT; ++j)
           acc[j] = DirectAcc<ROWS>::mfma(av[i], b[s & 1][i][j], acc[j]);
-      __builtin_amdgcn_sched_barrier(0);
+      spread();
     }
   }
+  // The order of a step's instructions.  A wavefront issues in order, so a
+  // load or LDS read that has to wait for its unit holds back the MFMAs behind
+  // it, and the eight wavefronts of a workgroup, which walk in step, all ask
+  // for those units at once.  With the step's prefetches dealt out among its
+  // MFMAs, one after every MFMA_PER of them together with a share of the
+  // address arithmetic, such a wait passes while the matrix pipe is still busy
+  // with the MFMA before it.  The prefetches stay inside the step.
+  static constexpr int MFMA_PER = NT >= 3 ? 2 : 1;
+  __device__ __forceinline__ void spread() {
+#pragma unroll
+    for (int i = 0; i < 4 * NT / MFMA_PER; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, MFMA_PER, 0); // MFMA
+      __builtin_amdgcn_sched_group_barrier(0x320, 1, 0); // a load, an LDS read or write
+      __builtin_amdgcn_sched_group_barrier(0x002, 2, 0); // vector arithmetic
+      __builtin_amdgcn_sched_group_barrier(0x004, 2, 0); // scalar arithmetic
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
   // SA k-steps whose W is the slab at wslab (lane-offset as wl is); b[0] holds
-  // its first step's W on entry.  Before the last step's MFMAs, handover()
-  // puts the next slab in place (stores + barrier): every wavefront has by
-  // then read all it needs of this slab, and the first W of the next slab
-  // (at wnext) is read under those MFMAs.
-  template <class Addr, class Handover>
+  // its first step's W on entry.  stage() puts the next slab into the other
+  // buffer, which nobody reads any more since the barrier before this slab:
+  // among the MFMAs of the last step but one when the slab is long enough for
+  // its loads to have arrived by then, else with the last step's.  Before the
+  // last step's MFMAs every wavefront has read all it needs of this slab:
+  // sync() is the barrier, and the first W of the next slab (at wnext) is read
+  // under those MFMAs.
+  template <class Addr, class Stage, class Sync>
   __device__ __forceinline__ void slab(int t0, Addr &addr, const float *wslab,
-                                       const float *wnext, Handover &handover) {
+                                       const float *wnext, Stage &stage,
+                                       Sync &sync) {
 #pragma unroll
     for (int s = 0; s < SA; ++s) {
       a[(s + SA - 1) % SA] =
           *reinterpret_cast<const float4 *>(addr(t0 + s + SA - 1));
-      if (s + 1 < SA) {
+      if (s + 1 < SA)
         read_w(wslab, s + 1, (s + 1) & 1);
-      } else {
-        handover();
+      if (s == (SA >= 4 ? SA - 2 : SA - 1))
+        stage();
+      if (s + 1 == SA) {
+        sync();
         read_w(wnext, 0, 0);
       }
-      __builtin_amdgcn_sched_barrier(0);
       const float av[4] = {a[s].x, a[s].y, a[s].z, a[s].w};
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int j = 0; j < NT; ++j)
           acc[j] = DirectAcc<ROWS>::mfma(av[i], b[s & 1][i][j], acc[j]);
-      __builtin_amdgcn_sched_barrier(0);
+      spread();
     }
   }
   // orow: row 4 q of the panel, column NT c of the slice
@@ -1075,8 +1096,8 @@ static bool wres_forward(scn_ctx *ctx, const float *A, const float *W,
 // eight consecutive 16-row panels and walk k in step, so one slab serves all
 // of them: one barrier per slab, none inside it.  Each thread fetches its part
 // of the next slab at the start of a slab and puts it into the other buffer
-// at the end; the slab after a panel's last is the next panel's first, so the
-// stream never drains.
+// towards the end; the slab after a panel's last is the next panel's first, so
+// the stream never drains.
 //
 // ONE (gathered A only): the input has a multiple of the slab's k channels, so
 // a slab lies within one filter position and its k-steps are consecutive
@@ -1279,12 +1300,10 @@ __global__ void __launch_bounds__(512, NT <= 4 ? 2 : 1)
         one.ruleNext = slab_rule(g + 2, one.chNext);
         one.cnt = 0;
       }
-      auto handover = [&]() {
-        w_store(cur ^ 1);
-        __syncthreads();
-      };
+      auto stage = [&]() { w_store(cur ^ 1); };
+      auto sync = [&]() { __syncthreads(); };
       pipe.slab(g * SA, addr, wl + cur * SLAB_FLOATS,
-                wl + (cur ^ 1) * SLAB_FLOATS, handover);
+                wl + (cur ^ 1) * SLAB_FLOATS, stage, sync);
       cur ^= 1;
     }
     // (the columns' constants are fetched here, once per panel of K / 16
