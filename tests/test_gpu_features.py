@@ -294,6 +294,8 @@ def test_argument_errors(scn, ctx):
                                            # W-streaming kernel: every width of slice, every size of rule load
                                            (1500, 27, 64, 64), (66001, 27, 64, 64), (33005, 9, 192, 96),
                                            (1100, 4, 504, 48),
+                                           # ... slabs of 32 k within one filter position (32 and 96 channels)
+                                           (2000, 27, 32, 64), (40001, 9, 96, 64),
                                            # few channels: the thin kernel (and the few-rows kernel) through the rules
                                            (83597, 4, 3, 32), (20000, 8, 1, 32), (300, 4, 3, 32), (400, 16, 2, 32),
                                            (9000, 16, 2, 64), (2500, 4, 2, 160), (5000, 2, 6, 36)])
