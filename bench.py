@@ -70,10 +70,14 @@ def parse():
     ap.add_argument("--from-host", action="store_true",
                     help="also time processDataset() on host-resident Pictures (CPU codify + PCIe upload included)")
     ap.add_argument("--producers", type=int, default=5,
-                    help="batch-producer threads / streams building rule books ahead of the forward pass.  HIP "
-                         "spreads streams over 4 hardware queues, and kernels of streams that share a queue run "
-                         "in order: with 5 producer streams the forward pass's stream (created first) still has "
-                         "its queue to itself (measured: 0.30 ms per batch of config 2, 0.35 with 6 or 4)")
+                    help="batch-producer threads building grids and rule books ahead of the forward pass (the "
+                         "reference's nBatchProducerThreads); they share at most five streams")
+    ap.add_argument("--producer-streams", type=int, default=-1,
+                    help="how many of those streams take part (SparseConvNetCUDA::setProducerStreams; 0: all).  HIP "
+                         "spreads streams over 4 hardware queues and kernels of streams that share a queue run in "
+                         "order: with two forward lanes, two producer streams leave every stream a queue of its "
+                         "own.  Default: 2 for the configs whose forward pass is the longer half (2, 4, 5), all "
+                         "for those that wait for their batches (1, 3)")
     ap.add_argument("--train", action="store_true",
                     help="time training batches instead (forward, backward pass, momentum step; Pictures on the host, "
                          "processDataset on a TRAINBATCH dataset): an auxiliary line, not the headline metric")
@@ -137,6 +141,9 @@ def main():
     cfg = synthetic.config(args.config, batch=args.batch)
     B = cfg.batch
     net = hostapi.Net(cfg.dimension, cfg.nInputFeatures, max(cfg.nClasses, 1), threads=max(1, args.producers))
+    if args.producer_streams < 0:
+        args.producer_streams = 2 if args.config in (2, 4, 5) and not args.train else 0
+    net.setProducerStreams(args.producer_streams)
     cfg.build(net)
     net.setFusedConvolutions(bool(args.fused))
     if args.precision != "fp32":
@@ -391,6 +398,7 @@ def main():
                               "note": "sites and features in pinned host memory, uploaded on the producer streams for "
                                       "every batch: forward time = rule build + H2D of inputs + kernels + D2H"},
         "varied_batches": varied,
+        "producer_streams_in_use": net.producerStreamsInUse(),
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,

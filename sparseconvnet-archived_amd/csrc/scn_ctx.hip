@@ -50,7 +50,11 @@ extern "C" int scn_ctx_create(int device, scn_ctx **out) {
   SCN_HIP_CHECK(hipMalloc((void **)&c->d_scalars, 16 * sizeof(int64_t)));
   SCN_HIP_CHECK(hipMemset(c->d_scalars, 0, 16 * sizeof(int64_t)));
   SCN_HIP_CHECK(hipMalloc((void **)&c->d_zeros, SCN_ZERO_FLOATS * sizeof(float)));
-  SCN_HIP_CHECK(hipMemset(c->d_zeros, 0, SCN_ZERO_FLOATS * sizeof(float)));
+  // (on the context's own stream: HIP gives a stream its hardware queue with
+  // the first work it gets, which takes about a millisecond -- here rather
+  // than in front of the first batch that happens to use the stream)
+  SCN_HIP_CHECK(hipMemsetAsync(c->d_zeros, 0, SCN_ZERO_FLOATS * sizeof(float), c->stream));
+  SCN_HIP_CHECK(hipStreamSynchronize(c->stream));
   *out = c;
   return SCN_OK;
 }

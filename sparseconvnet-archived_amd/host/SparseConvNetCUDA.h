@@ -16,6 +16,7 @@
 
 #define N_MAX_BATCH_PRODUCER_THREADS 20
 #define N_PRODUCER_STREAMS 5
+#define N_HARDWARE_QUEUES 4 // per process (GPU_MAX_HW_QUEUES, HIP's default)
 
 // A batch whose input is already in HBM: active sites (sample, key, row),
 // backgroundCol per sample, and the feature matrix [nSpatialSites x
@@ -58,6 +59,17 @@ public:
   // number goes first, so the consumer's next batch is never behind a later
   // one); the CPU halves of all threads run side by side.
   std::vector<std::unique_ptr<cudaMemStream>> batchMemStreams;
+  // How many of them are in use (all, unless told otherwise).  Kernels of
+  // streams that share a hardware queue run one after the other, and HIP has
+  // N_HARDWARE_QUEUES of them: with two forward lanes, two producer streams
+  // leave every stream a queue of its own, and no rule-book kernel then sits
+  // between two kernels of a forward pass.  That is the better choice for a
+  // net whose forward pass takes longer than the production of its batches
+  // (0.122 against 0.128 ms a batch on a five-level 2-D net); a net that waits
+  // for its batches (one layer; a 3-D net, whose rule books are the longer
+  // half) wants all of them.
+  void setProducerStreams(int n);
+  int producerStreamsInUse();
   // Forward lanes.  The kernels of one forward pass follow one another on one
   // stream, and most of them are too short to fill the GPU: with two lanes
   // the dataset loops keep the forward passes of two consecutive test batches
@@ -81,6 +93,7 @@ private:
   std::condition_variable streamPoolChanged;
   std::vector<cudaMemStream *> freeProducerStreams;
   std::multiset<int> waitingBatches;
+  int producerStreamsWanted; // 0: all
 
 public:
   std::mutex batchLock[N_MAX_BATCH_PRODUCER_THREADS];

@@ -21,7 +21,7 @@ SparseConvNetCUDA::SparseConvNetCUDA(int dimension, int nInputFeatures,
     : dimension(dimension), nClasses(nClasses), nTop(nTop),
       inputSpatialSize(0), nInputFeatures(nInputFeatures),
       nOutputFeatures(nInputFeatures), deviceID(0),
-      nBatchProducerThreads(nBatchProducerThreads) {
+      nBatchProducerThreads(nBatchProducerThreads), producerStreamsWanted(0) {
   (void)pciBusID; // one GPU per process: the context picks device 0
   assert(nBatchProducerThreads >= 1 &&
          nBatchProducerThreads <= N_MAX_BATCH_PRODUCER_THREADS);
@@ -44,6 +44,21 @@ SparseConvNetCUDA::SparseConvNetCUDA(int dimension, int nInputFeatures,
     batchPool.emplace_back(initialSubInterfaces.back());
     batchPool.back().preprocessStream = batchMemStreams[c % nStreams].get();
   }
+}
+// (between passes: no producer thread holds a stream)
+void SparseConvNetCUDA::setProducerStreams(int n) {
+  std::lock_guard<std::mutex> lock(streamPoolMutex);
+  producerStreamsWanted = n;
+  const int all = (int)batchMemStreams.size();
+  const int use = n < 1 || n > all ? all : n;
+  freeProducerStreams.clear();
+  for (int c = 0; c < use; c++)
+    freeProducerStreams.push_back(batchMemStreams[c].get());
+}
+int SparseConvNetCUDA::producerStreamsInUse() {
+  std::lock_guard<std::mutex> lock(streamPoolMutex);
+  const int all = (int)batchMemStreams.size();
+  return producerStreamsWanted < 1 || producerStreamsWanted > all ? all : producerStreamsWanted;
 }
 cudaMemStream *SparseConvNetCUDA::acquireProducerStream(int batchNumber) {
   std::unique_lock<std::mutex> lock(streamPoolMutex);
@@ -84,9 +99,7 @@ void SparseConvNetCUDA::limitBatchProducerThreads(int n) {
   const int nStreams = std::min(n, N_PRODUCER_STREAMS);
   while ((int)batchMemStreams.size() > nStreams)
     batchMemStreams.pop_back();
-  freeProducerStreams.clear();
-  for (auto &s : batchMemStreams)
-    freeProducerStreams.push_back(s.get());
+  setProducerStreams(producerStreamsWanted);
   for (int c = 0; c < n; c++)
     batchPool[c].preprocessStream = batchMemStreams[c % nStreams].get();
 }

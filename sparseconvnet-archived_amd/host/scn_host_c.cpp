@@ -107,6 +107,12 @@ int scnh_finish_headless(scnh_net *net, int topSpatialSize) {
 void scnh_set_fused_convolutions(scnh_net *net, int on) {
   net->cnn->setFusedConvolutions(on != 0);
 }
+void scnh_set_producer_streams(scnh_net *net, int n) {
+  net->cnn->setProducerStreams(n);
+}
+int scnh_producer_streams_in_use(scnh_net *net) {
+  return net->cnn->producerStreamsInUse();
+}
 void scnh_set_chained_rule_books(scnh_net *net, int on) {
   net->cnn->chainRuleBooks = on != 0;
 }

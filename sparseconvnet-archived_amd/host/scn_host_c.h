@@ -34,6 +34,11 @@ int scnh_finish_headless(scnh_net *net, int topSpatialSize);
 void scnh_set_precision(scnh_net *net, int precision);
 /* SparseConvNetCUDA::setFusedConvolutions */
 void scnh_set_fused_convolutions(scnh_net *net, int on);
+/* how many of the net's producer streams take part in batch production
+ * (SparseConvNetCUDA::setProducerStreams; n < 1: all of them), to be called
+ * between passes; and how many do */
+void scnh_set_producer_streams(scnh_net *net, int n);
+int scnh_producer_streams_in_use(scnh_net *net);
 /* rule books of consecutive layers built together (default) or layer by layer */
 void scnh_set_chained_rule_books(scnh_net *net, int on);
 int scnh_input_spatial_size(scnh_net *net);

@@ -43,6 +43,8 @@ def lib():
         "scnh_finish_headless": (i32, [vp, i32]),
         "scnh_set_precision": (None, [vp, i32]),
         "scnh_set_fused_convolutions": (None, [vp, i32]),
+        "scnh_set_producer_streams": (None, [vp, i32]),
+        "scnh_producer_streams_in_use": (i32, [vp]),
         "scnh_set_chained_rule_books": (None, [vp, i32]),
         "scnh_input_spatial_size": (i32, [vp]),
         "scnh_n_layers": (i32, [vp]),
@@ -251,6 +253,12 @@ class Net:
 
     def setFusedConvolutions(self, on=True):
         lib().scnh_set_fused_convolutions(self.h, int(on))
+
+    def setProducerStreams(self, n):
+        lib().scnh_set_producer_streams(self.h, int(n))
+
+    def producerStreamsInUse(self):
+        return lib().scnh_producer_streams_in_use(self.h)
 
     def setChainedRuleBooks(self, on=True):
         lib().scnh_set_chained_rule_books(self.h, int(on))

@@ -638,6 +638,36 @@ def test_ten_producer_threads_share_five_streams(scn):
     assert np.array_equal(results[0], results[1])
 
 
+def test_two_producer_streams_give_what_five_give(scn):
+    """setProducerStreams: five producer threads that share two streams (every stream then has a hardware queue of
+    its own beside the two forward lanes) give, bit for bit, what they give with all five."""
+    from sparseconvnet_archived_amd import hostapi, synthetic
+    cfg = synthetic.config(2, batch=11)
+    samples = synthetic.make_samples(cfg, 41, batch=11 * 12 + 5)
+    results = []
+    for streams in (0, 2, 1, 9):
+        net = hostapi.Net(cfg.dimension, cfg.nInputFeatures, cfg.nClasses, nTop=1, threads=5)
+        assert net.producerStreamsInUse() == 5
+        net.setProducerStreams(streams)
+        assert net.producerStreamsInUse() == (streams if 1 <= streams <= 5 else 5)
+        cfg.build(net)
+        net.setFusedConvolutions(True)
+        for i, (W, B, pr) in synthetic.he_normal_weights(net.layers(), 42).items():
+            net.set_weights(i, W, B, pr)
+        ds = hostapi.Dataset("many", 3, 100, hostapi.TESTBATCH)
+        for pts, f, label in samples:
+            ds.add_points(2, cfg.lattice, pts, f, label)
+        probs = []
+        net.begin(ds, 11)
+        while net.next_batch():
+            probs.extend(net.batch_outputs()["probabilities"])
+        net.close()
+        results.append(np.array(probs))
+    assert results[0].shape == (len(samples), 100)
+    for r in results[1:]:
+        assert np.array_equal(results[0], r)
+
+
 def test_resident_batches_taken_in_turn(scn):
     """scnh_forward_stream_timed_many: three different resident batches of different sizes taken in turn through five
     producer threads and two forward lanes; the probabilities left behind are those of the pass's last batch, bit for
