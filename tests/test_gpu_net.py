@@ -638,6 +638,44 @@ def test_ten_producer_threads_share_five_streams(scn):
     assert np.array_equal(results[0], results[1])
 
 
+@pytest.mark.parametrize("batch", [24, 420])
+def test_batches_in_pinned_host_memory_give_what_resident_ones_give(scn, batch):
+    """inputs_on_host: sites and features in pinned host memory, uploaded on the producer streams with every batch.
+    A small batch (under 4 MiB) is read over the bus by the kernels that use it, a large one goes through the copy
+    engine into the slot's staging first; either way the probabilities are those of the resident batch, bit for
+    bit."""
+    from sparseconvnet_archived_amd import hostapi, synthetic
+    cfg = synthetic.config(2, batch=batch)
+    net = hostapi.Net(cfg.dimension, cfg.nInputFeatures, cfg.nClasses, nTop=1, threads=5)
+    cfg.build(net)
+    net.setFusedConvolutions(True)
+    for i, (W, B, pr) in synthetic.he_normal_weights(net.layers(), 6).items():
+        net.set_weights(i, W, B, pr)
+    ctx = scn.Context(handle=net.context_handle())
+    samples = synthetic.make_samples(cfg, 400, batch=batch)
+    S, K, R, bg, feats, n = synthetic.codify(samples, 2, cfg.lattice, net.inputSpatialSize, 3)
+    nbytes = 16 * len(K) + 4 * feats.size
+    assert (nbytes >= 4 << 20) == (batch == 420)  # which side of the copy-engine threshold this case is on
+    dev = (ctx.array(S, np.int32), ctx.array(K, np.int64), ctx.array(R, np.int32), ctx.array(bg, np.int32),
+           ctx.array(feats, np.float32))
+    want = np.zeros((batch, 100), np.float32)
+    net.forward_resident(batch, dev[0].ptr, dev[1].ptr, dev[2].ptr, dev[3].ptr, len(K), n, dev[4].ptr, want)
+
+    def pinned(a):
+        h = ctx.host_alloc(a.nbytes)
+        np.frombuffer(h.buffer(), a.dtype, a.size)[:] = a.reshape(-1)
+        return h
+
+    host = [pinned(np.ascontiguousarray(x)) for x in (S.astype(np.int32), K.astype(np.int64), R.astype(np.int32),
+                                                      bg.astype(np.int32), feats.astype(np.float32))]
+    descr = [(batch, host[0].ptr, host[1].ptr, host[2].ptr, host[3].ptr, len(K), n, host[4].ptr)]
+    got = np.zeros((batch, 100), np.float32)
+    assert net.forward_stream_timed_many(3, 8, descr, inputs_on_host=True, h_probs=got) > 0
+    assert np.array_equal(got, want)
+    del host
+    net.close()
+
+
 def test_two_producer_streams_give_what_five_give(scn):
     """setProducerStreams: five producer threads that share two streams (every stream then has a hardware queue of
     its own beside the two forward lanes) give, bit for bit, what they give with all five."""
