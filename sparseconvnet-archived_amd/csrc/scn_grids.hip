@@ -69,7 +69,7 @@ __global__ void k_plan_count(GridView in, Geom g, const long long *ekey,
                              Count nEntries, const long long *inMeta,
                              unsigned *cntByRank, unsigned long long *ownMask,
                              unsigned *rankOf) {
-  long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  long long e = xcd_contiguous_block((count_now(nEntries) + 255) / 256) * blockDim.x + threadIdx.x;
   if (e >= nEntries.bound)
     return;
   // an input whose own deferred plan outgrew its bounds holds no entries worth
@@ -253,7 +253,8 @@ __global__ void k_plan_emit(GridView in, GridView out, Geom g,
                             const unsigned *base, const int *bgBefore,
                             const int *outBg, long long *okey, int *orow,
                             long long *siteKey) {
-  long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long live = count_now(nEntries) > in.batch ? count_now(nEntries) : in.batch;
+  long long e = xcd_contiguous_block((live + 255) / 256) * blockDim.x + threadIdx.x;
   if (outMeta[META_OVERFLOW])
     return; // the bounds did not hold: nothing may be written
   if (e < in.batch) { // background rows
@@ -295,7 +296,8 @@ __global__ void k_plan_emit_masked(GridView in, GridView out, Geom g,
                                    const int *bgBefore, const int *outBg,
                                    long long *okey, int *orow,
                                    long long *siteKey) {
-  long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long live = count_now(nEntries) > in.batch ? count_now(nEntries) : in.batch;
+  long long e = xcd_contiguous_block((live + 255) / 256) * blockDim.x + threadIdx.x;
   const int c = blockIdx.y;
   if (outMeta[META_OVERFLOW])
     return; // the bounds did not hold: nothing may be written
@@ -343,7 +345,8 @@ __global__ void k_plan_emit_walk(GridView in, GridView out, Geom g,
                                  const unsigned *rankOf, const int *bgBefore,
                                  const int *outBg, long long *okey, int *orow,
                                  long long *siteKey) {
-  long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long live = count_now(nEntries) > in.batch ? count_now(nEntries) : in.batch;
+  long long e = xcd_contiguous_block((live + 255) / 256) * blockDim.x + threadIdx.x;
   if (outMeta[META_OVERFLOW])
     return; // the bounds did not hold: nothing may be written
   if (e < in.batch) { // background rows
@@ -425,7 +428,12 @@ template <int D>
 __global__ void __launch_bounds__(256)
     k_mask_dilate(GridView in, Geom g, unsigned long long *outBits,
                   long long nWords, long long totalBits) {
-  const long long w = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  // Workgroups are dealt to the 8 XCDs round-robin and every XCD has an L2 of
+  // its own: each XCD takes one contiguous eighth of the words (the grid is a
+  // multiple of 8), so that the rows and planes a word's windows reach into
+  // are the ones its neighbours in the same L2 have just read.
+  const unsigned blk = (blockIdx.x % 8u) * (gridDim.x / 8u) + blockIdx.x / 8u;
+  const long long w = (long long)blk * blockDim.x + threadIdx.x;
   if (w >= nWords)
     return;
   unsigned long long res = 0;
@@ -653,6 +661,8 @@ __global__ void __launch_bounds__(256)
       return;
     }
     blk -= 1;
+  } else {
+    blk = xcd_contiguous_block((count_now(nSites) + rowsPerBlock - 1) / rowsPerBlock);
   }
   if (outMeta[META_OVERFLOW])
     return;
@@ -1064,7 +1074,7 @@ __global__ void k_grid_index(GridView g, const long long *ekey, const int *erow,
 // the rows by rank from the entry list
 __global__ void k_rank_rows(GridView g, const long long *ekey, const int *erow,
                             Count n, const long long *meta, int *rankRow) {
-  long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  long long e = xcd_contiguous_block((count_now(n) + 255) / 256) * blockDim.x + threadIdx.x;
   if (e >= n.bound || (meta && meta[META_OVERFLOW]) || e >= count_now(n))
     return;
   rankRow[rank_of(g, ekey[e])] = erow[e];
@@ -1121,7 +1131,7 @@ static int ensure_rank(scn_ctx *ctx, scn_grids *g) {
   if (!g->rankRowValid) {
     SCN_TRY(g->rankRow.reserve((size_t)g->nActive + 4));
     if (g->nActive > 0) {
-      hipLaunchKernelGGL(k_rank_rows, dim3(scn_ceil_div(g->nActive, 256)),
+      hipLaunchKernelGGL(k_rank_rows, dim3(xcd_grid(scn_ceil_div(g->nActive, 256))),
                          dim3(256), 0, ctx->stream, view_of(g), g->ekey.p,
                          g->erow.p, count_active(g),
                          g->pending ? g->meta.p : nullptr, g->rankRow.p);
@@ -1467,7 +1477,7 @@ static int plan_regions_d(scn_ctx *ctx, scn_grids *in, scn_grids *out,
     SCN_TRY(out->rankOf.reserve((size_t)nE + 2));
   }
   if (nE > 0) {
-    hipLaunchKernelGGL(k_plan_count<D>, dim3(scn_ceil_div(nE, 256)), dim3(256),
+    hipLaunchKernelGGL(k_plan_count<D>, dim3(xcd_grid(scn_ceil_div(nE, 256))), dim3(256),
                        0, ctx->stream, vin, g, in->ekey.p, nEc, inMeta, out->cnt.p,
                        masked ? out->ownMask.p : nullptr, out->rankOf.p);
     SCN_HIP_CHECK(hipGetLastError());
@@ -1512,14 +1522,15 @@ static int plan_regions_d(scn_ctx *ctx, scn_grids *in, scn_grids *out,
   GridView vout = view_of(out);
   if (g.mode == MODE_SQ_NOMIN && g.size <= 64) {
     const long long words = (long long)out->nWords + 2;
-    hipLaunchKernelGGL(k_mask_dilate<D>, dim3(scn_ceil_div(words, 256)), dim3(256),
+    const long long blocks = (scn_ceil_div(words, 256) + 7) / 8 * 8; // whole rounds of the 8 XCDs
+    hipLaunchKernelGGL(k_mask_dilate<D>, dim3((unsigned)blocks), dim3(256),
                        0, ctx->stream, vin, g, out->bits.p, words,
                        (long long)in->batch * g.volOut);
     SCN_HIP_CHECK(hipGetLastError());
     vout.bits = nullptr;
   }
   if (nThreads > 0 && masked && maxCand > 9) {
-    hipLaunchKernelGGL(k_plan_emit_walk<D>, dim3(scn_ceil_div(nThreads, 256)),
+    hipLaunchKernelGGL(k_plan_emit_walk<D>, dim3(xcd_grid(scn_ceil_div(nThreads, 256))),
                        dim3(256), 0, ctx->stream, vin, vout, g,
                        in->ekey.p, nEc, out->meta.p, out->base.p, out->ownMask.p,
                        out->rankOf.p, out->bgBefore.p, out->bg.p, out->ekey.p,
@@ -1527,14 +1538,14 @@ static int plan_regions_d(scn_ctx *ctx, scn_grids *in, scn_grids *out,
     SCN_HIP_CHECK(hipGetLastError());
   } else if (nThreads > 0 && masked) {
     hipLaunchKernelGGL(k_plan_emit_masked<D>,
-                       dim3(scn_ceil_div(nThreads, 256), (unsigned)maxCand),
+                       dim3(xcd_grid(scn_ceil_div(nThreads, 256)), (unsigned)maxCand),
                        dim3(256), 0, ctx->stream, vin, vout, g,
                        in->ekey.p, nEc, out->meta.p, out->base.p, out->ownMask.p,
                        out->rankOf.p, out->bgBefore.p, out->bg.p, out->ekey.p,
                        out->erow.p, out->siteKey.p);
     SCN_HIP_CHECK(hipGetLastError());
   } else if (nThreads > 0) {
-    hipLaunchKernelGGL(k_plan_emit<D>, dim3(scn_ceil_div(nThreads, 256)),
+    hipLaunchKernelGGL(k_plan_emit<D>, dim3(xcd_grid(scn_ceil_div(nThreads, 256))),
                        dim3(256), 0, ctx->stream, vin, vout, g,
                        in->ekey.p, nEc, out->meta.p, out->base.p, out->bgBefore.p,
                        out->bg.p,
@@ -1898,7 +1909,8 @@ extern "C" int scn_rules_fill(scn_ctx *ctx, const scn_grids *in,
     const int pitch = g.width | 1;
     const unsigned magicWidth = (unsigned)((1ull << 32) / (unsigned)g.width + 1);
     const unsigned magicSize = (unsigned)((1ull << 32) / (unsigned)g.size + 1);
-    dim3 runs(scn_ceil_div(out->nSites, rowsPerBlock) + extra);
+    dim3 runs(extra ? (unsigned)scn_ceil_div(out->nSites, rowsPerBlock) + extra
+                    : xcd_grid(scn_ceil_div(out->nSites, rowsPerBlock)));
 #define SCN_FILL_RUNS(D, SC)                                                   \
   if (g.size == 2)                                                             \
     hipLaunchKernelGGL((k_rules_fill_runs<D, SC, 2>), runs, block, 0,          \

@@ -60,6 +60,23 @@ __device__ __forceinline__ long long count_now(const Count &c) {
   const long long v = *c.live;
   return v < c.bound ? v : c.bound;
 }
+// The block a workgroup stands for.  Workgroups are dealt to the 8 XCDs
+// round-robin and every XCD has an L2 of its own; the kernels that walk
+// entries or rows in key order read, for each, the mask rows and rank rows of
+// its neighbourhood, which their neighbours in the walk read too.  So the
+// first nLive blocks (those that hold real work, rounded up to whole rounds of
+// the XCDs) are dealt out so that each XCD takes one contiguous eighth of
+// them; the rest keep their own number.  A permutation of the grid, which must
+// be a multiple of 8 blocks.
+__device__ __forceinline__ long long xcd_contiguous_block(long long nLive) {
+  const long long b = blockIdx.x;
+  const long long per = (nLive + 7) / 8;
+  return b < 8 * per ? (b % 8) * per + b / 8 : b;
+}
+// (host side: the grid such kernels are launched with)
+static inline unsigned xcd_grid(long long blocks) {
+  return (unsigned)((blocks + 7) / 8 * 8);
+}
 // per-grids device record
 enum { META_SITES = 0, META_ACTIVE = 1, META_OVERFLOW = 2, META_WIDTH = 3 };
 
