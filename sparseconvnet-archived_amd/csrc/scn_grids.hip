@@ -428,12 +428,9 @@ template <int D>
 __global__ void __launch_bounds__(256)
     k_mask_dilate(GridView in, Geom g, unsigned long long *outBits,
                   long long nWords, long long totalBits) {
-  // Workgroups are dealt to the 8 XCDs round-robin and every XCD has an L2 of
-  // its own: each XCD takes one contiguous eighth of the words (the grid is a
-  // multiple of 8), so that the rows and planes a word's windows reach into
-  // are the ones its neighbours in the same L2 have just read.
-  const unsigned blk = (blockIdx.x % 8u) * (gridDim.x / 8u) + blockIdx.x / 8u;
-  const long long w = (long long)blk * blockDim.x + threadIdx.x;
+  // (runs of blocks to one XCD: the rows and planes a word's windows reach into
+  // are the ones its neighbours in the same L2 have just read)
+  const long long w = xcd_contiguous_block((nWords + 255) / 256) * blockDim.x + threadIdx.x;
   if (w >= nWords)
     return;
   unsigned long long res = 0;

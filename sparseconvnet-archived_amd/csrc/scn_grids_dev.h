@@ -64,14 +64,20 @@ __device__ __forceinline__ long long count_now(const Count &c) {
 // round-robin and every XCD has an L2 of its own; the kernels that walk
 // entries or rows in key order read, for each, the mask rows and rank rows of
 // its neighbourhood, which their neighbours in the walk read too.  So the
-// first nLive blocks (those that hold real work, rounded up to whole rounds of
-// the XCDs) are dealt out so that each XCD takes one contiguous eighth of
-// them; the rest keep their own number.  A permutation of the grid, which must
+// blocks that hold real work (the first nLive) are dealt out in runs of
+// XCD_RUN consecutive blocks to one XCD, run after run round the XCDs: the
+// neighbours meet in one L2, and what the eight XCDs write at any moment still
+// lies close together.  The last, incomplete round of runs and the blocks
+// without work keep their own numbers.  A permutation of the grid, which must
 // be a multiple of 8 blocks.
+#define XCD_RUN 32
 __device__ __forceinline__ long long xcd_contiguous_block(long long nLive) {
   const long long b = blockIdx.x;
-  const long long per = (nLive + 7) / 8;
-  return b < 8 * per ? (b % 8) * per + b / 8 : b;
+  const long long whole = nLive / (8 * XCD_RUN) * (8 * XCD_RUN);
+  if (b >= whole)
+    return b;
+  const long long turn = b / 8, xcd = b % 8;
+  return ((turn / XCD_RUN) * 8 + xcd) * XCD_RUN + turn % XCD_RUN;
 }
 // (host side: the grid such kernels are launched with)
 static inline unsigned xcd_grid(long long blocks) {
