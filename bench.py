@@ -69,9 +69,10 @@ def parse():
                          "reported beside the headline figure (0 disables it)")
     ap.add_argument("--from-host", action="store_true",
                     help="also time processDataset() on host-resident Pictures (CPU codify + PCIe upload included)")
-    ap.add_argument("--producers", type=int, default=5,
+    ap.add_argument("--producers", type=int, default=10,
                     help="batch-producer threads building grids and rule books ahead of the forward pass (the "
-                         "reference's nBatchProducerThreads); they share at most five streams")
+                         "reference's nBatchProducerThreads, 10 by default there too); they share at most five "
+                         "streams")
     ap.add_argument("--producer-streams", type=int, default=-1,
                     help="how many of those streams take part (SparseConvNetCUDA::setProducerStreams; 0: all).  HIP "
                          "spreads streams over 4 hardware queues and kernels of streams that share a queue run in "
@@ -369,18 +370,22 @@ def main():
     if args.from_host:
         # the reference's own entry point: Pictures in host memory, codifyInputData on the producer threads, input
         # sites and features uploaded over PCIe for every batch
-        reps = max(2, min(args.steps, 20))
+        reps = max(2, min(3 * args.steps, 60))  # enough batches for the pass to outweigh its fill and drain
         ds = hostapi.Dataset(cfg.name, cfg.nInputFeatures, max(cfg.nClasses, 1), hostapi.TESTBATCH)
         for _ in range(reps):
             for pts, f, label in samples:
                 ds.add_points(cfg.dimension, cfg.lattice, pts, f, label)
         if net.layers()[-1]["act"] == synthetic.SOFTMAX:
+            streams = net.producerStreamsInUse()
+            net.setProducerStreams(0)  # production is the longer half here: every stream
             net.processDataset(ds, B)  # warm-up pass (buffers grow)
             t0 = time.perf_counter()
             net.processDataset(ds, B)
             dth = time.perf_counter() - t0
+            net.setProducerStreams(streams)
             from_host = {"ms_per_batch": 1e3 * dth / reps, "active_sites_per_s": active * reps / dth,
                          "samples_per_s": B * reps / dth, "batches": reps,
+                         "producer_streams_in_use": min(5, max(1, args.producers)),
                          "note": "processDataset on host Pictures: CPU codify + H2D of sites and features included"}
         ds.close()
 

@@ -32,6 +32,22 @@ struct BatchResultStage {
   BatchResultStage &operator=(const BatchResultStage &) = delete;
 };
 
+// Pinned host memory that only grows: what a batch slot flattens its input
+// grids into before it borrows a stream, so that the upload is four queued
+// copies and the stream is not held while the CPU walks the grids.
+struct PinnedStage {
+  void *p;
+  size_t bytes;
+  PinnedStage() : p(nullptr), bytes(0) {}
+  PinnedStage(PinnedStage &&o) : p(o.p), bytes(o.bytes) { o.p = nullptr, o.bytes = 0; }
+  PinnedStage(const PinnedStage &) = delete;
+  PinnedStage &operator=(const PinnedStage &) = delete;
+  ~PinnedStage();
+  // at least n bytes (the contents are not kept)
+  void reserve(size_t n);
+  template <typename T> T *as() { return static_cast<T *>(p); }
+};
+
 class SpatiallySparseBatch {
   SpatiallySparseBatchSubInterface *inputSub;
 
@@ -56,6 +72,12 @@ public:
   // device staging of the input sites (sample, key as two ints, row,
   // backgroundCol), reused from batch to batch
   vectorCUDA<int> stagingSample, stagingKey, stagingRow, stagingBackground;
+  // the same four arrays on the host, pinned, and how many sites they hold
+  PinnedStage hostSample, hostKey, hostRow, hostBackground;
+  size_t hostSites;
+  // ... and the input features, moved there from the interface's host vector
+  PinnedStage hostFeatures;
+  size_t hostFeatureCount;
   std::unique_ptr<BatchResultStage> result;
   void reset();
 };

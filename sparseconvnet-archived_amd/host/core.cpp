@@ -361,12 +361,27 @@ BatchResultStage::~BatchResultStage() {
     scn_host_free(scnDefaultContext(), pinned);
 }
 
+PinnedStage::~PinnedStage() {
+  if (p)
+    scn_host_free(scnDefaultContext(), p);
+}
+void PinnedStage::reserve(size_t n) {
+  if (n <= bytes)
+    return;
+  if (p)
+    SCN_CHECKED(scn_host_free(scnDefaultContext(), p));
+  p = nullptr;
+  bytes = n + n / 2 + 4096; // (pinning is slow: with room to grow)
+  SCN_CHECKED(scn_host_alloc(scnDefaultContext(), bytes, &p));
+}
+
 SpatiallySparseBatch::SpatiallySparseBatch(
     SpatiallySparseBatchSubInterface *inputSub)
     : inputSub(inputSub), preprocessStream(nullptr), forwardStream(nullptr),
       labels(false, 0),
       stagingSample(true, 0), stagingKey(true, 0), stagingRow(true, 0),
-      stagingBackground(true, 0), result(new BatchResultStage()) {
+      stagingBackground(true, 0), hostSites(0), hostFeatureCount(0),
+      result(new BatchResultStage()) {
   interfaces.emplace_back(inputSub);
   reset();
 }

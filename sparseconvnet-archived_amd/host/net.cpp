@@ -1,4 +1,5 @@
 // Net runtime, batch production, public facades and canned architectures.
+#include <cstring>
 #include <algorithm>
 #include <atomic>
 #include <cassert>
@@ -843,6 +844,36 @@ void BatchProducer::preprocessBatch(int c, int cc, RNG &rng) {
     for (size_t i = 0; i < features.size(); ++i)
       features[i] *= cnn.inputNormalizingConstants[i % in.nFeatures];
   }
+  // The grids as the four arrays scn_grids_build takes, and the features, in
+  // the slot's pinned staging: still on the CPU's time, no stream is held yet,
+  // and the upload is then five queued copies.
+  size_t n = 0;
+  for (auto &g : in.grids)
+    n += g.mp.size();
+  b.hostSample.reserve(n * sizeof(int32_t));
+  b.hostKey.reserve(n * sizeof(int64_t));
+  b.hostRow.reserve(n * sizeof(int32_t));
+  b.hostBackground.reserve((size_t)b.batchSize * sizeof(int32_t));
+  int32_t *sample = b.hostSample.as<int32_t>(), *row = b.hostRow.as<int32_t>(),
+          *bg = b.hostBackground.as<int32_t>();
+  int64_t *key = b.hostKey.as<int64_t>();
+  size_t at = 0;
+  for (int item = 0; item < b.batchSize; ++item) {
+    bg[item] = in.grids[item].backgroundCol;
+    for (auto &e : in.grids[item].mp.entries()) {
+      sample[at] = item;
+      key[at] = e.first;
+      row[at] = e.second;
+      ++at;
+    }
+  }
+  b.hostSites = n;
+  std::vector<float> &features = in.sub->features.hVector();
+  b.hostFeatureCount = features.size();
+  b.hostFeatures.reserve(features.size() * sizeof(float));
+  if (!features.empty())
+    std::memcpy(b.hostFeatures.p, features.data(), features.size() * sizeof(float));
+  features.clear();
 }
 // GPU half: the input grids go to HBM, then every layer builds its rule book,
 // all on the slot's stream
@@ -851,30 +882,17 @@ void BatchProducer::preprocessBatchOnDevice(int cc) {
   SpatiallySparseBatchInterface &in = b.interfaces[0];
   cudaMemStream &ms = b.preprocessStream ? *b.preprocessStream : cnn.memStream;
   scn_ctx *ctx = ms.ctx;
-  std::vector<int32_t> sample, row, bg;
-  std::vector<int64_t> key;
-  size_t n = 0;
-  for (auto &g : in.grids)
-    n += g.mp.size();
-  sample.reserve(n);
-  row.reserve(n);
-  key.reserve(n);
-  for (int item = 0; item < b.batchSize; ++item) {
-    bg.push_back(in.grids[item].backgroundCol);
-    for (auto &e : in.grids[item].mp.entries()) {
-      sample.push_back(item);
-      key.push_back(e.first);
-      row.push_back(e.second);
-    }
-  }
+  // (flattened into pinned memory by preprocessBatch)
+  const size_t n = b.hostSites;
   b.stagingSample.resize64(n);
   b.stagingKey.resize64(2 * n);
   b.stagingRow.resize64(n);
-  b.stagingBackground.resize64(bg.size());
-  SCN_CHECKED(scn_h2d(ctx, b.stagingSample.dPtr(), sample.data(), n * 4));
-  SCN_CHECKED(scn_h2d(ctx, b.stagingKey.dPtr(), key.data(), n * 8));
-  SCN_CHECKED(scn_h2d(ctx, b.stagingRow.dPtr(), row.data(), n * 4));
-  SCN_CHECKED(scn_h2d(ctx, b.stagingBackground.dPtr(), bg.data(), bg.size() * 4));
+  b.stagingBackground.resize64((size_t)b.batchSize);
+  SCN_CHECKED(scn_h2d_async(ctx, b.stagingSample.dPtr(), b.hostSample.p, n * 4));
+  SCN_CHECKED(scn_h2d_async(ctx, b.stagingKey.dPtr(), b.hostKey.p, n * 8));
+  SCN_CHECKED(scn_h2d_async(ctx, b.stagingRow.dPtr(), b.hostRow.p, n * 4));
+  SCN_CHECKED(scn_h2d_async(ctx, b.stagingBackground.dPtr(), b.hostBackground.p,
+                            (size_t)b.batchSize * 4));
   if (!in.deviceGrids) {
     SCN_CHECKED(scn_grids_create(ctx, &in.deviceGrids));
     in.ownsDeviceGrids = true;
@@ -886,7 +904,10 @@ void BatchProducer::preprocessBatchOnDevice(int cc) {
                               (const int64_t *)b.stagingKey.dPtr(),
                               b.stagingRow.dPtr(), (int64_t)n,
                               b.stagingBackground.dPtr(), in.nSpatialSites));
-  in.sub->features.copyToGPUAsync(ms);
+  in.sub->features.copyToGPU(); // (its host vector is empty: nothing moves)
+  in.sub->features.resize64(b.hostFeatureCount);
+  SCN_CHECKED(scn_h2d_async(ctx, in.sub->features.dPtr(), b.hostFeatures.p,
+                            b.hostFeatureCount * sizeof(float)));
   if (b.type == TRAINBATCH) {
     // the classifier's gradient reads the labels on the device: uploaded here,
     // on this slot's stream, so that the net's stream is never waited for
