@@ -40,14 +40,15 @@ TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic_bench.json")
 
 
 def measured_traffic():
-    """{(workload, kernel family, layer): bytes per launch}, the commit of the measurement (or {} and None)."""
+    """{(workload, kernel family, layer): bytes per launch}, the commit of the measurement and the digest of the
+    kernel sources it was made with (or {}, None, None)."""
     try:
         with open(TRAFFIC_FILE) as f:
             t = json.load(f)
     except (OSError, ValueError):
-        return {}, None
+        return {}, None, None
     table = {(e["workload"], e["kernel"], e["layer"]): e["read_bytes"] + e["written_bytes"] for e in t["entries"]}
-    return table, t.get("measured_at_commit")
+    return table, t.get("measured_at_commit"), t.get("csrc_sha256")
 
 
 def parse():
@@ -79,6 +80,14 @@ def parse():
                          "order: with two forward lanes, two producer streams leave every stream a queue of its "
                          "own.  Default: 2 for the configs whose forward pass is the longer half (2, 4, 5), all "
                          "for those that wait for their batches (1, 3)")
+    ap.add_argument("--regions", type=int, default=5,
+                    help="timed regions of --steps batches each; value is their median (min and max beside it)")
+    ap.add_argument("--other-configs", default="1,3,4,5,4:bf16,5:bf16",
+                    help="configurations (number[:precision]) given a short pass each after the headline one, "
+                         "reported under other_configs; empty: none")
+    ap.add_argument("--other-steps", type=int, default=20, help="timed batches per region of those passes (at most)")
+    ap.add_argument("--other-seconds", type=float, default=150.0,
+                    help="no further one of those passes is started after this many seconds")
     ap.add_argument("--train", action="store_true",
                     help="time training batches instead (forward, backward pass, momentum step; Pictures on the host, "
                          "processDataset on a TRAINBATCH dataset): an auxiliary line, not the headline metric")
@@ -124,39 +133,48 @@ def algorithmic_work(layers, ifaces, batch, precision):
     return work
 
 
-def main():
-    args = parse()
-    if args.gpus != 1:
-        print("bench.py: this build measures one GPU; --gpus %d is not supported (the forward path shards by sample "
-              "with no exchange between the GPUs)" % args.gpus, file=sys.stderr)
-        sys.exit(2)
-    # the host classes announce every layer on stdout like the reference does;
-    # keep stdout for the one JSON line and send that chatter to stderr
-    sys.stdout.flush()
-    saved_stdout = os.dup(1)
-    os.dup2(2, 1)
-    from __graft_entry__ import load_package
-    scn = load_package()
-    from sparseconvnet_archived_amd import hostapi, synthetic
+def csrc_digest():
+    """sha256 over the sources of libscn_hip.so (names and contents, sorted): what the byte counters were read for."""
+    import hashlib
+    h = hashlib.sha256()
+    d = os.path.join(ROOT, "sparseconvnet-archived_amd", "csrc")
+    for name in sorted(os.listdir(d)):
+        if name.endswith((".hip", ".h")) or name == "Makefile":
+            h.update(name.encode())
+            with open(os.path.join(d, name), "rb") as f:
+                h.update(f.read())
+    return h.hexdigest()
 
-    cfg = synthetic.config(args.config, batch=args.batch)
+
+def timed_regions(run, regions):
+    """`regions` timed regions one after the other -> (median, min, max, all) of the seconds each took"""
+    secs = [run() for _ in range(max(1, regions))]
+    return float(np.median(secs)), float(min(secs)), float(max(secs)), secs
+
+
+def measure(scn, hostapi, synthetic, args, number, precision, headline):
+    """One configuration through the pipeline bench.py times.  headline: everything the one JSON line carries for its
+    own workload; otherwise a short pass -- throughput with resident and with uploaded inputs, the dominant entry
+    and the NiN roofline."""
+    cfg = synthetic.config(number, batch=args.batch if headline else None)
     B = cfg.batch
-    net = hostapi.Net(cfg.dimension, cfg.nInputFeatures, max(cfg.nClasses, 1), threads=max(1, args.producers))
-    if args.producer_streams < 0:
-        args.producer_streams = 2 if args.config in (2, 4, 5) and not args.train else 0
-    net.setProducerStreams(args.producer_streams)
+    producers = max(1, args.producers)
+    steps = args.steps if headline else max(1, min(args.steps, args.other_steps))
+    warmup = args.warmup if headline else min(args.warmup, 5)
+    net = hostapi.Net(cfg.dimension, cfg.nInputFeatures, max(cfg.nClasses, 1), threads=producers)
+    streams = args.producer_streams
+    if streams < 0 or not headline:
+        streams = 2 if number in (2, 4, 5) else 0
+    net.setProducerStreams(streams)
     cfg.build(net)
     net.setFusedConvolutions(bool(args.fused))
-    if args.precision != "fp32":
-        net.setPrecision(scn.BF16 if args.precision == "bf16" else scn.BF16X3)
+    if precision != "fp32":
+        net.setPrecision(scn.BF16 if precision == "bf16" else scn.BF16X3)
     layers = net.layers()
     weights = synthetic.he_normal_weights(layers, args.seed + 1)
     for i, (W, Bv, pr) in weights.items():
         net.set_weights(i, W, Bv, pr)
     samples = synthetic.make_samples(cfg, args.seed)
-    if args.train:
-        train_leg(args, cfg, net, hostapi, samples, saved_stdout)
-        return
     S, K, R, bg, feats, nSites = synthetic.codify(samples, cfg.dimension, cfg.lattice, net.inputSpatialSize,
                                                   cfg.nInputFeatures)
     active = int(len(K))
@@ -167,7 +185,7 @@ def main():
     def step():
         net.forward_resident(B, dS.ptr, dK.ptr, dR.ptr, dBg.ptr, active, nSites, dF.ptr, probs)
 
-    if args.calibration_copy_mb > 0:
+    if headline and args.calibration_copy_mb > 0:
         # rows of 64 floats copied through the gather kernel with rules 0..n-1:
         # reads n*256 + n*4 bytes, writes n*256 bytes
         n_rows = args.calibration_copy_mb * (1 << 20) // 256
@@ -190,27 +208,47 @@ def main():
     hS, hK, hR, hBg, hF = (pinned(np.ascontiguousarray(x)) for x in
                            (S.astype(np.int32), K.astype(np.int64), R.astype(np.int32), bg.astype(np.int32),
                             feats.astype(np.float32)))
-    # warm-up and timed batches the way processDataset runs them, in ONE pass: producer threads build grids and
-    # rule books on their own streams while this thread runs the forward pass of the previous batch; the clock
-    # starts when the last warm-up batch is finished and the net's stream is idle, and the producers meanwhile
-    # hold the next batches ready, as in the middle of any dataset pass
+    # Warm-up, timed and tail batches the way processDataset runs them, in ONE pass: producer threads build grids and
+    # rule books on their own streams while the forward lanes run the batches before.  The clock starts when the last
+    # warm-up batch is finished and the forward streams are idle, and stops when the last timed batch's probabilities
+    # are on the host; `producers` more batches follow untimed, so the producers hold finished batches ready at both
+    # ends of the window and have to rebuild during it what the window consumes -- the middle of a long pass.
     # (set-up, before the warm-up: every batch slot's first batch is planned layer by layer and sizes the slot's
     # buffers, its second sizes the staging area of the recorded plans -- three batches per slot leave nothing to
     # allocate)
-    priming = 3 * max(1, args.producers)
+    priming = 3 * producers
     net.forward_stream_timed(0, priming, B, dS.ptr, dK.ptr, dR.ptr, dBg.ptr, active, nSites, dF.ptr,
                              inputs_on_host=False, h_probs=probs)
-    dt = net.forward_stream_timed(args.warmup, args.steps, B, dS.ptr, dK.ptr, dR.ptr, dBg.ptr, active, nSites, dF.ptr,
-                                  inputs_on_host=False, h_probs=probs)
+    net.setStreamTail(producers)
+    ready = []
+
+    def resident_region():
+        dt = net.forward_stream_timed(warmup, steps, B, dS.ptr, dK.ptr, dR.ptr, dBg.ptr, active, nSites, dF.ptr,
+                                      inputs_on_host=False, h_probs=probs)
+        ready.append(net.streamReadyAtStart())
+        return dt
+
+    def upload_region():
+        return net.forward_stream_timed(warmup, steps, B, hS.ptr, hK.ptr, hR.ptr, hBg.ptr, active, nSites, hF.ptr,
+                                        inputs_on_host=True, h_probs=probs)
+
+    regions = args.regions if headline else min(args.regions, 3)
+    dt, dt_min, dt_max, dt_all = timed_regions(resident_region, regions)
     ctx.sync()
-    ms_per_step = 1e3 * dt / args.steps
-    dt_up = net.forward_stream_timed(args.warmup, args.steps, B, hS.ptr, hK.ptr, hR.ptr, hBg.ptr, active, nSites,
-                                     hF.ptr, inputs_on_host=True, h_probs=probs)
+    ms_per_step = 1e3 * dt / steps
+    up, up_min, up_max, up_all = timed_regions(upload_region, regions)
     ctx.sync()
     upload_bytes = int(S.size * 4 + K.size * 8 + R.size * 4 + bg.size * 4 + feats.size * 4)
+    with_upload = {"active_sites_per_s": active * steps / up, "samples_per_s": B * steps / up,
+                   "ms_per_step": 1e3 * up / steps,
+                   "ms_per_step_min_max": [1e3 * up_min / steps, 1e3 * up_max / steps],
+                   "bytes_uploaded_per_step": upload_bytes,
+                   "note": "sites and features in pinned host memory, uploaded on the producer streams for every "
+                           "batch: forward time = rule build + H2D of inputs + all layer kernels + D2H of the "
+                           "probabilities (BatchProducer.cu:127-134 inside the clock of SparseConvNetCUDA.cu:277-324)"}
     # the same pass over several different batches taken in turn
     varied = None
-    if args.distinct_batches > 1:
+    if headline and args.distinct_batches > 1:
         keep, descr, actives = [], [], []
         for i in range(args.distinct_batches):
             Si, Ki, Ri, bgi, fi, ni = synthetic.codify(synthetic.make_samples(cfg, args.seed + 100 + i), cfg.dimension,
@@ -220,25 +258,30 @@ def main():
             keep.append(arrs)
             descr.append((B, arrs[0].ptr, arrs[1].ptr, arrs[2].ptr, arrs[3].ptr, int(len(Ki)), int(ni), arrs[4].ptr))
             actives.append(int(len(Ki)))
+        net.setStreamTail(0)
         net.forward_stream_timed_many(0, priming + args.distinct_batches, descr, h_probs=probs)
-        dt_var = net.forward_stream_timed_many(args.warmup, args.steps, descr, h_probs=probs)
+        net.setStreamTail(producers)
+        dv, dv_min, dv_max, _ = timed_regions(
+            lambda: net.forward_stream_timed_many(warmup, steps, descr, h_probs=probs), regions)
         ctx.sync()
-        timed_sites = sum(actives[(args.warmup + i) % len(actives)] for i in range(args.steps))
-        varied = {"distinct_batches": args.distinct_batches, "ms_per_step": 1e3 * dt_var / args.steps,
-                  "active_sites_per_s": timed_sites / dt_var, "samples_per_s": B * args.steps / dt_var,
+        timed_sites = sum(actives[(warmup + i) % len(actives)] for i in range(steps))
+        varied = {"distinct_batches": args.distinct_batches, "ms_per_step": 1e3 * dv / steps,
+                  "ms_per_step_min_max": [1e3 * dv_min / steps, 1e3 * dv_max / steps],
+                  "active_sites_per_s": timed_sites / dv, "samples_per_s": B * steps / dv,
                   "active_sites_min_max": [min(actives), max(actives)],
                   "note": "different batches in turn (seeds %d..%d), inputs resident" % (args.seed + 100,
                                                                                         args.seed + 99 + len(actives))}
         del keep
+    net.setStreamTail(0)
     # one batch at a time on one stream, nothing overlapped: the latency of a batch
     for _ in range(3):
         step()
     ctx.sync()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         step()
     ctx.sync()
-    ms_latency = 1e3 * (time.perf_counter() - t0) / args.steps
+    ms_latency = 1e3 * (time.perf_counter() - t0) / steps
     mac = hostapi.take_multiply_add_count()  # resets the counter
     step()
     mac = hostapi.take_multiply_add_count()
@@ -249,7 +292,7 @@ def main():
         info = net.interface(i, want_features=False)
         ifaces.append(dict(rows=info["nSpatialSites"], nFeatures=info["nFeatures"], nRules=int(info["rules"].size),
                            gridEntries=int(info["grids"][0].size)))
-    work = algorithmic_work(layers, ifaces, B, args.precision)
+    work = algorithmic_work(layers, ifaces, B, precision)
 
     # per-kernel durations: HIP events on the library's stream, same steps again
     ctx.prof_reset()
@@ -267,7 +310,7 @@ def main():
     span_floor_ms = float(np.median(bare))
     span_idle_kernel_ms = float(np.median(idle))
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         step()
     ctx.sync()
     dt_prof = time.perf_counter() - t0
@@ -281,9 +324,9 @@ def main():
     kernels = []
     for key, ms_total in tot.items():
         fam, tag = key
-        ms = ms_total / args.steps
+        ms = ms_total / steps
         byts, flops = work.get(key, (0, 0))
-        entry = dict(kernel=fam, layer=tag, ms_per_step=round(ms, 5), launches_per_step=cnt[key] / args.steps)
+        entry = dict(kernel=fam, layer=tag, ms_per_step=round(ms, 5), launches_per_step=cnt[key] / steps)
         if fam in ("gather", "nin", "conv_nin", "maxpool", "terminal", "softmax"):
             # one kernel per span: take off what the two events cost around nothing
             ms = max(ms - span_floor_ms * entry["launches_per_step"], 1e-6)
@@ -292,9 +335,9 @@ def main():
             K_, N_ = layers[tag]["nIn"], layers[tag]["nOut"]
             intensity = flops / max(byts, 1)
             entry["shape"] = [ifaces[tag + 1]["rows"], K_, N_]
-            if intensity >= BALANCE_FLOP_PER_BYTE[args.precision]:
+            if intensity >= BALANCE_FLOP_PER_BYTE[precision]:
                 a = flops / (ms * 1e-3) / 1e12
-                entry.update(bound="mfma", achieved=a, peak=MFMA_PEAK_TFLOPS[args.precision], unit="TFLOP/s")
+                entry.update(bound="mfma", achieved=a, peak=MFMA_PEAK_TFLOPS[precision], unit="TFLOP/s")
             else:
                 a = byts / (ms * 1e-3) / 1e9
                 entry.update(bound="hbm", achieved=a, peak=HBM_PEAK_GBS, unit="GB/s")
@@ -334,8 +377,14 @@ def main():
         else:
             rules_entry["note"] = ("layer by layer through masks, rank prefixes and rows by rank in HBM: a dozen "
                                    "launches per layer; the rule rows themselves leave at 4-6 TB/s")
-    traffic_table, traffic_commit = measured_traffic()
-    default_input = args.batch is None and args.seed == 2015 and args.precision == "fp32" and args.fused == 1
+    traffic_table, traffic_commit, traffic_digest = measured_traffic()
+    default_input = args.seed == 2015 and precision == "fp32" and args.fused == 1 and (not headline or args.batch is None)
+    traffic_note = None
+    if traffic_table and traffic_digest != csrc_digest():
+        # the byte counters were read for other kernels than the ones that ran just now
+        traffic_table = {}
+        traffic_note = ("the kernel sources have changed since the byte counters in profiles/hbm_traffic_bench.json "
+                        "were read (commit %s): no traffic figure is printed" % traffic_commit)
     fused_layers = {e["layer"] for e in kernels if e["kernel"] == "conv_nin"}
     for e in kernels:
         e["traffic"] = traffic_table.get((cfg.name, e["kernel"], e["layer"])) if default_input else None
@@ -364,28 +413,46 @@ def main():
     if roofline_nin and nin_ms > 0:
         roofline_nin["all_mfma_bound_layers"] = dict(
             layers=sorted(e["layer"] for e in nin_only), tflops=round(nin_flops / (nin_ms * 1e-3) / 1e12, 2),
-            frac=round(nin_flops / (nin_ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS[args.precision], 4))
+            frac=round(nin_flops / (nin_ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS[precision], 4),
+            per_layer_frac={str(e["layer"]): e["frac"] for e in sorted(nin_only, key=lambda e: e["layer"])})
+    pools = [e for e in single if e["kernel"] == "maxpool"]
+    roofline_pool = as_roofline(max(pools, key=lambda e: e["ms_kernel"])) if pools else None
+
+    if not headline:
+        net.close()
+        return {"workload": cfg.name, "batch": B, "precision": precision, "active_sites": active,
+                "steps": steps, "warmup": warmup, "regions": regions,
+                "ms_per_step": ms_per_step, "ms_per_step_min_max": [1e3 * dt_min / steps, 1e3 * dt_max / steps],
+                "active_sites_per_s": active * steps / dt, "samples_per_s": B * steps / dt,
+                "with_input_upload": {k: with_upload[k] for k in ("ms_per_step", "ms_per_step_min_max",
+                                                                  "active_sites_per_s", "samples_per_s")},
+                "batches_ready_at_t0": ready, "producer_streams_in_use": net_streams(streams, producers),
+                "ms_single_batch_latency": ms_latency, "roofline": roofline, "roofline_nin": roofline_nin,
+                "roofline_maxpool": roofline_pool,
+                "rules": None if not rules_entry else {k: rules_entry[k] for k in
+                                                       ("ms_kernel", "launches_per_step", "achieved", "frac",
+                                                        "algorithmic_bytes", "traffic")}}
 
     from_host = None
     if args.from_host:
         # the reference's own entry point: Pictures in host memory, codifyInputData on the producer threads, input
         # sites and features uploaded over PCIe for every batch
-        reps = max(2, min(3 * args.steps, 60))  # enough batches for the pass to outweigh its fill and drain
+        reps = max(2, min(3 * steps, 60))  # enough batches for the pass to outweigh its fill and drain
         ds = hostapi.Dataset(cfg.name, cfg.nInputFeatures, max(cfg.nClasses, 1), hostapi.TESTBATCH)
         for _ in range(reps):
             for pts, f, label in samples:
                 ds.add_points(cfg.dimension, cfg.lattice, pts, f, label)
         if net.layers()[-1]["act"] == synthetic.SOFTMAX:
-            streams = net.producerStreamsInUse()
+            inUse = net.producerStreamsInUse()
             net.setProducerStreams(0)  # production is the longer half here: every stream
             net.processDataset(ds, B)  # warm-up pass (buffers grow)
             t0 = time.perf_counter()
             net.processDataset(ds, B)
             dth = time.perf_counter() - t0
-            net.setProducerStreams(streams)
+            net.setProducerStreams(inUse)
             from_host = {"ms_per_batch": 1e3 * dth / reps, "active_sites_per_s": active * reps / dth,
                          "samples_per_s": B * reps / dth, "batches": reps,
-                         "producer_streams_in_use": min(5, max(1, args.producers)),
+                         "producer_streams_in_use": min(5, producers),
                          "note": "processDataset on host Pictures: CPU codify + H2D of sites and features included"}
         ds.close()
 
@@ -395,41 +462,51 @@ def main():
 
     out = {
         "metric": "active sites/sec + samples/sec fwd at 1 GPU; % HBM GB/s and % MFMA peak",
-        "value": active * args.steps / dt,
+        "value": active * steps / dt,
         "unit": "active sites/s",
-        "samples_per_s": B * args.steps / dt,
-        "with_input_upload": {"active_sites_per_s": active * args.steps / dt_up, "samples_per_s": B * args.steps / dt_up,
-                              "ms_per_step": 1e3 * dt_up / args.steps, "bytes_uploaded_per_step": upload_bytes,
-                              "note": "sites and features in pinned host memory, uploaded on the producer streams for "
-                                      "every batch: forward time = rule build + H2D of inputs + kernels + D2H"},
+        "value_definition": "median of %d timed regions of %d batches each; every region is the middle of one longer "
+                            "pass (warm-up before, %d more batches behind it); a batch's sites and features are "
+                            "resident in HBM when its region starts; the clock covers grid build, every rule book, "
+                            "all layer kernels and the copy of the probabilities to the host" % (regions, steps, producers),
+        "value_min_max": [active * steps / dt_max, active * steps / dt_min],
+        "samples_per_s": B * steps / dt,
+        "value_with_input_upload": with_upload["active_sites_per_s"],
+        "with_input_upload": with_upload,
         "varied_batches": varied,
         "producer_streams_in_use": net.producerStreamsInUse(),
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
+        "steps": steps,
+        "warmup": warmup,
+        "timed_regions": regions,
+        "tail_batches_per_region": producers,
+        "batches_ready_at_t0": ready,
         "ms_per_step": ms_per_step,
+        "ms_per_step_min_max": [1e3 * dt_min / steps, 1e3 * dt_max / steps],
+        "ms_per_step_regions": [round(1e3 * x / steps, 5) for x in dt_all],
         "ms_single_batch_latency": ms_latency,
-        "ms_per_step_with_event_timing": 1e3 * dt_prof / args.steps,
+        "ms_per_step_with_event_timing": 1e3 * dt_prof / steps,
         "event_span_floor_us": round(1e3 * span_floor_ms, 3),
         "event_span_idle_kernel_us": round(1e3 * span_idle_kernel_ms, 3),
-        "producer_threads": max(1, args.producers),
+        "producer_threads": producers,
         "priming_batches": priming,
         "fused_convolutions": sorted(fused_layers),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32" if args.precision == "fp32" else args.precision,
+        "dtype": "f32" if precision == "fp32" else precision,
         "data": "synthetic",
         "config": {"workload": cfg.name, "batch": B, "input_field": net.inputSpatialSize, "lattice": cfg.lattice,
                    "dimension": cfg.dimension, "active_sites": active, "input_rows": nSites,
-                   "stack": [list(c) for c in cfg.stack], "precision": args.precision, "seed": args.seed,
+                   "stack": [list(c) for c in cfg.stack], "precision": precision, "seed": args.seed,
                    "fused": bool(args.fused)},
         "mega_multiply_adds_per_sample": mac / B / 1e6,
         "giga_multiply_adds_per_s": mac / (ms_per_step * 1e-3) / 1e9,
         "roofline": roofline,
         "roofline_nin": roofline_nin,
+        "roofline_maxpool": roofline_pool,
         "rules": rules_entry,
         "traffic_measured_at_commit": traffic_commit,
+        "traffic_note": traffic_note,
         "kernel_family_ms_per_step": {k: round(v, 5) for k, v in fam_ms.items()},
         "kernels": kernels,
         "cpu_baseline": cpu_baseline,
@@ -437,6 +514,54 @@ def main():
     if from_host:
         out["from_host_pictures"] = from_host
     net.close()
+    return out
+
+
+def net_streams(wanted, producers):
+    pool = min(5, producers)
+    return pool if wanted < 1 or wanted > pool else wanted
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; --gpus %d is not supported (the forward path shards by sample "
+              "with no exchange between the GPUs)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    # the host classes announce every layer on stdout like the reference does;
+    # keep stdout for the one JSON line and send that chatter to stderr
+    sys.stdout.flush()
+    saved_stdout = os.dup(1)
+    os.dup2(2, 1)
+    from __graft_entry__ import load_package
+    scn = load_package()
+    from sparseconvnet_archived_amd import hostapi, synthetic
+
+    if args.train:
+        cfg = synthetic.config(args.config, batch=args.batch)
+        net = hostapi.Net(cfg.dimension, cfg.nInputFeatures, max(cfg.nClasses, 1), threads=max(1, args.producers))
+        net.setProducerStreams(max(0, args.producer_streams))
+        cfg.build(net)
+        net.setFusedConvolutions(bool(args.fused))
+        for i, (W, Bv, pr) in synthetic.he_normal_weights(net.layers(), args.seed + 1).items():
+            net.set_weights(i, W, Bv, pr)
+        train_leg(args, cfg, net, hostapi, synthetic.make_samples(cfg, args.seed), saved_stdout)
+        return
+    out = measure(scn, hostapi, synthetic, args, args.config, args.precision, True)
+    # the other configurations, a short pass each (the headline config's line stays the line)
+    others = []
+    t_start = time.perf_counter()
+    for item in [x for x in args.other_configs.split(",") if x]:
+        number, _, prec = item.partition(":")
+        number, prec = int(number), prec or "fp32"
+        if number == args.config and prec == args.precision:
+            continue
+        if time.perf_counter() - t_start > args.other_seconds:
+            others.append({"workload": "config %d %s" % (number, prec), "skipped": "time budget of the run"})
+            continue
+        print("bench.py: config %d, %s" % (number, prec), file=sys.stderr, flush=True)
+        others.append(measure(scn, hostapi, synthetic, args, number, prec, False))
+    out["other_configs"] = others
     sys.stdout.flush()
     os.dup2(saved_stdout, 1)
     print(json.dumps(out))

@@ -196,6 +196,65 @@ class Net:
                 out["predictions"] = np.stack([orc.top_indices(p, self.nTop) for p in probs])
         return out
 
+    # ---- the same pass in float64, through rule books that forward() has built
+    def forward64(self, fwd, every=False):
+        """Class probabilities (or the top feature matrix of a headless stack) of the batch behind `fwd` in float64
+        numpy arithmetic: the rule books are taken from fwd's interfaces, every feature layer is evaluated from its
+        definition (gather = indexing through the rules, NiN = p (A W + B) then the activation, max-pool = maximum
+        of the listed rows, terminal pooling = mean of the listed rows).  Shares no arithmetic with the C oracle; it is
+        what single-precision results are measured against.  Dropout subsets are taken from fwd; a RESCALEBATCH pass is not covered.
+        every: an iterator over all interfaces' feature matrices instead, the input first (one alive at a time)."""
+        it = self._forward64(fwd)
+        if every:
+            return it
+        x = None
+        for x in it:
+            pass
+        return x
+
+    def _forward64(self, fwd):
+        ifaces = fwd["interfaces"]
+        x = ifaces[0]["features"].astype(np.float64).reshape(ifaces[0]["nSpatialSites"], -1)
+        yield x
+        for i, l in enumerate(self.layers):
+            k, nxt = l["kind"], ifaces[i + 1]
+            n = nxt["nSpatialSites"]
+            if k in ("conv", "conv_tri"):
+                r = nxt["rules"].reshape(n, -1)
+                x = np.where((r >= 0)[:, :, None], x[np.maximum(r, 0)], 0.0).reshape(n, -1)
+            elif k in ("maxpool", "maxpool_tri", "fmp"):
+                r = nxt["rules"].reshape(n, -1)
+                cand = np.where((r >= 0)[:, :, None], x[np.maximum(r, 0)], -np.inf)
+                x = cand.max(1)
+            elif k in ("nin", "nin_prelu"):
+                W, B, pr = self.weights[i]
+                if "shrunk" in nxt:  # a training batch with dropout: the sub-matrix, unscaled
+                    _, outP, w = nxt["shrunk"]
+                    z = x @ w.astype(np.float64) + B[outP].astype(np.float64)
+                else:
+                    p = 1.0 - float(np.float32(l["dropout"]))
+                    z = p * (x @ W.astype(np.float64) + B.astype(np.float64))
+                act = l["act"]
+                if act == SOFTMAX:  # SigmoidLayer.cu:160-177
+                    e = np.exp(z - np.maximum(z.max(1, keepdims=True), -10000.0))
+                    x = e / e.sum(1, keepdims=True)
+                elif act == orc.TANH:
+                    x = np.tanh(z)
+                elif act == orc.SIGMOID:
+                    x = 1.0 / (1.0 + np.exp(-z))
+                elif act == orc.NOSIGMOID:
+                    x = z
+                else:
+                    slope = {RELU: 0.0, orc.VLEAKYRELU: float(np.float32(0.333)),
+                             orc.LEAKYRELU: float(np.float32(0.01))}.get(act)
+                    slope = pr.astype(np.float64) if act == PRELU else slope
+                    x = np.where(z > 0, z, z * slope)
+            elif k == "terminal":
+                r = nxt["rules"].reshape(n, -1)
+                cnt = np.maximum((r >= 0).sum(1), 1)
+                x = np.where((r >= 0)[:, :, None], x[np.maximum(r, 0)], 0.0).sum(1) / cnt[:, None]
+            yield x
+
     # ---- backward over the batch just forwarded, and the weight update
     def train_step(self, fwd, labels, learningRate, momentum):
         """SparseConvNetCUDA::processBatch for a TRAINBATCH without dropout (SparseConvNetCUDA.cu:247-252):

@@ -74,6 +74,8 @@ public:
   // still read batch i after asking for batch i + 1 (needs >= 2 slots).
   int keepAlive = 0;
   SpatiallySparseBatch *nextBatch();
+  // slots that hold a finished batch nobody has asked for yet
+  int slotsReady();
   void batchProducerThread(int nThread);
   // CPU half: fills slot cc with batch c (codify only)
   void preprocessBatch(int c, int cc, RNG &rng);

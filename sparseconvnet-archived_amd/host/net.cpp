@@ -947,6 +947,15 @@ void BatchProducer::batchProducerThread(int nThread) {
     slotChanged.notify_all();
   }
 }
+int BatchProducer::slotsReady() {
+  std::lock_guard<std::mutex> lock(slotMutex);
+  int n = 0;
+  for (char full : slotFull)
+    n += full != 0;
+  // (slots of batches already handed out stay marked until they are given back)
+  const int out = std::min(batchCounter + 1, keepAlive + 1);
+  return std::max(0, n - std::max(0, out));
+}
 SpatiallySparseBatch *BatchProducer::nextBatch() {
   if (batchCounter - keepAlive >= 0) { // hand a finished slot back to its worker
     int cc = (batchCounter - keepAlive) % cnn.nBatchProducerThreads;

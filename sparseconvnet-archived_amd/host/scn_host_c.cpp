@@ -20,6 +20,10 @@ struct scnh_net {
   SpatiallySparseBatch *batch = nullptr;
   bool hasClassifier = false;
   float learningRate = 0, momentum = 0; // of the batches scnh_next_batch runs
+  int streamTail = 0;    // batches that follow the timed ones of a stream pass
+  int readyAtStart = 0;  // slots that held a finished batch when the clock started
+  float *allProbs = nullptr; // where a stream pass leaves every batch's probabilities
+  int64_t allProbsCapacity = 0;
 };
 struct scnh_dataset {
   SpatiallySparseDataset ds;
@@ -595,9 +599,19 @@ int scnh_forward_stream_timed_many(
                              nActive[i], nSpatialSites[i], features[i]));
     rs.back().onHost = inputsOnHost != 0;
   }
-  BatchProducer bp(*cnn, rs, nWarmup + nTimed);
+  // The timed batches sit in the middle of a longer pass: nTail more batches
+  // follow them, so that the producers are as busy at the end of the timed
+  // window as they are at its start (they hold finished batches ready at both
+  // ends; without a tail the window would be served in part by work done before
+  // the clock started and never paid back).
+  const int nTail = net->streamTail > 0 ? net->streamTail : 0;
+  BatchProducer bp(*cnn, rs, nWarmup + nTimed + nTail);
   ForwardQueue queue(*cnn, bp, !net->hasClassifier); // (a headless net: layer by layer on lane 0)
   int done = 0, started = 0;
+  float *all = net->allProbs;
+  int64_t allLeft = net->allProbsCapacity;
+  auto t0 = std::chrono::steady_clock::now();
+  bool stopped = false;
   auto finish = [&](SpatiallySparseBatch *b) {
     if (net->hasClassifier) {
       std::ofstream f, g;
@@ -605,10 +619,23 @@ int scnh_forward_stream_timed_many(
       net->batch = b;
       if (h_probs)
         scnh_batch_probabilities(net, h_probs);
+      if (all) { // every batch's probabilities, in batch order, while they fit
+        const int64_t n = (int64_t)b->probabilities.size() * cnn->nClasses;
+        if (n <= allLeft) {
+          scnh_batch_probabilities(net, all);
+          all += n;
+          allLeft -= n;
+        }
+      }
     }
+    net->batch = b;
     ++done;
+    if (done == nWarmup + nTimed && !stopped) { // the last timed batch is on the host
+      if (seconds)
+        *seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+      stopped = true;
+    }
   };
-  auto t0 = std::chrono::steady_clock::now();
   SpatiallySparseBatch *headless = nullptr;
   while (SpatiallySparseBatch *b = bp.nextBatch()) {
     if (started == nWarmup) { // every warm-up batch done before the clock starts
@@ -618,18 +645,29 @@ int scnh_forward_stream_timed_many(
         finish(headless);
       headless = nullptr;
       cnn->synchronizeLanes();
+      net->readyAtStart = bp.slotsReady();
       t0 = std::chrono::steady_clock::now();
     }
+    const bool firstOfTail = started == nWarmup + nTimed;
     ++started;
     if (net->hasClassifier) {
       if (SpatiallySparseBatch *due = queue.push(b))
         finish(due);
     } else {
+      // (nothing is read back from a headless stack: a batch is finished when
+      // the net's stream has run it)
+      if (firstOfTail && headless) {
+        cnn->synchronizeLanes();
+        finish(headless);
+        headless = nullptr;
+      }
       forward_layers(net, *b);
       if (headless)
         finish(headless);
       headless = b;
       if (!bp.keepAlive) {
+        if (done + 1 == nWarmup + nTimed)
+          cnn->synchronizeLanes();
         finish(headless);
         headless = nullptr;
       }
@@ -637,13 +675,37 @@ int scnh_forward_stream_timed_many(
   }
   while (SpatiallySparseBatch *q = queue.pop())
     finish(q);
-  if (headless)
+  if (headless) {
+    cnn->synchronizeLanes();
     finish(headless);
+  }
   cnn->synchronizeLanes();
-  if (seconds)
-    *seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
-  net->batch = nullptr;
-  return done;
+  // net->batch stays at the last batch finished: its interfaces can be read
+  // (scnh_iface_*) until the next pass starts
+  return done - nTail;
+}
+void scnh_set_stream_tail(scnh_net *net, int nTail) { net->streamTail = nTail; }
+int scnh_stream_ready_at_start(scnh_net *net) { return net->readyAtStart; }
+void scnh_collect_probabilities(scnh_net *net, float *h_all, int64_t capacity) {
+  net->allProbs = h_all;
+  net->allProbsCapacity = h_all ? capacity : 0;
+}
+void scnh_chain_counts(scnh_net *net, int64_t *chains, int64_t *plans) {
+  SparseConvNetCUDA *cnn = net->cnn;
+  int64_t c = 0, p = 0;
+  auto add = [&](scn_ctx *ctx) {
+    int64_t a = 0, b = 0;
+    SCN_CHECKED(scn_ctx_chain_count(ctx, &a, &b));
+    c += a;
+    p += b;
+  };
+  add(cnn->memStream.ctx);
+  for (auto &s : cnn->batchMemStreams)
+    add(s->ctx);
+  if (chains)
+    *chains = c;
+  if (plans)
+    *plans = p;
 }
 void *scnh_context(scnh_net *net) { return net->cnn->memStream.ctx; }
 double scnh_take_multiply_add_count(void) {

@@ -221,6 +221,21 @@ int scnh_forward_stream_timed_many(
     const int64_t *nActive, const int *nSpatialSites,
     const float *const *features, int inputsOnHost, float *h_probs,
     double *seconds);
+/* nTail batches follow the timed ones of every later scnh_forward_stream_timed
+ * (_many) pass, untimed: the timed window then lies in the middle of a pass,
+ * with the producers as busy at its end as at its start (0: none). */
+void scnh_set_stream_tail(scnh_net *net, int nTail);
+/* how many batch slots held a finished batch when the clock of the last such
+ * pass started */
+int scnh_stream_ready_at_start(scnh_net *net);
+/* Every later such pass also leaves the probabilities of all its batches, in
+ * batch order, in h_all (capacity in floats; batches that no longer fit are
+ * left out; null: switched off).  After a pass the last batch finished stays
+ * readable through scnh_iface_* and scnh_batch_* until the next pass. */
+void scnh_collect_probabilities(scnh_net *net, float *h_all, int64_t capacity);
+/* recorded-plan runs so far on all streams of the net that build rule books
+ * (sums of scn_ctx_chain_count) */
+void scnh_chain_counts(scnh_net *net, int64_t *chains, int64_t *plans);
 /* the library context of the net (scn_ctx *), for timing and raw buffers */
 void *scnh_context(scnh_net *net);
 /* multiply-accumulates of the NiN layers since the last call */

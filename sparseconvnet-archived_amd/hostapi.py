@@ -99,6 +99,10 @@ def lib():
         "scnh_forward_resident_stream": (i32, [vp, i32, i32, vp, vp, vp, vp, i64, i32, vp, vp]),
         "scnh_forward_stream_timed": (i32, [vp, i32, i32, i32, vp, vp, vp, vp, i64, i32, vp, i32, vp, P(C.c_double)]),
         "scnh_forward_stream_timed_many": (i32, [vp, i32, i32, i32, vp, vp, vp, vp, vp, vp, vp, vp, i32, vp, P(C.c_double)]),
+        "scnh_set_stream_tail": (None, [vp, i32]),
+        "scnh_stream_ready_at_start": (i32, [vp]),
+        "scnh_collect_probabilities": (None, [vp, vp, i64]),
+        "scnh_chain_counts": (None, [vp, P(i64), P(i64)]),
         "scnh_context": (vp, [vp]),
         "scnh_take_multiply_add_count": (C.c_double, []),
     }
@@ -439,6 +443,25 @@ class Net:
                                                     _p(h_probs) if h_probs is not None else None, C.byref(sec))
         assert done == nWarmup + nTimed
         return sec.value
+
+    def setStreamTail(self, nTail):
+        """batches that follow the timed ones of every later forward_stream_timed(_many) pass, untimed"""
+        lib().scnh_set_stream_tail(self.h, int(nTail))
+
+    def streamReadyAtStart(self):
+        return lib().scnh_stream_ready_at_start(self.h)
+
+    def collect_probabilities(self, out):
+        """out: float32 array that later stream passes fill with every batch's probabilities in batch order
+        (None: switched off).  The caller keeps it alive."""
+        self._collect = out
+        lib().scnh_collect_probabilities(self.h, _p(out) if out is not None else None, 0 if out is None else out.size)
+
+    def chain_counts(self):
+        """(runs of recorded plans, plans in them) so far, over every stream that builds rule books"""
+        a, b = C.c_int64(), C.c_int64()
+        lib().scnh_chain_counts(self.h, C.byref(a), C.byref(b))
+        return a.value, b.value
 
     def context_handle(self):
         return lib().scnh_context(self.h)

@@ -6,6 +6,7 @@ import pytest
 import brute
 import oracle as orc
 from gpu_util import assert_same_grids, device_grids, oracle_grids
+from gpu_util import assert_probabilities
 
 pytestmark = pytest.mark.gpu
 
@@ -161,7 +162,7 @@ def test_net_with_fractional_max_pooling(scn, kind, train):
         if i > 0 and layers[i - 1]["kind"] == "fmp":
             assert np.array_equal(gi["choices"], wi["choices"])
     out = net.batch_outputs()
-    assert np.allclose(out["probabilities"], want["probabilities"], rtol=1e-3, atol=1e-6)
+    assert_probabilities(out["probabilities"], ora.forward64(want))
     if train:
         ora.train_step(want, labels, 0.01, 0.9)
         for i, wi in enumerate(want["interfaces"]):

@@ -7,6 +7,7 @@ import numpy as np
 import pytest
 
 from brute import rules_vectorized
+from gpu_util import assert_probabilities
 
 pytestmark = pytest.mark.gpu
 
@@ -29,7 +30,12 @@ def layer_geometry(stack):
     return out
 
 
-def check_net(scn, number, batch, seed, nin_rows=1500, fused=False, max_rows=1 << 16, precision=None, tol=1e-4):
+def check_net(scn, number, batch, seed, nin_rows=1500, fused=False, max_rows=1 << 16, precision=None, tol=1e-4, warm=0,
+              chained=None):
+    """warm: batches the slot is given before the one that is checked (its first batch is always planned layer by
+    layer through HBM; later ones through recorded plans where a sample's masks fit a compute unit's LDS, the second
+    with the widest arena, the third with one sized by what the slot has seen -- the path of every batch of a long
+    pass); chained: whether the checked batch must or must not have been planned that way."""
     from sparseconvnet_archived_amd import hostapi, synthetic
     cfg = synthetic.config(number, batch=batch)
     d = cfg.dimension
@@ -45,8 +51,15 @@ def check_net(scn, number, batch, seed, nin_rows=1500, fused=False, max_rows=1 <
     ds = hostapi.Dataset(cfg.name, cfg.nInputFeatures, max(cfg.nClasses, 1), hostapi.TESTBATCH)
     for pts, f, label in samples:
         ds.add_points(d, cfg.lattice, pts, f, label)
+    for _ in range(warm):
+        net.begin(ds, batch)
+        assert net.next_batch()
+        net.end()
+    chains = net.chain_counts()[0]
     net.begin(ds, batch)
     assert net.next_batch()
+    if chained is not None:
+        assert (net.chain_counts()[0] > chains) == chained
     layers = net.layers()
     geo = layer_geometry(cfg.stack)
     assert len(geo) == len(layers)
@@ -96,7 +109,7 @@ def check_net(scn, number, batch, seed, nin_rows=1500, fused=False, max_rows=1 <
                 assert np.allclose(fout.sum(1), 1, atol=1e-4)
                 e = np.exp(z - z.max(1, keepdims=True))
                 want = e / e.sum(1, keepdims=True)
-                assert np.allclose(fout[pick], want, rtol=max(1e-3, tol), atol=1e-6)
+                assert_probabilities(fout[pick], want, tol)  # each within tol of its row's largest
             else:
                 slope = {synthetic.RELU: 0.0, synthetic.PRELU: None}.get(act, 1.0)
                 want = np.where(z > 0, z, z * (pr if slope is None else slope))
@@ -129,14 +142,32 @@ def test_config2_full_batch_rule_books_and_layers(scn):
         alone = net.batch_outputs()["probabilities"][0]
         net.end()
         # (other kernels serve a batch of one: equal to rounding, not to the bit)
-        assert np.allclose(alone, out["probabilities"][pickOne], rtol=1e-3, atol=1e-6)
+        assert_probabilities(alone[None], out["probabilities"][pickOne][None])
     net.close()
 
 
 @pytest.mark.parametrize("number,batch,fused", [(1, 16, False), (3, 32, False), (4, 128, False), (4, 128, True),
                                                 (5, 96, True)])
 def test_full_batch_rule_books_and_layers(scn, number, batch, fused):
-    net, ds, samples, out = check_net(scn, number, batch, 100 * number + 5, fused=fused)
+    net, ds, samples, out = check_net(scn, number, batch, 100 * number + 5, fused=fused, chained=False)
+    net.close()
+
+
+@pytest.mark.parametrize("number,batch,fused,warm", [(1, 16, False, 2), (2, 100, True, 1), (2, 100, True, 2),
+                                                     (2, 100, False, 2), (3, 32, True, 1), (3, 32, True, 2),
+                                                     (3, 32, False, 2), (4, 128, True, 2), (4, 128, False, 2)])
+def test_full_batch_rule_books_from_recorded_plans(scn, number, batch, fused, warm):
+    """The rule books every batch of a long pass gets -- recorded plans run as k_chain_sample / k_chain_place -- at the
+    full field and batch of configs 1-4: the slot's second or third batch, rebuilt from the grids alone
+    (gridRules per sample, Regions.cu:528-653, ConvolutionalLayer.cu:114-118), and every feature layer on top."""
+    net, ds, samples, out = check_net(scn, number, batch, 100 * number + 7, fused=fused, warm=warm, chained=True)
+    net.close()
+
+
+def test_large_field_third_batch_is_planned_layer_by_layer(scn):
+    """Config 5 (128^3: a sample's masks do not fit LDS) never takes the recorded plans; its third batch, planned
+    with deferred counts through HBM, is checked like its first."""
+    net, ds, samples, out = check_net(scn, 5, 96, 512, fused=True, warm=2, chained=False)
     net.close()
 
 
@@ -148,3 +179,85 @@ def test_wide_net_full_batch_bf16(scn):
         net, ds, samples, out = check_net(scn, 4, 128, 405, fused=fused, precision=scn.BF16, tol=2e-2)
         assert np.allclose(out["probabilities"].sum(1), 1, atol=1e-4)
         net.close()
+
+
+@pytest.mark.parametrize("distinct,inputs_on_host", [(1, False), (1, True), (3, False)])
+def test_benchmark_pass_against_oracle(scn, distinct, inputs_on_host):
+    """The pass bench.py times, as it runs it: config 2 at batch 100, ten producer threads on two producer streams, two
+    forward lanes, fused convolutions, priming batches, then warm-up + timed + tail batches in one
+    scnh_forward_stream_timed(_many) pass, inputs resident in HBM or uploaded from pinned memory with every batch.
+    Every batch of that pass must have come from recorded plans; the probabilities of all of them are compared with
+    the float64 evaluation of the oracle's pass over the same batch, and the rule books, grids and background rows
+    the last batch left in its slot with the oracle's, bit for bit."""
+    import oracle_net
+    from sparseconvnet_archived_amd import hostapi, synthetic
+    cfg = synthetic.config(2)
+    B, producers, warmup, steps = cfg.batch, 10, 5, 20
+    assert B == 100
+    net = hostapi.Net(cfg.dimension, cfg.nInputFeatures, cfg.nClasses, threads=producers)
+    net.setProducerStreams(2)
+    ora = oracle_net.Net(cfg.dimension, cfg.nInputFeatures, cfg.nClasses)
+    cfg.build(net)
+    cfg.build(ora)
+    net.setFusedConvolutions(True)
+    for i, (W, Bv, pr) in synthetic.he_normal_weights(net.layers(), 2016).items():
+        net.set_weights(i, W, Bv, pr)
+        ora.set_weights(i, W, Bv, pr)
+    ctx = scn.Context(handle=net.context_handle())
+
+    def pinned(a):
+        h = ctx.host_alloc(a.nbytes)
+        np.frombuffer(h.buffer(), a.dtype, a.size)[:] = a.reshape(-1)
+        return h
+
+    keep, descr, wants, p64 = [], [], [], []
+    for i in range(distinct):
+        samples = synthetic.make_samples(cfg, 2015 + 100 * i)
+        S, K, R, bg, feats, n = synthetic.codify(samples, cfg.dimension, cfg.lattice, net.inputSpatialSize,
+                                                 cfg.nInputFeatures)
+        arrays = (S.astype(np.int32), K.astype(np.int64), R.astype(np.int32), bg.astype(np.int32),
+                  feats.astype(np.float32))
+        if inputs_on_host:
+            arrs = [pinned(np.ascontiguousarray(x)) for x in arrays]
+        else:
+            arrs = [ctx.array(x, x.dtype) for x in arrays]
+        keep.append(arrs)
+        descr.append((B, arrs[0].ptr, arrs[1].ptr, arrs[2].ptr, arrs[3].ptr, int(len(K)), int(n), arrs[4].ptr))
+        wants.append(ora.forward(B, S, K, R, bg, feats, n, np.array([s[2] for s in samples], np.int32)))
+        p64.append(ora.forward64(wants[-1]))
+    probs = np.zeros((B, cfg.nClasses), np.float32)
+    priming = 3 * producers + distinct
+    if distinct == 1:
+        net.forward_stream_timed(0, priming, *descr[0], inputs_on_host=inputs_on_host, h_probs=probs)
+    else:
+        net.forward_stream_timed_many(0, priming, descr, inputs_on_host=inputs_on_host, h_probs=probs)
+    net.setStreamTail(producers)
+    nPass = warmup + steps + producers
+    everything = np.zeros((nPass, B, cfg.nClasses), np.float32)
+    net.collect_probabilities(everything)
+    chains = net.chain_counts()[0]
+    if distinct == 1:
+        dt = net.forward_stream_timed(warmup, steps, *descr[0], inputs_on_host=inputs_on_host, h_probs=probs)
+    else:
+        dt = net.forward_stream_timed_many(warmup, steps, descr, inputs_on_host=inputs_on_host, h_probs=probs)
+    net.collect_probabilities(None)
+    print("benchmark pass: %.4f ms per batch, %d batches ready when the clock started"
+          % (1e3 * dt / steps, net.streamReadyAtStart()), flush=True)
+    # every batch of the pass had its rule books from recorded plans (k_chain_sample / k_chain_place)
+    assert net.chain_counts()[0] == chains + nPass
+    worst = 0.0
+    for i in range(nPass):
+        worst = max(worst, assert_probabilities(everything[i], p64[i % distinct]))
+        assert np.array_equal(everything[i], everything[i % distinct])  # the same batch gives the same bits every time
+    print("probabilities of %d batches: worst %.3g of the row's scale" % (nPass, worst), flush=True)
+    # what the last batch of the pass left in its slot
+    want = wants[(nPass - 1) % distinct]
+    for i, wi in enumerate(want["interfaces"]):
+        gi = net.interface(i, want_features=False)
+        assert gi["nSpatialSites"] == wi["nSpatialSites"]
+        assert np.array_equal(gi["rules"], wi["rules"])
+        s, k, r, b = gi["grids"]
+        os_, ok, or_, ob = wi["grids"].flat()
+        assert np.array_equal(s, os_) and np.array_equal(k, ok) and np.array_equal(r, or_) and np.array_equal(b, ob)
+    del keep
+    net.close()

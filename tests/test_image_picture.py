@@ -10,6 +10,7 @@ import pytest
 
 sys.path.insert(0, os.path.join(os.path.dirname(__file__), "..", "oracle"))
 import image_picture as img  # noqa: E402
+from gpu_util import assert_probabilities
 
 
 def hostapi():
@@ -179,6 +180,6 @@ def test_images_through_a_2d_net(scn):
     net.begin(ds, len(pics))
     assert net.next_batch()
     out = net.batch_outputs()
-    assert np.allclose(out["probabilities"], want["probabilities"], rtol=1e-3, atol=1e-6)
+    assert_probabilities(out["probabilities"], ora.forward64(want))
     net.end()
     net.close()

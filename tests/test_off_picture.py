@@ -9,6 +9,7 @@ import pytest
 
 sys.path.insert(0, os.path.join(os.path.dirname(__file__), "..", "oracle"))
 import off_picture as off  # noqa: E402
+from gpu_util import assert_probabilities
 
 
 def hostapi():
@@ -181,7 +182,7 @@ def test_meshes_through_a_3d_net(scn):
     net.begin(ds2, len(meshes))
     assert net.next_batch()
     out = net.batch_outputs()
-    assert np.allclose(out["probabilities"], want["probabilities"], rtol=1e-3, atol=1e-6)
+    assert_probabilities(out["probabilities"], ora.forward64(want))
     net.end()
     # the mesh pictures themselves: a probability row per mesh
     net.begin(ds, len(meshes))
