@@ -25,6 +25,8 @@
 // recorded layers get their entry lists, backgroundCol and counts; their hash
 // tables and masks are only built if somebody asks (ensure_index).
 #include "scn_grids_dev.h"
+#include "scn_pyr_dev.h"
+#include <stdlib.h>
 #include <string.h>
 #include <mutex>
 
@@ -34,6 +36,8 @@
 #endif
 #define CHAIN_WAVES (CHAIN_THREADS / 64)
 #define CHAIN_LDS_MAX (152 * 1024)
+// most LDS a workgroup of k_pyr_rules asks for
+#define PYR_LDS_MAX CHAIN_LDS_MAX
 #define CHAIN_HEADER_BYTES 512
 #define CHAIN_MIN_ARENA (16 * 1024)
 // bytes of arena per entry of the input grid (key, row, ownership mask, base)
@@ -96,6 +100,12 @@ struct ChainState {
   std::vector<ChainRec> recs;
   DevBuf<int> staging, counts;
   DevBuf<unsigned long long> flag;
+  // chains of square layers without a minimum, built from the output side
+  DevBuf<unsigned long long> pyramid;
+  bool pyramids = true; // (false: such chains go through k_chain_sample too)
+  bool pyrAtMax = false; // the last such chain had all the LDS there is
+  scn_grids *pyrSource = nullptr; // source of the last such chain: its largest sample comes back in h_pinned[13]
+  long long nPyramids = 0;
 };
 
 // ------------------------------------------------------------------ device
@@ -117,6 +127,23 @@ __device__ __forceinline__ unsigned wave_scan_incl(unsigned v, int lane) {
       v += up;
   }
   return v;
+}
+
+// The same sums through the lanes' cross-lane data path instead of the LDS
+// crossbar: shifts within a row of 16 lanes, then the last lane of rows 0 and 2
+// into the rows after them, then lane 31 into rows 2 and 3 (a lane that a step
+// does not reach adds 0).
+__device__ __forceinline__ unsigned wave_scan_incl_dpp(unsigned v) {
+  v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xf, 0xf, false); // row_shr:1
+  v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xf, 0xf, false); // row_shr:2
+  v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xf, 0xf, false); // row_shr:4
+  v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xf, 0xf, false); // row_shr:8
+  v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xa, 0xf, false); // row_bcast:15
+  v += (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xc, 0xf, false); // row_bcast:31
+  return v;
+}
+__device__ __forceinline__ unsigned wave_last(unsigned v) {
+  return (unsigned)__builtin_amdgcn_readlane((int)v, 63);
 }
 
 // Exclusive prefix sums over two sequences held in LDS at once, by the whole
@@ -744,11 +771,291 @@ __global__ void __launch_bounds__(PLACE_THREADS) k_chain_place(ChainArgs a) {
     L.bg[b] = hasBg ? (int)(rowBase + n) : -1;
 }
 
+// ------------------------------------------------ chains built from the output side
+//
+// scn_pyr_dev.h has the per-lane bodies; here are the two kernels around them.
+// k_pyr_masks, one workgroup per sample: the occupancy masks of all layers
+// (each the dilation of the one before), their rank prefixes and the sample's
+// site counts, left in global memory.  k_pyr_rules, one workgroup per sample:
+// everything per site, in sweeps over all layers at once -- the sums over the
+// samples before (which k_pyr_masks has finished writing), sites by rank,
+// owners, rows, entry lists and rule rows at their batch-global places.  Nothing
+// is staged and nothing is copied afterwards.
+// k_pyr_masks runs ONE wavefront per sample.  With four wavefronts per
+// workgroup the kernel was measured to give wrong mask words now and then --
+// only while workgroups of other streams' chains shared the compute units, with
+// either kind of barrier, its arguments, its input and its own first level
+// intact, and never with one chain at a time; the instruction stream shows
+// every wait in place.  The cause was not found.  A single wavefront has no
+// barrier to pass and gave no wrong word in any run; it costs about 2 us.
+#define PYR_A_THREADS 64
+#define PYR_A_BARRIER() lds_barrier()
+// keeps a wavefront-uniform value in a scalar register from here on
+#define PYR_PIN(v) asm volatile("" : "+s"(v))
+#define PYR_B_THREADS 512
+static_assert(sizeof(PyrArgs) <= 4096, "kernel arguments");
+
+// A layer's geometry as k_pyr_masks keeps it in LDS: one broadcast read a layer
+// instead of trips to the kernel arguments
+struct PyrGeoA {
+  int nIn, nOut, size, stride;
+  int words, offIn, offOut;
+  unsigned volOut, magicN, lenMax;
+  int pad[2];
+};
+static_assert(sizeof(PyrGeoA) == 48, "three 16-byte reads");
+#define PYR_A_EXTRA (128 + (PYR_MAX_LEVELS + 1) * (int)sizeof(PyrGeoA)) // counts, geometry: after the pyramid
+
+// One level of the pyramid by one wavefront: the words of the output mask (64 at
+// a time), and their rank prefixes in the same go; the level's site count comes back
+template <int D>
+__device__ __forceinline__ unsigned pyr_level(const PyrGeoA &g, pyr_u64 *masks, unsigned short *pref, int lane) {
+  const pyr_u64 *in = masks + g.offIn;
+  unsigned carry = 0;
+  for (int w0 = 0; w0 < g.words + 2; w0 += 64) {
+    const int w = w0 + lane;
+    const pyr_u64 v = w < g.words ? pyr_dilate_any<D>(in, g.nIn, g.nOut, g.size, g.stride, g.volOut, g.magicN, g.lenMax,
+                                                      (unsigned)w)
+                                  : 0ull;
+    const unsigned pc = (unsigned)pyr_popc64(v);
+    const unsigned incl = wave_scan_incl_dpp(pc);
+    if (w < g.words + 2) {
+      masks[g.offOut + w] = v;
+      pref[g.offOut + w] = (unsigned short)(carry + incl - pc);
+    }
+    carry += wave_last(incl);
+  }
+  return carry;
+}
+
+template <int D>
+__global__ void __launch_bounds__(PYR_A_THREADS) k_pyr_masks(PyrArgs a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  pyr_u64 *masks = reinterpret_cast<pyr_u64 *>(lds);
+  unsigned short *pref = reinterpret_cast<unsigned short *>(lds + 8ll * a.maskWords);
+  int *cnt = reinterpret_cast<int *>(lds + 8ll * a.pyrStride);
+  PyrGeoA *geo = reinterpret_cast<PyrGeoA *>(lds + 8ll * a.pyrStride + 128);
+  const int b = blockIdx.x, t = threadIdx.x;
+  static_assert(PYR_A_THREADS == 64, "one wavefront: the levels below pass no barrier");
+  if (t >= 1 && t < a.nMasks) {
+    const PyrLevel &L = a.lv[t];
+    PyrGeoA g;
+    g.nIn = L.nIn;
+    g.nOut = L.nOut;
+    g.size = L.size;
+    g.stride = L.stride;
+    g.words = L.words;
+    g.offIn = a.lv[t - 1].maskOff;
+    g.offOut = L.maskOff;
+    g.volOut = (unsigned)L.volOut;
+    g.magicN = L.magicN;
+    g.lenMax = L.lenMax;
+    g.pad[0] = g.pad[1] = 0;
+    geo[t] = g;
+  }
+  { // level 0: the sample's slice of the source mask
+    const PyrLevel &L = a.lv[0];
+    const int words = L.words;
+    const long long vol = L.volOut;
+    unsigned carry = 0;
+    for (int w0 = 0; w0 < words + 2; w0 += 64) {
+      const int w = w0 + t;
+      const pyr_u64 v = w < words ? pyr_source_word(a.bits, vol, b, (unsigned)w) : 0ull;
+      const unsigned pc = (unsigned)pyr_popc64(v);
+      const unsigned incl = wave_scan_incl_dpp(pc);
+      if (w < words + 2) {
+        masks[w] = v;
+        pref[w] = (unsigned short)(carry + incl - pc);
+      }
+      carry += wave_last(incl);
+    }
+    if (t == 0)
+      cnt[0] = (int)carry;
+  }
+  PYR_A_BARRIER();
+  for (int x = 1; x < a.nMasks; ++x) {
+    // (wavefront-uniform values, told to the compiler: the loops over a window's
+    // rows and a word's pieces then branch on scalars)
+    PyrGeoA g = geo[x];
+    g.nIn = __builtin_amdgcn_readfirstlane(g.nIn);
+    g.nOut = __builtin_amdgcn_readfirstlane(g.nOut);
+    g.size = __builtin_amdgcn_readfirstlane(g.size);
+    g.stride = __builtin_amdgcn_readfirstlane(g.stride);
+    g.words = __builtin_amdgcn_readfirstlane(g.words);
+    g.offIn = __builtin_amdgcn_readfirstlane(g.offIn);
+    g.offOut = __builtin_amdgcn_readfirstlane(g.offOut);
+    g.volOut = (unsigned)__builtin_amdgcn_readfirstlane((int)g.volOut);
+    g.magicN = (unsigned)__builtin_amdgcn_readfirstlane((int)g.magicN);
+    g.lenMax = (unsigned)__builtin_amdgcn_readfirstlane((int)g.lenMax);
+    const unsigned n = pyr_level<D>(g, masks, pref, t);
+    if (t == 0)
+      cnt[x] = (int)n;
+    PYR_A_BARRIER();
+  }
+  pyr_u64 *dst = a.pyramid + (long long)b * a.pyrStride;
+  const pyr_u64 *src = reinterpret_cast<const pyr_u64 *>(lds);
+  for (int i = t; i < a.pyrStride; i += PYR_A_THREADS)
+    dst[i] = src[i];
+  if (t < a.nMasks) {
+    int *c = a.counts + ((long long)t * a.batch + b) * 2;
+    c[0] = cnt[t];
+    c[1] = (long long)cnt[t] < a.lv[t].fullSize;
+  }
+  if (t == 0) {
+    bool fits = pyr_lds_need(a, cnt) <= a.ldsBytesB;
+    for (int x = 0; x < a.nMasks; ++x)
+      fits = fits && cnt[x] <= PYR_ROWS_MAX;
+    if (!fits)
+      atomicMax(a.flag, a.ticket);
+  }
+}
+
+template <int D>
+__global__ void __launch_bounds__(PYR_B_THREADS) k_pyr_rules(PyrArgs a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  PyrHdr *h = reinterpret_cast<PyrHdr *>(lds);
+  const int b = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  constexpr int T = PYR_B_THREADS;
+  const bool gaveUp = *reinterpret_cast<volatile unsigned long long *>(a.flag) == a.ticket;
+  const int nRegions = a.nMasks - 1;
+  if (t == 0)
+    h->over = 0;
+  { // the sample's masks and prefixes
+    const uint4 *src = reinterpret_cast<const uint4 *>(a.pyramid + (long long)b * a.pyrStride);
+    uint4 *dst = reinterpret_cast<uint4 *>(lds + PYR_HDR_BYTES);
+    for (int i = t; i < a.pyrStride / 2; i += T)
+      dst[i] = src[i];
+  }
+  // sums over the samples, a wavefront per level
+  for (int x = wave; x < a.nMasks; x += T / 64) {
+    const int *cnt = a.counts + (long long)x * a.batch * 2;
+    // (a batch's rows are numbered in 32 bits, so these sums fit)
+    unsigned v0 = 0, v1 = 0, v2 = 0, v3 = 0;
+    int mx = 0;
+    for (int s = lane; s < a.batch; s += 64) {
+      const int2 c = reinterpret_cast<const int2 *>(cnt)[s];
+      const int n = c.x, hb = c.y;
+      if (s < b) {
+        v0 += n;
+        v1 += hb;
+      }
+      v2 += n;
+      v3 += hb;
+      mx = n > mx ? n : mx;
+    }
+    v0 = wave_last(wave_scan_incl_dpp(v0));
+    v1 = wave_last(wave_scan_incl_dpp(v1));
+    v2 = wave_last(wave_scan_incl_dpp(v2));
+    v3 = wave_last(wave_scan_incl_dpp(v3));
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const int o = __shfl_xor(mx, off, 64);
+      mx = o > mx ? o : mx;
+    }
+    if (lane == 0) {
+      h->n[x] = cnt[2 * b];
+      h->hasBg[x] = cnt[2 * b + 1];
+      h->actBefore[x] = v0;
+      h->bgBefore[x] = v1;
+      h->actAll[x] = v2;
+      h->bgAll[x] = v3;
+      h->maxAct[x] = mx;
+    }
+  }
+  lds_barrier();
+  if (t <= a.nMasks) {
+    int sum = 0;
+    for (int x = 0; x < t; ++x)
+      sum += h->n[x];
+    h->siteOff[t] = sum;
+    if (t < a.nMasks)
+      pyr_fill_en(a, lds, t, sum);
+    if (t == a.nMasks)
+      h->total = sum;
+  }
+  if (t >= 1 && t <= nRegions + 1) {
+    int sum = 0;
+    for (int l = 1; l < t; ++l)
+      sum += h->n[l];
+    h->itemOff[t] = sum;
+  }
+  if (t >= 1 && t <= a.nLevels && pyr_report(a, h, t).over)
+    atomicOr(&h->over, 1);
+  if (t == 0 && pyr_lds_need(a, h->n) > a.ldsBytesB)
+    atomicOr(&h->over, 2);
+  lds_barrier();
+  const bool over = h->over != 0 || gaveUp;
+  if (b == 0 && t >= 1 && t <= a.nLevels) {
+    const PyrLevel &L = a.lv[t];
+    const PyrReport r = pyr_report(a, h, t);
+    L.meta[META_SITES] = over ? 0 : r.nSites;
+    L.meta[META_ACTIVE] = over ? 0 : r.nActive;
+    L.meta[META_OVERFLOW] = over;
+    L.meta[META_WIDTH] = L.kind == PYR_TERMINAL ? r.extra : 0;
+    volatile long long *slot = a.scalars + 16 + 4 * L.slot;
+    slot[0] = r.nSites;
+    slot[1] = r.nActive;
+    slot[2] = over;
+    slot[3] = r.extra;
+  }
+  if (b == 0 && t == 0) {
+    a.scalars[15] = *a.badSites;
+    a.scalars[13] = h->maxAct[0];
+  }
+  if (over)
+    return;
+  const PyrLds s = pyr_lds_view(a, lds, h->total, h->n[0]);
+  if (t >= 1 && t <= a.nLevels)
+    pyr_fill_level(a, s, t, b);
+  pyr_sweep_clear(s, t, T);
+  pyr_sweep_enumerate<D>(a, s, t, T);
+  lds_barrier();
+  { // the batch's rows of the source's sites: their loads go out first
+    const PyrLevel &L = a.lv[0];
+    const long long p0 = (long long)b * L.volOut;
+    const Slot *table = reinterpret_cast<const Slot *>(a.table);
+    for (int r = t; r < h->n[0]; r += T) {
+      int c[D];
+      pyr_unpack<D>(s.key[r], c);
+      long long p = p0 + pyr_key<D>(c, L.nOut);
+      p = p < (long long)a.batch * L.volOut ? p : 0; // (a mask never has a site beyond the field)
+      s.srcRow[r] = (unsigned)(a.dense ? a.dense[p] : hash_find(table, a.shift, a.mask, p));
+    }
+  }
+  pyr_sweep_owners<D>(s, nRegions, t, T);
+  lds_barrier();
+  // rows owned by the sites before, a wavefront per level
+  for (int x = wave; x < nRegions; x += T / 64) {
+    const int n = h->n[x];
+    const unsigned off = (unsigned)h->siteOff[x];
+    unsigned carry = 0;
+    for (int r0 = 0; r0 < n; r0 += 64) {
+      const int r = r0 + lane;
+      const unsigned v = r < n ? (unsigned)pyr_popc32(pyr_own_mask(s, off + r)) : 0u;
+      const unsigned incl = wave_scan_incl_dpp(v);
+      if (r < n)
+        s.base[off + r] = (unsigned short)(carry + incl - v);
+      carry += wave_last(incl);
+    }
+  }
+  lds_barrier();
+  pyr_sweep_rows<D>(s, nRegions, b, t, T);
+  lds_barrier();
+  pyr_sweep_rules<D>(s, nRegions, t, T);
+  pyr_sweep_tail(a, s, b, t, T);
+}
+
 // -------------------------------------------------------------------- host
 
 static ChainState *chain_state(scn_ctx *ctx) {
-  if (!ctx->chain)
+  if (!ctx->chain) {
     ctx->chain = new ChainState();
+    // SCN_CHAIN_PYRAMID=0: a diagnostic switch for A/B runs, every chain through
+    // k_chain_sample / k_chain_place (the rule books are the same)
+    const char *e = getenv("SCN_CHAIN_PYRAMID");
+    if (e && e[0] == '0')
+      ctx->chain->pyramids = false;
+  }
   return ctx->chain;
 }
 
@@ -758,6 +1065,7 @@ void scn_chain_release(scn_ctx *ctx) {
   ctx->chain->staging.release();
   ctx->chain->counts.release();
   ctx->chain->flag.release();
+  ctx->chain->pyramid.release();
   delete ctx->chain;
   ctx->chain = nullptr;
 }
@@ -986,6 +1294,163 @@ int scn_chain_record_fill(scn_ctx *ctx, const scn_grids *in, scn_grids *out,
   return SCN_OK;
 }
 
+// Chains of square layers without a minimum (and a terminal layer at the end)
+// are built from the output side by k_pyr_masks / k_pyr_rules.  *done = false:
+// this chain is not of that kind (or its masks do not fit), run it the other way.
+static int chain_flush_pyramid(scn_ctx *ctx, ChainState *cs, std::vector<ChainRec> &recs,
+                               bool *done) {
+  *done = false;
+  scn_grids *src = recs[0].in;
+  const int d = src->d;
+  for (size_t i = 0; i < recs.size(); ++i) {
+    const ChainLevel &L = recs[i].lv;
+    if (L.kind == CH_TERMINAL) {
+      if (i + 1 != recs.size())
+        return SCN_OK;
+      continue;
+    }
+    if (L.mode != MODE_SQ_NOMIN || L.cube > PYR_CUBE_MAX || L.size < 1 ||
+        (d >= 2 && L.size > 4) || L.stride < 1)
+      return SCN_OK;
+  }
+  if ((int)recs.size() > PYR_MAX_LEVELS)
+    return SCN_OK;
+  PyrArgs a;
+  memset(&a, 0, sizeof(a));
+  a.nLevels = (int)recs.size();
+  a.batch = src->batch;
+  a.d = d;
+  auto magic = [](long long x) { return (unsigned)((1ull << 32) / (unsigned long long)(x > 0 ? x : 1) + 1); };
+  long long maskWords = 0;
+  {
+    PyrLevel &L = a.lv[0];
+    L.kind = PYR_REGIONS;
+    L.nIn = L.nOut = src->n;
+    L.size = L.stride = L.width = 1;
+    L.volOut = src->vol;
+    L.fullSize = src->vol + 1; // (the source's background rows are the caller's)
+    L.words = (int)((src->vol + 63) / 64);
+    L.maskOff = 0;
+    L.magicN = magic(src->n);
+    L.magicS = magic(1);
+    maskWords = L.words + 2;
+  }
+  a.nMasks = 1;
+  for (int l = 1; l <= a.nLevels; ++l) {
+    const ChainRec &r = recs[l - 1];
+    PyrLevel &L = a.lv[l];
+    L.kind = r.lv.kind == CH_TERMINAL ? PYR_TERMINAL : PYR_REGIONS;
+    L.nIn = r.lv.nIn;
+    L.nOut = r.lv.nOut;
+    L.size = r.lv.size;
+    L.stride = r.lv.stride;
+    L.width = r.lv.width;
+    L.volOut = r.geom.volOut;
+    L.fullSize = r.lv.fullSize;
+    L.magicN = magic(L.nOut);
+    L.magicS = magic(L.size);
+    L.lenMax = pyr_len_max(L.size, L.stride);
+    L.rules = r.lv.rules;
+    L.capacity = r.lv.capacity;
+    L.ekey = r.lv.ekey;
+    L.erow = r.lv.erow;
+    L.bg = r.lv.bg;
+    L.meta = r.lv.meta;
+    L.boundRows = r.lv.boundRows;
+    L.boundActive = r.lv.boundActive;
+    L.slot = r.lv.slot;
+    if (L.kind == PYR_REGIONS) {
+      L.words = (int)((L.volOut + 63) / 64);
+      L.maskOff = (int)maskWords;
+      maskWords += L.words + 2;
+      a.nMasks = l + 1;
+    }
+  }
+  long long pyrStride = maskWords + (maskWords + 3) / 4;
+  pyrStride = (pyrStride + 1) / 2 * 2;
+  const long long fixedB = PYR_HDR_BYTES + 8 * pyrStride + 5 * 16;
+  if (fixedB + CHAIN_MIN_ARENA > PYR_LDS_MAX)
+    return SCN_OK;
+  a.maskWords = (int)maskWords;
+  a.pyrStride = (int)pyrStride;
+  // pass B's LDS: from the largest samples seen at every level, or all there is
+  long long ldsB = PYR_LDS_MAX;
+  {
+    bool known = !cs->wide && src->seenSample > 0;
+    long long sites = src->seenSample + src->seenSample / 2 + 64;
+    long long need = 14 * sites;
+    for (int l = 1; l < a.nMasks; ++l) {
+      const long long seen = recs[l - 1].out->seenSample;
+      known = known && seen > 0;
+      need += 10 * (seen + seen / 2 + 64);
+    }
+    if (known) {
+      need += fixedB;
+      ldsB = need < ldsB ? need : ldsB;
+    }
+  }
+  ldsB = (ldsB + 15) / 16 * 16;
+  a.ldsBytesB = (int)ldsB;
+  cs->pyrAtMax = ldsB >= PYR_LDS_MAX;
+  *done = true;
+  cs->nPyramids += 1;
+  SCN_TRY(scn_grids_ensure_table(ctx, src)); // pass B reads the source's rows through it
+  a.table = src->table.p;
+  a.dense = (long long)src->batch * src->vol <= SCN_DENSE_MAX_SITES ? src->dense.p : nullptr;
+  a.shift = 64 - src->log2cap;
+  a.mask = (1u << src->log2cap) - 1u;
+  a.bits = src->bits.p;
+  a.bg = src->bg.p;
+  SCN_TRY(cs->pyramid.reserve((size_t)a.batch * (size_t)pyrStride + 2));
+  SCN_TRY(cs->counts.reserve((size_t)a.nMasks * a.batch * 2 + 2));
+  if (!cs->flag.p) {
+    SCN_TRY(cs->flag.reserve(2));
+    SCN_TRY(scn_fill32(ctx, cs->flag.p, 0u, 4));
+  }
+  a.pyramid = cs->pyramid.p;
+  a.counts = cs->counts.p;
+  a.flag = cs->flag.p;
+  a.ticket = (unsigned long long)++ctx->ticket;
+  a.scalars = (long long *)ctx->d_pinned;
+  a.badSites = (const long long *)(ctx->d_scalars + 15);
+  cs->pyrSource = src;
+  {
+    // (above 64 KB of LDS a kernel has to be told so once)
+    static std::once_flag once;
+    static hipError_t attr = hipSuccess;
+    std::call_once(once, [] {
+      const void *k[6] = {reinterpret_cast<const void *>(&k_pyr_masks<1>),
+                          reinterpret_cast<const void *>(&k_pyr_masks<2>),
+                          reinterpret_cast<const void *>(&k_pyr_masks<3>),
+                          reinterpret_cast<const void *>(&k_pyr_rules<1>),
+                          reinterpret_cast<const void *>(&k_pyr_rules<2>),
+                          reinterpret_cast<const void *>(&k_pyr_rules<3>)};
+      for (int i = 0; i < 6 && attr == hipSuccess; ++i)
+        attr = hipFuncSetAttribute(k[i], hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   CHAIN_LDS_MAX);
+    });
+    SCN_HIP_CHECK(attr);
+  }
+  const size_t ldsA = (size_t)(8 * pyrStride + PYR_A_EXTRA);
+  const dim3 grid((unsigned)a.batch);
+  switch (d) {
+  case 1:
+    hipLaunchKernelGGL(k_pyr_masks<1>, grid, dim3(PYR_A_THREADS), ldsA, ctx->stream, a);
+    hipLaunchKernelGGL(k_pyr_rules<1>, grid, dim3(PYR_B_THREADS), (size_t)ldsB, ctx->stream, a);
+    break;
+  case 2:
+    hipLaunchKernelGGL(k_pyr_masks<2>, grid, dim3(PYR_A_THREADS), ldsA, ctx->stream, a);
+    hipLaunchKernelGGL(k_pyr_rules<2>, grid, dim3(PYR_B_THREADS), (size_t)ldsB, ctx->stream, a);
+    break;
+  default:
+    hipLaunchKernelGGL(k_pyr_masks<3>, grid, dim3(PYR_A_THREADS), ldsA, ctx->stream, a);
+    hipLaunchKernelGGL(k_pyr_rules<3>, grid, dim3(PYR_B_THREADS), (size_t)ldsB, ctx->stream, a);
+    break;
+  }
+  SCN_HIP_CHECK(hipGetLastError());
+  return SCN_OK;
+}
+
 int scn_chain_flush(scn_ctx *ctx) {
   ChainState *cs = ctx->chain;
   if (!cs || cs->recs.empty())
@@ -996,6 +1461,12 @@ int scn_chain_flush(scn_ctx *ctx) {
   cs->nPlans += (long long)recs.size();
   ProfScope ps(ctx, SCN_K_RULES);
   scn_grids *src = recs[0].in;
+  if (cs->pyramids) {
+    bool done = false;
+    SCN_TRY(chain_flush_pyramid(ctx, cs, recs, &done));
+    if (done)
+      return SCN_OK;
+  }
   SCN_TRY(scn_grids_ensure_table(ctx, src)); // the kernel reads the source's rows through it
   ChainArgs a;
   memset(&a, 0, sizeof(a));
@@ -1103,9 +1574,22 @@ int scn_chain_flush(scn_ctx *ctx) {
 // what scn_rules_settle learns about a chained plan from its pinned slot
 void scn_chain_settled(scn_ctx *ctx, scn_grids *g, long long sampleMax,
                        bool overflowed) {
+  if (ctx->chain && ctx->chain->pyrSource) {
+    // the source of a chain built from the output side: its largest sample
+    scn_grids *src = ctx->chain->pyrSource;
+    const long long m = ctx->h_pinned[13];
+    if (!overflowed)
+      src->seenSample = m > src->seenSample ? m : src->seenSample;
+    ctx->chain->pyrSource = nullptr;
+  }
   if (overflowed) {
-    if (ctx->chain)
+    if (ctx->chain) {
+      // a sample that does not fit with every layer's sites in LDS at once may
+      // still fit the other construction, which holds two layers at a time
+      if (ctx->chain->wide && ctx->chain->pyrAtMax)
+        ctx->chain->pyramids = false;
       ctx->chain->wide = true;
+    }
     return;
   }
   if (g->planKind == PLAN_REGIONS)

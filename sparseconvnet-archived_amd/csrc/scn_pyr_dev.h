@@ -1,0 +1,746 @@
+// Rule books of a whole net from the output side (square windows without a
+// minimum, Regions.cu:528-653), one sample at a time.
+//
+// gridRules walks the input map in ascending key and creates an output site
+// the first time one of its window's inputs is met (Regions.cu:557-576).  So an
+// output site exists iff its window holds an active input; it is *owned* by
+// the first active input of its window in row-major order; and the outputs get
+// their rows in the order (owner's key, output's key).  Everything a layer's
+// rule book needs therefore follows from occupancy masks alone:
+//
+//   pass A  the masks of all layers of the sample: each is its input mask
+//           OR-ed over the window and thinned by the stride, 64 sites at a time
+//           (pyr_dilate_word), plus a popcount prefix per word (the rank of a
+//           site = its position in iteration order);
+//   pass B  per output site, in five sweeps over ALL layers at once with one
+//           barrier between them: enumerate the sites by rank; find each
+//           site's owner (first set bit of its window) and mark, in the owner's
+//           16-bit ownership mask, which of its candidates this is (an LDS
+//           atomic OR); prefix sums of the owned counts per layer; a site's row
+//           = its owner's base + how many later candidates the owner also owns
+//           (a later candidate is an earlier output); and the rule rows, which
+//           look the input sites' rows up by rank.
+//
+// The code below is the per-lane body of every sweep.  It is written against
+// plain pointers ("lds" is just memory) so that the same text compiles for the
+// device (scn_chain.hip) and for the host, where a harness runs the lanes one
+// after the other with the barriers between sweeps (tests/chain_cpu_harness.cpp).
+#pragma once
+#include <stdint.h>
+#include <type_traits>
+
+#if defined(__HIPCC__)
+#define PYR_FN __host__ __device__ __forceinline__
+#else
+#define PYR_FN static inline
+#endif
+
+#define PYR_MAX_LEVELS 24  // recorded layers of a chain
+#define PYR_HDR_BYTES 5248 // pass B's header and level tables in LDS
+#define PYR_CUBE_MAX 16    // ownership masks are 16 bits
+#define PYR_ROWS_MAX 65000 // rows of one sample at one layer (16-bit rows)
+enum { PYR_REGIONS = 0, PYR_TERMINAL = 1 };
+
+typedef unsigned long long pyr_u64;
+
+// Level 0 is the source grid; level l >= 1 is the output of recorded layer l
+// (input: level l - 1).  A terminal layer can only be the last one.
+struct PyrLevel {
+  int kind;
+  int nIn, nOut, size, stride, width; // width = size^d
+  int words;   // 64-bit words of this level's mask (two spare words follow)
+  int maskOff; // of the mask in a sample's pyramid, in 64-bit words
+  unsigned magicN, magicS; // floor(2^32 / nOut) + 1, floor(2^32 / size) + 1
+  unsigned lenMax; // output sites a piece of the dilation may cover: its windows span at most 128 input sites
+  long long volOut, fullSize;
+  // where the layer's results go
+  int *rules;
+  long long capacity;
+  long long *ekey;
+  int *erow;
+  int *bg;
+  long long *meta;
+  long long boundRows, boundActive;
+  int slot;
+};
+
+struct PyrArgs {
+  int nLevels; // recorded layers: levels 1 .. nLevels
+  int nMasks;  // levels with a mask: 0 .. nMasks - 1 (the terminal layer has none)
+  int batch, d;
+  const int *dense; // row of every site of the source field, or
+  const void *table; // the source's hash table (device builds only)
+  unsigned shift, mask;
+  const pyr_u64 *bits; // the source batch's occupancy mask
+  const int *bg;       // and background rows
+  int maskWords;       // 64-bit words of all masks of a sample, spares included
+  int pyrStride;       // 64-bit words a sample takes in `pyramid`: masks, then 16-bit prefixes
+  pyr_u64 *pyramid;
+  int *counts; // [nLevels + 1][batch][2]: sites, has a background row
+  unsigned long long *flag;
+  unsigned long long ticket;
+  long long *scalars;
+  const long long *badSites;
+  int ldsBytesB; // dynamic LDS pass B is launched with
+  PyrLevel lv[PYR_MAX_LEVELS + 1];
+};
+
+// ---------------------------------------------------------------- bit helpers
+PYR_FN int pyr_popc64(pyr_u64 x) { return __builtin_popcountll(x); }
+PYR_FN int pyr_popc32(unsigned x) { return __builtin_popcount(x); }
+PYR_FN int pyr_ctz64(pyr_u64 x) { return __builtin_ctzll(x); }
+PYR_FN int pyr_ctz32(unsigned x) { return __builtin_ctz(x); }
+PYR_FN unsigned pyr_mulhi(unsigned a, unsigned b) {
+  return (unsigned)(((pyr_u64)a * (pyr_u64)b) >> 32);
+}
+// x / d for x d < 2^32, magic = floor(2^32 / d) + 1
+PYR_FN unsigned pyr_div(unsigned x, unsigned d, unsigned magic) {
+  return d == 1 ? x : pyr_mulhi(x, magic);
+}
+PYR_FN pyr_u64 pyr_even_bits(pyr_u64 x) {
+  x &= 0x5555555555555555ull;
+  x = (x | (x >> 1)) & 0x3333333333333333ull;
+  x = (x | (x >> 2)) & 0x0F0F0F0F0F0F0F0Full;
+  x = (x | (x >> 4)) & 0x00FF00FF00FF00FFull;
+  x = (x | (x >> 8)) & 0x0000FFFF0000FFFFull;
+  x = (x | (x >> 16)) & 0x00000000FFFFFFFFull;
+  return x;
+}
+struct PyrBits128 {
+  pyr_u64 lo, hi;
+};
+// 128 mask bits from position p on (the mask has two spare words)
+PYR_FN PyrBits128 pyr_bits128(const pyr_u64 *bits, unsigned p) {
+  const unsigned w = p >> 6, sh = p & 63;
+  const pyr_u64 a = bits[w], b = bits[w + 1], c = bits[w + 2];
+  PyrBits128 r;
+  r.lo = sh ? (a >> sh) | (b << (64 - sh)) : a;
+  r.hi = sh ? (b >> sh) | (c << (64 - sh)) : b;
+  return r;
+}
+// `len` (<= 16) mask bits from position p on
+PYR_FN unsigned pyr_bits(const pyr_u64 *bits, unsigned p, int len) {
+  const unsigned w = p >> 6, sh = p & 63;
+  pyr_u64 v = bits[w] >> sh;
+  if (sh)
+    v |= bits[w + 1] << (64 - sh);
+  return (unsigned)v & ((1u << len) - 1u);
+}
+PYR_FN unsigned pyr_rank(const pyr_u64 *bits, const unsigned short *pref, unsigned p) {
+  const unsigned w = p >> 6, sh = p & 63;
+  const pyr_u64 below = sh ? (bits[w] & ((1ull << sh) - 1ull)) : 0ull;
+  return pref[w] + (unsigned)pyr_popc64(below);
+}
+
+// Sites travel as packed coordinates: 30 bits in one dimension, 15 bits an axis
+// in two, 10 in three.
+template <int D> struct PyrPacked {
+  static constexpr int BITS = D == 1 ? 30 : (D == 2 ? 15 : 10);
+  static constexpr unsigned MASK = (1u << BITS) - 1u;
+};
+template <int D> PYR_FN unsigned pyr_pack(const int *c) {
+  unsigned v = 0;
+#if defined(__HIPCC__)
+#pragma unroll
+#endif
+  for (int q = 0; q < D; ++q)
+    v |= (unsigned)c[q] << (q * PyrPacked<D>::BITS);
+  return v;
+}
+template <int D> PYR_FN void pyr_unpack(unsigned v, int *c) {
+#if defined(__HIPCC__)
+#pragma unroll
+#endif
+  for (int q = 0; q < D; ++q)
+    c[q] = (int)((v >> (q * PyrPacked<D>::BITS)) & PyrPacked<D>::MASK);
+}
+template <int D> PYR_FN unsigned pyr_key(const int *c, int n) {
+  unsigned k = 0;
+#if defined(__HIPCC__)
+#pragma unroll
+#endif
+  for (int q = 0; q < D; ++q)
+    k = k * (unsigned)n + (unsigned)c[q];
+  return k;
+}
+
+// ------------------------------------------------------------------- pass A
+// Word w of a layer's output mask from its input mask `in` (one sample): the
+// word is cut into the pieces that lie in one row of the output field; a
+// piece ORs the size^(D-1) input rows of its windows (128 bits a request), ORs
+// `size` shifts of that and keeps every stride-th bit.
+// (a piece reads (len - 1) stride + size input bits, at most 128: at most this many sites)
+PYR_FN unsigned pyr_len_max(int size, int stride) {
+  return stride <= 1 ? 64u : (unsigned)((128 - size) / stride + 1);
+}
+// (SIZE, STRIDE: the layer's, when known at compile time; 0: take the arguments)
+template <int D, int SIZE = 0, int STRIDE = 0>
+PYR_FN pyr_u64 pyr_dilate_word(const pyr_u64 *in, int nIn, int nOut, int size_,
+                               int stride_, unsigned volOut, unsigned magicN,
+                               unsigned lenMax, unsigned w) {
+  const int size = SIZE ? SIZE : size_;
+  const int stride = STRIDE ? STRIDE : stride_;
+  unsigned pos = 64u * w;
+  if (pos >= volOut)
+    return 0ull;
+  const unsigned end = pos + 64u < volOut ? pos + 64u : volOut;
+  int j[D];
+  {
+    unsigned k = pos;
+    for (int a = D - 1; a >= 0; --a) {
+      const unsigned up = pyr_div(k, (unsigned)nOut, magicN);
+      j[a] = (int)(k - up * (unsigned)nOut);
+      k = up;
+    }
+  }
+  pyr_u64 res = 0;
+  while (pos < end) {
+    unsigned len = (unsigned)(nOut - j[D - 1]);
+    len = len < end - pos ? len : end - pos;
+    len = len < lenMax ? len : lenMax;
+    const int L = ((int)len - 1) * stride + size;
+    pyr_u64 lo = 0, hi = 0;
+    if (D == 1) {
+      const PyrBits128 x = pyr_bits128(in, (unsigned)(j[0] * stride));
+      lo = x.lo;
+      hi = x.hi;
+    } else if (D == 2) {
+      for (int q0 = 0; q0 < size; ++q0) {
+        const PyrBits128 x = pyr_bits128(
+            in, (unsigned)((j[0] * stride + q0) * nIn + j[D - 1] * stride));
+        lo |= x.lo;
+        hi |= x.hi;
+      }
+    } else {
+      for (int q0 = 0; q0 < size; ++q0)
+        for (int q1 = 0; q1 < size; ++q1) {
+          const PyrBits128 x = pyr_bits128(
+              in, (unsigned)(((j[0] * stride + q0) * nIn + (j[D > 1 ? 1 : 0] * stride + q1)) * nIn +
+                             j[D - 1] * stride));
+          lo |= x.lo;
+          hi |= x.hi;
+        }
+    }
+    // only the L bits of this piece's windows
+    if (L < 64) {
+      lo &= (1ull << L) - 1ull;
+      hi = 0;
+    } else if (L < 128) {
+      hi &= L == 64 ? 0ull : (1ull << (L - 64)) - 1ull;
+    }
+    // bit t: any of the `size` sites from t on
+    pyr_u64 ylo = lo, yhi = hi;
+    for (int q = 1; q < size; ++q) {
+      lo = (lo >> 1) | (hi << 63);
+      hi >>= 1;
+      ylo |= lo;
+      yhi |= hi;
+    }
+    pyr_u64 r;
+    if (stride == 1) {
+      r = ylo;
+    } else if (stride == 2) {
+      r = pyr_even_bits(ylo) | (pyr_even_bits(yhi) << 32);
+    } else {
+      r = 0;
+      for (unsigned t = 0; t < len; ++t) {
+        const unsigned at = t * (unsigned)stride;
+        const pyr_u64 bit = at < 64 ? (ylo >> at) : (yhi >> (at - 64));
+        r |= (bit & 1ull) << t;
+      }
+    }
+    if (len < 64)
+      r &= (1ull << len) - 1ull;
+    res |= r << (pos - 64u * w);
+    pos += len;
+    // the next piece starts where this one ended: carry through the axes
+    j[D - 1] += (int)len;
+    for (int a = D - 1; a > 0; --a)
+      if (j[a] >= nOut) {
+        j[a] = 0;
+        ++j[a - 1];
+      }
+  }
+  return res;
+}
+
+// The same with the usual windows (2/1, 3/2, 2/2, 3/1) compiled in
+template <int D>
+PYR_FN pyr_u64 pyr_dilate_any(const pyr_u64 *in, int nIn, int nOut, int size, int stride, unsigned volOut,
+                              unsigned magicN, unsigned lenMax, unsigned w) {
+  if (D >= 2 && size == 2 && stride == 1)
+    return pyr_dilate_word<D, 2, 1>(in, nIn, nOut, size, stride, volOut, magicN, lenMax, w);
+  if (D >= 2 && size == 3 && stride == 2)
+    return pyr_dilate_word<D, 3, 2>(in, nIn, nOut, size, stride, volOut, magicN, lenMax, w);
+  if (D >= 2 && size == 2 && stride == 2)
+    return pyr_dilate_word<D, 2, 2>(in, nIn, nOut, size, stride, volOut, magicN, lenMax, w);
+  if (D >= 2 && size == 3 && stride == 1)
+    return pyr_dilate_word<D, 3, 1>(in, nIn, nOut, size, stride, volOut, magicN, lenMax, w);
+  return pyr_dilate_word<D, 0, 0>(in, nIn, nOut, size, stride, volOut, magicN, lenMax, w);
+}
+
+// Word w of the source mask of sample b: its slice of the batch's mask
+PYR_FN pyr_u64 pyr_source_word(const pyr_u64 *bits, long long vol, int b, unsigned w) {
+  const long long left = vol - 64ll * w;
+  if (left <= 0)
+    return 0ull;
+  const long long p = (long long)b * vol + 64ll * w;
+  const long long gw = p >> 6;
+  const int sh = (int)(p & 63);
+  pyr_u64 v = bits[gw] >> sh;
+  if (sh)
+    v |= bits[gw + 1] << (64 - sh);
+  if (left < 64)
+    v &= (1ull << left) - 1ull;
+  return v;
+}
+
+// LDS bytes pass B needs for a sample with n[x] sites at level x (x < nMasks)
+PYR_FN long long pyr_lds_need(const PyrArgs &a, const int *n) {
+  long long total = 0;
+  for (int x = 0; x < a.nMasks; ++x)
+    total += n[x];
+  // per site: key (4), row, ownership mask, base (2 each); the source's rows
+  // are the batch's (4 more); every array padded to 16 bytes
+  return PYR_HDR_BYTES + 8ll * a.pyrStride + 10ll * total + 4ll * n[0] + 5 * 16;
+}
+
+// ------------------------------------------------------------------- pass B
+struct PyrHdr {
+  int n[PYR_MAX_LEVELS + 1];       // this sample's sites at level x
+  int hasBg[PYR_MAX_LEVELS + 1];   // and whether it has a background row there
+  int siteOff[PYR_MAX_LEVELS + 2]; // where level x starts in the per-site arrays
+  int itemOff[PYR_MAX_LEVELS + 2]; // output sites of the region layers before layer l (index l)
+  int maxAct[PYR_MAX_LEVELS + 1];  // largest sample of the batch at level x
+  long long actBefore[PYR_MAX_LEVELS + 1], bgBefore[PYR_MAX_LEVELS + 1]; // of the samples before this one
+  long long actAll[PYR_MAX_LEVELS + 1], bgAll[PYR_MAX_LEVELS + 1];
+  int over; // some layer outgrew its bounds, or a sample the LDS
+  int total; // sites of this sample over all levels with a mask
+};
+// What the sweeps need of layer l, once per item: kept in LDS (the kernel
+// arguments are far away for a lane that wants the entry of ITS layer), the
+// geometry in one 16-byte read, the rest as the sweeps come to it.
+struct PyrLv {
+  int size, stride, nIn, nOut;
+  int width;
+  unsigned magicS;
+  int inMaskOff, inSiteOff; // mask and sites of the layer's input (level l - 1)
+  int siteOff, n;           // sites of the layer's output (level l)
+  int bgIn;                 // batch-global row of the input's background row, or -1
+  int inIsSource;           // the input is the source grid: its rows are in srcRow
+  long long rowBase;        // batch-global row of this sample's row 0 at level l
+  long long actBefore;      // entries of the samples before this one at level l
+  long long inRowBase;      // rowBase of the input level (0 for the source)
+  long long volOut;
+  int *rules;
+  long long capacity;
+  long long *ekey;
+  int *erow;
+  long long boundActive;
+  long long pad;
+};
+// What the enumeration needs of level x (x < nMasks), in one 16-byte read
+struct PyrEn {
+  int maskOff, nOut;
+  unsigned magicN;
+  int siteOff;
+};
+#define PYR_LV_AT 1536
+#define PYR_EN_AT (PYR_LV_AT + (PYR_MAX_LEVELS + 1) * (int)sizeof(PyrLv))
+static_assert(sizeof(PyrHdr) <= PYR_LV_AT, "header");
+static_assert(PYR_EN_AT + (PYR_MAX_LEVELS + 1) * sizeof(PyrEn) <= PYR_HDR_BYTES, "level tables");
+static_assert(sizeof(PyrLv) % 16 == 0, "16-byte reads");
+
+// pass B's view of its LDS
+struct PyrLds {
+  PyrHdr *h;
+  PyrLv *lv;             // [nLevels + 1]
+  PyrEn *en;             // [nMasks]
+  pyr_u64 *masks;        // a.maskWords words
+  unsigned short *pref;  // one per mask word
+  unsigned *key;         // [total] packed coordinates by (level, rank)
+  unsigned *srcRow;      // [n[0]] batch-global rows of the source's sites
+  unsigned short *row;   // [total] rows, numbered from 0 within sample and level
+  unsigned *own;         // [total] 16-bit ownership masks, two to a word
+  unsigned short *base;  // [total] rows owned by the sites before, same level
+};
+PYR_FN PyrLds pyr_lds_view(const PyrArgs &a, unsigned char *lds, int total, int n0) {
+  PyrLds v;
+  v.h = reinterpret_cast<PyrHdr *>(lds);
+  v.lv = reinterpret_cast<PyrLv *>(lds + PYR_LV_AT);
+  v.en = reinterpret_cast<PyrEn *>(lds + PYR_EN_AT);
+  unsigned char *p = lds + PYR_HDR_BYTES;
+  v.masks = reinterpret_cast<pyr_u64 *>(p);
+  v.pref = reinterpret_cast<unsigned short *>(p + 8ll * a.maskWords);
+  p += 8ll * a.pyrStride;
+  auto pad = [](long long x) { return (x + 15) / 16 * 16; };
+  v.key = reinterpret_cast<unsigned *>(p);
+  p += pad(4ll * total);
+  v.srcRow = reinterpret_cast<unsigned *>(p);
+  p += pad(4ll * n0);
+  v.row = reinterpret_cast<unsigned short *>(p);
+  p += pad(2ll * total);
+  v.own = reinterpret_cast<unsigned *>(p);
+  p += pad(2ll * total);
+  v.base = reinterpret_cast<unsigned short *>(p);
+  return v;
+}
+
+// Entry l of the level table (lane l of the workgroup fills it, once)
+PYR_FN void pyr_fill_level(const PyrArgs &a, const PyrLds &s, int l, int b) {
+  const PyrHdr *h = s.h;
+  const PyrLevel &L = a.lv[l];
+  PyrLv v;
+  v.size = L.size;
+  v.stride = L.stride;
+  v.nIn = L.nIn;
+  v.nOut = L.nOut;
+  v.width = L.width;
+  v.magicS = L.magicS;
+  v.inMaskOff = a.lv[l - 1].maskOff;
+  v.inSiteOff = h->siteOff[l - 1];
+  const bool region = L.kind == PYR_REGIONS;
+  v.siteOff = region ? h->siteOff[l] : 0;
+  v.n = region ? h->n[l] : 0;
+  const int x = l - 1;
+  v.inIsSource = x == 0;
+  v.inRowBase = x == 0 ? 0 : h->actBefore[x] + h->bgBefore[x];
+  v.bgIn = x == 0 ? a.bg[b] : (h->hasBg[x] ? (int)v.inRowBase + h->n[x] : -1);
+  v.rowBase = region ? h->actBefore[l] + h->bgBefore[l] : 0;
+  v.actBefore = region ? h->actBefore[l] : 0;
+  v.volOut = L.volOut;
+  v.rules = L.rules;
+  v.capacity = L.capacity;
+  v.ekey = L.ekey;
+  v.erow = L.erow;
+  v.boundActive = L.boundActive;
+  s.lv[l] = v;
+}
+
+// Entry x of the enumeration's table (x < nMasks)
+PYR_FN void pyr_fill_en(const PyrArgs &a, unsigned char *lds, int x, int siteOff) {
+  const PyrLevel &L = a.lv[x];
+  PyrEn e;
+  e.maskOff = L.maskOff;
+  e.nOut = L.nOut;
+  e.magicN = L.magicN;
+  e.siteOff = siteOff;
+  reinterpret_cast<PyrEn *>(lds + PYR_EN_AT)[x] = e;
+}
+
+// The layer an item of the flattened sweeps belongs to: a lane's items come in
+// ascending order, so it moves a cursor (starts at 1)
+PYR_FN int pyr_item_level(const PyrHdr *h, int nRegions, int it, int l) {
+  while (l < nRegions && it >= h->itemOff[l + 1])
+    ++l;
+  return l;
+}
+
+// Window geometry known at compile time: S sites a side (in one dimension the
+// side is taken from the layer instead: one row of up to 16 sites), so that
+// the rows of a window live in registers.
+template <int D, int S> struct PyrGeo {
+  static constexpr int ROWS = D == 1 ? 1 : (D == 2 ? S : S * S);
+};
+template <int D, typename F> PYR_FN void pyr_by_size(int size, F f) {
+  if (D == 1 || size == 1) {
+    f(std::integral_constant<int, 1>());
+    return;
+  }
+  switch (size) {
+  case 2:
+    f(std::integral_constant<int, 2>());
+    break;
+  case 3:
+    f(std::integral_constant<int, 3>());
+    break;
+  default:
+    f(std::integral_constant<int, 4>());
+    break;
+  }
+}
+
+// The window of output site j over the input mask: bit k of the result =
+// window offset k (row-major) is active.  rowPos[i] = position of the window's
+// i-th row in the input field.
+template <int D, int S>
+PYR_FN unsigned pyr_window(const pyr_u64 *in, int size, int stride, int nIn, const int *j,
+                           unsigned *rowPos) {
+  const int side = D == 1 ? size : S; // sites of a window row
+  unsigned win = 0;
+  if (D == 1) {
+    rowPos[0] = (unsigned)(j[0] * stride);
+    win = pyr_bits(in, rowPos[0], side);
+  } else if (D == 2) {
+#if defined(__HIPCC__)
+#pragma unroll
+#endif
+    for (int q0 = 0; q0 < S; ++q0) {
+      rowPos[q0] = (unsigned)((j[0] * stride + q0) * nIn + j[D - 1] * stride);
+      win |= pyr_bits(in, rowPos[q0], side) << (q0 * S);
+    }
+  } else {
+#if defined(__HIPCC__)
+#pragma unroll
+#endif
+    for (int q0 = 0; q0 < S; ++q0)
+#if defined(__HIPCC__)
+#pragma unroll
+#endif
+      for (int q1 = 0; q1 < S; ++q1) {
+        const int i = q0 * S + q1;
+        rowPos[i] = (unsigned)(((j[0] * stride + q0) * nIn + (j[D > 1 ? 1 : 0] * stride + q1)) * nIn +
+                               j[D - 1] * stride);
+        win |= pyr_bits(in, rowPos[i], side) << (i * S);
+      }
+  }
+  return win;
+}
+
+// Owner of output site r of the layer v: which window offset (k) and which
+// input rank
+template <int D>
+PYR_FN void pyr_owner(const PyrLv &v, const PyrLds &s, int r, int *kStar, unsigned *ownerRank) {
+  const pyr_u64 *in = s.masks + v.inMaskOff;
+  const unsigned short *pref = s.pref + v.inMaskOff;
+  int j[D];
+  pyr_unpack<D>(s.key[v.siteOff + r], j);
+  const int size = v.size, stride = v.stride, nIn = v.nIn;
+  const unsigned magicS = v.magicS;
+  pyr_by_size<D>(size, [&](auto sz) {
+    constexpr int S = decltype(sz)::value;
+    constexpr int ROWS = PyrGeo<D, S>::ROWS;
+    unsigned rowPos[ROWS];
+    const unsigned win = pyr_window<D, S>(in, size, stride, nIn, j, rowPos);
+    const int k = pyr_ctz32(win); // (an output site's window holds an active input)
+    const int side = D == 1 ? size : S;
+    const int wr = D == 1 ? 0 : (int)pyr_div((unsigned)k, (unsigned)side, magicS);
+    unsigned p = rowPos[0];
+    // (a select over the rows instead of an indexed read of a register array)
+#if defined(__HIPCC__)
+#pragma unroll
+#endif
+    for (int i = 1; i < ROWS; ++i)
+      p = i == wr ? rowPos[i] : p;
+    p += (unsigned)(k - wr * side);
+    *kStar = k;
+    *ownerRank = pyr_rank(in, pref, p);
+  });
+}
+
+#if defined(__HIP_DEVICE_COMPILE__)
+#define PYR_ATOMIC_OR(ptr, v) atomicOr((ptr), (v))
+#else
+#define PYR_ATOMIC_OR(ptr, v) (*(ptr) |= (v))
+#endif
+
+// ---- sweep 0: the ownership masks start empty (no barrier is needed between
+// this and sweep 1: they touch different arrays)
+PYR_FN void pyr_sweep_clear(const PyrLds &s, int t, int T) {
+  for (int i = t; i < (s.h->total + 1) / 2; i += T)
+    s.own[i] = 0u;
+}
+
+// ---- sweep 1: the sites of every level by rank.  A lane takes mask words of
+// the whole pyramid (the spare words between the levels are zero); its words
+// come in ascending order, so the level is a cursor.
+template <int D>
+PYR_FN void pyr_sweep_enumerate(const PyrArgs &a, const PyrLds &s, int t, int T) {
+  int x = 0;
+  for (int g = t; g < a.maskWords; g += T) {
+    pyr_u64 v = s.masks[g];
+    if (!v)
+      continue;
+    while (x + 1 < a.nMasks && g >= s.en[x + 1].maskOff)
+      ++x;
+    const PyrEn e = s.en[x];
+    unsigned r = (unsigned)e.siteOff + s.pref[g];
+    const unsigned k0 = 64u * (unsigned)(g - e.maskOff);
+    while (v) {
+      unsigned k = k0 + (unsigned)pyr_ctz64(v);
+      v &= v - 1;
+      int c[D];
+      for (int q = D - 1; q >= 0; --q) {
+        const unsigned up = pyr_div(k, (unsigned)e.nOut, e.magicN);
+        c[q] = (int)(k - up * (unsigned)e.nOut);
+        k = up;
+      }
+      s.key[r++] = pyr_pack<D>(c);
+    }
+  }
+}
+
+// ---- sweep 2: every output site tells its owner which candidate it is
+template <int D>
+PYR_FN void pyr_sweep_owners(const PyrLds &s, int nRegions, int t, int T) {
+  const PyrHdr *h = s.h;
+  const int items = h->itemOff[nRegions + 1];
+  int l = 1;
+  for (int it = t; it < items; it += T) {
+    l = pyr_item_level(h, nRegions, it, l);
+    const PyrLv &v = s.lv[l];
+    int k;
+    unsigned rank;
+    pyr_owner<D>(v, s, it - h->itemOff[l], &k, &rank);
+    const unsigned at = (unsigned)v.inSiteOff + rank;
+    PYR_ATOMIC_OR(&s.own[at >> 1], 1u << (k + 16 * (int)(at & 1u)));
+  }
+}
+
+PYR_FN unsigned pyr_own_mask(const PyrLds &s, unsigned at) {
+  return (s.own[at >> 1] >> (16 * (at & 1u))) & 0xFFFFu;
+}
+
+// ---- sweep 4: rows of the output sites; the layers' entry lists
+template <int D>
+PYR_FN void pyr_sweep_rows(const PyrLds &s, int nRegions, int b, int t, int T) {
+  const PyrHdr *h = s.h;
+  const int items = h->itemOff[nRegions + 1];
+  int l = 1;
+  for (int it = t; it < items; it += T) {
+    l = pyr_item_level(h, nRegions, it, l);
+    const PyrLv &v = s.lv[l];
+    const int r = it - h->itemOff[l];
+    int k;
+    unsigned rank;
+    pyr_owner<D>(v, s, r, &k, &rank);
+    const unsigned at = (unsigned)v.inSiteOff + rank;
+    // the owner's candidates after this one are the outputs before it
+    const unsigned row = s.base[at] + (unsigned)pyr_popc32(pyr_own_mask(s, at) >> (k + 1));
+    s.row[v.siteOff + r] = (unsigned short)row;
+    int j[D];
+    pyr_unpack<D>(s.key[v.siteOff + r], j);
+    const long long entry = v.actBefore + row;
+    if (entry >= 0 && entry <= v.boundActive) { // (the entry list holds boundActive + 1)
+      v.ekey[entry] = (long long)b * v.volOut + pyr_key<D>(j, v.nOut);
+      v.erow[entry] = (int)(v.rowBase + row);
+    }
+  }
+}
+
+// batch-global row of the input site with rank `rank` of layer v
+PYR_FN int pyr_in_row(const PyrLv &v, const PyrLds &s, unsigned rank) {
+  if (v.inIsSource)
+    return (int)s.srcRow[rank];
+  return (int)v.inRowBase + (int)s.row[v.inSiteOff + rank];
+}
+// batch-global row of level x's background row of this sample (-1: none)
+PYR_FN int pyr_bg_row(const PyrArgs &a, const PyrLds &s, int x, int b) {
+  const PyrHdr *h = s.h;
+  if (x == 0)
+    return a.bg[b];
+  return h->hasBg[x] ? (int)(h->actBefore[x] + h->bgBefore[x]) + h->n[x] : -1;
+}
+
+// ---- sweep 5: rule rows
+template <int D>
+PYR_FN void pyr_sweep_rules(const PyrLds &s, int nRegions, int t, int T) {
+  const PyrHdr *h = s.h;
+  const int items = h->itemOff[nRegions + 1];
+  int l = 1;
+  for (int it = t; it < items; it += T) {
+    l = pyr_item_level(h, nRegions, it, l);
+    const PyrLv &v = s.lv[l];
+    if (!v.rules)
+      continue;
+    const int r = it - h->itemOff[l];
+    const pyr_u64 *in = s.masks + v.inMaskOff;
+    const unsigned short *pref = s.pref + v.inMaskOff;
+    int j[D];
+    pyr_unpack<D>(s.key[v.siteOff + r], j);
+    const int bgIn = v.bgIn;
+    const long long row = v.rowBase + s.row[v.siteOff + r];
+    if (row < 0 || (row + 1) * v.width > v.capacity)
+      continue; // (cannot happen while counts and masks agree; never write outside the caller's buffer)
+    int *dst = v.rules + row * v.width;
+    const int size = v.size, stride = v.stride, nIn = v.nIn;
+    pyr_by_size<D>(size, [&](auto sz) {
+      constexpr int S = decltype(sz)::value;
+      constexpr int ROWS = PyrGeo<D, S>::ROWS;
+      unsigned rowPos[ROWS];
+      const unsigned win = pyr_window<D, S>(in, size, stride, nIn, j, rowPos);
+      const int side = D == 1 ? size : S;
+#if defined(__HIPCC__)
+#pragma unroll
+#endif
+      for (int i = 0; i < ROWS; ++i) {
+        const unsigned present = (win >> (i * side)) & ((1u << side) - 1u);
+        // the active sites of a window row are neighbours in rank
+        unsigned rank = present ? pyr_rank(in, pref, rowPos[i]) : 0u;
+        for (int q = 0; q < side; ++q) {
+          int val = bgIn;
+          if ((present >> q) & 1u)
+            val = pyr_in_row(v, s, rank++);
+          dst[i * side + q] = val;
+        }
+      }
+    });
+  }
+}
+
+// ---- the all-background rows, backgroundCol, the terminal layer's rules
+PYR_FN void pyr_sweep_tail(const PyrArgs &a, const PyrLds &s, int b, int t, int T) {
+  const PyrHdr *h = s.h;
+  for (int l = 1; l <= a.nLevels; ++l) {
+    const PyrLevel &L = a.lv[l];
+    if (L.kind == PYR_TERMINAL) {
+      // terminalGridPoolingRules (TerminalPoolingLayer.cu:8-20): the rows in
+      // iteration order, or the background row of a sample without sites;
+      // padded with -1 to the batch's largest sample (:90-96)
+      const int x = l - 1;
+      const PyrLv &v = s.lv[l];
+      const long long width = h->maxAct[x] > 1 ? h->maxAct[x] : 1;
+      if (L.rules && ((long long)b + 1) * width <= L.capacity) {
+        const int n = h->n[x];
+        int *dst = L.rules + (long long)b * width;
+        for (long long i = t; i < width; i += T) {
+          int val = -1;
+          if (n == 0 && i == 0)
+            val = v.bgIn;
+          else if (i < n)
+            val = pyr_in_row(v, s, (unsigned)i);
+          dst[i] = val;
+        }
+      }
+      if (t == 0) { // the output grid: site 0 of sample b is row b
+        L.ekey[b] = b;
+        L.erow[b] = b;
+        L.bg[b] = -1;
+      }
+      continue;
+    }
+    const int bgOut = pyr_bg_row(a, s, l, b);
+    if (h->hasBg[l] && L.rules && bgOut >= 0 &&
+        ((long long)bgOut + 1) * L.width <= L.capacity) { // Regions.cu:647-652
+      const int bgIn = s.lv[l].bgIn;
+      int *dst = L.rules + (long long)bgOut * L.width;
+      for (int q = t; q < L.width; q += T)
+        dst[q] = bgIn;
+    }
+    if (t == 0)
+      L.bg[b] = bgOut;
+  }
+}
+
+// What a layer reports: sites, active sites, whether it outgrew its bounds,
+// and the terminal width or the largest sample (the header holds the sums)
+struct PyrReport {
+  long long nSites, nActive, over, extra;
+};
+PYR_FN PyrReport pyr_report(const PyrArgs &a, const PyrHdr *h, int l) {
+  const PyrLevel &L = a.lv[l];
+  PyrReport r;
+  if (L.kind == PYR_TERMINAL) {
+    const long long width = h->maxAct[l - 1] > 1 ? h->maxAct[l - 1] : 1;
+    r.nSites = r.nActive = a.batch;
+    r.extra = width;
+    r.over = width > L.boundRows || (L.rules && width * a.batch > L.capacity);
+  } else {
+    r.nSites = h->actAll[l] + h->bgAll[l];
+    r.nActive = h->actAll[l];
+    r.extra = h->maxAct[l];
+    r.over = r.nSites > L.boundRows || r.nActive > L.boundActive ||
+             (L.rules && r.nSites * L.width > L.capacity);
+  }
+  return r;
+}

@@ -261,3 +261,46 @@ def test_benchmark_pass_against_oracle(scn, distinct, inputs_on_host):
         assert np.array_equal(s, os_) and np.array_equal(k, ok) and np.array_equal(r, or_) and np.array_equal(b, ob)
     del keep
     net.close()
+
+
+def test_ten_producers_several_passes_against_oracle(scn):
+    """Ten producer threads, three batches (100, 100, 50) in flight at once on streams of their own, four passes over
+    the same dataset: a slot's first batch is planned layer by layer, its second from recorded plans with the widest
+    LDS arena, later ones with an arena sized by what the slot has seen -- with the chains of the three batches
+    running side by side.  Every batch of every pass: row counts and rule books of all interfaces bit for bit, and
+    the probabilities against float64."""
+    import oracle_net
+    from sparseconvnet_archived_amd import hostapi, synthetic
+    cfg = synthetic.config(2)
+    net = hostapi.Net(cfg.dimension, cfg.nInputFeatures, cfg.nClasses, threads=10)
+    ora = oracle_net.Net(cfg.dimension, cfg.nInputFeatures, cfg.nClasses)
+    cfg.build(net)
+    cfg.build(ora)
+    net.setFusedConvolutions(True)
+    for i, (W, Bv, pr) in synthetic.he_normal_weights(net.layers(), 4).items():
+        net.set_weights(i, W, Bv, pr)
+        ora.set_weights(i, W, Bv, pr)
+    samples = synthetic.make_samples(cfg, 11, batch=250)
+    ds = hostapi.Dataset("three", cfg.nInputFeatures, cfg.nClasses, hostapi.TESTBATCH)
+    for pts, f, label in samples:
+        ds.add_points(cfg.dimension, cfg.lattice, pts, f, label)
+    wants, p64 = [], []
+    for lo in range(0, 250, 100):
+        chunk = samples[lo:lo + 100]
+        S, K, R, bg, feats, n = synthetic.codify(chunk, cfg.dimension, cfg.lattice, net.inputSpatialSize,
+                                                 cfg.nInputFeatures)
+        wants.append(ora.forward(len(chunk), S, K, R, bg, feats, n, np.array([s[2] for s in chunk], np.int32)))
+        p64.append(ora.forward64(wants[-1]))
+    for p in range(4):
+        chains = net.chain_counts()[0]
+        net.begin(ds, 100)
+        for bi, want in enumerate(wants):
+            assert net.next_batch()
+            for i, wi in enumerate(want["interfaces"]):
+                gi = net.interface(i, want_features=False)
+                assert gi["nSpatialSites"] == wi["nSpatialSites"], "pass %d batch %d interface %d" % (p, bi, i)
+                assert np.array_equal(gi["rules"], wi["rules"]), "pass %d batch %d interface %d" % (p, bi, i)
+            assert_probabilities(net.batch_outputs()["probabilities"], p64[bi])
+        assert not net.next_batch()
+        assert net.chain_counts()[0] == chains + (3 if p else 0)
+    net.close()
