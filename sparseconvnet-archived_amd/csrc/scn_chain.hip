@@ -792,7 +792,7 @@ __global__ void __launch_bounds__(PLACE_THREADS) k_chain_place(ChainArgs a) {
 #define PYR_A_BARRIER() lds_barrier()
 // keeps a wavefront-uniform value in a scalar register from here on
 #define PYR_PIN(v) asm volatile("" : "+s"(v))
-#define PYR_B_THREADS 512
+#define PYR_B_THREADS 1024
 static_assert(sizeof(PyrArgs) <= 4096, "kernel arguments");
 
 // A layer's geometry as k_pyr_masks keeps it in LDS: one broadcast read a layer
@@ -800,29 +800,22 @@ static_assert(sizeof(PyrArgs) <= 4096, "kernel arguments");
 struct PyrGeoA {
   int nIn, nOut, size, stride;
   int words, offIn, offOut;
-  unsigned volOut, magicN, lenMax;
-  int pad[2];
+  unsigned magicN, seg, segs, magicSegs;
+  int pad;
 };
 static_assert(sizeof(PyrGeoA) == 48, "three 16-byte reads");
 #define PYR_A_EXTRA (128 + (PYR_MAX_LEVELS + 1) * (int)sizeof(PyrGeoA)) // counts, geometry: after the pyramid
 
-// One level of the pyramid by one wavefront: the words of the output mask (64 at
-// a time), and their rank prefixes in the same go; the level's site count comes back
-template <int D>
-__device__ __forceinline__ unsigned pyr_level(const PyrGeoA &g, pyr_u64 *masks, unsigned short *pref, int lane) {
-  const pyr_u64 *in = masks + g.offIn;
+// Rank prefixes of `words` mask words (the two spare words included) by one
+// wavefront; the number of set bits comes back
+__device__ __forceinline__ unsigned pyr_prefixes(const pyr_u64 *m, unsigned short *p, int words, int lane) {
   unsigned carry = 0;
-  for (int w0 = 0; w0 < g.words + 2; w0 += 64) {
+  for (int w0 = 0; w0 < words + 2; w0 += 64) {
     const int w = w0 + lane;
-    const pyr_u64 v = w < g.words ? pyr_dilate_any<D>(in, g.nIn, g.nOut, g.size, g.stride, g.volOut, g.magicN, g.lenMax,
-                                                      (unsigned)w)
-                                  : 0ull;
-    const unsigned pc = (unsigned)pyr_popc64(v);
+    const unsigned pc = w < words ? (unsigned)pyr_popc64(m[w]) : 0u;
     const unsigned incl = wave_scan_incl_dpp(pc);
-    if (w < g.words + 2) {
-      masks[g.offOut + w] = v;
-      pref[g.offOut + w] = (unsigned short)(carry + incl - pc);
-    }
+    if (w < words + 2)
+      p[w] = (unsigned short)(carry + incl - pc);
     carry += wave_last(incl);
   }
   return carry;
@@ -847,35 +840,47 @@ __global__ void __launch_bounds__(PYR_A_THREADS) k_pyr_masks(PyrArgs a) {
     g.words = L.words;
     g.offIn = a.lv[t - 1].maskOff;
     g.offOut = L.maskOff;
-    g.volOut = (unsigned)L.volOut;
     g.magicN = L.magicN;
-    g.lenMax = L.lenMax;
-    g.pad[0] = g.pad[1] = 0;
+    g.seg = L.seg;
+    g.segs = L.segs;
+    g.magicSegs = L.magicSegs;
+    g.pad = 0;
     geo[t] = g;
   }
-  { // level 0: the sample's slice of the source mask
+  { // level 0: the sample's slice of the source mask, four words a lane at a time
     const PyrLevel &L = a.lv[0];
     const int words = L.words;
     const long long vol = L.volOut;
     unsigned carry = 0;
-    for (int w0 = 0; w0 < words + 2; w0 += 64) {
-      const int w = w0 + t;
-      const pyr_u64 v = w < words ? pyr_source_word(a.bits, vol, b, (unsigned)w) : 0ull;
-      const unsigned pc = (unsigned)pyr_popc64(v);
-      const unsigned incl = wave_scan_incl_dpp(pc);
-      if (w < words + 2) {
-        masks[w] = v;
-        pref[w] = (unsigned short)(carry + incl - pc);
+    for (int w0 = 0; w0 < words + 2; w0 += 256) {
+      pyr_u64 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int w = w0 + 64 * u + t;
+        v[u] = w < words ? pyr_source_word(a.bits, vol, b, (unsigned)w) : 0ull;
       }
-      carry += wave_last(incl);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int w = w0 + 64 * u + t;
+        const unsigned pc = (unsigned)pyr_popc64(v[u]);
+        const unsigned incl = wave_scan_incl_dpp(pc);
+        if (w < words + 2) {
+          masks[w] = v[u];
+          pref[w] = (unsigned short)(carry + incl - pc);
+        }
+        carry += wave_last(incl);
+      }
     }
     if (t == 0)
       cnt[0] = (int)carry;
+    // the other levels start empty: their pieces are OR-ed in
+    for (int w = words + 2 + t; w < a.maskWords; w += PYR_A_THREADS)
+      masks[w] = 0ull;
   }
   PYR_A_BARRIER();
   for (int x = 1; x < a.nMasks; ++x) {
     // (wavefront-uniform values, told to the compiler: the loops over a window's
-    // rows and a word's pieces then branch on scalars)
+    // rows then branch on scalars)
     PyrGeoA g = geo[x];
     g.nIn = __builtin_amdgcn_readfirstlane(g.nIn);
     g.nOut = __builtin_amdgcn_readfirstlane(g.nOut);
@@ -884,18 +889,24 @@ __global__ void __launch_bounds__(PYR_A_THREADS) k_pyr_masks(PyrArgs a) {
     g.words = __builtin_amdgcn_readfirstlane(g.words);
     g.offIn = __builtin_amdgcn_readfirstlane(g.offIn);
     g.offOut = __builtin_amdgcn_readfirstlane(g.offOut);
-    g.volOut = (unsigned)__builtin_amdgcn_readfirstlane((int)g.volOut);
     g.magicN = (unsigned)__builtin_amdgcn_readfirstlane((int)g.magicN);
-    g.lenMax = (unsigned)__builtin_amdgcn_readfirstlane((int)g.lenMax);
-    const unsigned n = pyr_level<D>(g, masks, pref, t);
+    g.seg = (unsigned)__builtin_amdgcn_readfirstlane((int)g.seg);
+    g.segs = (unsigned)__builtin_amdgcn_readfirstlane((int)g.segs);
+    g.magicSegs = (unsigned)__builtin_amdgcn_readfirstlane((int)g.magicSegs);
+    pyr_sweep_dilate<D>(masks + g.offIn, masks + g.offOut, g.nIn, g.nOut, g.size, g.stride, g.magicN, g.seg, g.segs,
+                        g.magicSegs, t, PYR_A_THREADS);
+    PYR_A_BARRIER();
+    const unsigned n = pyr_prefixes(masks + g.offOut, pref + g.offOut, g.words, t);
     if (t == 0)
       cnt[x] = (int)n;
     PYR_A_BARRIER();
   }
-  pyr_u64 *dst = a.pyramid + (long long)b * a.pyrStride;
-  const pyr_u64 *src = reinterpret_cast<const pyr_u64 *>(lds);
-  for (int i = t; i < a.pyrStride; i += PYR_A_THREADS)
-    dst[i] = src[i];
+  {
+    uint4 *dst = reinterpret_cast<uint4 *>(a.pyramid + (long long)b * a.pyrStride);
+    const uint4 *src = reinterpret_cast<const uint4 *>(lds);
+    for (int i = t; i < a.pyrStride / 2; i += PYR_A_THREADS)
+      dst[i] = src[i];
+  }
   if (t < a.nMasks) {
     int *c = a.counts + ((long long)t * a.batch + b) * 2;
     c[0] = cnt[t];
@@ -918,6 +929,15 @@ __global__ void __launch_bounds__(PYR_B_THREADS) k_pyr_rules(PyrArgs a) {
   constexpr int T = PYR_B_THREADS;
   const bool gaveUp = *reinterpret_cast<volatile unsigned long long *>(a.flag) == a.ticket;
   const int nRegions = a.nMasks - 1;
+  // lane t keeps layer t's arguments from here on: fetched while the masks
+  // come in, not when the level table wants them
+  PyrLevel mine;
+  int inMaskOff = 0;
+  const int bgSource = a.bg[b];
+  if (t <= a.nLevels) {
+    mine = a.lv[t];
+    inMaskOff = a.lv[t > 0 ? t - 1 : 0].maskOff;
+  }
   if (t == 0)
     h->over = 0;
   { // the sample's masks and prefixes
@@ -969,7 +989,7 @@ __global__ void __launch_bounds__(PYR_B_THREADS) k_pyr_rules(PyrArgs a) {
       sum += h->n[x];
     h->siteOff[t] = sum;
     if (t < a.nMasks)
-      pyr_fill_en(a, lds, t, sum);
+      pyr_fill_en(mine, lds, t, sum);
     if (t == a.nMasks)
       h->total = sum;
   }
@@ -979,15 +999,15 @@ __global__ void __launch_bounds__(PYR_B_THREADS) k_pyr_rules(PyrArgs a) {
       sum += h->n[l];
     h->itemOff[t] = sum;
   }
-  if (t >= 1 && t <= a.nLevels && pyr_report(a, h, t).over)
+  if (t >= 1 && t <= a.nLevels && pyr_report(a, mine, h, t).over)
     atomicOr(&h->over, 1);
   if (t == 0 && pyr_lds_need(a, h->n) > a.ldsBytesB)
     atomicOr(&h->over, 2);
   lds_barrier();
   const bool over = h->over != 0 || gaveUp;
   if (b == 0 && t >= 1 && t <= a.nLevels) {
-    const PyrLevel &L = a.lv[t];
-    const PyrReport r = pyr_report(a, h, t);
+    const PyrLevel &L = mine;
+    const PyrReport r = pyr_report(a, mine, h, t);
     L.meta[META_SITES] = over ? 0 : r.nSites;
     L.meta[META_ACTIVE] = over ? 0 : r.nActive;
     L.meta[META_OVERFLOW] = over;
@@ -1006,7 +1026,7 @@ __global__ void __launch_bounds__(PYR_B_THREADS) k_pyr_rules(PyrArgs a) {
     return;
   const PyrLds s = pyr_lds_view(a, lds, h->total, h->n[0]);
   if (t >= 1 && t <= a.nLevels)
-    pyr_fill_level(a, s, t, b);
+    pyr_fill_level(mine, inMaskOff, bgSource, s, t);
   pyr_sweep_clear(s, t, T);
   pyr_sweep_enumerate<D>(a, s, t, T);
   lds_barrier();
@@ -1349,7 +1369,7 @@ static int chain_flush_pyramid(scn_ctx *ctx, ChainState *cs, std::vector<ChainRe
     L.fullSize = r.lv.fullSize;
     L.magicN = magic(L.nOut);
     L.magicS = magic(L.size);
-    L.lenMax = pyr_len_max(L.size, L.stride);
+    pyr_set_pieces(L);
     L.rules = r.lv.rules;
     L.capacity = r.lv.capacity;
     L.ekey = r.lv.ekey;
@@ -1368,7 +1388,7 @@ static int chain_flush_pyramid(scn_ctx *ctx, ChainState *cs, std::vector<ChainRe
   }
   long long pyrStride = maskWords + (maskWords + 3) / 4;
   pyrStride = (pyrStride + 1) / 2 * 2;
-  const long long fixedB = PYR_HDR_BYTES + 8 * pyrStride + 5 * 16;
+  const long long fixedB = PYR_HDR_BYTES + 8 * pyrStride + 6 * 16;
   if (fixedB + CHAIN_MIN_ARENA > PYR_LDS_MAX)
     return SCN_OK;
   a.maskWords = (int)maskWords;
@@ -1378,11 +1398,11 @@ static int chain_flush_pyramid(scn_ctx *ctx, ChainState *cs, std::vector<ChainRe
   {
     bool known = !cs->wide && src->seenSample > 0;
     long long sites = src->seenSample + src->seenSample / 2 + 64;
-    long long need = 14 * sites;
+    long long need = 15 * sites;
     for (int l = 1; l < a.nMasks; ++l) {
       const long long seen = recs[l - 1].out->seenSample;
       known = known && seen > 0;
-      need += 10 * (seen + seen / 2 + 64);
+      need += 11 * (seen + seen / 2 + 64);
     }
     if (known) {
       need += fixedB;

@@ -9,9 +9,9 @@
 // rule book needs therefore follows from occupancy masks alone:
 //
 //   pass A  the masks of all layers of the sample: each is its input mask
-//           OR-ed over the window and thinned by the stride, 64 sites at a time
-//           (pyr_dilate_word), plus a popcount prefix per word (the rank of a
-//           site = its position in iteration order);
+//           OR-ed over the window and thinned by the stride, up to 64 sites of
+//           a row at a time (pyr_dilate_pieces), plus a popcount prefix per
+//           word (the rank of a site = its position in iteration order);
 //   pass B  per output site, in five sweeps over ALL layers at once with one
 //           barrier between them: enumerate the sites by rank; find each
 //           site's owner (first set bit of its window) and mark, in the owner's
@@ -51,7 +51,7 @@ struct PyrLevel {
   int words;   // 64-bit words of this level's mask (two spare words follow)
   int maskOff; // of the mask in a sample's pyramid, in 64-bit words
   unsigned magicN, magicS; // floor(2^32 / nOut) + 1, floor(2^32 / size) + 1
-  unsigned lenMax; // output sites a piece of the dilation may cover: its windows span at most 128 input sites
+  unsigned seg;    // output sites a piece of the dilation covers (the last piece of a row: what is left)
   long long volOut, fullSize;
   // where the layer's results go
   int *rules;
@@ -62,6 +62,7 @@ struct PyrLevel {
   long long *meta;
   long long boundRows, boundActive;
   int slot;
+  unsigned segs, magicSegs; // pieces in a row of the output field, floor(2^32 / segs) + 1
 };
 
 struct PyrArgs {
@@ -165,58 +166,63 @@ template <int D> PYR_FN unsigned pyr_key(const int *c, int n) {
 }
 
 // ------------------------------------------------------------------- pass A
-// Word w of a layer's output mask from its input mask `in` (one sample): the
-// word is cut into the pieces that lie in one row of the output field; a
-// piece ORs the size^(D-1) input rows of its windows (128 bits a request), ORs
-// `size` shifts of that and keeps every stride-th bit.
-// (a piece reads (len - 1) stride + size input bits, at most 128: at most this many sites)
-PYR_FN unsigned pyr_len_max(int size, int stride) {
-  return stride <= 1 ? 64u : (unsigned)((128 - size) / stride + 1);
+// A layer's output mask from its input mask (one sample), a lane per PIECE: a
+// run of up to `seg` neighbouring output sites in one row of the output field.
+// The piece ORs the size^(D-1) input rows of its windows (128 bits a request),
+// ORs `size` shifts of that, keeps every stride-th bit and ORs the result into
+// the one or two words of the output mask it falls in (which start as zero).
+// (a piece reads (len - 1) stride + size input bits, at most 128, and gives at
+// most 64 bits)
+PYR_FN unsigned pyr_seg(int size, int stride) {
+  const unsigned most = stride <= 1 ? 64u : (unsigned)((128 - size) / stride + 1);
+  return most < 64u ? most : 64u;
 }
+PYR_FN void pyr_set_pieces(PyrLevel &L) {
+  L.seg = pyr_seg(L.size, L.stride);
+  L.segs = ((unsigned)L.nOut + L.seg - 1u) / L.seg;
+  L.magicSegs = (unsigned)((1ull << 32) / (L.segs > 0 ? L.segs : 1u) + 1ull);
+}
+#if defined(__HIPCC__) && defined(__HIP_DEVICE_COMPILE__)
+#define PYR_ATOMIC_OR64(ptr, v) atomicOr(reinterpret_cast<unsigned long long *>(ptr), (unsigned long long)(v))
+#else
+#define PYR_ATOMIC_OR64(ptr, v) (*(ptr) |= (v))
+#endif
 // (SIZE, STRIDE: the layer's, when known at compile time; 0: take the arguments)
-template <int D, int SIZE = 0, int STRIDE = 0>
-PYR_FN pyr_u64 pyr_dilate_word(const pyr_u64 *in, int nIn, int nOut, int size_,
-                               int stride_, unsigned volOut, unsigned magicN,
-                               unsigned lenMax, unsigned w) {
+template <int D, int SIZE, int STRIDE>
+PYR_FN void pyr_dilate_pieces(const pyr_u64 *in, pyr_u64 *out, int nIn, int nOut, int size_, int stride_,
+                              unsigned magicN, unsigned seg, unsigned segs, unsigned magicSegs, int t, int T) {
   const int size = SIZE ? SIZE : size_;
   const int stride = STRIDE ? STRIDE : stride_;
-  unsigned pos = 64u * w;
-  if (pos >= volOut)
-    return 0ull;
-  const unsigned end = pos + 64u < volOut ? pos + 64u : volOut;
-  int j[D];
-  {
-    unsigned k = pos;
-    for (int a = D - 1; a >= 0; --a) {
-      const unsigned up = pyr_div(k, (unsigned)nOut, magicN);
-      j[a] = (int)(k - up * (unsigned)nOut);
-      k = up;
-    }
-  }
-  pyr_u64 res = 0;
-  while (pos < end) {
-    unsigned len = (unsigned)(nOut - j[D - 1]);
-    len = len < end - pos ? len : end - pos;
-    len = len < lenMax ? len : lenMax;
+  unsigned rows = 1;
+  for (int q = 0; q < D - 1; ++q)
+    rows *= (unsigned)nOut;
+  const unsigned pieces = rows * segs;
+  for (unsigned p = (unsigned)t; p < pieces; p += (unsigned)T) {
+    const unsigned row = pyr_div(p, segs, magicSegs);
+    const unsigned jl = (p - row * segs) * seg; // the piece's first site along the last axis
+    unsigned len = (unsigned)nOut - jl;
+    len = len < seg ? len : seg;
     const int L = ((int)len - 1) * stride + size;
     pyr_u64 lo = 0, hi = 0;
     if (D == 1) {
-      const PyrBits128 x = pyr_bits128(in, (unsigned)(j[0] * stride));
+      const PyrBits128 x = pyr_bits128(in, jl * (unsigned)stride);
       lo = x.lo;
       hi = x.hi;
     } else if (D == 2) {
       for (int q0 = 0; q0 < size; ++q0) {
-        const PyrBits128 x = pyr_bits128(
-            in, (unsigned)((j[0] * stride + q0) * nIn + j[D - 1] * stride));
+        const PyrBits128 x = pyr_bits128(in, ((row * (unsigned)stride + (unsigned)q0) * (unsigned)nIn +
+                                              jl * (unsigned)stride));
         lo |= x.lo;
         hi |= x.hi;
       }
     } else {
+      const unsigned j0 = pyr_div(row, (unsigned)nOut, magicN), j1 = row - j0 * (unsigned)nOut;
       for (int q0 = 0; q0 < size; ++q0)
         for (int q1 = 0; q1 < size; ++q1) {
           const PyrBits128 x = pyr_bits128(
-              in, (unsigned)(((j[0] * stride + q0) * nIn + (j[D > 1 ? 1 : 0] * stride + q1)) * nIn +
-                             j[D - 1] * stride));
+              in, ((j0 * (unsigned)stride + (unsigned)q0) * (unsigned)nIn + (j1 * (unsigned)stride + (unsigned)q1)) *
+                          (unsigned)nIn +
+                      jl * (unsigned)stride);
           lo |= x.lo;
           hi |= x.hi;
         }
@@ -243,40 +249,36 @@ PYR_FN pyr_u64 pyr_dilate_word(const pyr_u64 *in, int nIn, int nOut, int size_,
       r = pyr_even_bits(ylo) | (pyr_even_bits(yhi) << 32);
     } else {
       r = 0;
-      for (unsigned t = 0; t < len; ++t) {
-        const unsigned at = t * (unsigned)stride;
+      for (unsigned i = 0; i < len; ++i) {
+        const unsigned at = i * (unsigned)stride;
         const pyr_u64 bit = at < 64 ? (ylo >> at) : (yhi >> (at - 64));
-        r |= (bit & 1ull) << t;
+        r |= (bit & 1ull) << i;
       }
     }
     if (len < 64)
       r &= (1ull << len) - 1ull;
-    res |= r << (pos - 64u * w);
-    pos += len;
-    // the next piece starts where this one ended: carry through the axes
-    j[D - 1] += (int)len;
-    for (int a = D - 1; a > 0; --a)
-      if (j[a] >= nOut) {
-        j[a] = 0;
-        ++j[a - 1];
-      }
+    if (!r)
+      continue;
+    const unsigned pos = row * (unsigned)nOut + jl, w = pos >> 6, sh = pos & 63u;
+    PYR_ATOMIC_OR64(&out[w], r << sh);
+    if (sh && (r >> (64u - sh)))
+      PYR_ATOMIC_OR64(&out[w + 1], r >> (64u - sh));
   }
-  return res;
 }
-
 // The same with the usual windows (2/1, 3/2, 2/2, 3/1) compiled in
 template <int D>
-PYR_FN pyr_u64 pyr_dilate_any(const pyr_u64 *in, int nIn, int nOut, int size, int stride, unsigned volOut,
-                              unsigned magicN, unsigned lenMax, unsigned w) {
+PYR_FN void pyr_sweep_dilate(const pyr_u64 *in, pyr_u64 *out, int nIn, int nOut, int size, int stride,
+                             unsigned magicN, unsigned seg, unsigned segs, unsigned magicSegs, int t, int T) {
   if (D >= 2 && size == 2 && stride == 1)
-    return pyr_dilate_word<D, 2, 1>(in, nIn, nOut, size, stride, volOut, magicN, lenMax, w);
-  if (D >= 2 && size == 3 && stride == 2)
-    return pyr_dilate_word<D, 3, 2>(in, nIn, nOut, size, stride, volOut, magicN, lenMax, w);
-  if (D >= 2 && size == 2 && stride == 2)
-    return pyr_dilate_word<D, 2, 2>(in, nIn, nOut, size, stride, volOut, magicN, lenMax, w);
-  if (D >= 2 && size == 3 && stride == 1)
-    return pyr_dilate_word<D, 3, 1>(in, nIn, nOut, size, stride, volOut, magicN, lenMax, w);
-  return pyr_dilate_word<D, 0, 0>(in, nIn, nOut, size, stride, volOut, magicN, lenMax, w);
+    pyr_dilate_pieces<D, 2, 1>(in, out, nIn, nOut, size, stride, magicN, seg, segs, magicSegs, t, T);
+  else if (D >= 2 && size == 3 && stride == 2)
+    pyr_dilate_pieces<D, 3, 2>(in, out, nIn, nOut, size, stride, magicN, seg, segs, magicSegs, t, T);
+  else if (D >= 2 && size == 2 && stride == 2)
+    pyr_dilate_pieces<D, 2, 2>(in, out, nIn, nOut, size, stride, magicN, seg, segs, magicSegs, t, T);
+  else if (D >= 2 && size == 3 && stride == 1)
+    pyr_dilate_pieces<D, 3, 1>(in, out, nIn, nOut, size, stride, magicN, seg, segs, magicSegs, t, T);
+  else
+    pyr_dilate_pieces<D, 0, 0>(in, out, nIn, nOut, size, stride, magicN, seg, segs, magicSegs, t, T);
 }
 
 // Word w of the source mask of sample b: its slice of the batch's mask
@@ -300,9 +302,10 @@ PYR_FN long long pyr_lds_need(const PyrArgs &a, const int *n) {
   long long total = 0;
   for (int x = 0; x < a.nMasks; ++x)
     total += n[x];
-  // per site: key (4), row, ownership mask, base (2 each); the source's rows
-  // are the batch's (4 more); every array padded to 16 bytes
-  return PYR_HDR_BYTES + 8ll * a.pyrStride + 10ll * total + 4ll * n[0] + 5 * 16;
+  // per site: key (4), row, ownership mask, base (2 each), which candidate of
+  // its owner it is (1); the source's rows are the batch's (4 more); every
+  // array padded to 16 bytes
+  return PYR_HDR_BYTES + 8ll * a.pyrStride + 11ll * total + 4ll * n[0] + 6 * 16;
 }
 
 // ------------------------------------------------------------------- pass B
@@ -327,7 +330,7 @@ struct PyrLv {
   int inMaskOff, inSiteOff; // mask and sites of the layer's input (level l - 1)
   int siteOff, n;           // sites of the layer's output (level l)
   int bgIn;                 // batch-global row of the input's background row, or -1
-  int inIsSource;           // the input is the source grid: its rows are in srcRow
+  int flags;                // PYR_LV_SOURCE: the input is the source grid, its rows are in srcRow; PYR_LV_TERMINAL
   long long rowBase;        // batch-global row of this sample's row 0 at level l
   long long actBefore;      // entries of the samples before this one at level l
   long long inRowBase;      // rowBase of the input level (0 for the source)
@@ -337,8 +340,9 @@ struct PyrLv {
   long long *ekey;
   int *erow;
   long long boundActive;
-  long long pad;
+  int *bg;
 };
+enum { PYR_LV_SOURCE = 1, PYR_LV_TERMINAL = 2 };
 // What the enumeration needs of level x (x < nMasks), in one 16-byte read
 struct PyrEn {
   int maskOff, nOut;
@@ -363,6 +367,7 @@ struct PyrLds {
   unsigned short *row;   // [total] rows, numbered from 0 within sample and level
   unsigned *own;         // [total] 16-bit ownership masks, two to a word
   unsigned short *base;  // [total] rows owned by the sites before, same level
+  unsigned char *kOf;    // [total] which of its owner's candidates a site is (the owner's rank waits in `row`)
 };
 PYR_FN PyrLds pyr_lds_view(const PyrArgs &a, unsigned char *lds, int total, int n0) {
   PyrLds v;
@@ -383,13 +388,16 @@ PYR_FN PyrLds pyr_lds_view(const PyrArgs &a, unsigned char *lds, int total, int 
   v.own = reinterpret_cast<unsigned *>(p);
   p += pad(2ll * total);
   v.base = reinterpret_cast<unsigned short *>(p);
+  p += pad(2ll * total);
+  v.kOf = p;
   return v;
 }
 
-// Entry l of the level table (lane l of the workgroup fills it, once)
-PYR_FN void pyr_fill_level(const PyrArgs &a, const PyrLds &s, int l, int b) {
+// Entry l of the level table (lane l of the workgroup fills it, once).  L:
+// layer l's arguments, which the lane has fetched already; inMaskOff: level
+// l - 1's; bgSource: the source's background row for this sample
+PYR_FN void pyr_fill_level(const PyrLevel &L, int inMaskOff, int bgSource, const PyrLds &s, int l) {
   const PyrHdr *h = s.h;
-  const PyrLevel &L = a.lv[l];
   PyrLv v;
   v.size = L.size;
   v.stride = L.stride;
@@ -397,15 +405,15 @@ PYR_FN void pyr_fill_level(const PyrArgs &a, const PyrLds &s, int l, int b) {
   v.nOut = L.nOut;
   v.width = L.width;
   v.magicS = L.magicS;
-  v.inMaskOff = a.lv[l - 1].maskOff;
+  v.inMaskOff = inMaskOff;
   v.inSiteOff = h->siteOff[l - 1];
   const bool region = L.kind == PYR_REGIONS;
   v.siteOff = region ? h->siteOff[l] : 0;
   v.n = region ? h->n[l] : 0;
   const int x = l - 1;
-  v.inIsSource = x == 0;
+  v.flags = (x == 0 ? PYR_LV_SOURCE : 0) | (region ? 0 : PYR_LV_TERMINAL);
   v.inRowBase = x == 0 ? 0 : h->actBefore[x] + h->bgBefore[x];
-  v.bgIn = x == 0 ? a.bg[b] : (h->hasBg[x] ? (int)v.inRowBase + h->n[x] : -1);
+  v.bgIn = x == 0 ? bgSource : (h->hasBg[x] ? (int)v.inRowBase + h->n[x] : -1);
   v.rowBase = region ? h->actBefore[l] + h->bgBefore[l] : 0;
   v.actBefore = region ? h->actBefore[l] : 0;
   v.volOut = L.volOut;
@@ -414,12 +422,12 @@ PYR_FN void pyr_fill_level(const PyrArgs &a, const PyrLds &s, int l, int b) {
   v.ekey = L.ekey;
   v.erow = L.erow;
   v.boundActive = L.boundActive;
+  v.bg = L.bg;
   s.lv[l] = v;
 }
 
 // Entry x of the enumeration's table (x < nMasks)
-PYR_FN void pyr_fill_en(const PyrArgs &a, unsigned char *lds, int x, int siteOff) {
-  const PyrLevel &L = a.lv[x];
+PYR_FN void pyr_fill_en(const PyrLevel &L, unsigned char *lds, int x, int siteOff) {
   PyrEn e;
   e.maskOff = L.maskOff;
   e.nOut = L.nOut;
@@ -541,32 +549,75 @@ PYR_FN void pyr_sweep_clear(const PyrLds &s, int t, int T) {
     s.own[i] = 0u;
 }
 
-// ---- sweep 1: the sites of every level by rank.  A lane takes mask words of
-// the whole pyramid (the spare words between the levels are zero); its words
+// Position of the k-th set bit of v (k < popcount(v)), by halving
+PYR_FN unsigned pyr_select64(pyr_u64 v, unsigned k) {
+  unsigned part = (unsigned)v, off = 0;
+  unsigned c = (unsigned)pyr_popc32(part);
+  if (k >= c) {
+    k -= c;
+    part = (unsigned)(v >> 32);
+    off = 32;
+  }
+  c = (unsigned)pyr_popc32(part & 0xFFFFu);
+  if (k >= c) {
+    k -= c;
+    part >>= 16;
+    off += 16;
+  }
+  c = (unsigned)pyr_popc32(part & 0xFFu);
+  if (k >= c) {
+    k -= c;
+    part >>= 8;
+    off += 8;
+  }
+  c = (unsigned)pyr_popc32(part & 0xFu);
+  if (k >= c) {
+    k -= c;
+    part >>= 4;
+    off += 4;
+  }
+  c = (unsigned)pyr_popc32(part & 3u);
+  if (k >= c) {
+    k -= c;
+    part >>= 2;
+    off += 2;
+  }
+  return off + (k >= (part & 1u) ? 1u : 0u);
+}
+
+// ---- sweep 1: the sites of every level by rank, a lane per SITE (a lane per
+// mask word leaves most lanes waiting for the one with the fullest word): the
+// word that holds rank r is the last one whose prefix is <= r, found by
+// bisection; the site is the (r - prefix)-th set bit of it.  A lane's sites
 // come in ascending order, so the level is a cursor.
 template <int D>
 PYR_FN void pyr_sweep_enumerate(const PyrArgs &a, const PyrLds &s, int t, int T) {
+  const int total = s.h->total;
   int x = 0;
-  for (int g = t; g < a.maskWords; g += T) {
-    pyr_u64 v = s.masks[g];
-    if (!v)
-      continue;
-    while (x + 1 < a.nMasks && g >= s.en[x + 1].maskOff)
+  for (int i = t; i < total; i += T) {
+    while (x + 1 < a.nMasks && i >= s.en[x + 1].siteOff)
       ++x;
     const PyrEn e = s.en[x];
-    unsigned r = (unsigned)e.siteOff + s.pref[g];
-    const unsigned k0 = 64u * (unsigned)(g - e.maskOff);
-    while (v) {
-      unsigned k = k0 + (unsigned)pyr_ctz64(v);
-      v &= v - 1;
-      int c[D];
-      for (int q = D - 1; q >= 0; --q) {
-        const unsigned up = pyr_div(k, (unsigned)e.nOut, e.magicN);
-        c[q] = (int)(k - up * (unsigned)e.nOut);
-        k = up;
-      }
-      s.key[r++] = pyr_pack<D>(c);
+    const unsigned r = (unsigned)(i - e.siteOff);
+    // (the level's two spare words have the level's count as prefix: > r)
+    const int span = (x + 1 < a.nMasks ? s.en[x + 1].maskOff : a.maskWords) - e.maskOff;
+    const unsigned short *pref = s.pref + e.maskOff;
+    int lo = 0, hi = span;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (pref[mid] <= r)
+        lo = mid;
+      else
+        hi = mid;
     }
+    unsigned k = 64u * (unsigned)lo + pyr_select64(s.masks[e.maskOff + lo], r - pref[lo]);
+    int c[D];
+    for (int q = D - 1; q >= 0; --q) {
+      const unsigned up = pyr_div(k, (unsigned)e.nOut, e.magicN);
+      c[q] = (int)(k - up * (unsigned)e.nOut);
+      k = up;
+    }
+    s.key[i] = pyr_pack<D>(c);
   }
 }
 
@@ -581,9 +632,13 @@ PYR_FN void pyr_sweep_owners(const PyrLds &s, int nRegions, int t, int T) {
     const PyrLv &v = s.lv[l];
     int k;
     unsigned rank;
-    pyr_owner<D>(v, s, it - h->itemOff[l], &k, &rank);
+    const int r = it - h->itemOff[l];
+    pyr_owner<D>(v, s, r, &k, &rank);
     const unsigned at = (unsigned)v.inSiteOff + rank;
     PYR_ATOMIC_OR(&s.own[at >> 1], 1u << (k + 16 * (int)(at & 1u)));
+    // (kept for sweep 4, which then has no window to look at)
+    s.row[v.siteOff + r] = (unsigned short)rank;
+    s.kOf[v.siteOff + r] = (unsigned char)k;
   }
 }
 
@@ -601,10 +656,8 @@ PYR_FN void pyr_sweep_rows(const PyrLds &s, int nRegions, int b, int t, int T) {
     l = pyr_item_level(h, nRegions, it, l);
     const PyrLv &v = s.lv[l];
     const int r = it - h->itemOff[l];
-    int k;
-    unsigned rank;
-    pyr_owner<D>(v, s, r, &k, &rank);
-    const unsigned at = (unsigned)v.inSiteOff + rank;
+    const int k = s.kOf[v.siteOff + r];
+    const unsigned at = (unsigned)v.inSiteOff + s.row[v.siteOff + r];
     // the owner's candidates after this one are the outputs before it
     const unsigned row = s.base[at] + (unsigned)pyr_popc32(pyr_own_mask(s, at) >> (k + 1));
     s.row[v.siteOff + r] = (unsigned short)row;
@@ -620,7 +673,7 @@ PYR_FN void pyr_sweep_rows(const PyrLds &s, int nRegions, int b, int t, int T) {
 
 // batch-global row of the input site with rank `rank` of layer v
 PYR_FN int pyr_in_row(const PyrLv &v, const PyrLds &s, unsigned rank) {
-  if (v.inIsSource)
+  if (v.flags & PYR_LV_SOURCE)
     return (int)s.srcRow[rank];
   return (int)v.inRowBase + (int)s.row[v.inSiteOff + rank];
 }
@@ -678,47 +731,51 @@ PYR_FN void pyr_sweep_rules(const PyrLds &s, int nRegions, int t, int T) {
   }
 }
 
-// ---- the all-background rows, backgroundCol, the terminal layer's rules
+// ---- the all-background rows, backgroundCol, the terminal layer's rules: a
+// wavefront per layer (the terminal layer, which can only be the last: all lanes)
 PYR_FN void pyr_sweep_tail(const PyrArgs &a, const PyrLds &s, int b, int t, int T) {
   const PyrHdr *h = s.h;
-  for (int l = 1; l <= a.nLevels; ++l) {
-    const PyrLevel &L = a.lv[l];
-    if (L.kind == PYR_TERMINAL) {
-      // terminalGridPoolingRules (TerminalPoolingLayer.cu:8-20): the rows in
-      // iteration order, or the background row of a sample without sites;
-      // padded with -1 to the batch's largest sample (:90-96)
-      const int x = l - 1;
-      const PyrLv &v = s.lv[l];
-      const long long width = h->maxAct[x] > 1 ? h->maxAct[x] : 1;
-      if (L.rules && ((long long)b + 1) * width <= L.capacity) {
-        const int n = h->n[x];
-        int *dst = L.rules + (long long)b * width;
-        for (long long i = t; i < width; i += T) {
-          int val = -1;
-          if (n == 0 && i == 0)
-            val = v.bgIn;
-          else if (i < n)
-            val = pyr_in_row(v, s, (unsigned)i);
-          dst[i] = val;
-        }
-      }
-      if (t == 0) { // the output grid: site 0 of sample b is row b
-        L.ekey[b] = b;
-        L.erow[b] = b;
-        L.bg[b] = -1;
-      }
+  const int W = T >= 64 ? 64 : T;
+  const int lane = t % W, wave = t / W, waves = T / W;
+  for (int l = 1 + wave; l <= a.nLevels; l += waves) {
+    const PyrLv &v = s.lv[l];
+    if (v.flags & PYR_LV_TERMINAL)
       continue;
-    }
     const int bgOut = pyr_bg_row(a, s, l, b);
-    if (h->hasBg[l] && L.rules && bgOut >= 0 &&
-        ((long long)bgOut + 1) * L.width <= L.capacity) { // Regions.cu:647-652
-      const int bgIn = s.lv[l].bgIn;
-      int *dst = L.rules + (long long)bgOut * L.width;
-      for (int q = t; q < L.width; q += T)
+    if (h->hasBg[l] && v.rules && bgOut >= 0 &&
+        ((long long)bgOut + 1) * v.width <= v.capacity) { // Regions.cu:647-652
+      const int bgIn = v.bgIn;
+      int *dst = v.rules + (long long)bgOut * v.width;
+      for (int q = lane; q < v.width; q += W)
         dst[q] = bgIn;
     }
-    if (t == 0)
-      L.bg[b] = bgOut;
+    if (lane == 0)
+      v.bg[b] = bgOut;
+  }
+  const PyrLv &v = s.lv[a.nLevels];
+  if (v.flags & PYR_LV_TERMINAL) {
+    // terminalGridPoolingRules (TerminalPoolingLayer.cu:8-20): the rows in
+    // iteration order, or the background row of a sample without sites;
+    // padded with -1 to the batch's largest sample (:90-96)
+    const int x = a.nLevels - 1;
+    const long long width = h->maxAct[x] > 1 ? h->maxAct[x] : 1;
+    if (v.rules && ((long long)b + 1) * width <= v.capacity) {
+      const int n = h->n[x];
+      int *dst = v.rules + (long long)b * width;
+      for (long long i = t; i < width; i += T) {
+        int val = -1;
+        if (n == 0 && i == 0)
+          val = v.bgIn;
+        else if (i < n)
+          val = pyr_in_row(v, s, (unsigned)i);
+        dst[i] = val;
+      }
+    }
+    if (t == 0) { // the output grid: site 0 of sample b is row b
+      v.ekey[b] = b;
+      v.erow[b] = b;
+      v.bg[b] = -1;
+    }
   }
 }
 
@@ -727,8 +784,7 @@ PYR_FN void pyr_sweep_tail(const PyrArgs &a, const PyrLds &s, int b, int t, int 
 struct PyrReport {
   long long nSites, nActive, over, extra;
 };
-PYR_FN PyrReport pyr_report(const PyrArgs &a, const PyrHdr *h, int l) {
-  const PyrLevel &L = a.lv[l];
+PYR_FN PyrReport pyr_report(const PyrArgs &a, const PyrLevel &L, const PyrHdr *h, int l) {
   PyrReport r;
   if (L.kind == PYR_TERMINAL) {
     const long long width = h->maxAct[l - 1] > 1 ? h->maxAct[l - 1] : 1;

@@ -32,15 +32,12 @@ template <int D> void pass_a(const PyrArgs &a, int b, int T, bool *gaveUp) {
       for (int w = t; w < L.words + 2; w += T)
         masks[w] = w < L.words ? pyr_source_word(a.bits, L.volOut, b, (unsigned)w) : 0ull;
   }
-  for (int x = 1; x < a.nMasks; ++x) {
+  for (int x = 1; x < a.nMasks; ++x) { // (the masks start as zero: the pieces are OR-ed in)
     const PyrLevel &L = a.lv[x];
     const pyr_u64 *in = masks + a.lv[x - 1].maskOff;
     pyr_u64 *out = masks + L.maskOff;
     for (int t = 0; t < T; ++t)
-      for (int w = t; w < L.words + 2; w += T)
-        out[w] = w < L.words ? pyr_dilate_any<D>(in, L.nIn, L.nOut, L.size, L.stride, (unsigned)L.volOut,
-                                                  L.magicN, L.lenMax, (unsigned)w)
-                             : 0ull;
+      pyr_sweep_dilate<D>(in, out, L.nIn, L.nOut, L.size, L.stride, L.magicN, L.seg, L.segs, L.magicSegs, t, T);
   }
   for (int x = 0; x < a.nMasks; ++x) {
     const PyrLevel &L = a.lv[x];
@@ -100,7 +97,7 @@ template <int D> void pass_b(const PyrArgs &a, int b, int T, bool gaveUp, long l
       sum += h->n[x];
     h->siteOff[t] = sum;
     if (t < a.nMasks)
-      pyr_fill_en(a, lds, t, sum);
+      pyr_fill_en(a.lv[t], lds, t, sum);
     if (t == a.nMasks)
       h->total = sum;
   }
@@ -111,14 +108,14 @@ template <int D> void pass_b(const PyrArgs &a, int b, int T, bool gaveUp, long l
     h->itemOff[t] = sum;
   }
   for (int t = 1; t <= a.nLevels; ++t)
-    if (pyr_report(a, h, t).over)
+    if (pyr_report(a, a.lv[t], h, t).over)
       h->over |= 1;
   if (pyr_lds_need(a, h->n) > a.ldsBytesB)
     h->over |= 2;
   const bool over = h->over != 0 || gaveUp;
   if (b == 0)
     for (int t = 1; t <= a.nLevels; ++t) {
-      const PyrReport r = pyr_report(a, h, t);
+      const PyrReport r = pyr_report(a, a.lv[t], h, t);
       report[4 * t + 0] = r.nSites;
       report[4 * t + 1] = r.nActive;
       report[4 * t + 2] = over;
@@ -130,12 +127,12 @@ template <int D> void pass_b(const PyrArgs &a, int b, int T, bool gaveUp, long l
   }
   const PyrLds s = pyr_lds_view(a, lds, h->total, h->n[0]);
   // (the last array must end inside what pass B was launched with)
-  if (reinterpret_cast<unsigned char *>(s.base + h->total) > lds + a.ldsBytesB) {
+  if (s.kOf + h->total > lds + a.ldsBytesB) {
     fprintf(stderr, "pyr_lds_need promises less than pyr_lds_view takes\n");
     abort();
   }
   for (int t = 1; t <= a.nLevels; ++t)
-    pyr_fill_level(a, s, t, b);
+    pyr_fill_level(a.lv[t], a.lv[t - 1].maskOff, a.bg[b], s, t);
   for (int t = 0; t < T; ++t)
     pyr_sweep_clear(s, t, T);
   for (int t = 0; t < T; ++t)
@@ -235,7 +232,7 @@ extern "C" int pyr_cpu_chain(int d, int batch, int n0, int nLevels, const int *g
     L.fullSize = L.volOut;
     L.magicN = magic(L.nOut);
     L.magicS = magic(L.size);
-    L.lenMax = pyr_len_max(L.size, L.stride);
+    pyr_set_pieces(L);
     L.rules = rules[l - 1];
     L.capacity = rulesCap[l - 1];
     L.ekey = ekey[l - 1];
