@@ -19,6 +19,7 @@ oracle timed on this host's cores.
 import argparse
 import json
 import os
+import subprocess
 import sys
 import time
 
@@ -600,7 +601,18 @@ def train_leg(args, cfg, net, hostapi, samples, saved_stdout):
 
 
 def cpu_leg(cfg, layers, weights, samples, spatialSize, budget_s):
-    """The CPU oracle on this host's cores, same batch, bounded wall time."""
+    """The CPU oracle on this host's cores, same batch, bounded wall time.  Timed in its -O3 -march=native build,
+    made here, on the host whose cores are timed (a library built with -march=native elsewhere may not run here);
+    the parity build (-mavx2 -ffp-contract=off) is timed instead if that build fails."""
+    odir = os.path.join(ROOT, "oracle")
+    flags_var = "CFLAGS"
+    try:
+        subprocess.check_call(["make", "-C", odir, "-s", "-B", "native"], stdout=subprocess.DEVNULL,
+                              stderr=subprocess.DEVNULL)
+        os.environ["SCN_ORACLE_LIB"] = os.path.join(odir, "libscn_oracle_native.so")
+        flags_var = "CFLAGS_NATIVE"
+    except (OSError, subprocess.CalledProcessError):
+        pass
     import oracle as orc
     import oracle_net
     from sparseconvnet_archived_amd import synthetic
@@ -659,7 +671,7 @@ def cpu_leg(cfg, layers, weights, samples, spatialSize, budget_s):
     flags = ""
     try:
         for line in open(os.path.join(ROOT, "oracle", "Makefile")):
-            if line.startswith("CFLAGS"):
+            if line.split("=", 1)[0].strip() == flags_var:
                 flags = line.split("=", 1)[1].strip()
     except OSError:
         pass

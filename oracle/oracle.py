@@ -22,9 +22,12 @@ def build():
 
 
 def _load():
-    if not os.path.exists(_LIB_PATH):
+    # SCN_ORACLE_LIB: another build of the same source (bench.py's cpu_baseline
+    # times the -march=native one; checkers never set it)
+    path = os.environ.get("SCN_ORACLE_LIB") or _LIB_PATH
+    if path == _LIB_PATH and not os.path.exists(_LIB_PATH):
         build()
-    lib = C.CDLL(_LIB_PATH)
+    lib = C.CDLL(path)
     vp, i32, i64, f32 = C.c_void_p, C.c_int32, C.c_int64, C.c_float
     sig = {
         "orc_grids_create": (vp, [C.c_int]),

@@ -104,6 +104,7 @@ struct ChainState {
   DevBuf<unsigned long long> pyramid;
   bool pyramids = true; // (false: such chains go through k_chain_sample too)
   bool pyrAtMax = false; // the last such chain had all the LDS there is
+  int pyrMisses = 0;     // such chains in a row that still outgrew it
   scn_grids *pyrSource = nullptr; // source of the last such chain: its largest sample comes back in h_pinned[13]
   long long nPyramids = 0;
 };
@@ -913,7 +914,7 @@ __global__ void __launch_bounds__(PYR_A_THREADS) k_pyr_masks(PyrArgs a) {
     c[1] = (long long)cnt[t] < a.lv[t].fullSize;
   }
   if (t == 0) {
-    bool fits = pyr_lds_need(a, cnt) <= a.ldsBytesB;
+    bool fits = pyr_fits(a, cnt);
     for (int x = 0; x < a.nMasks; ++x)
       fits = fits && cnt[x] <= PYR_ROWS_MAX;
     if (!fits)
@@ -928,7 +929,6 @@ __global__ void __launch_bounds__(PYR_B_THREADS) k_pyr_rules(PyrArgs a) {
   const int b = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6;
   constexpr int T = PYR_B_THREADS;
   const bool gaveUp = *reinterpret_cast<volatile unsigned long long *>(a.flag) == a.ticket;
-  const int nRegions = a.nMasks - 1;
   // lane t keeps layer t's arguments from here on: fetched while the masks
   // come in, not when the level table wants them
   PyrLevel mine;
@@ -983,25 +983,9 @@ __global__ void __launch_bounds__(PYR_B_THREADS) k_pyr_rules(PyrArgs a) {
     }
   }
   lds_barrier();
-  if (t <= a.nMasks) {
-    int sum = 0;
-    for (int x = 0; x < t; ++x)
-      sum += h->n[x];
-    h->siteOff[t] = sum;
-    if (t < a.nMasks)
-      pyr_fill_en(mine, lds, t, sum);
-    if (t == a.nMasks)
-      h->total = sum;
-  }
-  if (t >= 1 && t <= nRegions + 1) {
-    int sum = 0;
-    for (int l = 1; l < t; ++l)
-      sum += h->n[l];
-    h->itemOff[t] = sum;
-  }
   if (t >= 1 && t <= a.nLevels && pyr_report(a, mine, h, t).over)
     atomicOr(&h->over, 1);
-  if (t == 0 && pyr_lds_need(a, h->n) > a.ldsBytesB)
+  if (t == 0 && !pyr_fits(a, h->n))
     atomicOr(&h->over, 2);
   lds_barrier();
   const bool over = h->over != 0 || gaveUp;
@@ -1024,45 +1008,63 @@ __global__ void __launch_bounds__(PYR_B_THREADS) k_pyr_rules(PyrArgs a) {
   }
   if (over)
     return;
-  const PyrLds s = pyr_lds_view(a, lds, h->total, h->n[0]);
-  if (t >= 1 && t <= a.nLevels)
-    pyr_fill_level(mine, inMaskOff, bgSource, s, t);
-  pyr_sweep_clear(s, t, T);
-  pyr_sweep_enumerate<D>(a, s, t, T);
-  lds_barrier();
-  { // the batch's rows of the source's sites: their loads go out first
-    const PyrLevel &L = a.lv[0];
-    const long long p0 = (long long)b * L.volOut;
-    const Slot *table = reinterpret_cast<const Slot *>(a.table);
-    for (int r = t; r < h->n[0]; r += T) {
-      int c[D];
-      pyr_unpack<D>(s.key[r], c);
-      long long p = p0 + pyr_key<D>(c, L.nOut);
-      p = p < (long long)a.batch * L.volOut ? p : 0; // (a mask never has a site beyond the field)
-      s.srcRow[r] = (unsigned)(a.dense ? a.dense[p] : hash_find(table, a.shift, a.mask, p));
+  // the layers a window of levels at a time: as many as the LDS holds (all of
+  // them, for all but the largest samples)
+  for (int xa = 0;;) {
+    const int xb = pyr_window_end(a, h->n, xa);
+    const int la = xa + 1, lb = xb;
+    const bool last = xb == a.nMasks - 1;
+    pyr_fill_offsets(h, xa, xb, t);
+    lds_barrier();
+    if (t < a.nMasks)
+      pyr_fill_en(mine, lds, t, h->siteOff[t]);
+    const PyrLds s = pyr_lds_view(a, lds, h->total, h->n[xa]);
+    if ((t >= la && t <= lb) || (last && t == a.nLevels && t > lb))
+      pyr_fill_level(mine, inMaskOff, bgSource, s, t, xa);
+    pyr_sweep_clear(s, t, T);
+    lds_barrier();
+    pyr_sweep_enumerate<D>(a, s, xa, xb, t, T);
+    lds_barrier();
+    if (xa == 0) { // the batch's rows of the source's sites: their loads go out first
+      const PyrLevel &L = a.lv[0];
+      const long long p0 = (long long)b * L.volOut;
+      const Slot *table = reinterpret_cast<const Slot *>(a.table);
+      for (int r = t; r < h->n[0]; r += T) {
+        int c[D];
+        pyr_unpack<D>(s.key[r], c);
+        long long p = p0 + pyr_key<D>(c, L.nOut);
+        p = p < (long long)a.batch * L.volOut ? p : 0; // (a mask never has a site beyond the field)
+        s.srcRow[r] = (unsigned)(a.dense ? a.dense[p] : hash_find(table, a.shift, a.mask, p));
+      }
     }
-  }
-  pyr_sweep_owners<D>(s, nRegions, t, T);
-  lds_barrier();
-  // rows owned by the sites before, a wavefront per level
-  for (int x = wave; x < nRegions; x += T / 64) {
-    const int n = h->n[x];
-    const unsigned off = (unsigned)h->siteOff[x];
-    unsigned carry = 0;
-    for (int r0 = 0; r0 < n; r0 += 64) {
-      const int r = r0 + lane;
-      const unsigned v = r < n ? (unsigned)pyr_popc32(pyr_own_mask(s, off + r)) : 0u;
-      const unsigned incl = wave_scan_incl_dpp(v);
-      if (r < n)
-        s.base[off + r] = (unsigned short)(carry + incl - v);
-      carry += wave_last(incl);
+    pyr_sweep_owners<D>(s, la, lb, t, T);
+    lds_barrier();
+    // rows owned by the sites before, a wavefront per level
+    for (int x = xa + wave; x < xb; x += T / 64) {
+      const int n = h->n[x];
+      const unsigned off = (unsigned)h->siteOff[x];
+      unsigned carry = 0;
+      for (int r0 = 0; r0 < n; r0 += 64) {
+        const int r = r0 + lane;
+        const unsigned v = r < n ? (unsigned)pyr_popc32(pyr_own_mask(s, off + r)) : 0u;
+        const unsigned incl = wave_scan_incl_dpp(v);
+        if (r < n)
+          s.base[off + r] = (unsigned short)(carry + incl - v);
+        carry += wave_last(incl);
+      }
     }
+    lds_barrier();
+    pyr_sweep_rows<D>(s, la, lb, b, t, T);
+    lds_barrier();
+    pyr_sweep_rules<D>(s, la, lb, t, T);
+    pyr_sweep_tail(a, s, la, lb, b, t, T);
+    if (last)
+      break;
+    lds_barrier();
+    pyr_sweep_carry(s, lds, a, xb, t, T);
+    lds_barrier();
+    xa = xb;
   }
-  lds_barrier();
-  pyr_sweep_rows<D>(s, nRegions, b, t, T);
-  lds_barrier();
-  pyr_sweep_rules<D>(s, nRegions, t, T);
-  pyr_sweep_tail(a, s, b, t, T);
 }
 
 // -------------------------------------------------------------------- host
@@ -1594,24 +1596,29 @@ int scn_chain_flush(scn_ctx *ctx) {
 // what scn_rules_settle learns about a chained plan from its pinned slot
 void scn_chain_settled(scn_ctx *ctx, scn_grids *g, long long sampleMax,
                        bool overflowed) {
+  bool pyramid = false; // the first layer of a chain built from the output side
   if (ctx->chain && ctx->chain->pyrSource) {
-    // the source of a chain built from the output side: its largest sample
+    // its source's largest sample
     scn_grids *src = ctx->chain->pyrSource;
     const long long m = ctx->h_pinned[13];
     if (!overflowed)
       src->seenSample = m > src->seenSample ? m : src->seenSample;
     ctx->chain->pyrSource = nullptr;
+    pyramid = true;
   }
   if (overflowed) {
     if (ctx->chain) {
-      // a sample that does not fit with every layer's sites in LDS at once may
-      // still fit the other construction, which holds two layers at a time
-      if (ctx->chain->wide && ctx->chain->pyrAtMax)
+      // a sample one of whose layers does not fit the LDS with its input may
+      // still fit the other construction, which keeps less per site; a context
+      // that meets such samples time and again stops trying
+      if (pyramid && ctx->chain->wide && ctx->chain->pyrAtMax && ++ctx->chain->pyrMisses >= 3)
         ctx->chain->pyramids = false;
       ctx->chain->wide = true;
     }
     return;
   }
+  if (pyramid && ctx->chain)
+    ctx->chain->pyrMisses = 0;
   if (g->planKind == PLAN_REGIONS)
     g->seenSample = sampleMax > g->seenSample ? sampleMax : g->seenSample;
 }

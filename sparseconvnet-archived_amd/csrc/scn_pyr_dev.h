@@ -297,28 +297,49 @@ PYR_FN pyr_u64 pyr_source_word(const pyr_u64 *bits, long long vol, int b, unsign
   return v;
 }
 
-// LDS bytes pass B needs for a sample with n[x] sites at level x (x < nMasks)
-PYR_FN long long pyr_lds_need(const PyrArgs &a, const int *n) {
+// Pass B takes a sample's layers a WINDOW of levels xa .. xb at a time: level
+// xa as input only (its rows known: the source's, or from the window before),
+// layers xa + 1 .. xb built.  LDS bytes of a window for a sample with n[x]
+// sites at level x: per site key (4), row, ownership mask, base (2 each),
+// which candidate of its owner it is (1); the input level's batch-global rows
+// (4 more); every array padded to 16 bytes
+PYR_FN long long pyr_lds_window(const PyrArgs &a, const int *n, int xa, int xb) {
   long long total = 0;
-  for (int x = 0; x < a.nMasks; ++x)
+  for (int x = xa; x <= xb; ++x)
     total += n[x];
-  // per site: key (4), row, ownership mask, base (2 each), which candidate of
-  // its owner it is (1); the source's rows are the batch's (4 more); every
-  // array padded to 16 bytes
-  return PYR_HDR_BYTES + 8ll * a.pyrStride + 11ll * total + 4ll * n[0] + 6 * 16;
+  return PYR_HDR_BYTES + 8ll * a.pyrStride + 11ll * total + 4ll * n[xa] + 6 * 16;
+}
+// The window that starts at level xa: as many layers as fit (at least one,
+// when there is one)
+PYR_FN int pyr_window_end(const PyrArgs &a, const int *n, int xa) {
+  int xb = xa + 1 < a.nMasks ? xa + 1 : xa;
+  long long total = n[xa] + (xb > xa ? n[xb] : 0);
+  const long long fixed = PYR_HDR_BYTES + 8ll * a.pyrStride + 4ll * n[xa] + 6 * 16;
+  while (xb + 1 < a.nMasks && fixed + 11ll * (total + n[xb + 1]) <= a.ldsBytesB) {
+    total += n[xb + 1];
+    ++xb;
+  }
+  return xb;
+}
+// Whether every layer of the sample fits by itself
+PYR_FN bool pyr_fits(const PyrArgs &a, const int *n) {
+  bool fits = pyr_lds_window(a, n, 0, a.nMasks > 1 ? 1 : 0) <= a.ldsBytesB;
+  for (int x = 1; x + 1 < a.nMasks; ++x)
+    fits = fits && pyr_lds_window(a, n, x, x + 1) <= a.ldsBytesB;
+  return fits;
 }
 
 // ------------------------------------------------------------------- pass B
 struct PyrHdr {
   int n[PYR_MAX_LEVELS + 1];       // this sample's sites at level x
   int hasBg[PYR_MAX_LEVELS + 1];   // and whether it has a background row there
-  int siteOff[PYR_MAX_LEVELS + 2]; // where level x starts in the per-site arrays
-  int itemOff[PYR_MAX_LEVELS + 2]; // output sites of the region layers before layer l (index l)
+  int siteOff[PYR_MAX_LEVELS + 2]; // where level x of the current window starts in the per-site arrays
+  int itemOff[PYR_MAX_LEVELS + 2]; // output sites of the window's layers before layer l (index l)
   int maxAct[PYR_MAX_LEVELS + 1];  // largest sample of the batch at level x
   long long actBefore[PYR_MAX_LEVELS + 1], bgBefore[PYR_MAX_LEVELS + 1]; // of the samples before this one
   long long actAll[PYR_MAX_LEVELS + 1], bgAll[PYR_MAX_LEVELS + 1];
   int over; // some layer outgrew its bounds, or a sample the LDS
-  int total; // sites of this sample over all levels with a mask
+  int total; // sites of this sample over the levels of the current window
 };
 // What the sweeps need of layer l, once per item: kept in LDS (the kernel
 // arguments are far away for a lane that wants the entry of ITS layer), the
@@ -330,7 +351,7 @@ struct PyrLv {
   int inMaskOff, inSiteOff; // mask and sites of the layer's input (level l - 1)
   int siteOff, n;           // sites of the layer's output (level l)
   int bgIn;                 // batch-global row of the input's background row, or -1
-  int flags;                // PYR_LV_SOURCE: the input is the source grid, its rows are in srcRow; PYR_LV_TERMINAL
+  int flags;                // PYR_LV_SOURCE: the input is the window's first level, its rows are in srcRow; PYR_LV_TERMINAL
   long long rowBase;        // batch-global row of this sample's row 0 at level l
   long long actBefore;      // entries of the samples before this one at level l
   long long inRowBase;      // rowBase of the input level (0 for the source)
@@ -362,14 +383,17 @@ struct PyrLds {
   PyrEn *en;             // [nMasks]
   pyr_u64 *masks;        // a.maskWords words
   unsigned short *pref;  // one per mask word
+  unsigned *srcRow;      // [n[xa]] batch-global rows of the sites of the window's first level
   unsigned *key;         // [total] packed coordinates by (level, rank)
-  unsigned *srcRow;      // [n[0]] batch-global rows of the source's sites
   unsigned short *row;   // [total] rows, numbered from 0 within sample and level
   unsigned *own;         // [total] 16-bit ownership masks, two to a word
   unsigned short *base;  // [total] rows owned by the sites before, same level
   unsigned char *kOf;    // [total] which of its owner's candidates a site is (the owner's rank waits in `row`)
 };
-PYR_FN PyrLds pyr_lds_view(const PyrArgs &a, unsigned char *lds, int total, int n0) {
+// (total: sites of the window's levels, nFirst: of its first level.  srcRow
+// comes first: the rows a window leaves for the next one are written there
+// while the old window's arrays, which all lie behind it, are still read)
+PYR_FN PyrLds pyr_lds_view(const PyrArgs &a, unsigned char *lds, int total, int nFirst) {
   PyrLds v;
   v.h = reinterpret_cast<PyrHdr *>(lds);
   v.lv = reinterpret_cast<PyrLv *>(lds + PYR_LV_AT);
@@ -379,10 +403,10 @@ PYR_FN PyrLds pyr_lds_view(const PyrArgs &a, unsigned char *lds, int total, int 
   v.pref = reinterpret_cast<unsigned short *>(p + 8ll * a.maskWords);
   p += 8ll * a.pyrStride;
   auto pad = [](long long x) { return (x + 15) / 16 * 16; };
+  v.srcRow = reinterpret_cast<unsigned *>(p);
+  p += pad(4ll * nFirst);
   v.key = reinterpret_cast<unsigned *>(p);
   p += pad(4ll * total);
-  v.srcRow = reinterpret_cast<unsigned *>(p);
-  p += pad(4ll * n0);
   v.row = reinterpret_cast<unsigned short *>(p);
   p += pad(2ll * total);
   v.own = reinterpret_cast<unsigned *>(p);
@@ -393,10 +417,11 @@ PYR_FN PyrLds pyr_lds_view(const PyrArgs &a, unsigned char *lds, int total, int 
   return v;
 }
 
-// Entry l of the level table (lane l of the workgroup fills it, once).  L:
-// layer l's arguments, which the lane has fetched already; inMaskOff: level
-// l - 1's; bgSource: the source's background row for this sample
-PYR_FN void pyr_fill_level(const PyrLevel &L, int inMaskOff, int bgSource, const PyrLds &s, int l) {
+// Entry l of the level table (lane l of the workgroup fills it, once a
+// window).  L: layer l's arguments, which the lane has fetched already;
+// inMaskOff: level l - 1's; bgSource: the source's background row for this
+// sample; xa: the window's first level
+PYR_FN void pyr_fill_level(const PyrLevel &L, int inMaskOff, int bgSource, const PyrLds &s, int l, int xa) {
   const PyrHdr *h = s.h;
   PyrLv v;
   v.size = L.size;
@@ -411,7 +436,7 @@ PYR_FN void pyr_fill_level(const PyrLevel &L, int inMaskOff, int bgSource, const
   v.siteOff = region ? h->siteOff[l] : 0;
   v.n = region ? h->n[l] : 0;
   const int x = l - 1;
-  v.flags = (x == 0 ? PYR_LV_SOURCE : 0) | (region ? 0 : PYR_LV_TERMINAL);
+  v.flags = (x == xa ? PYR_LV_SOURCE : 0) | (region ? 0 : PYR_LV_TERMINAL);
   v.inRowBase = x == 0 ? 0 : h->actBefore[x] + h->bgBefore[x];
   v.bgIn = x == 0 ? bgSource : (h->hasBg[x] ? (int)v.inRowBase + h->n[x] : -1);
   v.rowBase = region ? h->actBefore[l] + h->bgBefore[l] : 0;
@@ -426,7 +451,21 @@ PYR_FN void pyr_fill_level(const PyrLevel &L, int inMaskOff, int bgSource, const
   s.lv[l] = v;
 }
 
-// Entry x of the enumeration's table (x < nMasks)
+// Where the levels of the window xa .. xb start in the per-site arrays, and
+// the window's layers among its items: lane t does entry t (t <= nMasks)
+PYR_FN void pyr_fill_offsets(PyrHdr *h, int xa, int xb, int t) {
+  if (t < xa || t > xb + 1)
+    return;
+  int sum = 0;
+  for (int x = xa; x < t; ++x)
+    sum += h->n[x];
+  h->siteOff[t] = sum;
+  h->itemOff[t] = t > xa ? sum - h->n[xa] : 0;
+  if (t == xb + 1)
+    h->total = sum;
+}
+
+// Entry x of the enumeration's table (x < nMasks; siteOff: in the current window)
 PYR_FN void pyr_fill_en(const PyrLevel &L, unsigned char *lds, int x, int siteOff) {
   PyrEn e;
   e.maskOff = L.maskOff;
@@ -437,9 +476,10 @@ PYR_FN void pyr_fill_en(const PyrLevel &L, unsigned char *lds, int x, int siteOf
 }
 
 // The layer an item of the flattened sweeps belongs to: a lane's items come in
-// ascending order, so it moves a cursor (starts at 1)
-PYR_FN int pyr_item_level(const PyrHdr *h, int nRegions, int it, int l) {
-  while (l < nRegions && it >= h->itemOff[l + 1])
+// ascending order, so it moves a cursor (starts at the window's first layer;
+// lb: its last)
+PYR_FN int pyr_item_level(const PyrHdr *h, int lb, int it, int l) {
+  while (l < lb && it >= h->itemOff[l + 1])
     ++l;
   return l;
 }
@@ -589,13 +629,14 @@ PYR_FN unsigned pyr_select64(pyr_u64 v, unsigned k) {
 // mask word leaves most lanes waiting for the one with the fullest word): the
 // word that holds rank r is the last one whose prefix is <= r, found by
 // bisection; the site is the (r - prefix)-th set bit of it.  A lane's sites
-// come in ascending order, so the level is a cursor.
+// come in ascending order, so the level is a cursor.  Of the window's first
+// level only the source needs its coordinates (to look its rows up).
 template <int D>
-PYR_FN void pyr_sweep_enumerate(const PyrArgs &a, const PyrLds &s, int t, int T) {
+PYR_FN void pyr_sweep_enumerate(const PyrArgs &a, const PyrLds &s, int xa, int xb, int t, int T) {
   const int total = s.h->total;
-  int x = 0;
-  for (int i = t; i < total; i += T) {
-    while (x + 1 < a.nMasks && i >= s.en[x + 1].siteOff)
+  int x = xa;
+  for (int i = (xa > 0 ? s.h->n[xa] : 0) + t; i < total; i += T) {
+    while (x + 1 <= xb && i >= s.en[x + 1].siteOff)
       ++x;
     const PyrEn e = s.en[x];
     const unsigned r = (unsigned)(i - e.siteOff);
@@ -623,12 +664,12 @@ PYR_FN void pyr_sweep_enumerate(const PyrArgs &a, const PyrLds &s, int t, int T)
 
 // ---- sweep 2: every output site tells its owner which candidate it is
 template <int D>
-PYR_FN void pyr_sweep_owners(const PyrLds &s, int nRegions, int t, int T) {
+PYR_FN void pyr_sweep_owners(const PyrLds &s, int la, int lb, int t, int T) {
   const PyrHdr *h = s.h;
-  const int items = h->itemOff[nRegions + 1];
-  int l = 1;
+  const int items = h->itemOff[lb + 1];
+  int l = la;
   for (int it = t; it < items; it += T) {
-    l = pyr_item_level(h, nRegions, it, l);
+    l = pyr_item_level(h, lb, it, l);
     const PyrLv &v = s.lv[l];
     int k;
     unsigned rank;
@@ -648,12 +689,12 @@ PYR_FN unsigned pyr_own_mask(const PyrLds &s, unsigned at) {
 
 // ---- sweep 4: rows of the output sites; the layers' entry lists
 template <int D>
-PYR_FN void pyr_sweep_rows(const PyrLds &s, int nRegions, int b, int t, int T) {
+PYR_FN void pyr_sweep_rows(const PyrLds &s, int la, int lb, int b, int t, int T) {
   const PyrHdr *h = s.h;
-  const int items = h->itemOff[nRegions + 1];
-  int l = 1;
+  const int items = h->itemOff[lb + 1];
+  int l = la;
   for (int it = t; it < items; it += T) {
-    l = pyr_item_level(h, nRegions, it, l);
+    l = pyr_item_level(h, lb, it, l);
     const PyrLv &v = s.lv[l];
     const int r = it - h->itemOff[l];
     const int k = s.kOf[v.siteOff + r];
@@ -687,12 +728,12 @@ PYR_FN int pyr_bg_row(const PyrArgs &a, const PyrLds &s, int x, int b) {
 
 // ---- sweep 5: rule rows
 template <int D>
-PYR_FN void pyr_sweep_rules(const PyrLds &s, int nRegions, int t, int T) {
+PYR_FN void pyr_sweep_rules(const PyrLds &s, int la, int lb, int t, int T) {
   const PyrHdr *h = s.h;
-  const int items = h->itemOff[nRegions + 1];
-  int l = 1;
+  const int items = h->itemOff[lb + 1];
+  int l = la;
   for (int it = t; it < items; it += T) {
-    l = pyr_item_level(h, nRegions, it, l);
+    l = pyr_item_level(h, lb, it, l);
     const PyrLv &v = s.lv[l];
     if (!v.rules)
       continue;
@@ -731,16 +772,27 @@ PYR_FN void pyr_sweep_rules(const PyrLds &s, int nRegions, int t, int T) {
   }
 }
 
-// ---- the all-background rows, backgroundCol, the terminal layer's rules: a
-// wavefront per layer (the terminal layer, which can only be the last: all lanes)
-PYR_FN void pyr_sweep_tail(const PyrArgs &a, const PyrLds &s, int b, int t, int T) {
+// ---- the rows of the window's last level, batch-global, where the next
+// window (which starts at that level) looks its input's rows up.  The
+// destination lies before everything the old window still holds.
+PYR_FN void pyr_sweep_carry(const PyrLds &s, unsigned char *lds, const PyrArgs &a, int xb, int t, int T) {
+  const PyrHdr *h = s.h;
+  const unsigned short *row = s.row + h->siteOff[xb];
+  unsigned *dst = reinterpret_cast<unsigned *>(lds + PYR_HDR_BYTES + 8ll * a.pyrStride);
+  const long long rowBase = h->actBefore[xb] + h->bgBefore[xb];
+  for (int i = t; i < h->n[xb]; i += T)
+    dst[i] = (unsigned)(rowBase + row[i]);
+}
+
+// ---- the all-background rows, backgroundCol of the window's layers, a
+// wavefront per layer; with the last window (xb = nMasks - 1) the terminal
+// layer's rules, if the chain ends in one (all lanes)
+PYR_FN void pyr_sweep_tail(const PyrArgs &a, const PyrLds &s, int la, int lb, int b, int t, int T) {
   const PyrHdr *h = s.h;
   const int W = T >= 64 ? 64 : T;
   const int lane = t % W, wave = t / W, waves = T / W;
-  for (int l = 1 + wave; l <= a.nLevels; l += waves) {
+  for (int l = la + wave; l <= lb; l += waves) {
     const PyrLv &v = s.lv[l];
-    if (v.flags & PYR_LV_TERMINAL)
-      continue;
     const int bgOut = pyr_bg_row(a, s, l, b);
     if (h->hasBg[l] && v.rules && bgOut >= 0 &&
         ((long long)bgOut + 1) * v.width <= v.capacity) { // Regions.cu:647-652
@@ -752,8 +804,10 @@ PYR_FN void pyr_sweep_tail(const PyrArgs &a, const PyrLds &s, int b, int t, int 
     if (lane == 0)
       v.bg[b] = bgOut;
   }
+  if (lb != a.nMasks - 1 || a.nLevels == lb)
+    return;
   const PyrLv &v = s.lv[a.nLevels];
-  if (v.flags & PYR_LV_TERMINAL) {
+  {
     // terminalGridPoolingRules (TerminalPoolingLayer.cu:8-20): the rows in
     // iteration order, or the background row of a sample without sites;
     // padded with -1 to the batch's largest sample (:90-96)

@@ -54,7 +54,7 @@ template <int D> void pass_a(const PyrArgs &a, int b, int T, bool *gaveUp) {
     c[0] = cnt[x];
     c[1] = (long long)cnt[x] < a.lv[x].fullSize;
   }
-  bool fits = pyr_lds_need(a, cnt) <= a.ldsBytesB;
+  bool fits = pyr_fits(a, cnt);
   for (int x = 0; x < a.nMasks; ++x)
     fits = fits && cnt[x] <= PYR_ROWS_MAX;
   if (!fits)
@@ -66,7 +66,6 @@ template <int D> void pass_b(const PyrArgs &a, int b, int T, bool gaveUp, long l
   std::vector<unsigned char> ldsv((size_t)a.ldsBytesB);
   unsigned char *lds = ldsv.data();
   PyrHdr *h = reinterpret_cast<PyrHdr *>(lds);
-  const int nRegions = a.nMasks - 1;
   h->over = 0;
   memcpy(lds + PYR_HDR_BYTES, a.pyramid + (long long)b * a.pyrStride, 8ll * a.pyrStride);
   for (int x = 0; x < a.nMasks; ++x) {
@@ -91,26 +90,10 @@ template <int D> void pass_b(const PyrArgs &a, int b, int T, bool gaveUp, long l
     h->bgAll[x] = v3;
     h->maxAct[x] = mx;
   }
-  for (int t = 0; t <= a.nMasks; ++t) {
-    int sum = 0;
-    for (int x = 0; x < t; ++x)
-      sum += h->n[x];
-    h->siteOff[t] = sum;
-    if (t < a.nMasks)
-      pyr_fill_en(a.lv[t], lds, t, sum);
-    if (t == a.nMasks)
-      h->total = sum;
-  }
-  for (int t = 1; t <= nRegions + 1; ++t) {
-    int sum = 0;
-    for (int l = 1; l < t; ++l)
-      sum += h->n[l];
-    h->itemOff[t] = sum;
-  }
   for (int t = 1; t <= a.nLevels; ++t)
     if (pyr_report(a, a.lv[t], h, t).over)
       h->over |= 1;
-  if (pyr_lds_need(a, h->n) > a.ldsBytesB)
+  if (!pyr_fits(a, h->n))
     h->over |= 2;
   const bool over = h->over != 0 || gaveUp;
   if (b == 0)
@@ -125,46 +108,65 @@ template <int D> void pass_b(const PyrArgs &a, int b, int T, bool gaveUp, long l
     *overOut = true;
     return;
   }
-  const PyrLds s = pyr_lds_view(a, lds, h->total, h->n[0]);
-  // (the last array must end inside what pass B was launched with)
-  if (s.kOf + h->total > lds + a.ldsBytesB) {
-    fprintf(stderr, "pyr_lds_need promises less than pyr_lds_view takes\n");
-    abort();
-  }
-  for (int t = 1; t <= a.nLevels; ++t)
-    pyr_fill_level(a.lv[t], a.lv[t - 1].maskOff, a.bg[b], s, t);
-  for (int t = 0; t < T; ++t)
-    pyr_sweep_clear(s, t, T);
-  for (int t = 0; t < T; ++t)
-    pyr_sweep_enumerate<D>(a, s, t, T);
-  {
-    const PyrLevel &L = a.lv[0];
-    const long long p0 = (long long)b * L.volOut;
-    for (int r = 0; r < h->n[0]; ++r) {
-      int c[D];
-      pyr_unpack<D>(s.key[r], c);
-      s.srcRow[r] = (unsigned)a.dense[p0 + pyr_key<D>(c, L.nOut)];
-    }
-  }
-  for (int t = 0; t < T; ++t)
-    pyr_sweep_owners<D>(s, nRegions, t, T);
-  for (int x = 0; x < nRegions; ++x) {
-    unsigned carry = 0;
-    for (int r = 0; r < h->n[x]; ++r) {
-      s.base[h->siteOff[x] + r] = (unsigned short)carry;
-      carry += (unsigned)pyr_popc32(pyr_own_mask(s, (unsigned)(h->siteOff[x] + r)));
-    }
-    if ((int)carry != h->n[x + 1]) {
-      fprintf(stderr, "level %d: %u sites owned, %d sites exist\n", x + 1, carry, h->n[x + 1]);
+  int windows = 0;
+  for (int xa = 0;;) {
+    const int xb = pyr_window_end(a, h->n, xa);
+    const int la = xa + 1, lb = xb;
+    const bool last = xb == a.nMasks - 1;
+    ++windows;
+    for (int t = 0; t <= a.nMasks; ++t)
+      pyr_fill_offsets(h, xa, xb, t);
+    for (int t = 0; t < a.nMasks; ++t)
+      pyr_fill_en(a.lv[t], lds, t, h->siteOff[t]);
+    const PyrLds s = pyr_lds_view(a, lds, h->total, h->n[xa]);
+    // (the last array must end inside what pass B was launched with)
+    if (s.kOf + h->total > lds + a.ldsBytesB || pyr_lds_window(a, h->n, xa, xb) > a.ldsBytesB) {
+      fprintf(stderr, "a window takes more LDS than pass B was launched with\n");
       abort();
     }
+    for (int t = 1; t <= a.nLevels; ++t)
+      if ((t >= la && t <= lb) || (last && t == a.nLevels && t > lb))
+        pyr_fill_level(a.lv[t], a.lv[t - 1].maskOff, a.bg[b], s, t, xa);
+    for (int t = 0; t < T; ++t)
+      pyr_sweep_clear(s, t, T);
+    for (int t = 0; t < T; ++t)
+      pyr_sweep_enumerate<D>(a, s, xa, xb, t, T);
+    if (xa == 0) {
+      const PyrLevel &L = a.lv[0];
+      const long long p0 = (long long)b * L.volOut;
+      for (int r = 0; r < h->n[0]; ++r) {
+        int c[D];
+        pyr_unpack<D>(s.key[r], c);
+        s.srcRow[r] = (unsigned)a.dense[p0 + pyr_key<D>(c, L.nOut)];
+      }
+    }
+    for (int t = 0; t < T; ++t)
+      pyr_sweep_owners<D>(s, la, lb, t, T);
+    for (int x = xa; x < xb; ++x) {
+      unsigned carry = 0;
+      for (int r = 0; r < h->n[x]; ++r) {
+        s.base[h->siteOff[x] + r] = (unsigned short)carry;
+        carry += (unsigned)pyr_popc32(pyr_own_mask(s, (unsigned)(h->siteOff[x] + r)));
+      }
+      if ((int)carry != h->n[x + 1]) {
+        fprintf(stderr, "level %d: %u sites owned, %d sites exist\n", x + 1, carry, h->n[x + 1]);
+        abort();
+      }
+    }
+    for (int t = 0; t < T; ++t)
+      pyr_sweep_rows<D>(s, la, lb, b, t, T);
+    for (int t = 0; t < T; ++t)
+      pyr_sweep_rules<D>(s, la, lb, t, T);
+    for (int t = 0; t < T; ++t)
+      pyr_sweep_tail(a, s, la, lb, b, t, T);
+    if (last)
+      break;
+    for (int t = 0; t < T; ++t)
+      pyr_sweep_carry(s, lds, a, xb, t, T);
+    xa = xb;
   }
-  for (int t = 0; t < T; ++t)
-    pyr_sweep_rows<D>(s, nRegions, b, t, T);
-  for (int t = 0; t < T; ++t)
-    pyr_sweep_rules<D>(s, nRegions, t, T);
-  for (int t = 0; t < T; ++t)
-    pyr_sweep_tail(a, s, b, t, T);
+  if (windows > report[0])
+    report[0] = windows; // (the most windows a sample took)
 }
 
 template <int D> int run(PyrArgs &a, int T, long long *report) {
@@ -182,7 +184,8 @@ template <int D> int run(PyrArgs &a, int T, long long *report) {
 // scn_grids_build takes them.  Per layer l (1-based) rules[l - 1] (capacity
 // rulesCap[l - 1] ints, may be null), ekey / erow / bgOut [l - 1]; bounds
 // [l - 1][2] = {rows, active}.  report: [nLevels + 1][4] = sites, active sites,
-// outgrew, terminal width or largest sample.  Returns 0, or 1 | 2 when a sample
+// outgrew, terminal width or largest sample; report[0][0] = the most windows of
+// levels a sample was built in.  Returns 0, or 1 | 2 when a sample
 // outgrew the LDS or a layer its bounds (nothing is written then).
 extern "C" int pyr_cpu_chain(int d, int batch, int n0, int nLevels, const int *geo, const int *sample,
                              const long long *key, const int *row, long long nActive, const int *bg,

@@ -180,6 +180,32 @@ def test_dense_and_sparse_extremes(harness):
     check(harness, 3, 11, CHAINS[3][2], 4, 903, fill=0.7)
 
 
+WINDOWED = [
+    (2, 70, [("c", 2, 1)] * 5 + [("c", 3, 2), ("c", 2, 1), ("t",)], 0.05),
+    (2, 70, [("c", 1, 1), ("c", 2, 1), ("c", 1, 1), ("c", 3, 1), ("c", 3, 2), ("c", 2, 1)], 0.05),
+    (3, 17, [("c", 2, 1), ("c", 1, 1), ("c", 2, 1), ("c", 2, 1), ("c", 2, 2), ("c", 2, 1), ("t",)], 0.03),
+    (1, 300, [("c", 3, 1), ("c", 2, 1), ("c", 5, 1), ("c", 3, 2), ("c", 3, 1), ("t",)], 0.2),
+]
+
+
+@pytest.mark.parametrize("case", range(len(WINDOWED)))
+def test_levels_taken_a_window_at_a_time(harness, case):
+    """With little LDS pass B builds a sample's layers in several windows of levels, the rows of a window's last
+    level carried into the next one; the rule books are the same."""
+    d, n0, layers, fill = WINDOWED[case]
+    seen = set()
+    for kb in list(range(7, 40)) + list(range(40, 153, 4)):
+        rc, want, report, *_ = run_chain(harness, d, n0, layers, 5, 700 + case, fill=fill, lds=kb * 1024, T=64)
+        if rc != 0:
+            continue  # (not even one layer of some sample fits: reported, nothing written)
+        w = int(report[0, 0])
+        if w not in seen:
+            check(harness, d, n0, layers, 5, 700 + case, fill=fill, lds=kb * 1024, T=64)
+            check(harness, d, n0, layers, 5, 700 + case, fill=fill, lds=kb * 1024, T=512)
+        seen.add(w)
+    assert max(seen) >= 3, seen
+
+
 def test_a_sample_that_outgrows_the_lds_is_reported(harness):
     d, n0, layers = CHAINS[1]
     rc, want, report, rules, *_ = run_chain(harness, d, n0, layers, 6, 5, fill=0.6, lds=8 * 1024)
