@@ -1334,6 +1334,8 @@ static int chain_flush_pyramid(scn_ctx *ctx, ChainState *cs, std::vector<ChainRe
     if (L.mode != MODE_SQ_NOMIN || L.cube > PYR_CUBE_MAX || L.size < 1 ||
         (d >= 2 && L.size > 4) || L.stride < 1)
       return SCN_OK;
+    if ((uintptr_t)L.rules & 15) // (rule rows are stored two or four entries at a time)
+      return SCN_OK;
   }
   if ((int)recs.size() > PYR_MAX_LEVELS)
     return SCN_OK;

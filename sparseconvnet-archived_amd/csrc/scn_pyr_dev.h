@@ -726,6 +726,13 @@ PYR_FN int pyr_bg_row(const PyrArgs &a, const PyrLds &s, int x, int b) {
   return h->hasBg[x] ? (int)(h->actBefore[x] + h->bgBefore[x]) + h->n[x] : -1;
 }
 
+struct alignas(8) PyrInt2 {
+  int x, y;
+};
+struct alignas(16) PyrInt4 {
+  int x, y, z, w;
+};
+
 // ---- sweep 5: rule rows
 template <int D>
 PYR_FN void pyr_sweep_rules(const PyrLds &s, int la, int lb, int t, int T) {
@@ -761,11 +768,32 @@ PYR_FN void pyr_sweep_rules(const PyrLds &s, int la, int lb, int t, int T) {
         const unsigned present = (win >> (i * side)) & ((1u << side) - 1u);
         // the active sites of a window row are neighbours in rank
         unsigned rank = present ? pyr_rank(in, pref, rowPos[i]) : 0u;
-        for (int q = 0; q < side; ++q) {
-          int val = bgIn;
-          if ((present >> q) & 1u)
-            val = pyr_in_row(v, s, rank++);
-          dst[i * side + q] = val;
+        if constexpr (D >= 2 && S % 2 == 0) {
+          // (a rule row of 4 or 8 or 16 ... entries starts on 16 bytes: two
+          // or four entries a store)
+          int val[S];
+#if defined(__HIPCC__)
+#pragma unroll
+#endif
+          for (int q = 0; q < S; ++q) {
+            val[q] = bgIn;
+            if ((present >> q) & 1u)
+              val[q] = pyr_in_row(v, s, rank++);
+          }
+          if constexpr (S == 2) {
+            PyrInt2 o = {val[0], val[1]};
+            *reinterpret_cast<PyrInt2 *>(dst + i * S) = o;
+          } else {
+            PyrInt4 o = {val[0], val[1], val[2], val[3]};
+            *reinterpret_cast<PyrInt4 *>(dst + i * S) = o;
+          }
+        } else {
+          for (int q = 0; q < side; ++q) {
+            int val = bgIn;
+            if ((present >> q) & 1u)
+              val = pyr_in_row(v, s, rank++);
+            dst[i * side + q] = val;
+          }
         }
       }
     });
