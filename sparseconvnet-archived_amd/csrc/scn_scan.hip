@@ -1,5 +1,9 @@
-// Exclusive prefix sums over uint32 counts (or popcounts of 64-bit words),
-// three-phase: per-tile totals, recursive scan of the totals, per-tile rescan.
+// Exclusive prefix sums over uint32 counts (or popcounts of 64-bit words).
+// Short arrays: one workgroup (scn_scan_dev.h).  Long ones: one pass with a
+// decoupled look-back -- every workgroup takes the next tile, sums it, publishes
+// the sum, adds up what the tiles before it have published (walking back until
+// it meets one that already knows its whole prefix) and writes its prefixes; the
+// input is read once and nothing is launched in between.
 #include "scn_common.h"
 #include "scn_scan_dev.h"
 
@@ -70,44 +74,35 @@ __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v,
   return before + incl - v;
 }
 
-// the block's sum in thread 0 (every thread gets it)
-__device__ __forceinline__ uint32_t block_sum(uint32_t v, uint32_t *lds) {
+// A tile's word of state: bits 63..62 say what the low 32 bits are -- nothing
+// yet (0), the tile's own sum (1), the sum of everything up to and including
+// the tile (2).  One 64-bit word, so flag and value arrive together.
+#define LB_SUM (1ull << 62)
+#define LB_PREFIX (2ull << 62)
+
+__global__ void k_scan_clear(unsigned long long *state, size_t words) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < words)
+    state[i] = 0ull;
+}
+
+// state[0 .. nb): the tiles' words; state[nb]: the ticket counter (tiles are
+// handed out in the order the workgroups arrive, so a workgroup only ever waits
+// for workgroups that are already running).  All zero at launch.
+template <bool POPC>
+__global__ void __launch_bounds__(SCAN_THREADS)
+    k_scan_lookback(const void *in, uint32_t *out, size_t n, unsigned long long *state,
+                    unsigned nb) {
+  __shared__ uint32_t lds[SCAN_THREADS];
+  __shared__ unsigned sTile;
+  __shared__ uint32_t sBefore;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1)
-    v += __shfl_xor(v, off, 64);
-  if (lane == 0)
-    lds[wave] = v;
-  __syncthreads();
-  return lds[0] + lds[1] + lds[2] + lds[3];
-}
-
-template <bool POPC>
-__global__ void __launch_bounds__(SCAN_THREADS)
-    k_scan_reduce(const void *in, size_t n, uint32_t *tileSums) {
-  __shared__ uint32_t lds[SCAN_THREADS];
-  size_t base = (size_t)blockIdx.x * SCAN_TILE + (size_t)threadIdx.x * SCAN_PER_THREAD;
-  const bool whole = ((size_t)blockIdx.x + 1) * SCAN_TILE <= n && ((uintptr_t)in & 15) == 0;
-  uint32_t v[SCAN_PER_THREAD];
-  scan_load_tile<POPC>(in, base, n, whole, v);
-  uint32_t s = 0;
-#pragma unroll
-  for (int k = 0; k < SCAN_PER_THREAD; ++k)
-    s += v[k];
-  const uint32_t total = block_sum(s, lds);
   if (threadIdx.x == 0)
-    tileSums[blockIdx.x] = total;
-}
-
-// out[i] = tileOffsets[tile] + exclusive prefix inside the tile; the block that
-// owns element n - 1 also writes out[n] = grand total.
-template <bool POPC>
-__global__ void __launch_bounds__(SCAN_THREADS)
-    k_scan_final(const void *in, uint32_t *out, size_t n,
-                 const uint32_t *tileOffsets) {
-  __shared__ uint32_t lds[SCAN_THREADS];
-  size_t base = (size_t)blockIdx.x * SCAN_TILE + (size_t)threadIdx.x * SCAN_PER_THREAD;
-  const bool whole = ((size_t)blockIdx.x + 1) * SCAN_TILE <= n && ((uintptr_t)in & 15) == 0 &&
+    sTile = atomicAdd(reinterpret_cast<unsigned *>(state + nb), 1u);
+  __syncthreads();
+  const unsigned tile = sTile;
+  const size_t base = (size_t)tile * SCAN_TILE + (size_t)threadIdx.x * SCAN_PER_THREAD;
+  const bool whole = ((size_t)tile + 1) * SCAN_TILE <= n && ((uintptr_t)in & 15) == 0 &&
                      ((uintptr_t)out & 15) == 0;
   uint32_t v[SCAN_PER_THREAD];
   scan_load_tile<POPC>(in, base, n, whole, v);
@@ -116,8 +111,44 @@ __global__ void __launch_bounds__(SCAN_THREADS)
   for (int k = 0; k < SCAN_PER_THREAD; ++k)
     s += v[k];
   uint32_t total;
-  uint32_t excl = block_exclusive_scan(s, lds, &total);
-  uint32_t off = tileOffsets ? tileOffsets[blockIdx.x] : 0u;
+  const uint32_t excl = block_exclusive_scan(s, lds, &total);
+  if (wave == 0) {
+    if (lane == 0)
+      __hip_atomic_store(&state[tile], (tile == 0 ? LB_PREFIX : LB_SUM) | total, __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+    uint32_t before = 0;
+    if (tile > 0) {
+      // lane i looks at tile - 1 - i, then 64 further back, ...; tiles before
+      // the first count as knowing their prefix: 0
+      long long j = (long long)tile - 1 - lane;
+      for (;;) {
+        unsigned long long w;
+        for (;;) {
+          w = j >= 0 ? __hip_atomic_load(&state[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : LB_PREFIX;
+          if (!__any((w >> 62) == 0ull))
+            break;
+          __builtin_amdgcn_s_sleep(1);
+        }
+        const unsigned long long known = __ballot((w >> 62) >= 2ull);
+        const int first = known ? __ffsll((long long)known) - 1 : 64;
+        uint32_t c = lane <= first ? (uint32_t)w : 0u;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1)
+          c += __shfl_xor(c, off, 64);
+        before += c;
+        if (known)
+          break;
+        j -= 64;
+      }
+      if (lane == 0)
+        __hip_atomic_store(&state[tile], LB_PREFIX | (unsigned long long)(uint32_t)(before + total),
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (lane == 0)
+      sBefore = before;
+  }
+  __syncthreads();
+  const uint32_t off = sBefore;
   uint32_t run = off + excl;
   if (whole) {
     uint32_t r[SCAN_PER_THREAD];
@@ -137,7 +168,7 @@ __global__ void __launch_bounds__(SCAN_THREADS)
       run += v[k];
     }
   }
-  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0)
+  if (tile == nb - 1 && threadIdx.x == 0)
     out[n] = off + total;
 }
 
@@ -149,13 +180,8 @@ __global__ void __launch_bounds__(SCAN1_THREADS)
 }
 
 size_t scn_scan_tmp_elems(size_t n) {
-  size_t total = 0;
-  while (n > SCAN_TILE) {
-    size_t nb = (n + SCAN_TILE - 1) / SCAN_TILE;
-    total += 2 * nb + 8; // tile sums + their exclusive scan (nb + 1)
-    n = nb;
-  }
-  return total + 8;
+  const size_t nb = (n + SCAN_TILE - 1) / SCAN_TILE;
+  return 2 * (nb + 1) + 8; // a 64-bit word a tile, one for the tickets, room to align them
 }
 
 template <bool POPC>
@@ -167,21 +193,15 @@ static int scan_impl(hipStream_t s, const void *in, uint32_t *out, size_t n,
     SCN_HIP_CHECK(hipGetLastError());
     return SCN_OK;
   }
-  size_t nb = (n + SCAN_TILE - 1) / SCAN_TILE;
-  if (nb <= 1) {
-    hipLaunchKernelGGL(k_scan_final<POPC>, dim3(1), dim3(SCAN_THREADS), 0, s, in,
-                       out, n, (const uint32_t *)nullptr);
-    SCN_HIP_CHECK(hipGetLastError());
-    return SCN_OK;
-  }
-  uint32_t *sums = tmp;
-  uint32_t *offs = tmp + nb + 4;
-  hipLaunchKernelGGL(k_scan_reduce<POPC>, dim3((unsigned)nb), dim3(SCAN_THREADS),
-                     0, s, in, n, sums);
+  const size_t nb = (n + SCAN_TILE - 1) / SCAN_TILE;
+  SCN_REQUIRE(nb < 0x7FFFFFFFull, SCN_ERR_CAPACITY, "scan: %zu elements", n);
+  unsigned long long *state =
+      reinterpret_cast<unsigned long long *>(((uintptr_t)tmp + 7) & ~(uintptr_t)7);
+  hipLaunchKernelGGL(k_scan_clear, dim3((unsigned)((nb + 1 + 255) / 256)), dim3(256), 0, s,
+                     state, nb + 1);
   SCN_HIP_CHECK(hipGetLastError());
-  SCN_TRY(scan_impl<false>(s, sums, offs, nb, tmp + 2 * nb + 8));
-  hipLaunchKernelGGL(k_scan_final<POPC>, dim3((unsigned)nb), dim3(SCAN_THREADS),
-                     0, s, in, out, n, (const uint32_t *)offs);
+  hipLaunchKernelGGL(k_scan_lookback<POPC>, dim3((unsigned)nb), dim3(SCAN_THREADS), 0, s, in,
+                     out, n, state, (unsigned)nb);
   SCN_HIP_CHECK(hipGetLastError());
   return SCN_OK;
 }

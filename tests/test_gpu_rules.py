@@ -76,6 +76,27 @@ def test_square_rules_rows_longer_than_a_mask_word(scn, ctx, d, size, stride, nO
         run_both(scn, ctx, samples, d, nIn, nOut, size, stride, 1, False, nSites)
 
 
+@pytest.mark.parametrize("d,nIn,size,stride,batch,density", [(2, 1025, 3, 2, 5, 0.02), (3, 130, 2, 1, 3, 0.015),
+                                                            (2, 1500, 2, 2, 2, 0.03)])
+def test_rule_books_whose_prefix_sums_take_many_tiles(scn, ctx, d, nIn, size, stride, batch, density):
+    """Masks of more than 65536 words and more than 65536 active sites: both prefix sums of a plan (set bits of the
+    mask, candidates per input) are then made in one pass over many tiles, each workgroup adding up what the tiles
+    before it have published."""
+    rng = np.random.default_rng(nIn + size)
+    nOut = (nIn - size) // stride + 1
+    samples, nSites = brute.random_samples(rng, batch, d, nIn, density)
+    assert batch * nIn ** d > 64 * 65536 and sum(len(m) for _, m in samples) > 65536
+    run_both(scn, ctx, samples, d, nIn, nOut, size, stride, 1, False, nSites)
+    # an input with a few very long runs of empty tiles between its sites
+    sparse = []
+    row = 0
+    for b in range(batch):
+        keys = rng.choice(nIn ** d, size=37, replace=False)
+        sparse.append((row, {int(k): row + 1 + i for i, k in enumerate(keys)}))
+        row += 38
+    run_both(scn, ctx, sparse, d, nIn, nOut, size, stride, 1, False, row)
+
+
 def test_find_on_grids_without_a_table(scn, ctx):
     """Look-ups by coordinate on grids whose hash table is only built when asked for: input grids of a batch too large
     for a dense row table, and the output grids of a rule-book plan (which never get either as they are built)."""
