@@ -111,6 +111,7 @@ static inline int scn_ceil_div(int64_t a, int64_t b) {
 
 // address of the static scratch of scn_sgemm_ABt_static on `device` (scn_train.hip)
 int scn_abt_static_setup(int device);
+void scn_abt_static_forget(const scn_ctx *ctx);
 
 // runs the recorded rule-book plans of the context, if any (scn_chain.hip)
 int scn_chain_flush(scn_ctx *ctx);

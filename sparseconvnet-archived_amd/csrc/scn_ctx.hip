@@ -42,7 +42,10 @@ extern "C" int scn_ctx_create(int device, scn_ctx **out) {
   hipDeviceProp_t prop;
   SCN_HIP_CHECK(hipGetDeviceProperties(&prop, device));
   c->numCU = prop.multiProcessorCount;
-  SCN_HIP_CHECK(hipStreamCreate(&c->stream)); // default priority
+  // default priority, and BLOCKING (hipStreamCreate, not hipStreamNonBlocking):
+  // a copy made with no context goes through the legacy stream and must wait
+  // for this one -- scn_h2d / scn_d2h with a null context count on that
+  SCN_HIP_CHECK(hipStreamCreate(&c->stream));
   SCN_HIP_CHECK(hipHostMalloc((void **)&c->h_pinned, SCN_PINNED_WORDS * sizeof(int64_t),
                               hipHostMallocMapped));
   memset(c->h_pinned, 0, SCN_PINNED_WORDS * sizeof(int64_t));
@@ -64,6 +67,7 @@ extern "C" int scn_ctx_destroy(scn_ctx *c) {
     return SCN_OK;
   (void)scn_chain_flush(c);
   (void)hipStreamSynchronize(c->stream);
+  scn_abt_static_forget(c);
   scn_chain_release(c);
   for (auto &s : c->spans) {
     (void)hipEventDestroy(s.a);

@@ -103,7 +103,8 @@ template <int VEC>
 __global__ void __launch_bounds__(256)
     k_maxpool(const float *__restrict__ in, float *__restrict__ out,
               const int *__restrict__ rules, long long nOutSites, int ps,
-              int C, int chunks, int *__restrict__ choice) {
+              int C, int chunks, int *__restrict__ choice,
+              const float *__restrict__ spare) {
   long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= nOutSites * chunks)
     return;
@@ -119,9 +120,10 @@ __global__ void __launch_bounds__(256)
   }
   bool none = true;
   // Nine candidates at a time: their rules are requested together, then
-  // their values (a skipped rule reads row 0 and is dropped below), so that a
-  // window costs two trips to memory rather than two per candidate; they
-  // are compared in rule order.
+  // their values (a skipped rule reads the context's spare row -- never `in`,
+  // which may have no rows at all -- and is dropped below), so that a window
+  // costs two trips to memory rather than two per candidate; they are
+  // compared in rule order.
   constexpr int MP = 9;
   for (int p0 = 0; p0 < ps; p0 += MP) {
     int rule[MP];
@@ -131,7 +133,8 @@ __global__ void __launch_bounds__(256)
     float v[MP][VEC];
 #pragma unroll
     for (int u = 0; u < MP; ++u) {
-      const float *src = in + (long long)(rule[u] > 0 ? rule[u] : 0) * C + c0;
+      const float *src = rule[u] >= 0 ? in + (long long)rule[u] * C + c0
+                                      : spare + (c0 & (SCN_ZERO_FLOATS - VEC));
       if (VEC == 4) {
         float4 t = *reinterpret_cast<const float4 *>(src);
         v[u][0] = t.x;
@@ -179,19 +182,22 @@ extern "C" int scn_maxpool(scn_ctx *ctx, const float *d_in, float *d_out,
               ps, C);
   if (nOutSites == 0)
     return SCN_OK;
-  SCN_REQUIRE(d_in && d_out && d_rules && d_choice, SCN_ERR_ARG,
+  // (d_in may be null: an input without rows, every rule negative)
+  SCN_REQUIRE(d_out && d_rules && d_choice, SCN_ERR_ARG,
               "scn_maxpool: null buffer");
   ProfScope prof(ctx, SCN_K_MAXPOOL);
   if (C % 4 == 0 && aligned16(d_in) && aligned16(d_out) && aligned16(d_choice)) {
     long long total = nOutSites * (C / 4);
     hipLaunchKernelGGL(k_maxpool<4>, dim3(scn_ceil_div(total, 256)), dim3(256),
                        0, ctx->stream, d_in, d_out, d_rules,
-                       (long long)nOutSites, ps, C, C / 4, d_choice);
+                       (long long)nOutSites, ps, C, C / 4, d_choice,
+                       (const float *)ctx->d_zeros);
   } else {
     long long total = nOutSites * C;
     hipLaunchKernelGGL(k_maxpool<1>, dim3(scn_ceil_div(total, 256)), dim3(256),
                        0, ctx->stream, d_in, d_out, d_rules,
-                       (long long)nOutSites, ps, C, C, d_choice);
+                       (long long)nOutSites, ps, C, C, d_choice,
+                       (const float *)ctx->d_zeros);
   }
   SCN_HIP_CHECK(hipGetLastError());
   return SCN_OK;
@@ -215,7 +221,7 @@ extern "C" int scn_maxpool_checked(scn_ctx *ctx, const float *d_in,
 __global__ void k_terminal_pool(const float *__restrict__ in,
                                 float *__restrict__ out,
                                 const int *__restrict__ rules, long long count,
-                                int S, int C) {
+                                int S, int C, const float *__restrict__ spare) {
   long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= count * C)
     return;
@@ -225,8 +231,8 @@ __global__ void k_terminal_pool(const float *__restrict__ in,
   float t = 0.f;
   int p = 0;
   // four rows at a time: their rules requested together, then their values
-  // (a rule past the sample's last reads row 0 and ends the sum); added in
-  // rule order
+  // (a rule past the sample's last reads the context's spare row, never `in`,
+  // and ends the sum); added in rule order
   bool more = true;
   for (int p0 = 0; p0 < S && more; p0 += 4) {
     int rule[4];
@@ -236,7 +242,7 @@ __global__ void k_terminal_pool(const float *__restrict__ in,
     float v[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u)
-      v[u] = in[(long long)(rule[u] > 0 ? rule[u] : 0) * C + j];
+      v[u] = rule[u] >= 0 ? in[(long long)rule[u] * C + j] : spare[j & (SCN_ZERO_FLOATS - 1)];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       more = more && rule[u] >= 0;
@@ -258,12 +264,13 @@ extern "C" int scn_terminal_pool(scn_ctx *ctx, const float *d_in, float *d_out,
               C);
   if (count == 0)
     return SCN_OK;
-  SCN_REQUIRE(d_in && d_out && d_rules, SCN_ERR_ARG,
+  // (d_in may be null: an input without rows, every rule negative)
+  SCN_REQUIRE(d_out && d_rules, SCN_ERR_ARG,
               "scn_terminal_pool: null buffer");
   ProfScope prof(ctx, SCN_K_TERMINAL);
   hipLaunchKernelGGL(k_terminal_pool, dim3(scn_ceil_div(count * C, 256)),
                      dim3(256), 0, ctx->stream, d_in, d_out, d_rules,
-                     (long long)count, S, C);
+                     (long long)count, S, C, (const float *)ctx->d_zeros);
   SCN_HIP_CHECK(hipGetLastError());
   return SCN_OK;
 }

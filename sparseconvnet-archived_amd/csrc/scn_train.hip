@@ -9,6 +9,7 @@
 //   convolution                dPropBackwardFromMatrixMultiplyOutput, ConvolutionalLayer.cu:42-63
 //   max-pooling                dMaxPoolBackProp, MaxPoolingLayer.cu:74-82
 //   terminal pooling           dTerminalPoolBackProp, TerminalPoolingLayer.cu:48-62
+#include <mutex>
 #include "scn_common.h"
 #include <hip/amd_detail/amd_hip_unsafe_atomics.h>
 
@@ -509,11 +510,17 @@ extern "C" int scn_sgemm_ABt(scn_ctx *ctx, const float *d_D, const float *d_W,
 #define ABT_STATIC_FLOATS (1 << 20) // 4 MiB per device
 static __device__ __align__(256) float scratch[ABT_STATIC_FLOATS];
 #define ABT_MAX_DEVICES 64
-static float *g_abtScratch[ABT_MAX_DEVICES]; // per device, set once by scn_ctx_create
+// per device, set once by scn_ctx_create: the array's address, an event that
+// marks the end of the last call that used it, and whose call that was
+static float *g_abtScratch[ABT_MAX_DEVICES];
+static hipEvent_t g_abtDone[ABT_MAX_DEVICES];
+static const scn_ctx *g_abtUser[ABT_MAX_DEVICES];
+static std::mutex g_abtMutex;
 
 int scn_abt_static_setup(int device) {
   SCN_REQUIRE(device >= 0 && device < ABT_MAX_DEVICES, SCN_ERR_ARG,
               "device %d: at most %d devices", device, ABT_MAX_DEVICES);
+  std::lock_guard<std::mutex> lock(g_abtMutex); // (contexts are made by several threads)
   if (g_abtScratch[device])
     return SCN_OK;
   float *ptr = nullptr;
@@ -521,8 +528,17 @@ int scn_abt_static_setup(int device) {
   SCN_HIP_CHECK(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
   SCN_REQUIRE(ptr != nullptr, SCN_ERR_HIP,
               "hipGetSymbolAddress returned no address for the static scratch");
+  SCN_HIP_CHECK(hipEventCreateWithFlags(&g_abtDone[device], hipEventDisableTiming));
   g_abtScratch[device] = ptr;
   return SCN_OK;
+}
+
+// a context that is destroyed gives the array up
+void scn_abt_static_forget(const scn_ctx *ctx) {
+  std::lock_guard<std::mutex> lock(g_abtMutex);
+  for (int d = 0; d < ABT_MAX_DEVICES; ++d)
+    if (g_abtUser[d] == ctx)
+      g_abtUser[d] = nullptr;
 }
 
 extern "C" int64_t scn_sgemm_ABt_static_limit(void) { return ABT_STATIC_FLOATS; }
@@ -539,15 +555,34 @@ extern "C" int scn_sgemm_ABt_static(scn_ctx *ctx, const float *d_D,
               "scratch, the static array holds %d; use scn_sgemm_ABt with a "
               "workspace",
               N, K, (long long)scn_sgemm_ABt_workspace(N, K), ABT_STATIC_FLOATS);
-  float *ptr = ctx->device >= 0 && ctx->device < ABT_MAX_DEVICES
-                   ? g_abtScratch[ctx->device]
-                   : nullptr;
+  const int dev = ctx->device;
+  float *ptr = dev >= 0 && dev < ABT_MAX_DEVICES ? g_abtScratch[dev] : nullptr;
   SCN_REQUIRE(ptr, SCN_ERR_STATE,
-              "scn_sgemm_ABt_static: no scratch address for device %d",
-              ctx->device);
+              "scn_sgemm_ABt_static: no scratch address for device %d", dev);
+  if (M == 0)
+    return SCN_OK;
+  // One array a device: calls of one context follow each other on its stream;
+  // a call of another context while the last one has not finished is refused.
+  // (a stream under capture records and queries nothing: its owner has to
+  // keep other users of the array away for as long as the graph may run)
+  std::lock_guard<std::mutex> lock(g_abtMutex);
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  SCN_HIP_CHECK(hipStreamIsCapturing(ctx->stream, &capturing));
+  if (g_abtUser[dev] && g_abtUser[dev] != ctx) {
+    const hipError_t busy = hipEventQuery(g_abtDone[dev]);
+    SCN_REQUIRE(busy != hipErrorNotReady, SCN_ERR_STATE,
+                "scn_sgemm_ABt_static: the device's static array is still in "
+                "use by a call of another context");
+    SCN_HIP_CHECK(busy);
+  }
   // (the kernels clear and fill what they use of the array: nothing of an
   // earlier call is read)
-  return scn_sgemm_ABt(ctx, d_D, d_W, d_dA, M, N, K, ptr);
+  SCN_TRY(scn_sgemm_ABt(ctx, d_D, d_W, d_dA, M, N, K, ptr));
+  if (capturing == hipStreamCaptureStatusNone) {
+    SCN_HIP_CHECK(hipEventRecord(g_abtDone[dev], ctx->stream));
+    g_abtUser[dev] = ctx;
+  }
+  return SCN_OK;
 }
 
 // ---------------------------------------------------------- weight update

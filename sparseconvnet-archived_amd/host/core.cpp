@@ -80,6 +80,12 @@ static std::mutex seedMutex;
 RNG::RNG() {
   std::lock_guard<std::mutex> lock(seedMutex);
   static unsigned bump = 0;
+  // SCN_SEED in the environment: generators seeded from that number instead
+  // of the clock, in the order they are made (a repeatable run)
+  if (const char *fixed = std::getenv("SCN_SEED")) {
+    gen.seed((unsigned)std::strtoul(fixed, nullptr, 10) + 7919u * bump++);
+    return;
+  }
   auto now = std::chrono::high_resolution_clock::now().time_since_epoch();
   gen.seed((unsigned)now.count() + 7919u * bump++);
 }
@@ -175,12 +181,18 @@ template <typename t> vectorCUDA<t>::~vectorCUDA() {
 // No stream named (vectorCUDA.cu:26-57, blocking cudaMemcpy): a copy with a
 // null context waits for the work of every stream of the device first, so the
 // data is complete whichever net's stream produced it.
+// The flip itself is serialised: the forward lanes' threads share the layers'
+// parameters, and two of them may ask for dPtr() of a vector that a host-side
+// writer left on the CPU.
+static std::mutex g_flipMutex;
 template <typename t> void vectorCUDA<t>::copyToCPU() {
+  std::lock_guard<std::mutex> lock(g_flipMutex);
   if (!onGPU)
     return;
   toCPU(nullptr);
 }
 template <typename t> void vectorCUDA<t>::copyToGPU() {
+  std::lock_guard<std::mutex> lock(g_flipMutex);
   if (onGPU)
     return;
   toGPU(nullptr);

@@ -60,6 +60,10 @@ public:
 };
 
 int main(int argc, char **argv) {
+  // weights, dropout and the order of the pictures come from generators that
+  // the reference seeds from the clock; here from a fixed number, so that the
+  // check on the training below means the same in every run
+  setenv("SCN_SEED", "20150101", 0);
   int nPictures = argc > 1 ? std::atoi(argv[1]) : 500;
   int batchSize = argc > 2 ? std::atoi(argv[2]) : 100;
   SpatiallySparseDataset testSet;
@@ -120,9 +124,7 @@ int main(int argc, char **argv) {
               << std::endl;
     return 1;
   }
-  // (weights, dropout and the order of the pictures are drawn from a
-  // clock-seeded generator, as in the reference: the margin allows for that)
-  if (!(after < 0.7f * before)) {
+  if (!(after < 0.25f * before)) {
     std::cout << "training did not lower the cost: " << before << " -> "
               << after << std::endl;
     return 1;

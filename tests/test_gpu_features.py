@@ -56,6 +56,26 @@ def test_terminal_pool_bit_exact(scn, ctx):
     assert np.array_equal(d_out.download(), orc.terminal_pool(inp, rules, B, S, C))
 
 
+@pytest.mark.parametrize("C", [32, 5])
+def test_pooling_over_an_input_without_rows(scn, ctx, C):
+    """Every rule negative and no input row at all (a null input): max-pooling gives zeros and choice 0, terminal
+    pooling 0 / 0, as the oracle does; nothing of the input is read."""
+    nOut, ps = 70, 9
+    rules = np.full((nOut, ps), -1, np.int32)
+    d_out = ctx.array(np.full((nOut, C), 7, np.float32))
+    d_choice = ctx.array(np.full((nOut, C), 7, np.int32))
+
+    class null:  # no input buffer at all
+        ptr = None
+
+    ctx.maxpool(null, d_out, ctx.array(rules), nOut, ps, C, d_choice)
+    o_out, o_choice = orc.maxpool(np.zeros((1, C), np.float32), rules, nOut, ps, C)
+    assert np.array_equal(d_out.download(), o_out) and np.array_equal(d_choice.download(), o_choice)
+    ctx.terminal_pool(null, d_out, ctx.array(rules), nOut, ps, C)
+    want = orc.terminal_pool(np.zeros((1, C), np.float32), rules, nOut, ps, C)
+    assert np.array_equal(np.isnan(d_out.download()), np.isnan(want)) and np.all(np.isnan(want))
+
+
 def test_softmax(scn, ctx):
     rng = np.random.default_rng(2)
     for M, N in ((100, 100), (7, 40), (3, 1), (130, 1000)):
