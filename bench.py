@@ -2,19 +2,26 @@
 """Forward-path benchmark on one MI355X.
 
 A step is one forward pass of one synthetic batch through the C++ host classes
-(SparseConvNet) on top of libscn_hip.so: grid hash build, every rule book,
-gather / NiN / max-pool / terminal pool / softmax kernels, and the copy of the
-class probabilities back to the host.  `value` is measured with the batch's
-active sites and input features already in HBM when the timed region starts;
-`with_input_upload` is the same pass with sites and features in pinned host
-memory, uploaded for every batch (the forward time that also counts the H2D of
-the inputs).  Warm-up and timed batches are one pass: the producer threads are
-not restarted in between.
+(SparseConvNet) on top of libscn_hip.so: grid build, every rule book, gather /
+NiN / max-pool / terminal pool / softmax kernels, and the copy of the class
+probabilities back to the host.  `value` is measured with the batch's active
+sites and input features already in HBM when the timed region starts;
+`value_with_input_upload` / `with_input_upload` is the same pass with sites and
+features in pinned host memory, uploaded for every batch (the forward time that
+also counts the H2D of the inputs); `value_definition` says which is which.
+
+Warm-up batches, timed batches and a tail of untimed batches are ONE pass
+through one batch producer: the clock starts when the last warm-up batch is
+finished and stops when the last timed batch is, with the producers busy on
+both sides of the region.  The line carries the MEDIAN of `--regions` such
+regions (the single figures in `ms_per_step_regions`), the other
+configurations in `other_configs`, and HBM traffic only while the kernel
+sources hash to what the traffic was measured with.
 
 Prints ONE JSON line: active sites/s (value) and samples/s, the roofline of the
 kernel -- or the rule-book construction as a whole -- that takes the most GPU
 time, the busiest NiN contraction beside it, a per-kernel table, and the CPU
-oracle timed on this host's cores.
+oracle (its -O3 -march=native build, made here) timed on this host's cores.
 """
 import argparse
 import json
@@ -373,8 +380,10 @@ def measure(scn, hostapi, synthetic, args, number, precision, headline):
                            launches_per_step=r_launches, bound="hbm", achieved=round(a, 3), peak=HBM_PEAK_GBS,
                            unit="GB/s", frac=round(a / HBM_PEAK_GBS, 5), algorithmic_bytes=int(r_bytes), traffic=None)
         if r_launches <= 2.5:
-            rules_entry["note"] = ("every layer's rule book in two launches, one workgroup per sample walking the layers "
-                                   "in LDS: latency-bound integer work, the HBM roofline is far from binding")
+            rules_entry["note"] = ("every layer's rule book in two launches, one workgroup per sample: all layers' "
+                                   "occupancy masks by dilation, then owners, rows and rule rows per output site "
+                                   "in LDS; integer work bound by instruction issue on one compute unit per sample, "
+                                   "the HBM roofline is far from binding")
         else:
             rules_entry["note"] = ("layer by layer through masks, rank prefixes and rows by rank in HBM: a dozen "
                                    "launches per layer; the rule rows themselves leave at 4-6 TB/s")
