@@ -264,6 +264,20 @@ int scn_conv_nin_forward_p(scn_ctx *ctx, const float *d_in,
                            const float *d_W, const float *d_B,
                            const float *d_prelu, float *d_out, int64_t M, int N,
                            float p, int act, int precision);
+/* scn_conv_nin_forward_p with SCN_BF16 for a caller that can spare room for a
+ * bf16 copy of the input matrix: the nInRows x nIn values are rounded once
+ * (nearest even) into d_in16 (2 bytes each, 16-byte aligned) and the
+ * contraction reads its rows from there, half the bytes for a matrix whose
+ * rows the rules visit many times over.  The operands that reach the MFMA are
+ * the ones scn_conv_nin_forward_p(SCN_BF16) rounds in registers, so the result
+ * is the same bit for bit; shapes the bf16 W-streaming kernel does not take
+ * run as scn_conv_nin_forward_p(SCN_BF16) does.  Same reference operator
+ * (NetworkInNetworkLayer.cu:187-200 after ConvolutionalLayer.cu:125-133). */
+int scn_conv_nin_forward_a16(scn_ctx *ctx, const float *d_in, int64_t nInRows,
+                             void *d_in16, const int32_t *d_rules, int fs,
+                             int nIn, const float *d_W, const float *d_B,
+                             const float *d_prelu, float *d_out, int64_t M,
+                             int N, float p, int act);
 /* maxPool (MaxPoolingLayer.h:6-7; MaxPoolingLayer.cu:9-72): first maximum
  * wins, negative rules skipped, choice = rule * C + channel. */
 int scn_maxpool(scn_ctx *ctx, const float *d_in, float *d_out,

@@ -113,6 +113,8 @@ def lib():
         "scn_conv_nin_supported_p": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int]),
         "scn_conv_nin_forward_p": (C.c_int, [vp, vp, vp, C.c_int, C.c_int, vp, vp, vp, vp, i64, C.c_int, f32, C.c_int,
                                              C.c_int]),
+        "scn_conv_nin_forward_a16": (C.c_int, [vp, vp, i64, vp, vp, C.c_int, C.c_int, vp, vp, vp, vp, i64, C.c_int, f32,
+                                               C.c_int]),
         "scn_maxpool": (C.c_int, [vp, vp, vp, vp, i64, C.c_int, C.c_int, vp]),
         "scn_maxpool_checked": (C.c_int, [vp, vp, i64, vp, vp, i64, C.c_int, C.c_int, vp]),
         "scn_terminal_pool": (C.c_int, [vp, vp, vp, vp, i64, C.c_int, C.c_int]),
@@ -293,6 +295,11 @@ class Context:
         _check(lib().scn_conv_nin_forward_p(self.h, d_in.ptr, d_rules.ptr, fs, nIn, d_W.ptr, d_B.ptr,
                                             d_prelu.ptr if d_prelu is not None else None, d_out.ptr, M, N, p, act,
                                             precision))
+
+    def conv_nin_forward_a16(self, d_in, nInRows, d_in16, d_rules, fs, nIn, d_W, d_B, d_prelu, d_out, M, N, p=1.0, act=RELU):
+        _check(lib().scn_conv_nin_forward_a16(self.h, d_in.ptr, nInRows, d_in16.ptr, d_rules.ptr, fs, nIn, d_W.ptr,
+                                              d_B.ptr, d_prelu.ptr if d_prelu is not None else None, d_out.ptr, M, N,
+                                              p, act))
 
     def maxpool(self, d_in, d_out, d_rules, nOutSites, ps, Cn, d_choice):
         _check(lib().scn_maxpool(self.h, d_in.ptr, d_out.ptr, d_rules.ptr, nOutSites, ps, Cn, d_choice.ptr))

@@ -1481,7 +1481,11 @@ __device__ __forceinline__ bf16x8 pack_bf16x8(const float4 &x, const float4 &y) 
   return __builtin_bit_cast(bf16x8, r);
 }
 
-template <int NT, int RD, int BL, int GRU>
+// A16: the rows the rules point at are bf16 already (a copy of the fp32 matrix
+// rounded once, nearest even, by k_to_bf16): a lane's eight k of a step are one
+// 16-byte load instead of two and need no conversion.  The values that reach
+// the MFMA are the same, so the results are too, bit for bit.
+template <int NT, int RD, int BL, int GRU, bool A16>
 __global__ void __launch_bounds__(512, NT <= 4 ? 2 : 1)
     k_nin_wstream_bf16(const float *__restrict__ A, const float *__restrict__ W,
                        float *__restrict__ out, long long M, int K, int N,
@@ -1489,6 +1493,8 @@ __global__ void __launch_bounds__(512, NT <= 4 ? 2 : 1)
   static_assert(BL % 2 == 0 && BL % RD == 0, "body = whole slabs and whole turns of the ring");
   constexpr int ROWS = 16, KS = 32, NW = ROWS * NT;
   constexpr bool GATHER = GRU > 0;
+  static_assert(GATHER || !A16, "bf16 rows are read through the rules only");
+  constexpr int ES = A16 ? 2 : 4; // bytes of an element of A
   constexpr int GROUP_BYTES = NW * 16 + 16;   // one group of 8 k: NW columns x 8 bf16, padded
   constexpr int SLAB_BYTES = 8 * GROUP_BYTES; // 64 k
   extern __shared__ __attribute__((aligned(16))) unsigned char sWb[]; // [2][SLAB_BYTES], then the rules
@@ -1524,12 +1530,14 @@ __global__ void __launch_bounds__(512, NT <= 4 ? 2 : 1)
     long long wrap;
     int bufCur, bufNext, rule, ch;
   } st;
-  // where this lane's 8 floats of step tt are; tt >= T: step tt - T of the next panel
-  auto addr = [&](int tt) -> const float * {
+  // where this lane's 8 elements of step tt are; tt >= T: step tt - T of the next panel
+  const unsigned char *const Ab = reinterpret_cast<const unsigned char *>(A);
+  const unsigned char *const zb = reinterpret_cast<const unsigned char *>(gs.zeros);
+  auto addr = [&](int tt) -> const unsigned char * {
     if (!GATHER)
-      return st.cur + KS * tt + (tt >= T ? st.wrap : 0ll);
-    const float *p =
-        (st.rule >= 0 ? A + (long long)st.rule * gs.nIn : gs.zeros) + st.ch;
+      return reinterpret_cast<const unsigned char *>(st.cur + KS * tt + (tt >= T ? st.wrap : 0ll));
+    const unsigned char *p =
+        (st.rule >= 0 ? Ab + (long long)st.rule * gs.nIn * ES : zb) + st.ch * ES;
     const int tn = tt + 1;
     const int kn = KS * (tn >= T ? tn - T : tn) + 8 * q;
     const int fn = (int)__umulhi((unsigned)kn, gs.magic);
@@ -1595,7 +1603,7 @@ __global__ void __launch_bounds__(512, NT <= 4 ? 2 : 1)
     }
   };
 
-  float4 a[RD][2];
+  float4 a[RD][A16 ? 1 : 2]; // (A16: eight bf16 in the one register quad)
   bf16x8 b[2][NT];
   floatx4 acc[NT];
   // this lane's W operands of step s (0, 1) of the slab in buffer buf
@@ -1607,9 +1615,10 @@ __global__ void __launch_bounds__(512, NT <= 4 ? 2 : 1)
       b[slot][j] = *reinterpret_cast<const bf16x8 *>(p + 256 * j);
   };
   auto load_a = [&](int slot, int tt) {
-    const float *p = addr(tt);
+    const unsigned char *p = addr(tt);
     a[slot][0] = *reinterpret_cast<const float4 *>(p);
-    a[slot][1] = *reinterpret_cast<const float4 *>(p + 4);
+    if (!A16)
+      a[slot][1] = *reinterpret_cast<const float4 *>(p + 16);
   };
 
   const bool more = pg + pgStep < pgEnd;
@@ -1675,7 +1684,8 @@ __global__ void __launch_bounds__(512, NT <= 4 ? 2 : 1)
           read_b(cur, 0, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
-        const bf16x8 av = pack_bf16x8(a[s % RD][0], a[s % RD][1]);
+        const bf16x8 av = A16 ? __builtin_bit_cast(bf16x8, a[s % RD][0])
+                              : pack_bf16x8(a[s % RD][0], a[s % RD][A16 ? 0 : 1]);
 #pragma unroll
         for (int j = 0; j < NT; ++j)
           acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, b[s & 1][j], acc[j], 0, 0, 0);
@@ -1728,7 +1738,8 @@ __global__ void __launch_bounds__(512, NT <= 4 ? 2 : 1)
 template <int NT, int RD, int BL>
 static int launch_wstream_bf16(scn_ctx *ctx, const float *A, const float *W,
                                float *out, long long M, int K, int N,
-                               const Epilogue &ep, const GatherSource *gs) {
+                               const Epilogue &ep, const GatherSource *gs,
+                               bool a16 = false) {
   constexpr int NW = 16 * NT;
   const int nSplits = N / NW;
   const size_t lds =
@@ -1740,29 +1751,36 @@ static int launch_wstream_bf16(scn_ctx *ctx, const float *A, const float *W,
   static OncePerDevice configured; // one set of attribute calls per instantiation and device
   const int rc = configured.run(ctx->device, [&]() {
     int rc = SCN_OK;
-#define SCN_WSB_LDS(G)                                                         \
+#define SCN_WSB_LDS(G, H)                                                      \
   if (hipFuncSetAttribute(                                                     \
-          reinterpret_cast<const void *>(k_nin_wstream_bf16<NT, RD, BL, G>),   \
+          reinterpret_cast<const void *>(k_nin_wstream_bf16<NT, RD, BL, G, H>), \
           hipFuncAttributeMaxDynamicSharedMemorySize,                          \
           WRES_LDS_BYTES) != hipSuccess)                                       \
     rc = SCN_ERR_HIP;
-    SCN_WSB_LDS(0) SCN_WSB_LDS(1) SCN_WSB_LDS(3) SCN_WSB_LDS(7)
+    SCN_WSB_LDS(0, false) SCN_WSB_LDS(1, false) SCN_WSB_LDS(3, false) SCN_WSB_LDS(7, false)
+    SCN_WSB_LDS(1, true) SCN_WSB_LDS(3, true) SCN_WSB_LDS(7, true)
 #undef SCN_WSB_LDS
     return rc;
   });
   SCN_REQUIRE(rc == SCN_OK, SCN_ERR_HIP, "hipFuncSetAttribute failed");
   const dim3 grid((unsigned)(wgs * nSplits));
-#define SCN_WSB_GO(G, src)                                                     \
-  hipLaunchKernelGGL((k_nin_wstream_bf16<NT, RD, BL, G>), grid, dim3(512),     \
+#define SCN_WSB_GO(G, H, src)                                                  \
+  hipLaunchKernelGGL((k_nin_wstream_bf16<NT, RD, BL, G, H>), grid, dim3(512),  \
                      lds, ctx->stream, A, W, out, M, K, N, ep, src, nSplits)
   if (!gs)
-    SCN_WSB_GO(0, GatherSource());
+    SCN_WSB_GO(0, false, GatherSource());
+  else if (a16 && gs->fs <= 4)
+    SCN_WSB_GO(1, true, *gs);
+  else if (a16 && gs->fs <= 12)
+    SCN_WSB_GO(3, true, *gs);
+  else if (a16)
+    SCN_WSB_GO(7, true, *gs);
   else if (gs->fs <= 4)
-    SCN_WSB_GO(1, *gs);
+    SCN_WSB_GO(1, false, *gs);
   else if (gs->fs <= 12)
-    SCN_WSB_GO(3, *gs);
+    SCN_WSB_GO(3, false, *gs);
   else
-    SCN_WSB_GO(7, *gs);
+    SCN_WSB_GO(7, false, *gs);
 #undef SCN_WSB_GO
   return SCN_OK;
 }
@@ -1776,8 +1794,9 @@ static bool wstream_bf16_shape(long long M, int K, int N) {
 }
 static bool wstream_bf16_forward(scn_ctx *ctx, const float *A, const float *W,
                                  float *out, long long M, int K, int N,
-                                 const Epilogue &ep, const GatherSource *gs) {
-  if (!wstream_bf16_shape(M, K, N) || (gs && gs->nIn % 8 != 0))
+                                 const Epilogue &ep, const GatherSource *gs,
+                                 bool a16 = false) {
+  if (!wstream_bf16_shape(M, K, N) || (gs && gs->nIn % 8 != 0) || (a16 && !gs))
     return false;
   const int T = K / 32;
   static const int widths[] = {6, 4, 2};
@@ -1795,10 +1814,10 @@ static bool wstream_bf16_forward(scn_ctx *ctx, const float *A, const float *W,
 #define SCN_WSB_CASE(NTV)                                                      \
   case NTV:                                                                    \
     if (T % 4 == 0)                                                            \
-      return launch_wstream_bf16<NTV, 4, 4>(ctx, A, W, out, M, K, N, ep, gs) == SCN_OK; \
+      return launch_wstream_bf16<NTV, 4, 4>(ctx, A, W, out, M, K, N, ep, gs, a16) == SCN_OK; \
     if (T % 6 == 0)                                                            \
-      return launch_wstream_bf16<NTV, 3, 6>(ctx, A, W, out, M, K, N, ep, gs) == SCN_OK; \
-    return launch_wstream_bf16<NTV, 2, 2>(ctx, A, W, out, M, K, N, ep, gs) == SCN_OK;
+      return launch_wstream_bf16<NTV, 3, 6>(ctx, A, W, out, M, K, N, ep, gs, a16) == SCN_OK; \
+    return launch_wstream_bf16<NTV, 2, 2>(ctx, A, W, out, M, K, N, ep, gs, a16) == SCN_OK;
   switch (nt) {
     SCN_WSB_CASE(2)
     SCN_WSB_CASE(4)
@@ -1982,10 +2001,11 @@ static void launch_mfma(scn_ctx *ctx, const float *A, const float *W,
                        ctx->stream, A, W, out, M, K, N, ep, GatherSource());
 }
 
+// rows16: a bf16 copy of the matrix the rules point into, or null
 static int nin_forward(scn_ctx *ctx, const float *d_A, const float *d_W,
                        const float *d_B, const float *d_prelu, float *d_out,
                        int64_t M, int K, int N, float p, int act, int precision,
-                       const GatherSource *gs) {
+                       const GatherSource *gs, const void *rows16 = nullptr) {
   SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_nin_forward: null context");
   SCN_REQUIRE(M >= 0 && K >= 1 && N >= 1, SCN_ERR_ARG,
               "scn_nin_forward: M %lld K %d N %d", (long long)M, K, N);
@@ -2014,8 +2034,12 @@ static int nin_forward(scn_ctx *ctx, const float *d_A, const float *d_W,
                    ((uintptr_t)d_W & 15) == 0 && ((uintptr_t)d_out & 15) == 0;
   // bf16 operands only where the contraction is big enough to matter; the
   // classifier head and the thin first layers stay fp32
-  if (vec && K >= 64 && act != SCN_SOFTMAX && precision == SCN_BF16 &&
-      wstream_bf16_forward(ctx, d_A, d_W, d_out, M, K, N, ep, gs)) {
+  if (vec && K >= 64 && act != SCN_SOFTMAX && precision == SCN_BF16 && rows16 && gs &&
+      ((uintptr_t)rows16 & 15) == 0 &&
+      wstream_bf16_forward(ctx, reinterpret_cast<const float *>(rows16), d_W, d_out, M, K, N, ep, gs, true)) {
+    // the same kernel reading rows that are bf16 already
+  } else if (vec && K >= 64 && act != SCN_SOFTMAX && precision == SCN_BF16 &&
+             wstream_bf16_forward(ctx, d_A, d_W, d_out, M, K, N, ep, gs)) {
     // W-streaming kernel with bf16 operands took it
   } else if (vec && K >= 64 && act != SCN_SOFTMAX && precision != SCN_FP32) {
     SCN_REQUIRE(!gs, SCN_ERR_ARG,
@@ -2125,6 +2149,55 @@ extern "C" int scn_conv_nin_supported_p(int fs, int nIn, int N, int precision) {
   // bf16 operands: the shapes of the bf16 W-streaming kernel, whatever M
   return precision == SCN_BF16 && nIn % 8 == 0 &&
          wstream_bf16_shape(1 << 20, fs * nIn, N);
+}
+
+// d_out16[i] = bf16(d_in[i]), nearest even (v_cvt_pk_bf16_f32), eight a lane
+__global__ void __launch_bounds__(256)
+    k_to_bf16(const float4 *__restrict__ in, uint4 *__restrict__ out, long long n8) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n8)
+    return;
+  const float4 x = in[2 * i], y = in[2 * i + 1];
+  uint4 r;
+  r.x = pack_bf16x2(x.x, x.y);
+  r.y = pack_bf16x2(x.z, x.w);
+  r.z = pack_bf16x2(y.x, y.y);
+  r.w = pack_bf16x2(y.z, y.w);
+  out[i] = r;
+}
+
+extern "C" int scn_conv_nin_forward_a16(scn_ctx *ctx, const float *d_in, int64_t nInRows,
+                                        void *d_in16, const int32_t *d_rules, int fs,
+                                        int nIn, const float *d_W, const float *d_B,
+                                        const float *d_prelu, float *d_out, int64_t M,
+                                        int N, float p, int act) {
+  SCN_REQUIRE(ctx, SCN_ERR_ARG, "scn_conv_nin_forward_a16: null context");
+  SCN_REQUIRE(scn_conv_nin_supported_p(fs, nIn, N, SCN_BF16), SCN_ERR_ARG,
+              "scn_conv_nin_forward_a16: fs %d nIn %d N %d is outside the bf16 fused kernel's range", fs,
+              nIn, N);
+  SCN_REQUIRE(nInRows >= 0 && (d_in16 || nInRows == 0), SCN_ERR_ARG,
+              "scn_conv_nin_forward_a16: %lld input rows, no room for their bf16 copy", (long long)nInRows);
+  SCN_REQUIRE(d_rules || M == 0, SCN_ERR_ARG, "scn_conv_nin_forward_a16: null rules");
+  SCN_REQUIRE(((uintptr_t)d_in & 15) == 0 && ((uintptr_t)d_W & 15) == 0 && ((uintptr_t)d_in16 & 15) == 0,
+              SCN_ERR_ARG, "scn_conv_nin_forward_a16: buffers must be 16-byte aligned");
+  if (M == 0)
+    return SCN_OK;
+  const bool copy = nIn % 8 == 0 && nInRows > 0 && d_in;
+  if (copy) {
+    ProfScope prof(ctx, SCN_K_GATHER);
+    const long long n8 = (long long)nInRows * nIn / 8;
+    hipLaunchKernelGGL(k_to_bf16, dim3(scn_ceil_div(n8, 256)), dim3(256), 0, ctx->stream,
+                       reinterpret_cast<const float4 *>(d_in), reinterpret_cast<uint4 *>(d_in16), n8);
+    SCN_HIP_CHECK(hipGetLastError());
+  }
+  GatherSource gs = GatherSource();
+  gs.rules = d_rules;
+  gs.fs = fs;
+  gs.nIn = nIn;
+  gs.magic = (unsigned)((1ull << 32) / (unsigned)nIn + 1);
+  gs.zeros = ctx->d_zeros;
+  return nin_forward(ctx, d_in, d_W, d_B, d_prelu, d_out, M, fs * nIn, N, p, act, SCN_BF16, &gs,
+                     copy ? d_in16 : nullptr);
 }
 
 extern "C" int scn_conv_nin_forward(scn_ctx *ctx, const float *d_in,

@@ -11,6 +11,10 @@ public:
   vectorCUDA<float> features;
   vectorCUDA<float> dfeatures; // gradient of the cost, training batches only
   vectorCUDA<int> poolingChoices;
+  // room for a bf16 copy of `features` (two bytes an element), made by a
+  // following fused convolution with bf16 operands whose window is large
+  // enough for the rows to be read many times over
+  vectorCUDA<float> features16;
   SpatiallySparseBatchSubInterface();
   void reset();
 };

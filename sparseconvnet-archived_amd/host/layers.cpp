@@ -311,6 +311,20 @@ static bool nin_fused(cudaMemStream &ms, SpatiallySparseBatchInterface &input,
     gather_now(ms, *src, input);
     return false;
   }
+  // bf16 operands, a window of eight or more sites and a matrix worth the
+  // pass: round the input once and let the contraction read the bf16 rows
+  // (the same result bit for bit, half the bytes through the caches)
+  if (precision == SCN_BF16 && fs >= 8 && nIn % 8 == 0 &&
+      (int64_t)output.nSpatialSites * fs >= (int64_t)1 << 20) {
+    const size_t elems = (size_t)src->nSpatialSites * nIn;
+    src->sub->features16.resize64(elems / 2 + 8);
+    SCN_CHECKED(scn_conv_nin_forward_a16(
+        ms.ctx, src->sub->features.dPtr(), src->nSpatialSites,
+        src->sub->features16.dPtr(), input.rules.dPtr(), fs, nIn, W.dPtr(),
+        B.dPtr(), prelu ? prelu->dPtr() : nullptr, output.sub->features.dPtr(),
+        output.nSpatialSites, nFeaturesOut, p, act));
+    return true;
+  }
   SCN_CHECKED(scn_conv_nin_forward_p(
       ms.ctx, src->sub->features.dPtr(), input.rules.dPtr(), fs, nIn, W.dPtr(),
       B.dPtr(), prelu ? prelu->dPtr() : nullptr, output.sub->features.dPtr(),

@@ -352,6 +352,39 @@ def test_fused_gather_nin_matches_the_two_kernels_bit_for_bit(scn, ctx, rows, fs
     assert not scn.lib().scn_conv_nin_supported(5, 3, 32)  # ... or not a multiple of 4
 
 
+@pytest.mark.parametrize("M,rows,fs,nIn,N,act", [
+    (40000, 9000, 27, 64, 64, "RELU"), (20011, 5000, 8, 64, 96, "PRELU"), (7000, 3000, 4, 32, 64, "VLEAKYRELU"),
+    (1030, 400, 9, 128, 160, "RELU"), (3, 10, 4, 64, 32, "NOSIGMOID"), (2600, 700, 4, 96, 128, "LEAKYRELU"),
+    # a shape the bf16 kernel does not take (few channels): what scn_conv_nin_forward_p(SCN_BF16) does
+    (5000, 1000, 4, 3, 32, "RELU")])
+def test_bf16_rows_rounded_once_give_the_same_bits(scn, ctx, M, rows, fs, nIn, N, act):
+    """scn_conv_nin_forward_a16 (the input matrix rounded to bf16 once, the contraction reading those rows) against
+    scn_conv_nin_forward_p with SCN_BF16 (rows rounded in registers as they are read): the same bits, and within the
+    bf16 bar (2e-2 of the row's scale) of the oracle."""
+    rng = np.random.default_rng(M + rows + N)
+    act_id = getattr(scn, act)
+    K = fs * nIn
+    src = rng.standard_normal((rows, nIn)).astype(np.float32)
+    rules = rng.integers(-1, rows, size=(M, fs)).astype(np.int32)
+    W = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float32)
+    B = rng.standard_normal(N).astype(np.float32)
+    prelu = rng.uniform(0.1, 0.4, N).astype(np.float32) if act == "PRELU" else None
+    d_src, d_rules, d_W, d_B = ctx.array(src), ctx.array(rules), ctx.array(W), ctx.array(B)
+    d_prelu = ctx.array(prelu) if prelu is not None else None
+    print("a16 M=%d rows=%d fs=%d nIn=%d N=%d %s" % (M, rows, fs, nIn, N, act), flush=True)
+    one = ctx.array(np.full((M, N), 9, np.float32))
+    two = ctx.array(np.full((M, N), 9, np.float32))
+    rows16 = ctx.empty((rows * nIn + 8) // 2, np.float32)  # two bytes an element
+    ctx.conv_nin_forward(d_src, d_rules, fs, nIn, d_W, d_B, d_prelu, one, M, N, 0.9, act_id, scn.BF16)
+    ctx.conv_nin_forward_a16(d_src, rows, rows16, d_rules, fs, nIn, d_W, d_B, d_prelu, two, M, N, 0.9, act_id)
+    got = two.download()
+    assert np.array_equal(got, one.download())
+    G = np.where(rules[:, :, None] >= 0, src[np.maximum(rules, 0)], 0).reshape(M, K).astype(np.float32)
+    want = orc.nin_forward(G, W, B, prelu, 0.9, act_id, f64=True)
+    scale = 0.9 * (np.abs(G).astype(np.float64) @ np.abs(W).astype(np.float64) + np.abs(B)) + 1e-6
+    assert np.max(np.abs(got - want) / scale) <= 2e-2
+
+
 def test_maxpool_refuses_inputs_beyond_32_bit_choices(scn, ctx):
     """poolingChoices are 32-bit element indices into the input (MaxPoolingLayer.cu:9-35): the entry point that is told
     the input's row count refuses 2^31 elements and more.  An argument check: nothing is launched, no such buffer
