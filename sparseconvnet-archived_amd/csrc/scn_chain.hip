@@ -7,7 +7,22 @@
 // layer at a time over the whole batch through tables in HBM, four launches
 // per layer; for a 2-D net that is some fifty dependent launches of a few
 // microseconds each.  Here the plan and fill calls of consecutive layers are
-// only recorded (scn_ctx_chain_rules) and then run together:
+// only recorded (scn_ctx_chain_rules) and then run together, in one of two ways.
+//
+// Chains of square windows without a minimum of active inputs (a terminal
+// layer may end them) are built from the output side (second half of this
+// file, per-lane bodies in scn_pyr_dev.h):
+//
+//   k_pyr_masks     one wavefront per sample: the occupancy masks of all
+//                   layers, each the dilation of the one before, their rank
+//                   prefixes and the sample's site counts;
+//   k_pyr_rules     one workgroup per sample: the counts of the samples before
+//                   it, then per output site in sweeps over all layers at once
+//                   -- sites by rank, owners, rows, entry lists, rule rows --
+//                   written at their batch-global places.
+//
+// Every other chain (a minimum of active inputs, triangular lattices, windows
+// of more than 16 sites) goes the older way, from the input side:
 //
 //   k_chain_sample  one workgroup per sample carries the sample's grid --
 //                   occupancy mask, rank prefix, (key, row) by rank -- in LDS
@@ -788,11 +803,10 @@ __global__ void __launch_bounds__(PLACE_THREADS) k_chain_place(ChainArgs a) {
 // either kind of barrier, its arguments, its input and its own first level
 // intact, and never with one chain at a time; the instruction stream shows
 // every wait in place.  The cause was not found.  A single wavefront has no
-// barrier to pass and gave no wrong word in any run; it costs about 2 us.
+// barrier to pass and gave no wrong word in any run; it costs a 126 x 126 field
+// about 2 us and a 47^3 one about 20.
 #define PYR_A_THREADS 64
 #define PYR_A_BARRIER() lds_barrier()
-// keeps a wavefront-uniform value in a scalar register from here on
-#define PYR_PIN(v) asm volatile("" : "+s"(v))
 #define PYR_B_THREADS 1024
 static_assert(sizeof(PyrArgs) <= 4096, "kernel arguments");
 

@@ -12,8 +12,10 @@
 //           OR-ed over the window and thinned by the stride, up to 64 sites of
 //           a row at a time (pyr_dilate_pieces), plus a popcount prefix per
 //           word (the rank of a site = its position in iteration order);
-//   pass B  per output site, in five sweeps over ALL layers at once with one
-//           barrier between them: enumerate the sites by rank; find each
+//   pass B  per output site, in five sweeps over ALL layers at once (or, for a
+//           sample too large for that, over as many consecutive layers as
+//           the LDS holds, window after window) with one barrier between
+//           them: enumerate the sites by rank; find each
 //           site's owner (first set bit of its window) and mark, in the owner's
 //           16-bit ownership mask, which of its candidates this is (an LDS
 //           atomic OR); prefix sums of the owned counts per layer; a site's row
