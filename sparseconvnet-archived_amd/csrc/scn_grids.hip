@@ -133,6 +133,9 @@ __device__ __forceinline__ void sample_ranks(const GridView &in, unsigned &rs,
 
 // per sample: does it need a background row, and how many were appended
 // before it.  One block of SCAN1_THREADS lanes.
+// OWNERS: `in` is the mask of the owning inputs with its prefix, so the rank
+// of a position is already the number of outputs before it and base is unused.
+template <bool OWNERS = false>
 __device__ __forceinline__ void
 plan_samples_body(const GridView &in, const unsigned *base, long long nEntries,
                   long long fullSize, int *outBg, int *bgBefore,
@@ -154,8 +157,11 @@ plan_samples_body(const GridView &in, const unsigned *base, long long nEntries,
       unsigned rs = b0 == 0 ? rs0 : rank_of(in, (long long)b * in.vol);
       re = b0 == 0 ? re0 : rank_of(in, (long long)(b + 1) * in.vol);
       sampleStart[b] = rs;
-      long long oc = (long long)base[re] - (long long)base[rs];
-      notFull = oc < fullSize;
+      if (!OWNERS) {
+        rs = base[rs];
+        re = base[re];
+      }
+      notFull = (long long)re - (long long)rs < fullSize;
     }
     // prefix of notFull over the lanes: shuffles inside a wavefront, the
     // wavefront totals through LDS (two sets of words: one barrier per round)
@@ -180,14 +186,15 @@ plan_samples_body(const GridView &in, const unsigned *base, long long nEntries,
     int excl = before + incl - notFull + carry;
     if (b < in.batch) {
       bgBefore[b] = excl;
-      outBg[b] = notFull ? (int)base[re] + excl : -1;
+      outBg[b] = notFull ? (int)re + excl : -1;
     }
     carry += total;
     flip ^= 1;
   }
   if (t == 0) {
-    const long long nSites = (long long)base[nEntries] + carry; // nOutputSpatialSites
-    const long long nActive = (long long)base[nEntries];        // active output sites
+    const long long nActive = // active output sites
+        OWNERS ? (long long)rank_of(in, (long long)in.batch * in.vol) : (long long)base[nEntries];
+    const long long nSites = nActive + carry; // nOutputSpatialSites
     const long long over = (inMeta && inMeta[META_OVERFLOW]) || nSites > boundRows ||
                            nActive > boundActive;
     meta[META_SITES] = nSites;
@@ -211,6 +218,7 @@ plan_samples_body(const GridView &in, const unsigned *base, long long nEntries,
   }
 }
 
+template <bool OWNERS>
 __global__ void __launch_bounds__(SCAN1_THREADS)
     k_plan_samples(GridView in, const unsigned *base, long long nEntries,
                    long long fullSize, int *outBg, int *bgBefore,
@@ -220,9 +228,9 @@ __global__ void __launch_bounds__(SCAN1_THREADS)
                    long long boundActive, int pinnedSlot) {
   unsigned rs0, re0;
   sample_ranks(in, rs0, re0);
-  plan_samples_body(in, base, nEntries, fullSize, outBg, bgBefore, sampleStart,
-                    scalars, badSites, ticket, meta, inMeta, boundRows,
-                    boundActive, pinnedSlot, rs0, re0);
+  plan_samples_body<OWNERS>(in, base, nEntries, fullSize, outBg, bgBefore, sampleStart,
+                            scalars, badSites, ticket, meta, inMeta, boundRows,
+                            boundActive, pinnedSlot, rs0, re0);
 }
 
 // small batches: prefix sum of the owned counts and the per-sample pass in
@@ -334,17 +342,77 @@ __global__ void k_plan_emit_masked(GridView in, GridView out, Geom g,
   siteKey[row] = pack_row_site<D>(b, j);
 }
 
-// The same with one lane per input walking the set bits of its ownership
-// mask: for boxes of many candidates (3-D: 27) of which an input owns a few,
-// where a lane per (input, candidate) would mostly read masks and leave.
+// position of the r-th (from 0) set bit of x, which has more than r
+__device__ __forceinline__ int select_bit64(unsigned long long x, unsigned r) {
+  int pos = 0;
+  unsigned v = (unsigned)x;
+  unsigned c = (unsigned)__popc(v);
+  if (r >= c) {
+    r -= c;
+    v = (unsigned)(x >> 32);
+    pos = 32;
+  }
+#pragma unroll
+  for (int half = 16; half >= 2; half >>= 1) {
+    c = (unsigned)__popc(v & ((1u << half) - 1u));
+    if (r >= c) {
+      r -= c;
+      v >>= half;
+      pos += half;
+    }
+  }
+  return pos + (r >= (v & 1u) ? 1 : 0);
+}
+
+// The lanes of a wavefront hold counts; their exclusive prefix goes to
+// before[0 .. 63] (LDS, this wavefront's part) and the total is returned.
+__device__ __forceinline__ unsigned wave_deal_prefix(unsigned cnt, unsigned *before) {
+  const int lane = threadIdx.x & 63;
+  unsigned incl = cnt;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const unsigned up = __shfl_up(incl, off, 64);
+    if (lane >= off)
+      incl += up;
+  }
+  before[lane] = incl - cnt;
+  return __shfl(incl, 63, 64);
+}
+// which lane's items hold item o of the wavefront (o < total): the last lane
+// with at most o items before it
+__device__ __forceinline__ int wave_deal_find(const unsigned *before, unsigned o) {
+  int l = 0;
+#pragma unroll
+  for (int step = 32; step; step >>= 1)
+    if (before[l + step] <= o)
+      l += step;
+  return l;
+}
+
+// The same for boxes of many candidates (3-D: 27) of which an input owns a
+// few, where a lane per (input, candidate) would mostly read masks and leave,
+// and a lane per input walking its own mask would leave most lanes idle.  A
+// lane takes its input apart once (sample, box of candidates, where its
+// outputs go) and leaves that in LDS; then the wavefront deals the set bits
+// of its 64 ownership masks out to its lanes, one output each.
+struct WalkItem {
+  unsigned long long mask;
+  int lo[3];
+  unsigned ext[3], inv[3];
+  unsigned idx;
+  int b, shiftRows;
+};
 template <int D>
-__global__ void k_plan_emit_walk(GridView in, GridView out, Geom g,
-                                 const long long *ekey, Count nEntries,
-                                 const long long *outMeta, const unsigned *base,
-                                 const unsigned long long *ownMask,
-                                 const unsigned *rankOf, const int *bgBefore,
-                                 const int *outBg, long long *okey, int *orow,
-                                 long long *siteKey) {
+__global__ void __launch_bounds__(256)
+    k_plan_emit_walk(GridView in, GridView out, Geom g,
+                     const long long *ekey, Count nEntries,
+                     const long long *outMeta, const unsigned *base,
+                     const unsigned long long *ownMask,
+                     const unsigned *rankOf, const int *bgBefore,
+                     const int *outBg, long long *okey, int *orow,
+                     long long *siteKey) {
+  __shared__ WalkItem items[256];
+  __shared__ unsigned before[256];
   const long long live = count_now(nEntries) > in.batch ? count_now(nEntries) : in.batch;
   long long e = xcd_contiguous_block((live + 255) / 256) * blockDim.x + threadIdx.x;
   if (outMeta[META_OVERFLOW])
@@ -354,43 +422,55 @@ __global__ void k_plan_emit_walk(GridView in, GridView out, Geom g,
     if (r >= 0)
       siteKey[r] = -1 - e;
   }
-  if (e >= count_now(nEntries))
-    return;
-  unsigned long long mask = ownMask[e];
-  const long long p = ekey[e];
-  const unsigned r = rankOf[e];
-  if (mask == 0)
-    return;
-  int i[D], lo[D], hi[D], j[D];
-  const int b = split_site<D>(p, g.volIn, g.nIn, i);
-  (void)cand_box<D>(g, b, i, lo, hi);
-  // a box is at most 64 candidates, so its sides are small: x / ext by a
-  // multiplication (exact for x < 64: the error of the factor stays below 1 / 64 ext)
-  unsigned ext[D], inv[D];
+  const int first = threadIdx.x & ~63;
+  unsigned long long mask = 0;
+  if (e < count_now(nEntries)) {
+    // all three at once: one memory latency instead of two in a row
+    mask = ownMask[e];
+    const long long p = ekey[e];
+    const unsigned r = rankOf[e];
+    if (mask) {
+      WalkItem &it = items[threadIdx.x];
+      int i[D], lo[D], hi[D];
+      const int b = split_site<D>(p, g.volIn, g.nIn, i);
+      (void)cand_box<D>(g, b, i, lo, hi);
+      // a box is at most 64 candidates, so its sides are small: x / ext by a
+      // multiplication (exact for x < 64: the error of the factor stays below 1 / 64 ext)
 #pragma unroll
-  for (int a = 0; a < D; ++a) {
-    ext[a] = (unsigned)(hi[a] - lo[a]);
-    inv[a] = 65536u / ext[a] + 1u;
+      for (int a = 0; a < D; ++a) {
+        it.lo[a] = lo[a];
+        it.ext[a] = (unsigned)(hi[a] - lo[a]);
+        it.inv[a] = 65536u / it.ext[a] + 1u;
+      }
+      it.mask = mask;
+      it.idx = base[r];
+      it.b = b;
+      it.shiftRows = bgBefore[b];
+    }
   }
-  unsigned idx = base[r];
-  const int shiftRows = bgBefore[b];
-  while (mask) { // ascending candidate = ascending output key
-    unsigned rem = (unsigned)(__ffsll((long long)mask) - 1);
-    mask &= mask - 1;
+  const unsigned total = wave_deal_prefix((unsigned)__popcll(mask), before + first);
+  __syncthreads();
+  for (unsigned o = threadIdx.x & 63; o < total; o += 64) {
+    const int l = wave_deal_find(before + first, o);
+    const WalkItem &it = items[first + l];
+    const unsigned nth = o - before[first + l];
+    // ascending candidate = ascending output key
+    unsigned rem = (unsigned)select_bit64(it.mask, nth);
+    int j[D];
 #pragma unroll
     for (int a = D - 1; a >= 0; --a) {
-      const unsigned up = (rem * inv[a]) >> 16;
-      j[a] = lo[a] + (int)(rem - up * ext[a]);
+      const unsigned up = (rem * it.inv[a]) >> 16;
+      j[a] = it.lo[a] + (int)(rem - up * it.ext[a]);
       rem = up;
     }
-    const long long po = (long long)b * g.volOut + encode_key<D>(j, g.nOut);
-    const int row = (int)idx + shiftRows;
+    const unsigned idx = it.idx + nth;
+    const long long po = (long long)it.b * g.volOut + encode_key<D>(j, g.nOut);
+    const int row = (int)idx + it.shiftRows;
     if (out.bits)
       atomicOr(&out.bits[po >> 6], 1ull << (po & 63));
     okey[idx] = po;
     orow[idx] = row;
-    siteKey[row] = pack_row_site<D>(b, j);
-    ++idx;
+    siteKey[row] = pack_row_site<D>(it.b, j);
   }
 }
 
@@ -517,6 +597,135 @@ __global__ void __launch_bounds__(256)
       }
   }
   outBits[w] = res;
+}
+
+// Windows of side 2 that tile the field (stride 2, no minimum): every input
+// lies in one window, a window's sites along the last axis are an even bit of
+// the mask and its odd neighbour (fields have an even side, so rows start at
+// even positions), and the owner of an output -- the first active site of its
+// window in key order -- can be told from the input mask a word at a time.
+// One lane per word of the input mask: a site owns its window's output when it
+// is active, no earlier row of the window holds an active site in its pair of
+// columns, and it is the first of its own pair.  The number of owners before
+// a position (prefix of this mask) is the number of outputs before it in the
+// reference's iteration order, so no per-input count is needed
+// (Regions.cu:528-653 for the order).
+template <int D>
+__global__ void __launch_bounds__(256)
+    k_tile2_owners(GridView in, Geom g, const long long *inMeta,
+                   unsigned long long *ownBits, long long nWords,
+                   long long totalBits) {
+  const long long w = xcd_contiguous_block((nWords + 255) / 256) * blockDim.x + threadIdx.x;
+  if (w >= nWords)
+    return;
+  unsigned long long res = 0;
+  long long pos = 64 * w;
+  const long long end = pos + 64 < totalBits ? pos + 64 : totalBits;
+  // (an input whose own deferred plan outgrew its bounds counts for nothing)
+  const unsigned long long X =
+      pos < end && !(inMeta && inMeta[META_OVERFLOW]) ? in.bits[w] : 0ull;
+  if (X) {
+    const unsigned long long EVEN = 0x5555555555555555ull;
+    int i[D];
+    (void)split_site<D>(pos, g.volIn, g.nIn, i);
+    const long long plane = (long long)g.nIn * g.nIn;
+    while (pos < end) {
+      long long len = g.nIn - i[D - 1];
+      len = len < end - pos ? len : end - pos;
+      const int at = (int)(pos - 64 * w); // even: rows and words start at even positions
+      const unsigned long long m = (len >= 64 ? ~0ull : (1ull << len) - 1ull) << at;
+      const unsigned long long x = X & m;
+      if (x) {
+        // the earlier rows of the windows, their bits under this piece's
+        unsigned long long earlier = 0;
+        if constexpr (D >= 2) {
+          const int dy = i[D - 2] & 1;
+          if (dy)
+            earlier |= get_bits128(in.bits, pos - g.nIn).lo;
+          if constexpr (D == 3) {
+            if (i[0] & 1) {
+              earlier |= get_bits128(in.bits, pos - plane - (long long)dy * g.nIn).lo;
+              earlier |= get_bits128(in.bits, pos - plane + (long long)(1 - dy) * g.nIn).lo;
+            }
+          }
+        }
+        earlier <<= at;
+        const unsigned long long taken =
+            earlier | ((earlier & EVEN) << 1) | ((earlier >> 1) & EVEN) | ((x & EVEN) << 1);
+        res |= x & ~taken;
+      }
+      pos += len;
+      i[D - 1] += (int)len;
+#pragma unroll
+      for (int a = D - 1; a > 0; --a)
+        if (i[a] >= g.nIn) {
+          i[a] = 0;
+          ++i[a - 1];
+        }
+      if (i[0] >= g.nIn) // the next sample
+        i[0] = 0;
+    }
+  }
+  ownBits[w] = res;
+}
+
+// The outputs of such windows, in ascending position of their owners = the
+// reference's order.  A wavefront takes 64 words of the owners' mask and deals
+// their set bits out to its lanes one each (prefix of the words' counts, a
+// search in it, the r-th set bit of the word found), so that the lanes write
+// consecutive entries whatever the words hold.  The wavefront's first position
+// is taken apart once; a site's coordinates follow from it by carries.
+template <int D>
+__global__ void __launch_bounds__(256)
+    k_tile2_emit(GridView in, Geom g, const unsigned long long *ownBits,
+                 const unsigned *ownPrefix, long long nWords,
+                 const long long *outMeta, const int *bgBefore,
+                 const int *outBg, long long *okey, int *orow,
+                 long long *siteKey) {
+  __shared__ unsigned long long sWord[256];
+  __shared__ unsigned sBefore[256];
+  const long long live = nWords > in.batch ? nWords : in.batch;
+  const long long w = xcd_contiguous_block((live + 255) / 256) * blockDim.x + threadIdx.x;
+  if (outMeta[META_OVERFLOW])
+    return; // the bounds did not hold: nothing may be written
+  if (w < in.batch) { // background rows
+    const int r = outBg[w];
+    if (r >= 0)
+      siteKey[r] = -1 - w;
+  }
+  const int lane = threadIdx.x & 63, first = threadIdx.x & ~63;
+  const unsigned long long word = w < nWords ? ownBits[w] : 0ull;
+  const unsigned total = wave_deal_prefix((unsigned)__popcll(word), sBefore + first);
+  sWord[threadIdx.x] = word;
+  __syncthreads();
+  if (total == 0)
+    return;
+  const long long w0 = w - lane; // the wavefront's first word, which exists as total > 0
+  const unsigned idx0 = ownPrefix[w0];
+  int i0[D];
+  const int b0 = split_site<D>(64 * w0, g.volIn, g.nIn, i0);
+  for (unsigned o = lane; o < total; o += 64) {
+    const int l = wave_deal_find(sBefore + first, o);
+    unsigned carry =
+        64u * (unsigned)l + (unsigned)select_bit64(sWord[first + l], o - sBefore[first + l]);
+    int j[D];
+#pragma unroll
+    for (int a = D - 1; a >= 0; --a) {
+      unsigned t = (unsigned)i0[a] + carry;
+      carry = 0;
+      if (t >= (unsigned)g.nIn) {
+        carry = t / (unsigned)g.nIn;
+        t -= carry * (unsigned)g.nIn;
+      }
+      j[a] = (int)(t >> 1);
+    }
+    const int b = b0 + (int)carry;
+    const unsigned idx = idx0 + o;
+    const int row = (int)idx + bgBefore[b];
+    okey[idx] = (long long)b * g.volOut + encode_key<D>(j, g.nOut);
+    orow[idx] = row;
+    siteKey[row] = pack_row_site<D>(b, j);
+  }
 }
 
 // clears a hash table (all-ones = empty slots) and an occupancy mask at once
@@ -1435,6 +1644,15 @@ static int triangle_size(int n, int d) { // utilities.cu:27-32
   return fs;
 }
 
+// SCN_TILE2_WORDWISE=0 sends windows of side 2, stride 2 down the general path
+static bool tile2_enabled() {
+  static const bool on = [] {
+    const char *e = getenv("SCN_TILE2_WORDWISE");
+    return !(e && e[0] == '0');
+  }();
+  return on;
+}
+
 template <int D>
 static int plan_regions_d(scn_ctx *ctx, scn_grids *in, scn_grids *out,
                           const Geom &g, long long fullSize,
@@ -1469,11 +1687,24 @@ static int plan_regions_d(scn_ctx *ctx, scn_grids *in, scn_grids *out,
   if (g.mode == MODE_SQ_FMP)
     maxCand = fmpCand; // from the tables themselves
   const bool masked = maxCand <= 64;
-  if (masked) {
+  // windows of side 2 that tile the field: owners and counts from the input
+  // mask a word at a time (k_tile2_owners)
+  const bool tiled = tile2_enabled() && g.mode == MODE_SQ_NOMIN && g.size == 2 &&
+                     g.stride == 2 && in->batch > 0;
+  const long long ownWords = (long long)in->nWords + 1; // one past: the rank of the end
+  if (tiled) {
+    SCN_TRY(out->ownMask.reserve((size_t)ownWords + 8)); // the scan reads whole 32-byte groups
+    SCN_TRY(out->base.reserve((size_t)ownWords + 2));
+    SCN_TRY(out->scanTmp.reserve(scn_scan_tmp_elems((size_t)ownWords)));
+    hipLaunchKernelGGL(k_tile2_owners<D>, dim3(xcd_grid(scn_ceil_div(ownWords, 256))),
+                       dim3(256), 0, ctx->stream, vin, g, inMeta, out->ownMask.p,
+                       ownWords, (long long)in->batch * g.volIn);
+    SCN_HIP_CHECK(hipGetLastError());
+  } else if (masked) {
     SCN_TRY(out->ownMask.reserve((size_t)nE + 2));
     SCN_TRY(out->rankOf.reserve((size_t)nE + 2));
   }
-  if (nE > 0) {
+  if (nE > 0 && !tiled) {
     hipLaunchKernelGGL(k_plan_count<D>, dim3(xcd_grid(scn_ceil_div(nE, 256))), dim3(256),
                        0, ctx->stream, vin, g, in->ekey.p, nEc, inMeta, out->cnt.p,
                        masked ? out->ownMask.p : nullptr, out->rankOf.p);
@@ -1481,7 +1712,17 @@ static int plan_regions_d(scn_ctx *ctx, scn_grids *in, scn_grids *out,
   }
   const long long *bad = (const long long *)(ctx->d_scalars + 15);
   const long long ticket = ++ctx->ticket;
-  if ((size_t)nE <= SCAN1_MAX_ELEMS) {
+  if (tiled) {
+    SCN_TRY(scn_scan_exclusive_popc64(ctx->stream, (const uint64_t *)out->ownMask.p,
+                                      out->base.p, (size_t)ownWords, out->scanTmp.p));
+    GridView owners = vin;
+    owners.bits = out->ownMask.p;
+    owners.prefix = out->base.p;
+    hipLaunchKernelGGL(k_plan_samples<true>, dim3(1), dim3(SCAN1_THREADS), 0, ctx->stream,
+                       owners, (const unsigned *)nullptr, 0ll, fullSize, out->bg.p,
+                       out->bgBefore.p, out->sampleStart.p, (long long *)ctx->d_pinned, bad,
+                       ticket, out->meta.p, inMeta, boundRows, boundActive, slot);
+  } else if ((size_t)nE <= SCAN1_MAX_ELEMS) {
     hipLaunchKernelGGL(k_plan_scan_samples, dim3(1), dim3(SCAN1_THREADS), 0,
                        ctx->stream, vin, out->cnt.p, out->base.p, nE, fullSize,
                        out->bg.p, out->bgBefore.p, out->sampleStart.p,
@@ -1490,7 +1731,7 @@ static int plan_regions_d(scn_ctx *ctx, scn_grids *in, scn_grids *out,
   } else {
     SCN_TRY(scn_scan_exclusive_u32(ctx->stream, out->cnt.p, out->base.p,
                                    (size_t)nE, out->scanTmp.p));
-    hipLaunchKernelGGL(k_plan_samples, dim3(1), dim3(SCAN1_THREADS), 0, ctx->stream, vin,
+    hipLaunchKernelGGL(k_plan_samples<false>, dim3(1), dim3(SCAN1_THREADS), 0, ctx->stream, vin,
                        out->base.p, nE, fullSize, out->bg.p, out->bgBefore.p,
                        out->sampleStart.p, (long long *)ctx->d_pinned, bad, ticket, out->meta.p,
                          inMeta, boundRows, boundActive, slot);
@@ -1526,7 +1767,14 @@ static int plan_regions_d(scn_ctx *ctx, scn_grids *in, scn_grids *out,
     SCN_HIP_CHECK(hipGetLastError());
     vout.bits = nullptr;
   }
-  if (nThreads > 0 && masked && maxCand > 9) {
+  if (tiled) {
+    const long long lanes = ownWords > in->batch ? ownWords : in->batch;
+    hipLaunchKernelGGL(k_tile2_emit<D>, dim3(xcd_grid(scn_ceil_div(lanes, 256))), dim3(256),
+                       0, ctx->stream, vin, g, out->ownMask.p, out->base.p, ownWords,
+                       out->meta.p, out->bgBefore.p, out->bg.p, out->ekey.p, out->erow.p,
+                       out->siteKey.p);
+    SCN_HIP_CHECK(hipGetLastError());
+  } else if (nThreads > 0 && masked && maxCand > 9) {
     hipLaunchKernelGGL(k_plan_emit_walk<D>, dim3(xcd_grid(scn_ceil_div(nThreads, 256))),
                        dim3(256), 0, ctx->stream, vin, vout, g,
                        in->ekey.p, nEc, out->meta.p, out->base.p, out->ownMask.p,

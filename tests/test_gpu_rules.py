@@ -47,7 +47,7 @@ def test_reference_executed_vectors_on_gpu(scn, ctx, case):
 
 
 GEOMS = [(1, 2, 1, 6), (1, 3, 2, 4), (2, 2, 1, 5), (2, 3, 1, 4), (2, 3, 2, 3), (2, 2, 2, 4), (2, 2, 3, 3),
-         (3, 2, 1, 3), (3, 3, 1, 2), (3, 2, 2, 2), (3, 3, 2, 2), (2, 3, 1, 30), (3, 3, 1, 9), (2, 5, 3, 7)]
+         (3, 2, 1, 3), (3, 3, 1, 2), (3, 2, 2, 2), (3, 3, 2, 2), (2, 3, 1, 30), (3, 3, 1, 9), (2, 5, 3, 7), (1, 2, 2, 5), (3, 2, 2, 5)]
 
 
 @pytest.mark.parametrize("d,size,stride,nOut", GEOMS)
@@ -62,7 +62,7 @@ def test_square_rules(scn, ctx, d, size, stride, nOut, minActive):
 
 
 WIDE_GEOMS = [(1, 3, 1, 300), (1, 3, 2, 150), (1, 5, 3, 90), (2, 2, 1, 100), (2, 3, 2, 70), (2, 4, 3, 45), (3, 3, 1, 70),
-              (3, 2, 2, 40)]
+              (3, 2, 2, 40), (1, 2, 2, 100), (2, 2, 2, 50), (3, 2, 2, 33)]
 
 
 @pytest.mark.parametrize("d,size,stride,nOut", WIDE_GEOMS)
