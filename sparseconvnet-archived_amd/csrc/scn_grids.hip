@@ -482,17 +482,44 @@ __global__ void __launch_bounds__(256)
 struct Bits128 {
   unsigned long long lo, hi;
 };
+// the L (at most 128) mask bits from position p on, and whatever follows them up to 128
 __device__ __forceinline__ Bits128 get_bits128(const unsigned long long *bits,
-                                               long long p) {
+                                               long long p, int L) {
   const long long w = p >> 6;
   const int sh = (int)(p & 63);
-  Words3 ww;
+  Words2 ww; // one request; a third word only when the L bits reach into it
   __builtin_memcpy(&ww, bits + w, sizeof(ww));
-  const unsigned long long a = ww.a, b = ww.b, c = ww.c;
+  const unsigned long long a = ww.a, b = ww.b;
+  unsigned long long c = 0;
+  if (sh + L > 128)
+    c = bits[w + 2];
   Bits128 r;
   r.lo = sh ? (a >> sh) | (b << (64 - sh)) : a;
   r.hi = sh ? (b >> sh) | (c << (64 - sh)) : b;
   return r;
+}
+// 96 mask bits from position p on, as three 32-bit words: one request at the
+// 4-byte boundary below p and three funnel shifts
+struct __attribute__((packed, aligned(4))) Dwords4 {
+  unsigned d[4];
+};
+__device__ __forceinline__ void get_bits96(const unsigned long long *bits, long long p,
+                                           unsigned &r0, unsigned &r1, unsigned &r2) {
+  Dwords4 v;
+  __builtin_memcpy(&v, reinterpret_cast<const unsigned *>(bits) + (p >> 5), sizeof(v));
+  const unsigned s = (unsigned)p & 31u;
+  r0 = __builtin_amdgcn_alignbit(v.d[1], v.d[0], s);
+  r1 = __builtin_amdgcn_alignbit(v.d[2], v.d[1], s);
+  r2 = __builtin_amdgcn_alignbit(v.d[3], v.d[2], s);
+}
+// 64 mask bits from position p on
+__device__ __forceinline__ unsigned long long get_bits64(const unsigned long long *bits,
+                                                         long long p) {
+  const long long w = p >> 6;
+  const int sh = (int)(p & 63);
+  Words2 ww;
+  __builtin_memcpy(&ww, bits + w, sizeof(ww));
+  return sh ? (ww.a >> sh) | (ww.b << (64 - sh)) : ww.a;
 }
 // the even bits of x, packed
 __device__ __forceinline__ unsigned long long even_bits(unsigned long long x) {
@@ -504,7 +531,9 @@ __device__ __forceinline__ unsigned long long even_bits(unsigned long long x) {
   x = (x | (x >> 16)) & 0x00000000FFFFFFFFull;
   return x;
 }
-template <int D>
+// S: the window's side when it is 2 or 3 (the loops over a window's rows unroll and all its rows are requested at
+// once), else 0 (read from g)
+template <int D, int S>
 __global__ void __launch_bounds__(256)
     k_mask_dilate(GridView in, Geom g, unsigned long long *outBits,
                   long long nWords, long long totalBits) {
@@ -513,71 +542,111 @@ __global__ void __launch_bounds__(256)
   const long long w = xcd_contiguous_block((nWords + 255) / 256) * blockDim.x + threadIdx.x;
   if (w >= nWords)
     return;
+  const int size = S ? S : g.size;
+  constexpr int UN = S ? S : 1; // (no unrolling of loops whose length is not known here)
   unsigned long long res = 0;
   long long pos = 64 * w;
   const long long end = pos + 64 < totalBits ? pos + 64 : totalBits;
   // a piece reads (len - 1) stride + size input bits: at most 128
-  const int lenMax = g.stride == 1 ? 64 : (128 - g.size) / g.stride + 1;
+  const int lenMax = g.stride == 1 ? 64 : (128 - size) / g.stride + 1;
   int j[D];
   int b = split_site<D>(pos, g.volOut, g.nOut, j);
   while (pos < end) {
     long long len = g.nOut - j[D - 1];
     len = len < end - pos ? len : end - pos;
     len = len < lenMax ? len : lenMax;
-    const int L = ((int)len - 1) * g.stride + g.size;
+    const int L = ((int)len - 1) * g.stride + size;
     const long long sampleBase = (long long)b * g.volIn;
-    unsigned long long lo = 0, hi = 0;
-    if (D == 1) {
-      const Bits128 x = get_bits128(in.bits, sampleBase + (long long)j[0] * g.stride);
-      lo = x.lo;
-      hi = x.hi;
-    } else if (D == 2) {
-      for (int q0 = 0; q0 < g.size; ++q0) {
-        const Bits128 x = get_bits128(
-            in.bits, sampleBase + (long long)(j[0] * g.stride + q0) * g.nIn +
-                         (long long)j[1] * g.stride);
-        lo |= x.lo;
-        hi |= x.hi;
+    unsigned long long r;
+    if (S && g.stride == 1) {
+      // at most 66 bits a row: three 32-bit words, shifted as such (64-bit
+      // shifts by a variable run at a quarter of the rate)
+      unsigned x0 = 0, x1 = 0, x2 = 0;
+      auto row = [&](long long p) {
+        unsigned a0, a1, a2;
+        get_bits96(in.bits, p, a0, a1, a2);
+        x0 |= a0;
+        x1 |= a1;
+        x2 |= a2;
+      };
+      if constexpr (D == 1) {
+        row(sampleBase + j[0]);
+      } else if constexpr (D == 2) {
+#pragma unroll
+        for (int q0 = 0; q0 < S; ++q0)
+          row(sampleBase + (long long)(j[0] + q0) * g.nIn + j[1]);
+      } else {
+#pragma unroll
+        for (int q0 = 0; q0 < S; ++q0)
+#pragma unroll
+          for (int q1 = 0; q1 < S; ++q1)
+            row(sampleBase + ((long long)(j[0] + q0) * g.nIn + (j[1] + q1)) * g.nIn + j[2]);
       }
+      // bit t: any of the S sites from t on (t below 64)
+      unsigned y0 = x0, y1 = x1;
+#pragma unroll
+      for (int q = 1; q < S; ++q) {
+        y0 |= __builtin_amdgcn_alignbit(x1, x0, q);
+        y1 |= __builtin_amdgcn_alignbit(x2, x1, q);
+      }
+      r = (unsigned long long)y0 | ((unsigned long long)y1 << 32);
     } else {
-      for (int q0 = 0; q0 < g.size; ++q0)
-        for (int q1 = 0; q1 < g.size; ++q1) {
+      unsigned long long lo = 0, hi = 0;
+      if (D == 1) {
+        const Bits128 x = get_bits128(in.bits, sampleBase + (long long)j[0] * g.stride, L);
+        lo = x.lo;
+        hi = x.hi;
+      } else if (D == 2) {
+#pragma unroll UN
+        for (int q0 = 0; q0 < size; ++q0) {
           const Bits128 x = get_bits128(
-              in.bits,
-              sampleBase +
-                  ((long long)(j[0] * g.stride + q0) * g.nIn +
-                   (j[D > 1 ? 1 : 0] * g.stride + q1)) * g.nIn +
-                  (long long)j[D - 1] * g.stride);
+              in.bits, sampleBase + (long long)(j[0] * g.stride + q0) * g.nIn +
+                           (long long)j[1] * g.stride, L);
           lo |= x.lo;
           hi |= x.hi;
         }
-    }
-    // only the L bits of this piece's windows
-    if (L < 64) {
-      lo &= (1ull << L) - 1ull;
-      hi = 0;
-    } else if (L < 128) {
-      hi &= L == 64 ? 0ull : (1ull << (L - 64)) - 1ull;
-    }
-    // bit t: any of the `size` sites from t on
-    unsigned long long ylo = lo, yhi = hi;
-    for (int q = 1; q < g.size; ++q) {
-      lo = (lo >> 1) | (hi << 63);
-      hi >>= 1;
-      ylo |= lo;
-      yhi |= hi;
-    }
-    unsigned long long r;
-    if (g.stride == 1) {
-      r = ylo;
-    } else if (g.stride == 2) {
-      r = even_bits(ylo) | (even_bits(yhi) << 32);
-    } else {
-      r = 0;
-      for (int t = 0; t < (int)len; ++t) {
-        const int at = t * g.stride;
-        const unsigned long long bit = at < 64 ? (ylo >> at) : (yhi >> (at - 64));
-        r |= (bit & 1ull) << t;
+      } else {
+#pragma unroll UN
+        for (int q0 = 0; q0 < size; ++q0)
+#pragma unroll UN
+          for (int q1 = 0; q1 < size; ++q1) {
+            const Bits128 x = get_bits128(
+                in.bits,
+                sampleBase +
+                    ((long long)(j[0] * g.stride + q0) * g.nIn +
+                     (j[D > 1 ? 1 : 0] * g.stride + q1)) * g.nIn +
+                    (long long)j[D - 1] * g.stride, L);
+            lo |= x.lo;
+            hi |= x.hi;
+          }
+      }
+      // only the L bits of this piece's windows
+      if (L < 64) {
+        lo &= (1ull << L) - 1ull;
+        hi = 0;
+      } else if (L < 128) {
+        hi &= L == 64 ? 0ull : (1ull << (L - 64)) - 1ull;
+      }
+      // bit t: any of the `size` sites from t on
+      unsigned long long ylo = lo, yhi = hi;
+#pragma unroll UN
+      for (int q = 1; q < size; ++q) {
+        lo = (lo >> 1) | (hi << 63);
+        hi >>= 1;
+        ylo |= lo;
+        yhi |= hi;
+      }
+      if (g.stride == 1) {
+        r = ylo;
+      } else if (g.stride == 2) {
+        r = even_bits(ylo) | (even_bits(yhi) << 32);
+      } else {
+        r = 0;
+        for (int t = 0; t < (int)len; ++t) {
+          const int at = t * g.stride;
+          const unsigned long long bit = at < 64 ? (ylo >> at) : (yhi >> (at - 64));
+          r |= (bit & 1ull) << t;
+        }
       }
     }
     if (len < 64)
@@ -641,11 +710,11 @@ __global__ void __launch_bounds__(256)
         if constexpr (D >= 2) {
           const int dy = i[D - 2] & 1;
           if (dy)
-            earlier |= get_bits128(in.bits, pos - g.nIn).lo;
+            earlier |= get_bits64(in.bits, pos - g.nIn);
           if constexpr (D == 3) {
             if (i[0] & 1) {
-              earlier |= get_bits128(in.bits, pos - plane - (long long)dy * g.nIn).lo;
-              earlier |= get_bits128(in.bits, pos - plane + (long long)(1 - dy) * g.nIn).lo;
+              earlier |= get_bits64(in.bits, pos - plane - (long long)dy * g.nIn);
+              earlier |= get_bits64(in.bits, pos - plane + (long long)(1 - dy) * g.nIn);
             }
           }
         }
@@ -859,7 +928,9 @@ __global__ void __launch_bounds__(256)
                       RankScan rs, int rowsPerBlock, int pitch,
                       unsigned magicWidth, unsigned magicSize) {
   __shared__ uint32_t ldsScan[SCAN1_LDS_WORDS];
-  __shared__ __attribute__((aligned(16))) int staged[FILL_LDS_INTS + 256];
+  // rowsPerBlock rows of `pitch` words (the launch says how many bytes: what the
+  // rows need and no more, so that short rows leave room for more workgroups)
+  extern __shared__ __attribute__((aligned(16))) int staged[];
   long long blk = blockIdx.x;
   if (SCAN) {
     if (blk == 0) {
@@ -928,12 +999,14 @@ __global__ void __launch_bounds__(256)
           unsigned present[U];
 #pragma unroll
           for (int u = 0; u < U; ++u) {
-            unsigned long long lo = w0[u] >> sh[u];
-            if (sh[u])
-              lo |= w1[u] << (64 - sh[u]);
-            present[u] = (unsigned)lo & ((1u << S) - 1u);
-            const unsigned rank0 =
-                pre[u] + (unsigned)__popcll(sh[u] ? (w0[u] & ((1ull << sh[u]) - 1ull)) : 0ull);
+            // in 32-bit pieces: 64-bit shifts by a variable run at a quarter of the rate
+            const unsigned d0 = (unsigned)w0[u], d1 = (unsigned)(w0[u] >> 32), d2 = (unsigned)w1[u];
+            const bool upper = sh[u] >= 32;
+            const unsigned s = (unsigned)sh[u] & 31u;
+            present[u] = __builtin_amdgcn_alignbit(upper ? d2 : d1, upper ? d1 : d0, s) & ((1u << S) - 1u);
+            const unsigned below = (1u << s) - 1u; // of the 32-bit word the run starts in
+            const unsigned rank0 = pre[u] + (upper ? (unsigned)__popc(d0) + (unsigned)__popc(d1 & below)
+                                                   : (unsigned)__popc(d0 & below));
             // the rows of the run's active sites are consecutive words: one
             // request (the array has spare words at its end)
             __builtin_memcpy(&val[u], in.rankRow + (present[u] ? rank0 : 0u), sizeof(Rows4));
@@ -1761,7 +1834,9 @@ static int plan_regions_d(scn_ctx *ctx, scn_grids *in, scn_grids *out,
   if (g.mode == MODE_SQ_NOMIN && g.size <= 64) {
     const long long words = (long long)out->nWords + 2;
     const long long blocks = (scn_ceil_div(words, 256) + 7) / 8 * 8; // whole rounds of the 8 XCDs
-    hipLaunchKernelGGL(k_mask_dilate<D>, dim3((unsigned)blocks), dim3(256),
+    auto dilate = g.size == 2 ? k_mask_dilate<D, 2>
+                              : (g.size == 3 ? k_mask_dilate<D, 3> : k_mask_dilate<D, 0>);
+    hipLaunchKernelGGL(dilate, dim3((unsigned)blocks), dim3(256),
                        0, ctx->stream, vin, g, out->bits.p, words,
                        (long long)in->batch * g.volOut);
     SCN_HIP_CHECK(hipGetLastError());
@@ -2156,19 +2231,20 @@ extern "C" int scn_rules_fill(scn_ctx *ctx, const scn_grids *in,
     const unsigned magicSize = (unsigned)((1ull << 32) / (unsigned)g.size + 1);
     dim3 runs(extra ? (unsigned)scn_ceil_div(out->nSites, rowsPerBlock) + extra
                     : xcd_grid(scn_ceil_div(out->nSites, rowsPerBlock)));
+    const size_t stagedBytes = ((size_t)rowsPerBlock * pitch + 4) * sizeof(int);
 #define SCN_FILL_RUNS(D, SC)                                                   \
   if (g.size == 2)                                                             \
-    hipLaunchKernelGGL((k_rules_fill_runs<D, SC, 2>), runs, block, 0,          \
+    hipLaunchKernelGGL((k_rules_fill_runs<D, SC, 2>), runs, block, stagedBytes,\
                        ctx->stream, vin, g, out->siteKey.p, count_sites(out),  \
                        out->meta.p, d_rules, rs, rowsPerBlock, pitch,          \
                        magicWidth, magicSize);                                 \
   else if (g.size == 3)                                                        \
-    hipLaunchKernelGGL((k_rules_fill_runs<D, SC, 3>), runs, block, 0,          \
+    hipLaunchKernelGGL((k_rules_fill_runs<D, SC, 3>), runs, block, stagedBytes,\
                        ctx->stream, vin, g, out->siteKey.p, count_sites(out),  \
                        out->meta.p, d_rules, rs, rowsPerBlock, pitch,          \
                        magicWidth, magicSize);                                 \
   else                                                                         \
-    hipLaunchKernelGGL((k_rules_fill_runs<D, SC, 0>), runs, block, 0,          \
+    hipLaunchKernelGGL((k_rules_fill_runs<D, SC, 0>), runs, block, stagedBytes,\
                        ctx->stream, vin, g, out->siteKey.p, count_sites(out),  \
                        out->meta.p, d_rules, rs, rowsPerBlock, pitch,          \
                        magicWidth, magicSize);

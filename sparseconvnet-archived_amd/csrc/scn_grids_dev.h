@@ -186,13 +186,13 @@ __device__ __forceinline__ int hash_find(const Slot *t, unsigned shift,
   }
 }
 
-// two or three consecutive mask words fetched as one request (global memory
-// takes 16-byte loads at any 4-byte boundary)
+// consecutive mask words fetched as one request (global memory takes 16-byte
+// loads at any 4-byte boundary)
 struct __attribute__((packed, aligned(8))) Words2 {
   unsigned long long a, b;
 };
-struct __attribute__((packed, aligned(8))) Words3 {
-  unsigned long long a, b, c;
+struct __attribute__((packed, aligned(4))) Dwords2 {
+  unsigned a, b;
 };
 
 // row of the site at packed position p, -1 when it is not active
@@ -215,10 +215,15 @@ __device__ __forceinline__ unsigned get_bits(const unsigned long long *bits,
 }
 
 __device__ __forceinline__ unsigned rank_of(const GridView &g, long long p) {
-  long long w = p >> 6;
-  int sh = (int)(p & 63);
-  unsigned long long below = sh ? (g.bits[w] & ((1ull << sh) - 1ull)) : 0ull;
-  return g.prefix[w] + (unsigned)__popcll(below);
+  const long long w = p >> 6;
+  const unsigned long long word = g.bits[w];
+  // the set bits below p in its word, counted in 32-bit halves (64-bit shifts
+  // by a variable run at a quarter of the rate)
+  const unsigned d0 = (unsigned)word, d1 = (unsigned)(word >> 32);
+  const unsigned below = (1u << ((unsigned)p & 31u)) - 1u;
+  const unsigned n = p & 32 ? (unsigned)__popc(d0) + (unsigned)__popc(d1 & below)
+                            : (unsigned)__popc(d0 & below);
+  return g.prefix[w] + n;
 }
 
 __device__ __forceinline__ int sq_outputL(int size, int stride, int i) {
@@ -451,25 +456,24 @@ __device__ __forceinline__ unsigned row_bits(const unsigned long long *bits,
   if (!inside || hi <= lo)
     p = 0; // any valid address; the result is masked away
   p += base;
-  const Pos w = p >> 6;
-  const unsigned sh = (unsigned)(p & 63);
-  unsigned long long a, b;
-  if constexpr (sizeof(Pos) == 8) { // global memory: one 16-byte request
-    Words2 ww;
-    __builtin_memcpy(&ww, bits + w, sizeof(ww));
-    a = ww.a;
-    b = ww.b;
-  } else {
-    a = bits[w];
-    b = bits[w + 1];
-  }
-  unsigned long long v = a >> sh;
-  if (sh)
-    v |= b << (64 - sh);
+  // the two 32-bit words at the 4-byte boundary below p in one request, and a
+  // funnel shift (64-bit shifts by a variable run at a quarter of the rate)
+  Dwords2 ww;
+  __builtin_memcpy(&ww, reinterpret_cast<const unsigned *>(bits) + (p >> 5), sizeof(ww));
+  const unsigned v = __builtin_amdgcn_alignbit(ww.b, ww.a, (unsigned)p & 31u);
   const int m = hi - lo;
-  unsigned r = (unsigned)v & (m >= 32 ? 0xFFFFFFFFu : ((1u << (m > 0 ? m : 0)) - 1u));
+  unsigned r = v & (m >= 32 ? 0xFFFFFFFFu : ((1u << (m > 0 ? m : 0)) - 1u));
   r = (!inside || hi <= lo) ? 0u : r;
   return r << (lo - c0 > 0 ? lo - c0 : 0);
+}
+
+// `len` (<= 32) mask bits from bit position p on, no questions asked
+template <typename Pos>
+__device__ __forceinline__ unsigned bits_at(const unsigned long long *bits, Pos p, int len) {
+  Dwords2 ww;
+  __builtin_memcpy(&ww, reinterpret_cast<const unsigned *>(bits) + (p >> 5), sizeof(ww));
+  const unsigned v = __builtin_amdgcn_alignbit(ww.b, ww.a, (unsigned)p & 31u);
+  return v & (len >= 32 ? 0xFFFFFFFFu : ((1u << len) - 1u));
 }
 
 // Square regions without a minimum (Regions.cu:528-653), window side S: which
@@ -533,12 +537,25 @@ owned_nomin(const unsigned long long *bits, Pos base, const int *i,
   constexpr int W = 2 * S - 1;
   constexpr unsigned FULL = (1u << S) - 1u;
   unsigned m = 0;
+  // a site whose whole neighbourhood lies inside the field (nearly all) needs
+  // no clipping: its rows are at fixed distances from the first
+  bool interior = i[0] >= S - 1;
+#pragma unroll
+  for (int a = 1; a < D; ++a)
+    interior = interior && i[a] >= S - 1 && i[a] + S - 1 < nIn;
   if (D == 2) {
     unsigned nb[S];
+    if (interior) {
+      const Pos p0 = base + (Pos)(i[0] - (S - 1)) * (Pos)nIn + (Pos)(i[1] - (S - 1));
 #pragma unroll
-    for (int r = 0; r < S; ++r) {
-      const int lead[1] = {i[0] - (S - 1) + r};
-      nb[r] = row_bits<2>(bits, base, lead, i[1] - (S - 1), W, nIn);
+      for (int r = 0; r < S; ++r)
+        nb[r] = bits_at(bits, p0 + (Pos)(r * nIn), W);
+    } else {
+#pragma unroll
+      for (int r = 0; r < S; ++r) {
+        const int lead[1] = {i[0] - (S - 1) + r};
+        nb[r] = row_bits<2>(bits, base, lead, i[1] - (S - 1), W, nIn);
+      }
     }
 #pragma unroll
     for (int a0 = 0; a0 < S; ++a0) {
@@ -565,13 +582,24 @@ owned_nomin(const unsigned long long *bits, Pos base, const int *i,
     }
   } else {
     unsigned nb[S][W];
+    if (interior) {
+      const Pos plane = (Pos)nIn * (Pos)nIn;
+      const Pos p0 = base + (Pos)(i[0] - (S - 1)) * plane + (Pos)(i[1] - (S - 1)) * (Pos)nIn +
+                     (Pos)(i[2] - (S - 1));
 #pragma unroll
-    for (int pl = 0; pl < S; ++pl)
+      for (int pl = 0; pl < S; ++pl)
 #pragma unroll
-      for (int r = 0; r < W; ++r) {
-        const int lead[2] = {i[0] - (S - 1) + pl, i[1] - (S - 1) + r};
-        nb[pl][r] = row_bits<3>(bits, base, lead, i[2] - (S - 1), W, nIn);
-      }
+        for (int r = 0; r < W; ++r)
+          nb[pl][r] = bits_at(bits, p0 + (Pos)pl * plane + (Pos)(r * nIn), W);
+    } else {
+#pragma unroll
+      for (int pl = 0; pl < S; ++pl)
+#pragma unroll
+        for (int r = 0; r < W; ++r) {
+          const int lead[2] = {i[0] - (S - 1) + pl, i[1] - (S - 1) + r};
+          nb[pl][r] = row_bits<3>(bits, base, lead, i[2] - (S - 1), W, nIn);
+        }
+    }
 #pragma unroll
     for (int a0 = 0; a0 < S; ++a0) {
       const int d0 = i[0] - a0;
@@ -645,7 +673,9 @@ __device__ __forceinline__ int unpack_row_site(long long sk, int *j) {
 template <int D>
 __device__ __forceinline__ int split_site(long long p, long long vol, int n,
                                           int *c) {
-  const int b = (int)(p / vol);
+  // (64-bit division is a long routine: most batches' masks have fewer than 2^32 bits)
+  const int b = ((unsigned long long)(p | vol) >> 32) == 0 ? (int)((unsigned)p / (unsigned)vol)
+                                                           : (int)(p / vol);
   const long long key = p - (long long)b * vol;
   if (vol < (1ll << 31)) {
     unsigned k = (unsigned)key;
