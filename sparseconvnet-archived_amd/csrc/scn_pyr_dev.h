@@ -109,30 +109,42 @@ PYR_FN pyr_u64 pyr_even_bits(pyr_u64 x) {
   x = (x | (x >> 16)) & 0x00000000FFFFFFFFull;
   return x;
 }
+// Bits that straddle words are taken out in 32-bit pieces: (hi:lo) >> s for s
+// below 32 is one instruction on the device, where a 64-bit shift by a
+// variable amount issues at a quarter of the rate of a 32-bit operation.
+PYR_FN unsigned pyr_alignbit(unsigned hi, unsigned lo, unsigned s) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_amdgcn_alignbit(hi, lo, s);
+#else
+  s &= 31u;
+  return s ? (lo >> s) | (hi << (32u - s)) : lo;
+#endif
+}
 struct PyrBits128 {
-  pyr_u64 lo, hi;
+  unsigned w[4];
 };
-// 128 mask bits from position p on (the mask has two spare words)
+// 128 mask bits from position p on, as four 32-bit words (the mask has two spare words)
 PYR_FN PyrBits128 pyr_bits128(const pyr_u64 *bits, unsigned p) {
-  const unsigned w = p >> 6, sh = p & 63;
-  const pyr_u64 a = bits[w], b = bits[w + 1], c = bits[w + 2];
+  unsigned d[5];
+  __builtin_memcpy(d, reinterpret_cast<const unsigned *>(bits) + (p >> 5), sizeof(d));
   PyrBits128 r;
-  r.lo = sh ? (a >> sh) | (b << (64 - sh)) : a;
-  r.hi = sh ? (b >> sh) | (c << (64 - sh)) : b;
+  for (int i = 0; i < 4; ++i)
+    r.w[i] = pyr_alignbit(d[i + 1], d[i], p & 31u);
   return r;
 }
 // `len` (<= 16) mask bits from position p on
 PYR_FN unsigned pyr_bits(const pyr_u64 *bits, unsigned p, int len) {
-  const unsigned w = p >> 6, sh = p & 63;
-  pyr_u64 v = bits[w] >> sh;
-  if (sh)
-    v |= bits[w + 1] << (64 - sh);
-  return (unsigned)v & ((1u << len) - 1u);
+  unsigned d[2];
+  __builtin_memcpy(d, reinterpret_cast<const unsigned *>(bits) + (p >> 5), sizeof(d));
+  return pyr_alignbit(d[1], d[0], p & 31u) & ((1u << len) - 1u);
 }
 PYR_FN unsigned pyr_rank(const pyr_u64 *bits, const unsigned short *pref, unsigned p) {
-  const unsigned w = p >> 6, sh = p & 63;
-  const pyr_u64 below = sh ? (bits[w] & ((1ull << sh) - 1ull)) : 0ull;
-  return pref[w] + (unsigned)pyr_popc64(below);
+  const unsigned w = p >> 6;
+  const pyr_u64 word = bits[w];
+  const unsigned d0 = (unsigned)word, d1 = (unsigned)(word >> 32);
+  const unsigned below = (1u << (p & 31u)) - 1u;
+  const int n = p & 32u ? pyr_popc32(d0) + pyr_popc32(d1 & below) : pyr_popc32(d0 & below);
+  return pref[w] + (unsigned)n;
 }
 
 // Sites travel as packed coordinates: 30 bits in one dimension, 15 bits an axis
@@ -204,46 +216,33 @@ PYR_FN void pyr_dilate_pieces(const pyr_u64 *in, pyr_u64 *out, int nIn, int nOut
     const unsigned jl = (p - row * segs) * seg; // the piece's first site along the last axis
     unsigned len = (unsigned)nOut - jl;
     len = len < seg ? len : seg;
-    const int L = ((int)len - 1) * stride + size;
-    pyr_u64 lo = 0, hi = 0;
+    // (a piece reads (len - 1) stride + size bits; what lies beyond them in
+    // the 128 fetched only reaches result bits from len on, cleared below)
+    unsigned x[5] = {0u, 0u, 0u, 0u, 0u};
+    auto add = [&](unsigned from) {
+      const PyrBits128 v = pyr_bits128(in, from);
+      for (int i = 0; i < 4; ++i)
+        x[i] |= v.w[i];
+    };
     if (D == 1) {
-      const PyrBits128 x = pyr_bits128(in, jl * (unsigned)stride);
-      lo = x.lo;
-      hi = x.hi;
+      add(jl * (unsigned)stride);
     } else if (D == 2) {
-      for (int q0 = 0; q0 < size; ++q0) {
-        const PyrBits128 x = pyr_bits128(in, ((row * (unsigned)stride + (unsigned)q0) * (unsigned)nIn +
-                                              jl * (unsigned)stride));
-        lo |= x.lo;
-        hi |= x.hi;
-      }
+      for (int q0 = 0; q0 < size; ++q0)
+        add((row * (unsigned)stride + (unsigned)q0) * (unsigned)nIn + jl * (unsigned)stride);
     } else {
       const unsigned j0 = pyr_div(row, (unsigned)nOut, magicN), j1 = row - j0 * (unsigned)nOut;
       for (int q0 = 0; q0 < size; ++q0)
-        for (int q1 = 0; q1 < size; ++q1) {
-          const PyrBits128 x = pyr_bits128(
-              in, ((j0 * (unsigned)stride + (unsigned)q0) * (unsigned)nIn + (j1 * (unsigned)stride + (unsigned)q1)) *
-                          (unsigned)nIn +
-                      jl * (unsigned)stride);
-          lo |= x.lo;
-          hi |= x.hi;
-        }
-    }
-    // only the L bits of this piece's windows
-    if (L < 64) {
-      lo &= (1ull << L) - 1ull;
-      hi = 0;
-    } else if (L < 128) {
-      hi &= L == 64 ? 0ull : (1ull << (L - 64)) - 1ull;
+        for (int q1 = 0; q1 < size; ++q1)
+          add(((j0 * (unsigned)stride + (unsigned)q0) * (unsigned)nIn + (j1 * (unsigned)stride + (unsigned)q1)) *
+                  (unsigned)nIn +
+              jl * (unsigned)stride);
     }
     // bit t: any of the `size` sites from t on
-    pyr_u64 ylo = lo, yhi = hi;
-    for (int q = 1; q < size; ++q) {
-      lo = (lo >> 1) | (hi << 63);
-      hi >>= 1;
-      ylo |= lo;
-      yhi |= hi;
-    }
+    unsigned y[4] = {x[0], x[1], x[2], x[3]};
+    for (int q = 1; q < size; ++q)
+      for (int i = 0; i < 4; ++i)
+        y[i] |= pyr_alignbit(x[i + 1], x[i], (unsigned)q); // (sides stay below 32)
+    const pyr_u64 ylo = (pyr_u64)y[0] | ((pyr_u64)y[1] << 32), yhi = (pyr_u64)y[2] | ((pyr_u64)y[3] << 32);
     pyr_u64 r;
     if (stride == 1) {
       r = ylo;
