@@ -1331,6 +1331,7 @@ __global__ void __launch_bounds__(512, NT <= 4 ? 2 : 1)
 }
 
 #define WSTREAM_LDS_BYTES(nw, sa) (2 * 16 * (sa) * ((nw) + 4) * 4)
+#define WSTREAM_ROUNDS 32
 template <int NT, int SA>
 static int launch_wstream(scn_ctx *ctx, const float *A, const float *W,
                           float *out, long long M, int K, int N,
@@ -1340,7 +1341,15 @@ static int launch_wstream(scn_ctx *ctx, const float *A, const float *W,
   const size_t lds =
       WSTREAM_LDS_BYTES(NW, SA) + (gs ? WRES_RULE_BYTES(gs->fs) : 0);
   long long wgs = scn_ceil_div(scn_ceil_div(M, 16), 8);
-  const long long cap = (long long)ctx->numCU * (lds * 2 <= WRES_LDS_BYTES ? 2 : 1);
+  // Not one workgroup per slot that walks to the end of the matrix: 32 times as
+  // many, each with a 32nd of the panel groups.  Alone the kernel takes the same
+  // time (a workgroup's start is hidden behind its neighbour on the compute
+  // unit, the MFMA pipe is the bound); beside other streams it lets their
+  // kernels onto the chip whenever a workgroup retires instead of after the
+  // last one (a batch of 6.3 M rows: 17.7 -> 16.7 ms in the pipeline, whose
+  // producer otherwise waits out every launch).
+  const long long cap =
+      (long long)ctx->numCU * (lds * 2 <= WRES_LDS_BYTES ? 2 : 1) * WSTREAM_ROUNDS;
   if (wgs > cap)
     wgs = cap;
   static OncePerDevice configured; // one set of attribute calls per instantiation and device
@@ -1745,6 +1754,8 @@ static int launch_wstream_bf16(scn_ctx *ctx, const float *A, const float *W,
   const size_t lds =
       WSTREAM_BF16_LDS_BYTES(NW) + (gs ? WRES_RULE_BYTES(gs->fs) : 0);
   long long wgs = scn_ceil_div(scn_ceil_div(M, 16), 8);
+  // (one workgroup per slot: this kernel is bound by the rows it gathers, a
+  // workgroup's start is not hidden, and more of them cost 9 us each a slot)
   const long long cap = (long long)ctx->numCU * (lds * 2 <= WRES_LDS_BYTES ? 2 : 1);
   if (wgs > cap)
     wgs = cap;
