@@ -1348,10 +1348,17 @@ static int launch_wstream(scn_ctx *ctx, const float *A, const float *W,
   // kernels onto the chip whenever a workgroup retires instead of after the
   // last one (a batch of 6.3 M rows: 17.7 -> 16.7 ms in the pipeline, whose
   // producer otherwise waits out every launch).
-  const long long cap =
-      (long long)ctx->numCU * (lds * 2 <= WRES_LDS_BYTES ? 2 : 1) * WSTREAM_ROUNDS;
-  if (wgs > cap)
-    wgs = cap;
+  // At least two panel groups a workgroup and a multiple of 8 workgroups: the
+  // kernel then gives every XCD a range of the matrix of its own, and the rows
+  // that neighbouring panels gather meet in one L2 (without that a matrix of
+  // 3.3 M rows took twice the bytes from HBM).
+  const long long slots = (long long)ctx->numCU * (lds * 2 <= WRES_LDS_BYTES ? 2 : 1);
+  if (wgs > slots) {
+    long long many = wgs / 2 / 8 * 8;
+    if (many > slots * WSTREAM_ROUNDS)
+      many = slots * WSTREAM_ROUNDS;
+    wgs = many > slots ? many : slots;
+  }
   static OncePerDevice configured; // one set of attribute calls per instantiation and device
   const int rc = configured.run(ctx->device, [&]() {
     int rc = SCN_OK;
