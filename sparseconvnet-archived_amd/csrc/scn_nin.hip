@@ -1129,30 +1129,24 @@ __global__ void __launch_bounds__(512, NT <= 4 ? 2 : 1)
   // panels which gather the same input rows -- neighbours in the rule book --
   // meet in one L2; otherwise workgroup w takes groups w, w + wgs, ...
   // Within its XCD's range a workgroup takes every (wgs / 8)-th group, so the
-  // workgroups on the chip work side by side and move through the range
-  // together -- when all of them are on the chip at once.  With more
-  // workgroups than that (`chunks` > 0: how many of an XCD's are on the chip at
-  // once; they come and go through the launch) the range is cut into as many
-  // pieces as there are rounds of workgroups, and the `chunks` workgroups of a
-  // round walk their piece side by side in the same way.
+  // workgroups on the chip work side by side -- when all of them are on the
+  // chip at once.  With more workgroups than that (`chunks`: they come and go
+  // through the launch) each takes a run of consecutive groups instead, and
+  // the ones on the chip at any moment are again neighbours.
   const int wgs = gridDim.x / nSplits;
   const bool ranges = nSplits == 1 && wgs % 8 == 0 && nGroups >= 2ll * wgs;
-  const bool rounds = ranges && chunks > 0 && (wgs / 8) % chunks == 0;
+  const bool runs = ranges && chunks;
   const int split = blockIdx.x % nSplits;
   const int xcd = blockIdx.x % 8;
   const long long perXcd = (nGroups + 7) / 8;
-  const int pgStep = rounds ? chunks : (ranges ? wgs / 8 : wgs);
+  const long long perWg = (perXcd + wgs / 8 - 1) / (wgs / 8 > 0 ? wgs / 8 : 1);
+  const int pgStep = runs ? 1 : (ranges ? wgs / 8 : wgs);
   const int n0 = split * NW;
-  long long pg = ranges ? xcd * perXcd + blockIdx.x / 8 : blockIdx.x / nSplits;
+  long long pg = runs ? xcd * perXcd + (long long)(blockIdx.x / 8) * perWg
+                      : (ranges ? xcd * perXcd + blockIdx.x / 8 : blockIdx.x / nSplits);
   long long pgEnd = ranges && (xcd + 1) * perXcd < nGroups ? (xcd + 1) * perXcd : nGroups;
-  if (rounds) {
-    const long long perWg = (perXcd + wgs / 8 - 1) / (wgs / 8); // groups a workgroup takes
-    const long long piece = perWg * chunks;
-    const long long first = xcd * perXcd + (long long)((blockIdx.x / 8) / chunks) * piece;
-    pg = first + (blockIdx.x / 8) % chunks;
-    if (first + piece < pgEnd)
-      pgEnd = first + piece;
-  }
+  if (runs && pg + perWg < pgEnd)
+    pgEnd = pg + perWg;
   long long panel = pg * 8 + wave; // may lie past the end
 
   int *const sRw = reinterpret_cast<int *>(sW + 2 * SLAB_FLOATS) +
@@ -1368,14 +1362,11 @@ static int launch_wstream(scn_ctx *ctx, const float *A, const float *W,
   // that neighbouring panels gather meet in one L2 (without that a matrix of
   // 3.3 M rows took twice the bytes from HBM).
   const long long slots = (long long)ctx->numCU * (lds * 2 <= WRES_LDS_BYTES ? 2 : 1);
-  int chunks = 0; // workgroups of an XCD on the chip at once, when they come in rounds
   if (wgs > slots) {
-    long long rounds = wgs / 2 / slots;
-    if (rounds > WSTREAM_ROUNDS)
-      rounds = WSTREAM_ROUNDS;
-    if (rounds >= 2 && slots % 8 == 0)
-      chunks = (int)(slots / 8);
-    wgs = chunks ? slots * rounds : slots;
+    long long many = wgs / 2 / 8 * 8;
+    if (many > slots * WSTREAM_ROUNDS)
+      many = slots * WSTREAM_ROUNDS;
+    wgs = many > slots ? many : slots;
   }
   static OncePerDevice configured; // one set of attribute calls per instantiation and device
   const int rc = configured.run(ctx->device, [&]() {
@@ -1397,7 +1388,7 @@ static int launch_wstream(scn_ctx *ctx, const float *A, const float *W,
 #define SCN_WSTREAM_GO(G, ONE, src)                                            \
   hipLaunchKernelGGL((k_nin_wstream<NT, SA, G, ONE>), grid, dim3(512), lds,    \
                      ctx->stream, A, W, out, M, K, N, ep, src, nSplits,        \
-                     chunks)
+                     wgs > slots ? 1 : 0)
 #define SCN_WSTREAM_EITHER(G)                                                  \
   do {                                                                         \
     if (one)                                                                   \
