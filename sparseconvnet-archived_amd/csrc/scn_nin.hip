@@ -1107,7 +1107,7 @@ template <int NT, int SA, int GRU, bool ONE>
 __global__ void __launch_bounds__(512, NT <= 4 ? 2 : 1)
     k_nin_wstream(const float *__restrict__ A, const float *__restrict__ W,
                   float *__restrict__ out, long long M, int K, int N,
-                  Epilogue ep, GatherSource gs, int nSplits, int chunks) {
+                  Epilogue ep, GatherSource gs, int nSplits) {
   constexpr int ROWS = 16;
   typedef WresPipe<ROWS, NT, SA> Pipe;
   constexpr bool GATHER = GRU > 0;
@@ -1128,25 +1128,16 @@ __global__ void __launch_bounds__(512, NT <= 4 ? 2 : 1)
   // is therefore cut into eight contiguous ranges, one per XCD, so that
   // panels which gather the same input rows -- neighbours in the rule book --
   // meet in one L2; otherwise workgroup w takes groups w, w + wgs, ...
-  // Within its XCD's range a workgroup takes every (wgs / 8)-th group, so the
-  // workgroups on the chip work side by side -- when all of them are on the
-  // chip at once.  With more workgroups than that (`chunks`: they come and go
-  // through the launch) each takes a run of consecutive groups instead, and
-  // the ones on the chip at any moment are again neighbours.
   const int wgs = gridDim.x / nSplits;
   const bool ranges = nSplits == 1 && wgs % 8 == 0 && nGroups >= 2ll * wgs;
-  const bool runs = ranges && chunks;
   const int split = blockIdx.x % nSplits;
   const int xcd = blockIdx.x % 8;
   const long long perXcd = (nGroups + 7) / 8;
-  const long long perWg = (perXcd + wgs / 8 - 1) / (wgs / 8 > 0 ? wgs / 8 : 1);
-  const int pgStep = runs ? 1 : (ranges ? wgs / 8 : wgs);
+  const int pgStep = ranges ? wgs / 8 : wgs;
+  const long long pgEnd =
+      ranges && (xcd + 1) * perXcd < nGroups ? (xcd + 1) * perXcd : nGroups;
   const int n0 = split * NW;
-  long long pg = runs ? xcd * perXcd + (long long)(blockIdx.x / 8) * perWg
-                      : (ranges ? xcd * perXcd + blockIdx.x / 8 : blockIdx.x / nSplits);
-  long long pgEnd = ranges && (xcd + 1) * perXcd < nGroups ? (xcd + 1) * perXcd : nGroups;
-  if (runs && pg + perWg < pgEnd)
-    pgEnd = pg + perWg;
+  long long pg = ranges ? xcd * perXcd + blockIdx.x / 8 : blockIdx.x / nSplits;
   long long panel = pg * 8 + wave; // may lie past the end
 
   int *const sRw = reinterpret_cast<int *>(sW + 2 * SLAB_FLOATS) +
@@ -1387,8 +1378,7 @@ static int launch_wstream(scn_ctx *ctx, const float *A, const float *W,
   const dim3 grid((unsigned)(wgs * nSplits));
 #define SCN_WSTREAM_GO(G, ONE, src)                                            \
   hipLaunchKernelGGL((k_nin_wstream<NT, SA, G, ONE>), grid, dim3(512), lds,    \
-                     ctx->stream, A, W, out, M, K, N, ep, src, nSplits,        \
-                     wgs > slots ? 1 : 0)
+                     ctx->stream, A, W, out, M, K, N, ep, src, nSplits)
 #define SCN_WSTREAM_EITHER(G)                                                  \
   do {                                                                         \
     if (one)                                                                   \
