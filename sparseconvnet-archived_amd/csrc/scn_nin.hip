@@ -1341,23 +1341,23 @@ static int launch_wstream(scn_ctx *ctx, const float *A, const float *W,
   const size_t lds =
       WSTREAM_LDS_BYTES(NW, SA) + (gs ? WRES_RULE_BYTES(gs->fs) : 0);
   long long wgs = scn_ceil_div(scn_ceil_div(M, 16), 8);
-  // Not one workgroup per slot that walks to the end of the matrix: 32 times as
-  // many, each with a 32nd of the panel groups.  Alone the kernel takes the same
-  // time (a workgroup's start is hidden behind its neighbour on the compute
-  // unit, the MFMA pipe is the bound); beside other streams it lets their
-  // kernels onto the chip whenever a workgroup retires instead of after the
-  // last one (a batch of 6.3 M rows: 17.7 -> 16.7 ms in the pipeline, whose
-  // producer otherwise waits out every launch).
-  // At least two panel groups a workgroup and a multiple of 8 workgroups: the
-  // kernel then gives every XCD a range of the matrix of its own, and the rows
-  // that neighbouring panels gather meet in one L2 (without that a matrix of
-  // 3.3 M rows took twice the bytes from HBM).
+  // Not one workgroup per slot that walks to the end of the matrix, but up to
+  // 32 times as many, each with at least three panel groups.  Alone the kernel
+  // takes the same time (a workgroup's start is hidden behind its neighbour on
+  // the compute unit, the MFMA pipe is the bound); beside other streams it
+  // lets their kernels onto the chip whenever a workgroup retires instead of
+  // after the last one (a batch of 6.3 M rows: 17.7 -> 16.6 ms in the
+  // pipeline, whose producer otherwise waits out every launch).  The price is
+  // in the gathered rows: workgroups that come and go drift apart, the panels
+  // that share input rows meet less often in L2, and the kernel reads 8 %
+  // more from HBM at three groups a workgroup (50 % more at one).  A multiple
+  // of 8 workgroups and two groups each keep the kernel's per-XCD ranges.
   const long long slots = (long long)ctx->numCU * (lds * 2 <= WRES_LDS_BYTES ? 2 : 1);
   if (wgs > slots) {
-    long long many = wgs / 2 / 8 * 8;
-    if (many > slots * WSTREAM_ROUNDS)
-      many = slots * WSTREAM_ROUNDS;
-    wgs = many > slots ? many : slots;
+    long long rounds = wgs / (3 * slots);
+    if (rounds > WSTREAM_ROUNDS)
+      rounds = WSTREAM_ROUNDS;
+    wgs = slots * (rounds > 1 ? rounds : 1);
   }
   static OncePerDevice configured; // one set of attribute calls per instantiation and device
   const int rc = configured.run(ctx->device, [&]() {
