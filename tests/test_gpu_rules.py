@@ -225,13 +225,15 @@ def _chain(scn, ctx, dg, outs, term, samples, sizes, geoms):
     return got
 
 
-def test_deferred_counts(scn, ctx):
+@pytest.mark.parametrize("sizes,geoms", [([18, 17, 8, 7], [(2, 1), (3, 2), (2, 1)]),
+                                         ([19, 18, 9, 7], [(2, 1), (2, 2), (3, 1)])])
+def test_deferred_counts(scn, ctx, sizes, geoms):
     """scn_ctx_defer_counts / scn_rules_settle: a batch that fits the bounds of
     the previous one is planned without waiting and gives the same rule books
-    and grids; a batch that outgrows them is reported and planned again."""
+    and grids; a batch that outgrows them is reported and planned again.  (The
+    second chain has windows of side 2 at stride 2, whose owners are read off
+    the input mask a word at a time.)"""
     rng = np.random.default_rng(31)
-    sizes = [18, 17, 8, 7]
-    geoms = [(2, 1), (3, 2), (2, 1)]
     dg = scn.Grids(ctx)
     outs = [scn.Grids(ctx) for _ in geoms]
     term = scn.Grids(ctx)
